@@ -1,0 +1,284 @@
+"""Headline benchmark: INT4 g128 weight-only-quantized linear on one MI355X.
+
+A step is one woq_linear call (through the C ABI) over one synthetic batch.  The default
+workload is the decode shape the metric is quoted on -- activations bf16 [1, 4096], weights
+uint4 [14336, 4096], group 128, lowp_mode BF16 -- with the weight rotated over enough distinct
+copies (> 512 MB in total) that no launch finds its weights in the 256 MB Infinity Cache.
+The same JSON line carries the prefill figure (M = 2048, TFLOP/s), the roofline fraction of
+the dominant kernel and a CPU baseline (the oracle's C port on the host cores).
+
+    python bench.py --gpus 1 --steps 2000 --warmup 200
+"""
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for _p in (ROOT, os.path.join(ROOT, "intel-extension-for-pytorch_amd")):
+    if _p not in sys.path:
+        sys.path.insert(0, _p)
+
+HBM_PEAK_GBS = 8000.0       # MI355X HBM3E, published
+MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
+
+
+def algorithmic_bytes(M, K, N, G):
+    """INT4 weights 1/2 B, bf16 scales 2 B and packed uint4 zeros 1/2 B per (n, group),
+    bf16 activations and outputs."""
+    kg = K // G
+    return N * K // 2 + N * kg * 2 + N * kg // 2 + M * K * 2 + M * N * 2
+
+
+def build_params(lib_mod, x, ctx, out, lowp_mode, act_quant_mode=-1, workspace=None):
+    p = lib_mod.LinearParams()
+    p.struct_size = ctypes.sizeof(lib_mod.LinearParams)
+    p.x = x.data_ptr()
+    p.x_dtype = lib_mod.ACT_BF16
+    p.M, p.K, p.N = x.shape[0], ctx.weight_shape_[1], ctx.weight_shape_[0]
+    p.qweight = ctx.at_weight_.data_ptr()
+    p.weight_dtype = ctx.weight_dtype_
+    p.scales_f32 = ctx.scales_list_[0].data_ptr()
+    p.scales_f16 = ctx.scales_list_[1].data_ptr()
+    p.scales_bf16 = ctx.scales_list_[2].data_ptr()
+    p.zeros_u8 = ctx.zeros_u8_.data_ptr() if ctx.zeros_u8_ is not None else None
+    p.group_size = ctx.group_size_
+    p.bias = ctx.bias_f32_.data_ptr() if ctx.bias_f32_ is not None else None
+    p.lowp_mode = lowp_mode
+    p.act_quant_mode = act_quant_mode
+    p.fusion = 0
+    p.out = out.data_ptr()
+    p.out_dtype = lib_mod.ACT_BF16
+    if workspace is not None:
+        p.workspace = workspace.data_ptr()
+        p.workspace_bytes = workspace.numel()
+    p.force_kernel = 0
+    return p
+
+
+def time_steps(torch, lib, params, steps, warmup, stream):
+    """Launches params round-robin; returns (wall seconds, event milliseconds) for `steps`."""
+    n = len(params)
+    for i in range(warmup):
+        rc = lib.woq_hip_linear(ctypes.byref(params[i % n]))
+        assert rc == 0, lib.woq_hip_last_error()
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    start.record(stream)
+    for i in range(steps):
+        lib.woq_hip_linear(ctypes.byref(params[i % n]))
+    stop.record(stream)
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    return t1 - t0, start.elapsed_time(stop)
+
+
+def time_graph(torch, lib, params, steps, warmup):
+    """Same launches captured once into a HIP graph (one node per weight copy) and replayed."""
+    n = len(params)
+    g = torch.cuda.CUDAGraph()
+    s = torch.cuda.Stream()
+    s.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(s):
+        for p in params:
+            p.stream = s.cuda_stream
+            lib.woq_hip_linear(ctypes.byref(p))
+        torch.cuda.synchronize()
+        with torch.cuda.graph(g, stream=s):
+            for p in params:
+                p.stream = torch.cuda.current_stream().cuda_stream
+                rc = lib.woq_hip_linear(ctypes.byref(p))
+                assert rc == 0, lib.woq_hip_last_error()
+    reps = max(1, steps // n)
+    for _ in range(max(1, warmup // n)):
+        g.replay()
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    start.record()
+    for _ in range(reps):
+        g.replay()
+    stop.record()
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    return reps * n, t1 - t0, start.elapsed_time(stop)
+
+
+def cpu_baseline_decode(case, K, N, G, budget_s=12.0):
+    """The oracle's C port (bf16-regime arithmetic, OpenMP over output channels) on the same
+    decode workload, timed on the host cores this process may use."""
+    import numpy as np
+
+    so = os.path.join(ROOT, "oracle", "libwoq_oracle.so")
+    if not os.path.exists(so):
+        return None
+    cores = len(os.sched_getaffinity(0))
+    os.environ.setdefault("OMP_NUM_THREADS", str(cores))
+    lib = ctypes.CDLL(so)
+    x = case["x"].view(__import__("torch").int16).numpy().astype(np.uint16)
+    qw = np.ascontiguousarray(case["qweight"].numpy())
+    sc = np.ascontiguousarray(case["scales"].float().numpy())
+    zp = np.ascontiguousarray(case["zeros"].float().numpy())
+    acc = np.zeros((1, N), dtype=np.float32)
+    vp = ctypes.c_void_p
+    i64 = ctypes.c_int64
+    lib.woq_ref_linear_int4.argtypes = [vp, i64, i64, i64, vp, vp, vp, i64, vp, ctypes.c_int, i64, i64, vp]
+
+    def run():
+        lib.woq_ref_linear_int4(x.ctypes.data, 1, K, N, qw.ctypes.data, sc.ctypes.data, zp.ctypes.data, G, None, 1,
+                                0, N, acc.ctypes.data)
+
+    run()
+    times = []
+    t_end = time.perf_counter() + budget_s
+    while len(times) < 10 or (time.perf_counter() < t_end and len(times) < 200):
+        t0 = time.perf_counter()
+        run()
+        times.append(time.perf_counter() - t0)
+    med = sorted(times)[len(times) // 2]
+    return {
+        "value": round(algorithmic_bytes(1, K, N, G) / med / 1e9, 3),
+        "unit": "GB/s",
+        "cores": cores,
+        "kind": "port",
+        "sample": f"full workload (M=1, K={K}, N={N}), median of {len(times)} passes of oracle/woq_ref.c",
+        "ms_per_step": round(med * 1e3, 4),
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=4000)
+    ap.add_argument("--warmup", type=int, default=400)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-prefill", action="store_true", help="skip the M=2048 measurement")
+    ap.add_argument("--M", type=int, default=1, help="decode batch (1..16)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path; run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+
+    import ipex_amd  # noqa: F401
+    from ipex_amd import _lib, ops
+    from ipex_amd.utils import synthetic
+
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    lib = _lib.load()
+    dev = torch.device("cuda", 0)
+    stream = torch.cuda.current_stream()
+    K, N, G, M = 4096, 14336, 128, args.M
+
+    case = synthetic.make_int4_case(2, M, K, N, G)
+    ctx0 = ops.WoqLinearOpContext(
+        case["qweight"].to(dev), 2, [N, K], case["scales"].to(dev), case["zeros"].to(dev), None, None, None, G, 2, -1
+    )
+    per_copy = ctx0.at_weight_.numel() + sum(t.numel() * t.element_size() for t in ctx0.scales_list_) + ctx0.zeros_u8_.numel()
+    copies = int(640e6 // per_copy) + 1
+    x = case["x"].to(dev)
+    out = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
+
+    class Copy:
+        pass
+
+    params = []
+    keep = []
+    for i in range(copies):
+        c = Copy()
+        c.__dict__.update(ctx0.__dict__)
+        if i > 0:
+            c.at_weight_ = ctx0.at_weight_.clone()
+            c.scales_list_ = [t.clone() for t in ctx0.scales_list_]
+            c.zeros_u8_ = ctx0.zeros_u8_.clone()
+        keep.append(c)
+        p = build_params(_lib, x, c, out, 2)
+        p.stream = stream.cuda_stream
+        params.append(p)
+
+    nbytes = algorithmic_bytes(M, K, N, G)
+    wall, ev_ms = time_steps(torch, lib, params, args.steps, args.warmup, stream)
+    g_steps, g_wall, g_ev_ms = time_graph(torch, lib, params, args.steps, args.warmup)
+    for p in params:
+        p.stream = stream.cuda_stream
+    # cache-resident figure: the same weight every launch
+    _, hot_ms = time_steps(torch, lib, params[:1], args.steps, args.warmup, stream)
+
+    us_launch = ev_ms * 1e3 / args.steps
+    us_graph = g_ev_ms * 1e3 / g_steps
+    best_us = min(us_launch, us_graph)
+    value = nbytes / (min(wall / args.steps, g_wall / g_steps)) / 1e9
+    achieved = nbytes / (best_us * 1e-6) / 1e9
+
+    result = {
+        "metric": "INT4 WOQ linear: GB/s (% of HBM peak) at M=1; TFLOPS at M=2048",
+        "value": round(value, 1),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(min(wall / args.steps, g_wall / g_steps) * 1e3, 6),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "fp16 x int4 -> fp32 accumulate (lowp_mode BF16, M < 5)" if M < 5 else "bf16 x int4 -> fp32 accumulate",
+        "data": "synthetic",
+        "config": {
+            "workload": f"INT4 g128 woq_linear decode, M={M}, K={K}, N={N}, lowp_mode=BF16, "
+                        f"{copies} rotating weight copies ({copies * per_copy / 1e6:.0f} MB)",
+            "algorithmic_bytes_per_step": nbytes,
+        },
+        "roofline": {
+            "bound": "hbm",
+            "achieved": round(achieved, 1),
+            "peak": HBM_PEAK_GBS,
+            "unit": "GB/s",
+            "frac": round(achieved / HBM_PEAK_GBS, 4),
+            "traffic": None,
+            "kernel": "woq_small_m_kernel",
+            "us_per_launch_stream": round(us_launch, 3),
+            "us_per_launch_graph": round(us_graph, 3),
+            "us_per_launch_cache_resident": round(hot_ms * 1e3 / args.steps, 3),
+        },
+    }
+
+    if not args.no_prefill:
+        Mp = 2048
+        casep = synthetic.make_int4_case(3, Mp, K, N, G, outliers=True)
+        xp = casep["x"].to(dev)
+        outp = torch.empty(Mp, N, dtype=torch.bfloat16, device=dev)
+        flops = 2.0 * Mp * K * N
+        pre = {}
+        for name, lowp, aq in (("bf16", 2, -1), ("int8", 3, 6)):
+            ws = None
+            wbytes = lib.woq_hip_linear_workspace_bytes(Mp, K, lowp, aq, G)
+            if wbytes:
+                ws = torch.empty(wbytes, dtype=torch.uint8, device=dev)
+            pp = build_params(_lib, xp, keep[0], outp, lowp, aq, ws)
+            pp.stream = stream.cuda_stream
+            steps_p = max(10, min(200, args.steps // 20))
+            _, ms = time_steps(torch, lib, [pp], steps_p, max(3, steps_p // 5), stream)
+            us = ms * 1e3 / steps_p
+            pre[name] = {"us_per_step": round(us, 2), "tflops": round(flops / (us * 1e-6) / 1e12, 1)}
+        result["prefill_m2048"] = {
+            "workload": f"INT4 g128 woq_linear prefill, M={Mp}, K={K}, N={N}",
+            "flops_per_step": flops,
+            "lowp_bf16": pre["bf16"],
+            "lowp_int8_per_row": pre["int8"],
+            "frac_of_bf16_mfma_peak": round(pre["bf16"]["tflops"] / MFMA_BF16_PEAK_TFLOPS, 4),
+            "peak_tflops": MFMA_BF16_PEAK_TFLOPS,
+        }
+
+    if not args.no_cpu:
+        result["cpu_baseline"] = cpu_baseline_decode(synthetic.make_int4_case(2, 1, K, N, G), K, N, G)
+    else:
+        result["cpu_baseline"] = None
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

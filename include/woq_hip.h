@@ -1,0 +1,215 @@
+/*
+ * woq_hip.h -- C ABI of the MI355X (gfx950) weight-only-quantized linear library.
+ *
+ * Every entry point takes plain device pointers, sizes and a hipStream_t (passed as
+ * void*).  Nothing here allocates device memory: callers own every buffer, including
+ * the workspace that lowp_mode=INT8 needs.  All work is enqueued on the given stream;
+ * no entry point synchronises the host.
+ *
+ * Return value: 0 on success, non-zero on error; woq_hip_last_error() then returns a
+ * description (thread-local).  Argument errors are reported before anything is
+ * launched, mirroring the TORCH_CHECK behaviour of the reference op
+ * (csrc/cpu/jit/cpu/kernels/LinearWoqPacked.cpp:537-543, csrc/cpu/aten/Linear.cpp:574-577).
+ *
+ * Reference interfaces replaced (paths relative to the reference tree):
+ *   woq_hip_pack_weight      <- woq_linear_pack_weight / qlinear_woq_pack
+ *                               (csrc/cpu/aten/Linear.cpp:379-438,
+ *                                csrc/cpu/aten/kernels/WoqUtilKrnl.cpp:32-249)
+ *   woq_hip_unpack_weight    <- woq_linear_unpack_weight / qlinear_woq_unpack
+ *                               (csrc/cpu/aten/Linear.cpp:464-495,
+ *                                csrc/cpu/aten/kernels/WoqUtilKrnl.cpp:251-324)
+ *   woq_hip_pack_qparams     <- ContextLinearWoq constructor: dtype copies and the
+ *                               [N, K/G] -> [N/Nb, K/G, Nb] permutation of scales / zero
+ *                               points (csrc/cpu/jit/cpu/kernels/ContextLinearWoq.h:37-133)
+ *   woq_hip_unpack_int4_zeros<- int32-compressed zero points -> one value per group
+ *                               (csrc/cpu/jit/cpu/kernels/LinearWoqPacked.cpp:98-103)
+ *   woq_hip_dynamic_quant    <- dynamic_quantize_per_block
+ *                               (csrc/cpu/aten/utils/woq_dynamic_quant.h:1526-1750)
+ *   woq_hip_linear           <- woq_linear_kernel -> qlinear_woq_affine
+ *                               (csrc/cpu/aten/Linear.cpp:499-546,
+ *                                csrc/cpu/aten/kernels/WoqLinearKrnl.cpp:56-161) including the
+ *                               fused post-ops of woq_linear_unary_kernel /
+ *                               woq_linear_binary_kernel (csrc/cpu/aten/Linear.cpp:619-801)
+ *   woq_hip_dequant_weight   <- dequantize_woq_weight (csrc/cpu/aten/utils/woq_utils.h:79-163)
+ */
+#ifndef WOQ_HIP_H_
+#define WOQ_HIP_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* weight dtype, csrc/cpu/aten/utils/woq_defines.h:6-9 */
+#define WOQ_HIP_DTYPE_INT8 1
+#define WOQ_HIP_DTYPE_INT4 2
+#define WOQ_HIP_DTYPE_NF4 3
+
+/* lowp_mode, csrc/cpu/aten/utils/woq_defines.h:21-24 */
+#define WOQ_HIP_LOWP_NONE 0
+#define WOQ_HIP_LOWP_FP16 1
+#define WOQ_HIP_LOWP_BF16 2
+#define WOQ_HIP_LOWP_INT8 3
+
+/* act_quant_mode, csrc/cpu/aten/utils/woq_defines.h:11-19 */
+#define WOQ_HIP_QUANT_A_NONE (-1)
+#define WOQ_HIP_QUANT_A_PER_TENSOR 0
+#define WOQ_HIP_QUANT_A_PER_K_BLOCK 1
+#define WOQ_HIP_QUANT_A_PER_M 2
+#define WOQ_HIP_QUANT_A_PER_M_K_BLOCK 3
+#define WOQ_HIP_QUANT_A_PER_TENSOR_SYM 4
+#define WOQ_HIP_QUANT_A_PER_K_BLOCK_SYM 5
+#define WOQ_HIP_QUANT_A_PER_M_SYM 6
+#define WOQ_HIP_QUANT_A_PER_M_K_BLOCK_SYM 7
+
+/* fused post-op, csrc/cpu/aten/utils/woq_defines.h:27-36 */
+#define WOQ_HIP_FUSE_NONE 0x0
+#define WOQ_HIP_FUSE_GELU_ERF 0x1
+#define WOQ_HIP_FUSE_GELU_TANH 0x2
+#define WOQ_HIP_FUSE_RELU 0x3
+#define WOQ_HIP_FUSE_SILU 0x4
+#define WOQ_HIP_FUSE_ADD 0x10
+#define WOQ_HIP_FUSE_ADD_ADD 0x20
+#define WOQ_HIP_FUSE_MUL 0x30
+
+/* element types of activations / outputs */
+#define WOQ_HIP_ACT_FP32 0
+#define WOQ_HIP_ACT_FP16 1
+#define WOQ_HIP_ACT_BF16 2
+
+/* Tile geometry of the packed layouts (see woq_hip_pack_weight). */
+#define WOQ_HIP_TILE_N 16      /* output rows per tile                     */
+#define WOQ_HIP_TILE_BYTES 1024 /* one tile = one dwordx4 load per lane of a wave64 */
+#define WOQ_HIP_TILE_K_INT4 128 /* K values per tile row, 4-bit weights    */
+#define WOQ_HIP_TILE_K_INT8 64  /* K values per tile row, 8-bit weights    */
+
+const char* woq_hip_last_error(void);
+
+/* ABI version; bumped whenever a struct or a layout below changes. */
+int woq_hip_abi_version(void);
+
+/* Padded extents of the packed layout: N up to a multiple of 16, K up to a multiple of
+ * the tile K extent.  packed bytes = Np/16 * Kp/tile_k * 1024. */
+int64_t woq_hip_padded_n(int64_t N);
+int64_t woq_hip_padded_k(int weight_dtype, int64_t K);
+int64_t woq_hip_packed_weight_bytes(int weight_dtype, int64_t N, int64_t K);
+
+/*
+ * Plain -> packed.
+ *   INT4 / NF4: plain is uint8 [N, ceil(K/2)], byte j of a row holds element 2j in the
+ *               low nibble and 2j+1 in the high nibble
+ *               (intel_extension_for_pytorch/quantization/_quantize_utils.py:1184).
+ *   INT8:       plain is int8 [N, K].
+ * Packed layout (the same bytes serve the small-M kernel, the MFMA GEMM and the int8 path):
+ *   tiles [Np/16][Kp/tile_k], 1024 bytes each, K-tiles of one row block contiguous.
+ *   Lane l = r + 16*c of a wave64 owns bytes [16*l, 16*l+16) of a tile: output row
+ *   n0 + r, and
+ *     INT4: K offsets 32*c .. 32*c+31 as 4 dwords; dword j holds offsets 8*j .. 8*j+7 with
+ *           element e stored in nibble position (e even ? e/2 : 4 + e/2), so that
+ *           (dword >> 4*v) & 0x000F000F yields elements (2v, 2v+1) in the two 16-bit halves;
+ *     INT8: K offsets 16*c .. 16*c+15, one per byte, stored offset-binary (value + 128).
+ *   Padding rows / columns hold zero-weight encodings and never contribute.
+ */
+int woq_hip_pack_weight(const void* plain, int weight_dtype, int64_t N, int64_t K,
+                        void* packed, void* stream);
+
+/* Exact inverse of woq_hip_pack_weight (padding dropped). */
+int woq_hip_unpack_weight(const void* packed, int weight_dtype, int64_t N, int64_t K,
+                          void* plain, void* stream);
+
+/*
+ * Quantization parameters -> kernel layout.
+ *   scales: fp32 [N, KG] (KG = number of K groups; 1 for per-channel)
+ *   zeros : fp32 [N, KG] or NULL (symmetric).  Must be integral, in [0,255] for 4-bit and
+ *           [-128,127] for 8-bit weights (checked by the host wrapper).
+ * Outputs are laid out [Np/16][KG][16] (row-in-tile fastest):
+ *   scales_f32 / scales_f16 / scales_bf16: the three roundings the reference keeps
+ *   (ContextLinearWoq.h:104-106); zeros_u8: zero point as one byte, the value itself for
+ *   4-bit weights and value + 128 for 8-bit weights (the same offset-binary shift as the
+ *   weight bytes, so stored_weight - stored_zero == q - z in both cases).
+ * Padding rows get scale 1, zero 0 (LinearWoqPacked.cpp:344-361).
+ */
+int woq_hip_pack_qparams(const float* scales, const float* zeros, int weight_dtype, int64_t N,
+                         int64_t KG, float* scales_f32, void* scales_f16, void* scales_bf16,
+                         uint8_t* zeros_u8, void* stream);
+
+/* zp[i][j] = (zp32[i][j/8] >> (4*(j%8))) & 0xf, written as fp32 [rows, cols]. */
+int woq_hip_unpack_int4_zeros(const int32_t* zp32, int64_t rows, int64_t cols,
+                              int64_t cols_zp32, float* out, void* stream);
+
+/*
+ * Dynamic activation quantization.
+ *   x: [M, K] (x_dtype), q: int8 (symmetric modes 4..7) or uint8 (asymmetric 0..3) [M, K],
+ *   scales: fp32, zps: int32 (asymmetric only, may be NULL for symmetric modes); shapes
+ *   per mode: per-tensor [1], per-K-block [Kc], per-M [M], per-M-K-block [M, Kc] with
+ *   Kc = ceil(K / quant_block_k).
+ *   scale = max(|max|,|min|)/127 (sym) or (max-min)/255 (asym); q = clamp(rint(x/scale + zp)).
+ */
+int woq_hip_dynamic_quant(const void* x, int x_dtype, int64_t M, int64_t K,
+                          int64_t quant_block_k, int act_quant_mode, void* q, float* scales,
+                          int32_t* zps, void* stream);
+
+typedef struct woq_hip_linear_params {
+  uint32_t struct_size; /* sizeof(woq_hip_linear_params), checked */
+
+  /* activations, row-major [M, K], 16-byte aligned rows (K % 8 == 0) */
+  const void* x;
+  int32_t x_dtype; /* WOQ_HIP_ACT_* */
+  int64_t M, K, N;
+
+  /* packed weight + parameters (woq_hip_pack_weight / woq_hip_pack_qparams) */
+  const void* qweight;
+  int32_t weight_dtype; /* WOQ_HIP_DTYPE_* */
+  const float* scales_f32;
+  const void* scales_f16;
+  const void* scales_bf16;
+  const uint8_t* zeros_u8; /* NULL: symmetric weights */
+  int64_t group_size;       /* <= 0: per output channel */
+  const float* bias;        /* fp32 [N] or NULL */
+
+  int32_t lowp_mode;      /* WOQ_HIP_LOWP_* */
+  int32_t act_quant_mode; /* WOQ_HIP_QUANT_A_*, used when lowp_mode == INT8 */
+
+  /* fused post-op; others[i] is [M, N] in x_dtype */
+  int32_t fusion;
+  const void* others[2];
+
+  /* output [M, N]; out_dtype = x_dtype, or WOQ_HIP_ACT_FP32 to receive the fp32
+   * accumulator (bias added, no output rounding, no post-op) for parity checks */
+  void* out;
+  int32_t out_dtype;
+
+  /* workspace for lowp_mode == INT8 (size from woq_hip_linear_workspace_bytes) */
+  void* workspace;
+  int64_t workspace_bytes;
+
+  /* optional, lowp_mode == INT8 only: receives the exact int32 sum of every
+   * (m, n, K-block) as int32 [M, N, Kp/block_k] (tests only, small shapes) */
+  int32_t* debug_block_sums;
+
+  /* force_kernel: 0 = automatic; 1 = small-M streaming kernel; 2 = tiled MFMA GEMM */
+  int32_t force_kernel;
+
+  void* stream;
+} woq_hip_linear_params;
+
+int64_t woq_hip_linear_workspace_bytes(int64_t M, int64_t K, int32_t lowp_mode,
+                                       int32_t act_quant_mode, int64_t group_size);
+
+/* K-block of the int8 path: min(group_size, 128), per-channel -> 128
+ * (get_block_k, csrc/cpu/aten/Linear.cpp:362-376). */
+int64_t woq_hip_int8_block_k(int64_t group_size, int64_t K);
+
+int woq_hip_linear(const woq_hip_linear_params* p);
+
+/* Packed weight -> dense [N, K] in out_dtype (fp32: (q - z) * s exactly; fp16 / bf16: that
+ * value rounded to nearest even).  Used by the weight cache and by tests. */
+int woq_hip_dequant_weight(const void* qweight, int weight_dtype, int64_t N, int64_t K,
+                           const float* scales_f32, const uint8_t* zeros_u8,
+                           int64_t group_size, void* out, int out_dtype, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* WOQ_HIP_H_ */

@@ -1,0 +1,221 @@
+// extern "C" entry points: argument validation, regime / kernel selection, launches.
+#include <stdarg.h>
+#include <stdio.h>
+#include <string.h>
+
+#include "woq_common.h"
+#include "woq_internal.h"
+
+namespace woq {
+
+static thread_local char g_err[512] = "";
+
+int set_error(const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+  return 1;
+}
+
+int check_launch(const char* what) {
+  hipError_t err = hipGetLastError();
+  if (err != hipSuccess) return set_error("%s: %s", what, hipGetErrorString(err));
+  return 0;
+}
+
+static bool valid_wdtype(int d) { return d == WOQ_HIP_DTYPE_INT8 || d == WOQ_HIP_DTYPE_INT4; }
+
+}  // namespace woq
+
+using namespace woq;
+
+extern "C" {
+
+const char* woq_hip_last_error(void) { return g_err; }
+
+int woq_hip_abi_version(void) { return 1; }
+
+int64_t woq_hip_padded_n(int64_t N) { return (N + kTileN - 1) / kTileN * kTileN; }
+
+int64_t woq_hip_padded_k(int weight_dtype, int64_t K) {
+  const int tk = weight_dtype == WOQ_HIP_DTYPE_INT8 ? kTileK8 : kTileK4;
+  return (K + tk - 1) / tk * tk;
+}
+
+int64_t woq_hip_packed_weight_bytes(int weight_dtype, int64_t N, int64_t K) {
+  const int tk = weight_dtype == WOQ_HIP_DTYPE_INT8 ? kTileK8 : kTileK4;
+  return woq_hip_padded_n(N) / kTileN * (woq_hip_padded_k(weight_dtype, K) / tk) * kTileBytes;
+}
+
+int woq_hip_pack_weight(const void* plain, int weight_dtype, int64_t N, int64_t K, void* packed,
+                        void* stream) {
+  if (!valid_wdtype(weight_dtype)) return set_error("pack_weight: unsupported weight dtype %d", weight_dtype);
+  if (N < 0 || K < 0) return set_error("pack_weight: negative shape");
+  if ((N > 0 && K > 0) && (!plain || !packed)) return set_error("pack_weight: null pointer");
+  return launch_pack_weight(plain, weight_dtype, N, K, packed, (hipStream_t)stream);
+}
+
+int woq_hip_unpack_weight(const void* packed, int weight_dtype, int64_t N, int64_t K, void* plain,
+                          void* stream) {
+  if (!valid_wdtype(weight_dtype)) return set_error("unpack_weight: unsupported weight dtype %d", weight_dtype);
+  if (N < 0 || K < 0) return set_error("unpack_weight: negative shape");
+  if ((N > 0 && K > 0) && (!plain || !packed)) return set_error("unpack_weight: null pointer");
+  return launch_unpack_weight(packed, weight_dtype, N, K, plain, (hipStream_t)stream);
+}
+
+int woq_hip_pack_qparams(const float* scales, const float* zeros, int weight_dtype, int64_t N, int64_t KG,
+                         float* scales_f32, void* scales_f16, void* scales_bf16, uint8_t* zeros_u8,
+                         void* stream) {
+  if (!valid_wdtype(weight_dtype)) return set_error("pack_qparams: unsupported weight dtype %d", weight_dtype);
+  if (N < 0 || KG < 1) return set_error("pack_qparams: bad shape N=%lld KG=%lld", (long long)N, (long long)KG);
+  if (N > 0 && (!scales || !scales_f32 || !scales_f16 || !scales_bf16))
+    return set_error("pack_qparams: null scales pointer");
+  if (zeros && !zeros_u8) return set_error("pack_qparams: zeros given but zeros_u8 is null");
+  return launch_pack_qparams(scales, zeros, weight_dtype, N, KG, scales_f32, scales_f16, scales_bf16, zeros_u8,
+                             (hipStream_t)stream);
+}
+
+int woq_hip_unpack_int4_zeros(const int32_t* zp32, int64_t rows, int64_t cols, int64_t cols_zp32, float* out,
+                              void* stream) {
+  if (rows < 0 || cols < 0 || cols_zp32 * 8 < cols)
+    return set_error("unpack_int4_zeros: bad shape rows=%lld cols=%lld cols_zp32=%lld", (long long)rows,
+                     (long long)cols, (long long)cols_zp32);
+  return launch_unpack_int4_zeros(zp32, rows, cols, cols_zp32, out, (hipStream_t)stream);
+}
+
+int woq_hip_dynamic_quant(const void* x, int x_dtype, int64_t M, int64_t K, int64_t quant_block_k,
+                          int act_quant_mode, void* q, float* scales, int32_t* zps, void* stream) {
+  if (act_quant_mode < 0 || act_quant_mode > 7) return set_error("dynamic_quant: bad act_quant_mode %d", act_quant_mode);
+  if (x_dtype < 0 || x_dtype > 2) return set_error("dynamic_quant: bad x_dtype %d", x_dtype);
+  if (K % 8 != 0) return set_error("dynamic_quant: K (%lld) must be a multiple of 8", (long long)K);
+  if (act_quant_mode < 4 && !zps) return set_error("dynamic_quant: asymmetric mode needs a zps buffer");
+  return launch_dynamic_quant(x, x_dtype, M, K, K, quant_block_k, act_quant_mode, q, scales, zps,
+                              (hipStream_t)stream);
+}
+
+int64_t woq_hip_int8_block_k(int64_t group_size, int64_t K) {
+  int64_t bk = group_size > 0 ? (group_size < 128 ? group_size : 128) : 128;
+  while (bk > 0 && K % bk != 0) bk /= 2;
+  return bk;
+}
+
+int64_t woq_hip_linear_workspace_bytes(int64_t M, int64_t K, int32_t lowp_mode, int32_t act_quant_mode,
+                                       int64_t group_size) {
+  if (lowp_mode != WOQ_HIP_LOWP_INT8) return 0;
+  (void)act_quant_mode;
+  const int64_t kp = (K + 127) / 128 * 128;
+  const int64_t qbytes = (M * kp + 255) / 256 * 256;
+  int64_t qbk = group_size > 0 ? group_size : woq_hip_int8_block_k(-1, K);
+  if (qbk <= 0) qbk = 1;
+  const int64_t Kc = (K + qbk - 1) / qbk;
+  return qbytes + (M * Kc + 64) * 8;
+}
+
+int woq_hip_linear(const woq_hip_linear_params* p) {
+  if (!p) return set_error("woq_linear: null params");
+  if (p->struct_size != sizeof(woq_hip_linear_params))
+    return set_error("woq_linear: struct_size %u does not match this library (%zu)", p->struct_size,
+                     sizeof(woq_hip_linear_params));
+  if (!valid_wdtype(p->weight_dtype)) return set_error("woq_linear: unsupported weight dtype %d", p->weight_dtype);
+  if (p->M < 0 || p->K <= 0 || p->N <= 0)
+    return set_error("woq_linear: bad shape M=%lld K=%lld N=%lld", (long long)p->M, (long long)p->K, (long long)p->N);
+  if (p->x_dtype != WOQ_HIP_ACT_BF16 && p->x_dtype != WOQ_HIP_ACT_FP16 && p->x_dtype != WOQ_HIP_ACT_FP32)
+    return set_error("woq_linear: bad x_dtype %d", p->x_dtype);
+  if (p->out_dtype != p->x_dtype && p->out_dtype != WOQ_HIP_ACT_FP32)
+    return set_error("woq_linear: out_dtype must equal x_dtype or be fp32");
+  if (p->lowp_mode < 0 || p->lowp_mode > 3) return set_error("woq_linear: bad lowp_mode %d", p->lowp_mode);
+  if (p->M == 0) return 0;
+  if (!p->x || !p->qweight || !p->out || !p->scales_f32 || !p->scales_f16 || !p->scales_bf16)
+    return set_error("woq_linear: null pointer argument");
+  if (p->group_size > 0 && p->group_size % 32 != 0)
+    return set_error("woq_linear: group_size %lld must be a multiple of 32 (or <= 0 for per-channel)",
+                     (long long)p->group_size);
+  switch (p->fusion) {
+    case WOQ_HIP_FUSE_NONE: case WOQ_HIP_FUSE_GELU_ERF: case WOQ_HIP_FUSE_GELU_TANH:
+    case WOQ_HIP_FUSE_RELU: case WOQ_HIP_FUSE_SILU:
+      break;
+    case WOQ_HIP_FUSE_ADD: case WOQ_HIP_FUSE_MUL:
+      if (!p->others[0]) return set_error("woq_linear: fusion 0x%x needs others[0]", p->fusion);
+      break;
+    case WOQ_HIP_FUSE_ADD_ADD:
+      if (!p->others[0] || !p->others[1]) return set_error("woq_linear: add_add needs two others");
+      break;
+    default:
+      return set_error("woq_linear: unexpected fusion type 0x%x", p->fusion);
+  }
+  if (p->out_dtype == WOQ_HIP_ACT_FP32 && p->x_dtype != WOQ_HIP_ACT_FP32 && p->fusion != WOQ_HIP_FUSE_NONE)
+    return set_error("woq_linear: the fp32 accumulator output does not take a post-op");
+
+  const int wbits = p->weight_dtype == WOQ_HIP_DTYPE_INT8 ? 8 : 4;
+  const int tk = wbits == 4 ? kTileK4 : kTileK8;
+  const int64_t NT = woq_hip_padded_n(p->N) / kTileN;
+  const int64_t KT = woq_hip_padded_k(p->weight_dtype, p->K) / tk;
+  const int64_t Kpad = KT * tk;
+  const int64_t G = p->group_size > 0 ? p->group_size : Kpad;
+  const int64_t KG = p->group_size > 0 ? (p->K + G - 1) / G : 1;
+  hipStream_t st = (hipStream_t)p->stream;
+
+  int lowp = p->lowp_mode;
+  if (lowp == WOQ_HIP_LOWP_INT8) {
+    const int64_t bk = woq_hip_int8_block_k(p->group_size, p->K);
+    const bool blocks_ok = bk == 32 || bk == 64 || bk == 128;
+    const bool mode_ok = p->act_quant_mode >= WOQ_HIP_QUANT_A_PER_TENSOR_SYM &&
+                         p->act_quant_mode <= WOQ_HIP_QUANT_A_PER_M_K_BLOCK_SYM;
+    if (p->weight_dtype == WOQ_HIP_DTYPE_INT8 && p->zeros_u8)
+      return set_error("woq_linear: symmetric quantization is required for INT8 weights with lowp_mode INT8");
+    if (p->x_dtype == WOQ_HIP_ACT_FP32 || !blocks_ok) {
+      // Shapes the blocked int8 kernel does not take run unquantized in the activation dtype,
+      // which is what the reference's fallback does for lowp_mode INT8
+      // (csrc/cpu/aten/kernels/WoqInt8GemmAPerMKrnl.cpp:143-169).
+      lowp = WOQ_HIP_LOWP_NONE;
+    } else if (!mode_ok) {
+      return set_error("woq_linear: act_quant_mode %d is not supported (symmetric modes 4..7 only)",
+                       p->act_quant_mode);
+    } else {
+      Int8Args a;
+      a.x = p->x; a.x_dtype = p->x_dtype; a.M = p->M; a.K = p->K; a.N = p->N; a.NT = NT; a.KT = KT;
+      a.qweight = (const uint8_t*)p->qweight; a.wbits = wbits; a.scales = p->scales_f32;
+      a.zeros = p->zeros_u8; a.G = G; a.KG = KG; a.bias = p->bias; a.act_quant_mode = p->act_quant_mode;
+      a.fusion = p->fusion; a.other0 = p->others[0]; a.other1 = p->others[1]; a.out = p->out;
+      a.out_dtype = p->out_dtype; a.workspace = p->workspace; a.workspace_bytes = p->workspace_bytes;
+      a.debug_block_sums = p->debug_block_sums;
+      return launch_int8_linear(a, st);
+    }
+  }
+
+  // Floating-point regimes (csrc/cpu/aten/kernels/WoqLinearKrnl.cpp:75-112; the small-batch
+  // threshold 5 is IPEX_WOQ_SMALL_BATCH_THRESHOLD, csrc/cpu/aten/utils/woq.h:24).
+  int regime;
+  if (lowp == WOQ_HIP_LOWP_FP16 || (lowp == WOQ_HIP_LOWP_NONE && p->x_dtype == WOQ_HIP_ACT_FP16) ||
+      (lowp == WOQ_HIP_LOWP_BF16 && p->M < 5)) {
+    regime = kRegimeF16;
+  } else if ((lowp == WOQ_HIP_LOWP_NONE && p->x_dtype == WOQ_HIP_ACT_BF16) || lowp == WOQ_HIP_LOWP_BF16) {
+    regime = kRegimeBF16;
+  } else {
+    return set_error("woq_linear: fp32 compute (lowp_mode NONE with fp32 activations) is not supported");
+  }
+
+  FpArgs f;
+  f.x = p->x; f.x_dtype = p->x_dtype; f.M = p->M; f.K = p->K; f.N = p->N; f.NT = NT; f.KT = KT;
+  f.qweight = (const uint8_t*)p->qweight;
+  f.scales = (const uint16_t*)(regime == kRegimeF16 ? p->scales_f16 : p->scales_bf16);
+  f.zeros = p->zeros_u8; f.G = G; f.KG = KG; f.bias = p->bias; f.fusion = p->fusion;
+  f.other0 = p->others[0]; f.other1 = p->others[1]; f.out = p->out; f.out_dtype = p->out_dtype;
+
+  int kernel = p->force_kernel;
+  if (kernel == 0) kernel = p->M <= 64 ? 1 : 2;
+  if (kernel == 1 && p->M > 64) return set_error("woq_linear: the small-M kernel takes M <= 64");
+  return kernel == 1 ? launch_small_m(f, wbits, regime, st) : launch_gemm(f, wbits, regime, st);
+}
+
+int woq_hip_dequant_weight(const void* qweight, int weight_dtype, int64_t N, int64_t K, const float* scales_f32,
+                           const uint8_t* zeros_u8, int64_t group_size, void* out, int out_dtype, void* stream) {
+  if (!valid_wdtype(weight_dtype)) return set_error("dequant_weight: unsupported weight dtype %d", weight_dtype);
+  if (out_dtype < 0 || out_dtype > 2) return set_error("dequant_weight: bad out_dtype %d", out_dtype);
+  if (N > 0 && K > 0 && (!qweight || !scales_f32 || !out)) return set_error("dequant_weight: null pointer");
+  return launch_dequant_weight(qweight, weight_dtype, N, K, scales_f32, zeros_u8, group_size, out, out_dtype,
+                               (hipStream_t)stream);
+}
+
+}  // extern "C"

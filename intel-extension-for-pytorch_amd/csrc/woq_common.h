@@ -1,0 +1,222 @@
+// Shared device helpers for the gfx950 WOQ linear kernels: vector types, the packed
+// tile geometry, nibble decoding and the rounding helpers every kernel uses.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/woq_hip.h"
+
+namespace woq {
+
+typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+typedef _Float16 h8 __attribute__((ext_vector_type(8)));
+typedef __bf16 b2 __attribute__((ext_vector_type(2)));
+typedef __bf16 b8 __attribute__((ext_vector_type(8)));
+typedef float f2 __attribute__((ext_vector_type(2)));
+typedef float f4 __attribute__((ext_vector_type(4)));
+typedef float f16v __attribute__((ext_vector_type(16)));
+typedef int i4 __attribute__((ext_vector_type(4)));
+typedef int i16v __attribute__((ext_vector_type(16)));
+typedef unsigned u2 __attribute__((ext_vector_type(2)));
+typedef unsigned u4 __attribute__((ext_vector_type(4)));
+
+constexpr int kTileN = WOQ_HIP_TILE_N;
+constexpr int kTileBytes = WOQ_HIP_TILE_BYTES;
+constexpr int kTileK4 = WOQ_HIP_TILE_K_INT4;
+constexpr int kTileK8 = WOQ_HIP_TILE_K_INT8;
+
+// Compute regimes of the floating-point kernels.  The reference picks fp16 for
+// lowp_mode FP16, for NONE with half activations and for BF16 with M < 5, and bf16 for
+// NONE with bf16 activations and for BF16 with M >= 5
+// (csrc/cpu/aten/kernels/WoqLinearKrnl.cpp:75-112).
+enum Regime { kRegimeF16 = 0, kRegimeBF16 = 1 };
+
+template <typename T, typename U>
+__device__ __forceinline__ T bitcast(U u) {
+  static_assert(sizeof(T) == sizeof(U), "size mismatch");
+  return __builtin_bit_cast(T, u);
+}
+
+__device__ __forceinline__ float bf16_bits_to_f32(uint16_t b) {
+  return bitcast<float>((uint32_t)b << 16);
+}
+
+// fp32 -> bf16, round to nearest even (NaN kept quiet); v_cvt_pk_bf16_f32 on gfx950.
+__device__ __forceinline__ uint16_t f32_to_bf16_bits(float f) {
+  __bf16 b = (__bf16)f;
+  return bitcast<uint16_t>(b);
+}
+
+__device__ __forceinline__ uint16_t f32_to_f16_bits(float f) {
+  _Float16 h = (_Float16)f;
+  return bitcast<uint16_t>(h);
+}
+
+__device__ __forceinline__ float f16_bits_to_f32(uint16_t b) {
+  return (float)bitcast<_Float16>(b);
+}
+
+// Nibble position of K-element e (0..7) inside one dword of the packed INT4 layout.
+__host__ __device__ __forceinline__ constexpr int nibble_pos(int e) {
+  return (e & 1) ? 4 + (e >> 1) : (e >> 1);
+}
+
+// ---- 4-bit decode -------------------------------------------------------------------
+// (d >> 4v) & 0x000F000F | 0x6400_6400 is the fp16 pair (1024 + q[2v], 1024 + q[2v+1]).
+__device__ __forceinline__ h2 nib_pair_f16(uint32_t d, int v, uint32_t mask, uint32_t magic) {
+  return bitcast<h2>(((d >> (4 * v)) & mask) | magic);
+}
+
+// fp16 regime: w = fp16((q - z) * s).  nz = -(1024 + z) (exact in fp16 for integral z < 1024),
+// so the add is exact and the product is rounded once, which is fp16((q - z) * s) whenever s
+// is an fp16 value (csrc/cpu/aten/utils/woq_utils.h:79-163 followed by .to(half),
+// csrc/cpu/aten/utils/woq.h:3565-3567).
+__device__ __forceinline__ h8 dequant8_f16(uint32_t d, h2 nz, h2 s2) {
+  const uint32_t mask = 0x000F000Fu, magic = 0x64006400u;
+  h8 r;
+#pragma unroll
+  for (int v = 0; v < 4; ++v) {
+    h2 h = nib_pair_f16(d, v, mask, magic);
+    h = (h + nz) * s2;
+    r[2 * v] = h[0];
+    r[2 * v + 1] = h[1];
+  }
+  return r;
+}
+
+// bf16 regime: w = bf16((q - z) * s) with s a bf16 value held in fp32.  c = -(1024 + z) * s is
+// exact in fp32 (11 bits x 8 bits), and fma(1024 + q, s, c) has the exactly representable
+// value (q - z) * s, so the only rounding is the final RNE to bf16
+// (csrc/cpu/aten/utils/woq.h:1495-1581: separate sub and mul in fp32, then store as bf16).
+__device__ __forceinline__ b8 dequant8_bf16(uint32_t d, float s, float c) {
+  const uint32_t mask = 0x000F000Fu, magic = 0x64006400u;
+  b8 r;
+#pragma unroll
+  for (int v = 0; v < 4; ++v) {
+    h2 h = nib_pair_f16(d, v, mask, magic);
+    f2 f;
+    f[0] = __builtin_fmaf((float)h[0], s, c);
+    f[1] = __builtin_fmaf((float)h[1], s, c);
+    b2 b = __builtin_convertvector(f, b2);
+    r[2 * v] = b[0];
+    r[2 * v + 1] = b[1];
+  }
+  return r;
+}
+
+// ---- 8-bit decode (bytes are offset-binary: stored = q + 128) ---------------------------
+// 8 consecutive K elements live in two dwords.
+__device__ __forceinline__ h8 dequant8_f16_w8(uint32_t d0, uint32_t d1, float s, float c) {
+  // w = fp16((u - uz) * s), computed as fma(u, s, -uz * s) in fp32 (exact for fp16/bf16-valued
+  // scales: 8 bits x 11 bits) and rounded once to fp16.
+  h8 r;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    r[i] = (_Float16)__builtin_fmaf((float)((d0 >> (8 * i)) & 0xFFu), s, c);
+    r[4 + i] = (_Float16)__builtin_fmaf((float)((d1 >> (8 * i)) & 0xFFu), s, c);
+  }
+  return r;
+}
+
+__device__ __forceinline__ b8 dequant8_bf16_w8(uint32_t d0, uint32_t d1, float s, float c) {
+  b8 r;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    r[i] = (__bf16)__builtin_fmaf((float)((d0 >> (8 * i)) & 0xFFu), s, c);
+    r[4 + i] = (__bf16)__builtin_fmaf((float)((d1 >> (8 * i)) & 0xFFu), s, c);
+  }
+  return r;
+}
+
+// Output rounding of one accumulator.
+//   fp16 regime: the reference GEMM result is an fp16 tensor, the fp16 bias is added in
+//   fp16, and the result is cast to the activation dtype
+//   (csrc/cpu/aten/utils/woq.h:3569-3576, 3612).
+//   bf16 regime: fp32 accumulator initialised with the fp32 bias, one rounding to the
+//   output dtype (csrc/cpu/aten/utils/woq.h:3298-3310, 3452).
+template <int REGIME>
+__device__ __forceinline__ float finalize_acc(float acc, bool has_bias, float bias) {
+  if (REGIME == kRegimeF16) {
+    _Float16 h = (_Float16)acc;
+    if (has_bias) h = (_Float16)((float)h + (float)(_Float16)bias);
+    return (float)h;
+  } else {
+    return has_bias ? acc + bias : acc;
+  }
+}
+
+__device__ __forceinline__ float gelu_erf(float x) {
+  return 0.5f * x * (1.0f + erff(x * 0.70710678118654752440f));
+}
+__device__ __forceinline__ float gelu_tanh(float x) {
+  const float k0 = 0.7978845608028654f, k1 = 0.044715f;
+  return 0.5f * x * (1.0f + tanhf(k0 * (x + k1 * x * x * x)));
+}
+__device__ __forceinline__ float silu(float x) { return x / (1.0f + __expf(-x)); }
+
+__device__ __forceinline__ float load_act(const void* p, int dtype, int64_t i) {
+  if (dtype == WOQ_HIP_ACT_BF16) return bf16_bits_to_f32(((const uint16_t*)p)[i]);
+  if (dtype == WOQ_HIP_ACT_FP16) return f16_bits_to_f32(((const uint16_t*)p)[i]);
+  return ((const float*)p)[i];
+}
+
+// Round v to the activation dtype and return it as fp32 (the reference applies post-ops on
+// the output-dtype tile, csrc/cpu/aten/utils/woq.h:2924-2967).
+__device__ __forceinline__ float round_to_act(float v, int dtype) {
+  if (dtype == WOQ_HIP_ACT_BF16) return bf16_bits_to_f32(f32_to_bf16_bits(v));
+  if (dtype == WOQ_HIP_ACT_FP16) return f16_bits_to_f32(f32_to_f16_bits(v));
+  return v;
+}
+
+__device__ __forceinline__ void store_act(void* p, int dtype, int64_t i, float v) {
+  if (dtype == WOQ_HIP_ACT_BF16)
+    ((uint16_t*)p)[i] = f32_to_bf16_bits(v);
+  else if (dtype == WOQ_HIP_ACT_FP16)
+    ((uint16_t*)p)[i] = f32_to_f16_bits(v);
+  else
+    ((float*)p)[i] = v;
+}
+
+// Epilogue shared by every kernel: bias + regime rounding, optional post-op, store.
+struct Epilogue {
+  const float* bias;
+  int fusion;
+  const void* other0;
+  const void* other1;
+  void* out;
+  int out_dtype;  // WOQ_HIP_ACT_*; fp32 means "raw accumulator + bias"
+  int act_dtype;  // dtype post-ops round through
+  int64_t N;      // logical N (row stride of out / others)
+};
+
+template <int REGIME>
+__device__ __forceinline__ void epilogue_store(const Epilogue& e, int64_t m, int64_t n, float acc) {
+  const bool hb = e.bias != nullptr;
+  const float b = hb ? e.bias[n] : 0.0f;
+  const int64_t idx = m * e.N + n;
+  if (e.out_dtype == WOQ_HIP_ACT_FP32 && e.act_dtype != WOQ_HIP_ACT_FP32) {
+    ((float*)e.out)[idx] = hb ? acc + b : acc;
+    return;
+  }
+  float y = finalize_acc<REGIME>(acc, hb, b);
+  if (e.fusion != WOQ_HIP_FUSE_NONE) {
+    y = round_to_act(y, e.act_dtype);
+    switch (e.fusion) {
+      case WOQ_HIP_FUSE_GELU_ERF: y = gelu_erf(y); break;
+      case WOQ_HIP_FUSE_GELU_TANH: y = gelu_tanh(y); break;
+      case WOQ_HIP_FUSE_RELU: y = y > 0.0f ? y : 0.0f; break;
+      case WOQ_HIP_FUSE_SILU: y = silu(y); break;
+      case WOQ_HIP_FUSE_ADD: y = y + load_act(e.other0, e.act_dtype, idx); break;
+      case WOQ_HIP_FUSE_ADD_ADD:
+        y = round_to_act(y + load_act(e.other0, e.act_dtype, idx), e.act_dtype);
+        y = y + load_act(e.other1, e.act_dtype, idx);
+        break;
+      case WOQ_HIP_FUSE_MUL: y = y * load_act(e.other0, e.act_dtype, idx); break;
+      default: break;
+    }
+  }
+  store_act(e.out, e.out_dtype, idx, y);
+}
+
+}  // namespace woq

@@ -1,0 +1,569 @@
+// lowp_mode = INT8: dynamic activation quantization and int8 x int8 -> int32 MFMA kernels.
+//
+// Reference counterparts:
+//   dynamic_quantize_per_block (csrc/cpu/aten/utils/woq_dynamic_quant.h:1526-1750)
+//   Dequantize<int8_t> + BrgemmTPP<int8,int32> + fp32 epilogue (csrc/cpu/aten/utils/woq.h:1664-1734,
+//   2133-2199), small-M VNNI micro-kernel (woq.h:953-1127).
+//
+// Arithmetic contract (bit-exact parts): q_a = clamp(rint(x / s_a + zp_a)), B = q_w - z_w as int8,
+// qC[m, n, kb] = sum over the K block kb of q_a * B in int32.  Float epilogue, blocks in ascending
+// K order inside a wave: C += (float(qC) * s_a) * s_w  (woq.h:2172-2186, unfused mul, mul, add).
+#include "woq_common.h"
+#include "woq_internal.h"
+
+namespace woq {
+
+__host__ __device__ inline bool quant_a_is_sym(int mode) { return mode >= WOQ_HIP_QUANT_A_PER_TENSOR_SYM; }
+__host__ __device__ inline bool quant_a_per_m(int mode) {
+  return mode == WOQ_HIP_QUANT_A_PER_M || mode == WOQ_HIP_QUANT_A_PER_M_K_BLOCK ||
+         mode == WOQ_HIP_QUANT_A_PER_M_SYM || mode == WOQ_HIP_QUANT_A_PER_M_K_BLOCK_SYM;
+}
+__host__ __device__ inline bool quant_a_per_k(int mode) {
+  return mode == WOQ_HIP_QUANT_A_PER_K_BLOCK || mode == WOQ_HIP_QUANT_A_PER_M_K_BLOCK ||
+         mode == WOQ_HIP_QUANT_A_PER_K_BLOCK_SYM || mode == WOQ_HIP_QUANT_A_PER_M_K_BLOCK_SYM;
+}
+
+// ---- statistics: one workgroup per quantization group -------------------------------------
+// group id -> (row range, k range); writes scale (and zero point for asymmetric modes).
+__global__ __launch_bounds__(256) void act_stats_kernel(const void* __restrict__ x, int x_dtype, int64_t M,
+                                                        int64_t K, int64_t qbk, int64_t Kc, int mode,
+                                                        float* __restrict__ scales, int32_t* __restrict__ zps) {
+  const int64_t gid = blockIdx.x;
+  const bool per_m = quant_a_per_m(mode), per_k = quant_a_per_k(mode);
+  int64_t m_lo = 0, m_hi = M, k_lo = 0, k_hi = K;
+  if (per_m && per_k) {
+    m_lo = gid / Kc;
+    m_hi = m_lo + 1;
+    k_lo = (gid % Kc) * qbk;
+    k_hi = k_lo + qbk < K ? k_lo + qbk : K;
+  } else if (per_m) {
+    m_lo = gid;
+    m_hi = gid + 1;
+  } else if (per_k) {
+    k_lo = gid * qbk;
+    k_hi = k_lo + qbk < K ? k_lo + qbk : K;
+  }
+  const int64_t kw = k_hi - k_lo;
+  const int64_t total = (m_hi - m_lo) * kw;
+  float mn = __builtin_inff(), mx = -__builtin_inff();
+  for (int64_t i = threadIdx.x; i < total; i += blockDim.x) {
+    const int64_t m = m_lo + i / kw, k = k_lo + i % kw;
+    const float v = load_act(x, x_dtype, m * K + k);
+    mn = fminf(mn, v);
+    mx = fmaxf(mx, v);
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+    mn = fminf(mn, __shfl_xor(mn, off));
+    mx = fmaxf(mx, __shfl_xor(mx, off));
+  }
+  __shared__ float smn[4], smx[4];
+  const int wave = threadIdx.x >> 6;
+  if ((threadIdx.x & 63) == 0) {
+    smn[wave] = mn;
+    smx[wave] = mx;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int w = 1; w < (int)(blockDim.x >> 6); ++w) {
+      mn = fminf(mn, smn[w]);
+      mx = fmaxf(mx, smx[w]);
+    }
+    if (quant_a_is_sym(mode)) {
+      scales[gid] = __fdiv_rn(fmaxf(fabsf(mx), fabsf(mn)), 127.0f);
+    } else {
+      const float s = __fdiv_rn(__fsub_rn(mx, mn), 255.0f);
+      scales[gid] = s;
+      zps[gid] = (int32_t)(-rintf(__fdiv_rn(mn, s)));
+    }
+  }
+}
+
+// ---- quantize: one thread per 8 consecutive K elements -------------------------------------
+// ldq: row stride of q in bytes (>= K, the tail is zero-filled up to ldq).
+// permute: store each group of 8 as [e0 e4 e1 e5 e2 e6 e3 e7], the byte order the 4-bit decode
+// produces, so the int8 kernels can use the activations without a shuffle.
+__global__ void act_quant_kernel(const void* __restrict__ x, int x_dtype, int64_t M, int64_t K, int64_t ldq,
+                                 int64_t qbk, int64_t Kc, int mode, const float* __restrict__ scales,
+                                 const int32_t* __restrict__ zps, uint8_t* __restrict__ q, int permute) {
+  const int64_t g8 = ldq / 8;
+  const int64_t gid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (gid >= M * g8) return;
+  const int64_t m = gid / g8, k0 = (gid % g8) * 8;
+  const bool per_m = quant_a_per_m(mode), per_k = quant_a_per_k(mode), sym = quant_a_is_sym(mode);
+  uint8_t o[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    const int64_t k = k0 + e;
+    uint8_t b = 0;
+    if (k < K) {
+      const int64_t gi = (per_m ? m * (per_k ? Kc : 1) : 0) + (per_k ? k / qbk : 0);
+      const float s = scales[gi];
+      const float zp = sym ? 0.0f : (float)zps[gi];
+      const float v = load_act(x, x_dtype, m * K + k);
+      float t = __fadd_rn(__fdiv_rn(v, s), zp);
+      t = rintf(t);
+      const float lo = sym ? -128.0f : 0.0f, hi = sym ? 127.0f : 255.0f;
+      t = fminf(fmaxf(t, lo), hi);
+      if (s == 0.0f || t != t) t = sym ? 0.0f : zp;  // all-zero group: the reference divides 0 by 0
+      b = sym ? (uint8_t)(int8_t)(int)t : (uint8_t)(int)t;
+    }
+    o[e] = b;
+  }
+  uint32_t d0, d1;
+  if (permute) {
+    d0 = o[0] | (o[4] << 8) | (o[1] << 16) | ((uint32_t)o[5] << 24);
+    d1 = o[2] | (o[6] << 8) | (o[3] << 16) | ((uint32_t)o[7] << 24);
+  } else {
+    d0 = o[0] | (o[1] << 8) | (o[2] << 16) | ((uint32_t)o[3] << 24);
+    d1 = o[4] | (o[5] << 8) | (o[6] << 16) | ((uint32_t)o[7] << 24);
+  }
+  *(u2*)(q + m * ldq + k0) = u2{d0, d1};
+}
+
+static int64_t num_quant_groups(int64_t M, int64_t Kc, int mode) {
+  const bool per_m = quant_a_per_m(mode), per_k = quant_a_per_k(mode);
+  return (per_m ? M : 1) * (per_k ? Kc : 1);
+}
+
+static int launch_quant_impl(const void* x, int x_dtype, int64_t M, int64_t K, int64_t ldq, int64_t qbk,
+                             int mode, void* q, float* scales, int32_t* zps, int permute, hipStream_t st) {
+  if (M == 0 || K == 0) return 0;
+  if (qbk <= 0) qbk = K;
+  const int64_t Kc = (K + qbk - 1) / qbk;
+  const int64_t groups = num_quant_groups(M, Kc, mode);
+  act_stats_kernel<<<(unsigned)groups, 256, 0, st>>>(x, x_dtype, M, K, qbk, Kc, mode, scales, zps);
+  if (int rc = check_launch("act_stats_kernel")) return rc;
+  const int64_t total = M * (ldq / 8);
+  act_quant_kernel<<<(unsigned)((total + 255) / 256), 256, 0, st>>>(x, x_dtype, M, K, ldq, qbk, Kc, mode,
+                                                                    scales, zps, (uint8_t*)q, permute);
+  return check_launch("act_quant_kernel");
+}
+
+int launch_dynamic_quant(const void* x, int x_dtype, int64_t M, int64_t K, int64_t ldq, int64_t qbk, int mode,
+                         void* q, float* scales, int32_t* zps, hipStream_t st) {
+  return launch_quant_impl(x, x_dtype, M, K, ldq, qbk, mode, q, scales, zps, 0, st);
+}
+
+// ---- weight nibbles / bytes -> int8 (q - z) --------------------------------------------------
+// Four bytes at once: ((b | 0x80808080) - z * 0x01010101) ^ 0x80808080 never borrows across bytes
+// for |q - z| < 128 and leaves q - z in two's complement.
+__device__ __forceinline__ uint32_t sub_bytes(uint32_t b, uint32_t z4) {
+  return ((b | 0x80808080u) - z4) ^ 0x80808080u;
+}
+
+// 16 K elements of one lane for one 16x16x64 MFMA, from two packed dwords (4-bit) or four
+// dwords (8-bit); 4-bit yields the permuted order [e0 e4 e1 e5][e2 e6 e3 e7].
+template <int WBITS>
+__device__ __forceinline__ i4 decode16_i8(const uint32_t* d, uint32_t z4) {
+  i4 r;
+  if (WBITS == 4) {
+    r[0] = (int)sub_bytes(d[0] & 0x0F0F0F0Fu, z4);
+    r[1] = (int)sub_bytes((d[0] >> 4) & 0x0F0F0F0Fu, z4);
+    r[2] = (int)sub_bytes(d[1] & 0x0F0F0F0Fu, z4);
+    r[3] = (int)sub_bytes((d[1] >> 4) & 0x0F0F0F0Fu, z4);
+  } else {
+    // offset-binary bytes u = q + 128 and zero uz = z + 128: (u - uz) needs 9 bits when both are
+    // extreme; the reference restricts 8-bit weights to symmetric (z = 0) in this mode
+    // (csrc/cpu/aten/kernels/WoqInt8GemmAPerMKrnl.cpp:69-73), where it is exact.
+#pragma unroll
+    for (int i = 0; i < 4; ++i) r[i] = (int)(d[i] ^ 0x80808080u);
+  }
+  return r;
+}
+
+struct Int8KArgs {
+  Int8Args a;
+  const uint8_t* xq;   // [M][ldq]
+  int64_t ldq;
+  const float* sa;     // activation scales
+  int64_t sa_m_stride, sa_k_stride, qbk;
+  int64_t block_k;     // K block of the int32 accumulation
+  int W;
+  int64_t Kpad;
+};
+
+// Small-M int8 kernel; same work decomposition as the floating-point small-M kernel.
+template <int WBITS, int MT, int KPW, int NTW>
+__global__ __launch_bounds__(1024) void woq_small_m_i8_kernel(const Int8KArgs p) {
+  constexpr int TK = WBITS == 4 ? kTileK4 : kTileK8;
+  constexpr int STEPS = WBITS == 4 ? 2 : 1;  // 16x16x64 MFMAs per tile
+  constexpr int CK = TK / 4;
+  extern __shared__ __align__(16) uint8_t smem[];
+  const Int8Args& a = p.a;
+  const int W = p.W;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int r = lane & 15, c = lane >> 4;
+  const int64_t nt0 = (int64_t)blockIdx.x * NTW;
+  const int64_t KC = (int64_t)W * KPW * TK;
+  f4* red = (f4*)smem;
+
+  f4 acc[NTW][MT];
+#pragma unroll
+  for (int t = 0; t < NTW; ++t)
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) acc[t][mt] = f4{0.f, 0.f, 0.f, 0.f};
+
+  // blocks per tile (block_k <= TK) or tiles per block (block_k > TK, 8-bit only: 128 / 64)
+  const int bpt = p.block_k <= TK ? (int)(TK / p.block_k) : 1;
+
+  for (int64_t kc0 = 0; kc0 < p.Kpad; kc0 += KC) {
+    const int64_t ktw = kc0 / TK + (int64_t)wave * KPW;
+    u4 wreg[NTW][KPW];
+    uint8_t zreg[NTW][KPW];
+#pragma unroll
+    for (int t = 0; t < NTW; ++t) {
+      const int64_t nt = nt0 + t;
+#pragma unroll
+      for (int i = 0; i < KPW; ++i) {
+        const int64_t kt = ktw + i;
+        wreg[t][i] = WBITS == 4 ? u4{0u, 0u, 0u, 0u} : u4{0x80808080u, 0x80808080u, 0x80808080u, 0x80808080u};
+        zreg[t][i] = WBITS == 4 ? 0 : 128;
+        if (nt < a.NT && kt < a.KT) {
+          wreg[t][i] = __builtin_nontemporal_load((const u4*)(a.qweight + ((nt * a.KT + kt) * 64 + lane) * 16));
+          if (a.zeros) {
+            int64_t g = (kt * TK + c * CK) / a.G;
+            if (g >= a.KG) g = a.KG - 1;
+            zreg[t][i] = a.zeros[(nt * a.KG + g) * kTileN + r];
+          } else {
+            zreg[t][i] = WBITS == 4 ? 8 : 128;
+          }
+        }
+      }
+    }
+    i4 xb[KPW][STEPS][MT];
+#pragma unroll
+    for (int i = 0; i < KPW; ++i)
+#pragma unroll
+      for (int j = 0; j < STEPS; ++j) {
+        const int64_t k = (ktw + i) * TK + c * CK + j * 16;
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+          const int64_t row = mt * 16 + r;
+          i4 v = i4{0, 0, 0, 0};
+          if (row < a.M && k < p.ldq) v = *(const i4*)(p.xq + row * p.ldq + k);
+          xb[i][j][mt] = v;
+        }
+      }
+
+#pragma unroll
+    for (int t = 0; t < NTW; ++t) {
+      const int64_t nt = nt0 + t;
+      i4 qc[MT];
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) qc[mt] = i4{0, 0, 0, 0};
+#pragma unroll
+      for (int i = 0; i < KPW; ++i) {
+        const int64_t kt = ktw + i;
+        const uint32_t z4 = (uint32_t)zreg[t][i] * 0x01010101u;
+#pragma unroll
+        for (int j = 0; j < STEPS; ++j) {
+          const uint32_t* d = (const uint32_t*)&wreg[t][i] + (WBITS == 4 ? 2 * j : 0);
+          const i4 aop = decode16_i8<WBITS>(d, z4);
+#pragma unroll
+          for (int mt = 0; mt < MT; ++mt)
+            qc[mt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(aop, xb[i][j][mt], qc[mt], 0, 0, 0);
+          // a K block ends here when the K extent accumulated so far is a multiple of block_k
+          const int64_t kend = kt * TK + (WBITS == 4 ? (j + 1) * 64 : 64);
+          const bool flush = (kend % p.block_k) == 0 || (i == KPW - 1 && j == STEPS - 1);
+          if (flush) {
+            const int64_t kb = (kend - 1) / p.block_k;          // block index
+            const int64_t kq = kb * p.block_k;                   // first k of the block
+            int64_t g = kq / a.G;
+            if (g >= a.KG) g = a.KG - 1;
+            const bool live = nt < a.NT && kt < a.KT;
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) {
+              const int64_t m = mt * 16 + (lane & 15);
+              const float sa = (m < a.M && live) ? p.sa[m * p.sa_m_stride + (kq / p.qbk) * p.sa_k_stride] : 0.0f;
+#pragma unroll
+              for (int e = 0; e < 4; ++e) {
+                const int64_t n = nt * kTileN + 4 * (lane >> 4) + e;
+                const float sw = live ? a.scales[(nt * a.KG + g) * kTileN + 4 * (lane >> 4) + e] : 0.0f;
+                const float cterm = __fmul_rn(__fmul_rn((float)qc[mt][e], sa), sw);
+                acc[t][mt][e] = __fadd_rn(acc[t][mt][e], cterm);
+                if (a.debug_block_sums && live && m < a.M && n < a.N)
+                  a.debug_block_sums[(m * a.N + n) * (p.Kpad / p.block_k) + kb] = qc[mt][e];
+              }
+              qc[mt] = i4{0, 0, 0, 0};
+            }
+          }
+        }
+      }
+    }
+  }
+  (void)bpt;
+
+#pragma unroll
+  for (int t = 0; t < NTW; ++t)
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) red[((t * MT + mt) * W + wave) * 64 + lane] = acc[t][mt];
+  __syncthreads();
+
+  Epilogue e{a.bias, a.fusion, a.other0, a.other1, a.out, a.out_dtype, a.x_dtype, a.N};
+  for (int idx = threadIdx.x; idx < NTW * MT * 64; idx += blockDim.x) {
+    const int ln = idx & 63, tm = idx >> 6;
+    const int t = tm / MT, mt = tm % MT;
+    f4 s = red[(tm * W) * 64 + ln];
+    for (int w = 1; w < W; ++w) {
+      const f4 v = red[(tm * W + w) * 64 + ln];
+      s[0] = __fadd_rn(s[0], v[0]);
+      s[1] = __fadd_rn(s[1], v[1]);
+      s[2] = __fadd_rn(s[2], v[2]);
+      s[3] = __fadd_rn(s[3], v[3]);
+    }
+    const int64_t m = mt * 16 + (ln & 15);
+    const int64_t n = (nt0 + t) * kTileN + 4 * (ln >> 4);
+    if (m < a.M) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        if (n + i < a.N) epilogue_store<kRegimeBF16>(e, m, n + i, s[i]);
+    }
+  }
+}
+
+// ---- tiled int8 GEMM for large M -------------------------------------------------------------
+// 128 x 128 output tile, K step 128 bytes, 4 waves (2 x 2), v_mfma_i32_32x32x32_i8.
+constexpr int IBM = 128, IBN = 128, IBK = 128;
+constexpr int ILDS = IBK + 16;
+
+template <int WBITS>
+__global__ __launch_bounds__(256) void woq_gemm_i8_kernel(const Int8KArgs p) {
+  constexpr int TK = WBITS == 4 ? kTileK4 : kTileK8;
+  const Int8Args& a = p.a;
+  __shared__ __align__(16) uint8_t sA[IBM * ILDS];
+  __shared__ __align__(16) uint8_t sB[IBN * ILDS];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+  const int64_t m0 = (int64_t)blockIdx.y * IBM, n0 = (int64_t)blockIdx.x * IBN;
+  const int64_t nt0 = n0 / kTileN;
+
+  f16v acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
+
+  const int sub_blocks = (int)(IBK / p.block_k);  // block_k in {32, 64, 128}
+
+  for (int64_t k0 = 0; k0 < p.Kpad; k0 += IBK) {
+    // activations: 128 rows x 128 bytes = 1024 x 16 B -> 4 per thread
+    u4 xa[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int row = (tid >> 3) + 32 * i;
+      const int64_t m = m0 + row, k = k0 + (tid & 7) * 16;
+      xa[i] = u4{0u, 0u, 0u, 0u};
+      if (m < a.M && k < p.ldq) xa[i] = *(const u4*)(p.xq + m * p.ldq + k);
+    }
+    // weights: 8 row blocks x 128 K.  4-bit: one tile per row block -> 512 lane slots;
+    // 8-bit: two tiles per row block -> 1024 lane slots.
+    constexpr int WL = WBITS == 4 ? 2 : 4;
+    u4 wo[WL][WBITS == 4 ? 2 : 1];
+    int wrow[WL], wcol[WL];
+#pragma unroll
+    for (int q = 0; q < WL; ++q) {
+      const int slot = tid + 256 * q;
+      int ntl, li, kt_off;
+      if (WBITS == 4) {
+        ntl = slot >> 6;
+        li = slot & 63;
+        kt_off = 0;
+      } else {
+        ntl = slot >> 7;
+        kt_off = (slot >> 6) & 1;
+        li = slot & 63;
+      }
+      const int r = li & 15, c = li >> 4;
+      wrow[q] = ntl * 16 + r;
+      wcol[q] = WBITS == 4 ? c * 32 : kt_off * 64 + c * 16;
+      const int64_t nt = nt0 + ntl, kt = k0 / TK + kt_off;
+      u4 wv = WBITS == 4 ? u4{0u, 0u, 0u, 0u} : u4{0x80808080u, 0x80808080u, 0x80808080u, 0x80808080u};
+      uint32_t z = WBITS == 4 ? 8u : 128u;
+      if (nt < a.NT && kt < a.KT) {
+        wv = *(const u4*)(a.qweight + ((nt * a.KT + kt) * 64 + li) * 16);
+        if (a.zeros) {
+          int64_t g = (kt * TK + c * (TK / 4)) / a.G;
+          if (g >= a.KG) g = a.KG - 1;
+          z = a.zeros[(nt * a.KG + g) * kTileN + r];
+        }
+      } else if (WBITS == 4) {
+        z = 0;
+      }
+      const uint32_t z4 = z * 0x01010101u;
+      if (WBITS == 4) {
+        const i4 lo = decode16_i8<4>((const uint32_t*)&wv, z4);
+        const i4 hi = decode16_i8<4>((const uint32_t*)&wv + 2, z4);
+        wo[q][0] = bitcast<u4>(lo);
+        wo[q][WBITS == 4 ? 1 : 0] = bitcast<u4>(hi);
+      } else {
+        wo[q][0] = bitcast<u4>(decode16_i8<8>((const uint32_t*)&wv, z4));
+      }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int row = (tid >> 3) + 32 * i;
+      *(u4*)(sA + row * ILDS + (tid & 7) * 16) = xa[i];
+    }
+#pragma unroll
+    for (int q = 0; q < WL; ++q) {
+      *(u4*)(sB + wrow[q] * ILDS + wcol[q]) = wo[q][0];
+      if (WBITS == 4) *(u4*)(sB + wrow[q] * ILDS + wcol[q] + 16) = wo[q][WBITS == 4 ? 1 : 0];
+    }
+    __syncthreads();
+
+    for (int sb = 0; sb < sub_blocks; ++sb) {
+      i16v qc[2][2];
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+          for (int e = 0; e < 16; ++e) qc[i][j][e] = 0;
+      const int kbeg = sb * (int)p.block_k;
+      for (int ks = 0; ks < (int)p.block_k; ks += 32) {
+        i4 af[2], bf[2];
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+          af[i] = *(const i4*)(sA + (wm * 64 + i * 32 + (lane & 31)) * ILDS + kbeg + ks + (lane >> 5) * 16);
+          bf[i] = *(const i4*)(sB + (wn * 64 + i * 32 + (lane & 31)) * ILDS + kbeg + ks + (lane >> 5) * 16);
+        }
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+          for (int j = 0; j < 2; ++j)
+            qc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[i], bf[j], qc[i][j], 0, 0, 0);
+      }
+      // fp32 epilogue of this K block
+      const int64_t kq = k0 + kbeg;
+      const int64_t kb = kq / p.block_k;
+      int64_t g = kq / a.G;
+      if (g >= a.KG) g = a.KG - 1;
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        const int64_t n = n0 + wn * 64 + j * 32 + (lane & 31);
+        const float sw = n < a.NT * kTileN ? a.scales[((n / kTileN) * a.KG + g) * kTileN + (n % kTileN)] : 0.0f;
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+#pragma unroll
+          for (int e = 0; e < 16; ++e) {
+            const int64_t m = m0 + wm * 64 + i * 32 + 8 * (e >> 2) + 4 * (lane >> 5) + (e & 3);
+            const float sa = m < a.M ? p.sa[m * p.sa_m_stride + (kq / p.qbk) * p.sa_k_stride] : 0.0f;
+            const float cterm = __fmul_rn(__fmul_rn((float)qc[i][j][e], sa), sw);
+            acc[i][j][e] = __fadd_rn(acc[i][j][e], cterm);
+            if (a.debug_block_sums && m < a.M && n < a.N)
+              a.debug_block_sums[(m * a.N + n) * (p.Kpad / p.block_k) + kb] = qc[i][j][e];
+          }
+        }
+      }
+    }
+  }
+
+  Epilogue ep{a.bias, a.fusion, a.other0, a.other1, a.out, a.out_dtype, a.x_dtype, a.N};
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int64_t n = n0 + wn * 64 + j * 32 + (lane & 31);
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const int64_t m = m0 + wm * 64 + i * 32 + 8 * (e >> 2) + 4 * (lane >> 5) + (e & 3);
+        if (m < a.M && n < a.N) epilogue_store<kRegimeBF16>(ep, m, n, acc[i][j][e]);
+      }
+    }
+}
+
+template <int WBITS, int MT, int KPW, int NTW>
+static int launch_small_i8_cfg(Int8KArgs& p, hipStream_t st) {
+  const size_t smem = (size_t)NTW * MT * p.W * 64 * sizeof(f4);
+  auto kern = woq_small_m_i8_kernel<WBITS, MT, KPW, NTW>;
+  if (smem > 64 * 1024) {
+    hipError_t err = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+    if (err != hipSuccess) return set_error("hipFuncSetAttribute: %s", hipGetErrorString(err));
+  }
+  const unsigned grid = (unsigned)((p.a.NT + NTW - 1) / NTW);
+  kern<<<grid, p.W * 64, smem, st>>>(p);
+  return check_launch("woq_small_m_i8_kernel");
+}
+
+template <int WBITS>
+static int dispatch_small_i8(Int8KArgs& p, hipStream_t st) {
+  const int64_t KT = p.a.KT, NT = p.a.NT, M = p.a.M;
+  auto pick_w = [&](int kpw) {
+    int64_t w = (KT + kpw - 1) / kpw;
+    if (w > 16) {
+      const int64_t rounds = (KT + 16 * kpw - 1) / (16 * kpw);
+      w = (KT + rounds * kpw - 1) / (rounds * kpw);
+    }
+    return (int)(w < 1 ? 1 : w);
+  };
+  if (M <= 16) {
+    p.W = pick_w(2);
+    if (NT >= 512) return launch_small_i8_cfg<WBITS, 1, 2, 2>(p, st);
+    return launch_small_i8_cfg<WBITS, 1, 2, 1>(p, st);
+  } else if (M <= 32) {
+    p.W = pick_w(2);
+    if (NT >= 512) return launch_small_i8_cfg<WBITS, 2, 2, 2>(p, st);
+    return launch_small_i8_cfg<WBITS, 2, 2, 1>(p, st);
+  }
+  p.W = pick_w(2);
+  if (NT >= 512) return launch_small_i8_cfg<WBITS, 4, 2, 2>(p, st);
+  return launch_small_i8_cfg<WBITS, 4, 2, 1>(p, st);
+}
+
+int launch_int8_linear(const Int8Args& a, hipStream_t st) {
+  const int mode = a.act_quant_mode;
+  if (!quant_a_is_sym(mode) || mode > WOQ_HIP_QUANT_A_PER_M_K_BLOCK_SYM)
+    return set_error(
+        "lowp_mode INT8: act_quant_mode %d is not supported by this build (symmetric modes 4..7 only)", mode);
+  const int TK = a.wbits == 4 ? kTileK4 : kTileK8;
+  Int8KArgs p;
+  p.a = a;
+  p.Kpad = a.KT * TK;
+  p.ldq = p.Kpad;
+  const int64_t G = a.G;  // per-channel callers pass G >= Kpad
+  const bool per_channel = G >= p.Kpad;
+  p.block_k = woq_hip_int8_block_k(per_channel ? -1 : G, a.K);
+  if (p.block_k % 32 != 0 || 128 % p.block_k != 0)
+    return set_error("lowp_mode INT8: K block %lld (from group_size / K) must be 32, 64 or 128",
+                     (long long)p.block_k);
+  p.qbk = per_channel ? p.block_k : G;
+  const int64_t Kc = (a.K + p.qbk - 1) / p.qbk;
+  const bool per_m = quant_a_per_m(mode), per_k = quant_a_per_k(mode);
+  p.sa_m_stride = per_m ? (per_k ? Kc : 1) : 0;
+  p.sa_k_stride = per_k ? 1 : 0;
+  if (!per_k) p.qbk = p.Kpad + 1;  // k / qbk == 0 for every k
+
+  // workspace: q [M][ldq] | scales [groups] | (zps unused for symmetric modes)
+  const int64_t qbytes = (a.M * p.ldq + 255) / 256 * 256;
+  const int64_t groups = (per_m ? a.M : 1) * (per_k ? Kc : 1);
+  const int64_t need = qbytes + groups * (int64_t)sizeof(float);
+  if (a.workspace == nullptr || a.workspace_bytes < need)
+    return set_error("lowp_mode INT8: workspace too small (%lld < %lld bytes)", (long long)a.workspace_bytes,
+                     (long long)need);
+  uint8_t* xq = (uint8_t*)a.workspace;
+  float* sa = (float*)((uint8_t*)a.workspace + qbytes);
+  p.xq = xq;
+  p.sa = sa;
+  const int64_t qbk_quant = per_k ? (per_channel ? p.block_k : G) : a.K;
+  if (int rc = launch_quant_impl(a.x, a.x_dtype, a.M, a.K, p.ldq, qbk_quant, mode, xq, sa, nullptr,
+                                 a.wbits == 4 ? 1 : 0, st))
+    return rc;
+
+  // The small-M kernel accumulates whole tiles per MFMA, so it needs K blocks that are whole
+  // tiles; finer blocks (group_size 32 / 64 with 4-bit weights) go through the tiled kernel,
+  // which re-lays the weights in LDS in plain K order.
+  if (a.M <= 64 && p.block_k % TK == 0)
+    return a.wbits == 4 ? dispatch_small_i8<4>(p, st) : dispatch_small_i8<8>(p, st);
+  dim3 grid((unsigned)((a.NT * kTileN + IBN - 1) / IBN), (unsigned)((a.M + IBM - 1) / IBM));
+  if (a.wbits == 4)
+    woq_gemm_i8_kernel<4><<<grid, 256, 0, st>>>(p);
+  else
+    woq_gemm_i8_kernel<8><<<grid, 256, 0, st>>>(p);
+  return check_launch("woq_gemm_i8_kernel");
+}
+
+}  // namespace woq

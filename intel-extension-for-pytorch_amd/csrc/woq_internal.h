@@ -1,0 +1,78 @@
+// Host-side declarations shared by the translation units of libwoq_hip.so.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/woq_hip.h"
+
+namespace woq {
+
+// Records msg as the thread's last error and returns 1.
+int set_error(const char* fmt, ...);
+// hipGetLastError() after a launch; records and returns non-zero on failure.
+int check_launch(const char* what);
+
+struct Epilogue;
+
+// Arguments common to the floating-point kernels (small-M streaming and tiled GEMM).
+struct FpArgs {
+  const void* x;
+  int x_dtype;
+  int64_t M, K, N;       // logical sizes
+  int64_t NT, KT;        // tiles along N and K of the packed weight
+  const uint8_t* qweight;
+  const uint16_t* scales;  // fp16 bits (fp16 regime) or bf16 bits (bf16 regime), [NT][KG][16]
+  const uint8_t* zeros;    // [NT][KG][16] or nullptr
+  int64_t G;               // group size in K elements (per-channel: >= padded K)
+  int64_t KG;
+  const float* bias;
+  int fusion;
+  const void* other0;
+  const void* other1;
+  void* out;
+  int out_dtype;
+};
+
+int launch_pack_weight(const void* plain, int weight_dtype, int64_t N, int64_t K, void* packed,
+                       hipStream_t st);
+int launch_unpack_weight(const void* packed, int weight_dtype, int64_t N, int64_t K, void* plain,
+                         hipStream_t st);
+int launch_pack_qparams(const float* scales, const float* zeros, int weight_dtype, int64_t N, int64_t KG,
+                        float* s32, void* s16, void* sb16, uint8_t* z8, hipStream_t st);
+int launch_unpack_int4_zeros(const int32_t* zp32, int64_t rows, int64_t cols, int64_t cols_zp32,
+                             float* out, hipStream_t st);
+int launch_dequant_weight(const void* qweight, int weight_dtype, int64_t N, int64_t K, const float* s32,
+                          const uint8_t* z8, int64_t G, void* out, int out_dtype, hipStream_t st);
+
+// regime: 0 = fp16, 1 = bf16 (woq::Regime)
+int launch_small_m(const FpArgs& a, int wbits, int regime, hipStream_t st);
+int launch_gemm(const FpArgs& a, int wbits, int regime, hipStream_t st);
+
+struct Int8Args {
+  const void* x;
+  int x_dtype;
+  int64_t M, K, N;
+  int64_t NT, KT;
+  const uint8_t* qweight;
+  int wbits;
+  const float* scales;   // fp32 [NT][KG][16]
+  const uint8_t* zeros;  // [NT][KG][16] or nullptr
+  int64_t G, KG;
+  const float* bias;
+  int act_quant_mode;
+  int fusion;
+  const void* other0;
+  const void* other1;
+  void* out;
+  int out_dtype;
+  void* workspace;
+  int64_t workspace_bytes;
+  int32_t* debug_block_sums;
+};
+
+int launch_dynamic_quant(const void* x, int x_dtype, int64_t M, int64_t K, int64_t ldq, int64_t qbk,
+                         int mode, void* q, float* scales, int32_t* zps, hipStream_t st);
+int launch_int8_linear(const Int8Args& a, hipStream_t st);
+
+}  // namespace woq

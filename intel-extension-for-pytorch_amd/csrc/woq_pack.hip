@@ -1,0 +1,241 @@
+// Weight prepack / unpack and quantization-parameter layout kernels.
+//
+// The reference blocks weights for AVX-512 / AMX as [N/32][K/Kb][Kb][16] bytes
+// (csrc/cpu/aten/kernels/WoqUtilKrnl.cpp:32-249).  Here the unit is what one wave64 fetches
+// with a single global_load_dwordx4 per lane: a 1 KiB tile of 16 output rows.  Both
+// directions are integer-exact and invertible, as the reference's pack / unpack pair is
+// (tests/cpu/test_quantization_default_recipe.py:1848-1854).
+#include "woq_common.h"
+#include "woq_internal.h"
+
+namespace woq {
+
+// One thread per packed dword.
+__global__ void pack_int4_kernel(const uint8_t* __restrict__ plain, uint32_t* __restrict__ packed,
+                                 int64_t N, int64_t K, int64_t KT, int64_t total_dwords) {
+  const int64_t gid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (gid >= total_dwords) return;
+  const int j = gid & 3;
+  const int lane = (gid >> 2) & 63;
+  const int64_t tile = gid >> 8;
+  const int64_t nt = tile / KT, kt = tile % KT;
+  const int r = lane & 15, c = lane >> 4;
+  const int64_t n = nt * kTileN + r;
+  const int64_t kbase = kt * kTileK4 + c * 32 + j * 8;
+  const int64_t row_bytes = (K + 1) / 2;
+  uint32_t out = 0;
+  if (n < N) {
+#pragma unroll
+    for (int b = 0; b < 4; ++b) {
+      const int64_t k = kbase + 2 * b;
+      if (k < K) {
+        const uint32_t byte = plain[n * row_bytes + (k >> 1)];
+        out |= (byte & 0xFu) << (4 * b);
+        if (k + 1 < K) out |= (byte >> 4) << (16 + 4 * b);
+      }
+    }
+  }
+  packed[gid] = out;
+}
+
+// One thread per plain byte (two K elements).
+__global__ void unpack_int4_kernel(const uint32_t* __restrict__ packed, uint8_t* __restrict__ plain,
+                                   int64_t N, int64_t K, int64_t KT) {
+  const int64_t row_bytes = (K + 1) / 2;
+  const int64_t gid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (gid >= N * row_bytes) return;
+  const int64_t n = gid / row_bytes, kb = gid % row_bytes;
+  const int64_t k = kb * 2;
+  const int64_t nt = n / kTileN, kt = k / kTileK4;
+  const int r = n % kTileN;
+  const int koff = k % kTileK4;
+  const int c = koff / 32, j = (koff % 32) / 8, b = (koff % 8) / 2;
+  const uint32_t d = packed[((nt * KT + kt) * 64 + (r + 16 * c)) * 4 + j];
+  const uint32_t lo = (d >> (4 * b)) & 0xFu;
+  const uint32_t hi = (d >> (16 + 4 * b)) & 0xFu;
+  plain[gid] = (uint8_t)(lo | (hi << 4));
+}
+
+// One thread per packed dword (4 K elements of one row).
+__global__ void pack_int8_kernel(const int8_t* __restrict__ plain, uint32_t* __restrict__ packed,
+                                 int64_t N, int64_t K, int64_t KT, int64_t total_dwords) {
+  const int64_t gid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (gid >= total_dwords) return;
+  const int j = gid & 3;
+  const int lane = (gid >> 2) & 63;
+  const int64_t tile = gid >> 8;
+  const int64_t nt = tile / KT, kt = tile % KT;
+  const int r = lane & 15, c = lane >> 4;
+  const int64_t n = nt * kTileN + r;
+  const int64_t kbase = kt * kTileK8 + c * 16 + j * 4;
+  uint32_t out = 0x80808080u;  // offset-binary zero
+  if (n < N) {
+    out = 0;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int64_t k = kbase + i;
+      const uint32_t u = (k < K) ? (uint32_t)(uint8_t)(plain[n * K + k] ^ (int8_t)0x80) : 0x80u;
+      out |= u << (8 * i);
+    }
+  }
+  packed[gid] = out;
+}
+
+__global__ void unpack_int8_kernel(const uint8_t* __restrict__ packed, int8_t* __restrict__ plain,
+                                   int64_t N, int64_t K, int64_t KT) {
+  const int64_t gid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (gid >= N * K) return;
+  const int64_t n = gid / K, k = gid % K;
+  const int64_t nt = n / kTileN, kt = k / kTileK8;
+  const int r = n % kTileN;
+  const int koff = k % kTileK8;
+  const int c = koff / 16, i = koff % 16;
+  const uint8_t u = packed[((nt * KT + kt) * 64 + (r + 16 * c)) * 16 + i];
+  plain[gid] = (int8_t)(u ^ 0x80u);
+}
+
+__global__ void pack_qparams_kernel(const float* __restrict__ scales, const float* __restrict__ zeros,
+                                    int weight_dtype, int64_t N, int64_t Np, int64_t KG,
+                                    float* __restrict__ s32, uint16_t* __restrict__ s16,
+                                    uint16_t* __restrict__ sb16, uint8_t* __restrict__ z8) {
+  const int64_t gid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (gid >= Np * KG) return;
+  const int r = gid % kTileN;
+  const int64_t g = (gid / kTileN) % KG;
+  const int64_t nt = gid / (kTileN * KG);
+  const int64_t n = nt * kTileN + r;
+  float s = 1.0f, z = 0.0f;
+  if (n < N) {
+    s = scales[n * KG + g];
+    if (zeros) z = zeros[n * KG + g];
+  }
+  s32[gid] = s;
+  s16[gid] = f32_to_f16_bits(s);
+  sb16[gid] = f32_to_bf16_bits(s);
+  if (z8) {
+    int zi = (int)z;
+    if (weight_dtype == WOQ_HIP_DTYPE_INT8) zi += 128;
+    z8[gid] = (uint8_t)zi;
+  }
+}
+
+__global__ void unpack_int4_zeros_kernel(const uint32_t* __restrict__ zp32, int64_t rows, int64_t cols,
+                                         int64_t cols_zp32, float* __restrict__ out) {
+  const int64_t gid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (gid >= rows * cols) return;
+  const int64_t i = gid / cols, j = gid % cols;
+  out[gid] = (float)((zp32[i * cols_zp32 + j / 8] >> ((j % 8) * 4)) & 0xFu);
+}
+
+// Dense dequantization of a packed weight: one thread per (n, 8 consecutive k).
+__global__ void dequant_weight_kernel(const uint8_t* __restrict__ packed, int weight_dtype, int64_t N,
+                                      int64_t K, int64_t KT, const float* __restrict__ s32,
+                                      const uint8_t* __restrict__ z8, int64_t G, int64_t KG,
+                                      void* __restrict__ out, int out_dtype) {
+  const int64_t K8 = (K + 7) / 8;
+  const int64_t gid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (gid >= N * K8) return;
+  const int64_t n = gid / K8, k0 = (gid % K8) * 8;
+  const int64_t nt = n / kTileN;
+  const int r = n % kTileN;
+  const bool w4 = weight_dtype != WOQ_HIP_DTYPE_INT8;
+  const int tile_k = w4 ? kTileK4 : kTileK8;
+  const int64_t kt = k0 / tile_k;
+  const int koff = k0 % tile_k;
+  int64_t g = G > 0 ? k0 / G : 0;
+  if (g >= KG) g = KG - 1;
+  const float s = s32[(nt * KG + g) * kTileN + r];
+  float z = 0.0f;
+  if (z8)
+    z = (float)z8[(nt * KG + g) * kTileN + r];
+  else
+    z = w4 ? 8.0f : 128.0f;  // symmetric: INT4 stored +8, INT8 bytes are offset-binary
+  float w[8];
+  if (w4) {
+    const int c = koff / 32, j = (koff % 32) / 8;
+    const uint32_t d = ((const uint32_t*)packed)[((nt * KT + kt) * 64 + (r + 16 * c)) * 4 + j];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) w[e] = (float)((d >> (4 * nibble_pos(e))) & 0xFu);
+  } else {
+    const int c = koff / 16, i0 = koff % 16;
+    const uint8_t* p = packed + ((nt * KT + kt) * 64 + (r + 16 * c)) * 16 + i0;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) w[e] = (float)p[e];
+  }
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    const int64_t k = k0 + e;
+    if (k >= K) break;
+    // (q - z) first, then the scale, each in fp32 (woq_utils.h:147-161)
+    const float v = __fmul_rn(__fsub_rn(w[e], z), s);
+    store_act(out, out_dtype, n * K + k, v);
+  }
+}
+
+static inline unsigned blocks_for(int64_t n, int bs) { return (unsigned)((n + bs - 1) / bs); }
+
+int launch_pack_weight(const void* plain, int weight_dtype, int64_t N, int64_t K, void* packed,
+                       hipStream_t st) {
+  const int64_t Np = woq_hip_padded_n(N), Kp = woq_hip_padded_k(weight_dtype, K);
+  const int tile_k = weight_dtype == WOQ_HIP_DTYPE_INT8 ? kTileK8 : kTileK4;
+  const int64_t KT = Kp / tile_k;
+  const int64_t total = (Np / kTileN) * KT * (kTileBytes / 4);
+  if (total == 0) return 0;
+  if (weight_dtype == WOQ_HIP_DTYPE_INT8)
+    pack_int8_kernel<<<blocks_for(total, 256), 256, 0, st>>>((const int8_t*)plain, (uint32_t*)packed, N,
+                                                             K, KT, total);
+  else
+    pack_int4_kernel<<<blocks_for(total, 256), 256, 0, st>>>((const uint8_t*)plain, (uint32_t*)packed,
+                                                             N, K, KT, total);
+  return check_launch("pack_weight");
+}
+
+int launch_unpack_weight(const void* packed, int weight_dtype, int64_t N, int64_t K, void* plain,
+                         hipStream_t st) {
+  const int64_t Kp = woq_hip_padded_k(weight_dtype, K);
+  if (N == 0 || K == 0) return 0;
+  if (weight_dtype == WOQ_HIP_DTYPE_INT8) {
+    unpack_int8_kernel<<<blocks_for(N * K, 256), 256, 0, st>>>((const uint8_t*)packed, (int8_t*)plain, N,
+                                                               K, Kp / kTileK8);
+  } else {
+    const int64_t total = N * ((K + 1) / 2);
+    unpack_int4_kernel<<<blocks_for(total, 256), 256, 0, st>>>((const uint32_t*)packed, (uint8_t*)plain,
+                                                               N, K, Kp / kTileK4);
+  }
+  return check_launch("unpack_weight");
+}
+
+int launch_pack_qparams(const float* scales, const float* zeros, int weight_dtype, int64_t N, int64_t KG,
+                        float* s32, void* s16, void* sb16, uint8_t* z8, hipStream_t st) {
+  const int64_t Np = woq_hip_padded_n(N);
+  const int64_t total = Np * KG;
+  if (total == 0) return 0;
+  pack_qparams_kernel<<<blocks_for(total, 256), 256, 0, st>>>(scales, zeros, weight_dtype, N, Np, KG, s32,
+                                                              (uint16_t*)s16, (uint16_t*)sb16,
+                                                              zeros ? z8 : nullptr);
+  return check_launch("pack_qparams");
+}
+
+int launch_unpack_int4_zeros(const int32_t* zp32, int64_t rows, int64_t cols, int64_t cols_zp32,
+                             float* out, hipStream_t st) {
+  const int64_t total = rows * cols;
+  if (total == 0) return 0;
+  unpack_int4_zeros_kernel<<<blocks_for(total, 256), 256, 0, st>>>((const uint32_t*)zp32, rows, cols,
+                                                                   cols_zp32, out);
+  return check_launch("unpack_int4_zeros");
+}
+
+int launch_dequant_weight(const void* qweight, int weight_dtype, int64_t N, int64_t K, const float* s32,
+                          const uint8_t* z8, int64_t G, void* out, int out_dtype, hipStream_t st) {
+  if (N == 0 || K == 0) return 0;
+  const int64_t Kp = woq_hip_padded_k(weight_dtype, K);
+  const int tile_k = weight_dtype == WOQ_HIP_DTYPE_INT8 ? kTileK8 : kTileK4;
+  const int64_t KG = G > 0 ? (K + G - 1) / G : 1;
+  const int64_t total = N * ((K + 7) / 8);
+  dequant_weight_kernel<<<blocks_for(total, 256), 256, 0, st>>>((const uint8_t*)qweight, weight_dtype, N,
+                                                                K, Kp / tile_k, s32, z8, G, KG, out,
+                                                                out_dtype);
+  return check_launch("dequant_weight");
+}
+
+}  // namespace woq

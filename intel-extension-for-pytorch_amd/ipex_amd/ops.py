@@ -1,0 +1,524 @@
+"""Operator boundary: the ``torch_ipex`` / ``ipex_prepack`` ops and the prepack context.
+
+Same op names, argument order and error behaviour as the reference
+(csrc/cpu/aten/Linear.cpp:1013-1112, csrc/cpu/jit/cpu/kernels/RegisterOpContextClass.cpp:127-223),
+registered for tensors that live on the GPU:
+
+    torch.ops.torch_ipex.ipex_woq_linear(x, ctx.get_data_handle())
+    torch.ops.torch_ipex.woq_linear_{gelu,new_gelu,relu,silu}(x, handle)
+    torch.ops.torch_ipex.woq_linear_{add,add_add,mul}(x, handle, others)
+    torch.ops.torch_ipex.woq_linear(x, packed_w, "int4", [N, K], scales, zeros, bias, g_idx, G, lowp, aq, comp)
+    torch.ops.ipex_prepack.weight_only_qlinear_prepack(...)      -> WoqLinearOpContext
+    torch.ops.ipex_prepack.weight_only_qlinear_prepack_int4(...) -> WoqLinearOpContext
+    torch.ops.ipex_prepack.woq_linear_pack_weight(...) / woq_linear_unpack_weight(...)
+
+The context is a Python object here (the reference's is a TorchScript custom class); its
+``get_data_handle()`` returns a 1-element CPU int64 tensor, as the reference's does
+(csrc/cpu/jit/cpu/kernels/OpContext.cpp:396-400), and the ops resolve it through a registry
+of live contexts, so a stale handle raises instead of dereferencing freed memory.
+"""
+import os
+import threading
+import weakref
+from typing import List, Optional
+
+import torch
+
+from . import _kernels, _lib
+
+WOQ_DTYPE_MAP = {"int8": _lib.DTYPE_INT8, "int4": _lib.DTYPE_INT4, "nf4": _lib.DTYPE_NF4}
+PLAIN_WEIGHT_FORMAT, GPTQ_WEIGHT_FORMAT, AWQ_WEIGHT_FORMAT = 0, 1, 2
+
+# M at and above which a cached dequantized weight is used (IPEX_WOQ_WEIGHT_CACHE_BATCH_THRESHOLD,
+# csrc/cpu/jit/cpu/kernels/LinearWoqPacked.cpp:17-18).
+WEIGHT_CACHE_BATCH_THRESHOLD = int(os.environ.get("IPEX_WOQ_WEIGHT_CACHE_BATCH_THRESHOLD", "64"))
+
+_contexts = {}
+_contexts_lock = threading.Lock()
+_next_handle = [1]
+
+
+def _to_gpu(t, device=None):
+    if t is None:
+        return None
+    if t.is_cuda:
+        return t
+    if not torch.cuda.is_available():
+        raise RuntimeError(
+            "WOQ linear: no GPU is available; this build runs on MI355X only and has no CPU path"
+        )
+    return t.to(device if device is not None else torch.device("cuda", torch.cuda.current_device()))
+
+
+def _check_integral_zeros(zeros, weight_dtype):
+    lo, hi = (-128, 127) if weight_dtype == _lib.DTYPE_INT8 else (0, 255)
+    z = zeros.to(torch.float32)
+    ok = torch.equal(z, z.round()) and bool((z >= lo).all()) and bool((z <= hi).all())
+    if not ok:
+        raise RuntimeError(
+            f"WOQ linear: zero points must be integers in [{lo}, {hi}] for this weight dtype"
+        )
+
+
+class WoqLinearOpContext:
+    """Prepacked weight + quantization parameters of one linear layer
+    (ContextLinearWoq / IpexWoqLinearOpContext of the reference,
+    csrc/cpu/jit/cpu/kernels/ContextLinearWoq.h:12-139, OpContext.cpp:364-507).
+
+    ``weight`` is the plain checkpoint format: uint8 [N, ceil(K/2)] for 4-bit, int8 [N, K] for
+    8-bit weights.
+    """
+
+    def __init__(
+        self,
+        weight,
+        weight_dtype,
+        weight_shape,
+        scales,
+        zero_points=None,
+        bias=None,
+        g_idx=None,
+        batch_size=None,
+        group_size=-1,
+        lowp_mode=0,
+        act_quant_mode=0,
+        cache_weight_for_large_batch=False,
+    ):
+        weight_dtype = int(weight_dtype)
+        if weight_dtype not in (_lib.DTYPE_INT8, _lib.DTYPE_INT4):
+            raise RuntimeError(f"WOQ linear: unsupported weight dtype {weight_dtype} (INT8 and INT4 are built)")
+        if g_idx is not None:
+            raise RuntimeError("WOQ linear: g_idx (GPTQ act-order) is not supported by this build")
+        N, K = int(weight_shape[0]), int(weight_shape[1])
+        weight = _to_gpu(weight)
+        dev = weight.device
+        if weight_dtype == _lib.DTYPE_INT4:
+            weight = weight.view(torch.uint8) if weight.dtype != torch.uint8 else weight
+            if tuple(weight.shape) != (N, (K + 1) // 2):
+                raise RuntimeError(
+                    f"WOQ linear: int4 weight has shape {tuple(weight.shape)}, expected {(N, (K + 1) // 2)}"
+                )
+        else:
+            if weight.dtype != torch.int8 or tuple(weight.shape) != (N, K):
+                raise RuntimeError(f"WOQ linear: int8 weight must be int8 [{N}, {K}]")
+        scales = _to_gpu(scales, dev).to(torch.float32)
+        group_size = int(group_size)
+        if group_size > 0:
+            KG = (K + group_size - 1) // group_size
+            scales = scales.reshape(N, -1)
+            if scales.shape[1] != KG:
+                raise RuntimeError(
+                    f"WOQ linear: scales have {scales.shape[1]} groups, expected {KG} for group_size {group_size}"
+                )
+        else:
+            scales = scales.reshape(N, 1)
+        if zero_points is not None:
+            zero_points = _to_gpu(zero_points, dev).to(torch.float32).reshape(scales.shape)
+            _check_integral_zeros(zero_points, weight_dtype)
+        if weight_dtype == _lib.DTYPE_INT8 and int(lowp_mode) == _lib.LOWP_INT8 and zero_points is not None:
+            raise RuntimeError("WOQ: symmetric quantization is required for NF4 or INT8 with lowp-mode INT8")
+
+        self.weight_dtype_ = weight_dtype
+        self.weight_shape_ = [N, K]
+        self.group_size_ = group_size
+        self.lowp_mode_ = int(lowp_mode)
+        self.act_quant_mode_ = int(act_quant_mode)
+        self.batch_size_ = batch_size
+        self.cache_weight_for_large_batch_ = bool(cache_weight_for_large_batch)
+        self.g_idx_ = None
+        self.at_bias_ = _to_gpu(bias, dev)
+        self.bias_f32_ = self.at_bias_.to(torch.float32).contiguous() if self.at_bias_ is not None else None
+        self.at_weight_ = _kernels.pack_weight(weight, weight_dtype, N, K)
+        s32, s16, sb16, z8 = _kernels.pack_qparams(scales, zero_points, weight_dtype)
+        self.scales_list_ = [s32, s16, sb16]
+        self.zeros_u8_ = z8
+        self.scales_plain_ = scales if group_size > 0 else scales.reshape(N)
+        self.zero_points_plain_ = (
+            None if zero_points is None else (zero_points if group_size > 0 else zero_points.reshape(N))
+        )
+        self.cached_weight_ = None
+        self.cached_compensation_ = None
+        with _contexts_lock:
+            self._handle = _next_handle[0]
+            _next_handle[0] += 1
+            _contexts[self._handle] = weakref.ref(self)
+
+    def __del__(self):
+        try:
+            with _contexts_lock:
+                _contexts.pop(self._handle, None)
+        except Exception:
+            pass
+
+    # ---- reference method surface ----
+    def get_weight(self):
+        return self.at_weight_
+
+    def get_bias(self):
+        return self.at_bias_
+
+    def get_scales(self):
+        return self.scales_plain_
+
+    def get_zero_points(self):
+        return self.zero_points_plain_
+
+    def get_weight_shape(self):
+        return list(self.weight_shape_)
+
+    def get_g_idx(self):
+        return self.g_idx_
+
+    def get_cached_weight(self):
+        return self.cached_weight_
+
+    def get_cached_compensation(self):
+        return self.cached_compensation_
+
+    def pack(self, tensor):
+        return tensor
+
+    def to_public(self, tensor):
+        """Packed tensor -> plain [N, K/2] (or [N, K]) checkpoint layout."""
+        N, K = self.weight_shape_
+        return _kernels.unpack_weight(tensor, self.weight_dtype_, N, K)
+
+    def get_data_handle(self):
+        return torch.tensor([self._handle], dtype=torch.int64)
+
+    def load_from_ctx(self, other):
+        self.__dict__.update({k: v for k, v in other.__dict__.items() if k != "_handle"})
+
+    # ---- pickling: always the plain format, re-prepacked on load (OpContext.h:363-403) ----
+    def __getstate__(self):
+        cpu = lambda t: None if t is None else t.detach().cpu()
+        return (
+            cpu(self.to_public(self.at_weight_)),
+            self.weight_dtype_,
+            list(self.weight_shape_),
+            cpu(self.scales_plain_),
+            cpu(self.zero_points_plain_),
+            cpu(self.at_bias_),
+            None,
+            self.batch_size_,
+            self.group_size_,
+            self.lowp_mode_,
+            self.act_quant_mode_,
+            self.cache_weight_for_large_batch_,
+        )
+
+    def __setstate__(self, state):
+        self.__init__(*state)
+
+    # ---- execution ----
+    def _cached_bf16_weight(self):
+        if self.cached_weight_ is None:
+            N, K = self.weight_shape_
+            # the bf16-rounded scales are what the bf16 kernel dequantizes with
+            s = self.scales_list_[2].to(torch.float32)
+            self.cached_weight_ = _kernels.dequant_weight(
+                self.at_weight_, self.weight_dtype_, N, K, s, self.zeros_u8_, self.group_size_, torch.bfloat16
+            )
+        return self.cached_weight_
+
+    def run(self, x, fusion=_lib.FUSE_NONE, others=(), **kw):
+        N, K = self.weight_shape_
+        if x.shape[-1] != K:
+            raise RuntimeError(
+                f"WOQ linear: input and weight shapes do not match, got k = {x.shape[-1]} and {K} respectively."
+            )
+        M = x.numel() // K if x.numel() > 0 else 0
+        if M == 0:
+            return x.new_empty(*x.shape[:-1], N)
+        if (
+            self.cache_weight_for_large_batch_
+            and self.lowp_mode_ == _lib.LOWP_BF16
+            and M >= WEIGHT_CACHE_BATCH_THRESHOLD
+            and fusion == _lib.FUSE_NONE
+            and not kw
+        ):
+            # first-token path on a cached dequantized weight: a plain bf16 GEMM
+            # (csrc/cpu/jit/cpu/kernels/LinearWoqPacked.cpp:517-526)
+            w = self._cached_bf16_weight()
+            b = self.at_bias_.to(torch.bfloat16) if self.at_bias_ is not None else None
+            return torch.nn.functional.linear(x.to(torch.bfloat16), w, b).to(x.dtype)
+        return _kernels.linear(
+            x,
+            self.at_weight_,
+            self.weight_dtype_,
+            N,
+            K,
+            self.scales_list_[0],
+            self.scales_list_[1],
+            self.scales_list_[2],
+            self.zeros_u8_,
+            self.group_size_,
+            self.bias_f32_,
+            self.lowp_mode_,
+            self.act_quant_mode_,
+            fusion=fusion,
+            others=others,
+            **kw,
+        )
+
+
+def _context_from_handle(handle):
+    if handle.dtype != torch.int64 or handle.numel() != 1:
+        raise RuntimeError("ipex_woq_linear: W_prepack must be the 1-element int64 tensor of get_data_handle()")
+    key = int(handle.reshape(-1)[0])
+    with _contexts_lock:
+        ref = _contexts.get(key)
+    ctx = ref() if ref is not None else None
+    if ctx is None:
+        raise RuntimeError("ipex_woq_linear: the prepack context behind this handle no longer exists")
+    return ctx
+
+
+# ---- prepack entry points -----------------------------------------------------------------------
+def weight_only_qlinear_prepack(
+    W,
+    W_dtype,
+    W_shape,
+    scales,
+    zero_points,
+    B,
+    g_idx,
+    batch_size,
+    group_size,
+    lowp_mode,
+    act_quant_mode,
+    cache_weight_for_large_batch=False,
+):
+    """createWoqLinearPrePackOpContext (csrc/cpu/jit/cpu/kernels/LinearWoqPacked.cpp:20-51)."""
+    return WoqLinearOpContext(
+        W, W_dtype, list(W_shape), scales, zero_points, B, g_idx, batch_size, group_size, lowp_mode,
+        act_quant_mode, cache_weight_for_large_batch,
+    )
+
+
+def weight_only_qlinear_prepack_int4(
+    W,
+    scales,
+    zeros,
+    B,
+    g_idx,
+    batch_size,
+    group_size,
+    lowp_mode,
+    act_quant_mode,
+    cache_weight_for_large_batch=False,
+    weight_format=PLAIN_WEIGHT_FORMAT,
+):
+    """INT4 checkpoint ingest (createWoqLinearPrePackOpContextInt4,
+    csrc/cpu/jit/cpu/kernels/LinearWoqPacked.cpp:53-202): scales -> fp32, int32-compressed
+    zero points -> one value per group, int32 / uint8 weight viewed as bytes, or a float weight
+    re-quantized with the given parameters."""
+    from .utils.weight_only_quantization import gptq_to_plain, awq_to_plain
+
+    W = _to_gpu(W)
+    dev = W.device
+    scales_f32 = _to_gpu(scales, dev).squeeze().to(torch.float32)
+    zp_f32 = None
+    if zeros is not None:
+        zeros = _to_gpu(zeros, dev)
+        if zeros.dtype == torch.int32 and zeros.numel() != scales_f32.numel():
+            if scales_f32.dim() != 2 or zeros.dim() != 2 or scales_f32.size(0) != zeros.size(0):
+                raise RuntimeError("IPEX WOQ INT4: unexpected zero points size")
+            zp_f32 = _kernels.unpack_int4_zeros(zeros, scales_f32.size(1))
+        elif zeros.numel() == scales_f32.numel():
+            zp_f32 = zeros.squeeze().to(torch.float32)
+        else:
+            raise RuntimeError("IPEX WOQ INT4: unexpected zero points size")
+    if W.dtype in (torch.int32, torch.uint8):
+        if weight_format == GPTQ_WEIGHT_FORMAT:
+            plain = gptq_to_plain(W)
+        elif weight_format == AWQ_WEIGHT_FORMAT:
+            plain = awq_to_plain(W)
+        else:
+            plain = W.contiguous().view(torch.uint8)
+        N, K = plain.shape[0], plain.shape[1] * 2
+    elif W.dtype in (torch.bfloat16, torch.float32, torch.float16):
+        N, K = W.shape
+        w = W.to(torch.float32)
+        if group_size > 0:
+            wv = w.view(N, K // group_size, group_size)
+            q = wv / scales_f32.unsqueeze(2)
+            if zp_f32 is not None:
+                q = q + zp_f32.unsqueeze(2)
+        else:
+            q = w / scales_f32.unsqueeze(1)
+            if zp_f32 is not None:
+                q = q + zp_f32.unsqueeze(1)
+        q = torch.round(q).to(torch.uint8).view(N, K)
+        plain = (q[:, 1::2] << 4).bitwise_or(q[:, ::2])
+    else:
+        raise RuntimeError(f"IPEX WOQ INT4: unexpected weight data type: {W.dtype}")
+    return WoqLinearOpContext(
+        plain, _lib.DTYPE_INT4, [N, K], scales_f32, zp_f32, B, g_idx, batch_size, group_size, lowp_mode,
+        act_quant_mode, cache_weight_for_large_batch,
+    )
+
+
+def woq_linear_pack_weight(W, W_dtype, W_shape, scales, zero_points, B, g_idx, group_size, lowp_mode):
+    """packWoqLinearWeight (csrc/cpu/jit/cpu/kernels/LinearWoqPacked.cpp:212-256): returns
+    (packed weight, [scales fp32, fp16, bf16], zeros list or None, bias list or None, compensation)."""
+    ctx = WoqLinearOpContext(
+        W, WOQ_DTYPE_MAP[W_dtype], list(W_shape), scales, zero_points, B, g_idx, None, group_size, lowp_mode, 0
+    )
+    zeros = None
+    if ctx.zeros_u8_ is not None:
+        zf = ctx.zeros_u8_.to(torch.float32)
+        if ctx.weight_dtype_ == _lib.DTYPE_INT8:
+            zf = zf - 128
+        zeros = [zf, zf.to(torch.float16), zf.to(torch.bfloat16), ctx.zeros_u8_]
+    bias = None
+    if ctx.at_bias_ is not None:
+        b = ctx.at_bias_
+        bias = [b.to(torch.float32), b.to(torch.float16), b.to(torch.bfloat16)]
+    return ctx.at_weight_, list(ctx.scales_list_), zeros, bias, None
+
+
+def woq_linear_unpack_weight(W, W_dtype, W_shape, lowp_mode):
+    """unpackWoqLinearWeight (csrc/cpu/jit/cpu/kernels/LinearWoqPacked.cpp:258-275)."""
+    return _kernels.unpack_weight(W, WOQ_DTYPE_MAP[W_dtype], int(W_shape[0]), int(W_shape[1]))
+
+
+# ---- forward ops --------------------------------------------------------------------------------
+def _require_gpu_input(x, name):
+    if not x.is_cuda:
+        raise RuntimeError(
+            f"{name}: the input must be on the GPU (got {x.device}); there is no CPU implementation in this build"
+        )
+
+
+def ipex_woq_linear(input, W_prepack):
+    _require_gpu_input(input, "torch_ipex::ipex_woq_linear")
+    return _context_from_handle(W_prepack).run(input)
+
+
+def _unary(fusion, name):
+    def op(input, W_prepack):
+        _require_gpu_input(input, f"torch_ipex::{name}")
+        return _context_from_handle(W_prepack).run(input, fusion=fusion)
+
+    op.__name__ = name
+    return op
+
+
+def _binary(fusion, name, n_others):
+    def op(input, W_prepack, others):
+        _require_gpu_input(input, f"torch_ipex::{name}")
+        if len(others) < n_others:
+            raise RuntimeError(f"torch_ipex::{name}: expected {n_others} extra input(s), got {len(others)}")
+        return _context_from_handle(W_prepack).run(input, fusion=fusion, others=tuple(others[:n_others]))
+
+    op.__name__ = name
+    return op
+
+
+woq_linear_gelu = _unary(_lib.FUSE_GELU_ERF, "woq_linear_gelu")
+woq_linear_new_gelu = _unary(_lib.FUSE_GELU_TANH, "woq_linear_new_gelu")
+woq_linear_relu = _unary(_lib.FUSE_RELU, "woq_linear_relu")
+woq_linear_silu = _unary(_lib.FUSE_SILU, "woq_linear_silu")
+woq_linear_add = _binary(_lib.FUSE_ADD, "woq_linear_add", 1)
+woq_linear_add_add = _binary(_lib.FUSE_ADD_ADD, "woq_linear_add_add", 2)
+woq_linear_mul = _binary(_lib.FUSE_MUL, "woq_linear_mul", 1)
+
+
+def woq_linear(
+    input,
+    qweight,
+    weight_dtype: str,
+    weight_shape: List[int],
+    weight_scales: List[torch.Tensor],
+    weight_zeros: Optional[List[torch.Tensor]],
+    bias: Optional[List[torch.Tensor]],
+    g_idx: Optional[torch.Tensor],
+    group_size: int,
+    lowp_mode: int,
+    act_quant_mode: int,
+    compensation: Optional[torch.Tensor] = None,
+):
+    """Context-free forward (woq_linear_forward_v2, csrc/cpu/aten/Linear.cpp:556-617); the
+    tensor arguments are the outputs of ``woq_linear_pack_weight``."""
+    _require_gpu_input(input, "torch_ipex::woq_linear")
+    if weight_dtype not in WOQ_DTYPE_MAP:
+        raise RuntimeError(f"Unsupported weight dtype: {weight_dtype}")
+    if g_idx is not None:
+        raise RuntimeError("torch_ipex::woq_linear: g_idx is not supported by this build")
+    if weight_zeros is not None and len(weight_zeros) != 4:
+        raise RuntimeError("IPEX WOQ: expect list of zeros has length 4")
+    if bias is not None and len(bias) != 3:
+        raise RuntimeError("IPEX WOQ: expect list of bias has length 3")
+    if len(weight_scales) != 3:
+        raise RuntimeError("IPEX WOQ: expect list of scales has length 3")
+    N, K = int(weight_shape[0]), int(weight_shape[1])
+    return _kernels.linear(
+        input,
+        qweight,
+        WOQ_DTYPE_MAP[weight_dtype],
+        N,
+        K,
+        weight_scales[0],
+        weight_scales[1],
+        weight_scales[2],
+        weight_zeros[3] if weight_zeros is not None else None,
+        group_size,
+        bias[0].contiguous() if bias is not None else None,
+        lowp_mode,
+        act_quant_mode,
+    )
+
+
+_registered = False
+_libs = []
+
+
+def register():
+    """Registers the ops under ``torch.ops.torch_ipex`` / ``torch.ops.ipex_prepack`` (idempotent)."""
+    global _registered
+    if _registered:
+        return
+    tl = torch.library.Library("torch_ipex", "FRAGMENT")
+    _libs.append(tl)
+    key = "CompositeExplicitAutograd"
+    tl.define("ipex_woq_linear(Tensor input, Tensor W_prepack) -> Tensor")
+    tl.impl("ipex_woq_linear", ipex_woq_linear, key)
+    for name, fn in (
+        ("woq_linear_gelu", woq_linear_gelu),
+        ("woq_linear_new_gelu", woq_linear_new_gelu),
+        ("woq_linear_relu", woq_linear_relu),
+        ("woq_linear_silu", woq_linear_silu),
+    ):
+        tl.define(f"{name}(Tensor input, Tensor W_prepack) -> Tensor")
+        tl.impl(name, fn, key)
+    for name, fn in (
+        ("woq_linear_add", woq_linear_add),
+        ("woq_linear_add_add", woq_linear_add_add),
+        ("woq_linear_mul", woq_linear_mul),
+    ):
+        tl.define(f"{name}(Tensor input, Tensor W_prepack, Tensor[] others) -> Tensor")
+        tl.impl(name, fn, key)
+    tl.define(
+        "woq_linear(Tensor input, Tensor qweight, str weight_dtype, int[] weight_shape, "
+        "Tensor[] weight_scales, Tensor[]? weight_zeros, Tensor[]? bias, Tensor? g_idx, "
+        "int group_size, int lowp_mode, int act_quant_mode, Tensor? compensation=None) -> Tensor"
+    )
+    tl.impl("woq_linear", woq_linear, key)
+
+    pl = torch.library.Library("ipex_prepack", "FRAGMENT")
+    _libs.append(pl)
+    pl.define(
+        "woq_linear_pack_weight(Tensor W, str W_dtype, int[] W_shape, Tensor scales, Tensor? zero_points, "
+        "Tensor? B, Tensor? g_idx, int group_size, int lowp_mode) -> (Tensor, Tensor[], Tensor[]?, Tensor[]?, Tensor?)"
+    )
+    pl.impl("woq_linear_pack_weight", woq_linear_pack_weight, key)
+    pl.define("woq_linear_unpack_weight(Tensor W, str W_dtype, int[] W_shape, int lowp_mode) -> Tensor")
+    pl.impl("woq_linear_unpack_weight", woq_linear_unpack_weight, key)
+    # The two context-returning entry points cannot be torch.library ops (their result is a
+    # Python object); they are attached to the same namespace so that the reference call sites
+    # `torch.ops.ipex_prepack.weight_only_qlinear_prepack[_int4](...)` work unchanged.
+    ns = torch.ops.ipex_prepack
+    setattr(ns, "weight_only_qlinear_prepack", weight_only_qlinear_prepack)
+    setattr(ns, "weight_only_qlinear_prepack_int4", weight_only_qlinear_prepack_int4)
+    _registered = True

@@ -1,0 +1,389 @@
+"""GPU parity: the HIP path (through the C ABI) against the CPU oracle on identical inputs.
+
+Bars: integer results (pack / unpack, activation quantization, int32 block sums) bit-exact;
+fp32 accumulators max-abs <= 1e-2; bf16 outputs relative-L2 <= 2e-3 (two correct
+implementations with different summation orders can differ by one bf16 ulp, which at
+|y| in [8, 16) is 0.0625, so the max-abs bar is applied to the accumulators).
+"""
+import numpy as np
+import pytest
+import torch
+
+from helpers import bf16_ulp_diff, case_np, make_context, max_abs, rel_l2, to_np_f32
+from oracle import woq_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+MAX_ABS_ACC = 1e-2
+REL_L2_OUT = 2e-3
+
+
+def _kernels():
+    from ipex_amd import _kernels
+
+    return _kernels
+
+
+def _synthetic():
+    from ipex_amd.utils import synthetic
+
+    return synthetic
+
+
+# ---------------------------------------------------------------------------------------------
+# prepack: integer-exact, invertible
+# ---------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("N,K", [(16, 128), (4096, 4096), (500, 4096), (33, 200), (1, 2), (48, 4095)])
+def test_int4_pack_unpack_roundtrip(cuda, N, K):
+    k = _kernels()
+    g = torch.Generator().manual_seed(N * 7 + K)
+    plain = torch.randint(0, 256, (N, (K + 1) // 2), dtype=torch.uint8, generator=g)
+    if K % 2:
+        plain[:, -1] &= 0x0F  # the pad nibble of an odd K is zero in the format
+    packed = k.pack_weight(plain.to(cuda), 2, N, K)
+    assert packed.shape == ((N + 15) // 16, (K + 127) // 128, 1024)
+    back = k.unpack_weight(packed, 2, N, K)
+    assert torch.equal(back.cpu(), plain)
+
+
+def test_int4_pack_layout_matches_definition(cuda):
+    # lane l = r + 16c owns row r, K offsets 32c..32c+31; dword j holds offsets 8j..8j+7 with
+    # element e in nibble (e even ? e/2 : 4 + e/2)
+    k = _kernels()
+    N, K = 32, 256
+    q = torch.randint(0, 16, (N, K), dtype=torch.uint8, generator=torch.Generator().manual_seed(1))
+    plain = (q[:, 1::2] << 4) | q[:, ::2]
+    packed = k.pack_weight(plain.to(cuda), 2, N, K).cpu().numpy().view(np.uint32).reshape(2, 2, 64, 4)
+    qn = q.numpy()
+    for nt, kt, lane, j in [(0, 0, 0, 0), (1, 1, 37, 3), (0, 1, 63, 2), (1, 0, 16, 1)]:
+        r, c = lane % 16, lane // 16
+        word = int(packed[nt, kt, lane, j])
+        for e in range(8):
+            pos = e // 2 if e % 2 == 0 else 4 + e // 2
+            assert (word >> (4 * pos)) & 0xF == qn[nt * 16 + r, kt * 128 + c * 32 + j * 8 + e]
+
+
+@pytest.mark.parametrize("N,K", [(16, 64), (11008, 4096), (37, 100)])
+def test_int8_pack_unpack_roundtrip(cuda, N, K):
+    k = _kernels()
+    plain = torch.randint(-128, 128, (N, K), dtype=torch.int8, generator=torch.Generator().manual_seed(N + K))
+    packed = k.pack_weight(plain.to(cuda), 1, N, K)
+    assert torch.equal(k.unpack_weight(packed, 1, N, K).cpu(), plain)
+
+
+def test_qparams_layout(cuda):
+    k = _kernels()
+    N, KG = 40, 3
+    s = torch.rand(N, KG) + 0.5
+    z = torch.randint(0, 16, (N, KG)).float()
+    s32, s16, sb16, z8 = k.pack_qparams(s.to(cuda), z.to(cuda), 2)
+    assert s32.shape == (3, KG, 16)
+    sp = torch.ones(48, KG)
+    sp[:N] = s
+    zp = torch.zeros(48, KG)
+    zp[:N] = z
+    assert torch.equal(s32.cpu(), sp.view(3, 16, KG).permute(0, 2, 1))
+    assert torch.equal(s16.cpu(), sp.view(3, 16, KG).permute(0, 2, 1).half())
+    assert torch.equal(sb16.cpu(), sp.view(3, 16, KG).permute(0, 2, 1).bfloat16())
+    assert torch.equal(z8.cpu().float(), zp.view(3, 16, KG).permute(0, 2, 1))
+
+
+def test_compressed_zero_points(cuda):
+    k = _kernels()
+    zp32 = torch.randint(-(2**31), 2**31 - 1, (9, 5), dtype=torch.int32, generator=torch.Generator().manual_seed(2))
+    got = k.unpack_int4_zeros(zp32.to(cuda), 37).cpu().numpy()
+    assert np.array_equal(got, O.unpack_compressed_zeros(zp32.numpy(), 37))
+
+
+@pytest.mark.parametrize("G", [32, 128, -1])
+def test_dequant_weight_bit_exact(cuda, G):
+    syn, k = _synthetic(), _kernels()
+    case = syn.make_int4_case(9, 1, 512, 80, G, scale_dtype=torch.float32)
+    ctx = make_context(case, 2)
+    c = case_np(case)
+    want = O.dequantize_woq_weight(c["qw"], 80, 512, c["scales"], c["zps"], 2, G)
+    got = k.dequant_weight(ctx.at_weight_, 2, 80, 512, ctx.scales_list_[0], ctx.zeros_u8_, G)
+    assert np.array_equal(got.cpu().numpy(), want)
+    got16 = k.dequant_weight(ctx.at_weight_, 2, 80, 512, ctx.scales_list_[0], ctx.zeros_u8_, G, torch.bfloat16)
+    assert np.array_equal(to_np_f32(got16), O.bf16_round(want))
+
+
+# ---------------------------------------------------------------------------------------------
+# floating-point paths
+# ---------------------------------------------------------------------------------------------
+def _check_fp(case, lowp_mode, ctx=None, cols=None, force_kernel=0, label=""):
+    """Runs the HIP path twice (output dtype and fp32 accumulator) and checks both oracles."""
+    k = _kernels()
+    ctx = ctx or make_context(case, lowp_mode)
+    x = case["x"].cuda()
+    N, K, G = case["N"], case["K"], case["group_size"]
+    kw = dict(force_kernel=force_kernel)
+    y = to_np_f32(ctx.run(x, **kw))
+    acc = ctx.run(x, out_fp32=True, **kw).cpu().numpy()
+    c = case_np(case)
+    M = c["x"].shape[0]
+    cd = O.select_compute(lowp_mode, "bf16", M)
+    qw, sc, zp, b = c["qw"], c["scales"], c["zps"], c["bias"]
+    if cols is not None:  # check a subset of output columns against the oracle
+        qw, sc = qw[cols], sc[cols]
+        zp = None if zp is None else zp[cols]
+        b = None if b is None else b[cols]
+        y, acc = y[:, cols], acc[:, cols]
+        N = len(cols)
+    wd = case["weight_dtype"]
+    acc_ref, y_ref = O.woq_linear_ref(c["x"], "bf16", qw, N, K, sc, zp, b, wd, G, cd)
+    stats = {"max_abs_acc_vs_ref": max_abs(acc, acc_ref), "rel_l2_out_vs_ref": rel_l2(y, y_ref)}
+    assert stats["max_abs_acc_vs_ref"] <= MAX_ABS_ACC, (label, stats)
+    assert stats["rel_l2_out_vs_ref"] <= REL_L2_OUT, (label, stats)
+    if cd == "bf16":
+        acc_opt, y_opt = O.woq_linear_opt_bf16(c["x"], "bf16", qw, N, K, sc, zp, b, wd, G)
+        stats["max_abs_acc_vs_opt"] = max_abs(acc, acc_opt)
+        stats["rel_l2_out_vs_opt"] = rel_l2(y, y_opt)
+        ulps = bf16_ulp_diff(y, y_opt)
+        stats["out_ulp_max_vs_opt"] = int(ulps.max())
+        stats["out_exact_frac_vs_opt"] = float((ulps == 0).mean())
+        assert stats["max_abs_acc_vs_opt"] <= MAX_ABS_ACC, (label, stats)
+        assert stats["rel_l2_out_vs_opt"] <= REL_L2_OUT, (label, stats)
+        assert stats["out_ulp_max_vs_opt"] <= 1, (label, stats)
+    elif wd == 2 and M <= 4 and N * K <= 4096 * 4096:
+        # the optimized fp16 kernel accumulates in fp16; its own rounding noise exceeds 1e-2 at
+        # these magnitudes, so only the relative-L2 bar applies against it
+        y_h = O.woq_linear_opt_fp16(c["x"], qw, N, K, sc, zp, b, wd, G)
+        stats["rel_l2_out_vs_opt_fp16"] = rel_l2(y, y_h)
+        stats["max_abs_out_vs_opt_fp16"] = max_abs(y, y_h)
+        assert stats["rel_l2_out_vs_opt_fp16"] <= 6e-3, (label, stats)
+    print(label, stats)
+    return stats
+
+
+def test_c0_int4_g128_m1(cuda):
+    case = _synthetic().make_int4_case(0, 1, 4096, 4096, 128)
+    _check_fp(case, O.LOWP_BF16, label="C0")
+
+
+@pytest.mark.parametrize("M", [1, 4, 8, 16])
+@pytest.mark.parametrize("K,N", [(4096, 14336), (14336, 4096)])
+def test_c2_decode_sweep(cuda, M, K, N):
+    case = _synthetic().make_int4_case(2, M, K, N, 128)
+    cols = np.arange(0, N, 7)  # every 7th output column keeps the oracle in seconds
+    _check_fp(case, O.LOWP_BF16, cols=cols, label=f"C2 M={M} K={K} N={N}")
+
+
+def test_c1_int8_per_channel_bias(cuda):
+    case = _synthetic().make_int8_case(1, 32, 4096, 11008)
+    _check_fp(case, O.LOWP_BF16, cols=np.arange(0, 11008, 5), label="C1")
+
+
+@pytest.mark.parametrize("K,N", [(4096, 6144), (4096, 4096), (4096, 28672), (14336, 4096)])
+def test_c4_block_g32_m16(cuda, K, N):
+    case = _synthetic().make_int4_case(4, 16, K, N, 32)
+    _check_fp(case, O.LOWP_BF16, cols=np.arange(0, N, 9), label=f"C4 K={K} N={N}")
+
+
+def test_c3_prefill_bf16(cuda):
+    case = _synthetic().make_int4_case(3, 2048, 4096, 14336, 128, outliers=True)
+    _check_fp(case, O.LOWP_BF16, cols=np.arange(0, 14336, 29), label="C3 bf16")
+
+
+@pytest.mark.parametrize("M", [1, 3, 5, 17, 33, 64, 65, 130, 257])
+def test_ragged_m_small_shapes(cuda, M):
+    case = _synthetic().make_int4_case(11, M, 512, 272, 128, bias=True)
+    _check_fp(case, O.LOWP_BF16, label=f"ragged M={M}")
+
+
+@pytest.mark.parametrize("N,K,G", [(500, 1024, 128), (30, 384, 32), (100, 640, 64), (64, 1000, -1), (17, 136, -1)])
+def test_ragged_n_k(cuda, N, K, G):
+    case = _synthetic().make_int4_case(12, 6, K, N, G, bias=True)
+    _check_fp(case, O.LOWP_BF16, label=f"ragged N={N} K={K} G={G}")
+    case = _synthetic().make_int4_case(13, 2, K, N, G)
+    _check_fp(case, O.LOWP_BF16, label=f"ragged fp16 N={N} K={K} G={G}")
+    case = _synthetic().make_int4_case(14, 150, K, N, G, bias=True)
+    _check_fp(case, O.LOWP_BF16, label=f"ragged gemm N={N} K={K} G={G}")
+
+
+@pytest.mark.parametrize("M", [2, 40, 100])
+def test_both_kernels_agree_on_mid_m(cuda, M):
+    case = _synthetic().make_int4_case(15, M, 1024, 256, 128, bias=True)
+    if M <= 64:
+        _check_fp(case, O.LOWP_BF16, force_kernel=1, label=f"small-M kernel M={M}")
+    _check_fp(case, O.LOWP_BF16, force_kernel=2, label=f"tiled kernel M={M}")
+
+
+def test_int8_weights_small_and_tiled(cuda):
+    for M in (1, 8, 40, 200):
+        case = _synthetic().make_int8_case(16, M, 512, 144)
+        _check_fp(case, O.LOWP_BF16, label=f"int8 weights M={M}")
+
+
+def test_lowp_none_and_fp16_modes(cuda):
+    case = _synthetic().make_int4_case(17, 3, 512, 64, 128)
+    _check_fp(case, O.LOWP_NONE, label="lowp NONE (bf16 compute at M=3)")
+    _check_fp(case, O.LOWP_FP16, label="lowp FP16")
+    case = _synthetic().make_int4_case(17, 70, 512, 64, 128)
+    _check_fp(case, O.LOWP_FP16, label="lowp FP16 tiled")
+
+
+def test_symmetric_int4(cuda):
+    case = _synthetic().make_int4_case(18, 7, 512, 96, 128)
+    case["zeros"] = None
+    _check_fp(case, O.LOWP_BF16, label="sym int4")
+
+
+def test_empty_batch(cuda):
+    case = _synthetic().make_int4_case(19, 1, 256, 32, 128)
+    ctx = make_context(case, O.LOWP_BF16)
+    y = ctx.run(torch.empty(0, 256, dtype=torch.bfloat16, device=cuda))
+    assert y.shape == (0, 32)
+    y = ctx.run(torch.randn(2, 3, 256, device=cuda).bfloat16())
+    assert y.shape == (2, 3, 32)
+
+
+# ---------------------------------------------------------------------------------------------
+# lowp_mode INT8
+# ---------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("mode", [4, 5, 6, 7])
+@pytest.mark.parametrize("M,K", [(1, 512), (37, 4096), (300, 1024)])
+def test_dynamic_quant_bit_exact(cuda, mode, M, K):
+    k = _kernels()
+    x = torch.randn(M, K, generator=torch.Generator().manual_seed(M + K + mode))
+    x[0, :5] = torch.tensor([0.5, -0.5, 1.5, 2.5, 1e-3])
+    x = x.to(torch.bfloat16)
+    q, s, zp = k.dynamic_quant(x.to(cuda), 128, mode)
+    q_ref, s_ref, _ = O.dynamic_quantize_per_block(to_np_f32(x), 128, mode)
+    assert np.array_equal(s.cpu().numpy(), s_ref)
+    assert np.array_equal(q.cpu().numpy(), q_ref)
+
+
+def test_dynamic_quant_all_bf16_patterns(cuda):
+    k = _kernels()
+    bits = torch.arange(65536, dtype=torch.int32).to(torch.int16)
+    vals = bits.view(torch.bfloat16)
+    vals = vals[torch.isfinite(vals.float()) & (vals.float().abs() < 3e4)]
+    n = (vals.numel() // 1024) * 1024
+    x = vals[torch.randperm(vals.numel(), generator=torch.Generator().manual_seed(0))][:n].reshape(-1, 1024)
+    for mode in (6, 7):
+        q, s, _ = k.dynamic_quant(x.to(cuda), 128, mode)
+        q_ref, s_ref, _ = O.dynamic_quantize_per_block(to_np_f32(x), 128, mode)
+        assert np.array_equal(s.cpu().numpy(), s_ref)
+        assert np.array_equal(q.cpu().numpy(), q_ref)
+
+
+def _check_int8(case, mode, cols=None, debug=True, label=""):
+    ctx = make_context(case, O.LOWP_INT8, mode)
+    x = case["x"].cuda()
+    N, K, G = case["N"], case["K"], case["group_size"]
+    c = case_np(case)
+    y = to_np_f32(ctx.run(x))
+    if debug:
+        acc, sums = ctx.run(x, out_fp32=True, debug_block_sums=True)
+        sums = sums.cpu().numpy()
+    else:
+        acc, sums = ctx.run(x, out_fp32=True), None
+    acc = acc.cpu().numpy()
+    qw, sc, zp, b = c["qw"], c["scales"], c["zps"], c["bias"]
+    if cols is not None:
+        qw, sc = qw[cols], sc[cols]
+        zp = None if zp is None else zp[cols]
+        b = None if b is None else b[cols]
+        y, acc = y[:, cols], acc[:, cols]
+        sums = None if sums is None else sums[:, cols]
+        N = len(cols)
+    r = O.woq_linear_opt_int8(c["x"], "bf16", qw, N, K, sc, zp, b, case["weight_dtype"], G, mode)
+    if sums is not None:
+        assert np.array_equal(sums[:, :, : r["sums"].shape[2]], r["sums"]), label  # int32, bit-exact
+    stats = {"max_abs_acc": max_abs(acc, r["acc"]), "rel_l2_out": rel_l2(y, r["y"])}
+    print(label, stats)
+    assert stats["max_abs_acc"] <= MAX_ABS_ACC and stats["rel_l2_out"] <= REL_L2_OUT, (label, stats)
+    return stats
+
+
+@pytest.mark.parametrize("mode", [6, 7, 4, 5])
+@pytest.mark.parametrize("M", [1, 4, 16, 48, 150])
+def test_int8_lowp_int4_g128(cuda, mode, M):
+    case = _synthetic().make_int4_case(20, M, 1024, 272, 128, bias=True, outliers=True)
+    _check_int8(case, mode, label=f"int8 lowp mode={mode} M={M}")
+
+
+@pytest.mark.parametrize("G", [32, 64, -1, 256])
+@pytest.mark.parametrize("M", [3, 130])
+def test_int8_lowp_other_groups(cuda, G, M):
+    case = _synthetic().make_int4_case(21, M, 1024, 144, G, bias=True)
+    _check_int8(case, 7, label=f"int8 lowp G={G} M={M}")
+    _check_int8(case, 6, label=f"int8 lowp G={G} M={M} per-M")
+
+
+def test_int8_lowp_int8_weights(cuda):
+    for M in (2, 20, 140):
+        case = _synthetic().make_int8_case(22, M, 512, 80)
+        _check_int8(case, 6, label=f"int8 lowp int8 weights M={M}")
+
+
+def test_c3_prefill_int8(cuda):
+    case = _synthetic().make_int4_case(3, 2048, 4096, 14336, 128, outliers=True)
+    _check_int8(case, 6, cols=np.arange(0, 14336, 61), debug=False, label="C3 int8 per-M")
+    # bit-exact int32 block sums on a slice small enough to hold [M, N, K/128]
+    small = dict(case)
+    small["x"] = case["x"][:96]
+    small["qweight"], small["scales"], small["zeros"] = case["qweight"][:512], case["scales"][:512], case["zeros"][:512]
+    small["N"], small["M"] = 512, 96
+    _check_int8(small, 6, label="C3 int8 block sums slice")
+
+
+# ---------------------------------------------------------------------------------------------
+# post-ops and size-independent properties
+# ---------------------------------------------------------------------------------------------
+def test_fused_post_ops(cuda):
+    from ipex_amd import _lib
+
+    case = _synthetic().make_int4_case(23, 9, 512, 96, 128, bias=True)
+    ctx = make_context(case, O.LOWP_BF16)
+    x = case["x"].cuda()
+    base = ctx.run(x)
+    o1 = torch.randn(9, 96, device=cuda).bfloat16()
+    o2 = torch.randn(9, 96, device=cuda).bfloat16()
+    F = torch.nn.functional
+    checks = {
+        _lib.FUSE_RELU: F.relu(base.float()),
+        _lib.FUSE_SILU: F.silu(base.float()),
+        _lib.FUSE_GELU_ERF: F.gelu(base.float()),
+        _lib.FUSE_GELU_TANH: F.gelu(base.float(), approximate="tanh"),
+    }
+    for fusion, want in checks.items():
+        got = ctx.run(x, fusion=fusion)
+        assert torch.allclose(got.float(), want.bfloat16().float(), atol=2e-2, rtol=2e-2), fusion
+    assert torch.equal(ctx.run(x, fusion=_lib.FUSE_ADD, others=(o1,)), (base.float() + o1.float()).bfloat16())
+    assert torch.equal(ctx.run(x, fusion=_lib.FUSE_MUL, others=(o1,)), (base.float() * o1.float()).bfloat16())
+    want = ((base.float() + o1.float()).bfloat16().float() + o2.float()).bfloat16()
+    assert torch.equal(ctx.run(x, fusion=_lib.FUSE_ADD_ADD, others=(o1, o2)), want)
+
+
+def test_linearity_in_scales_at_full_size(cuda):
+    # doubling every scale doubles the fp32 accumulator exactly (powers of two commute with
+    # every rounding on the path); run at the full decode shape
+    syn = _synthetic()
+    case = syn.make_int4_case(2, 4, 4096, 14336, 128)
+    a1 = make_context(case, O.LOWP_BF16).run(case["x"].cuda(), out_fp32=True)
+    case2 = dict(case)
+    case2["scales"] = case["scales"] * 2
+    a2 = make_context(case2, O.LOWP_BF16).run(case["x"].cuda(), out_fp32=True)
+    assert torch.equal(a2, a1 * 2)
+
+
+def test_zero_point_equal_to_weight_gives_bias(cuda):
+    # q == z everywhere -> every dequantized weight is 0 -> output is exactly the bias
+    syn = _synthetic()
+    case = syn.make_int4_case(24, 5, 1024, 272, 128, bias=True)
+    q = torch.full((272, 1024), 7, dtype=torch.uint8)
+    case["qweight"] = (q[:, 1::2] << 4) | q[:, ::2]
+    case["zeros"] = torch.full_like(case["zeros"], 7.0)
+    y = make_context(case, O.LOWP_BF16).run(case["x"].cuda())
+    assert torch.equal(y.cpu(), case["bias"].unsqueeze(0).expand(5, -1))
+    y = make_context(case, O.LOWP_INT8, 6).run(case["x"].cuda())
+    assert torch.equal(y.cpu(), case["bias"].unsqueeze(0).expand(5, -1))
+
+
+def test_determinism(cuda):
+    case = _synthetic().make_int4_case(2, 8, 4096, 14336, 128)
+    ctx = make_context(case, O.LOWP_BF16)
+    x = case["x"].cuda()
+    assert torch.equal(ctx.run(x), ctx.run(x))

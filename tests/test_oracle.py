@@ -1,0 +1,282 @@
+"""Pins the CPU oracle: every function is checked against something the oracle did not
+compute itself -- hand-built bytes, brute force in exact arithmetic, invariants of the
+definition, or the AWQ tensors the reference's own test holds."""
+import fractions
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import woq_oracle as O
+
+GOLDEN = os.path.join(os.path.dirname(__file__), "golden")
+
+
+def test_nibble_order_closed_form():
+    # byte j = q[2j] | q[2j+1] << 4
+    q = np.array([[1, 2, 3, 4, 15, 0]], dtype=np.uint8)
+    packed = O.pack_int4(q)
+    assert packed.tolist() == [[0x21, 0x43, 0x0F]]
+    assert O.unpack_int4(packed).tolist() == q.tolist()
+    # odd K pads one zero element
+    assert O.pack_int4(np.array([[7, 9, 5]], dtype=np.uint8)).tolist() == [[0x97, 0x05]]
+
+
+def test_compressed_zero_points_closed_form():
+    # 8 zero points per int32, value j in nibble j
+    word = sum(((j + 3) % 16) << (4 * j) for j in range(8))
+    zp32 = np.array([[word, 0x0000_00A5]], dtype=np.uint32).view(np.int32)
+    out = O.unpack_compressed_zeros(zp32, 10)
+    assert out.tolist() == [[(j + 3) % 16 for j in range(8)] + [5, 10]]
+    # high bit set in the word must not sign-extend
+    zp32 = np.array([[0xF000_0000]], dtype=np.uint32).view(np.int32)
+    assert O.unpack_compressed_zeros(zp32, 8).tolist() == [[0, 0, 0, 0, 0, 0, 0, 15]]
+
+
+def test_dequantize_brute_force_all_codes():
+    # every code x every zero point, one group each: (q - z) * s in exact rationals
+    codes = np.arange(16, dtype=np.uint8)
+    K = 16
+    for z in range(16):
+        qw = O.pack_int4(codes[None, :])
+        s = np.float32(0.0123)
+        got = O.dequantize_woq_weight(qw, 1, K, np.array([[s]]), np.array([[float(z)]]), O.WOQ_DTYPE_INT4, 16)
+        want = [float(fractions.Fraction(int(c) - z) * fractions.Fraction(float(s))) for c in codes]
+        assert np.array_equal(got[0], np.array(want, dtype=np.float32))
+    # symmetric int4 is stored +8
+    got = O.dequantize_woq_weight(O.pack_int4(codes[None, :]), 1, K, np.array([2.0]), None, O.WOQ_DTYPE_INT4, -1)
+    assert got[0].tolist() == [2.0 * (c - 8) for c in range(16)]
+
+
+def test_dequantize_group_indexing():
+    # group g of row n must use scales[n, g]: make each group's scale identify it
+    N, K, G = 3, 96, 32
+    q = np.full((N, K), 5, dtype=np.uint8)
+    scales = np.arange(1, N * 3 + 1, dtype=np.float32).reshape(N, 3)
+    zps = np.full((N, 3), 4.0, dtype=np.float32)
+    w = O.dequantize_woq_weight(O.pack_int4(q), N, K, scales, zps, O.WOQ_DTYPE_INT4, G)
+    for n in range(N):
+        for k in range(K):
+            assert w[n, k] == scales[n, k // G]
+    # trailing partial group
+    w = O.dequantize_woq_weight(O.pack_int4(q[:, :80]), N, 80, scales, zps, O.WOQ_DTYPE_INT4, G)
+    assert w[1, 79] == scales[1, 2] and w.shape == (N, 80)
+
+
+def test_bf16_round_matches_torch_on_all_halfway_cases():
+    rng = np.random.default_rng(0)
+    x = rng.standard_normal(200000).astype(np.float32) * rng.choice([1e-3, 1.0, 300.0], 200000).astype(np.float32)
+    # exact ties: mantissa low 16 bits = 0x8000
+    ties = (x.view(np.uint32) & 0xFFFF0000 | 0x8000).view(np.float32)
+    for arr in (x, ties):
+        want = torch.from_numpy(arr).to(torch.bfloat16).float().numpy()
+        assert np.array_equal(O.bf16_round(arr), want)
+
+
+def test_fma16_is_single_rounding():
+    # a*b + c where the double rounding fp32->fp16 would differ from one rounding
+    rng = np.random.default_rng(1)
+    a = rng.standard_normal(20000).astype(np.float16)
+    b = rng.integers(-15, 16, 20000).astype(np.float16)
+    c = (rng.standard_normal(20000) * 30).astype(np.float16)
+    got = O._fma16(a, b, c)
+    want = np.array(
+        [
+            np.float16(float(fractions.Fraction(float(x)) * fractions.Fraction(float(y)) + fractions.Fraction(float(z))))
+            for x, y, z in zip(a[:3000], b[:3000], c[:3000])
+        ],
+        dtype=np.float16,
+    )
+    assert np.array_equal(got[:3000], want)
+
+
+def _tiny_case(M=3, N=5, K=64, G=32, seed=0, bias=True):
+    rng = np.random.default_rng(seed)
+    x = O.bf16_round(rng.standard_normal((M, K)).astype(np.float32))
+    q = rng.integers(0, 16, (N, K)).astype(np.uint8)
+    scales = O.bf16_round((0.005 + 0.015 * rng.random((N, K // G))).astype(np.float32))
+    zps = rng.integers(0, 16, (N, K // G)).astype(np.float32)
+    b = O.bf16_round((0.02 * rng.standard_normal(N)).astype(np.float32)) if bias else None
+    return x, q, O.pack_int4(q), scales, zps, b
+
+
+def test_gemm_paths_against_exact_rational_matmul():
+    M, N, K, G = 3, 5, 64, 32
+    x, q, qw, scales, zps, b = _tiny_case(M, N, K, G)
+    F = fractions.Fraction
+    exact = np.zeros((M, N))
+    for m in range(M):
+        for n in range(N):
+            acc = F(0)
+            for k in range(K):
+                acc += F(float(x[m, k])) * F(int(q[n, k]) - int(zps[n, k // G])) * F(float(scales[n, k // G]))
+            exact[m, n] = float(acc + F(float(b[n])))
+    # fallback path with fp32 compute: no weight rounding -> equals the exact value to fp64 accuracy
+    acc, _ = O.woq_linear_ref(x, "bf16", qw, N, K, scales, zps, b, O.WOQ_DTYPE_INT4, G, "fp32")
+    assert np.max(np.abs(acc - exact)) < 1e-5
+    # bf16 path: weights rounded to bf16 first -> within K * 2^-9 * |x||w| of exact, and equal to
+    # an explicit per-element evaluation
+    acc_b, y_b = O.woq_linear_opt_bf16(x, "bf16", qw, N, K, scales, zps, b, O.WOQ_DTYPE_INT4, G)
+    manual = np.zeros((M, N))
+    for m in range(M):
+        for n in range(N):
+            tot = F(float(b[n]))
+            for k in range(K):
+                w = np.float32(np.float32(int(q[n, k]) - zps[n, k // G]) * scales[n, k // G])
+                w = torch.tensor(float(w)).to(torch.bfloat16).item()
+                tot += F(float(x[m, k])) * F(w)
+            manual[m, n] = float(tot)
+    assert np.max(np.abs(acc_b - manual)) < 1e-9
+    assert np.max(np.abs(acc_b - exact)) < 0.05
+    assert np.array_equal(y_b, torch.from_numpy(acc_b.astype(np.float32)).to(torch.bfloat16).float().numpy())
+    # fp16 chain: stays within the fp16 accumulation error of the exact value
+    y_h = O.woq_linear_opt_fp16(x[:2], qw, N, K, scales, zps, b, O.WOQ_DTYPE_INT4, G)
+    assert np.max(np.abs(y_h - exact[:2])) < 0.08
+
+
+def test_fp16_chain_order_matters_and_is_sequential():
+    # one output, K = 4: ((x0*w0 + x1*w1) + x2*w2) + x3*w3 in fp16, chosen so that another order differs
+    x = np.array([[1024.0, 0.25, 0.25, -1024.0]], dtype=np.float32)
+    q = np.array([[9, 9, 9, 9]], dtype=np.uint8)  # z = 8 -> w = 1
+    zps = np.array([[8.0]], dtype=np.float32)
+    scales = np.array([[1.0]], dtype=np.float32)
+    y = O.woq_linear_opt_fp16(x, O.pack_int4(q), 1, 4, scales, zps, None, O.WOQ_DTYPE_INT4, 4, block_k=4)
+    # sequential: 1024 + .25 -> 1024 (fp16 ulp at 1024 is 1), again 1024, then 0
+    assert y[0, 0] == 0.0
+    # per-block scaling happens after the block sum: two blocks of 2
+    y2 = O.woq_linear_opt_fp16(x, O.pack_int4(q), 1, 4, np.array([[1.0, 1.0]], np.float32),
+                               np.array([[8.0, 8.0]], np.float32), None, O.WOQ_DTYPE_INT4, 2, block_k=2)
+    # block0: 1024 (0.25 lost); block1: 0.25 - 1024 -> -1024 (fp16); C = 1024 + (-1024) = 0
+    assert y2[0, 0] == 0.0
+
+
+def test_select_compute_table():
+    assert O.select_compute(O.LOWP_BF16, "bf16", 1) == "fp16"
+    assert O.select_compute(O.LOWP_BF16, "bf16", 4) == "fp16"
+    assert O.select_compute(O.LOWP_BF16, "bf16", 5) == "bf16"
+    assert O.select_compute(O.LOWP_NONE, "bf16", 1) == "bf16"
+    assert O.select_compute(O.LOWP_NONE, "fp16", 100) == "fp16"
+    assert O.select_compute(O.LOWP_FP16, "bf16", 100) == "fp16"
+    assert O.select_compute(O.LOWP_INT8, "bf16", 1) == "int8"
+    assert O.select_compute(O.LOWP_NONE, "fp32", 1) == "fp32"
+    assert [O.int8_block_k(g, 4096) for g in (-1, 32, 64, 128, 256)] == [128, 32, 64, 128, 128]
+    assert O.int8_block_k(-1, 4160) == 64
+
+
+def _all_bf16_values():
+    bits = np.arange(65536, dtype=np.uint32)
+    v = (bits << 16).view(np.float32)
+    return v[np.isfinite(v)]
+
+
+@pytest.mark.parametrize("mode", [4, 6, 7, 0, 2])
+def test_dynamic_quant_invariants_over_all_bf16_patterns(mode):
+    vals = _all_bf16_values()
+    vals = vals[np.abs(vals) < 1e4]
+    rng = np.random.default_rng(3)
+    x = rng.permutation(vals)[: 64 * 512].reshape(64, 512).astype(np.float32)
+    qbk = 128
+    q, s, zp = O.dynamic_quantize_per_block(x, qbk, mode)
+    sym = mode >= 4
+    per_m = mode in (2, 3, 6, 7)
+    per_k = mode in (1, 3, 5, 7)
+    assert q.dtype == (np.int8 if sym else np.uint8)
+    for m in range(64):
+        for kc in range(4 if per_k else 1):
+            rows = slice(m, m + 1) if per_m else slice(0, 64)
+            cols = slice(kc * qbk, (kc + 1) * qbk) if per_k else slice(0, 512)
+            blk, qb = x[rows, cols], q[rows, cols].astype(np.float64)
+            idx = tuple(([m] if per_m else []) + ([kc] if per_k else [])) or (0,)
+            sc = float(s[idx])
+            if sym:
+                amax = np.abs(blk).max()
+                # the definition: scale = absmax / 127 as an fp32 division
+                assert sc == float(np.float32(amax) / np.float32(127))
+                # the extreme element lands on +-127, nothing exceeds it
+                assert np.abs(qb).max() == 127
+                assert np.all(np.abs(blk - qb * sc) <= sc * 0.5 * (1 + 1e-4))
+            else:
+                z = float(zp[idx])
+                assert sc == float(np.float32(blk.max() - blk.min()) / np.float32(255))
+                assert qb.min() >= 0 and qb.max() <= 255
+                inside = (qb > 0) & (qb < 255)
+                assert np.all(np.abs(blk - (qb - z) * sc)[inside] <= sc * 0.5 * (1 + 1e-3))
+        if not per_m:
+            break
+
+
+def test_dynamic_quant_rounds_half_to_even():
+    # scale = 127/127 = 1 -> q = rint(x): halves go to the even neighbour
+    x = np.array([[127.0, 0.5, 1.5, 2.5, -0.5, -1.5, -2.5, 3.5]], dtype=np.float32)
+    q, s, _ = O.dynamic_quantize_per_block(x, 8, 6)
+    assert s.tolist() == [1.0]
+    assert q.tolist() == [[127, 0, 2, 2, 0, -2, -2, 4]]
+    # asymmetric: zp = -rint(min / s), q = rint(x / s + zp), clamped to 0..255
+    x = np.array([[-1.0, 0.0, 1.0, 254.0]], dtype=np.float32)
+    q, s, zp = O.dynamic_quantize_per_block(x, 4, 2)
+    assert s.tolist() == [1.0] and zp.tolist() == [1]
+    assert q.tolist() == [[0, 1, 2, 255]]
+    # symmetric clamps at -128..127 only through rounding: -absmax maps to -127
+    x = np.array([[-4.0, 4.0, 0.0, 2.0]], dtype=np.float32)
+    q, _, _ = O.dynamic_quantize_per_block(x, 4, 6)
+    assert q.tolist() == [[-127, 127, 0, 64]]  # 2 / (4/127) = 63.5 -> 64 (even)
+
+
+def test_int8_block_sums_against_python_integers():
+    rng = np.random.default_rng(5)
+    M, N, K, G = 3, 4, 256, 128
+    xq = rng.integers(-128, 128, (M, K)).astype(np.int8)
+    q = rng.integers(0, 16, (N, K)).astype(np.uint8)
+    zps = rng.integers(0, 16, (N, K // G)).astype(np.float32)
+    sums = O.int8_block_sums(xq, O.pack_int4(q), N, K, zps, O.WOQ_DTYPE_INT4, G, 128)
+    for m in range(M):
+        for n in range(N):
+            for kb in range(2):
+                want = sum(int(xq[m, k]) * (int(q[n, k]) - int(zps[n, k // G])) for k in range(kb * 128, kb * 128 + 128))
+                assert sums[m, n, kb] == want
+
+
+def test_int8_linear_epilogue_close_to_exact():
+    x, q, qw, scales, zps, b = _tiny_case(M=6, N=5, K=256, G=128, seed=7)
+    r = O.woq_linear_opt_int8(x, "bf16", qw, 5, 256, scales, zps, b, O.WOQ_DTYPE_INT4, 128, 6)
+    # against the unquantized product: int8 activations carry ~1/127 relative error per element
+    acc_exact, _ = O.woq_linear_ref(x, "bf16", qw, 5, 256, scales, zps, b, O.WOQ_DTYPE_INT4, 128, "fp32")
+    assert np.max(np.abs(r["acc"] - acc_exact)) < 0.1
+    # and exactly the definition when re-evaluated in float64 from the integer sums
+    sa = r["sa"].astype(np.float64).reshape(-1, 1)
+    want = b.astype(np.float64)[None, :] + sum(
+        r["sums"][:, :, kb].astype(np.float64) * sa * scales[:, kb].astype(np.float64)[None, :] for kb in range(2)
+    )
+    assert np.max(np.abs(r["acc"] - want)) < 1e-5
+
+
+def _awq_decode_independent(qweight, qzeros, scales, group_size):
+    """AutoAWQ GEMM packing, restated from its definition: word [k, j] holds column
+    8j + ORDER[i] in nibble i, ORDER = [0, 2, 4, 6, 1, 3, 5, 7]."""
+    order = [0, 2, 4, 6, 1, 3, 5, 7]
+    K, N8 = qweight.shape
+    w = np.zeros((K, N8 * 8), dtype=np.int64)
+    z = np.zeros((qzeros.shape[0], N8 * 8), dtype=np.int64)
+    qwu = qweight.astype(np.int64) & 0xFFFFFFFF
+    qzu = qzeros.astype(np.int64) & 0xFFFFFFFF
+    for i in range(8):
+        w[:, order[i]::8] = (qwu >> (4 * i)) & 0xF
+        z[:, order[i]::8] = (qzu >> (4 * i)) & 0xF
+    g = np.arange(K) // group_size
+    return ((w - z[g]) * scales[g].astype(np.float64)).T  # [N, K]
+
+
+def test_awq_fixture_decode():
+    p = os.path.join(GOLDEN, "awq_fixture.pt")
+    d = torch.load(p, weights_only=True)
+    qweight, qzeros, scales = d["qweight"].numpy(), d["qzeros"].numpy(), d["scales"].float().numpy()
+    want = _awq_decode_independent(qweight, qzeros, scales, 128)
+    # the product's converters + the oracle's dequantize must reproduce it
+    from ipex_amd.utils.weight_only_quantization import _convert_awq_scales_qzeros, awq_to_plain
+
+    plain = awq_to_plain(d["qweight"]).numpy()
+    s2, z2 = _convert_awq_scales_qzeros(d["scales"], d["qzeros"])
+    K, N = qweight.shape[0], qweight.shape[1] * 8
+    got = O.dequantize_woq_weight(plain, N, K, s2.float().numpy(), z2.float().numpy(), O.WOQ_DTYPE_INT4, 128)
+    assert np.max(np.abs(got - want)) < 1e-6
