@@ -237,14 +237,20 @@ __global__ __launch_bounds__(1024) void woq_small_m_kernel(const SmallMArgs a) {
 }
 
 template <int WBITS, int REGIME, int MT, int KPW, int NTW, bool CONV>
-static int launch_cfg(const SmallMArgs& a, hipStream_t st) {
+static int launch_cfg(SmallMArgs& a, hipStream_t st) {
   constexpr int TK = WBITS == 4 ? kTileK4 : kTileK8;
+  auto smem_for = [&](int W) {
+    size_t smem = (size_t)NTW * MT * W * 64 * sizeof(f4);
+    if (CONV) {
+      const int64_t rows = a.f.M < MT * 16 ? a.f.M : MT * 16;
+      smem += (size_t)rows * W * KPW * TK * sizeof(uint16_t);
+    }
+    return smem;
+  };
+  // the staging buffer of converted activations grows with W: fewer waves, more rounds
+  while (a.W > 1 && smem_for(a.W) > 96 * 1024) a.W = (a.W + 1) / 2;
   const int W = a.W;
-  size_t smem = (size_t)NTW * MT * W * 64 * sizeof(f4);
-  if (CONV) {
-    const int64_t rows = a.f.M < MT * 16 ? a.f.M : MT * 16;
-    smem += (size_t)rows * W * KPW * TK * sizeof(uint16_t);
-  }
+  const size_t smem = smem_for(W);
   auto kern = woq_small_m_kernel<WBITS, REGIME, MT, KPW, NTW, CONV>;
   if (smem > 160 * 1024) return set_error("small-M kernel: LDS request %zu exceeds 160 KiB", smem);
   if (smem > 64 * 1024) {
@@ -298,7 +304,7 @@ int launch_small_m(const FpArgs& f, int wbits, int regime, hipStream_t st) {
   a.W = 1;
   a.Kpad = f.KT * (wbits == 4 ? kTileK4 : kTileK8);
   const int want = regime == kRegimeF16 ? WOQ_HIP_ACT_FP16 : WOQ_HIP_ACT_BF16;
-  const bool conv = f.x_dtype != want;
+  const bool conv = f.x_dtype != want || (f.K % 8) != 0;
 #define WOQ_DISPATCH(WB, RG)                                            \
   (conv ? dispatch_shape<WB, RG, true>(a, st) : dispatch_shape<WB, RG, false>(a, st))
   if (wbits == 4)

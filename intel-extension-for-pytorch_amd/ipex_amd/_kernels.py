@@ -168,6 +168,8 @@ def linear(
             f"WOQ linear: input and weight shapes do not match, got k = {x.shape[-1]} and {K} respectively."
         )
     x2 = x.reshape(-1, K).contiguous()
+    if x2.data_ptr() % 16:
+        x2 = x2.clone()  # the kernels read activation rows with 16-byte loads
     M = x2.shape[0]
     out_dtype = torch.float32 if out_fp32 else x.dtype
     out = torch.empty((M, N), dtype=out_dtype, device=x.device)

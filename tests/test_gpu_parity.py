@@ -131,10 +131,22 @@ def _check_fp(case, lowp_mode, ctx=None, cols=None, force_kernel=0, label=""):
         y, acc = y[:, cols], acc[:, cols]
         N = len(cols)
     wd = case["weight_dtype"]
-    acc_ref, y_ref = O.woq_linear_ref(c["x"], "bf16", qw, N, K, sc, zp, b, wd, G, cd)
+    # The optimized kernels read the scales in the compute dtype (ContextLinearWoq.h:104-106) and
+    # so does the HIP path; the fallback keeps fp32 scales.  The fallback oracle is therefore
+    # evaluated with the scales rounded the same way (a no-op for fp16 / bf16 checkpoints), and
+    # the distance to the unrounded-scale fallback is reported.
+    sc_cd = O._round_to(sc, cd)
+    acc_ref, y_ref = O.woq_linear_ref(c["x"], "bf16", qw, N, K, sc_cd, zp, b, wd, G, cd)
     stats = {"max_abs_acc_vs_ref": max_abs(acc, acc_ref), "rel_l2_out_vs_ref": rel_l2(y, y_ref)}
+    if not np.array_equal(sc_cd, sc):
+        acc_f32s, _ = O.woq_linear_ref(c["x"], "bf16", qw, N, K, sc, zp, b, wd, G, cd)
+        stats["max_abs_acc_vs_ref_fp32_scales"] = max_abs(acc, acc_f32s)
     assert stats["max_abs_acc_vs_ref"] <= MAX_ABS_ACC, (label, stats)
-    assert stats["rel_l2_out_vs_ref"] <= REL_L2_OUT, (label, stats)
+    # fp16 regime: the HIP path follows the fallback's rounding chain (fp16 result, fp16 bias add,
+    # cast).  bf16 regime: it follows the optimized kernel (fp32 bias, one rounding), which the
+    # fallback's extra bf16 rounding of a biased result does not match to 2e-3.
+    if cd == "fp16" or b is None:
+        assert stats["rel_l2_out_vs_ref"] <= REL_L2_OUT, (label, stats)
     if cd == "bf16":
         acc_opt, y_opt = O.woq_linear_opt_bf16(c["x"], "bf16", qw, N, K, sc, zp, b, wd, G)
         stats["max_abs_acc_vs_opt"] = max_abs(acc, acc_opt)
@@ -144,7 +156,8 @@ def _check_fp(case, lowp_mode, ctx=None, cols=None, force_kernel=0, label=""):
         stats["out_exact_frac_vs_opt"] = float((ulps == 0).mean())
         assert stats["max_abs_acc_vs_opt"] <= MAX_ABS_ACC, (label, stats)
         assert stats["rel_l2_out_vs_opt"] <= REL_L2_OUT, (label, stats)
-        assert stats["out_ulp_max_vs_opt"] <= 1, (label, stats)
+        # one bf16 ulp at most, except next to zero where an ulp is far below the accumulator bar
+        assert bool(np.all((ulps <= 1) | (np.abs(y - y_opt) <= 1e-4))), (label, stats)
     elif wd == 2 and M <= 4 and N * K <= 4096 * 4096:
         # the optimized fp16 kernel accumulates in fp16; its own rounding noise exceeds 1e-2 at
         # these magnitudes, so only the relative-L2 bar applies against it
