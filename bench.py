@@ -44,6 +44,7 @@ def build_params(lib_mod, x, ctx, out, lowp_mode, act_quant_mode=-1, workspace=N
     p.scales_f16 = ctx.scales_list_[1].data_ptr()
     p.scales_bf16 = ctx.scales_list_[2].data_ptr()
     p.zeros_u8 = ctx.zeros_u8_.data_ptr() if ctx.zeros_u8_ is not None else None
+    p.scale_zero_f16x2 = ctx.scale_zero_f16x2_.data_ptr() if ctx.scale_zero_f16x2_ is not None else None
     p.group_size = ctx.group_size_
     p.bias = ctx.bias_f32_.data_ptr() if ctx.bias_f32_ is not None else None
     p.lowp_mode = lowp_mode
@@ -195,6 +196,7 @@ def main():
             c.at_weight_ = ctx0.at_weight_.clone()
             c.scales_list_ = [t.clone() for t in ctx0.scales_list_]
             c.zeros_u8_ = ctx0.zeros_u8_.clone()
+            c.scale_zero_f16x2_ = ctx0.scale_zero_f16x2_.clone()
         keep.append(c)
         p = build_params(_lib, x, c, out, 2)
         p.stream = stream.cuda_stream
@@ -239,7 +241,7 @@ def main():
             "unit": "GB/s",
             "frac": round(achieved / HBM_PEAK_GBS, 4),
             "traffic": None,
-            "kernel": "woq_small_m_kernel",
+            "kernel": "woq_decode_kernel",
             "us_per_launch_stream": round(us_launch, 3),
             "us_per_launch_graph": round(us_graph, 3),
             "us_per_launch_cache_resident": round(hot_ms * 1e3 / args.steps, 3),

@@ -121,18 +121,21 @@ int woq_hip_unpack_weight(const void* packed, int weight_dtype, int64_t N, int64
 /*
  * Quantization parameters -> kernel layout.
  *   scales: fp32 [N, KG] (KG = number of K groups; 1 for per-channel)
- *   zeros : fp32 [N, KG] or NULL (symmetric).  Must be integral, in [0,255] for 4-bit and
+ *   zeros : fp32 [N, KG] or NULL (symmetric).  Must be integral, in [0,127] for 4-bit and
  *           [-128,127] for 8-bit weights (checked by the host wrapper).
  * Outputs are laid out [Np/16][KG][16] (row-in-tile fastest):
  *   scales_f32 / scales_f16 / scales_bf16: the three roundings the reference keeps
  *   (ContextLinearWoq.h:104-106); zeros_u8: zero point as one byte, the value itself for
  *   4-bit weights and value + 128 for 8-bit weights (the same offset-binary shift as the
  *   weight bytes, so stored_weight - stored_zero == q - z in both cases).
+ *   scale_zero_f16x2 (may be NULL): one dword per (row, group) for the decode kernel, low half =
+ *   fp16 scale, high half = fp16 (128 + zero point) (symmetric 4-bit weights: 128 + 8); only
+ *   meaningful for 4-bit weights.
  * Padding rows get scale 1, zero 0 (LinearWoqPacked.cpp:344-361).
  */
 int woq_hip_pack_qparams(const float* scales, const float* zeros, int weight_dtype, int64_t N,
                          int64_t KG, float* scales_f32, void* scales_f16, void* scales_bf16,
-                         uint8_t* zeros_u8, void* stream);
+                         uint8_t* zeros_u8, uint32_t* scale_zero_f16x2, void* stream);
 
 /* zp[i][j] = (zp32[i][j/8] >> (4*(j%8))) & 0xf, written as fp32 [rows, cols]. */
 int woq_hip_unpack_int4_zeros(const int32_t* zp32, int64_t rows, int64_t cols,
@@ -165,6 +168,7 @@ typedef struct woq_hip_linear_params {
   const void* scales_f16;
   const void* scales_bf16;
   const uint8_t* zeros_u8; /* NULL: symmetric weights */
+  const uint32_t* scale_zero_f16x2; /* from woq_hip_pack_qparams; NULL disables the decode kernel */
   int64_t group_size;       /* <= 0: per output channel */
   const float* bias;        /* fp32 [N] or NULL */
 

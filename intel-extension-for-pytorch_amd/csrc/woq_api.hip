@@ -66,14 +66,14 @@ int woq_hip_unpack_weight(const void* packed, int weight_dtype, int64_t N, int64
 
 int woq_hip_pack_qparams(const float* scales, const float* zeros, int weight_dtype, int64_t N, int64_t KG,
                          float* scales_f32, void* scales_f16, void* scales_bf16, uint8_t* zeros_u8,
-                         void* stream) {
+                         uint32_t* scale_zero_f16x2, void* stream) {
   if (!valid_wdtype(weight_dtype)) return set_error("pack_qparams: unsupported weight dtype %d", weight_dtype);
   if (N < 0 || KG < 1) return set_error("pack_qparams: bad shape N=%lld KG=%lld", (long long)N, (long long)KG);
   if (N > 0 && (!scales || !scales_f32 || !scales_f16 || !scales_bf16))
     return set_error("pack_qparams: null scales pointer");
   if (zeros && !zeros_u8) return set_error("pack_qparams: zeros given but zeros_u8 is null");
   return launch_pack_qparams(scales, zeros, weight_dtype, N, KG, scales_f32, scales_f16, scales_bf16, zeros_u8,
-                             (hipStream_t)stream);
+                             scale_zero_f16x2, (hipStream_t)stream);
 }
 
 int woq_hip_unpack_int4_zeros(const int32_t* zp32, int64_t rows, int64_t cols, int64_t cols_zp32, float* out,
@@ -204,6 +204,8 @@ int woq_hip_linear(const woq_hip_linear_params* p) {
   f.other0 = p->others[0]; f.other1 = p->others[1]; f.out = p->out; f.out_dtype = p->out_dtype;
 
   int kernel = p->force_kernel;
+  if (kernel == 0 && decode_kernel_applies(f, wbits, regime, p->scale_zero_f16x2))
+    return launch_decode(f, p->scale_zero_f16x2, st);
   if (kernel == 0) kernel = p->M <= 64 ? 1 : 2;
   if (kernel == 1 && p->M > 64) return set_error("woq_linear: the small-M kernel takes M <= 64");
   return kernel == 1 ? launch_small_m(f, wbits, regime, st) : launch_gemm(f, wbits, regime, st);

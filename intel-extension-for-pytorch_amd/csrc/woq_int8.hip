@@ -216,19 +216,22 @@ __global__ __launch_bounds__(1024) void woq_small_m_i8_kernel(const Int8KArgs p)
       const int64_t nt = nt0 + t;
 #pragma unroll
       for (int i = 0; i < KPW; ++i) {
-        const int64_t kt = ktw + i;
-        wreg[t][i] = WBITS == 4 ? u4{0u, 0u, 0u, 0u} : u4{0x80808080u, 0x80808080u, 0x80808080u, 0x80808080u};
-        zreg[t][i] = WBITS == 4 ? 0 : 128;
-        if (nt < a.NT && kt < a.KT) {
-          wreg[t][i] = __builtin_nontemporal_load((const u4*)(a.qweight + ((nt * a.KT + kt) * 64 + lane) * 16));
-          if (a.zeros) {
-            int64_t g = (kt * TK + c * CK) / a.G;
-            if (g >= a.KG) g = a.KG - 1;
-            zreg[t][i] = a.zeros[(nt * a.KG + g) * kTileN + r];
-          } else {
-            zreg[t][i] = WBITS == 4 ? 8 : 128;
-          }
+        // unconditional loads from clamped indices; a clamped tile is replaced by the zero
+        // encoding (q == z) afterwards
+        const int64_t ktr = ktw + i;
+        const bool live = nt < a.NT && ktr < a.KT;
+        const int64_t ntc = nt < a.NT ? nt : a.NT - 1;
+        const int64_t kt = ktr < a.KT ? ktr : a.KT - 1;
+        const u4 wv = __builtin_nontemporal_load((const u4*)(a.qweight + ((ntc * a.KT + kt) * 64 + lane) * 16));
+        uint8_t zb = WBITS == 4 ? 8 : 128;
+        if (a.zeros) {
+          int64_t g = (kt * TK + c * CK) / a.G;
+          if (g >= a.KG) g = a.KG - 1;
+          zb = a.zeros[(ntc * a.KG + g) * kTileN + r];
         }
+        const uint32_t dead = WBITS == 4 ? 0u : 0x80808080u;
+        wreg[t][i] = live ? wv : u4{dead, dead, dead, dead};
+        zreg[t][i] = live ? zb : (uint8_t)(WBITS == 4 ? 0 : 128);
       }
     }
     i4 xb[KPW][STEPS][MT];
@@ -240,8 +243,9 @@ __global__ __launch_bounds__(1024) void woq_small_m_i8_kernel(const Int8KArgs p)
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) {
           const int64_t row = mt * 16 + r;
-          i4 v = i4{0, 0, 0, 0};
-          if (row < a.M && k < p.ldq) v = *(const i4*)(p.xq + row * p.ldq + k);
+          const bool ok = row < a.M && k < p.ldq;
+          const i4 v0 = *(const i4*)(p.xq + (row < a.M ? row : a.M - 1) * p.ldq + (k < p.ldq ? k : 0));
+          const i4 v = ok ? v0 : i4{0, 0, 0, 0};
           xb[i][j][mt] = v;
         }
       }

@@ -39,11 +39,30 @@ int launch_pack_weight(const void* plain, int weight_dtype, int64_t N, int64_t K
 int launch_unpack_weight(const void* packed, int weight_dtype, int64_t N, int64_t K, void* plain,
                          hipStream_t st);
 int launch_pack_qparams(const float* scales, const float* zeros, int weight_dtype, int64_t N, int64_t KG,
-                        float* s32, void* s16, void* sb16, uint8_t* z8, hipStream_t st);
+                        float* s32, void* s16, void* sb16, uint8_t* z8, uint32_t* sz, hipStream_t st);
 int launch_unpack_int4_zeros(const int32_t* zp32, int64_t rows, int64_t cols, int64_t cols_zp32,
                              float* out, hipStream_t st);
 int launch_dequant_weight(const void* qweight, int weight_dtype, int64_t N, int64_t K, const float* s32,
                           const uint8_t* z8, int64_t G, void* out, int out_dtype, hipStream_t st);
+
+// Arguments of the fp16-regime decode kernel (4-bit weights, groups that are multiples of 128).
+struct DecodeArgs {
+  const uint16_t* x;
+  int x_dtype;
+  int64_t M, K, N, NT, KT, Kpad;
+  const uint8_t* qweight;
+  const uint32_t* sz;  // [NT][KG][16]: fp16 scale | fp16 (128 + zero) << 16
+  int64_t G, KG;
+  const float* bias;
+  int fusion;
+  const void* other0;
+  const void* other1;
+  void* out;
+  int out_dtype;
+  int W;
+};
+bool decode_kernel_applies(const FpArgs& f, int wbits, int regime, const uint32_t* sz);
+int launch_decode(const FpArgs& f, const uint32_t* sz, hipStream_t st);
 
 // regime: 0 = fp16, 1 = bf16 (woq::Regime)
 int launch_small_m(const FpArgs& a, int wbits, int regime, hipStream_t st);

@@ -97,7 +97,8 @@ __global__ void unpack_int8_kernel(const uint8_t* __restrict__ packed, int8_t* _
 __global__ void pack_qparams_kernel(const float* __restrict__ scales, const float* __restrict__ zeros,
                                     int weight_dtype, int64_t N, int64_t Np, int64_t KG,
                                     float* __restrict__ s32, uint16_t* __restrict__ s16,
-                                    uint16_t* __restrict__ sb16, uint8_t* __restrict__ z8) {
+                                    uint16_t* __restrict__ sb16, uint8_t* __restrict__ z8,
+                                    uint32_t* __restrict__ sz) {
   const int64_t gid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (gid >= Np * KG) return;
   const int r = gid % kTileN;
@@ -116,6 +117,10 @@ __global__ void pack_qparams_kernel(const float* __restrict__ scales, const floa
     int zi = (int)z;
     if (weight_dtype == WOQ_HIP_DTYPE_INT8) zi += 128;
     z8[gid] = (uint8_t)zi;
+  }
+  if (sz) {
+    const float zz = 128.0f + (zeros ? z : (n < N ? 8.0f : 0.0f));
+    sz[gid] = (uint32_t)f32_to_f16_bits(s) | ((uint32_t)f32_to_f16_bits(zz) << 16);
   }
 }
 
@@ -206,13 +211,13 @@ int launch_unpack_weight(const void* packed, int weight_dtype, int64_t N, int64_
 }
 
 int launch_pack_qparams(const float* scales, const float* zeros, int weight_dtype, int64_t N, int64_t KG,
-                        float* s32, void* s16, void* sb16, uint8_t* z8, hipStream_t st) {
+                        float* s32, void* s16, void* sb16, uint8_t* z8, uint32_t* sz, hipStream_t st) {
   const int64_t Np = woq_hip_padded_n(N);
   const int64_t total = Np * KG;
   if (total == 0) return 0;
   pack_qparams_kernel<<<blocks_for(total, 256), 256, 0, st>>>(scales, zeros, weight_dtype, N, Np, KG, s32,
                                                               (uint16_t*)s16, (uint16_t*)sb16,
-                                                              zeros ? z8 : nullptr);
+                                                              zeros ? z8 : nullptr, sz);
   return check_launch("pack_qparams");
 }
 

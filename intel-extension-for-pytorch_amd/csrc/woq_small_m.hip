@@ -137,18 +137,20 @@ __global__ __launch_bounds__(1024) void woq_small_m_kernel(const SmallMArgs a) {
       const int64_t nt = nt0 + t;
 #pragma unroll
       for (int i = 0; i < KPW; ++i) {
-        const int64_t kt = ktw + i;
-        wreg[t][i] = u4{0u, 0u, 0u, 0u};
-        sreg[t][i] = 0;
-        zreg[t][i] = 0;
-        if (nt < f.NT && kt < f.KT) {
-          wreg[t][i] = __builtin_nontemporal_load((const u4*)(f.qweight + ((nt * f.KT + kt) * 64 + lane) * 16));
-          int64_t g = (kt * TK + c * CK) / f.G;
-          if (g >= f.KG) g = f.KG - 1;
-          const int64_t qi = (nt * f.KG + g) * kTileN + r;
-          sreg[t][i] = f.scales[qi];
-          if (f.zeros) zreg[t][i] = f.zeros[qi];
-        }
+        // unconditional loads from clamped indices: the compiler can then count outstanding
+        // loads and start on the first tile while the others are in flight; a zero scale
+        // cancels a clamped tile
+        const int64_t ktr = ktw + i;
+        const bool live = nt < f.NT && ktr < f.KT;
+        const int64_t ntc = nt < f.NT ? nt : f.NT - 1;
+        const int64_t kt = ktr < f.KT ? ktr : f.KT - 1;
+        wreg[t][i] = __builtin_nontemporal_load((const u4*)(f.qweight + ((ntc * f.KT + kt) * 64 + lane) * 16));
+        int64_t g = (kt * TK + c * CK) / f.G;
+        if (g >= f.KG) g = f.KG - 1;
+        const int64_t qi = (ntc * f.KG + g) * kTileN + r;
+        const uint16_t sb = f.scales[qi];
+        sreg[t][i] = live ? sb : (uint16_t)0;
+        zreg[t][i] = f.zeros ? f.zeros[qi] : (uint8_t)0;
       }
     }
 
@@ -178,13 +180,15 @@ __global__ __launch_bounds__(1024) void woq_small_m_kernel(const SmallMArgs a) {
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) {
           const int64_t row = mt * 16 + r;
-          u4 v = u4{0u, 0u, 0u, 0u};
-          if (row < f.M && k < f.K) {
-            if (CONV)
-              v = *(const u4*)(sx + row * KC + (k - kc0));
-            else
-              v = *(const u4*)((const uint16_t*)f.x + row * f.K + k);
-          }
+          const bool ok = row < f.M && k < f.K;
+          const int64_t rowc = row < f.M ? row : f.M - 1;
+          const int64_t kc = k < f.K ? k : 0;
+          u4 v;
+          if (CONV)
+            v = *(const u4*)(sx + (rowc < rows ? rowc : 0) * KC + (ok ? k - kc0 : 0));
+          else
+            v = *(const u4*)((const uint16_t*)f.x + rowc * f.K + kc);
+          v = ok ? v : u4{0u, 0u, 0u, 0u};
           xb[i][j][mt] = bitcast<vec8>(v);
         }
       }

@@ -63,7 +63,8 @@ def unpack_weight(packed, weight_dtype, N, K):
 
 
 def pack_qparams(scales, zeros, weight_dtype):
-    """scales / zeros: fp32 [N, KG] -> ([NT, KG, 16] fp32, fp16, bf16, uint8-or-None)."""
+    """scales / zeros: fp32 [N, KG] -> ([NT, KG, 16] fp32, fp16, bf16, uint8-or-None, packed
+    (fp16 scale, fp16 128 + zero) dwords-or-None)."""
     lib = _lib.load()
     _require_cuda(scales, "scales")
     scales = scales.to(torch.float32).contiguous()
@@ -78,14 +79,18 @@ def pack_qparams(scales, zeros, weight_dtype):
         zeros = zeros.to(torch.float32).contiguous()
         assert zeros.shape == scales.shape
         z8 = torch.empty((nt, KG, _lib.TILE_N), dtype=torch.uint8, device=dev)
+    sz = None
+    if weight_dtype != _lib.DTYPE_INT8:
+        sz = torch.empty((nt, KG, _lib.TILE_N), dtype=torch.int32, device=dev)
     with torch.cuda.device(dev):
         _lib.check(
             lib.woq_hip_pack_qparams(
-                _ptr(scales), _ptr(zeros), weight_dtype, N, KG, _ptr(s32), _ptr(s16), _ptr(sb16), _ptr(z8), _stream()
+                _ptr(scales), _ptr(zeros), weight_dtype, N, KG, _ptr(s32), _ptr(s16), _ptr(sb16), _ptr(z8), _ptr(sz),
+                _stream()
             ),
             "pack_qparams",
         )
-    return s32, s16, sb16, z8
+    return s32, s16, sb16, z8, sz
 
 
 def unpack_int4_zeros(zp32, cols):
@@ -150,6 +155,7 @@ def linear(
     bias_f32,
     lowp_mode,
     act_quant_mode,
+    scale_zero_f16x2=None,
     fusion=_lib.FUSE_NONE,
     others=(),
     out_fp32=False,
@@ -184,6 +190,7 @@ def linear(
     p.scales_f16 = scales_f16.data_ptr()
     p.scales_bf16 = scales_bf16.data_ptr()
     p.zeros_u8 = zeros_u8.data_ptr() if zeros_u8 is not None else None
+    p.scale_zero_f16x2 = scale_zero_f16x2.data_ptr() if scale_zero_f16x2 is not None else None
     p.group_size = group_size
     p.bias = bias_f32.data_ptr() if bias_f32 is not None else None
     p.lowp_mode = lowp_mode

@@ -52,6 +52,7 @@ class LinearParams(ctypes.Structure):
         ("scales_f16", ctypes.c_void_p),
         ("scales_bf16", ctypes.c_void_p),
         ("zeros_u8", ctypes.c_void_p),
+        ("scale_zero_f16x2", ctypes.c_void_p),
         ("group_size", ctypes.c_int64),
         ("bias", ctypes.c_void_p),
         ("lowp_mode", ctypes.c_int32),
@@ -102,7 +103,7 @@ def load():
         lib.woq_hip_unpack_weight.restype = i32
         lib.woq_hip_unpack_weight.argtypes = [vp, i32, i64, i64, vp, vp]
         lib.woq_hip_pack_qparams.restype = i32
-        lib.woq_hip_pack_qparams.argtypes = [vp, vp, i32, i64, i64, vp, vp, vp, vp, vp]
+        lib.woq_hip_pack_qparams.argtypes = [vp, vp, i32, i64, i64, vp, vp, vp, vp, vp, vp]
         lib.woq_hip_unpack_int4_zeros.restype = i32
         lib.woq_hip_unpack_int4_zeros.argtypes = [vp, i64, i64, i64, vp, vp]
         lib.woq_hip_dynamic_quant.restype = i32

@@ -51,7 +51,7 @@ def _to_gpu(t, device=None):
 
 
 def _check_integral_zeros(zeros, weight_dtype):
-    lo, hi = (-128, 127) if weight_dtype == _lib.DTYPE_INT8 else (0, 255)
+    lo, hi = (-128, 127) if weight_dtype == _lib.DTYPE_INT8 else (0, 127)
     z = zeros.to(torch.float32)
     ok = torch.equal(z, z.round()) and bool((z >= lo).all()) and bool((z <= hi).all())
     if not ok:
@@ -129,9 +129,10 @@ class WoqLinearOpContext:
         self.at_bias_ = _to_gpu(bias, dev)
         self.bias_f32_ = self.at_bias_.to(torch.float32).contiguous() if self.at_bias_ is not None else None
         self.at_weight_ = _kernels.pack_weight(weight, weight_dtype, N, K)
-        s32, s16, sb16, z8 = _kernels.pack_qparams(scales, zero_points, weight_dtype)
+        s32, s16, sb16, z8, sz = _kernels.pack_qparams(scales, zero_points, weight_dtype)
         self.scales_list_ = [s32, s16, sb16]
         self.zeros_u8_ = z8
+        self.scale_zero_f16x2_ = sz
         self.scales_plain_ = scales if group_size > 0 else scales.reshape(N)
         self.zero_points_plain_ = (
             None if zero_points is None else (zero_points if group_size > 0 else zero_points.reshape(N))
@@ -256,6 +257,7 @@ class WoqLinearOpContext:
             self.bias_f32_,
             self.lowp_mode_,
             self.act_quant_mode_,
+            scale_zero_f16x2=self.scale_zero_f16x2_,
             fusion=fusion,
             others=others,
             **kw,

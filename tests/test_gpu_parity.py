@@ -76,7 +76,7 @@ def test_qparams_layout(cuda):
     N, KG = 40, 3
     s = torch.rand(N, KG) + 0.5
     z = torch.randint(0, 16, (N, KG)).float()
-    s32, s16, sb16, z8 = k.pack_qparams(s.to(cuda), z.to(cuda), 2)
+    s32, s16, sb16, z8, sz = k.pack_qparams(s.to(cuda), z.to(cuda), 2)
     assert s32.shape == (3, KG, 16)
     sp = torch.ones(48, KG)
     sp[:N] = s
@@ -86,6 +86,10 @@ def test_qparams_layout(cuda):
     assert torch.equal(s16.cpu(), sp.view(3, 16, KG).permute(0, 2, 1).half())
     assert torch.equal(sb16.cpu(), sp.view(3, 16, KG).permute(0, 2, 1).bfloat16())
     assert torch.equal(z8.cpu().float(), zp.view(3, 16, KG).permute(0, 2, 1))
+    halves = sz.cpu().view(torch.float16).view(3, KG, 16, 2)
+    assert torch.equal(halves[..., 0], s16.cpu())
+    want_z = 128 + zp.view(3, 16, KG).permute(0, 2, 1)
+    assert torch.equal(halves[..., 1].float(), want_z)
 
 
 def test_compressed_zero_points(cuda):
