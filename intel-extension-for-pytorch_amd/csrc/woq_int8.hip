@@ -331,7 +331,7 @@ __global__ __launch_bounds__(1024) void woq_small_m_i8_kernel(const Int8KArgs p)
 constexpr int IBM = 128, IBN = 128, IBK = 128;
 constexpr int ILDS = IBK + 16;
 
-template <int WBITS>
+template <int WBITS, int BLOCK_K, bool PER_K, bool DEBUG>
 __global__ __launch_bounds__(256) void woq_gemm_i8_kernel(const Int8KArgs p) {
   constexpr int TK = WBITS == 4 ? kTileK4 : kTileK8;
   const Int8Args& a = p.a;
@@ -350,7 +350,21 @@ __global__ __launch_bounds__(256) void woq_gemm_i8_kernel(const Int8KArgs p) {
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
 
-  const int sub_blocks = (int)(IBK / p.block_k);  // block_k in {32, 64, 128}
+  constexpr int sub_blocks = IBK / BLOCK_K;  // BLOCK_K in {32, 64, 128}
+
+  // rows / columns of this lane's accumulator elements: m = mrow0 + 32 i + 8 (e / 4) + e % 4,
+  // n = ncol0 + 32 j
+  const int mrow0 = (int)m0 + wm * 64 + 4 * (lane >> 5);
+  const int ncol0 = (int)n0 + wn * 64 + (lane & 31);
+  // activation scales of those rows; constant over K unless the mode is per K block
+  float sa_reg[2][16];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) {
+      const int m = mrow0 + i * 32 + 8 * (e >> 2) + (e & 3);
+      sa_reg[i][e] = p.sa[(int64_t)(m < (int)a.M ? m : (int)a.M - 1) * p.sa_m_stride];
+    }
 
   for (int64_t k0 = 0; k0 < p.Kpad; k0 += IBK) {
     // activations: 128 rows x 128 bytes = 1024 x 16 B -> 4 per thread
@@ -419,6 +433,7 @@ __global__ __launch_bounds__(256) void woq_gemm_i8_kernel(const Int8KArgs p) {
     }
     __syncthreads();
 
+#pragma unroll
     for (int sb = 0; sb < sub_blocks; ++sb) {
       i16v qc[2][2];
 #pragma unroll
@@ -427,8 +442,9 @@ __global__ __launch_bounds__(256) void woq_gemm_i8_kernel(const Int8KArgs p) {
         for (int j = 0; j < 2; ++j)
 #pragma unroll
           for (int e = 0; e < 16; ++e) qc[i][j][e] = 0;
-      const int kbeg = sb * (int)p.block_k;
-      for (int ks = 0; ks < (int)p.block_k; ks += 32) {
+      const int kbeg = sb * BLOCK_K;
+#pragma unroll
+      for (int ks = 0; ks < BLOCK_K; ks += 32) {
         i4 af[2], bf[2];
 #pragma unroll
         for (int i = 0; i < 2; ++i) {
@@ -441,25 +457,36 @@ __global__ __launch_bounds__(256) void woq_gemm_i8_kernel(const Int8KArgs p) {
           for (int j = 0; j < 2; ++j)
             qc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[i], bf[j], qc[i][j], 0, 0, 0);
       }
-      // fp32 epilogue of this K block
-      const int64_t kq = k0 + kbeg;
-      const int64_t kb = kq / p.block_k;
-      int64_t g = kq / a.G;
-      if (g >= a.KG) g = a.KG - 1;
+      // fp32 epilogue of this K block: C += (float(qC) * s_a[m]) * s_w[n, g]
+      const int kq = (int)k0 + kbeg;
+      int g = (int)((unsigned)kq / (unsigned)a.G);
+      if (g >= (int)a.KG) g = (int)a.KG - 1;
+      if (PER_K) {
+        const int kcol = (int)((unsigned)kq / (unsigned)p.qbk);
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+          for (int e = 0; e < 16; ++e) {
+            const int m = mrow0 + i * 32 + 8 * (e >> 2) + (e & 3);
+            sa_reg[i][e] = p.sa[(int64_t)(m < (int)a.M ? m : (int)a.M - 1) * p.sa_m_stride + kcol];
+          }
+      }
 #pragma unroll
       for (int j = 0; j < 2; ++j) {
-        const int64_t n = n0 + wn * 64 + j * 32 + (lane & 31);
-        const float sw = n < a.NT * kTileN ? a.scales[((n / kTileN) * a.KG + g) * kTileN + (n % kTileN)] : 0.0f;
+        const int n = ncol0 + j * 32;  // < NT * 16 by construction of the grid? clamp below
+        const int nc = n < (int)a.NT * kTileN ? n : (int)a.NT * kTileN - 1;
+        const float sw = a.scales[((nc >> 4) * (int)a.KG + g) * kTileN + (nc & 15)];
 #pragma unroll
         for (int i = 0; i < 2; ++i) {
 #pragma unroll
           for (int e = 0; e < 16; ++e) {
-            const int64_t m = m0 + wm * 64 + i * 32 + 8 * (e >> 2) + 4 * (lane >> 5) + (e & 3);
-            const float sa = m < a.M ? p.sa[m * p.sa_m_stride + (kq / p.qbk) * p.sa_k_stride] : 0.0f;
-            const float cterm = __fmul_rn(__fmul_rn((float)qc[i][j][e], sa), sw);
+            const float cterm = __fmul_rn(__fmul_rn((float)qc[i][j][e], sa_reg[i][e]), sw);
             acc[i][j][e] = __fadd_rn(acc[i][j][e], cterm);
-            if (a.debug_block_sums && m < a.M && n < a.N)
-              a.debug_block_sums[(m * a.N + n) * (p.Kpad / p.block_k) + kb] = qc[i][j][e];
+            if (DEBUG) {
+              const int64_t m = mrow0 + i * 32 + 8 * (e >> 2) + (e & 3);
+              if (m < a.M && n < a.N)
+                a.debug_block_sums[(m * a.N + n) * (p.Kpad / BLOCK_K) + kq / BLOCK_K] = qc[i][j][e];
+            }
           }
         }
       }
@@ -563,10 +590,27 @@ int launch_int8_linear(const Int8Args& a, hipStream_t st) {
   if (a.M <= 64 && p.block_k % TK == 0)
     return a.wbits == 4 ? dispatch_small_i8<4>(p, st) : dispatch_small_i8<8>(p, st);
   dim3 grid((unsigned)((a.NT * kTileN + IBN - 1) / IBN), (unsigned)((a.M + IBM - 1) / IBM));
-  if (a.wbits == 4)
-    woq_gemm_i8_kernel<4><<<grid, 256, 0, st>>>(p);
-  else
-    woq_gemm_i8_kernel<8><<<grid, 256, 0, st>>>(p);
+  const bool dbg = a.debug_block_sums != nullptr;
+#define WOQ_I8_GEMM_B(WB, BK)                                                            \
+  if (dbg)                                                                               \
+    woq_gemm_i8_kernel<WB, BK, true, true><<<grid, 256, 0, st>>>(p);                     \
+  else if (per_k)                                                                        \
+    woq_gemm_i8_kernel<WB, BK, true, false><<<grid, 256, 0, st>>>(p);                    \
+  else                                                                                   \
+    woq_gemm_i8_kernel<WB, BK, false, false><<<grid, 256, 0, st>>>(p);
+#define WOQ_I8_GEMM(WB)                                   \
+  switch (p.block_k) {                                    \
+    case 32: { WOQ_I8_GEMM_B(WB, 32) } break;             \
+    case 64: { WOQ_I8_GEMM_B(WB, 64) } break;             \
+    default: { WOQ_I8_GEMM_B(WB, 128) } break;            \
+  }
+  if (a.wbits == 4) {
+    WOQ_I8_GEMM(4)
+  } else {
+    WOQ_I8_GEMM(8)
+  }
+#undef WOQ_I8_GEMM
+#undef WOQ_I8_GEMM_B
   return check_launch("woq_gemm_i8_kernel");
 }
 
