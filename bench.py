@@ -158,6 +158,9 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-prefill", action="store_true", help="skip the M=2048 measurement")
     ap.add_argument("--M", type=int, default=1, help="decode batch (1..16)")
+    ap.add_argument("--traffic-probe", action="store_true",
+                    help="short run for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE: a few decode launches plus a "
+                         "plain device copy of known size that calibrates the counter")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path; run with --gpus 1", file=sys.stderr)
@@ -203,6 +206,18 @@ def main():
         params.append(p)
 
     nbytes = algorithmic_bytes(M, K, N, G)
+    if args.traffic_probe:
+        # 64 launches over distinct weight copies, then one 256 MiB device-to-device copy kernel
+        for i in range(64):
+            lib.woq_hip_linear(ctypes.byref(params[i % len(params)]))
+        src = torch.empty(256 << 20, dtype=torch.uint8, device=dev)
+        dst = torch.empty_like(src)
+        torch.cuda.synchronize()
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"traffic_probe": True, "decode_launches": 64, "copy_bytes": 256 << 20,
+                          "algorithmic_bytes_per_launch": nbytes}))
+        return
     wall, ev_ms = time_steps(torch, lib, params, args.steps, args.warmup, stream)
     g_steps, g_wall, g_ev_ms = time_graph(torch, lib, params, args.steps, args.warmup)
     for p in params:

@@ -1,0 +1,246 @@
+"""Front-door tests on the GPU, modelled on the reference's own WOQ tests
+(tests/cpu/test_quantization_default_recipe.py:261-2227, tests/cpu/test_ipex_llm_quantization.py):
+build the module the way a user does, compare with matmul on the dequantized weight."""
+import copy
+import os
+import pickle
+
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+GOLDEN = os.path.join(os.path.dirname(__file__), "golden")
+
+
+def _ipex():
+    import ipex_amd
+
+    return ipex_amd
+
+
+@pytest.mark.parametrize("weight_dtype,group_size,lowp", [
+    ("INT8", -1, "NONE"), ("INT8", -1, "BF16"), ("INT4", -1, "BF16"), ("INT4", 128, "BF16"), ("INT4", 32, "BF16"),
+    ("INT4", 64, "FP16"), ("INT4", 128, "INT8"), ("INT8", -1, "INT8"),
+])
+@pytest.mark.parametrize("M", [1, 4, 33, 196])
+def test_prepare_convert_matches_dequantized_matmul(cuda, weight_dtype, group_size, lowp, M):
+    ipex = _ipex()
+    q = ipex.quantization
+    torch.manual_seed(0)
+    K, N = 512, 272
+    lin = torch.nn.Linear(K, N, bias=True).to(torch.bfloat16)
+    model = torch.nn.Sequential(lin).eval()
+    qmap = q.get_weight_only_quant_qconfig_mapping(
+        weight_dtype=getattr(q.WoqWeightDtype, weight_dtype),
+        lowp_mode=getattr(q.WoqLowpMode, lowp),
+        act_quant_mode=q.WoqActQuantMode.PER_BATCH_IC_BLOCK_SYM,
+        group_size=group_size,
+    )
+    w_float = lin.weight.detach().float().clone()
+    qmodel = q.convert(q.prepare(copy.deepcopy(model).to(cuda), qmap, inplace=True), inplace=True)
+    woq = qmodel[0]
+    assert type(woq).__name__ == "WeightOnlyQuantizedLinear"
+    assert woq.weight.is_cuda and woq.weight.dtype == torch.uint8
+    x = torch.randn(M, K).to(torch.bfloat16)
+    y = qmodel(x.to(cuda)).float().cpu()
+    # expected: quantize with the same helpers, dequantize, matmul in fp32
+    dt = getattr(q.WoqWeightDtype, weight_dtype)
+    sym = qmap.global_qconfig.weight_qscheme == q.WoqWeightQScheme.SYMMETRIC
+    if group_size == -1:
+        qw, s, z = q.quantize_per_channel(w_float, dt, None, None, sym)
+        dq = q.dequantize_per_channel(qw, s, z, dt, [N, K])
+    else:
+        qw, s, z = q.quantize_per_block(w_float, dt, group_size, None, None, sym)
+        dq = q.dequantize_per_block(qw, s, z, dt, group_size, [N, K])
+    ref = x.float() @ dq.t() + lin.bias.float()
+    tol = 5e-2 if lowp == "INT8" else 2e-2
+    assert torch.allclose(y, ref, atol=tol, rtol=2e-2), float((y - ref).abs().max())
+    # context accessors return the un-permuted, un-padded parameters and the plain weight
+    ctx = woq._op_context
+    assert torch.equal(ctx.to_public(ctx.get_weight()).cpu(), qw)
+    assert torch.equal(ctx.get_scales().cpu(), s.float())
+    assert ctx.get_weight_shape() == [N, K]
+    if z is not None:
+        assert torch.equal(ctx.get_zero_points().cpu(), z.float())
+
+
+def test_all_zero_bias_is_dropped_and_weight_emptied(cuda):
+    ipex = _ipex()
+    q = ipex.quantization
+    lin = torch.nn.Linear(256, 64, bias=True).to(cuda)
+    with torch.no_grad():
+        lin.bias.zero_()
+    lin.qconfig = q.get_weight_only_quant_qconfig_mapping(weight_dtype=q.WoqWeightDtype.INT4).global_qconfig
+    woq = ipex.nn.modules.WeightOnlyQuantizedLinear.from_float(lin)
+    assert woq.bias is False and woq._op_context.get_bias() is None
+    assert lin.weight.numel() == 0
+
+
+def test_awq_fixture_through_llm_front_door(cuda):
+    """The reference's own AutoAWQ tensors (tests/cpu/test_ipex_llm_quantization.py:112-151),
+    checked against an independent decode at the reference's precision (0.1) and tighter."""
+    ipex = _ipex()
+    d = torch.load(os.path.join(GOLDEN, "awq_fixture.pt"), weights_only=True)
+    K, N, G = 768, 2304, 128
+    order = [0, 2, 4, 6, 1, 3, 5, 7]
+    qw = d["qweight"].numpy().astype(np.int64) & 0xFFFFFFFF
+    qz = d["qzeros"].numpy().astype(np.int64) & 0xFFFFFFFF
+    w = np.zeros((K, N), dtype=np.int64)
+    z = np.zeros((K // G, N), dtype=np.int64)
+    for i in range(8):
+        w[:, order[i]::8] = (qw >> (4 * i)) & 0xF
+        z[:, order[i]::8] = (qz >> (4 * i)) & 0xF
+    sc = d["scales"].float().numpy()
+    g = np.arange(K) // G
+    dq = ((w - z[g]) * sc[g]).astype(np.float32)  # [K, N]
+    act = d["act"]
+    ref = act.float().numpy() @ dq + d["bias"].float().numpy()
+    lm = ipex.llm.quantization
+    lin = lm.IPEXWeightOnlyQuantizedLinear.from_weight(
+        d["qweight"], d["scales"], d["qzeros"], K, N, None, d["bias"], G, None, lm.QuantMethod.AWQ_GEMM,
+        lm.QuantDtype.INT4,
+    )
+    y = lin(act.to(cuda)).float().cpu().numpy()
+    assert np.max(np.abs(y - ref)) < 0.1
+    assert np.linalg.norm(y - ref) / np.linalg.norm(ref) < 4e-3  # bf16 weights + bf16 output rounding
+
+
+def test_gptq_checkpoint_through_llm_front_door(cuda):
+    ipex = _ipex()
+    gen = torch.Generator().manual_seed(3)
+    K, N, G = 512, 256, 128
+    q = torch.randint(0, 16, (K, N), generator=gen)  # [K, N]
+    zp = torch.randint(0, 16, (K // G, N), generator=gen)
+    scales = (0.005 + 0.015 * torch.rand(K // G, N, generator=gen)).half()
+    qv = q.view(K // 8, 8, N)
+    qweight = torch.zeros(K // 8, N, dtype=torch.int64)
+    for i in range(8):
+        qweight |= qv[:, i, :] << (4 * i)
+    qweight = (qweight - (qweight >= 2**31) * 2**32).to(torch.int32)
+    zv = ((zp - 1) % 16).view(K // G, N // 8, 8)
+    qzeros = torch.zeros(K // G, N // 8, dtype=torch.int64)
+    for i in range(8):
+        qzeros |= zv[:, :, i] << (4 * i)
+    qzeros = (qzeros - (qzeros >= 2**31) * 2**32).to(torch.int32)
+    lm = ipex.llm.quantization
+    lin = lm.IPEXWeightOnlyQuantizedLinear.from_weight(qweight, scales, qzeros, K, N, None, None, G)
+    x = torch.randn(7, K, generator=gen).to(torch.bfloat16)
+    y = lin(x.to(cuda)).float().cpu()
+    gidx = torch.arange(K) // G
+    dq = (q - zp[gidx]).float() * scales.float()[gidx]
+    ref = x.float() @ dq
+    assert torch.allclose(y, ref, atol=3e-2, rtol=2e-2)
+
+
+def test_context_pickle_roundtrip(cuda):
+    from ipex_amd.utils import synthetic
+    from helpers import make_context
+
+    case = synthetic.make_int4_case(30, 3, 512, 80, 128, bias=True)
+    ctx = make_context(case, 2)
+    x = case["x"].to(cuda)
+    y0 = ctx.run(x)
+    ctx2 = pickle.loads(pickle.dumps(ctx))
+    assert torch.equal(ctx2.run(x), y0)
+    assert torch.equal(ctx2.to_public(ctx2.get_weight()).cpu(), case["qweight"])
+    assert ctx2.get_data_handle().item() != ctx.get_data_handle().item()
+
+
+def test_stale_handle_raises(cuda):
+    from ipex_amd.utils import synthetic
+    from helpers import make_context
+
+    case = synthetic.make_int4_case(31, 1, 256, 32, 128)
+    ctx = make_context(case, 2)
+    handle = ctx.get_data_handle()
+    x = case["x"].to(cuda)
+    torch.ops.torch_ipex.ipex_woq_linear(x, handle)
+    del ctx
+    with pytest.raises(RuntimeError, match="no longer exists"):
+        torch.ops.torch_ipex.ipex_woq_linear(x, handle)
+    with pytest.raises(RuntimeError, match="GPU"):
+        torch.ops.torch_ipex.ipex_woq_linear(x.cpu(), handle)
+
+
+def test_context_free_op_matches_module(cuda):
+    """ipex_prepack::woq_linear_pack_weight -> unpack round trip and torch_ipex::woq_linear
+    (tests/cpu/test_quantization_default_recipe.py:1805-1901)."""
+    from ipex_amd.utils import synthetic
+    from helpers import make_context
+
+    for lowp, M in ((2, 3), (2, 20), (3, 9)):
+        case = synthetic.make_int4_case(32, M, 512, 96, 128, bias=True)
+        ctx = make_context(case, lowp, 6 if lowp == 3 else -1)
+        x = case["x"].to(cuda)
+        packed, scales, zeros, bias, comp = torch.ops.ipex_prepack.woq_linear_pack_weight(
+            case["qweight"].to(cuda), "int4", [96, 512], case["scales"].to(cuda), case["zeros"].to(cuda),
+            case["bias"].to(cuda), None, 128, lowp,
+        )
+        back = torch.ops.ipex_prepack.woq_linear_unpack_weight(packed, "int4", [96, 512], lowp)
+        assert torch.equal(back.cpu(), case["qweight"])
+        y = torch.ops.torch_ipex.woq_linear(
+            x, packed, "int4", [96, 512], scales, zeros, bias, None, 128, lowp, 6 if lowp == 3 else -1, comp
+        )
+        want = ctx.run(x)
+        # the context-free op has no decode-kernel parameters, so M < 5 takes the general kernel
+        assert torch.allclose(y.float(), want.float(), atol=2e-2, rtol=1e-2)
+    with pytest.raises(RuntimeError, match="Unsupported weight dtype"):
+        torch.ops.torch_ipex.woq_linear(x, packed, "int3", [96, 512], scales, zeros, bias, None, 128, 2, -1, None)
+
+
+def test_k_mismatch_and_bad_arguments(cuda):
+    from ipex_amd import ops
+    from ipex_amd.utils import synthetic
+    from helpers import make_context
+
+    case = synthetic.make_int4_case(33, 2, 256, 32, 128)
+    ctx = make_context(case, 2)
+    with pytest.raises(RuntimeError, match="input and weight shapes do not match"):
+        ctx.run(torch.zeros(2, 128, dtype=torch.bfloat16, device=cuda))
+    with pytest.raises(RuntimeError, match="zero points must be integers"):
+        ops.WoqLinearOpContext(case["qweight"].to(cuda), 2, [32, 256], case["scales"].to(cuda),
+                               case["zeros"].to(cuda) + 0.5, None, None, None, 128, 2, -1)
+    with pytest.raises(RuntimeError, match="g_idx"):
+        ops.WoqLinearOpContext(case["qweight"].to(cuda), 2, [32, 256], case["scales"].to(cuda),
+                               case["zeros"].to(cuda), None, torch.zeros(256, dtype=torch.int32), None, 128, 2, -1)
+    with pytest.raises(RuntimeError, match="symmetric quantization is required"):
+        ops.WoqLinearOpContext(torch.zeros(32, 256, dtype=torch.int8, device=cuda), 1, [32, 256],
+                               torch.ones(32, device=cuda), torch.zeros(32, device=cuda), None, None, None, -1, 3, 6)
+
+
+def test_weight_cache_for_large_batch(cuda):
+    """cache_weight_for_large_batch: M >= 64 runs a plain bf16 GEMM on a cached dequantized weight
+    and must agree with the uncached path (tests/cpu/test_quantization_default_recipe.py:1522-1579)."""
+    from ipex_amd.utils import synthetic
+    from helpers import make_context
+
+    case = synthetic.make_int4_case(34, 80, 512, 144, 128, bias=True)
+    x = case["x"].to(cuda)
+    y_plain = make_context(case, 2).run(x)
+    cached = make_context(case, 2, cache=True)
+    y_cached = cached.run(x)
+    assert cached.get_cached_weight() is not None and cached.get_cached_weight().dtype == torch.bfloat16
+    assert torch.allclose(y_cached.float(), y_plain.float(), atol=6e-2, rtol=2e-2)
+    # small batches do not touch the cache
+    cached2 = make_context(case, 2, cache=True)
+    cached2.run(x[:8])
+    assert cached2.get_cached_weight() is None
+
+
+def test_fused_ops_through_torch_ops(cuda):
+    from ipex_amd.utils import synthetic
+    from helpers import make_context
+
+    case = synthetic.make_int4_case(35, 6, 256, 48, 128, bias=True)
+    ctx = make_context(case, 2)
+    h = ctx.get_data_handle()
+    x = case["x"].to(cuda)
+    base = torch.ops.torch_ipex.ipex_woq_linear(x, h)
+    o = torch.randn(6, 48, device=cuda).bfloat16()
+    assert torch.equal(torch.ops.torch_ipex.woq_linear_add(x, h, [o]), (base.float() + o.float()).bfloat16())
+    assert torch.equal(torch.ops.torch_ipex.woq_linear_mul(x, h, [o]), (base.float() * o.float()).bfloat16())
+    assert torch.equal(torch.ops.torch_ipex.woq_linear_relu(x, h), torch.relu(base))
+    got = torch.ops.torch_ipex.woq_linear_silu(x, h)
+    assert torch.allclose(got.float(), torch.nn.functional.silu(base.float()), atol=2e-2, rtol=2e-2)
