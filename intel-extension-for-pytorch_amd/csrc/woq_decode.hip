@@ -48,18 +48,21 @@ __device__ __forceinline__ f4 mfma16(u4 a, u4 b, f4 c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_bf16(bitcast<b8>(a), bitcast<b8>(b), c, 0, 0, 0);
 }
 
-template <bool XF16, int NTW, int MAXM>
+template <bool XF16, int NTW, int MAXM, bool ONE_ROUND>
 __global__ __launch_bounds__(1024, 8) void woq_decode_kernel(const DecodeArgs a) {
   constexpr int KPW = kDecodeKPW;
   constexpr int SLICE = KPW * kTileK4;  // K elements of one wave per round
   extern __shared__ __align__(16) uint8_t smem[];
   const int W = a.W;
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63;
+  // the wave index is uniform: keeping it in an SGPR moves the tile / group address arithmetic to
+  // the scalar unit and leaves one VGPR offset per stream
+  const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
   const int r = lane & 15, c = lane >> 4;
   const int64_t nt0 = (int64_t)blockIdx.x * NTW;
 
   uint16_t* sx = (uint16_t*)smem + (size_t)wave * MAXM * SLICE;            // private [MAXM][SLICE]
-  f4* red = (f4*)(smem + (size_t)W * MAXM * SLICE * sizeof(uint16_t));     // [NTW][W][64]
+  f4* red = (f4*)(smem + (size_t)W * MAXM * SLICE * sizeof(uint16_t));     // [NTW][W][16]
 
   uint32_t mask, magic;
   asm volatile("s_mov_b32 %0, 0x000F000F" : "=s"(mask));
@@ -75,72 +78,80 @@ __global__ __launch_bounds__(1024, 8) void woq_decode_kernel(const DecodeArgs a)
   for (int t = 0; t < NTW; ++t) acc[t] = f4{0.f, 0.f, 0.f, 0.f};
 
   const int NT = (int)a.NT, KT = (int)a.KT, KG = (int)a.KG;
-  const int tpg = (int)(a.G / kTileK4);  // tiles per group
+  const int tpg_shift = a.tpg_shift;  // log2(tiles per group)
   const int xlane = lane & (KPW * 16 - 1);  // lanes 32..63 mirror 0..31
+  (void)NT;
   const int xrow = r < MAXM ? r : 0;
 
   // 32-bit offsets from uniform base pointers keep the per-lane address state in one VGPR each
   // (the packed weight, its parameters and the activations are each far below 4 GiB)
   const int K = (int)a.K, M = (int)a.M;
-  const int rounds = (KT + W * KPW - 1) / (W * KPW);
+  // ONE_ROUND: the W waves cover K exactly once (K == W * KPW * 128), the common decode case
+  const int rounds = ONE_ROUND ? 1 : (KT + W * KPW - 1) / (W * KPW);
+#pragma unroll 1
   for (int rd = 0; rd < rounds; ++rd) {
     const int ktw = (rd * W + wave) * KPW;
+    // The launcher guarantees K % (KPW * 128) == 0 and NT % NTW == 0, so a wave either has a
+    // full slice of work or none: no clamped addresses, no selects between the loads.
+    if (!ONE_ROUND && ktw >= KT) break;
 
     // ---- this wave's slice of the activations: issued first, so it is the first to return ----
     u4 xs[MAXM];
-    {
-      const int k = ktw * kTileK4 + xlane * 8;
-      const int kk = k < K ? k : 0;
+    const uint8_t* xbase = (const uint8_t*)a.x + (size_t)ktw * kTileK4 * 2;  // uniform
 #pragma unroll
-      for (int m = 0; m < MAXM; ++m) {
-        const int mm = m < M ? m : M - 1;
-        const u4 v = *(const u4*)((const uint8_t*)a.x + (uint32_t)(mm * K + kk) * 2u);
-        xs[m] = k < K ? v : u4{0u, 0u, 0u, 0u};
-      }
+    for (int m = 0; m < MAXM; ++m) {
+      const int mm = m < M ? m : M - 1;
+      xs[m] = *(const u4*)(xbase + (size_t)mm * K * 2 + (uint32_t)xlane * 16u);
     }
 
-    // ---- the weight stream of this round: one KiB tile per load, all in flight together ----
+    // ---- the weight stream of this round, in the order it is consumed: one KiB tile per load,
+    // all in flight together; uniform bases + one per-lane offset ----
     u4 wreg[NTW][KPW];
     uint32_t szreg[NTW][KPW];
 #pragma unroll
-    for (int t = 0; t < NTW; ++t) {
+    for (int i = 0; i < KPW; ++i) {
+      const int kt = ktw + i;
+      int g = kt >> tpg_shift;
+      g = g < KG ? g : KG - 1;
 #pragma unroll
-      for (int i = 0; i < KPW; ++i) {
-        int nt = (int)nt0 + t, kt = ktw + i;
-        const bool live = nt < NT && kt < KT;
-        nt = nt < NT ? nt : NT - 1;
-        kt = kt < KT ? kt : KT - 1;
-        wreg[t][i] = __builtin_nontemporal_load((const u4*)(a.qweight + (uint32_t)((nt * KT + kt) * 64 + lane) * 16u));
-        int g = tpg == 1 ? kt : (int)((unsigned)kt / (unsigned)tpg);
-        g = g < KG ? g : KG - 1;
-        const uint32_t sz = *(const uint32_t*)((const uint8_t*)a.sz + (uint32_t)((nt * KG + g) * kTileN + r) * 4u);
-        szreg[t][i] = live ? sz : 0u;  // scale 0 cancels a clamped tile
+      for (int t = 0; t < NTW; ++t) {
+        const size_t nt = (size_t)nt0 + t;
+        const uint8_t* wb = a.qweight + (nt * KT + kt) * kTileBytes;                      // uniform
+        const uint8_t* sb = (const uint8_t*)a.sz + (nt * KG + g) * (kTileN * sizeof(uint32_t));  // uniform
+        wreg[t][i] = __builtin_nontemporal_load((const u4*)(wb + (uint32_t)lane * 16u));
+        szreg[t][i] = *(const uint32_t*)(sb + (uint32_t)r * 4u);
       }
     }
 
+    // Every load of the round stays ahead of the first use: the scheduler would otherwise sink
+    // some of them below the first s_waitcnt to save registers, exposing a full memory round
+    // trip in the middle of the round.
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int m = 0; m < MAXM; ++m) *(u4*)(sx + m * SLICE + xlane * 8) = xs[m];
 
 #pragma unroll
     for (int i = 0; i < KPW; ++i) {
-      u4 xa[4];
-#pragma unroll
-      for (int j = 0; j < 4; ++j) xa[j] = *(const u4*)(sx + xrow * SLICE + i * kTileK4 + c * 32 + j * 8);
+      // -sum_k x of this K tile (shared by the NTW weight tiles)
       f4 d1 = f4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int j = 0; j < 4; ++j) d1 = mfma16<XF16>(xa[j], neg1, d1);
+      for (int j = 0; j < 4; ++j) {
+        const u4 xa = *(const u4*)(sx + xrow * SLICE + i * kTileK4 + c * 32 + j * 8);
+        d1 = mfma16<XF16>(xa, neg1, d1);
+      }
 #pragma unroll
       for (int t = 0; t < NTW; ++t) {
         f4 dw = f4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
+          const u4 xa = *(const u4*)(sx + xrow * SLICE + i * kTileK4 + c * 32 + j * 8);
           const uint32_t d = wreg[t][i][j];
           u4 bop;
           bop[0] = v_and_or(d, mask, magic);
           bop[1] = v_and_or(d >> 4, mask, magic);
           bop[2] = v_and_or(d >> 8, mask, magic);
           bop[3] = v_and_or(d >> 12, mask, magic);
-          dw = mfma16<XF16>(xa[j], bop, dw);
+          dw = mfma16<XF16>(xa, bop, dw);
         }
         // dw = sum x (c + q), d1 = -sum x;  group term = s * (dw + (128 + z) * d1 [+ 896 * d1])
 #pragma unroll
@@ -155,39 +166,41 @@ __global__ __launch_bounds__(1024, 8) void woq_decode_kernel(const DecodeArgs a)
   }
 
   // ---- combine the waves' partial sums in wave order, then bias / rounding / store ----
+  // Only lanes 0..15 hold rows m = 0..3 (M <= 4); they publish their four accumulators.
+  if (c == 0) {
 #pragma unroll
-  for (int t = 0; t < NTW; ++t) red[(t * W + wave) * 64 + lane] = acc[t];
+    for (int t = 0; t < NTW; ++t) red[(t * W + wave) * 16 + r] = acc[t];
+  }
   __syncthreads();
 
   Epilogue ep{a.bias, a.fusion, a.other0, a.other1, a.out, a.out_dtype, a.x_dtype, a.N};
+  const float* redf = (const float*)red;
+  // one thread per output element (tile, column, row); its W <= 16 partial sums are fetched with
+  // independent LDS reads (a rolled loop would pay one LDS round trip per wave) and added in wave
+  // order
   for (int idx = threadIdx.x; idx < NTW * 64; idx += blockDim.x) {
-    const int ln = idx & 63, t = idx >> 6;
-    const int64_t m0 = 4 * (ln >> 4);
-    const int64_t n = (nt0 + t) * kTileN + (ln & 15);
-    if (m0 >= a.M || n >= a.N) continue;
-    f4 s = red[(t * W) * 64 + ln];
-    for (int w = 1; w < W; ++w) {
-      const f4 v = red[(t * W + w) * 64 + ln];
-      s[0] += v[0];
-      s[1] += v[1];
-      s[2] += v[2];
-      s[3] += v[3];
-    }
-    // one copy of the generic epilogue (bias, post-ops, output dtype): it runs on a handful of
-    // lanes once per workgroup, so the loop is kept rolled to keep the kernel small
-#pragma unroll 1
-    for (int e = 0; e < 4; ++e) {
-      const float v = e == 0 ? s[0] : (e == 1 ? s[1] : (e == 2 ? s[2] : s[3]));
-      if (m0 + e < a.M) epilogue_store<kRegimeF16>(ep, m0 + e, n, v);
-    }
+    const int e = idx & 3, col = (idx >> 2) & 15, t = idx >> 6;
+    const int64_t n = (nt0 + t) * kTileN + col;
+    if (e >= M || n >= a.N) continue;
+    float part[16];
+#pragma unroll
+    for (int w = 0; w < 16; ++w) part[w] = w < W ? redf[((t * W + w) * 16 + col) * 4 + e] : 0.0f;
+    float s = part[0];
+#pragma unroll
+    for (int w = 1; w < 16; ++w) s += part[w];
+    // plain case first: bf16 in / out, no bias, no post-op -> fp16 rounding then bf16 store
+    if (a.fusion == WOQ_HIP_FUSE_NONE && a.bias == nullptr && a.out_dtype == WOQ_HIP_ACT_BF16)
+      ((uint16_t*)a.out)[(int64_t)e * a.N + n] = f32_to_bf16_bits((float)(_Float16)s);
+    else
+      epilogue_store<kRegimeF16>(ep, e, n, s);
   }
 }
 
-template <bool XF16, int NTW, int MAXM>
+template <bool XF16, int NTW, int MAXM, bool ONE_ROUND>
 static int launch_decode_cfg(const DecodeArgs& a, hipStream_t st) {
-  const size_t smem = (size_t)NTW * a.W * 64 * sizeof(f4) +
+  const size_t smem = (size_t)NTW * a.W * 16 * sizeof(f4) +
                       (size_t)a.W * MAXM * kDecodeKPW * kTileK4 * sizeof(uint16_t);
-  auto kern = woq_decode_kernel<XF16, NTW, MAXM>;
+  auto kern = woq_decode_kernel<XF16, NTW, MAXM, ONE_ROUND>;
   if (smem > 64 * 1024) {
     hipError_t err = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
     if (err != hipSuccess) return set_error("hipFuncSetAttribute: %s", hipGetErrorString(err));
@@ -198,8 +211,9 @@ static int launch_decode_cfg(const DecodeArgs& a, hipStream_t st) {
 }
 
 bool decode_kernel_applies(const FpArgs& f, int wbits, int regime, const uint32_t* sz) {
+  const int64_t tpg = f.G / kTileK4;
   return sz != nullptr && wbits == 4 && regime == kRegimeF16 && f.M <= 4 && (f.G % kTileK4) == 0 &&
-         (f.K % 8) == 0 && (f.x_dtype == WOQ_HIP_ACT_BF16 || f.x_dtype == WOQ_HIP_ACT_FP16);
+         (tpg & (tpg - 1)) == 0 && (f.K % (kDecodeKPW * kTileK4)) == 0 && (f.x_dtype == WOQ_HIP_ACT_BF16 || f.x_dtype == WOQ_HIP_ACT_FP16);
 }
 
 int launch_decode(const FpArgs& f, const uint32_t* sz, hipStream_t st) {
@@ -213,6 +227,8 @@ int launch_decode(const FpArgs& f, const uint32_t* sz, hipStream_t st) {
   a.bias = f.bias; a.fusion = f.fusion; a.other0 = f.other0; a.other1 = f.other1;
   a.out = f.out; a.out_dtype = f.out_dtype;
   a.Kpad = f.KT * kTileK4;
+  a.tpg_shift = 0;
+  while ((int64_t)kTileK4 << (a.tpg_shift + 1) <= f.G && a.tpg_shift < 30) ++a.tpg_shift;
   // waves per workgroup: cover K in as few equal rounds as possible, at most 16 waves
   int64_t w = (f.KT + kDecodeKPW - 1) / kDecodeKPW;
   if (w > 16) {
@@ -221,10 +237,12 @@ int launch_decode(const FpArgs& f, const uint32_t* sz, hipStream_t st) {
   }
   a.W = (int)w;
   const bool xf16 = f.x_dtype == WOQ_HIP_ACT_FP16;
-  const bool two = f.NT >= 512;
+  const bool two = f.NT >= 512 && f.NT % 2 == 0;
   const bool one_row = f.M == 1;
-#define WOQ_DECODE(XF, NTW) \
-  (one_row ? launch_decode_cfg<XF, NTW, 1>(a, st) : launch_decode_cfg<XF, NTW, 4>(a, st))
+  const bool one_round = f.KT == (int64_t)a.W * kDecodeKPW;
+#define WOQ_DECODE(XF, NTW)                                                                             \
+  (one_row ? (one_round ? launch_decode_cfg<XF, NTW, 1, true>(a, st) : launch_decode_cfg<XF, NTW, 1, false>(a, st)) \
+           : (one_round ? launch_decode_cfg<XF, NTW, 4, true>(a, st) : launch_decode_cfg<XF, NTW, 4, false>(a, st)))
   if (xf16) return two ? WOQ_DECODE(true, 2) : WOQ_DECODE(true, 1);
   return two ? WOQ_DECODE(false, 2) : WOQ_DECODE(false, 1);
 #undef WOQ_DECODE

@@ -60,6 +60,7 @@ struct DecodeArgs {
   void* out;
   int out_dtype;
   int W;
+  int tpg_shift;  // log2(G / 128)
 };
 bool decode_kernel_applies(const FpArgs& f, int wbits, int regime, const uint32_t* sz);
 int launch_decode(const FpArgs& f, const uint32_t* sz, hipStream_t st);
