@@ -192,7 +192,8 @@ typedef struct woq_hip_linear_params {
    * (m, n, K-block) as int32 [M, N, Kp/block_k] (tests only, small shapes) */
   int32_t* debug_block_sums;
 
-  /* force_kernel: 0 = automatic; 1 = small-M streaming kernel; 2 = tiled MFMA GEMM */
+  /* force_kernel: 0 = automatic; 1 = small-M streaming kernel; 2 = tiled MFMA GEMM (any shape);
+   * 3 = 4-bit prefill GEMM (K % 128 == 0, power-of-two or per-channel groups, x in the compute dtype) */
   int32_t force_kernel;
 
   void* stream;

@@ -206,9 +206,13 @@ int woq_hip_linear(const woq_hip_linear_params* p) {
   int kernel = p->force_kernel;
   if (kernel == 0 && decode_kernel_applies(f, wbits, regime, p->scale_zero_f16x2))
     return launch_decode(f, p->scale_zero_f16x2, st);
-  if (kernel == 0) kernel = p->M <= 64 ? 1 : 2;
+  if (kernel == 0) kernel = p->M <= 64 ? 1 : (gemm_w4_applies(f, wbits, regime) ? 3 : 2);
   if (kernel == 1 && p->M > 64) return set_error("woq_linear: the small-M kernel takes M <= 64");
-  return kernel == 1 ? launch_small_m(f, wbits, regime, st) : launch_gemm(f, wbits, regime, st);
+  if (kernel == 3 && !gemm_w4_applies(f, wbits, regime))
+    return set_error("woq_linear: the 4-bit prefill kernel takes 4-bit weights, K %% 128 == 0, a power-of-two or "
+                     "per-channel group size and activations in the compute dtype");
+  if (kernel == 1) return launch_small_m(f, wbits, regime, st);
+  return kernel == 3 ? launch_gemm_w4(f, regime, st) : launch_gemm(f, wbits, regime, st);
 }
 
 int woq_hip_dequant_weight(const void* qweight, int weight_dtype, int64_t N, int64_t K, const float* scales_f32,

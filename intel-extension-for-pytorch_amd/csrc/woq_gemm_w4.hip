@@ -1,0 +1,352 @@
+// MFMA GEMM for 4-bit weights and large M (prefill): y[M, N] = x[M, K] * dequant(W)[N, K]^T.
+//
+// Reference counterpart: DequantGemmTPP (dequantize a [Kb x 32] weight block to a stack
+// buffer, then libxsmm BRGEMM) driven by qlinear_woq_affine_impl
+// (csrc/cpu/aten/utils/woq.h:1847-1944, 3104-3477).  There the block is re-dequantized for
+// every M block of 64 rows; here a wave dequantizes a weight tile once per 128 rows.
+//
+//   * v_mfma_f32_16x16x32 with A = activations and B = weights, as in the decode kernel: the
+//     dequantized registers of one packed dword ARE the B operand, so weights never touch LDS;
+//   * a workgroup (4 waves) computes 128 rows x 448 columns; each wave owns 7 weight row-blocks
+//     (112 columns) for all 128 rows: 8 x 7 accumulator tiles = 224 registers, and every weight
+//     is dequantized by exactly one wave; 14336 / 448 = 32 and 2048 / 128 = 16 give 512
+//     workgroups = two full generations on 256 CUs;
+//   * per K step of 128 (one packed tile per row-block) the activations of the 128 rows go from
+//     global memory straight into LDS (global_load_lds_dwordx4, no staging registers), double
+//     buffered; 16-byte chunk p of row m is stored at chunk p ^ (m % 16), which makes the
+//     A-fragment reads (16 rows, one chunk) conflict-free without padding;
+//   * the step is software pipelined over its 4 K sub-steps: while the MFMAs of sub-step j run,
+//     the VALU dequantizes the dwords of sub-step j + 1 (the first sub-step of the next K step in
+//     the last one), ordered by sched_group_barrier as 1 MFMA : 3 VALU.
+#include "woq_common.h"
+#include "woq_internal.h"
+
+namespace woq {
+
+constexpr int G4_BM = 128;               // rows per workgroup
+constexpr int G4_MT = G4_BM / 16;        // 16-row accumulator tiles
+constexpr int G4_NTW = 7;                // weight row-blocks (16 columns each) per wave
+constexpr int G4_WAVES = 4;
+constexpr int G4_BN = G4_WAVES * G4_NTW * kTileN;  // 448
+constexpr int G4_XBYTES = G4_BM * kTileK4 * 2;     // one activation buffer: 32 KiB
+constexpr int G4_SSTRIDE = G4_NTW * kTileN + 4;    // fp32 row stride of the epilogue staging tile
+
+template <int REGIME>
+__device__ __forceinline__ f4 g4_mfma(u4 a, u4 b, f4 c) {
+  if constexpr (REGIME == kRegimeF16)
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(bitcast<h8>(a), bitcast<h8>(b), c, 0, 0, 0);
+  else
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(bitcast<b8>(a), bitcast<b8>(b), c, 0, 0, 0);
+}
+
+// Per-lane dequantization constants of one row-block and K step.
+template <int REGIME>
+struct G4Consts;
+// bf16 regime: w = bf16((q - z) * s).  The fp16 value 1024 + q (or 1024 + 16 q for a nibble taken
+// in place at bits 4..7) times s (or s / 16) plus c is the exact product (q - z) * s in fp32: one
+// fma, then one round-to-nearest-even to bf16.
+template <>
+struct G4Consts<kRegimeBF16> {
+  float s, c, s16, c16;
+  __device__ __forceinline__ void set(uint16_t sbits, float z) {
+    s = bf16_bits_to_f32(sbits);
+    c = -((1024.0f + z) * s);
+    s16 = s * 0.0625f;
+    c16 = -((64.0f + z) * s);
+  }
+};
+// fp16 regime: w = fp16((q - z) * s): exact subtraction, one rounding in the product.
+template <>
+struct G4Consts<kRegimeF16> {
+  h2 nz, s2;
+  __device__ __forceinline__ void set(uint16_t sbits, float z) {
+    const _Float16 s = bitcast<_Float16>(sbits);
+    const _Float16 n = (_Float16)(-(1024.0f + z));
+    nz = h2{n, n};
+    s2 = h2{s, s};
+  }
+};
+
+struct G4Masks {
+  uint32_t lo, hi, magic;  // 0x000F000F, 0x00F000F0, fp16 1024 twice
+};
+
+__device__ __forceinline__ uint32_t g4_pair_bf16(uint32_t hbits, float s, float c) {
+  const h2 h = bitcast<h2>(hbits);
+  f2 f;
+  f[0] = __builtin_fmaf((float)h[0], s, c);
+  f[1] = __builtin_fmaf((float)h[1], s, c);
+  return bitcast<uint32_t>(__builtin_convertvector(f, b2));
+}
+
+// One packed dword (8 weights of one row) -> MFMA B operand.
+__device__ __forceinline__ u4 g4_dequant(uint32_t d, const G4Masks& k, const G4Consts<kRegimeBF16>& q) {
+  const uint32_t d8 = d >> 8;
+  u4 r;
+  r[0] = g4_pair_bf16((d & k.lo) | k.magic, q.s, q.c);
+  r[1] = g4_pair_bf16((d & k.hi) | k.magic, q.s16, q.c16);
+  r[2] = g4_pair_bf16((d8 & k.lo) | k.magic, q.s, q.c);
+  r[3] = g4_pair_bf16((d8 & k.hi) | k.magic, q.s16, q.c16);
+  return r;
+}
+__device__ __forceinline__ u4 g4_dequant(uint32_t d, const G4Masks& k, const G4Consts<kRegimeF16>& q) {
+  u4 r;
+#pragma unroll
+  for (int v = 0; v < 4; ++v) {
+    h2 h = bitcast<h2>(((d >> (4 * v)) & k.lo) | k.magic);
+    h = (h + q.nz) * q.s2;
+    r[v] = bitcast<uint32_t>(h);
+  }
+  return r;
+}
+
+typedef __attribute__((address_space(3))) void* lds_ptr_t;
+typedef const __attribute__((address_space(1))) void* global_ptr_t;
+
+template <int REGIME>
+__global__ __launch_bounds__(256) void woq_gemm_w4_kernel(const FpArgs f, const int g_shift) {
+  __shared__ __align__(1024) uint8_t sX[2 * G4_XBYTES];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int r = lane & 15, c = lane >> 4;
+  const int M = (int)f.M, K = (int)f.K, NT = (int)f.NT, KT = (int)f.KT, KG = (int)f.KG;
+  const int m0 = blockIdx.y * G4_BM;
+  const int nt0 = (blockIdx.x * G4_WAVES + wave) * G4_NTW;  // first row-block of this wave
+
+  G4Masks km;
+  asm volatile("s_mov_b32 %0, 0x000F000F" : "=s"(km.lo));
+  asm volatile("s_mov_b32 %0, 0x00F000F0" : "=s"(km.hi));
+  asm volatile("v_mov_b32 %0, 0x64006400" : "=v"(km.magic));
+
+  f4 acc[G4_MT][G4_NTW];
+#pragma unroll
+  for (int mt = 0; mt < G4_MT; ++mt)
+#pragma unroll
+    for (int t = 0; t < G4_NTW; ++t) acc[mt][t] = f4{0.f, 0.f, 0.f, 0.f};
+
+  // ---- activations: wave w, load i fills LDS bytes [(8 w + i) * 1024, +1024): rows
+  // 4 (8 w + i) + lane / 16, physical chunk lane % 16 = logical chunk ^ (row % 16).  Rows past M
+  // re-read row M - 1; their results are never stored.
+  uint32_t xoff[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int rowl = (wave * 8 + i) * 4 + c;
+    const int rowc = m0 + rowl < M ? rowl : M - 1 - m0;
+    const int chunk = r ^ (rowl & 15);
+    xoff[i] = (uint32_t)(rowc * K + chunk * 8) * 2u;
+  }
+  // All global addresses are a wave-uniform 64-bit base plus a 32-bit per-lane byte offset that
+  // carries the K step, which keeps the bases in scalar registers.
+  const uint8_t* xbase = (const uint8_t*)f.x + (int64_t)m0 * K * 2;
+  auto load_x = [&](int kt, int buf) {
+    const uint32_t ko = (uint32_t)kt * (kTileK4 * 2);
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+      __builtin_amdgcn_global_load_lds((global_ptr_t)(xbase + (uint32_t)(xoff[i] + ko)),
+                                       (lds_ptr_t)(sX + buf * G4_XBYTES + (wave * 8 + i) * 1024), 16, 0, 0);
+  };
+  // A fragment of row tile mt, sub-step j: row 16 mt + r, logical chunk 4 c + j
+  uint32_t rd[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) rd[j] = (uint32_t)(r * 256 + (((c * 4 + j) ^ r) << 4));
+
+  // ---- weights of one K tile: one dwordx4 + one (scale, zero) per row-block and lane.  Symmetric
+  // weights carry no zero points: scale bytes are read (and ignored) instead of branching. ----
+  const bool has_z = f.zeros != nullptr;
+  const uint8_t* wbase[G4_NTW];
+  const uint8_t* sbase[G4_NTW];
+  const uint8_t* zbase[G4_NTW];
+#pragma unroll
+  for (int t = 0; t < G4_NTW; ++t) {
+    const int nt = nt0 + t < NT ? nt0 + t : NT - 1;
+    wbase[t] = f.qweight + (size_t)nt * KT * kTileBytes;
+    sbase[t] = (const uint8_t*)(f.scales + (size_t)nt * KG * kTileN);
+    zbase[t] = has_z ? f.zeros + (size_t)nt * KG * kTileN : sbase[t];
+  }
+  const uint32_t woff = (uint32_t)lane * 16u;
+  auto load_w = [&](int kt, u4 (&w)[G4_NTW], uint16_t (&s)[G4_NTW], uint8_t (&z)[G4_NTW]) {
+    int g = (kt * kTileK4 + c * 32) >> g_shift;
+    g = g < KG ? g : KG - 1;
+    const uint32_t qoff = (uint32_t)(g * kTileN + r);
+    const uint32_t wo = (uint32_t)kt * kTileBytes + woff;
+#pragma unroll
+    for (int t = 0; t < G4_NTW; ++t) {
+      w[t] = *(const u4*)(wbase[t] + wo);
+      s[t] = *(const uint16_t*)(sbase[t] + (uint32_t)(qoff * 2u));
+      const uint8_t zb = *(zbase[t] + qoff);
+      z[t] = has_z ? zb : (uint8_t)8;
+    }
+  };
+
+  u4 wr[G4_NTW], wn[G4_NTW];
+  uint16_t sr[G4_NTW];
+  uint8_t zr[G4_NTW];
+  G4Consts<REGIME> qc[G4_NTW];
+  u4 bop[2];    // B operand in use / being dequantized
+  u4 xa[2][G4_MT];  // A fragments of the sub-step in use / of the next one
+
+  load_x(0, 0);
+  load_w(0, wr, sr, zr);
+#pragma unroll
+  for (int t = 0; t < G4_NTW; ++t) qc[t].set(sr[t], (float)zr[t]);
+  bop[0] = g4_dequant(wr[0][0], km, qc[0]);
+  __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the LDS writes of load_x have landed
+  __syncthreads();
+#pragma unroll
+  for (int mt = 0; mt < G4_MT; ++mt) xa[0][mt] = *(const u4*)(sX + mt * 4096 + rd[0]);
+
+  // The accumulator tiles pass through an opaque statement on both sides of the K loop: without it
+  // the optimizer splits each loop-carried vector into four scalars (the epilogue reads single
+  // elements), and the tiles are then copied between registers in every iteration.
+#pragma unroll
+  for (int mt = 0; mt < G4_MT; ++mt)
+#pragma unroll
+    for (int t = 0; t < G4_NTW; ++t) asm volatile("" : "+a"(acc[mt][t]));
+
+  for (int kt = 0; kt < KT; ++kt) {
+    const uint8_t* xs = sX + (kt & 1) * G4_XBYTES;
+    const uint8_t* xsn = sX + ((kt & 1) ^ 1) * G4_XBYTES;
+    // ---- prefetch step kt + 1 (the last step re-reads itself into the idle buffer) ----
+    const int ktn = kt + 1 < KT ? kt + 1 : kt;
+    load_x(ktn, (kt & 1) ^ 1);
+    load_w(ktn, wn, sr, zr);
+    __builtin_amdgcn_sched_barrier(0);
+
+    // 28 blocks of 8 MFMAs (one row-block t of one K sub-step j against the 8 row tiles); the VALU
+    // dequantizes the B operand of the next block meanwhile.  The last block of a sub-step also
+    // fetches the A fragments of the next sub-step; in the last block of the step these come from
+    // the other buffer, so the block starts with the wait for this step's prefetch and the barrier.
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+#pragma unroll
+      for (int t = 0; t < G4_NTW; ++t) {
+        const int cur = (j * G4_NTW + t) & 1;
+        const bool last_t = t == G4_NTW - 1;
+        if (last_t && j == 3) {
+          __builtin_amdgcn_s_waitcnt(0x0F70);
+          __syncthreads();
+#pragma unroll
+          for (int u = 0; u < G4_NTW; ++u) qc[u].set(sr[u], (float)zr[u]);
+          bop[cur ^ 1] = g4_dequant(wn[0][0], km, qc[0]);
+        } else if (last_t) {
+          bop[cur ^ 1] = g4_dequant(wr[0][j + 1], km, qc[0]);
+        } else {
+          bop[cur ^ 1] = g4_dequant(wr[t + 1][j], km, qc[t + 1]);
+        }
+#pragma unroll
+        for (int mt = 0; mt < G4_MT; ++mt) {
+          acc[mt][t] = g4_mfma<REGIME>(xa[j & 1][mt], bop[cur], acc[mt][t]);
+          if (last_t)
+            xa[(j & 1) ^ 1][mt] = j == 3 ? *(const u4*)(xsn + mt * 4096 + rd[0])
+                                         : *(const u4*)(xs + mt * 4096 + rd[j + 1]);
+        }
+#pragma unroll
+        for (int mt = 0; mt < G4_MT; ++mt) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          if (last_t) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x002, 3, 0);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+
+    // ---- publish step kt + 1 ----
+#pragma unroll
+    for (int t = 0; t < G4_NTW; ++t) wr[t] = wn[t];
+  }
+
+#pragma unroll
+  for (int mt = 0; mt < G4_MT; ++mt)
+#pragma unroll
+    for (int t = 0; t < G4_NTW; ++t) asm volatile("" : "+a"(acc[mt][t]));
+
+  // ---- epilogue: D[m][n], lane (n = r, c) holds rows m = 16 mt + 4 c + e.  Each wave transposes
+  // one 16 x 112 accumulator tile at a time through its own LDS region (the activation buffers are
+  // idle after the last barrier), so that consecutive lanes store consecutive columns. ----
+  float* stage = (float*)sX + wave * (16 * G4_SSTRIDE);
+  const int64_t ncol0 = (int64_t)nt0 * kTileN;
+  const int act = REGIME == kRegimeF16 ? WOQ_HIP_ACT_FP16 : WOQ_HIP_ACT_BF16;
+  const bool fast = f.fusion == WOQ_HIP_FUSE_NONE && f.out_dtype == act && (f.N % 8) == 0 &&
+                    ncol0 + G4_NTW * kTileN <= f.N && (((uintptr_t)f.out | (uintptr_t)f.bias) & 15) == 0;
+  const bool hb = f.bias != nullptr;
+  Epilogue ep{f.bias, f.fusion, f.other0, f.other1, f.out, f.out_dtype, f.x_dtype, f.N};
+#pragma unroll
+  for (int mt = 0; mt < G4_MT; ++mt) {
+#pragma unroll
+    for (int t = 0; t < G4_NTW; ++t)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) stage[(4 * c + e) * G4_SSTRIDE + t * kTileN + r] = acc[mt][t][e];
+    if (fast) {
+      // 16 rows x 14 chunks of 8 columns: one 16-byte store per chunk
+#pragma unroll
+      for (int it = 0; it < 4; ++it) {
+        const int idx = it * 64 + lane;
+        const int row = idx / 14, ch = idx - row * 14;
+        const int m = m0 + mt * 16 + row;
+        if (idx < 16 * 14 && m < M) {
+          const f4 v0 = *(const f4*)(stage + row * G4_SSTRIDE + ch * 8);
+          const f4 v1 = *(const f4*)(stage + row * G4_SSTRIDE + ch * 8 + 4);
+          const int64_t n = ncol0 + ch * 8;
+          f4 b0 = f4{0.f, 0.f, 0.f, 0.f}, b1 = b0;
+          if (hb) {
+            b0 = *(const f4*)(f.bias + n);
+            b1 = *(const f4*)(f.bias + n + 4);
+          }
+          u4 o;
+#pragma unroll
+          for (int i = 0; i < 2; ++i) {
+            const float y0 = finalize_acc<REGIME>(v0[2 * i], hb, b0[2 * i]);
+            const float y1 = finalize_acc<REGIME>(v0[2 * i + 1], hb, b0[2 * i + 1]);
+            const float y2 = finalize_acc<REGIME>(v1[2 * i], hb, b1[2 * i]);
+            const float y3 = finalize_acc<REGIME>(v1[2 * i + 1], hb, b1[2 * i + 1]);
+            if constexpr (REGIME == kRegimeF16) {
+              o[i] = (uint32_t)f32_to_f16_bits(y0) | ((uint32_t)f32_to_f16_bits(y1) << 16);
+              o[i + 2] = (uint32_t)f32_to_f16_bits(y2) | ((uint32_t)f32_to_f16_bits(y3) << 16);
+            } else {
+              o[i] = bitcast<uint32_t>(__builtin_convertvector(f2{y0, y1}, b2));
+              o[i + 2] = bitcast<uint32_t>(__builtin_convertvector(f2{y2, y3}, b2));
+            }
+          }
+          *(u4*)((uint16_t*)f.out + (int64_t)m * f.N + n) = o;
+        }
+      }
+    } else {
+#pragma unroll 1
+      for (int it = 0; it < 16 * G4_NTW * kTileN / 64; ++it) {
+        const int idx = it * 64 + lane;
+        const int row = idx / (G4_NTW * kTileN), col = idx - row * (G4_NTW * kTileN);
+        const int m = m0 + mt * 16 + row;
+        const int64_t n = ncol0 + col;
+        if (m < M && n < f.N) epilogue_store<REGIME>(ep, m, n, stage[row * G4_SSTRIDE + col]);
+      }
+    }
+  }
+}
+
+// The kernel needs whole K tiles, activations already in the regime's dtype, and a group size whose
+// boundaries never split a lane's 32 consecutive K values.
+bool gemm_w4_applies(const FpArgs& f, int wbits, int regime) {
+  const int want = regime == kRegimeF16 ? WOQ_HIP_ACT_FP16 : WOQ_HIP_ACT_BF16;
+  if (wbits != 4 || f.x_dtype != want || ((uintptr_t)f.x & 15) != 0) return false;
+  if (f.K % kTileK4 != 0 || f.K * G4_BM * 2 >= (int64_t)1 << 31) return false;
+  if (f.G >= f.KT * kTileK4) return true;                 // per-channel: one group
+  return f.G >= 32 && (f.G & (f.G - 1)) == 0;
+}
+
+int launch_gemm_w4(const FpArgs& f, int regime, hipStream_t st) {
+  int g_shift = 30;
+  if (f.G < f.KT * kTileK4) {
+    g_shift = 0;
+    while (((int64_t)1 << g_shift) < f.G) ++g_shift;
+  }
+  dim3 grid((unsigned)((f.NT * kTileN + G4_BN - 1) / G4_BN), (unsigned)((f.M + G4_BM - 1) / G4_BM));
+  if (regime == kRegimeF16)
+    woq_gemm_w4_kernel<kRegimeF16><<<grid, 256, 0, st>>>(f, g_shift);
+  else
+    woq_gemm_w4_kernel<kRegimeBF16><<<grid, 256, 0, st>>>(f, g_shift);
+  return check_launch("woq_gemm_w4_kernel");
+}
+
+}  // namespace woq

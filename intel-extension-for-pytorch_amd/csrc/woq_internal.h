@@ -68,6 +68,9 @@ int launch_decode(const FpArgs& f, const uint32_t* sz, hipStream_t st);
 // regime: 0 = fp16, 1 = bf16 (woq::Regime)
 int launch_small_m(const FpArgs& a, int wbits, int regime, hipStream_t st);
 int launch_gemm(const FpArgs& a, int wbits, int regime, hipStream_t st);
+// 4-bit prefill GEMM with register-resident dequantization (woq_gemm_w4.hip)
+bool gemm_w4_applies(const FpArgs& f, int wbits, int regime);
+int launch_gemm_w4(const FpArgs& f, int regime, hipStream_t st);
 
 struct Int8Args {
   const void* x;
