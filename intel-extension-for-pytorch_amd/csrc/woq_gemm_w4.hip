@@ -6,30 +6,46 @@
 // every M block of 64 rows; here a wave dequantizes a weight tile once per 128 rows.
 //
 //   * v_mfma_f32_16x16x32 with A = activations and B = weights, as in the decode kernel: the
-//     dequantized registers of one packed dword ARE the B operand, so weights never touch LDS;
-//   * a workgroup (4 waves) computes 128 rows x 448 columns; each wave owns 7 weight row-blocks
-//     (112 columns) for all 128 rows: 8 x 7 accumulator tiles = 224 registers, and every weight
-//     is dequantized by exactly one wave; 14336 / 448 = 32 and 2048 / 128 = 16 give 512
-//     workgroups = two full generations on 256 CUs;
-//   * per K step of 128 (one packed tile per row-block) the activations of the 128 rows go from
-//     global memory straight into LDS (global_load_lds_dwordx4, no staging registers), double
-//     buffered; 16-byte chunk p of row m is stored at chunk p ^ (m % 16), which makes the
-//     A-fragment reads (16 rows, one chunk) conflict-free without padding;
-//   * the step is software pipelined over its 4 K sub-steps: while the MFMAs of sub-step j run,
-//     the VALU dequantizes the dwords of sub-step j + 1 (the first sub-step of the next K step in
-//     the last one), ordered by sched_group_barrier as 1 MFMA : 3 VALU.
+//     dequantized registers of one packed dword ARE the B operand, so weights never touch LDS
+//     in dequantized form and every weight is dequantized by exactly one wave;
+//   * a workgroup is 4 waves, one per SIMD with the whole 512-entry register file; wave w owns NTW
+//     weight row-blocks (16 columns each) for all 16 * MT rows of the workgroup, i.e. MT x NTW
+//     accumulator tiles.  The shape built is 128 x 448 (MT 8, NTW 7: 224 accumulator registers;
+//     14336 / 448 = 32 and 2048 / 128 = 16 give 512 workgroups = two full generations on 256 CUs).
+//     One wave hides about two VALU instructions behind each MFMA (measured: 16.4 cycles per MFMA
+//     with 0..2 independent VALU instructions in between, +4 cycles for each further one); a
+//     dequantized dword costs 17 and feeds MT = 8 MFMAs, so the loop is VALU-issue-bound;
+//   * per K step of 128 (one packed tile per row-block) the activations of the rows go from global
+//     memory straight into LDS (global_load_lds_dwordx4, no staging registers), double buffered;
+//     16-byte chunk p of row m is stored at chunk p ^ (m % 16), which makes the A-fragment reads
+//     (16 rows, one chunk) conflict-free without padding.  The packed tiles take the same route
+//     into a per-wave LDS stage two steps ahead and are read into registers during the last K
+//     sub-step of the step before;
+//   * the step is software pipelined over its 4 K sub-steps and NTW row-blocks: while the MT MFMAs
+//     of one (sub-step, row-block) run, the VALU dequantizes the dword of the next one.
 #include "woq_common.h"
 #include "woq_internal.h"
 
 namespace woq {
 
-constexpr int G4_BM = 128;               // rows per workgroup
-constexpr int G4_MT = G4_BM / 16;        // 16-row accumulator tiles
-constexpr int G4_NTW = 7;                // weight row-blocks (16 columns each) per wave
 constexpr int G4_WAVES = 4;
-constexpr int G4_BN = G4_WAVES * G4_NTW * kTileN;  // 448
-constexpr int G4_XBYTES = G4_BM * kTileK4 * 2;     // one activation buffer: 32 KiB
-constexpr int G4_SSTRIDE = G4_NTW * kTileN + 4;    // fp32 row stride of the epilogue staging tile
+template <int MT_, int NTW_>
+struct G4Shape {
+  static constexpr int MT = MT_;                        // 16-row accumulator tiles
+  static constexpr int NTW = NTW_;                      // weight row-blocks (16 columns) per wave
+  static constexpr int BM = 16 * MT;                    // rows per workgroup
+  static constexpr int BN = G4_WAVES * NTW * kTileN;    // columns per workgroup
+  static constexpr int XBYTES = BM * kTileK4 * 2;       // one activation buffer
+  static constexpr int XLOADS = XBYTES / (G4_WAVES * 1024);  // LDS loads per wave and buffer
+  static constexpr int WSTAGE = G4_WAVES * NTW * kTileBytes;  // one weight stage
+  static constexpr int LDS_BYTES = 2 * XBYTES + 2 * WSTAGE;
+  static constexpr int SSTRIDE = NTW * kTileN + 4;      // fp32 row stride of the epilogue staging tile
+  // Row-block during whose MFMAs the A fragments of the next K sub-step are read from LDS.  One
+  // block ahead of their first use needs a second set of MT fragment registers; with 16 row tiles
+  // a block is long enough (256 cycles) to read them in the last block, each into the registers of
+  // the fragment whose last MFMA has just been issued.
+  static constexpr int FETCH_T = MT >= 16 ? NTW - 1 : NTW - 2;
+};
 
 template <int REGIME>
 __device__ __forceinline__ f4 g4_mfma(u4 a, u4 b, f4 c) {
@@ -103,9 +119,13 @@ __device__ __forceinline__ u4 g4_dequant(uint32_t d, const G4Masks& k, const G4C
 typedef __attribute__((address_space(3))) void* lds_ptr_t;
 typedef const __attribute__((address_space(1))) void* global_ptr_t;
 
-template <int REGIME>
+template <int REGIME, class S>
 __global__ __launch_bounds__(256) void woq_gemm_w4_kernel(const FpArgs f, const int g_shift) {
-  __shared__ __align__(1024) uint8_t sX[2 * G4_XBYTES];
+  constexpr int G4_MT = S::MT, G4_NTW = S::NTW, G4_BM = S::BM, G4_XBYTES = S::XBYTES, G4_XLOADS = S::XLOADS,
+                G4_WSTAGE = S::WSTAGE, G4_SSTRIDE = S::SSTRIDE;
+  // two activation buffers, then two weight stages of 4 waves x NTW tiles x 1 KiB
+  extern __shared__ __align__(1024) uint8_t sX[];
+  uint8_t* const sW = sX + 2 * G4_XBYTES;
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -126,13 +146,13 @@ __global__ __launch_bounds__(256) void woq_gemm_w4_kernel(const FpArgs f, const 
 #pragma unroll
     for (int t = 0; t < G4_NTW; ++t) acc[mt][t] = f4{0.f, 0.f, 0.f, 0.f};
 
-  // ---- activations: wave w, load i fills LDS bytes [(8 w + i) * 1024, +1024): rows
-  // 4 (8 w + i) + lane / 16, physical chunk lane % 16 = logical chunk ^ (row % 16).  Rows past M
-  // re-read row M - 1; their results are never stored.
-  uint32_t xoff[8];
+  // ---- activations: load i of wave w fills LDS KiB number w * XLOADS + i of a buffer: rows
+  // 4 (w * XLOADS + i) + lane / 16, physical chunk lane % 16 = logical chunk ^ (row % 16).  Rows
+  // past M re-read row M - 1; their results are never stored.
+  uint32_t xoff[G4_XLOADS];
 #pragma unroll
-  for (int i = 0; i < 8; ++i) {
-    const int rowl = (wave * 8 + i) * 4 + c;
+  for (int i = 0; i < G4_XLOADS; ++i) {
+    const int rowl = (wave * G4_XLOADS + i) * 4 + c;
     const int rowc = m0 + rowl < M ? rowl : M - 1 - m0;
     const int chunk = r ^ (rowl & 15);
     xoff[i] = (uint32_t)(rowc * K + chunk * 8) * 2u;
@@ -143,9 +163,10 @@ __global__ __launch_bounds__(256) void woq_gemm_w4_kernel(const FpArgs f, const 
   auto load_x = [&](int kt, int buf) {
     const uint32_t ko = (uint32_t)kt * (kTileK4 * 2);
 #pragma unroll
-    for (int i = 0; i < 8; ++i)
+    for (int i = 0; i < G4_XLOADS; ++i)
       __builtin_amdgcn_global_load_lds((global_ptr_t)(xbase + (uint32_t)(xoff[i] + ko)),
-                                       (lds_ptr_t)(sX + buf * G4_XBYTES + (wave * 8 + i) * 1024), 16, 0, 0);
+                                       (lds_ptr_t)(sX + buf * G4_XBYTES + (wave * G4_XLOADS + i) * 1024), 16, 0,
+                                       0);
   };
   // A fragment of row tile mt, sub-step j: row 16 mt + r, logical chunk 4 c + j
   uint32_t rd[4];
@@ -166,34 +187,57 @@ __global__ __launch_bounds__(256) void woq_gemm_w4_kernel(const FpArgs f, const 
     zbase[t] = has_z ? f.zeros + (size_t)nt * KG * kTileN : sbase[t];
   }
   const uint32_t woff = (uint32_t)lane * 16u;
-  auto load_w = [&](int kt, u4 (&w)[G4_NTW], uint16_t (&s)[G4_NTW], uint8_t (&z)[G4_NTW]) {
+  auto load_q = [&](int kt, uint16_t (&s)[G4_NTW], uint8_t (&z)[G4_NTW]) {
     int g = (kt * kTileK4 + c * 32) >> g_shift;
     g = g < KG ? g : KG - 1;
     const uint32_t qoff = (uint32_t)(g * kTileN + r);
-    const uint32_t wo = (uint32_t)kt * kTileBytes + woff;
 #pragma unroll
     for (int t = 0; t < G4_NTW; ++t) {
-      w[t] = *(const u4*)(wbase[t] + wo);
       s[t] = *(const uint16_t*)(sbase[t] + (uint32_t)(qoff * 2u));
       const uint8_t zb = *(zbase[t] + qoff);
       z[t] = has_z ? zb : (uint8_t)8;
     }
   };
+  // The packed tiles of a K step travel global -> LDS -> registers: the LDS stage costs no
+  // registers while the load is in flight, which lets the tiles be requested two steps ahead.
+  // Each wave fills and reads only its own NTW KiB of a stage.
+  uint8_t* const wmine = sW + wave * (G4_NTW * kTileBytes);
+  auto dma_w = [&](int kt, int stage) {
+    const uint32_t wo = (uint32_t)kt * kTileBytes + woff;
+#pragma unroll
+    for (int t = 0; t < G4_NTW; ++t)
+      __builtin_amdgcn_global_load_lds((global_ptr_t)(wbase[t] + wo),
+                                       (lds_ptr_t)(wmine + stage * G4_WSTAGE + t * kTileBytes), 16, 0, 0);
+  };
+  auto read_w = [&](int stage, int t) { return *(const u4*)(wmine + stage * G4_WSTAGE + t * kTileBytes + woff); };
 
-  u4 wr[G4_NTW], wn[G4_NTW];
+  u4 wr[G4_NTW];
   uint16_t sr[G4_NTW];
   uint8_t zr[G4_NTW];
   G4Consts<REGIME> qc[G4_NTW];
-  u4 bop[2];    // B operand in use / being dequantized
+  u4 bop[2];        // B operand in use / being dequantized
   u4 xa[2][G4_MT];  // A fragments of the sub-step in use / of the next one
 
+  // s_waitcnt immediates (vmcnt in bits 3:0 and 15:14; expcnt 6:4 and lgkmcnt 11:8 left at maximum)
+  constexpr int kVmcnt0 = 0x0F70, kLgkmcnt0 = 0xC07F;
+  constexpr int kVmcntW = 0x0F70 | G4_NTW;  // all but the last NTW loads (one weight stage) have landed
+  // everything older than one whole step of loads (2 NTW parameter loads, XLOADS + NTW LDS loads)
+  constexpr int kStepLoads = 3 * G4_NTW + G4_XLOADS;
+  static_assert(kStepLoads < 64 && G4_NTW < 16, "s_waitcnt vmcnt is a 6-bit field");
+  constexpr int kVmcntStep = 0x0F70 | (kStepLoads & 15) | ((kStepLoads >> 4) << 14);
+
   load_x(0, 0);
-  load_w(0, wr, sr, zr);
-#pragma unroll
-  for (int t = 0; t < G4_NTW; ++t) qc[t].set(sr[t], (float)zr[t]);
-  bop[0] = g4_dequant(wr[0][0], km, qc[0]);
-  __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the LDS writes of load_x have landed
+  dma_w(0, 0);
+  dma_w(KT > 1 ? 1 : 0, 1);
+  load_q(0, sr, zr);
+  __builtin_amdgcn_s_waitcnt(kVmcnt0);
   __syncthreads();
+#pragma unroll
+  for (int t = 0; t < G4_NTW; ++t) {
+    wr[t] = read_w(0, t);
+    qc[t].set(sr[t], (float)zr[t]);
+  }
+  bop[0] = g4_dequant(wr[0][0], km, qc[0]);
 #pragma unroll
   for (int mt = 0; mt < G4_MT; ++mt) xa[0][mt] = *(const u4*)(sX + mt * 4096 + rd[0]);
 
@@ -208,28 +252,44 @@ __global__ __launch_bounds__(256) void woq_gemm_w4_kernel(const FpArgs f, const 
   for (int kt = 0; kt < KT; ++kt) {
     const uint8_t* xs = sX + (kt & 1) * G4_XBYTES;
     const uint8_t* xsn = sX + ((kt & 1) ^ 1) * G4_XBYTES;
-    // ---- prefetch step kt + 1 (the last step re-reads itself into the idle buffer) ----
-    const int ktn = kt + 1 < KT ? kt + 1 : kt;
-    load_x(ktn, (kt & 1) ^ 1);
-    load_w(ktn, wn, sr, zr);
+    // ---- requests, in this order (s_waitcnt vmcnt counts from the youngest): parameters and
+    // activations of step kt + 1, then (behind the first MFMA block) the weight tiles of step
+    // kt + 2 into the stage that held step kt.  Past the end the last step is requested again. ----
+    const int kt1 = kt + 1 < KT ? kt + 1 : KT - 1;
+    const int kt2 = kt + 2 < KT ? kt + 2 : KT - 1;
+    load_q(kt1, sr, zr);
+    load_x(kt1, (kt & 1) ^ 1);
     __builtin_amdgcn_sched_barrier(0);
 
-    // 28 blocks of 8 MFMAs (one row-block t of one K sub-step j against the 8 row tiles); the VALU
-    // dequantizes the B operand of the next block meanwhile.  The last block of a sub-step also
-    // fetches the A fragments of the next sub-step; in the last block of the step these come from
-    // the other buffer, so the block starts with the wait for this step's prefetch and the barrier.
+    // 4 NTW blocks of MT MFMAs (one row-block t of one K sub-step j against the MT row tiles); the VALU
+    // dequantizes the B operand of the next block meanwhile.  Block FETCH_T of a sub-step also
+    // fetches the A fragments of the next sub-step; in the last sub-step these come from the other
+    // buffer, so that block starts with the wait for this step's activations and the barrier.  Block t of the last sub-step reads the
+    // tile of row-block t for the next step from LDS; its registers were last used one block before.
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
 #pragma unroll
       for (int t = 0; t < G4_NTW; ++t) {
         const int cur = (j * G4_NTW + t) & 1;
         const bool last_t = t == G4_NTW - 1;
+        const bool fetch_t = t == S::FETCH_T;
+        if (j == 0 && t == 1) {
+          // the LDS reads of the previous step's last blocks have returned: their stage is free
+          __builtin_amdgcn_s_waitcnt(kLgkmcnt0);
+          dma_w(kt2, kt & 1);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+        if (j == 3 && t == 0) __builtin_amdgcn_s_waitcnt(kVmcntStep);  // tiles of step kt + 1 are in LDS
+        if (fetch_t && j == 3) {
+          // Written as an instruction, not as the barrier builtin: before that one the compiler
+          // waits for every outstanding load, the tiles requested for step kt + 2 included.
+          __builtin_amdgcn_s_waitcnt(kVmcntW);
+          asm volatile("s_barrier" ::: "memory");
+        }
         if (last_t && j == 3) {
-          __builtin_amdgcn_s_waitcnt(0x0F70);
-          __syncthreads();
 #pragma unroll
           for (int u = 0; u < G4_NTW; ++u) qc[u].set(sr[u], (float)zr[u]);
-          bop[cur ^ 1] = g4_dequant(wn[0][0], km, qc[0]);
+          bop[cur ^ 1] = g4_dequant(wr[0][0], km, qc[0]);
         } else if (last_t) {
           bop[cur ^ 1] = g4_dequant(wr[0][j + 1], km, qc[0]);
         } else {
@@ -238,32 +298,31 @@ __global__ __launch_bounds__(256) void woq_gemm_w4_kernel(const FpArgs f, const 
 #pragma unroll
         for (int mt = 0; mt < G4_MT; ++mt) {
           acc[mt][t] = g4_mfma<REGIME>(xa[j & 1][mt], bop[cur], acc[mt][t]);
-          if (last_t)
+          if (fetch_t)
             xa[(j & 1) ^ 1][mt] = j == 3 ? *(const u4*)(xsn + mt * 4096 + rd[0])
                                          : *(const u4*)(xs + mt * 4096 + rd[j + 1]);
         }
+        if (j == 3) wr[t] = read_w((kt & 1) ^ 1, t);
 #pragma unroll
         for (int mt = 0; mt < G4_MT; ++mt) {
           __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-          if (last_t) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+          if (fetch_t) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
           __builtin_amdgcn_sched_group_barrier(0x002, 3, 0);
         }
         __builtin_amdgcn_sched_barrier(0);
       }
     }
-
-    // ---- publish step kt + 1 ----
-#pragma unroll
-    for (int t = 0; t < G4_NTW; ++t) wr[t] = wn[t];
   }
 
+  // The requests past the last step are still writing LDS: drain them before the workgroup can end.
+  __builtin_amdgcn_s_waitcnt(kVmcnt0);
 #pragma unroll
   for (int mt = 0; mt < G4_MT; ++mt)
 #pragma unroll
     for (int t = 0; t < G4_NTW; ++t) asm volatile("" : "+a"(acc[mt][t]));
 
   // ---- epilogue: D[m][n], lane (n = r, c) holds rows m = 16 mt + 4 c + e.  Each wave transposes
-  // one 16 x 112 accumulator tile at a time through its own LDS region (the activation buffers are
+  // one 16 x (16 NTW) accumulator tile at a time through its own LDS region (the activation buffers are
   // idle after the last barrier), so that consecutive lanes store consecutive columns. ----
   float* stage = (float*)sX + wave * (16 * G4_SSTRIDE);
   const int64_t ncol0 = (int64_t)nt0 * kTileN;
@@ -279,13 +338,14 @@ __global__ __launch_bounds__(256) void woq_gemm_w4_kernel(const FpArgs f, const 
 #pragma unroll
       for (int e = 0; e < 4; ++e) stage[(4 * c + e) * G4_SSTRIDE + t * kTileN + r] = acc[mt][t][e];
     if (fast) {
-      // 16 rows x 14 chunks of 8 columns: one 16-byte store per chunk
+      // 16 rows x 2 NTW chunks of 8 columns: one 16-byte store per chunk
+      constexpr int CH = 2 * G4_NTW;
 #pragma unroll
-      for (int it = 0; it < 4; ++it) {
+      for (int it = 0; it < (16 * CH + 63) / 64; ++it) {
         const int idx = it * 64 + lane;
-        const int row = idx / 14, ch = idx - row * 14;
+        const int row = idx / CH, ch = idx - row * CH;
         const int m = m0 + mt * 16 + row;
-        if (idx < 16 * 14 && m < M) {
+        if (idx < 16 * CH && m < M) {
           const f4 v0 = *(const f4*)(stage + row * G4_SSTRIDE + ch * 8);
           const f4 v1 = *(const f4*)(stage + row * G4_SSTRIDE + ch * 8 + 4);
           const int64_t n = ncol0 + ch * 8;
@@ -330,9 +390,22 @@ __global__ __launch_bounds__(256) void woq_gemm_w4_kernel(const FpArgs f, const 
 bool gemm_w4_applies(const FpArgs& f, int wbits, int regime) {
   const int want = regime == kRegimeF16 ? WOQ_HIP_ACT_FP16 : WOQ_HIP_ACT_BF16;
   if (wbits != 4 || f.x_dtype != want || ((uintptr_t)f.x & 15) != 0) return false;
-  if (f.K % kTileK4 != 0 || f.K * G4_BM * 2 >= (int64_t)1 << 31) return false;
+  if (f.K % kTileK4 != 0 || f.K * 256 * 2 >= (int64_t)1 << 31) return false;
   if (f.G >= f.KT * kTileK4) return true;                 // per-channel: one group
   return f.G >= 32 && (f.G & (f.G - 1)) == 0;
+}
+
+template <int REGIME, class S>
+static int launch_shape(const FpArgs& f, int g_shift, hipStream_t st) {
+  // more than 64 KiB of LDS per workgroup needs an opt-in (once per kernel and process)
+  static const hipError_t lds_optin =
+      hipFuncSetAttribute(reinterpret_cast<const void*>(&woq_gemm_w4_kernel<REGIME, S>),
+                          hipFuncAttributeMaxDynamicSharedMemorySize, S::LDS_BYTES);
+  if (lds_optin != hipSuccess)
+    return set_error("woq_gemm_w4_kernel: LDS opt-in failed: %s", hipGetErrorString(lds_optin));
+  dim3 grid((unsigned)((f.NT * kTileN + S::BN - 1) / S::BN), (unsigned)((f.M + S::BM - 1) / S::BM));
+  woq_gemm_w4_kernel<REGIME, S><<<grid, 256, S::LDS_BYTES, st>>>(f, g_shift);
+  return check_launch("woq_gemm_w4_kernel");
 }
 
 int launch_gemm_w4(const FpArgs& f, int regime, hipStream_t st) {
@@ -341,12 +414,12 @@ int launch_gemm_w4(const FpArgs& f, int regime, hipStream_t st) {
     g_shift = 0;
     while (((int64_t)1 << g_shift) < f.G) ++g_shift;
   }
-  dim3 grid((unsigned)((f.NT * kTileN + G4_BN - 1) / G4_BN), (unsigned)((f.M + G4_BM - 1) / G4_BM));
-  if (regime == kRegimeF16)
-    woq_gemm_w4_kernel<kRegimeF16><<<grid, 256, 0, st>>>(f, g_shift);
-  else
-    woq_gemm_w4_kernel<kRegimeBF16><<<grid, 256, 0, st>>>(f, g_shift);
-  return check_launch("woq_gemm_w4_kernel");
+  // 128 x 448 per workgroup.  A 256 x 256 shape (MT 16, NTW 4) would halve the dequantization work
+  // per MFMA, but its 256 accumulator registers leave the register allocator no spare tile and the
+  // generated loop copies accumulators through VGPRs and scratch; it measured slower and is not built.
+  using Shape = G4Shape<8, 7>;
+  return regime == kRegimeF16 ? launch_shape<kRegimeF16, Shape>(f, g_shift, st)
+                              : launch_shape<kRegimeBF16, Shape>(f, g_shift, st);
 }
 
 }  // namespace woq

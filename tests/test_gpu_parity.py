@@ -226,6 +226,58 @@ def test_both_kernels_agree_on_mid_m(cuda, M):
     _check_fp(case, O.LOWP_BF16, force_kernel=2, label=f"tiled kernel M={M}")
 
 
+@pytest.mark.parametrize(
+    "M,K,N,G,bias",
+    [
+        (128, 256, 448, 128, False),  # exactly one workgroup tile
+        (300, 1024, 1000, 32, True),  # ragged M, last wave of the last workgroup partly outside N
+        (129, 512, 464, 64, True),
+        (200, 384, 96, -1, False),  # per-channel, fewer row-blocks than one wave owns
+        (513, 2048, 912, 256, True),
+        (70, 128, 16, 128, False),  # a single K step
+        (150, 256, 450, 128, True),  # N not a multiple of 8: element-wise stores
+    ],
+)
+def test_w4_prefill_kernel(cuda, M, K, N, G, bias):
+    case = _synthetic().make_int4_case(20, M, K, N, G, bias=bias)
+    _check_fp(case, O.LOWP_BF16, force_kernel=3, label=f"w4 prefill M={M} K={K} N={N} G={G}")
+
+
+def test_w4_prefill_kernel_symmetric_and_close_to_tiled(cuda):
+    case = _synthetic().make_int4_case(21, 260, 512, 464, 128, bias=True)
+    case["zeros"] = None
+    _check_fp(case, O.LOWP_BF16, force_kernel=3, label="w4 prefill, symmetric")
+    # the two GEMM kernels sum the K products in different orders: same values up to the last bit
+    ctx = make_context(case, O.LOWP_BF16)
+    x = case["x"].cuda()
+    a, b = to_np_f32(ctx.run(x, force_kernel=3)), to_np_f32(ctx.run(x, force_kernel=2))
+    assert bool(np.all((bf16_ulp_diff(a, b) <= 1) | (np.abs(a - b) <= 1e-4)))
+
+
+def test_w4_prefill_kernel_fp16_regime(cuda):
+    """lowp_mode FP16 with fp16 activations: w = fp16((q - z) * s), fp16 result and bias add."""
+    syn = _synthetic()
+    M, K, N, G = 140, 512, 464, 128
+    case = syn.make_int4_case(22, M, K, N, G, bias=True, scale_dtype=torch.float16)
+    case["x"] = case["x"].to(torch.float16)
+    ctx = make_context(case, O.LOWP_FP16)
+    x = case["x"].cuda()
+    y = to_np_f32(ctx.run(x, force_kernel=3))
+    acc = ctx.run(x, out_fp32=True, force_kernel=3).cpu().numpy()
+    c = case_np(case)
+    acc_ref, y_ref = O.woq_linear_ref(c["x"], "fp16", c["qw"], N, K, c["scales"], c["zps"], c["bias"], 2, G, "fp16")
+    assert max_abs(acc, acc_ref) <= MAX_ABS_ACC
+    assert rel_l2(y, y_ref) <= REL_L2_OUT
+    assert rel_l2(y, to_np_f32(ctx.run(x, force_kernel=2))) <= 1e-3
+
+
+def test_w4_prefill_kernel_rejects_other_shapes(cuda):
+    case = _synthetic().make_int4_case(23, 70, 1000, 64, -1)  # K is not a multiple of 128
+    ctx = make_context(case, O.LOWP_BF16)
+    with pytest.raises(RuntimeError, match="4-bit prefill kernel"):
+        ctx.run(case["x"].cuda(), force_kernel=3)
+
+
 def test_int8_weights_small_and_tiled(cuda):
     for M in (1, 8, 40, 200):
         case = _synthetic().make_int8_case(16, M, 512, 144)
