@@ -25,6 +25,12 @@ HBM_PEAK_GBS = 8000.0       # MI355X HBM3E, published
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
 
 
+# HBM bytes per launch of the dominant kernel, from two rocprofv3 --pmc runs of `bench.py --traffic-probe`
+# (FETCH_SIZE 15310.55 KiB and WRITE_SIZE 28.00 KiB per dispatch, scaled by what the same counters read for a
+# 256 MiB copy: x2.000 and x1.000); keyed by (M, K, N, group size).  Other shapes have not been measured.
+MEASURED_HBM_BYTES_PER_LAUNCH = {(1, 4096, 14336, 128): 31384678}
+
+
 def algorithmic_bytes(M, K, N, G):
     """INT4 weights 1/2 B, bf16 scales 2 B and packed uint4 zeros 1/2 B per (n, group),
     bf16 activations and outputs."""
@@ -255,7 +261,7 @@ def main():
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": round(achieved / HBM_PEAK_GBS, 4),
-            "traffic": None,
+            "traffic": MEASURED_HBM_BYTES_PER_LAUNCH.get((M, K, N, G)),
             "kernel": "woq_decode_kernel",
             "us_per_launch_stream": round(us_launch, 3),
             "us_per_launch_graph": round(us_graph, 3),
