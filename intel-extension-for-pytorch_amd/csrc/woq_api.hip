@@ -208,11 +208,13 @@ int woq_hip_linear(const woq_hip_linear_params* p) {
     return launch_decode(f, p->scale_zero_f16x2, st);
   if (kernel == 0) kernel = p->M <= 64 ? 1 : (gemm_w4_applies(f, wbits, regime) ? 3 : 2);
   if (kernel == 1 && p->M > 64) return set_error("woq_linear: the small-M kernel takes M <= 64");
+  const int w4_shape = kernel == 4 ? 7 : kernel == 5 ? 4 : kernel == 6 ? 2 : 0;
+  if (kernel >= 4 && kernel <= 6) kernel = 3;
   if (kernel == 3 && !gemm_w4_applies(f, wbits, regime))
     return set_error("woq_linear: the 4-bit prefill kernel takes 4-bit weights, K %% 128 == 0, a power-of-two or "
                      "per-channel group size and activations in the compute dtype");
   if (kernel == 1) return launch_small_m(f, wbits, regime, st);
-  return kernel == 3 ? launch_gemm_w4(f, regime, st) : launch_gemm(f, wbits, regime, st);
+  return kernel == 3 ? launch_gemm_w4(f, regime, st, w4_shape) : launch_gemm(f, wbits, regime, st);
 }
 
 int woq_hip_dequant_weight(const void* qweight, int weight_dtype, int64_t N, int64_t K, const float* scales_f32,

@@ -408,18 +408,39 @@ static int launch_shape(const FpArgs& f, int g_shift, hipStream_t st) {
   return check_launch("woq_gemm_w4_kernel");
 }
 
-int launch_gemm_w4(const FpArgs& f, int regime, hipStream_t st) {
+// Relative time of a shape: generations of 256 workgroups times the length of one K step, which
+// is proportional to the row-blocks per wave plus a fixed part (requests, barrier, pipeline fill).
+template <class S>
+static double shape_cost(const FpArgs& f) {
+  const double wgs = (double)((f.NT * kTileN + S::BN - 1) / S::BN) * (double)((f.M + S::BM - 1) / S::BM);
+  return (double)(int64_t)((wgs + 255) / 256) * (S::NTW + 1.0);
+}
+
+int launch_gemm_w4(const FpArgs& f, int regime, hipStream_t st, int shape) {
   int g_shift = 30;
   if (f.G < f.KT * kTileK4) {
     g_shift = 0;
     while (((int64_t)1 << g_shift) < f.G) ++g_shift;
   }
-  // 128 x 448 per workgroup.  A 256 x 256 shape (MT 16, NTW 4) would halve the dequantization work
-  // per MFMA, but its 256 accumulator registers leave the register allocator no spare tile and the
-  // generated loop copies accumulators through VGPRs and scratch; it measured slower and is not built.
-  using Shape = G4Shape<8, 7>;
-  return regime == kRegimeF16 ? launch_shape<kRegimeF16, Shape>(f, g_shift, st)
-                              : launch_shape<kRegimeBF16, Shape>(f, g_shift, st);
+  // 128 rows x 448, 256 or 128 columns per workgroup: the widest shape does the most work per
+  // activation fragment, the narrower ones make enough workgroups to fill the chip when M * N is
+  // small (e.g. N = 4096: 10 column blocks of 448 but 16 of 256).  A 256 x 256 shape (MT 16, NTW 4)
+  // would halve the dequantization work per MFMA, but its 256 accumulator registers leave the
+  // register allocator no spare tile and the generated loop copies accumulators through VGPRs and
+  // scratch; it measured slower and is not built.
+  using S7 = G4Shape<8, 7>;
+  using S4 = G4Shape<8, 4>;
+  using S2 = G4Shape<8, 2>;
+  const double c7 = shape_cost<S7>(f), c4 = shape_cost<S4>(f), c2 = shape_cost<S2>(f);
+  if (shape == 0) shape = (c7 <= c4 && c7 <= c2) ? 7 : (c4 <= c2 ? 4 : 2);
+  if (shape == 7)
+    return regime == kRegimeF16 ? launch_shape<kRegimeF16, S7>(f, g_shift, st)
+                                : launch_shape<kRegimeBF16, S7>(f, g_shift, st);
+  if (shape == 4)
+    return regime == kRegimeF16 ? launch_shape<kRegimeF16, S4>(f, g_shift, st)
+                                : launch_shape<kRegimeBF16, S4>(f, g_shift, st);
+  return regime == kRegimeF16 ? launch_shape<kRegimeF16, S2>(f, g_shift, st)
+                              : launch_shape<kRegimeBF16, S2>(f, g_shift, st);
 }
 
 }  // namespace woq

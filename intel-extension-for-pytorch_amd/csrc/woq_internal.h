@@ -70,7 +70,8 @@ int launch_small_m(const FpArgs& a, int wbits, int regime, hipStream_t st);
 int launch_gemm(const FpArgs& a, int wbits, int regime, hipStream_t st);
 // 4-bit prefill GEMM with register-resident dequantization (woq_gemm_w4.hip)
 bool gemm_w4_applies(const FpArgs& f, int wbits, int regime);
-int launch_gemm_w4(const FpArgs& f, int regime, hipStream_t st);
+// shape: row-blocks per wave (7, 4 or 2: 448, 256 or 128 columns per workgroup), 0 = by cost model
+int launch_gemm_w4(const FpArgs& f, int regime, hipStream_t st, int shape = 0);
 
 struct Int8Args {
   const void* x;

@@ -238,9 +238,10 @@ def test_both_kernels_agree_on_mid_m(cuda, M):
         (150, 256, 450, 128, True),  # N not a multiple of 8: element-wise stores
     ],
 )
-def test_w4_prefill_kernel(cuda, M, K, N, G, bias):
+@pytest.mark.parametrize("shape", [3, 4, 5, 6])  # cost model, then 448 / 256 / 128 columns per workgroup
+def test_w4_prefill_kernel(cuda, M, K, N, G, bias, shape):
     case = _synthetic().make_int4_case(20, M, K, N, G, bias=bias)
-    _check_fp(case, O.LOWP_BF16, force_kernel=3, label=f"w4 prefill M={M} K={K} N={N} G={G}")
+    _check_fp(case, O.LOWP_BF16, force_kernel=shape, label=f"w4 prefill M={M} K={K} N={N} G={G} kernel={shape}")
 
 
 def test_w4_prefill_kernel_symmetric_and_close_to_tiled(cuda):
