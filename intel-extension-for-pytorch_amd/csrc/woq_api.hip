@@ -206,6 +206,13 @@ int woq_hip_linear(const woq_hip_linear_params* p) {
   int kernel = p->force_kernel;
   if (kernel == 0 && decode_kernel_applies(f, wbits, regime, p->scale_zero_f16x2))
     return launch_decode(f, p->scale_zero_f16x2, st);
+  if (kernel == 0 && decode_dq_applies(f, wbits, regime)) kernel = 7;
+  if (kernel >= 7 && kernel <= 10) {
+    if (!decode_dq_applies(f, wbits, regime))
+      return set_error("woq_linear: the dequantizing decode kernel takes 4-bit weights, M <= 16, K %% 128 == 0, a "
+                       "power-of-two or per-channel group size and activations in the compute dtype");
+    return launch_decode_dq(f, regime, st, kernel == 10 ? 4 : kernel - 7);
+  }
   if (kernel == 0) kernel = p->M <= 64 ? 1 : (gemm_w4_applies(f, wbits, regime) ? 3 : 2);
   if (kernel == 1 && p->M > 64) return set_error("woq_linear: the small-M kernel takes M <= 64");
   const int w4_shape = kernel == 4 ? 7 : kernel == 5 ? 4 : kernel == 6 ? 2 : 0;

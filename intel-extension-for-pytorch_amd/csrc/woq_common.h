@@ -219,4 +219,67 @@ __device__ __forceinline__ void epilogue_store(const Epilogue& e, int64_t m, int
   store_act(e.out, e.out_dtype, idx, y);
 }
 
+// ---- 4-bit weights as MFMA operands: one packed dword (8 weights of one row) -> 8 bf16 / fp16 ----
+// Per-lane dequantization constants of one weight row and quantization group.
+template <int REGIME>
+struct G4Consts;
+// bf16 regime: w = bf16((q - z) * s).  The fp16 value 1024 + q (or 1024 + 16 q for a nibble taken
+// in place at bits 4..7) times s (or s / 16) plus c is the exact product (q - z) * s in fp32: one
+// fma, then one round-to-nearest-even to bf16.
+template <>
+struct G4Consts<kRegimeBF16> {
+  float s, c, s16, c16;
+  __device__ __forceinline__ void set(uint16_t sbits, float z) {
+    s = bf16_bits_to_f32(sbits);
+    c = -((1024.0f + z) * s);
+    s16 = s * 0.0625f;
+    c16 = -((64.0f + z) * s);
+  }
+};
+// fp16 regime: w = fp16((q - z) * s): exact subtraction, one rounding in the product.
+template <>
+struct G4Consts<kRegimeF16> {
+  h2 nz, s2;
+  __device__ __forceinline__ void set(uint16_t sbits, float z) {
+    const _Float16 s = bitcast<_Float16>(sbits);
+    const _Float16 n = (_Float16)(-(1024.0f + z));
+    nz = h2{n, n};
+    s2 = h2{s, s};
+  }
+};
+
+struct G4Masks {
+  uint32_t lo, hi, magic;  // 0x000F000F, 0x00F000F0, fp16 1024 twice
+};
+
+__device__ __forceinline__ uint32_t g4_pair_bf16(uint32_t hbits, float s, float c) {
+  const h2 h = bitcast<h2>(hbits);
+  f2 f;
+  f[0] = __builtin_fmaf((float)h[0], s, c);
+  f[1] = __builtin_fmaf((float)h[1], s, c);
+  return bitcast<uint32_t>(__builtin_convertvector(f, b2));
+}
+
+// One packed dword (8 weights of one row) -> MFMA B operand.
+__device__ __forceinline__ u4 g4_dequant(uint32_t d, const G4Masks& k, const G4Consts<kRegimeBF16>& q) {
+  const uint32_t d8 = d >> 8;
+  u4 r;
+  r[0] = g4_pair_bf16((d & k.lo) | k.magic, q.s, q.c);
+  r[1] = g4_pair_bf16((d & k.hi) | k.magic, q.s16, q.c16);
+  r[2] = g4_pair_bf16((d8 & k.lo) | k.magic, q.s, q.c);
+  r[3] = g4_pair_bf16((d8 & k.hi) | k.magic, q.s16, q.c16);
+  return r;
+}
+__device__ __forceinline__ u4 g4_dequant(uint32_t d, const G4Masks& k, const G4Consts<kRegimeF16>& q) {
+  u4 r;
+#pragma unroll
+  for (int v = 0; v < 4; ++v) {
+    h2 h = bitcast<h2>(((d >> (4 * v)) & k.lo) | k.magic);
+    h = (h + q.nz) * q.s2;
+    r[v] = bitcast<uint32_t>(h);
+  }
+  return r;
+}
+
+
 }  // namespace woq

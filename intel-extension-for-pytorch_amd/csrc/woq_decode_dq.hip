@@ -1,0 +1,219 @@
+// Decode kernel with per-weight dequantization: 4-bit weights, M <= 16, HBM-bound weight streaming.
+//
+// Reference counterpart: the M >= 5 path of lowp_mode BF16 -- Dequantize<bfloat16> into a bf16
+// block, then a bf16 x bf16 -> fp32 BRGEMM (csrc/cpu/aten/utils/woq.h:1495-1581, 1847-1944) -- at
+// the batch sizes of a decode step.  Each weight becomes w = bf16((q - z) * s) with the scale read
+// as bf16 (fp16 regime: w = fp16((q - z) * s)), exactly as there; the products accumulate in fp32.
+//
+// Same decomposition as the integer-weight decode kernel: a workgroup owns NTW weight row-blocks
+// (16 output columns each) and all of K, its W <= 8 waves take one K tile each per round, the
+// partial sums meet in LDS and are added in wave order.  v_mfma_f32_16x16x32 with A = activations
+// (row m = lane % 16) and B = weights (column n = lane % 16): the dequantized registers of one
+// packed dword are the B operand.
+// The dequantization is ~17 VALU instructions per packed dword, about as much time chip-wide as
+// the weight stream itself, so the rounds are software pipelined: the requests of round r + 1
+// (tiles and parameters into registers, activations into the other LDS buffer) are issued before
+// round r is computed.
+// Activations: a wave copies the 16 rows x 256 bytes of its K tile straight into its private 4 KiB
+// of LDS (global_load_lds_dwordx4: four fully coalesced instructions, no registers) and reads the
+// operand fragments from there; chunk p of row m sits at p ^ m so the fragment reads are
+// conflict-free.  Reading the fragments from global memory directly costs the same number of
+// instructions but each one gathers 64 separate 16-byte pieces, which made the texture addresser
+// the bottleneck (M = 16: 19.7 us against 13.9 us at M = 8 for the same weights).  Rows past M
+// re-read row M - 1 and their results are dropped.  The 64 KiB of slices are reused for the
+// cross-wave sum, so two workgroups fit on a CU.
+#include "woq_common.h"
+#include "woq_internal.h"
+
+namespace woq {
+
+constexpr int kDqSlice = kTileN * kTileK4 * 2;  // one wave's activation slice: 16 rows x 128 K, 4 KiB
+
+struct DecodeDqArgs {
+  FpArgs f;
+  int W;        // waves per workgroup
+  int g_shift;  // log2(group size); 30 for per-channel
+};
+
+template <int REGIME>
+__device__ __forceinline__ f4 dq_mfma(u4 a, u4 b, f4 c) {
+  if constexpr (REGIME == kRegimeF16)
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(bitcast<h8>(a), bitcast<h8>(b), c, 0, 0, 0);
+  else
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(bitcast<b8>(a), bitcast<b8>(b), c, 0, 0, 0);
+}
+
+typedef __attribute__((address_space(3))) void* dq_lds_ptr_t;
+typedef const __attribute__((address_space(1))) void* dq_global_ptr_t;
+
+template <int REGIME, int NTW>
+__global__ __launch_bounds__(512, 4) void woq_decode_dq_kernel(const DecodeDqArgs a) {
+  extern __shared__ __align__(1024) uint8_t smem[];
+  const FpArgs& f = a.f;
+  const int W = a.W;
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+  const int r = lane & 15, c = lane >> 4;
+  const int M = (int)f.M, K = (int)f.K, KT = (int)f.KT, KG = (int)f.KG;
+  const int64_t nt0 = (int64_t)blockIdx.x * NTW;
+  uint8_t* const sx = smem + wave * (2 * kDqSlice);  // this wave's two activation buffers
+  f4* const red = (f4*)smem;                         // [NTW][W][64], after the K loop
+
+  G4Masks km;
+  asm volatile("s_mov_b32 %0, 0x000F000F" : "=s"(km.lo));
+  asm volatile("s_mov_b32 %0, 0x00F000F0" : "=s"(km.hi));
+  asm volatile("v_mov_b32 %0, 0x64006400" : "=v"(km.magic));
+
+  f4 acc[NTW];
+#pragma unroll
+  for (int t = 0; t < NTW; ++t) acc[t] = f4{0.f, 0.f, 0.f, 0.f};
+
+  // wave-uniform bases + one 32-bit per-lane offset per stream.
+  // Activation load i fills LDS bytes [1024 i, +1024) of a buffer: rows 4 i + lane / 16,
+  // physical chunk lane % 16 = logical chunk ^ row.
+  uint32_t xoff[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int row = 4 * i + c;
+    const int rowc = row < M ? row : M - 1;
+    xoff[i] = (uint32_t)(rowc * K + ((r ^ row) & 15) * 8) * 2u;
+  }
+  uint32_t rdo[4];  // fragment j of this lane: row r, logical chunk 4 c + j
+#pragma unroll
+  for (int j = 0; j < 4; ++j) rdo[j] = (uint32_t)(r * 256 + (((c * 4 + j) ^ r) << 4));
+  const uint32_t woff = (uint32_t)lane * 16u;
+  const bool has_z = f.zeros != nullptr;
+  const uint8_t* wbase[NTW];
+  const uint8_t* sbase[NTW];
+  const uint8_t* zbase[NTW];
+#pragma unroll
+  for (int t = 0; t < NTW; ++t) {
+    wbase[t] = f.qweight + (size_t)(nt0 + t) * KT * kTileBytes;
+    sbase[t] = (const uint8_t*)(f.scales + (size_t)(nt0 + t) * KG * kTileN);
+    zbase[t] = has_z ? f.zeros + (size_t)(nt0 + t) * KG * kTileN : sbase[t];
+  }
+
+  u4 wnext[NTW];
+  uint16_t snext[NTW];
+  uint8_t znext[NTW];
+  // every request of one round: activations into LDS buffer `buf`, tiles and parameters into registers
+  auto request = [&](int kt, int buf) {
+    // uniform base + 32-bit offset; groups of four rows that lie entirely past M are not loaded
+    // (their LDS bytes stay undefined: an MFMA output row depends on its own A row only)
+    const uint32_t ko = (uint32_t)kt * (kTileK4 * 2);
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      if (4 * i < M)
+        __builtin_amdgcn_global_load_lds((dq_global_ptr_t)((const uint8_t*)f.x + (uint32_t)(xoff[i] + ko)),
+                                         (dq_lds_ptr_t)(sx + buf * kDqSlice + i * 1024), 16, 0, 0);
+    int g = (kt * kTileK4 + c * 32) >> a.g_shift;
+    g = g < KG ? g : KG - 1;
+    const uint32_t qoff = (uint32_t)(g * kTileN + r);
+    const uint32_t wo = (uint32_t)kt * kTileBytes + woff;
+#pragma unroll
+    for (int t = 0; t < NTW; ++t) {
+      wnext[t] = __builtin_nontemporal_load((const u4*)(wbase[t] + wo));
+      snext[t] = *(const uint16_t*)(sbase[t] + (uint32_t)(qoff * 2u));
+      znext[t] = *(zbase[t] + qoff);  // raw: any use here would wait for the load inside the request
+    }
+  };
+
+  // Rounds: wave w takes K tiles w, w + W, ...; a wave with no tile left idles until the sum.
+  if (wave < KT) request(wave, 0);
+#pragma unroll 1
+  for (int kt = wave, buf = 0; kt < KT; kt += W, buf ^= 1) {
+    u4 wreg[NTW];
+    G4Consts<REGIME> qc[NTW];
+#pragma unroll
+    for (int t = 0; t < NTW; ++t) {
+      wreg[t] = wnext[t];
+      qc[t].set(snext[t], has_z ? (float)znext[t] : 8.0f);
+    }
+    // The compiler does not order LDS reads after the LDS-writing loads: wait for them here.
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+    if (kt + W < KT) request(kt + W, buf ^ 1);
+    __builtin_amdgcn_sched_barrier(0);
+
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const u4 xa = *(const u4*)(sx + buf * kDqSlice + rdo[j]);
+#pragma unroll
+      for (int t = 0; t < NTW; ++t) {
+        const u4 bop = g4_dequant(wreg[t][j], km, qc[t]);
+        acc[t] = dq_mfma<REGIME>(xa, bop, acc[t]);
+      }
+    }
+  }
+
+  // ---- combine the waves' partial sums in wave order, then bias / rounding / store ----
+  __syncthreads();  // every wave is done with its activation slices: the region becomes `red`
+#pragma unroll
+  for (int t = 0; t < NTW; ++t) red[(t * W + wave) * 64 + lane] = acc[t];
+  __syncthreads();
+
+  Epilogue ep{f.bias, f.fusion, f.other0, f.other1, f.out, f.out_dtype, f.x_dtype, f.N};
+  const float* redf = (const float*)red;
+  const bool plain = REGIME == kRegimeBF16 && f.fusion == WOQ_HIP_FUSE_NONE && f.bias == nullptr &&
+                     f.out_dtype == WOQ_HIP_ACT_BF16;
+  // one thread per output element, consecutive threads on consecutive columns; D[m][n] sits in
+  // lane n + 16 (m / 4), register m % 4
+  for (int idx = threadIdx.x; idx < NTW * 256; idx += blockDim.x) {
+    const int col = idx & 15, m = (idx >> 4) & 15, t = idx >> 8;
+    const int64_t n = (nt0 + t) * kTileN + col;
+    if (m >= M || n >= f.N) continue;
+    const int slot = (col + 16 * (m >> 2)) * 4 + (m & 3);
+    float part[8];
+#pragma unroll
+    for (int w = 0; w < 8; ++w) part[w] = w < W ? redf[(t * W + w) * 256 + slot] : 0.0f;
+    float s = part[0];
+#pragma unroll
+    for (int w = 1; w < 8; ++w) s += part[w];
+    if (plain)
+      ((uint16_t*)f.out)[(int64_t)m * f.N + n] = f32_to_bf16_bits(s);
+    else
+      epilogue_store<REGIME>(ep, m, n, s);
+  }
+}
+
+template <int REGIME, int NTW>
+static int launch_dq_cfg(const DecodeDqArgs& a, hipStream_t st) {
+  const size_t smem = (size_t)a.W * 2 * kDqSlice;  // >= NTW * W * 1 KiB of partial sums
+  const unsigned grid = (unsigned)(a.f.NT / NTW);
+  woq_decode_dq_kernel<REGIME, NTW><<<grid, a.W * 64, smem, st>>>(a);
+  return check_launch("woq_decode_dq_kernel");
+}
+
+// 4-bit weights, at most 16 rows already in the compute dtype, whole K tiles, and a group
+// size whose boundaries never split a lane's 32 consecutive K values.
+bool decode_dq_applies(const FpArgs& f, int wbits, int regime) {
+  const int want = regime == kRegimeF16 ? WOQ_HIP_ACT_FP16 : WOQ_HIP_ACT_BF16;
+  if (wbits != 4 || f.M > 16 || f.x_dtype != want || ((uintptr_t)f.x & 15) != 0) return false;
+  if (f.K % kTileK4 != 0 || f.M * f.K * 2 >= (int64_t)1 << 31) return false;
+  if (f.G >= f.KT * kTileK4) return true;
+  return f.G >= 32 && (f.G & (f.G - 1)) == 0;
+}
+
+int launch_decode_dq(const FpArgs& f, int regime, hipStream_t st, int ntw) {
+  DecodeDqArgs a;
+  a.f = f;
+  a.g_shift = 30;
+  if (f.G < f.KT * kTileK4) {
+    a.g_shift = 0;
+    while (((int64_t)1 << a.g_shift) < f.G) ++a.g_shift;
+  }
+  a.W = (int)(f.KT < 8 ? f.KT : 8);
+  if (ntw != 0 && f.NT % ntw != 0)
+    return set_error("woq_decode_dq_kernel: %d row-blocks per workgroup do not divide %lld", ntw, (long long)f.NT);
+  // Two row-blocks per workgroup re-read the activations half as often; with one there are twice
+  // as many workgroups, which small N needs to fill the chip (two workgroups per CU are resident).
+  if (ntw == 0) ntw = (f.NT >= 512 && f.NT % 2 == 0) ? 2 : 1;
+  if (ntw == 4)
+    return regime == kRegimeF16 ? launch_dq_cfg<kRegimeF16, 4>(a, st) : launch_dq_cfg<kRegimeBF16, 4>(a, st);
+  if (ntw == 2)
+    return regime == kRegimeF16 ? launch_dq_cfg<kRegimeF16, 2>(a, st) : launch_dq_cfg<kRegimeBF16, 2>(a, st);
+  if (ntw == 1)
+    return regime == kRegimeF16 ? launch_dq_cfg<kRegimeF16, 1>(a, st) : launch_dq_cfg<kRegimeBF16, 1>(a, st);
+  return set_error("woq_decode_dq_kernel: 1, 2 or 4 row-blocks per workgroup, got %d", ntw);
+}
+
+}  // namespace woq

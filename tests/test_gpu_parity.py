@@ -279,6 +279,57 @@ def test_w4_prefill_kernel_rejects_other_shapes(cuda):
         ctx.run(case["x"].cuda(), force_kernel=3)
 
 
+@pytest.mark.parametrize(
+    "M,K,N,G,bias",
+    [
+        (5, 1024, 64, 128, False),
+        (16, 4096, 1024, 32, True),  # eight waves, four rounds, one group per lane column
+        (8, 512, 48, 64, True),  # fewer K tiles than waves
+        (13, 1152, 96, -1, False),  # per-channel, nine K tiles: a partial last round
+        (16, 128, 16, 128, False),  # a single K tile
+        (3, 256, 80, 256, True),  # bf16 regime is forced below by lowp NONE
+    ],
+)
+@pytest.mark.parametrize("kernel", [7, 8, 9, 10])  # automatic, then 1 / 2 / 4 row-blocks per workgroup
+def test_dequantizing_decode_kernel(cuda, M, K, N, G, bias, kernel):
+    ntw = {7: 1, 8: 1, 9: 2, 10: 4}[kernel]
+    if (N // 16) % ntw:
+        pytest.skip("row-blocks per workgroup must divide N / 16")
+    case = _synthetic().make_int4_case(24, M, K, N, G, bias=bias)
+    lowp = O.LOWP_NONE if M < 5 else O.LOWP_BF16  # bf16 compute at every M
+    _check_fp(case, lowp, force_kernel=kernel, label=f"decode dq M={M} K={K} N={N} G={G} kernel={kernel}")
+
+
+def test_dequantizing_decode_kernel_fp16_regime_and_symmetric(cuda):
+    """fp16 regime with a group size the integer-weight decode kernel does not take, and weights
+    without zero points."""
+    syn = _synthetic()
+    M, K, N, G = 11, 1024, 96, 32
+    case = syn.make_int4_case(25, M, K, N, G, bias=True, scale_dtype=torch.float16)
+    case["x"] = case["x"].to(torch.float16)
+    ctx = make_context(case, O.LOWP_FP16)
+    x = case["x"].cuda()
+    y = to_np_f32(ctx.run(x, force_kernel=7))
+    acc = ctx.run(x, out_fp32=True, force_kernel=7).cpu().numpy()
+    c = case_np(case)
+    acc_ref, y_ref = O.woq_linear_ref(c["x"], "fp16", c["qw"], N, K, c["scales"], c["zps"], c["bias"], 2, G, "fp16")
+    assert max_abs(acc, acc_ref) <= MAX_ABS_ACC
+    assert rel_l2(y, y_ref) <= REL_L2_OUT
+    case = _synthetic().make_int4_case(26, 9, 768, 64, 128)
+    case["zeros"] = None
+    _check_fp(case, O.LOWP_BF16, force_kernel=7, label="decode dq, symmetric")
+
+
+def test_dequantizing_decode_kernel_close_to_small_m_kernel(cuda):
+    case = _synthetic().make_int4_case(27, 16, 2048, 1024, 128, bias=True)
+    ctx = make_context(case, O.LOWP_BF16)
+    x = case["x"].cuda()
+    a, b = to_np_f32(ctx.run(x, force_kernel=7)), to_np_f32(ctx.run(x, force_kernel=1))
+    assert bool(np.all((bf16_ulp_diff(a, b) <= 1) | (np.abs(a - b) <= 1e-4)))
+    with pytest.raises(RuntimeError, match="dequantizing decode kernel"):
+        ctx.run(torch.randn(17, 2048, device=cuda).bfloat16(), force_kernel=7)
+
+
 def test_int8_weights_small_and_tiled(cuda):
     for M in (1, 8, 40, 200):
         case = _synthetic().make_int8_case(16, M, 512, 144)
