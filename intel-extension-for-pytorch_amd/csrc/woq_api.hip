@@ -160,7 +160,7 @@ int woq_hip_linear(const woq_hip_linear_params* p) {
   if (lowp == WOQ_HIP_LOWP_INT8) {
     const int64_t bk = woq_hip_int8_block_k(p->group_size, p->K);
     const bool blocks_ok = bk == 32 || bk == 64 || bk == 128;
-    const bool mode_ok = p->act_quant_mode >= WOQ_HIP_QUANT_A_PER_TENSOR_SYM &&
+    const bool mode_ok = p->act_quant_mode >= WOQ_HIP_QUANT_A_PER_TENSOR &&
                          p->act_quant_mode <= WOQ_HIP_QUANT_A_PER_M_K_BLOCK_SYM;
     if (p->weight_dtype == WOQ_HIP_DTYPE_INT8 && p->zeros_u8)
       return set_error("woq_linear: symmetric quantization is required for INT8 weights with lowp_mode INT8");
@@ -170,8 +170,7 @@ int woq_hip_linear(const woq_hip_linear_params* p) {
       // (csrc/cpu/aten/kernels/WoqInt8GemmAPerMKrnl.cpp:143-169).
       lowp = WOQ_HIP_LOWP_NONE;
     } else if (!mode_ok) {
-      return set_error("woq_linear: act_quant_mode %d is not supported (symmetric modes 4..7 only)",
-                       p->act_quant_mode);
+      return set_error("woq_linear: lowp_mode INT8 needs an act_quant_mode in 0..7, got %d", p->act_quant_mode);
     } else {
       Int8Args a;
       a.x = p->x; a.x_dtype = p->x_dtype; a.M = p->M; a.K = p->K; a.N = p->N; a.NT = NT; a.KT = KT;

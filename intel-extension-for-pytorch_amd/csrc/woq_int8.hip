@@ -79,13 +79,84 @@ __global__ __launch_bounds__(256) void act_stats_kernel(const void* __restrict__
   }
 }
 
+// ---- statistics of groups that span all rows (per-tensor, per-K-block modes) ----------------
+// One workgroup per group would scan M * K (or M * qbk) elements alone.  Instead many workgroups
+// scan 8 rows x one K range each and combine through integer atomics on an order-preserving key
+// of the float (min / max are exact in any order, so the result is deterministic).  The keys live
+// in the output arrays themselves: max (or max |x| for the symmetric modes) in `scales`, min in
+// `zps`; a last pass turns them into scale and zero point in place.
+__device__ __forceinline__ int32_t float_key(float f) {
+  const int32_t b = bitcast<int32_t>(f);
+  return b ^ ((b >> 31) & 0x7fffffff);
+}
+__device__ __forceinline__ float key_float(int32_t k) { return bitcast<float>(k ^ ((k >> 31) & 0x7fffffff)); }
+
+__global__ void act_stats_init_kernel(int64_t groups, int32_t* __restrict__ maxk, int32_t* __restrict__ mink) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= groups) return;
+  maxk[i] = float_key(-__builtin_inff());
+  if (mink) mink[i] = float_key(__builtin_inff());
+}
+
+constexpr int kStatRows = 8, kStatChunk = 2048;
+
+__global__ __launch_bounds__(256) void act_stats_partial_kernel(const void* __restrict__ x, int x_dtype, int64_t M,
+                                                                int64_t K, int64_t qbk, int per_k, int sym,
+                                                                int32_t* __restrict__ maxk,
+                                                                int32_t* __restrict__ mink) {
+  // blockIdx.x: K range (a quantization block, or a chunk of the row for per-tensor), blockIdx.y: 8 rows
+  const int64_t kw = per_k ? qbk : kStatChunk;
+  const int64_t k_lo = (int64_t)blockIdx.x * kw;
+  const int64_t k_hi = k_lo + kw < K ? k_lo + kw : K;
+  const int64_t m_lo = (int64_t)blockIdx.y * kStatRows;
+  const int64_t m_hi = m_lo + kStatRows < M ? m_lo + kStatRows : M;
+  const int64_t w = k_hi - k_lo, total = (m_hi - m_lo) * w;
+  float mn = __builtin_inff(), mx = -__builtin_inff();
+  for (int64_t i = threadIdx.x; i < total; i += blockDim.x) {
+    const float v = load_act(x, x_dtype, (m_lo + i / w) * K + k_lo + i % w);
+    mn = fminf(mn, v);
+    mx = fmaxf(mx, v);
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+    mn = fminf(mn, __shfl_xor(mn, off));
+    mx = fmaxf(mx, __shfl_xor(mx, off));
+  }
+  if ((threadIdx.x & 63) == 0 && mx >= mn) {  // a wave that saw no element still holds (+inf, -inf)
+    const int64_t g = per_k ? blockIdx.x : 0;
+    if (sym) {
+      atomicMax(maxk + g, float_key(fmaxf(fabsf(mx), fabsf(mn))));
+    } else {
+      atomicMax(maxk + g, float_key(mx));
+      atomicMin(mink + g, float_key(mn));
+    }
+  }
+}
+
+__global__ void act_stats_finalize_kernel(int64_t groups, int sym, float* __restrict__ scales,
+                                          int32_t* __restrict__ zps) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= groups) return;
+  const float mx = key_float(bitcast<int32_t>(scales[i]));
+  if (sym) {
+    scales[i] = __fdiv_rn(mx, 127.0f);
+  } else {
+    const float mn = key_float(zps[i]);
+    const float s = __fdiv_rn(__fsub_rn(mx, mn), 255.0f);
+    scales[i] = s;
+    zps[i] = (int32_t)(-rintf(__fdiv_rn(mn, s)));
+  }
+}
+
 // ---- quantize: one thread per 8 consecutive K elements -------------------------------------
 // ldq: row stride of q in bytes (>= K, the tail is zero-filled up to ldq).
 // permute: store each group of 8 as [e0 e4 e1 e5 e2 e6 e3 e7], the byte order the 4-bit decode
-// produces, so the int8 kernels can use the activations without a shuffle.
+// produces, so the int8 kernels can use the activations without a shuffle.  Padding bytes up to
+// ldq hold 0 (symmetric) or, with offset128, whatever: the weights there are padded with q = z.
 __global__ void act_quant_kernel(const void* __restrict__ x, int x_dtype, int64_t M, int64_t K, int64_t ldq,
                                  int64_t qbk, int64_t Kc, int mode, const float* __restrict__ scales,
-                                 const int32_t* __restrict__ zps, uint8_t* __restrict__ q, int permute) {
+                                 const int32_t* __restrict__ zps, uint8_t* __restrict__ q, int permute,
+                                 int offset128) {
   const int64_t g8 = ldq / 8;
   const int64_t gid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (gid >= M * g8) return;
@@ -106,7 +177,8 @@ __global__ void act_quant_kernel(const void* __restrict__ x, int x_dtype, int64_
       const float lo = sym ? -128.0f : 0.0f, hi = sym ? 127.0f : 255.0f;
       t = fminf(fmaxf(t, lo), hi);
       if (s == 0.0f || t != t) t = sym ? 0.0f : zp;  // all-zero group: the reference divides 0 by 0
-      b = sym ? (uint8_t)(int8_t)(int)t : (uint8_t)(int)t;
+      // offset128: the asymmetric value 0..255 stored as the int8 number q - 128 for the signed MFMA
+      b = sym ? (uint8_t)(int8_t)(int)t : (uint8_t)((int)t ^ (offset128 ? 0x80 : 0));
     }
     o[e] = b;
   }
@@ -127,22 +199,37 @@ static int64_t num_quant_groups(int64_t M, int64_t Kc, int mode) {
 }
 
 static int launch_quant_impl(const void* x, int x_dtype, int64_t M, int64_t K, int64_t ldq, int64_t qbk,
-                             int mode, void* q, float* scales, int32_t* zps, int permute, hipStream_t st) {
+                             int mode, void* q, float* scales, int32_t* zps, int permute, int offset128,
+                             hipStream_t st) {
   if (M == 0 || K == 0) return 0;
   if (qbk <= 0) qbk = K;
   const int64_t Kc = (K + qbk - 1) / qbk;
   const int64_t groups = num_quant_groups(M, Kc, mode);
-  act_stats_kernel<<<(unsigned)groups, 256, 0, st>>>(x, x_dtype, M, K, qbk, Kc, mode, scales, zps);
-  if (int rc = check_launch("act_stats_kernel")) return rc;
+  if (quant_a_per_m(mode)) {
+    act_stats_kernel<<<(unsigned)groups, 256, 0, st>>>(x, x_dtype, M, K, qbk, Kc, mode, scales, zps);
+    if (int rc = check_launch("act_stats_kernel")) return rc;
+  } else {
+    const int sym = quant_a_is_sym(mode), per_k = quant_a_per_k(mode);
+    if (!sym && zps == nullptr) return set_error("dynamic_quant: asymmetric modes need a zero-point array");
+    int32_t* maxk = (int32_t*)scales;
+    int32_t* mink = sym ? nullptr : zps;
+    act_stats_init_kernel<<<(unsigned)((groups + 255) / 256), 256, 0, st>>>(groups, maxk, mink);
+    if (int rc = check_launch("act_stats_init_kernel")) return rc;
+    dim3 grid((unsigned)(per_k ? Kc : (K + kStatChunk - 1) / kStatChunk), (unsigned)((M + kStatRows - 1) / kStatRows));
+    act_stats_partial_kernel<<<grid, 256, 0, st>>>(x, x_dtype, M, K, qbk, per_k, sym, maxk, mink);
+    if (int rc = check_launch("act_stats_partial_kernel")) return rc;
+    act_stats_finalize_kernel<<<(unsigned)((groups + 255) / 256), 256, 0, st>>>(groups, sym, scales, zps);
+    if (int rc = check_launch("act_stats_finalize_kernel")) return rc;
+  }
   const int64_t total = M * (ldq / 8);
   act_quant_kernel<<<(unsigned)((total + 255) / 256), 256, 0, st>>>(x, x_dtype, M, K, ldq, qbk, Kc, mode,
-                                                                    scales, zps, (uint8_t*)q, permute);
+                                                                    scales, zps, (uint8_t*)q, permute, offset128);
   return check_launch("act_quant_kernel");
 }
 
 int launch_dynamic_quant(const void* x, int x_dtype, int64_t M, int64_t K, int64_t ldq, int64_t qbk, int mode,
                          void* q, float* scales, int32_t* zps, hipStream_t st) {
-  return launch_quant_impl(x, x_dtype, M, K, ldq, qbk, mode, q, scales, zps, 0, st);
+  return launch_quant_impl(x, x_dtype, M, K, ldq, qbk, mode, q, scales, zps, 0, 0, st);
 }
 
 // ---- weight nibbles / bytes -> int8 (q - z) --------------------------------------------------
@@ -177,7 +264,9 @@ struct Int8KArgs {
   const uint8_t* xq;   // [M][ldq]
   int64_t ldq;
   const float* sa;     // activation scales
+  const int32_t* za;   // activation zero points (asymmetric modes), indexed like sa
   int64_t sa_m_stride, sa_k_stride, qbk;
+  int sa_kc;           // activation-scale groups along K (1 unless the mode is per K block)
   int64_t block_k;     // K block of the int32 accumulation
   int W;
   int64_t Kpad;
@@ -331,12 +420,20 @@ __global__ __launch_bounds__(1024) void woq_small_m_i8_kernel(const Int8KArgs p)
 constexpr int IBM = 128, IBN = 128, IBK = 128;
 constexpr int ILDS = IBK + 16;
 
-template <int WBITS, int BLOCK_K, bool PER_K, bool DEBUG>
+// ASYM: asymmetric activations (uint8 q_a with zero point zp_a; csrc/cpu/aten/utils/woq.h:2172-2186).
+// The activations arrive as int8 q_a - 128, the zero points are used as zp_a - 128, and the weight
+// column sums of the K block ("compensation") come from one more MFMA against a row of ones:
+// (sum (q_a - 128) B) - (zp_a - 128) sum B = sum q_a B - zp_a sum B, exactly the reference's integer.
+template <int WBITS, int BLOCK_K, bool PER_K, bool DEBUG, bool ASYM>
 __global__ __launch_bounds__(256) void woq_gemm_i8_kernel(const Int8KArgs p) {
+  static_assert(!ASYM || PER_K, "the asymmetric variant reloads scales and zero points per K block");
   constexpr int TK = WBITS == 4 ? kTileK4 : kTileK8;
   const Int8Args& a = p.a;
   __shared__ __align__(16) uint8_t sA[IBM * ILDS];
   __shared__ __align__(16) uint8_t sB[IBN * ILDS];
+  // activation scales of the K blocks of one step (per-K-block modes): [IBK / BLOCK_K][IBM]
+  __shared__ __align__(16) float sSA[PER_K ? (IBK / BLOCK_K) * IBM : 4];
+  __shared__ __align__(16) int32_t sZA[ASYM ? (IBK / BLOCK_K) * IBM : 4];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave >> 1, wn = wave & 1;
   const int64_t m0 = (int64_t)blockIdx.y * IBM, n0 = (int64_t)blockIdx.x * IBN;
@@ -358,6 +455,7 @@ __global__ __launch_bounds__(256) void woq_gemm_i8_kernel(const Int8KArgs p) {
   const int ncol0 = (int)n0 + wn * 64 + (lane & 31);
   // activation scales of those rows; constant over K unless the mode is per K block
   float sa_reg[2][16];
+  int za_reg[ASYM ? 2 : 1][16];
 #pragma unroll
   for (int i = 0; i < 2; ++i)
 #pragma unroll
@@ -420,7 +518,31 @@ __global__ __launch_bounds__(256) void woq_gemm_i8_kernel(const Int8KArgs p) {
         wo[q][0] = bitcast<u4>(decode16_i8<8>((const uint32_t*)&wv, z4));
       }
     }
+    // per-K-block activation scales of this step: one coalesced pass into LDS instead of 32
+    // strided loads per thread and block
+    float sa_stage[PER_K ? (IBK / BLOCK_K) * IBM / 256 + 1 : 1];
+    int32_t za_stage[ASYM ? (IBK / BLOCK_K) * IBM / 256 + 1 : 1];
+    if (PER_K) {
+#pragma unroll
+      for (int q = 0; q * 256 < (IBK / BLOCK_K) * IBM; ++q) {
+        const int idx = tid + 256 * q;
+        const int sb = idx / IBM, row = idx % IBM;
+        const int64_t m = m0 + row < a.M ? m0 + row : a.M - 1;
+        int kcol = (int)((unsigned)((int)k0 + sb * BLOCK_K) / (unsigned)p.qbk);
+        kcol = kcol < p.sa_kc ? kcol : p.sa_kc - 1;  // K blocks of the padding past K
+        sa_stage[q] = idx < (IBK / BLOCK_K) * IBM ? p.sa[m * p.sa_m_stride + kcol] : 0.0f;
+        if (ASYM) za_stage[q] = idx < (IBK / BLOCK_K) * IBM ? p.za[m * p.sa_m_stride + kcol] - 128 : 0;
+      }
+    }
     __syncthreads();
+    if (PER_K) {
+#pragma unroll
+      for (int q = 0; q * 256 < (IBK / BLOCK_K) * IBM; ++q)
+        if (tid + 256 * q < (IBK / BLOCK_K) * IBM) {
+          sSA[tid + 256 * q] = sa_stage[q];
+          if (ASYM) sZA[tid + 256 * q] = za_stage[q];
+        }
+    }
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int row = (tid >> 3) + 32 * i;
@@ -442,6 +564,15 @@ __global__ __launch_bounds__(256) void woq_gemm_i8_kernel(const Int8KArgs p) {
         for (int j = 0; j < 2; ++j)
 #pragma unroll
           for (int e = 0; e < 16; ++e) qc[i][j][e] = 0;
+      i16v qcomp[2];  // column sums of the weights of this K block (every row of the tile alike)
+      if (ASYM) {
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+          for (int e = 0; e < 16; ++e) qcomp[j][e] = 0;
+      }
+      const int ones1 = 0x01010101;
+      const i4 ones = i4{ones1, ones1, ones1, ones1};
       const int kbeg = sb * BLOCK_K;
 #pragma unroll
       for (int ks = 0; ks < BLOCK_K; ks += 32) {
@@ -456,19 +587,33 @@ __global__ __launch_bounds__(256) void woq_gemm_i8_kernel(const Int8KArgs p) {
 #pragma unroll
           for (int j = 0; j < 2; ++j)
             qc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[i], bf[j], qc[i][j], 0, 0, 0);
+        if (ASYM) {
+          // padded K positions hold weights q = 0, not q = z: keep them out of the column sums
+          const bool in_k = (int)k0 + kbeg + ks + (lane >> 5) * 16 < (int)a.K;
+          const i4 ones_k = in_k ? ones : i4{0, 0, 0, 0};
+#pragma unroll
+          for (int j = 0; j < 2; ++j)
+            qcomp[j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(ones_k, bf[j], qcomp[j], 0, 0, 0);
+        }
       }
       // fp32 epilogue of this K block: C += (float(qC) * s_a[m]) * s_w[n, g]
       const int kq = (int)k0 + kbeg;
       int g = (int)((unsigned)kq / (unsigned)a.G);
       if (g >= (int)a.KG) g = (int)a.KG - 1;
       if (PER_K) {
-        const int kcol = (int)((unsigned)kq / (unsigned)p.qbk);
 #pragma unroll
         for (int i = 0; i < 2; ++i)
 #pragma unroll
-          for (int e = 0; e < 16; ++e) {
-            const int m = mrow0 + i * 32 + 8 * (e >> 2) + (e & 3);
-            sa_reg[i][e] = p.sa[(int64_t)(m < (int)a.M ? m : (int)a.M - 1) * p.sa_m_stride + kcol];
+          for (int e4 = 0; e4 < 4; ++e4) {
+            // rows wm * 64 + 32 i + 8 e4 + 4 (lane / 32) + 0..3 of the workgroup tile
+            const f4 v = *(const f4*)(sSA + sb * IBM + wm * 64 + i * 32 + 8 * e4 + 4 * (lane >> 5));
+#pragma unroll
+            for (int e = 0; e < 4; ++e) sa_reg[i][4 * e4 + e] = v[e];
+            if (ASYM) {
+              const i4 z = *(const i4*)(sZA + sb * IBM + wm * 64 + i * 32 + 8 * e4 + 4 * (lane >> 5));
+#pragma unroll
+              for (int e = 0; e < 4; ++e) za_reg[i][4 * e4 + e] = z[e];
+            }
           }
       }
 #pragma unroll
@@ -480,12 +625,15 @@ __global__ __launch_bounds__(256) void woq_gemm_i8_kernel(const Int8KArgs p) {
         for (int i = 0; i < 2; ++i) {
 #pragma unroll
           for (int e = 0; e < 16; ++e) {
-            const float cterm = __fmul_rn(__fmul_rn((float)qc[i][j][e], sa_reg[i][e]), sw);
+            const int qv = ASYM ? qc[i][j][e] - qcomp[j][e] * za_reg[i][e] : qc[i][j][e];
+            const float cterm = __fmul_rn(__fmul_rn((float)qv, sa_reg[i][e]), sw);
             acc[i][j][e] = __fadd_rn(acc[i][j][e], cterm);
             if (DEBUG) {
+              // the block sum as the reference defines it: unsigned activations times weights
               const int64_t m = mrow0 + i * 32 + 8 * (e >> 2) + (e & 3);
               if (m < a.M && n < a.N)
-                a.debug_block_sums[(m * a.N + n) * (p.Kpad / BLOCK_K) + kq / BLOCK_K] = qc[i][j][e];
+                a.debug_block_sums[(m * a.N + n) * (p.Kpad / BLOCK_K) + kq / BLOCK_K] =
+                    ASYM ? qc[i][j][e] + 128 * qcomp[j][e] : qc[i][j][e];
             }
           }
         }
@@ -547,9 +695,9 @@ static int dispatch_small_i8(Int8KArgs& p, hipStream_t st) {
 
 int launch_int8_linear(const Int8Args& a, hipStream_t st) {
   const int mode = a.act_quant_mode;
-  if (!quant_a_is_sym(mode) || mode > WOQ_HIP_QUANT_A_PER_M_K_BLOCK_SYM)
-    return set_error(
-        "lowp_mode INT8: act_quant_mode %d is not supported by this build (symmetric modes 4..7 only)", mode);
+  if (mode < WOQ_HIP_QUANT_A_PER_TENSOR || mode > WOQ_HIP_QUANT_A_PER_M_K_BLOCK_SYM)
+    return set_error("lowp_mode INT8: bad act_quant_mode %d", mode);
+  const bool asym = !quant_a_is_sym(mode);
   const int TK = a.wbits == 4 ? kTileK4 : kTileK8;
   Int8KArgs p;
   p.a = a;
@@ -567,37 +715,45 @@ int launch_int8_linear(const Int8Args& a, hipStream_t st) {
   p.sa_m_stride = per_m ? (per_k ? Kc : 1) : 0;
   p.sa_k_stride = per_k ? 1 : 0;
   if (!per_k) p.qbk = p.Kpad + 1;  // k / qbk == 0 for every k
+  p.sa_kc = per_k ? (int)Kc : 1;
 
-  // workspace: q [M][ldq] | scales [groups] | (zps unused for symmetric modes)
+  // workspace: q [M][ldq] | scales [groups] | zero points [groups] (asymmetric modes)
   const int64_t qbytes = (a.M * p.ldq + 255) / 256 * 256;
   const int64_t groups = (per_m ? a.M : 1) * (per_k ? Kc : 1);
-  const int64_t need = qbytes + groups * (int64_t)sizeof(float);
+  const int64_t need = qbytes + groups * (int64_t)(sizeof(float) + (asym ? sizeof(int32_t) : 0));
   if (a.workspace == nullptr || a.workspace_bytes < need)
     return set_error("lowp_mode INT8: workspace too small (%lld < %lld bytes)", (long long)a.workspace_bytes,
                      (long long)need);
   uint8_t* xq = (uint8_t*)a.workspace;
   float* sa = (float*)((uint8_t*)a.workspace + qbytes);
+  int32_t* za = asym ? (int32_t*)(sa + groups) : nullptr;
   p.xq = xq;
   p.sa = sa;
+  p.za = za;
   const int64_t qbk_quant = per_k ? (per_channel ? p.block_k : G) : a.K;
-  if (int rc = launch_quant_impl(a.x, a.x_dtype, a.M, a.K, p.ldq, qbk_quant, mode, xq, sa, nullptr,
-                                 a.wbits == 4 ? 1 : 0, st))
+  if (int rc = launch_quant_impl(a.x, a.x_dtype, a.M, a.K, p.ldq, qbk_quant, mode, xq, sa, za,
+                                 a.wbits == 4 ? 1 : 0, asym ? 1 : 0, st))
     return rc;
 
   // The small-M kernel accumulates whole tiles per MFMA, so it needs K blocks that are whole
   // tiles; finer blocks (group_size 32 / 64 with 4-bit weights) go through the tiled kernel,
   // which re-lays the weights in LDS in plain K order.
-  if (a.M <= 64 && p.block_k % TK == 0)
+  // Asymmetric activations (rare: the reference's default is symmetric) always take the tiled kernel.
+  if (!asym && a.M <= 64 && p.block_k % TK == 0)
     return a.wbits == 4 ? dispatch_small_i8<4>(p, st) : dispatch_small_i8<8>(p, st);
   dim3 grid((unsigned)((a.NT * kTileN + IBN - 1) / IBN), (unsigned)((a.M + IBM - 1) / IBM));
   const bool dbg = a.debug_block_sums != nullptr;
 #define WOQ_I8_GEMM_B(WB, BK)                                                            \
-  if (dbg)                                                                               \
-    woq_gemm_i8_kernel<WB, BK, true, true><<<grid, 256, 0, st>>>(p);                     \
+  if (asym && dbg)                                                                       \
+    woq_gemm_i8_kernel<WB, BK, true, true, true><<<grid, 256, 0, st>>>(p);               \
+  else if (asym)                                                                         \
+    woq_gemm_i8_kernel<WB, BK, true, false, true><<<grid, 256, 0, st>>>(p);              \
+  else if (dbg)                                                                          \
+    woq_gemm_i8_kernel<WB, BK, true, true, false><<<grid, 256, 0, st>>>(p);              \
   else if (per_k)                                                                        \
-    woq_gemm_i8_kernel<WB, BK, true, false><<<grid, 256, 0, st>>>(p);                    \
+    woq_gemm_i8_kernel<WB, BK, true, false, false><<<grid, 256, 0, st>>>(p);             \
   else                                                                                   \
-    woq_gemm_i8_kernel<WB, BK, false, false><<<grid, 256, 0, st>>>(p);
+    woq_gemm_i8_kernel<WB, BK, false, false, false><<<grid, 256, 0, st>>>(p);
 #define WOQ_I8_GEMM(WB)                                   \
   switch (p.block_k) {                                    \
     case 32: { WOQ_I8_GEMM_B(WB, 32) } break;             \

@@ -274,6 +274,26 @@ def dynamic_quantize_per_block(x, quant_block_k, mode):
     return q, scales, (None if sym else zps)
 
 
+def _int8_weights(qw, N, K, zps, weight_dtype, group_size):
+    """B[n, k] = q - z as integers (the int8 operand of the lowp-INT8 kernels, woq.h:1701-1704,
+    614-625)."""
+    if weight_dtype == WOQ_DTYPE_INT4:
+        q = unpack_int4(qw)[:, :K].astype(np.int64)
+        if zps is None:
+            return q - 8
+        z = np.asarray(zps).reshape(N, -1).astype(np.int64)
+        g = (np.arange(K) // group_size) if group_size > 0 else np.zeros(K, dtype=np.int64)
+        return q - z[:, g]
+    return np.asarray(qw, dtype=np.int8).astype(np.int64)
+
+
+def int8_weight_block_sums(qw, N, K, zps, weight_dtype, group_size, block_k):
+    """compensation[n, kb] = sum_{k in block kb} (q[n, k] - z[n, g(k)]) (woq.h:1679-1727)."""
+    B = _int8_weights(qw, N, K, zps, weight_dtype, group_size)
+    KB = K // block_k
+    return B[:, : KB * block_k].reshape(N, KB, block_k).sum(axis=2).astype(np.int32)
+
+
 def int8_block_sums(xq, qw, N, K, zps, weight_dtype, group_size, block_k):
     """Exact int32 sums qC[m, n, kb] = sum_{k in block kb} xq[m, k] * (q[n, k] - z[n, g(k)])."""
     if weight_dtype == WOQ_DTYPE_INT4:
@@ -297,30 +317,40 @@ def int8_block_sums(xq, qw, N, K, zps, weight_dtype, group_size, block_k):
 
 
 def woq_linear_opt_int8(x, act_dtype, qw, N, K, scales, zps, bias, weight_dtype, group_size, act_quant_mode):
-    """lowp_mode INT8 with symmetric activation quantization (modes 4..7).
-    C = fp32 bias or 0; for each K block kb ascending: C += (float(qC[kb]) * s_a) * s_w[n, g(kb)].
-    Returns dict(xq, sa, sums, acc (fp32), y)."""
-    assert act_quant_mode >= 4
+    """lowp_mode INT8.  C = fp32 bias or 0; for each K block kb ascending:
+    C += (float(qC[kb]) * s_a) * s_w[n, g(kb)] for the symmetric activation modes 4..7, and
+    C += (float(qC[kb] - compensation[n, kb] * zp_a) * s_a) * s_w[n, g(kb)] for the asymmetric
+    modes 0..3 (integer subtraction first, woq.h:2172-2186).  Returns dict(xq, sa, za, sums, acc
+    (fp32), y)."""
     M = x.shape[0]
+    asym = act_quant_mode < 4
     bk = int8_block_k(group_size, K)
     qbk = group_size if group_size > 0 else bk
-    xq, sa, _ = dynamic_quantize_per_block(x, qbk, act_quant_mode)
+    xq, sa, za = dynamic_quantize_per_block(x, qbk, act_quant_mode)
     sums = int8_block_sums(xq, qw, N, K, zps, weight_dtype, group_size, bk)
     s = np.asarray(scales, dtype=np.float32).reshape(N, -1)
-    per_m = act_quant_mode in (6, 7)
-    per_k = act_quant_mode in (5, 7)
+    per_m = act_quant_mode in (2, 3, 6, 7)
+    per_k = act_quant_mode in (1, 3, 5, 7)
     Kc = (K + qbk - 1) // qbk
     sa2 = np.asarray(sa, dtype=np.float32).reshape(M if per_m else 1, Kc if per_k else 1)
+    if asym:
+        comp = int8_weight_block_sums(qw, N, K, zps, weight_dtype, group_size, bk).astype(np.int64)
+        za2 = np.asarray(za, dtype=np.int64).reshape(M if per_m else 1, Kc if per_k else 1)
     C = np.zeros((M, N), dtype=np.float32)
     if bias is not None:
         C[:] = np.asarray(bias, dtype=np.float32)[None, :]
     for kb in range(K // bk):
         g = (kb * bk) // group_size if group_size > 0 else 0
-        sa_col = sa2[:, (kb * bk) // qbk if per_k else 0].reshape(-1, 1)
-        c = (sums[:, :, kb].astype(np.float32) * sa_col).astype(np.float32)
+        kc = (kb * bk) // qbk if per_k else 0
+        sa_col = sa2[:, kc].reshape(-1, 1)
+        qv = sums[:, :, kb].astype(np.int64)
+        if asym:
+            qv = qv - comp[:, kb][None, :] * za2[:, kc].reshape(-1, 1)
+            assert np.abs(qv).max() < 2**31
+        c = (qv.astype(np.float32) * sa_col).astype(np.float32)
         c = (c * s[:, g][None, :]).astype(np.float32)
         C = (C + c).astype(np.float32)
-    return {"xq": xq, "sa": sa, "sums": sums, "acc": C, "y": _round_to(C, act_dtype)}
+    return {"xq": xq, "sa": sa, "za": za, "sums": sums, "acc": C, "y": _round_to(C, act_dtype)}
 
 
 def woq_linear(x, act_dtype, qw, N, K, scales, zps, bias, weight_dtype, group_size, lowp_mode, act_quant_mode=-1,

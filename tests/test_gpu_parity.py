@@ -362,7 +362,7 @@ def test_empty_batch(cuda):
 # ---------------------------------------------------------------------------------------------
 # lowp_mode INT8
 # ---------------------------------------------------------------------------------------------
-@pytest.mark.parametrize("mode", [4, 5, 6, 7])
+@pytest.mark.parametrize("mode", [0, 1, 2, 3, 4, 5, 6, 7])
 @pytest.mark.parametrize("M,K", [(1, 512), (37, 4096), (300, 1024)])
 def test_dynamic_quant_bit_exact(cuda, mode, M, K):
     k = _kernels()
@@ -370,9 +370,11 @@ def test_dynamic_quant_bit_exact(cuda, mode, M, K):
     x[0, :5] = torch.tensor([0.5, -0.5, 1.5, 2.5, 1e-3])
     x = x.to(torch.bfloat16)
     q, s, zp = k.dynamic_quant(x.to(cuda), 128, mode)
-    q_ref, s_ref, _ = O.dynamic_quantize_per_block(to_np_f32(x), 128, mode)
-    assert np.array_equal(s.cpu().numpy(), s_ref)
+    q_ref, s_ref, zp_ref = O.dynamic_quantize_per_block(to_np_f32(x), 128, mode)
+    assert np.array_equal(s.cpu().numpy().reshape(-1), s_ref.reshape(-1))
     assert np.array_equal(q.cpu().numpy(), q_ref)
+    if mode < 4:
+        assert np.array_equal(zp.cpu().numpy().reshape(-1), zp_ref.reshape(-1))
 
 
 def test_dynamic_quant_all_bf16_patterns(cuda):
@@ -423,6 +425,21 @@ def _check_int8(case, mode, cols=None, debug=True, label=""):
 def test_int8_lowp_int4_g128(cuda, mode, M):
     case = _synthetic().make_int4_case(20, M, 1024, 272, 128, bias=True, outliers=True)
     _check_int8(case, mode, label=f"int8 lowp mode={mode} M={M}")
+
+
+@pytest.mark.parametrize("mode", [0, 1, 2, 3])
+@pytest.mark.parametrize("M,K,N,G", [(1, 1024, 272, 128), (37, 512, 144, 32), (150, 1024, 272, 128), (20, 768, 80, -1)])
+def test_int8_lowp_asymmetric_activations(cuda, mode, M, K, N, G):
+    """uint8 activations with a zero point: block sums bit-exact (as the reference defines them,
+    unsigned activations times weights), compensation applied in integers."""
+    case = _synthetic().make_int4_case(28, M, K, N, G, bias=True, outliers=True)
+    case["x"] = (case["x"].float() + 0.5).to(torch.bfloat16)  # off-centre: zero points far from 128
+    _check_int8(case, mode, label=f"int8 lowp asym mode={mode} M={M} K={K} N={N} G={G}")
+
+
+def test_int8_lowp_asymmetric_activations_int8_weights(cuda):
+    case = _synthetic().make_int8_case(29, 70, 512, 80)
+    _check_int8(case, 2, label="int8 lowp asym, int8 weights")
 
 
 @pytest.mark.parametrize("G", [32, 64, -1, 256])

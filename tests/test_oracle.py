@@ -251,6 +251,40 @@ def test_int8_linear_epilogue_close_to_exact():
     assert np.max(np.abs(r["acc"] - want)) < 1e-5
 
 
+@pytest.mark.parametrize("mode", [0, 1, 2, 3])
+def test_int8_linear_asymmetric_activations_is_the_dequantized_product(mode):
+    """Pins the compensation term (its sign, its block index, which zero point multiplies it):
+    sum_k (q_a - zp_a) s_a (q_w - z_w) s_w, evaluated exactly from the quantized tensors, must be
+    what the integer-compensation form gives; a wrong sign or index is off by whole units."""
+    x, q, qw, scales, zps, b = _tiny_case(M=6, N=5, K=256, G=128, seed=11)
+    x = x + np.float32(0.75)  # an offset makes the zero points large
+    r = O.woq_linear_opt_int8(x, "bf16", qw, 5, 256, scales, zps, b, O.WOQ_DTYPE_INT4, 128, mode)
+    assert r["xq"].dtype == np.uint8 and r["za"] is not None
+    per_m, per_k = mode in (2, 3), mode in (1, 3)
+    sa = np.asarray(r["sa"], dtype=np.float64).reshape(6 if per_m else 1, 2 if per_k else 1)
+    za = np.asarray(r["za"], dtype=np.float64).reshape(6 if per_m else 1, 2 if per_k else 1)
+    kcol = (np.arange(256) // 128) if per_k else np.zeros(256, dtype=np.int64)
+    xdq = (r["xq"].astype(np.float64) - za[:, kcol]) * sa[:, kcol]  # broadcasts over rows if not per_m
+    g = np.arange(256) // 128
+    wdq = (q.astype(np.float64) - zps.astype(np.float64)[:, g]) * scales.astype(np.float64)[:, g]
+    want = xdq @ wdq.T + b.astype(np.float64)[None, :]
+    assert np.max(np.abs(r["acc"] - want)) < 1e-4
+    # and it approximates the unquantized product
+    acc_exact, _ = O.woq_linear_ref(x, "bf16", qw, 5, 256, scales, zps, b, O.WOQ_DTYPE_INT4, 128, "fp32")
+    assert np.max(np.abs(r["acc"] - acc_exact)) < 0.1
+
+
+def test_int8_weight_block_sums_closed_form():
+    rng = np.random.default_rng(12)
+    N, K, G = 3, 256, 64
+    q = rng.integers(0, 16, (N, K)).astype(np.uint8)
+    zps = rng.integers(0, 16, (N, K // G)).astype(np.float32)
+    comp = O.int8_weight_block_sums(O.pack_int4(q), N, K, zps, O.WOQ_DTYPE_INT4, G, 64)
+    for n in range(N):
+        for kb in range(K // 64):
+            assert comp[n, kb] == sum(int(q[n, k]) - int(zps[n, k // G]) for k in range(kb * 64, kb * 64 + 64))
+
+
 def _awq_decode_independent(qweight, qzeros, scales, group_size):
     """AutoAWQ GEMM packing, restated from its definition: word [k, j] holds column
     8j + ORDER[i] in nibble i, ORDER = [0, 2, 4, 6, 1, 3, 5, 7]."""
