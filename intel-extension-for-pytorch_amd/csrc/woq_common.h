@@ -252,22 +252,29 @@ struct G4Masks {
   uint32_t lo, hi, magic;  // 0x000F000F, 0x00F000F0, fp16 1024 twice
 };
 
-__device__ __forceinline__ uint32_t g4_pair_bf16(uint32_t hbits, float s, float c) {
+__device__ __forceinline__ f2 g4_fma_pair(uint32_t hbits, float s, float c) {
   const h2 h = bitcast<h2>(hbits);
   f2 f;
   f[0] = __builtin_fmaf((float)h[0], s, c);
   f[1] = __builtin_fmaf((float)h[1], s, c);
-  return bitcast<uint32_t>(__builtin_convertvector(f, b2));
+  return f;
 }
+__device__ __forceinline__ uint32_t g4_cvt_pair(f2 f) { return bitcast<uint32_t>(__builtin_convertvector(f, b2)); }
 
-// One packed dword (8 weights of one row) -> MFMA B operand.
+// One packed dword (8 weights of one row) -> MFMA B operand.  Written so that no conversion
+// directly follows the fma that feeds it: v_cvt_pk_bf16_f32 one instruction behind its producer
+// costs a wait state.
 __device__ __forceinline__ u4 g4_dequant(uint32_t d, const G4Masks& k, const G4Consts<kRegimeBF16>& q) {
-  const uint32_t d8 = d >> 8;
   u4 r;
-  r[0] = g4_pair_bf16((d & k.lo) | k.magic, q.s, q.c);
-  r[1] = g4_pair_bf16((d & k.hi) | k.magic, q.s16, q.c16);
-  r[2] = g4_pair_bf16((d8 & k.lo) | k.magic, q.s, q.c);
-  r[3] = g4_pair_bf16((d8 & k.hi) | k.magic, q.s16, q.c16);
+  const f2 f0 = g4_fma_pair((d & k.lo) | k.magic, q.s, q.c);
+  const f2 f1 = g4_fma_pair((d & k.hi) | k.magic, q.s16, q.c16);
+  r[0] = g4_cvt_pair(f0);
+  const uint32_t d8 = d >> 8;
+  const f2 f2_ = g4_fma_pair((d8 & k.lo) | k.magic, q.s, q.c);
+  r[1] = g4_cvt_pair(f1);
+  const f2 f3 = g4_fma_pair((d8 & k.hi) | k.magic, q.s16, q.c16);
+  r[2] = g4_cvt_pair(f2_);
+  r[3] = g4_cvt_pair(f3);
   return r;
 }
 __device__ __forceinline__ u4 g4_dequant(uint32_t d, const G4Masks& k, const G4Consts<kRegimeF16>& q) {
