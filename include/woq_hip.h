@@ -31,6 +31,11 @@
  *                               fused post-ops of woq_linear_unary_kernel /
  *                               woq_linear_binary_kernel (csrc/cpu/aten/Linear.cpp:619-801)
  *   woq_hip_dequant_weight   <- dequantize_woq_weight (csrc/cpu/aten/utils/woq_utils.h:79-163)
+ *   woq_hip_shuffle_activations, woq_hip_shuffle_int4_weight
+ *                            <- woq_shuffle_tensor_by_group_idx /
+ *                               woq_shuffle_weight_back_by_group_idx, the channel shuffles of
+ *                               GPTQ act-order (csrc/cpu/jit/cpu/kernels/LinearWoqPacked.cpp:407-421,
+ *                               777-954)
  */
 #ifndef WOQ_HIP_H_
 #define WOQ_HIP_H_
@@ -216,6 +221,16 @@ int woq_hip_linear(const woq_hip_linear_params* p);
 int woq_hip_dequant_weight(const void* qweight, int weight_dtype, int64_t N, int64_t K,
                            const float* scales_f32, const uint8_t* zeros_u8,
                            int64_t group_size, void* out, int out_dtype, void* stream);
+
+/* GPTQ act-order.  src[p] (int32, K entries, a permutation of 0..K-1) is the input channel that
+ * belongs at position p once the channels are sorted by group (stable in the channel index).
+ *   shuffle_activations: out[m, p] = x[m, src[p]], x and out [M, K] in x_dtype.
+ *   shuffle_int4_weight: the same on plain int4 rows [N, (K + 1) / 2] (low nibble = even index);
+ *   with the inverse permutation it restores the checkpoint order. */
+int woq_hip_shuffle_activations(const void* x, int x_dtype, int64_t M, int64_t K, const int32_t* src,
+                                void* out, void* stream);
+int woq_hip_shuffle_int4_weight(const void* plain, int64_t N, int64_t K, const int32_t* src, void* out,
+                                void* stream);
 
 #ifdef __cplusplus
 }

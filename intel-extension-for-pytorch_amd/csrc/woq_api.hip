@@ -232,4 +232,21 @@ int woq_hip_dequant_weight(const void* qweight, int weight_dtype, int64_t N, int
                                (hipStream_t)stream);
 }
 
+int woq_hip_shuffle_activations(const void* x, int x_dtype, int64_t M, int64_t K, const int32_t* src, void* out,
+                                void* stream) {
+  if (x_dtype < 0 || x_dtype > 2) return set_error("shuffle_activations: bad x_dtype %d", x_dtype);
+  if (M < 0 || K < 0) return set_error("shuffle_activations: bad shape M=%lld K=%lld", (long long)M, (long long)K);
+  if (M > 0 && K > 0 && (!x || !src || !out)) return set_error("shuffle_activations: null pointer");
+  if (x == out && M > 0) return set_error("shuffle_activations: in-place shuffling is not supported");
+  return launch_shuffle_activations(x, x_dtype, M, K, src, out, (hipStream_t)stream);
+}
+
+int woq_hip_shuffle_int4_weight(const void* plain, int64_t N, int64_t K, const int32_t* src, void* out,
+                                void* stream) {
+  if (N < 0 || K < 0) return set_error("shuffle_int4_weight: bad shape N=%lld K=%lld", (long long)N, (long long)K);
+  if (N > 0 && K > 0 && (!plain || !src || !out)) return set_error("shuffle_int4_weight: null pointer");
+  if (plain == out && N > 0) return set_error("shuffle_int4_weight: in-place shuffling is not supported");
+  return launch_shuffle_int4_weight(plain, N, K, src, out, (hipStream_t)stream);
+}
+
 }  // extern "C"

@@ -243,4 +243,60 @@ int launch_dequant_weight(const void* qweight, int weight_dtype, int64_t N, int6
   return check_launch("dequant_weight");
 }
 
+// ---- GPTQ act-order (g_idx): channel shuffles -------------------------------------------------
+// Reference: woq_shuffle_tensor_by_group_idx / woq_shuffle_weight_back_by_group_idx
+// (csrc/cpu/jit/cpu/kernels/LinearWoqPacked.cpp:777-954).  Channel j moves to position
+// g_idx[j] * group_size + (number of earlier channels of the same group); `src` is that map
+// read backwards (src[p] = the channel that lands at position p), which serves both directions.
+template <typename T>
+__global__ void shuffle_activations_kernel(const T* __restrict__ x, int64_t M, int64_t K,
+                                           const int32_t* __restrict__ src, T* __restrict__ out) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= M * K) return;
+  const int64_t m = i / K, p = i - m * K;
+  out[i] = x[m * K + src[p]];
+}
+
+// plain int4 rows (two values per byte, low nibble first): one thread per output byte
+__global__ void shuffle_int4_weight_kernel(const uint8_t* __restrict__ plain, int64_t N, int64_t K,
+                                           const int32_t* __restrict__ src, uint8_t* __restrict__ out) {
+  const int64_t stride = (K + 1) / 2;
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= N * stride) return;
+  const int64_t n = i / stride, b = i - n * stride;
+  uint8_t v = 0;
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    const int64_t pos = 2 * b + h;
+    if (pos < K) {
+      const int64_t j = src[pos];
+      const uint8_t byte = plain[n * stride + j / 2];
+      v |= (uint8_t)(((j & 1) ? byte >> 4 : byte & 15) << (4 * h));
+    }
+  }
+  out[i] = v;
+}
+
+int launch_shuffle_activations(const void* x, int x_dtype, int64_t M, int64_t K, const int32_t* src, void* out,
+                               hipStream_t st) {
+  const int64_t total = M * K;
+  if (total == 0) return 0;
+  if (x_dtype == WOQ_HIP_ACT_FP32)
+    shuffle_activations_kernel<uint32_t><<<blocks_for(total, 256), 256, 0, st>>>((const uint32_t*)x, M, K, src,
+                                                                                   (uint32_t*)out);
+  else
+    shuffle_activations_kernel<uint16_t><<<blocks_for(total, 256), 256, 0, st>>>((const uint16_t*)x, M, K, src,
+                                                                                   (uint16_t*)out);
+  return check_launch("shuffle_activations");
+}
+
+int launch_shuffle_int4_weight(const void* plain, int64_t N, int64_t K, const int32_t* src, void* out,
+                               hipStream_t st) {
+  const int64_t total = N * ((K + 1) / 2);
+  if (total == 0) return 0;
+  shuffle_int4_weight_kernel<<<blocks_for(total, 256), 256, 0, st>>>((const uint8_t*)plain, N, K, src,
+                                                                     (uint8_t*)out);
+  return check_launch("shuffle_int4_weight");
+}
+
 }  // namespace woq

@@ -240,3 +240,31 @@ def dequant_weight(qweight, weight_dtype, N, K, scales_f32, zeros_u8, group_size
             "dequant_weight",
         )
     return out
+
+
+def shuffle_activations(x, src):
+    """out[..., p] = x[..., src[p]] (GPTQ act-order: channels sorted by group)."""
+    lib = _lib.load()
+    _require_cuda(x, "input")
+    if x.dtype not in _ACT_CODE:
+        raise RuntimeError(f"shuffle_activations: unsupported dtype {x.dtype}")
+    K = x.shape[-1]
+    x2 = x.reshape(-1, K).contiguous()
+    out = torch.empty_like(x2)
+    with torch.cuda.device(x.device):
+        _lib.check(
+            lib.woq_hip_shuffle_activations(_ptr(x2), _ACT_CODE[x.dtype], x2.shape[0], K, _ptr(src), _ptr(out), _stream()),
+            "shuffle_activations",
+        )
+    return out.reshape(x.shape)
+
+
+def shuffle_int4_weight(plain, N, K, src):
+    """Plain int4 rows [N, (K + 1) // 2] with nibble p taken from nibble src[p]."""
+    lib = _lib.load()
+    _require_cuda(plain, "weight")
+    plain = plain.contiguous()
+    out = torch.empty_like(plain)
+    with torch.cuda.device(plain.device):
+        _lib.check(lib.woq_hip_shuffle_int4_weight(_ptr(plain), N, K, _ptr(src), _ptr(out), _stream()), "shuffle_int4_weight")
+    return out

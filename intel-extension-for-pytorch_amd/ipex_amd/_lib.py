@@ -33,6 +33,8 @@ EXPORTS = [
     "woq_hip_int8_block_k",
     "woq_hip_linear",
     "woq_hip_dequant_weight",
+    "woq_hip_shuffle_activations",
+    "woq_hip_shuffle_int4_weight",
 ]
 
 
@@ -116,6 +118,10 @@ def load():
         lib.woq_hip_linear.argtypes = [ctypes.POINTER(LinearParams)]
         lib.woq_hip_dequant_weight.restype = i32
         lib.woq_hip_dequant_weight.argtypes = [vp, i32, i64, i64, vp, vp, i64, vp, i32, vp]
+        lib.woq_hip_shuffle_activations.restype = i32
+        lib.woq_hip_shuffle_activations.argtypes = [vp, i32, i64, i64, vp, vp, vp]
+        lib.woq_hip_shuffle_int4_weight.restype = i32
+        lib.woq_hip_shuffle_int4_weight.argtypes = [vp, i64, i64, vp, vp, vp]
         if lib.woq_hip_abi_version() != 1:
             raise RuntimeError("libwoq_hip.so has an unexpected ABI version")
         _lib = lib

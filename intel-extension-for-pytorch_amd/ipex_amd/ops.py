@@ -87,8 +87,6 @@ class WoqLinearOpContext:
         weight_dtype = int(weight_dtype)
         if weight_dtype not in (_lib.DTYPE_INT8, _lib.DTYPE_INT4):
             raise RuntimeError(f"WOQ linear: unsupported weight dtype {weight_dtype} (INT8 and INT4 are built)")
-        if g_idx is not None:
-            raise RuntimeError("WOQ linear: g_idx (GPTQ act-order) is not supported by this build")
         N, K = int(weight_shape[0]), int(weight_shape[1])
         weight = _to_gpu(weight)
         dev = weight.device
@@ -125,7 +123,28 @@ class WoqLinearOpContext:
         self.act_quant_mode_ = int(act_quant_mode)
         self.batch_size_ = batch_size
         self.cache_weight_for_large_batch_ = bool(cache_weight_for_large_batch)
+        # GPTQ act-order: input channel k belongs to group g_idx[k].  As the reference does for
+        # 4-bit group-wise weights (LinearWoqPacked.cpp:306-316, 407-421), the weight's input channels
+        # are sorted by group once here and the activations are shuffled the same way per call.
         self.g_idx_ = None
+        self.g_src_ = None  # position -> source channel
+        self.g_dst_ = None  # inverse permutation
+        if g_idx is not None and weight_dtype == _lib.DTYPE_INT4 and group_size > 0:
+            g = _to_gpu(g_idx, dev).to(torch.int64).reshape(-1)
+            KG = (K + group_size - 1) // group_size
+            if g.numel() != K:
+                raise RuntimeError("g_idx size and weight shape mismatch")
+            if int(g.min()) < 0 or int(g.max()) >= KG:
+                raise RuntimeError(f"WOQ linear: g_idx values must lie in [0, {KG})")
+            want = torch.full((KG,), group_size, dtype=torch.int64, device=dev)
+            want[-1] = K - (KG - 1) * group_size
+            if not torch.equal(torch.bincount(g, minlength=KG), want):
+                raise RuntimeError("WOQ linear: g_idx must assign exactly group_size channels to every group")
+            src = torch.argsort(g, stable=True)
+            self.g_idx_ = g_idx
+            self.g_src_ = src.to(torch.int32).contiguous()
+            self.g_dst_ = torch.argsort(src).to(torch.int32).contiguous()
+            weight = _kernels.shuffle_int4_weight(weight, N, K, self.g_src_)
         self.at_bias_ = _to_gpu(bias, dev)
         self.bias_f32_ = self.at_bias_.to(torch.float32).contiguous() if self.at_bias_ is not None else None
         self.at_weight_ = _kernels.pack_weight(weight, weight_dtype, N, K)
@@ -182,7 +201,10 @@ class WoqLinearOpContext:
     def to_public(self, tensor):
         """Packed tensor -> plain [N, K/2] (or [N, K]) checkpoint layout."""
         N, K = self.weight_shape_
-        return _kernels.unpack_weight(tensor, self.weight_dtype_, N, K)
+        plain = _kernels.unpack_weight(tensor, self.weight_dtype_, N, K)
+        if self.g_dst_ is not None:  # back to the checkpoint's channel order (LinearWoqPacked.cpp:755-765)
+            plain = _kernels.shuffle_int4_weight(plain, N, K, self.g_dst_)
+        return plain
 
     def get_data_handle(self):
         return torch.tensor([self._handle], dtype=torch.int64)
@@ -200,7 +222,7 @@ class WoqLinearOpContext:
             cpu(self.scales_plain_),
             cpu(self.zero_points_plain_),
             cpu(self.at_bias_),
-            None,
+            cpu(self.g_idx_),
             self.batch_size_,
             self.group_size_,
             self.lowp_mode_,
@@ -231,6 +253,8 @@ class WoqLinearOpContext:
         M = x.numel() // K if x.numel() > 0 else 0
         if M == 0:
             return x.new_empty(*x.shape[:-1], N)
+        if self.g_src_ is not None:
+            x = _kernels.shuffle_activations(x, self.g_src_)
         if (
             self.cache_weight_for_large_batch_
             and self.lowp_mode_ == _lib.LOWP_BF16
@@ -446,8 +470,10 @@ def woq_linear(
     _require_gpu_input(input, "torch_ipex::woq_linear")
     if weight_dtype not in WOQ_DTYPE_MAP:
         raise RuntimeError(f"Unsupported weight dtype: {weight_dtype}")
-    if g_idx is not None:
-        raise RuntimeError("torch_ipex::woq_linear: g_idx is not supported by this build")
+    if g_idx is not None and WOQ_DTYPE_MAP[weight_dtype] == _lib.DTYPE_INT4 and group_size > 0:
+        # the packed weight from woq_linear_pack_weight is already sorted by group
+        src = torch.argsort(g_idx.to(input.device).to(torch.int64).reshape(-1), stable=True).to(torch.int32)
+        input = _kernels.shuffle_activations(input, src.contiguous())
     if weight_zeros is not None and len(weight_zeros) != 4:
         raise RuntimeError("IPEX WOQ: expect list of zeros has length 4")
     if bias is not None and len(bias) != 3:

@@ -5,6 +5,8 @@ fp32 accumulators max-abs <= 1e-2; bf16 outputs relative-L2 <= 2e-3 (two correct
 implementations with different summation orders can differ by one bf16 ulp, which at
 |y| in [8, 16) is 0.0625, so the max-abs bar is applied to the accumulators).
 """
+import pickle
+
 import numpy as np
 import pytest
 import torch
@@ -525,3 +527,74 @@ def test_determinism(cuda):
     ctx = make_context(case, O.LOWP_BF16)
     x = case["x"].cuda()
     assert torch.equal(ctx.run(x), ctx.run(x))
+
+
+# ---------------------------------------------------------------------------------------------
+# GPTQ act-order (g_idx)
+# ---------------------------------------------------------------------------------------------
+def _g_idx_cases(K, G):
+    n_groups = K // G
+    yield "interleaved", torch.arange(n_groups).repeat(G)  # as the reference's tests build it
+    perm = torch.randperm(K, generator=torch.Generator().manual_seed(K + G))
+    yield "random", (torch.arange(K) // G)[perm]
+
+
+class _Unshuffled:
+    """Feeds a context built with g_idx the activations in checkpoint order when the caller holds
+    them sorted by group."""
+
+    def __init__(self, ctx, dst):
+        self.ctx, self.dst = ctx, dst
+
+    def run(self, x_sorted, **kw):
+        return self.ctx.run(x_sorted[:, self.dst.to(x_sorted.device)].contiguous(), **kw)
+
+
+@pytest.mark.parametrize("M", [3, 9, 80])
+def test_g_idx_matches_the_group_sorted_problem(cuda, M):
+    """w[n, k] = (q[n, k] - z[n, g_idx[k]]) * s[n, g_idx[k]]: sorting the channels by group with
+    numpy gives an ordinary group-wise problem, which the oracle evaluates; the context built with
+    g_idx must give the same result on the unsorted activations."""
+    from ipex_amd import ops
+
+    K, N, G = 512, 96, 128
+    for name, g_idx in _g_idx_cases(K, G):
+        case = _synthetic().make_int4_case(31, M, K, N, G, bias=True)
+        src = np.argsort(g_idx.numpy(), kind="stable")
+        dst = torch.from_numpy(np.argsort(src))
+        q = O.unpack_int4(case["qweight"].numpy())[:, :K]
+        sorted_case = dict(case)
+        sorted_case["x"] = case["x"][:, torch.from_numpy(src)].contiguous()
+        sorted_case["qweight"] = torch.from_numpy(O.pack_int4(np.ascontiguousarray(q[:, src])))
+        ctx = ops.WoqLinearOpContext(
+            case["qweight"].cuda(), 2, [N, K], case["scales"].cuda(), case["zeros"].cuda(), case["bias"].cuda(),
+            g_idx, None, G, O.LOWP_BF16, -1,
+        )
+        _check_fp(sorted_case, O.LOWP_BF16, ctx=_Unshuffled(ctx, dst), label=f"g_idx {name} M={M}")
+        # the checkpoint layout comes back bit-exactly, and the context pickles with its g_idx
+        assert torch.equal(ctx.to_public(ctx.get_weight()).cpu(), case["qweight"])
+        assert torch.equal(ctx.get_g_idx().cpu(), g_idx)
+        ctx2 = pickle.loads(pickle.dumps(ctx))
+        x = case["x"].cuda()
+        assert torch.equal(ctx2.run(x), ctx.run(x))
+        # lowp INT8 goes through the same shuffles: identical to the context of the sorted problem
+        ctx_i8 = ops.WoqLinearOpContext(
+            case["qweight"].cuda(), 2, [N, K], case["scales"].cuda(), case["zeros"].cuda(), case["bias"].cuda(),
+            g_idx, None, G, O.LOWP_INT8, 6,
+        )
+        ref_i8 = make_context(sorted_case, O.LOWP_INT8, 6)
+        assert torch.equal(ctx_i8.run(x), ref_i8.run(sorted_case["x"].cuda()))
+
+
+def test_g_idx_validation(cuda):
+    from ipex_amd import ops
+
+    case = _synthetic().make_int4_case(32, 2, 256, 32, 128)
+    args = lambda g: (case["qweight"].cuda(), 2, [32, 256], case["scales"].cuda(), case["zeros"].cuda(), None, g, None,
+                      128, O.LOWP_BF16, -1)
+    with pytest.raises(RuntimeError, match="mismatch"):
+        ops.WoqLinearOpContext(*args(torch.zeros(100, dtype=torch.int64)))
+    with pytest.raises(RuntimeError, match="exactly group_size"):
+        ops.WoqLinearOpContext(*args(torch.zeros(256, dtype=torch.int64)))
+    with pytest.raises(RuntimeError, match="must lie in"):
+        ops.WoqLinearOpContext(*args(torch.full((256,), 5, dtype=torch.int64)))
