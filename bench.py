@@ -114,6 +114,73 @@ def time_graph(torch, lib, params, steps, warmup):
     return reps * n, t1 - t0, start.elapsed_time(stop)
 
 
+def _rotating_params(torch, lib_mod, ops_mod, case, lowp_mode, dev, stream, min_bytes=640e6):
+    """One op context per weight copy (enough copies that the working set exceeds the Infinity
+    Cache), the launch parameters of each, and the objects that keep the memory alive."""
+    M, K, N, G = case["M"], case["K"], case["N"], case["group_size"]
+    ctx0 = ops_mod.WoqLinearOpContext(
+        case["qweight"].to(dev), case["weight_dtype"], [N, K], case["scales"].to(dev),
+        None if case["zeros"] is None else case["zeros"].to(dev),
+        None if case["bias"] is None else case["bias"].to(dev), None, None, G, lowp_mode, -1,
+    )
+    copies = int(min_bytes // ctx0.at_weight_.numel()) + 1
+    x = case["x"].to(dev)
+    out = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
+
+    class Copy:
+        pass
+
+    params, keep = [], [x, out]
+    for i in range(copies):
+        c = Copy()
+        c.__dict__.update(ctx0.__dict__)
+        if i > 0:
+            c.at_weight_ = ctx0.at_weight_.clone()
+            c.scales_list_ = [t.clone() for t in ctx0.scales_list_]
+            c.zeros_u8_ = None if ctx0.zeros_u8_ is None else ctx0.zeros_u8_.clone()
+            c.scale_zero_f16x2_ = None if ctx0.scale_zero_f16x2_ is None else ctx0.scale_zero_f16x2_.clone()
+        keep.append(c)
+        p = build_params(lib_mod, x, c, out, lowp_mode)
+        p.stream = stream.cuda_stream
+        params.append(p)
+    return params, keep
+
+
+def config_sweep(torch, lib, lib_mod, ops_mod, synthetic, dev, stream, steps):
+    """The other named configurations, each timed like the headline (rotating weight copies, HIP
+    events over back-to-back launches) and reported against its own algorithmic bytes: weights at
+    their stored width, bf16 scales (fp32 for the INT8 case), uint4 zeros, bf16 activations, bias
+    and outputs."""
+    rows = []
+
+    def run(name, case):
+        M, K, N, G = case["M"], case["K"], case["N"], case["group_size"]
+        params, keep = _rotating_params(torch, lib_mod, ops_mod, case, 2, dev, stream)
+        _, ms = time_steps(torch, lib, params, steps, max(10, steps // 10), stream)
+        us = ms * 1e3 / steps
+        if case["weight_dtype"] == 2:
+            nbytes = algorithmic_bytes(M, K, N, G)
+        else:
+            nbytes = N * K + N * 4 + M * K * 2 + M * N * 2 + (N * 2 if case["bias"] is not None else 0)
+        rows.append({"config": name, "M": M, "K": K, "N": N, "group_size": G, "us_per_launch": round(us, 2),
+                     "GB_per_s": round(nbytes / us / 1e3, 1), "frac_of_hbm_peak": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 3)})
+        del params, keep
+        torch.cuda.empty_cache()
+
+    run("C0 int4 g128 M=1 4096->4096", synthetic.make_int4_case(0, 1, 4096, 4096, 128))
+    run("C1 int8 per-channel M=32 4096->11008 +bias", synthetic.make_int8_case(1, 32, 4096, 11008))
+    for M in (4, 8, 16):
+        run(f"C2 int4 g128 M={M} 4096->14336", synthetic.make_int4_case(2, M, 4096, 14336, 128))
+    for M in (1, 4, 8, 16):
+        run(f"C2 int4 g128 M={M} 14336->4096", synthetic.make_int4_case(2, M, 14336, 4096, 128))
+    block = 0.0
+    for K, N, what in ((4096, 6144, "qkv"), (4096, 4096, "o"), (4096, 28672, "gate+up"), (14336, 4096, "down")):
+        run(f"C4 int4 g32 M=16 {what} {K}->{N}", synthetic.make_int4_case(4, 16, K, N, 32))
+        block += rows[-1]["us_per_launch"]
+    rows.append({"config": "C4 decoder block, summed WOQ-linear time per token step", "us": round(block, 2)})
+    return rows
+
+
 def cpu_baseline_decode(case, K, N, G, budget_s=12.0):
     """The oracle's C port (bf16-regime arithmetic, OpenMP over output channels) on the same
     decode workload, timed on the host cores this process may use."""
@@ -163,6 +230,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=400)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-prefill", action="store_true", help="skip the M=2048 measurement")
+    ap.add_argument("--no-sweep", action="store_true", help="skip the other named configurations")
     ap.add_argument("--M", type=int, default=1, help="decode batch (1..16)")
     ap.add_argument("--traffic-probe", action="store_true",
                     help="short run for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE: a few decode launches plus a "
@@ -295,6 +363,12 @@ def main():
             "frac_of_bf16_mfma_peak": round(pre["bf16"]["tflops"] / MFMA_BF16_PEAK_TFLOPS, 4),
             "peak_tflops": MFMA_BF16_PEAK_TFLOPS,
         }
+
+    if not args.no_sweep and M == 1:
+        del params, keep
+        torch.cuda.empty_cache()
+        result["other_configs"] = config_sweep(torch, lib, _lib, ops, synthetic, dev, stream,
+                                               max(50, min(400, args.steps // 10)))
 
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline_decode(synthetic.make_int4_case(2, 1, K, N, G), K, N, G)
