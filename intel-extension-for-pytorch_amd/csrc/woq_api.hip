@@ -208,9 +208,9 @@ int woq_hip_linear(const woq_hip_linear_params* p) {
   if (kernel == 0 && decode_dq_applies(f, wbits, regime)) kernel = 7;
   if (kernel >= 7 && kernel <= 10) {
     if (!decode_dq_applies(f, wbits, regime))
-      return set_error("woq_linear: the dequantizing decode kernel takes 4-bit weights, M <= 16, K %% 128 == 0, a "
+      return set_error("woq_linear: the dequantizing decode kernel takes M <= 32, K a multiple of the weight tile, a "
                        "power-of-two or per-channel group size and activations in the compute dtype");
-    return launch_decode_dq(f, regime, st, kernel == 10 ? 4 : kernel - 7);
+    return launch_decode_dq(f, wbits, regime, st, kernel == 10 ? 4 : kernel - 7);
   }
   if (kernel == 0) kernel = p->M <= 64 ? 1 : (gemm_w4_applies(f, wbits, regime) ? 3 : 2);
   if (kernel == 1 && p->M > 64) return set_error("woq_linear: the small-M kernel takes M <= 64");

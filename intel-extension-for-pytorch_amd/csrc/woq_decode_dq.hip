@@ -1,4 +1,5 @@
-// Decode kernel with per-weight dequantization: 4-bit weights, M <= 16, HBM-bound weight streaming.
+// Decode kernel with per-weight dequantization: 4- or 8-bit weights, M <= 32, HBM-bound weight
+// streaming.
 //
 // Reference counterpart: the M >= 5 path of lowp_mode BF16 -- Dequantize<bfloat16> into a bf16
 // block, then a bf16 x bf16 -> fp32 BRGEMM (csrc/cpu/aten/utils/woq.h:1495-1581, 1847-1944) -- at
@@ -14,20 +15,18 @@
 // the weight stream itself, so the rounds are software pipelined: the requests of round r + 1
 // (tiles and parameters into registers, activations into the other LDS buffer) are issued before
 // round r is computed.
-// Activations: a wave copies the 16 rows x 256 bytes of its K tile straight into its private 4 KiB
-// of LDS (global_load_lds_dwordx4: four fully coalesced instructions, no registers) and reads the
-// operand fragments from there; chunk p of row m sits at p ^ m so the fragment reads are
-// conflict-free.  Reading the fragments from global memory directly costs the same number of
+// Activations: a wave copies the rows of its K tile (16 or 32 rows x 256 bytes for 4-bit weights,
+// x 128 bytes for 8-bit ones) straight into its private slice of LDS (global_load_lds_dwordx4: four fully coalesced instructions, no registers) and reads the
+// operand fragments from there; chunk p of row m sits at p ^ m (p ^ (m / 2) for the 128-byte rows)
+// so the fragment reads are conflict-free.  Reading the fragments from global memory directly costs the same number of
 // instructions but each one gathers 64 separate 16-byte pieces, which made the texture addresser
 // the bottleneck (M = 16: 19.7 us against 13.9 us at M = 8 for the same weights).  Rows past M
-// re-read row M - 1 and their results are dropped.  The 64 KiB of slices are reused for the
-// cross-wave sum, so two workgroups fit on a CU.
+// re-read row M - 1 and their results are dropped.  The at most 64 KiB of slices are reused for
+// the cross-wave sum, so two workgroups fit on a CU.
 #include "woq_common.h"
 #include "woq_internal.h"
 
 namespace woq {
-
-constexpr int kDqSlice = kTileN * kTileK4 * 2;  // one wave's activation slice: 16 rows x 128 K, 4 KiB
 
 struct DecodeDqArgs {
   FpArgs f;
@@ -46,8 +45,30 @@ __device__ __forceinline__ f4 dq_mfma(u4 a, u4 b, f4 c) {
 typedef __attribute__((address_space(3))) void* dq_lds_ptr_t;
 typedef const __attribute__((address_space(1))) void* dq_global_ptr_t;
 
-template <int REGIME, int NTW>
+// Geometry of one K tile (1 KiB of packed weights: 16 rows x 128 int4 or x 64 int8) and of the
+// activation slice that goes with it.
+template <int WBITS, int MT>
+struct DqGeom {
+  static constexpr int TK = WBITS == 4 ? kTileK4 : kTileK8;
+  static constexpr int ROWB = TK * 2;             // bytes of one activation row of the tile
+  static constexpr int LPR = ROWB / 16;           // lanes (16-byte chunks) per row
+  static constexpr int RPI = 64 / LPR;            // rows per LDS-load instruction
+  static constexpr int SLICE = MT * 16 * ROWB;    // one buffer of one wave
+  static constexpr int NX = SLICE / 1024;         // LDS-load instructions per buffer
+  static constexpr int NJ = TK / 32;              // MFMAs (32 K values each) per tile
+  static __device__ __forceinline__ int swz(int row) { return WBITS == 4 ? (row & 15) : ((row >> 1) & 7); }
+};
+
+// 8-bit weights: per-lane scale and offset of one row, c = -(128 + z) * s for the offset-binary
+// bytes (symmetric: z = 0).
+struct G8Consts {
+  float s, c;
+};
+
+template <int REGIME, int WBITS, int MT, int NTW>
 __global__ __launch_bounds__(512, 4) void woq_decode_dq_kernel(const DecodeDqArgs a) {
+  using Geo = DqGeom<WBITS, MT>;
+  constexpr int TK = Geo::TK, NJ = Geo::NJ, NX = Geo::NX, SLICE = Geo::SLICE;
   extern __shared__ __align__(1024) uint8_t smem[];
   const FpArgs& f = a.f;
   const int W = a.W;
@@ -56,31 +77,34 @@ __global__ __launch_bounds__(512, 4) void woq_decode_dq_kernel(const DecodeDqArg
   const int r = lane & 15, c = lane >> 4;
   const int M = (int)f.M, K = (int)f.K, KT = (int)f.KT, KG = (int)f.KG;
   const int64_t nt0 = (int64_t)blockIdx.x * NTW;
-  uint8_t* const sx = smem + wave * (2 * kDqSlice);  // this wave's two activation buffers
-  f4* const red = (f4*)smem;                         // [NTW][W][64], after the K loop
+  uint8_t* const sx = smem + wave * (2 * SLICE);  // this wave's two activation buffers
+  f4* const red = (f4*)smem;                      // [NTW * MT][W][64], after the K loop
 
   G4Masks km;
   asm volatile("s_mov_b32 %0, 0x000F000F" : "=s"(km.lo));
   asm volatile("s_mov_b32 %0, 0x00F000F0" : "=s"(km.hi));
   asm volatile("v_mov_b32 %0, 0x64006400" : "=v"(km.magic));
 
-  f4 acc[NTW];
+  f4 acc[NTW][MT];
 #pragma unroll
-  for (int t = 0; t < NTW; ++t) acc[t] = f4{0.f, 0.f, 0.f, 0.f};
+  for (int t = 0; t < NTW; ++t)
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) acc[t][mt] = f4{0.f, 0.f, 0.f, 0.f};
 
   // wave-uniform bases + one 32-bit per-lane offset per stream.
-  // Activation load i fills LDS bytes [1024 i, +1024) of a buffer: rows 4 i + lane / 16,
-  // physical chunk lane % 16 = logical chunk ^ row.
-  uint32_t xoff[4];
+  // Activation load i fills LDS bytes [1024 i, +1024) of a buffer: rows RPI * i + lane / LPR,
+  // physical chunk lane % LPR = logical chunk ^ swz(row).
+  uint32_t xoff[NX];
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int row = 4 * i + c;
+  for (int i = 0; i < NX; ++i) {
+    const int row = Geo::RPI * i + lane / Geo::LPR;
     const int rowc = row < M ? row : M - 1;
-    xoff[i] = (uint32_t)(rowc * K + ((r ^ row) & 15) * 8) * 2u;
+    const int chunk = ((lane % Geo::LPR) ^ Geo::swz(row)) & (Geo::LPR - 1);
+    xoff[i] = (uint32_t)(rowc * K + chunk * 8) * 2u;
   }
-  uint32_t rdo[4];  // fragment j of this lane: row r, logical chunk 4 c + j
+  uint32_t rdo[NJ];  // fragment j of this lane in row tile 0: row r, logical chunk NJ c + j
 #pragma unroll
-  for (int j = 0; j < 4; ++j) rdo[j] = (uint32_t)(r * 256 + (((c * 4 + j) ^ r) << 4));
+  for (int j = 0; j < NJ; ++j) rdo[j] = (uint32_t)(r * Geo::ROWB + (((c * NJ + j) ^ Geo::swz(r)) << 4));
   const uint32_t woff = (uint32_t)lane * 16u;
   const bool has_z = f.zeros != nullptr;
   const uint8_t* wbase[NTW];
@@ -98,15 +122,15 @@ __global__ __launch_bounds__(512, 4) void woq_decode_dq_kernel(const DecodeDqArg
   uint8_t znext[NTW];
   // every request of one round: activations into LDS buffer `buf`, tiles and parameters into registers
   auto request = [&](int kt, int buf) {
-    // uniform base + 32-bit offset; groups of four rows that lie entirely past M are not loaded
+    // uniform base + 32-bit offset; instructions whose rows lie entirely past M are skipped
     // (their LDS bytes stay undefined: an MFMA output row depends on its own A row only)
-    const uint32_t ko = (uint32_t)kt * (kTileK4 * 2);
+    const uint32_t ko = (uint32_t)kt * Geo::ROWB;
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
-      if (4 * i < M)
+    for (int i = 0; i < NX; ++i)
+      if (Geo::RPI * i < M)
         __builtin_amdgcn_global_load_lds((dq_global_ptr_t)((const uint8_t*)f.x + (uint32_t)(xoff[i] + ko)),
-                                         (dq_lds_ptr_t)(sx + buf * kDqSlice + i * 1024), 16, 0, 0);
-    int g = (kt * kTileK4 + c * 32) >> a.g_shift;
+                                         (dq_lds_ptr_t)(sx + buf * SLICE + i * 1024), 16, 0, 0);
+    int g = (kt * TK + c * (TK / 4)) >> a.g_shift;
     g = g < KG ? g : KG - 1;
     const uint32_t qoff = (uint32_t)(g * kTileN + r);
     const uint32_t wo = (uint32_t)kt * kTileBytes + woff;
@@ -123,11 +147,17 @@ __global__ __launch_bounds__(512, 4) void woq_decode_dq_kernel(const DecodeDqArg
 #pragma unroll 1
   for (int kt = wave, buf = 0; kt < KT; kt += W, buf ^= 1) {
     u4 wreg[NTW];
-    G4Consts<REGIME> qc[NTW];
+    G4Consts<REGIME> qc4[WBITS == 4 ? NTW : 1];
+    G8Consts qc8[WBITS == 8 ? NTW : 1];
 #pragma unroll
     for (int t = 0; t < NTW; ++t) {
       wreg[t] = wnext[t];
-      qc[t].set(snext[t], has_z ? (float)znext[t] : 8.0f);
+      if constexpr (WBITS == 4) {
+        qc4[t].set(snext[t], has_z ? (float)znext[t] : 8.0f);
+      } else {
+        qc8[t].s = REGIME == kRegimeF16 ? f16_bits_to_f32(snext[t]) : bf16_bits_to_f32(snext[t]);
+        qc8[t].c = -((has_z ? (float)znext[t] : 128.0f) * qc8[t].s);
+      }
     }
     // The compiler does not order LDS reads after the LDS-writing loads: wait for them here.
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
@@ -135,12 +165,22 @@ __global__ __launch_bounds__(512, 4) void woq_decode_dq_kernel(const DecodeDqArg
     __builtin_amdgcn_sched_barrier(0);
 
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const u4 xa = *(const u4*)(sx + buf * kDqSlice + rdo[j]);
+    for (int j = 0; j < NJ; ++j) {
+      u4 xa[MT];
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) xa[mt] = *(const u4*)(sx + buf * SLICE + mt * 16 * Geo::ROWB + rdo[j]);
 #pragma unroll
       for (int t = 0; t < NTW; ++t) {
-        const u4 bop = g4_dequant(wreg[t][j], km, qc[t]);
-        acc[t] = dq_mfma<REGIME>(xa, bop, acc[t]);
+        u4 bop;
+        if constexpr (WBITS == 4) {
+          bop = g4_dequant(wreg[t][j], km, qc4[t]);
+        } else if constexpr (REGIME == kRegimeF16) {
+          bop = bitcast<u4>(dequant8_f16_w8(wreg[t][2 * j], wreg[t][2 * j + 1], qc8[t].s, qc8[t].c));
+        } else {
+          bop = bitcast<u4>(dequant8_bf16_w8(wreg[t][2 * j], wreg[t][2 * j + 1], qc8[t].s, qc8[t].c));
+        }
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) acc[t][mt] = dq_mfma<REGIME>(xa[mt], bop, acc[t][mt]);
       }
     }
   }
@@ -148,23 +188,27 @@ __global__ __launch_bounds__(512, 4) void woq_decode_dq_kernel(const DecodeDqArg
   // ---- combine the waves' partial sums in wave order, then bias / rounding / store ----
   __syncthreads();  // every wave is done with its activation slices: the region becomes `red`
 #pragma unroll
-  for (int t = 0; t < NTW; ++t) red[(t * W + wave) * 64 + lane] = acc[t];
+  for (int t = 0; t < NTW; ++t)
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) red[((t * MT + mt) * W + wave) * 64 + lane] = acc[t][mt];
   __syncthreads();
 
   Epilogue ep{f.bias, f.fusion, f.other0, f.other1, f.out, f.out_dtype, f.x_dtype, f.N};
   const float* redf = (const float*)red;
   const bool plain = REGIME == kRegimeBF16 && f.fusion == WOQ_HIP_FUSE_NONE && f.bias == nullptr &&
                      f.out_dtype == WOQ_HIP_ACT_BF16;
-  // one thread per output element, consecutive threads on consecutive columns; D[m][n] sits in
-  // lane n + 16 (m / 4), register m % 4
-  for (int idx = threadIdx.x; idx < NTW * 256; idx += blockDim.x) {
-    const int col = idx & 15, m = (idx >> 4) & 15, t = idx >> 8;
+  // one thread per output element, consecutive threads on consecutive columns; D[m][n] of a row
+  // tile sits in lane n + 16 (m / 4), register m % 4
+  for (int idx = threadIdx.x; idx < NTW * MT * 256; idx += blockDim.x) {
+    const int col = idx & 15, m16 = (idx >> 4) & 15, tm = idx >> 8;
+    const int t = tm / MT, mt = tm - t * MT;
+    const int m = mt * 16 + m16;
     const int64_t n = (nt0 + t) * kTileN + col;
     if (m >= M || n >= f.N) continue;
-    const int slot = (col + 16 * (m >> 2)) * 4 + (m & 3);
+    const int slot = (col + 16 * (m16 >> 2)) * 4 + (m16 & 3);
     float part[8];
 #pragma unroll
-    for (int w = 0; w < 8; ++w) part[w] = w < W ? redf[(t * W + w) * 256 + slot] : 0.0f;
+    for (int w = 0; w < 8; ++w) part[w] = w < W ? redf[(tm * W + w) * 256 + slot] : 0.0f;
     float s = part[0];
 #pragma unroll
     for (int w = 1; w < 8; ++w) s += part[w];
@@ -175,45 +219,61 @@ __global__ __launch_bounds__(512, 4) void woq_decode_dq_kernel(const DecodeDqArg
   }
 }
 
-template <int REGIME, int NTW>
-static int launch_dq_cfg(const DecodeDqArgs& a, hipStream_t st) {
-  const size_t smem = (size_t)a.W * 2 * kDqSlice;  // >= NTW * W * 1 KiB of partial sums
+template <int REGIME, int WBITS, int MT, int NTW>
+static int launch_dq_cfg(DecodeDqArgs a, hipStream_t st) {
+  using Geo = DqGeom<WBITS, MT>;
+  // at most 64 KiB of activation buffers per workgroup, so that two workgroups share a CU
+  const int max_w = 65536 / (2 * Geo::SLICE);
+  a.W = (int)(a.f.KT < max_w ? a.f.KT : max_w);
+  if (a.W > 8) a.W = 8;
+  size_t smem = (size_t)a.W * 2 * Geo::SLICE;
+  const size_t red = (size_t)NTW * MT * a.W * 64 * sizeof(f4);
+  if (red > smem) smem = red;
   const unsigned grid = (unsigned)(a.f.NT / NTW);
-  woq_decode_dq_kernel<REGIME, NTW><<<grid, a.W * 64, smem, st>>>(a);
+  woq_decode_dq_kernel<REGIME, WBITS, MT, NTW><<<grid, a.W * 64, smem, st>>>(a);
   return check_launch("woq_decode_dq_kernel");
 }
 
-// 4-bit weights, at most 16 rows already in the compute dtype, whole K tiles, and a group
-// size whose boundaries never split a lane's 32 consecutive K values.
+// At most 32 rows already in the compute dtype, whole K tiles, and (4-bit) a group size whose
+// boundaries never split a lane's 32 consecutive K values (8-bit: 16).
 bool decode_dq_applies(const FpArgs& f, int wbits, int regime) {
   const int want = regime == kRegimeF16 ? WOQ_HIP_ACT_FP16 : WOQ_HIP_ACT_BF16;
-  if (wbits != 4 || f.M > 16 || f.x_dtype != want || ((uintptr_t)f.x & 15) != 0) return false;
-  if (f.K % kTileK4 != 0 || f.M * f.K * 2 >= (int64_t)1 << 31) return false;
-  if (f.G >= f.KT * kTileK4) return true;
-  return f.G >= 32 && (f.G & (f.G - 1)) == 0;
+  const int tk = wbits == 4 ? kTileK4 : kTileK8;
+  if (f.M > 32 || f.x_dtype != want || ((uintptr_t)f.x & 15) != 0) return false;
+  if (f.K % tk != 0 || f.M * f.K * 2 >= (int64_t)1 << 31) return false;
+  if (f.G >= f.KT * tk) return true;
+  return f.G >= (wbits == 4 ? 32 : 16) && (f.G & (f.G - 1)) == 0;
 }
 
-int launch_decode_dq(const FpArgs& f, int regime, hipStream_t st, int ntw) {
+template <int REGIME, int WBITS>
+static int launch_dq_regime(const DecodeDqArgs& a, int ntw, hipStream_t st) {
+  const bool two_rows = a.f.M > 16;
+  if (ntw == 4) return two_rows ? launch_dq_cfg<REGIME, WBITS, 2, 4>(a, st) : launch_dq_cfg<REGIME, WBITS, 1, 4>(a, st);
+  if (ntw == 2) return two_rows ? launch_dq_cfg<REGIME, WBITS, 2, 2>(a, st) : launch_dq_cfg<REGIME, WBITS, 1, 2>(a, st);
+  return two_rows ? launch_dq_cfg<REGIME, WBITS, 2, 1>(a, st) : launch_dq_cfg<REGIME, WBITS, 1, 1>(a, st);
+}
+
+int launch_decode_dq(const FpArgs& f, int wbits, int regime, hipStream_t st, int ntw) {
   DecodeDqArgs a;
   a.f = f;
+  a.W = 1;
   a.g_shift = 30;
-  if (f.G < f.KT * kTileK4) {
+  if (f.G < f.KT * (wbits == 4 ? kTileK4 : kTileK8)) {
     a.g_shift = 0;
     while (((int64_t)1 << a.g_shift) < f.G) ++a.g_shift;
   }
-  a.W = (int)(f.KT < 8 ? f.KT : 8);
+  if (ntw != 0 && ntw != 1 && ntw != 2 && ntw != 4)
+    return set_error("woq_decode_dq_kernel: 1, 2 or 4 row-blocks per workgroup, got %d", ntw);
   if (ntw != 0 && f.NT % ntw != 0)
     return set_error("woq_decode_dq_kernel: %d row-blocks per workgroup do not divide %lld", ntw, (long long)f.NT);
   // Two row-blocks per workgroup re-read the activations half as often; with one there are twice
   // as many workgroups, which small N needs to fill the chip (two workgroups per CU are resident).
   if (ntw == 0) ntw = (f.NT >= 512 && f.NT % 2 == 0) ? 2 : 1;
-  if (ntw == 4)
-    return regime == kRegimeF16 ? launch_dq_cfg<kRegimeF16, 4>(a, st) : launch_dq_cfg<kRegimeBF16, 4>(a, st);
-  if (ntw == 2)
-    return regime == kRegimeF16 ? launch_dq_cfg<kRegimeF16, 2>(a, st) : launch_dq_cfg<kRegimeBF16, 2>(a, st);
-  if (ntw == 1)
-    return regime == kRegimeF16 ? launch_dq_cfg<kRegimeF16, 1>(a, st) : launch_dq_cfg<kRegimeBF16, 1>(a, st);
-  return set_error("woq_decode_dq_kernel: 1, 2 or 4 row-blocks per workgroup, got %d", ntw);
+  if (wbits == 4)
+    return regime == kRegimeF16 ? launch_dq_regime<kRegimeF16, 4>(a, ntw, st)
+                                : launch_dq_regime<kRegimeBF16, 4>(a, ntw, st);
+  return regime == kRegimeF16 ? launch_dq_regime<kRegimeF16, 8>(a, ntw, st)
+                              : launch_dq_regime<kRegimeBF16, 8>(a, ntw, st);
 }
 
 }  // namespace woq

@@ -69,10 +69,10 @@ struct DecodeArgs {
 bool decode_kernel_applies(const FpArgs& f, int wbits, int regime, const uint32_t* sz);
 int launch_decode(const FpArgs& f, const uint32_t* sz, hipStream_t st);
 
-// Decode kernel with per-weight dequantization (woq_decode_dq.hip): 4-bit, M <= 16.
-// ntw: weight row-blocks per workgroup (1 or 2), 0 = automatic
+// Decode kernel with per-weight dequantization (woq_decode_dq.hip): 4- or 8-bit weights, M <= 32.
+// ntw: weight row-blocks per workgroup (1, 2 or 4), 0 = automatic
 bool decode_dq_applies(const FpArgs& f, int wbits, int regime);
-int launch_decode_dq(const FpArgs& f, int regime, hipStream_t st, int ntw = 0);
+int launch_decode_dq(const FpArgs& f, int wbits, int regime, hipStream_t st, int ntw = 0);
 
 // regime: 0 = fp16, 1 = bf16 (woq::Regime)
 int launch_small_m(const FpArgs& a, int wbits, int regime, hipStream_t st);

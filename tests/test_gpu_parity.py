@@ -302,6 +302,21 @@ def test_dequantizing_decode_kernel(cuda, M, K, N, G, bias, kernel):
     _check_fp(case, lowp, force_kernel=kernel, label=f"decode dq M={M} K={K} N={N} G={G} kernel={kernel}")
 
 
+@pytest.mark.parametrize("M", [1, 7, 16, 17, 32])
+@pytest.mark.parametrize("kernel", [7, 9, 10])
+def test_dequantizing_decode_kernel_int8_weights(cuda, M, kernel):
+    """8-bit weights (64 K values per tile) and two row tiles (M > 16)."""
+    case = _synthetic().make_int8_case(33, M, 704, 128)  # 11 K tiles: a partial last round
+    lowp = O.LOWP_NONE if M < 5 else O.LOWP_BF16
+    _check_fp(case, lowp, force_kernel=kernel, label=f"decode dq int8 weights M={M} kernel={kernel}")
+
+
+@pytest.mark.parametrize("M,K,N,G", [(20, 1024, 96, 128), (32, 2048, 64, 32), (17, 384, 48, -1)])
+def test_dequantizing_decode_kernel_two_row_tiles_int4(cuda, M, K, N, G):
+    case = _synthetic().make_int4_case(34, M, K, N, G, bias=True)
+    _check_fp(case, O.LOWP_BF16, force_kernel=7, label=f"decode dq int4 M={M} K={K} N={N} G={G}")
+
+
 def test_dequantizing_decode_kernel_fp16_regime_and_symmetric(cuda):
     """fp16 regime with a group size the integer-weight decode kernel does not take, and weights
     without zero points."""
@@ -329,7 +344,7 @@ def test_dequantizing_decode_kernel_close_to_small_m_kernel(cuda):
     a, b = to_np_f32(ctx.run(x, force_kernel=7)), to_np_f32(ctx.run(x, force_kernel=1))
     assert bool(np.all((bf16_ulp_diff(a, b) <= 1) | (np.abs(a - b) <= 1e-4)))
     with pytest.raises(RuntimeError, match="dequantizing decode kernel"):
-        ctx.run(torch.randn(17, 2048, device=cuda).bfloat16(), force_kernel=7)
+        ctx.run(torch.randn(33, 2048, device=cuda).bfloat16(), force_kernel=7)
 
 
 def test_int8_weights_small_and_tiled(cuda):
