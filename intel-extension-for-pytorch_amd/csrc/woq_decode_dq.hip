@@ -16,13 +16,14 @@
 // (tiles and parameters into registers, activations into the other LDS buffer) are issued before
 // round r is computed.
 // Activations: a wave copies the rows of its K tile (16 or 32 rows x 256 bytes for 4-bit weights,
-// x 128 bytes for 8-bit ones) straight into its private slice of LDS (global_load_lds_dwordx4: four fully coalesced instructions, no registers) and reads the
-// operand fragments from there; chunk p of row m sits at p ^ m (p ^ (m / 2) for the 128-byte rows)
-// so the fragment reads are conflict-free.  Reading the fragments from global memory directly costs the same number of
-// instructions but each one gathers 64 separate 16-byte pieces, which made the texture addresser
-// the bottleneck (M = 16: 19.7 us against 13.9 us at M = 8 for the same weights).  Rows past M
-// re-read row M - 1 and their results are dropped.  The at most 64 KiB of slices are reused for
-// the cross-wave sum, so two workgroups fit on a CU.
+// x 128 bytes for 8-bit ones) straight into its private slice of LDS (global_load_lds_dwordx4:
+// fully coalesced, no registers) and reads the operand fragments from there; chunk p of row m sits
+// at p ^ m (p ^ (m / 2) for the 128-byte rows) so the fragment reads are conflict-free.  Reading
+// the fragments from global memory directly costs the same number of instructions but each one
+// gathers 64 separate 16-byte pieces, which made the texture addresser the bottleneck (M = 16:
+// 19.7 us against 13.9 us at M = 8 for the same weights).  Rows past M re-read row M - 1 and their
+// results are dropped.  The at most 64 KiB of slices are reused for the cross-wave sum, so two
+// workgroups fit on a CU.
 #include "woq_common.h"
 #include "woq_internal.h"
 
