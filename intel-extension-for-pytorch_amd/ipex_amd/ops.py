@@ -17,6 +17,7 @@ The context is a Python object here (the reference's is a TorchScript custom cla
 (csrc/cpu/jit/cpu/kernels/OpContext.cpp:396-400), and the ops resolve it through a registry
 of live contexts, so a stale handle raises instead of dereferencing freed memory.
 """
+import ctypes
 import os
 import threading
 import weakref
@@ -210,7 +211,8 @@ class WoqLinearOpContext:
         return torch.tensor([self._handle], dtype=torch.int64)
 
     def load_from_ctx(self, other):
-        self.__dict__.update({k: v for k, v in other.__dict__.items() if k != "_handle"})
+        self.__dict__.pop("_tls", None)  # cached parameter blocks point at the old tensors
+        self.__dict__.update({k: v for k, v in other.__dict__.items() if k not in ("_handle", "_tls")})
 
     # ---- pickling: always the plain format, re-prepacked on load (OpContext.h:363-403) ----
     def __getstate__(self):
@@ -234,6 +236,59 @@ class WoqLinearOpContext:
         self.__init__(*state)
 
     # ---- execution ----
+    def _run_planned(self, x, M, fusion, others):
+        """The common call (floating-point regimes, no debugging options) through a parameter
+        block that is filled once per context and thread: per call only the activation / output
+        pointers, M, the post-op and the stream change."""
+        N, K = self.weight_shape_
+        tl = self.__dict__.setdefault("_tls", threading.local())
+        p = getattr(tl, "plan", None)
+        if p is None:
+            p = _lib.LinearParams()
+            p.struct_size = ctypes.sizeof(_lib.LinearParams)
+            p.K, p.N = K, N
+            p.qweight = self.at_weight_.data_ptr()
+            p.weight_dtype = self.weight_dtype_
+            p.scales_f32 = self.scales_list_[0].data_ptr()
+            p.scales_f16 = self.scales_list_[1].data_ptr()
+            p.scales_bf16 = self.scales_list_[2].data_ptr()
+            p.zeros_u8 = self.zeros_u8_.data_ptr() if self.zeros_u8_ is not None else None
+            p.scale_zero_f16x2 = self.scale_zero_f16x2_.data_ptr() if self.scale_zero_f16x2_ is not None else None
+            p.group_size = self.group_size_
+            p.bias = self.bias_f32_.data_ptr() if self.bias_f32_ is not None else None
+            p.lowp_mode = self.lowp_mode_
+            p.act_quant_mode = self.act_quant_mode_
+            tl.plan = p
+        x2 = x if x.is_contiguous() else x.contiguous()
+        if x2.data_ptr() % 16:
+            x2 = x2.clone()  # the kernels read activation rows with 16-byte loads
+        out = torch.empty((*x.shape[:-1], N), dtype=x.dtype, device=x.device)
+        code = _kernels._ACT_CODE[x.dtype]
+        p.x, p.x_dtype, p.M = x2.data_ptr(), code, M
+        p.out, p.out_dtype = out.data_ptr(), code
+        p.fusion = fusion
+        keep = []
+        for i in range(2):
+            if i < len(others):
+                o = others[i]
+                if o.numel() != M * N:
+                    raise RuntimeError("woq_linear: post-op operand must have the output's shape")
+                o = o.to(x.dtype).contiguous()
+                keep.append(o)
+                p.others[i] = o.data_ptr()
+            else:
+                p.others[i] = None
+        lib = _lib.load()
+        if x.device.index == torch.cuda.current_device():
+            p.stream = torch.cuda.current_stream().cuda_stream
+            rc = lib.woq_hip_linear(ctypes.byref(p))
+        else:
+            with torch.cuda.device(x.device):
+                p.stream = torch.cuda.current_stream().cuda_stream
+                rc = lib.woq_hip_linear(ctypes.byref(p))
+        _lib.check(rc, "woq_linear")
+        return out
+
     def _cached_bf16_weight(self):
         if self.cached_weight_ is None:
             N, K = self.weight_shape_
@@ -267,6 +322,8 @@ class WoqLinearOpContext:
             w = self._cached_bf16_weight()
             b = self.at_bias_.to(torch.bfloat16) if self.at_bias_ is not None else None
             return torch.nn.functional.linear(x.to(torch.bfloat16), w, b).to(x.dtype)
+        if not kw and self.lowp_mode_ != _lib.LOWP_INT8 and x.dtype in _kernels._ACT_CODE and x.is_cuda:
+            return self._run_planned(x, M, fusion, others)
         return _kernels.linear(
             x,
             self.at_weight_,
