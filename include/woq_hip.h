@@ -46,7 +46,9 @@
 extern "C" {
 #endif
 
-/* weight dtype, csrc/cpu/aten/utils/woq_defines.h:6-9 */
+/* weight dtype, csrc/cpu/aten/utils/woq_defines.h:6-9.  NF4: 4-bit codes into the NormalFloat4 table
+ * (csrc/cpu/aten/utils/woq_utils.h:34-51), packed like INT4, symmetric only, floating-point
+ * lowp modes only (woq_hip_linear returns an error for NF4 with WOQ_HIP_LOWP_INT8). */
 #define WOQ_HIP_DTYPE_INT8 1
 #define WOQ_HIP_DTYPE_INT4 2
 #define WOQ_HIP_DTYPE_NF4 3
@@ -201,7 +203,8 @@ typedef struct woq_hip_linear_params {
    * 3 = 4-bit prefill GEMM (K % 128 == 0, power-of-two or per-channel groups, x in the compute dtype),
    * workgroup shape by cost model; 4 / 5 / 6 = the same kernel with 448 / 256 / 128 columns per workgroup;
    * 7 = dequantizing decode kernel (M <= 32, K % 128 == 0 for 4-bit and K % 64 == 0 for 8-bit weights, x in the
-   * compute dtype), 8 / 9 / 10 = the same with one / two / four weight row-blocks per workgroup */
+   * compute dtype), 8 / 9 / 10 = the same with one / two / four weight row-blocks per workgroup.
+   * NF4 weights: 0, 1, 2, 7, 8, 9 only */
   int32_t force_kernel;
 
   void* stream;

@@ -24,7 +24,9 @@ int check_launch(const char* what) {
   return 0;
 }
 
-static bool valid_wdtype(int d) { return d == WOQ_HIP_DTYPE_INT8 || d == WOQ_HIP_DTYPE_INT4; }
+static bool valid_wdtype(int d) {
+  return d == WOQ_HIP_DTYPE_INT8 || d == WOQ_HIP_DTYPE_INT4 || d == WOQ_HIP_DTYPE_NF4;
+}
 
 }  // namespace woq
 
@@ -156,6 +158,10 @@ int woq_hip_linear(const woq_hip_linear_params* p) {
   const int64_t KG = p->group_size > 0 ? (p->K + G - 1) / G : 1;
   hipStream_t st = (hipStream_t)p->stream;
 
+  const bool nf4 = p->weight_dtype == WOQ_HIP_DTYPE_NF4;
+  if (nf4 && p->zeros_u8) return set_error("woq_linear: symmetric quantization is required for NF4 weights");
+  if (nf4 && p->lowp_mode == WOQ_HIP_LOWP_INT8)
+    return set_error("woq_linear: NF4 weights run in the floating-point regimes only (lowp_mode NONE, FP16 or BF16)");
   int lowp = p->lowp_mode;
   if (lowp == WOQ_HIP_LOWP_INT8) {
     const int64_t bk = woq_hip_int8_block_k(p->group_size, p->K);
@@ -201,8 +207,16 @@ int woq_hip_linear(const woq_hip_linear_params* p) {
   f.scales = (const uint16_t*)(regime == kRegimeF16 ? p->scales_f16 : p->scales_bf16);
   f.zeros = p->zeros_u8; f.G = G; f.KG = KG; f.bias = p->bias; f.fusion = p->fusion;
   f.other0 = p->others[0]; f.other1 = p->others[1]; f.out = p->out; f.out_dtype = p->out_dtype;
+  f.nf4 = nf4 ? 1 : 0;
 
   int kernel = p->force_kernel;
+  if (nf4) {
+    // table lookups instead of the integer decode: the dequantizing decode kernel and the two
+    // general kernels carry them
+    if (kernel == 0) kernel = decode_dq_applies(f, wbits, regime) ? 7 : (p->M <= 64 ? 1 : 2);
+    if (kernel != 1 && kernel != 2 && (kernel < 7 || kernel > 9))
+      return set_error("woq_linear: NF4 weights run on kernels 1, 2 and 7..9 only");
+  }
   if (kernel == 0 && decode_kernel_applies(f, wbits, regime, p->scale_zero_f16x2))
     return launch_decode(f, p->scale_zero_f16x2, st);
   if (kernel == 0 && decode_dq_applies(f, wbits, regime)) kernel = 7;

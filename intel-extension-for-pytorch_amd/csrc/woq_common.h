@@ -288,5 +288,31 @@ __device__ __forceinline__ u4 g4_dequant(uint32_t d, const G4Masks& k, const G4C
   return r;
 }
 
+// ---- NF4 weights: 4-bit codes into a fixed table of 16 values in [-1, 1] ----------------------
+// The table of csrc/cpu/aten/utils/woq_utils.h:34-51 (the NormalFloat4 code book); w = table[q] *
+// scale, the product rounded to fp32 and then once to the compute dtype
+// (csrc/cpu/aten/utils/woq_utils.h:165-262).
+static __constant__ const float kNf4Values[16] = {
+    -1.0f, -0.6961928009986877f, -0.5250730514526367f, -0.39491748809814453f,
+    -0.28444138169288635f, -0.18477343022823334f, -0.09105003625154495f, 0.0f,
+    0.07958029955625534f, 0.16093020141124725f, 0.24611230194568634f, 0.33791524171829224f,
+    0.44070982933044434f, 0.5626170039176941f, 0.7229568362236023f, 1.0f};
+
+// One packed dword (8 codes of one row) -> 8 compute-dtype weights in K order.  `lut` is a copy
+// of the table in LDS: the 64 lanes read at most 16 distinct words, one per bank.
+template <int REGIME>
+__device__ __forceinline__ u4 nf4_dequant(uint32_t d, const float* lut, float s) {
+  u4 r;
+#pragma unroll
+  for (int v = 0; v < 4; ++v) {
+    const float lo = __fmul_rn(lut[(d >> (4 * v)) & 15u], s);
+    const float hi = __fmul_rn(lut[(d >> (16 + 4 * v)) & 15u], s);
+    if constexpr (REGIME == kRegimeF16)
+      r[v] = (uint32_t)f32_to_f16_bits(lo) | ((uint32_t)f32_to_f16_bits(hi) << 16);
+    else
+      r[v] = g4_cvt_pair(f2{lo, hi});
+  }
+  return r;
+}
 
 }  // namespace woq

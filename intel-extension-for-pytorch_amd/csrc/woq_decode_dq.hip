@@ -66,11 +66,18 @@ struct G8Consts {
   float s, c;
 };
 
-template <int REGIME, int WBITS, int MT, int NTW>
+// NF4: the 4-bit codes index the NormalFloat4 table (a copy in LDS) and there are no zero points.
+template <int REGIME, int WBITS, int MT, int NTW, bool NF4>
 __global__ __launch_bounds__(512, 4) void woq_decode_dq_kernel(const DecodeDqArgs a) {
   using Geo = DqGeom<WBITS, MT>;
   constexpr int TK = Geo::TK, NJ = Geo::NJ, NX = Geo::NX, SLICE = Geo::SLICE;
+  static_assert(!NF4 || WBITS == 4, "NF4 codes are 4 bits wide");
   extern __shared__ __align__(1024) uint8_t smem[];
+  __shared__ float sNf4[16];
+  if constexpr (NF4) {
+    if (threadIdx.x < 16) sNf4[threadIdx.x] = kNf4Values[threadIdx.x];
+    __syncthreads();
+  }
   const FpArgs& f = a.f;
   const int W = a.W;
   const int lane = threadIdx.x & 63;
@@ -149,11 +156,13 @@ __global__ __launch_bounds__(512, 4) void woq_decode_dq_kernel(const DecodeDqArg
   for (int kt = wave, buf = 0; kt < KT; kt += W, buf ^= 1) {
     u4 wreg[NTW];
     G4Consts<REGIME> qc4[WBITS == 4 ? NTW : 1];
-    G8Consts qc8[WBITS == 8 ? NTW : 1];
+    G8Consts qc8[WBITS == 8 || NF4 ? NTW : 1];
 #pragma unroll
     for (int t = 0; t < NTW; ++t) {
       wreg[t] = wnext[t];
-      if constexpr (WBITS == 4) {
+      if constexpr (NF4) {
+        qc8[t].s = REGIME == kRegimeF16 ? f16_bits_to_f32(snext[t]) : bf16_bits_to_f32(snext[t]);
+      } else if constexpr (WBITS == 4) {
         qc4[t].set(snext[t], has_z ? (float)znext[t] : 8.0f);
       } else {
         qc8[t].s = REGIME == kRegimeF16 ? f16_bits_to_f32(snext[t]) : bf16_bits_to_f32(snext[t]);
@@ -173,7 +182,9 @@ __global__ __launch_bounds__(512, 4) void woq_decode_dq_kernel(const DecodeDqArg
 #pragma unroll
       for (int t = 0; t < NTW; ++t) {
         u4 bop;
-        if constexpr (WBITS == 4) {
+        if constexpr (NF4) {
+          bop = nf4_dequant<REGIME>(wreg[t][j], sNf4, qc8[t].s);
+        } else if constexpr (WBITS == 4) {
           bop = g4_dequant(wreg[t][j], km, qc4[t]);
         } else if constexpr (REGIME == kRegimeF16) {
           bop = bitcast<u4>(dequant8_f16_w8(wreg[t][2 * j], wreg[t][2 * j + 1], qc8[t].s, qc8[t].c));
@@ -220,7 +231,7 @@ __global__ __launch_bounds__(512, 4) void woq_decode_dq_kernel(const DecodeDqArg
   }
 }
 
-template <int REGIME, int WBITS, int MT, int NTW>
+template <int REGIME, int WBITS, int MT, int NTW, bool NF4 = false>
 static int launch_dq_cfg(DecodeDqArgs a, hipStream_t st) {
   using Geo = DqGeom<WBITS, MT>;
   // at most 64 KiB of activation buffers per workgroup, so that two workgroups share a CU
@@ -231,7 +242,7 @@ static int launch_dq_cfg(DecodeDqArgs a, hipStream_t st) {
   const size_t red = (size_t)NTW * MT * a.W * 64 * sizeof(f4);
   if (red > smem) smem = red;
   const unsigned grid = (unsigned)(a.f.NT / NTW);
-  woq_decode_dq_kernel<REGIME, WBITS, MT, NTW><<<grid, a.W * 64, smem, st>>>(a);
+  woq_decode_dq_kernel<REGIME, WBITS, MT, NTW, NF4><<<grid, a.W * 64, smem, st>>>(a);
   return check_launch("woq_decode_dq_kernel");
 }
 
@@ -254,6 +265,14 @@ static int launch_dq_regime(const DecodeDqArgs& a, int ntw, hipStream_t st) {
   return two_rows ? launch_dq_cfg<REGIME, WBITS, 2, 1>(a, st) : launch_dq_cfg<REGIME, WBITS, 1, 1>(a, st);
 }
 
+// NF4: one or two row-blocks per workgroup.
+template <int REGIME>
+static int launch_dq_nf4(const DecodeDqArgs& a, int ntw, hipStream_t st) {
+  const bool two_rows = a.f.M > 16;
+  if (ntw == 2) return two_rows ? launch_dq_cfg<REGIME, 4, 2, 2, true>(a, st) : launch_dq_cfg<REGIME, 4, 1, 2, true>(a, st);
+  return two_rows ? launch_dq_cfg<REGIME, 4, 2, 1, true>(a, st) : launch_dq_cfg<REGIME, 4, 1, 1, true>(a, st);
+}
+
 int launch_decode_dq(const FpArgs& f, int wbits, int regime, hipStream_t st, int ntw) {
   DecodeDqArgs a;
   a.f = f;
@@ -270,6 +289,11 @@ int launch_decode_dq(const FpArgs& f, int wbits, int regime, hipStream_t st, int
   // Two row-blocks per workgroup re-read the activations half as often; with one there are twice
   // as many workgroups, which small N needs to fill the chip (two workgroups per CU are resident).
   if (ntw == 0) ntw = (f.NT >= 512 && f.NT % 2 == 0) ? 2 : 1;
+  if (f.nf4) {
+    if (wbits != 4 || f.zeros) return set_error("woq_decode_dq_kernel: NF4 weights are 4-bit and symmetric");
+    if (ntw == 4) return set_error("woq_decode_dq_kernel: NF4 weights take 1 or 2 row-blocks per workgroup");
+    return regime == kRegimeF16 ? launch_dq_nf4<kRegimeF16>(a, ntw, st) : launch_dq_nf4<kRegimeBF16>(a, ntw, st);
+  }
   if (wbits == 4)
     return regime == kRegimeF16 ? launch_dq_regime<kRegimeF16, 4>(a, ntw, st)
                                 : launch_dq_regime<kRegimeBF16, 4>(a, ntw, st);

@@ -55,6 +55,13 @@ __global__ __launch_bounds__(256) void woq_gemm_kernel(const FpArgs f) {
   const int64_t nt0 = n0 / kTileN;
   const int64_t Kpad = f.KT * TK;
 
+  __shared__ float sNf4[16];
+  const bool nf4 = WBITS == 4 && f.nf4 != 0;
+  if (nf4) {
+    if (tid < 16) sNf4[tid] = kNf4Values[tid];
+    __syncthreads();
+  }
+
   f16v acc[2][2];
 #pragma unroll
   for (int i = 0; i < 2; ++i)
@@ -124,7 +131,11 @@ __global__ __launch_bounds__(256) void woq_gemm_kernel(const FpArgs f) {
         if (f.zeros) zb = f.zeros[qi];
       }
       const float z = f.zeros ? (float)zb : (WBITS == 4 ? 8.0f : 128.0f);
-      if (WBITS == 4) {
+      if (nf4) {
+        const float s = REGIME == kRegimeF16 ? f16_bits_to_f32(sbits) : bf16_bits_to_f32(sbits);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) wd[j] = bitcast<vec8>(nf4_dequant<REGIME>(wv[q][j], sNf4, s));
+      } else if (WBITS == 4) {
         if constexpr (REGIME == kRegimeF16) {
           const _Float16 s = bitcast<_Float16>(sbits);
           const _Float16 nz = (_Float16)(-(1024.0f + z));

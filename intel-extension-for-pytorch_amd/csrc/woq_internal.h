@@ -32,6 +32,7 @@ struct FpArgs {
   const void* other1;
   void* out;
   int out_dtype;
+  int nf4;  // 4-bit codes index the NF4 table instead of standing for integers (zeros == nullptr)
 };
 
 int launch_pack_weight(const void* plain, int weight_dtype, int64_t N, int64_t K, void* packed,

@@ -167,12 +167,14 @@ __global__ void dequant_weight_kernel(const uint8_t* __restrict__ packed, int we
 #pragma unroll
     for (int e = 0; e < 8; ++e) w[e] = (float)p[e];
   }
+  const bool nf4 = weight_dtype == WOQ_HIP_DTYPE_NF4;
 #pragma unroll
   for (int e = 0; e < 8; ++e) {
     const int64_t k = k0 + e;
     if (k >= K) break;
-    // (q - z) first, then the scale, each in fp32 (woq_utils.h:147-161)
-    const float v = __fmul_rn(__fsub_rn(w[e], z), s);
+    // (q - z) first, then the scale, each in fp32 (woq_utils.h:147-161); NF4: table value times
+    // scale (woq_utils.h:165-262)
+    const float v = nf4 ? __fmul_rn(kNf4Values[(int)w[e]], s) : __fmul_rn(__fsub_rn(w[e], z), s);
     store_act(out, out_dtype, n * K + k, v);
   }
 }

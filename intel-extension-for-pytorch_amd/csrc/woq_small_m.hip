@@ -119,6 +119,13 @@ __global__ __launch_bounds__(1024) void woq_small_m_kernel(const SmallMArgs a) {
   uint16_t* sx = (uint16_t*)(smem + (size_t)NTW * MT * W * 64 * sizeof(f4));  // [rows][KC]
   const int rows = (int)(f.M < MT * 16 ? f.M : MT * 16);
 
+  __shared__ float sNf4[16];
+  const bool nf4 = WBITS == 4 && f.nf4 != 0;
+  if (nf4) {
+    if (threadIdx.x < 16) sNf4[threadIdx.x] = kNf4Values[threadIdx.x];
+    __syncthreads();
+  }
+
   f4 acc[NTW][MT];
 #pragma unroll
   for (int t = 0; t < NTW; ++t)
@@ -201,7 +208,13 @@ __global__ __launch_bounds__(1024) void woq_small_m_kernel(const SmallMArgs a) {
       for (int i = 0; i < KPW; ++i) {
         const LaneQ<WBITS, REGIME> q = make_laneq<WBITS, REGIME>(sreg[t][i], f.zeros != nullptr, zreg[t][i]);
         vec8 aop[STEPS];
-        dequant_tile<WBITS, REGIME>(wreg[t][i], q, aop);
+        if (nf4) {
+          const float s = REGIME == kRegimeF16 ? f16_bits_to_f32(sreg[t][i]) : bf16_bits_to_f32(sreg[t][i]);
+#pragma unroll
+          for (int j = 0; j < STEPS; ++j) aop[j] = bitcast<vec8>(nf4_dequant<REGIME>(wreg[t][i][j], sNf4, s));
+        } else {
+          dequant_tile<WBITS, REGIME>(wreg[t][i], q, aop);
+        }
 #pragma unroll
         for (int j = 0; j < STEPS; ++j)
 #pragma unroll

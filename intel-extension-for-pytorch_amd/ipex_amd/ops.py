@@ -86,16 +86,20 @@ class WoqLinearOpContext:
         cache_weight_for_large_batch=False,
     ):
         weight_dtype = int(weight_dtype)
-        if weight_dtype not in (_lib.DTYPE_INT8, _lib.DTYPE_INT4):
-            raise RuntimeError(f"WOQ linear: unsupported weight dtype {weight_dtype} (INT8 and INT4 are built)")
+        if weight_dtype not in (_lib.DTYPE_INT8, _lib.DTYPE_INT4, _lib.DTYPE_NF4):
+            raise RuntimeError(f"WOQ linear: unsupported weight dtype {weight_dtype}")
+        if weight_dtype == _lib.DTYPE_NF4 and zero_points is not None:
+            raise RuntimeError("WOQ: symmetric quantization is required for NF4 or INT8 with lowp-mode INT8")
+        if weight_dtype == _lib.DTYPE_NF4 and int(lowp_mode) == _lib.LOWP_INT8:
+            raise RuntimeError("WOQ linear: NF4 weights run with lowp_mode NONE, FP16 or BF16 (INT8 is not built)")
         N, K = int(weight_shape[0]), int(weight_shape[1])
         weight = _to_gpu(weight)
         dev = weight.device
-        if weight_dtype == _lib.DTYPE_INT4:
+        if weight_dtype != _lib.DTYPE_INT8:
             weight = weight.view(torch.uint8) if weight.dtype != torch.uint8 else weight
             if tuple(weight.shape) != (N, (K + 1) // 2):
                 raise RuntimeError(
-                    f"WOQ linear: int4 weight has shape {tuple(weight.shape)}, expected {(N, (K + 1) // 2)}"
+                    f"WOQ linear: 4-bit weight has shape {tuple(weight.shape)}, expected {(N, (K + 1) // 2)}"
                 )
         else:
             if weight.dtype != torch.int8 or tuple(weight.shape) != (N, K):

@@ -31,6 +31,16 @@ def make_int4_case(cfg, M, K, N, group_size, outliers=False, bias=False, scale_d
                 group_size=group_size, weight_dtype=2)
 
 
+def make_nf4_case(cfg, M, K, N, group_size, bias=False, scale_dtype=torch.bfloat16):
+    """NF4 weights: codes uniform in 0..15 packed like int4, absmax scales uniform in [0.02, 0.08],
+    no zero points."""
+    case = make_int4_case(cfg, M, K, N, group_size, bias=bias, scale_dtype=scale_dtype)
+    case["scales"] = (case["scales"] * 4).to(scale_dtype).float()
+    case["zeros"] = None
+    case["weight_dtype"] = 3
+    return case
+
+
 def make_int8_case(cfg, M, K, N, bias=True):
     """Per-output-channel symmetric int8 weights uniform in -127..127, fp32 scales uniform in
     [0.001, 0.01], bf16 bias ~ N(0, 0.02)."""

@@ -101,10 +101,28 @@ def unpack_compressed_zeros(zp32, cols):
     return ((z[:, j // 8] >> ((j % 8) * 4).astype(np.uint32)) & 0xF).astype(np.float32)
 
 
+# The NormalFloat4 code book (csrc/cpu/aten/utils/woq_utils.h:34-51): 16 values in [-1, 1], code 7
+# is exactly zero.
+NF4_DEQUANT_TABLE = np.array(
+    [
+        -1.0, -0.6961928009986877, -0.5250730514526367, -0.39491748809814453,
+        -0.28444138169288635, -0.18477343022823334, -0.09105003625154495, 0.0,
+        0.07958029955625534, 0.16093020141124725, 0.24611230194568634, 0.33791524171829224,
+        0.44070982933044434, 0.5626170039176941, 0.7229568362236023, 1.0,
+    ],
+    dtype=np.float32,
+)
+
+
 def dequantize_woq_weight(qw, N, K, scales, zps, weight_dtype, group_size):
     """fp32 (q - z) * s; q - z first, then the scale, both in fp32.  zps None: symmetric (INT4
-    codes stand for code - 8).  scales / zps: [N] or [N, ceil(K / group_size)]."""
-    if weight_dtype == WOQ_DTYPE_INT4:
+    codes stand for code - 8).  NF4: table[code] * s, no zero point
+    (csrc/cpu/aten/utils/woq_utils.h:64-77, 108-131).  scales / zps: [N] or
+    [N, ceil(K / group_size)]."""
+    if weight_dtype == WOQ_DTYPE_NF4:
+        assert zps is None, "NF4 is symmetric"
+        q = NF4_DEQUANT_TABLE[unpack_int4(qw)[:, :K]]
+    elif weight_dtype == WOQ_DTYPE_INT4:
         q = unpack_int4(qw)[:, :K].astype(np.float32)
         if zps is None:
             q = q - np.float32(8)
@@ -189,14 +207,19 @@ def _fma16(a, b, c):
 def woq_linear_opt_fp16(x, qw, N, K, scales, zps, bias, weight_dtype, group_size, block_k=None):
     """The M < 5 path with bf16 activations: everything in fp16, including the accumulators.
     Per output: C = fp16(bias) or 0; per K block of Kb = min(group_size, 64):
-    vc = 0; for k ascending: vc = fma(x_k, q_k - z, vc); then C = fma(s, vc, C); y = bf16(C)."""
-    assert weight_dtype == WOQ_DTYPE_INT4
+    vc = 0; for k ascending: vc = fma(x_k, q_k - z, vc); then C = fma(s, vc, C); y = bf16(C).
+    NF4: q_k is the table value rounded to fp16 and there is no z (the fp16 lookup table of
+    csrc/cpu/aten/utils/woq.h:827-836)."""
+    assert weight_dtype in (WOQ_DTYPE_INT4, WOQ_DTYPE_NF4)
+    nf4 = weight_dtype == WOQ_DTYPE_NF4
+    assert not (nf4 and zps is not None), "NF4 is symmetric"
     M = x.shape[0]
     if block_k is None:
         block_k = min(group_size, 64) if group_size > 0 else 64
         while K % block_k:
             block_k //= 2
-    q = unpack_int4(qw)[:, :K].astype(np.float16)
+    q = unpack_int4(qw)[:, :K]
+    q = NF4_DEQUANT_TABLE[q].astype(np.float16) if nf4 else q.astype(np.float16)
     s = np.asarray(scales, dtype=np.float32).reshape(N, -1).astype(np.float16)
     z = None if zps is None else np.asarray(zps, dtype=np.float32).reshape(N, -1).astype(np.float16)
     xh = np.asarray(x, dtype=np.float32).astype(np.float16)
@@ -205,7 +228,7 @@ def woq_linear_opt_fp16(x, qw, N, K, scales, zps, bias, weight_dtype, group_size
         C[:] = np.asarray(bias, dtype=np.float32).astype(np.float16)[None, :]
     for kb in range(K // block_k):
         g = (kb * block_k) // group_size if group_size > 0 else 0
-        zg = z[:, g] if z is not None else np.float16(8)
+        zg = z[:, g] if z is not None else np.float16(0 if nf4 else 8)
         vc = np.zeros((M, N), dtype=np.float16)
         for k in range(kb * block_k, (kb + 1) * block_k):
             w = (q[:, k] - zg).astype(np.float16)  # exact small integers

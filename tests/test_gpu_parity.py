@@ -164,7 +164,7 @@ def _check_fp(case, lowp_mode, ctx=None, cols=None, force_kernel=0, label=""):
         assert stats["rel_l2_out_vs_opt"] <= REL_L2_OUT, (label, stats)
         # one bf16 ulp at most, except next to zero where an ulp is far below the accumulator bar
         assert bool(np.all((ulps <= 1) | (np.abs(y - y_opt) <= 1e-4))), (label, stats)
-    elif wd == 2 and M <= 4 and N * K <= 4096 * 4096:
+    elif wd in (2, 3) and M <= 4 and N * K <= 4096 * 4096:
         # the optimized fp16 kernel accumulates in fp16; its own rounding noise exceeds 1e-2 at
         # these magnitudes, so only the relative-L2 bar applies against it
         y_h = O.woq_linear_opt_fp16(c["x"], qw, N, K, sc, zp, b, wd, G)
@@ -365,6 +365,80 @@ def test_symmetric_int4(cuda):
     case = _synthetic().make_int4_case(18, 7, 512, 96, 128)
     case["zeros"] = None
     _check_fp(case, O.LOWP_BF16, label="sym int4")
+
+
+# ---------------------------------------------------------------------------------------------
+# NF4 weights (table lookups; floating-point regimes)
+# ---------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("M", [1, 4, 5, 16, 40, 64, 65, 200])
+@pytest.mark.parametrize("K,N,G", [(1024, 272, 128), (384, 48, 32), (1000, 100, -1)])
+def test_nf4_linear(cuda, M, K, N, G):
+    case = _synthetic().make_nf4_case(21, M, K, N, G, bias=(M % 2 == 0))
+    _check_fp(case, O.LOWP_BF16, label=f"nf4 M={M} K={K} N={N} G={G}")
+
+
+@pytest.mark.parametrize("M", [1, 4, 7, 16, 17, 32])
+@pytest.mark.parametrize("kernel", [1, 7, 8, 9])  # small-M kernel, then the decode kernel: automatic, 1, 2 row-blocks
+def test_nf4_decode_kernels(cuda, M, kernel):
+    case = _synthetic().make_nf4_case(27, M, 1024, 544, 128, bias=(M == 7))
+    # lowp_mode BF16 computes in fp16 below 5 rows, where bf16 activations need the converting
+    # small-M kernel; lowp_mode NONE keeps them in bf16 for the decode kernel
+    lowp = O.LOWP_NONE if (M < 5 and kernel >= 7) else O.LOWP_BF16
+    _check_fp(case, lowp, force_kernel=kernel, label=f"nf4 kernel {kernel} M={M}")
+
+
+def test_nf4_other_lowp_modes_and_fp16_activations(cuda):
+    syn = _synthetic()
+    for M in (3, 70):
+        case = syn.make_nf4_case(22, M, 512, 96, 64, bias=True)
+        _check_fp(case, O.LOWP_NONE, label=f"nf4 lowp NONE M={M}")
+        _check_fp(case, O.LOWP_FP16, label=f"nf4 lowp FP16 M={M}")
+    # fp16 activations, fp16 scales: w = fp16(table * s), fp32 accumulation
+    case = syn.make_nf4_case(23, 9, 256, 64, 32, scale_dtype=torch.float16)
+    ctx = make_context(case, O.LOWP_FP16)
+    xh = case["x"].to(torch.float16)
+    y = to_np_f32(ctx.run(xh.cuda()))
+    c = case_np(case)
+    _, y_ref = O.woq_linear_ref(to_np_f32(xh), "fp16", c["qw"], 64, 256, c["scales"], None, None, 3, 32, "fp16")
+    assert rel_l2(y, y_ref) <= REL_L2_OUT
+
+
+@pytest.mark.parametrize("G", [32, 128, -1])
+def test_nf4_dequant_weight_bit_exact_and_pack_roundtrip(cuda, G):
+    syn, k = _synthetic(), _kernels()
+    case = syn.make_nf4_case(24, 1, 512, 80, G, scale_dtype=torch.float32)
+    ctx = make_context(case, 2)
+    c = case_np(case)
+    want = O.dequantize_woq_weight(c["qw"], 80, 512, c["scales"], None, 3, G)
+    got = k.dequant_weight(ctx.at_weight_, 3, 80, 512, ctx.scales_list_[0], None, G)
+    assert np.array_equal(got.cpu().numpy(), want)
+    got16 = k.dequant_weight(ctx.at_weight_, 3, 80, 512, ctx.scales_list_[0], None, G, torch.bfloat16)
+    assert np.array_equal(to_np_f32(got16), O.bf16_round(want))
+    assert torch.equal(k.unpack_weight(ctx.at_weight_, 3, 80, 512).cpu(), case["qweight"])
+
+
+def test_nf4_rejections(cuda):
+    syn = _synthetic()
+    case = syn.make_nf4_case(25, 4, 256, 32, 64)
+    with pytest.raises(RuntimeError, match="NF4"):
+        make_context(case, O.LOWP_INT8, 6)
+    bad = dict(case, zeros=torch.zeros(32, 4))
+    with pytest.raises(RuntimeError, match="symmetric"):
+        make_context(bad, O.LOWP_BF16)
+    ctx = make_context(case, O.LOWP_BF16)
+    with pytest.raises(RuntimeError, match="NF4"):
+        ctx.run(case["x"].cuda(), force_kernel=3)
+    with pytest.raises(RuntimeError, match="NF4"):
+        ctx.run(case["x"].cuda(), force_kernel=10)
+
+
+def test_nf4_weight_cache_for_large_batch_matches_oracle(cuda):
+    case = _synthetic().make_nf4_case(26, 1200, 256, 64, 64)
+    ctx = make_context(case, O.LOWP_BF16, cache=True)
+    y = to_np_f32(ctx.run(case["x"].cuda()))
+    c = case_np(case)
+    _, y_opt = O.woq_linear_opt_bf16(c["x"], "bf16", c["qw"], 64, 256, c["scales"], None, None, 3, 64)
+    assert rel_l2(y, y_opt) <= REL_L2_OUT
 
 
 def test_empty_batch(cuda):

@@ -49,6 +49,84 @@ def test_dequantize_brute_force_all_codes():
     assert got[0].tolist() == [2.0 * (c - 8) for c in range(16)]
 
 
+def test_nf4_table_is_the_normal_quantile_code_book():
+    # The published construction of NormalFloat4 (QLoRA): 8 positive quantiles of N(0, 1) at
+    # linspace(offset, 0.5, 9)[:-1], zero, 7 negative ones at linspace(offset, 0.5, 8)[:-1],
+    # sorted and divided by the largest.  A mistyped or swapped entry misses it by far more than
+    # the fp32 rounding of the published digits.
+    from scipy.stats import norm
+
+    off = 0.9677083
+    pos = norm.ppf(np.linspace(off, 0.5, 9)[:-1])
+    neg = -norm.ppf(np.linspace(off, 0.5, 8)[:-1])
+    v = np.sort(np.concatenate([pos, [0.0], neg]))
+    v /= v.max()
+    t = O.NF4_DEQUANT_TABLE
+    assert t.dtype == np.float32 and t.shape == (16,)
+    assert np.abs(v - t).max() <= 2e-7
+    assert t[0] == -1.0 and t[7] == 0.0 and t[15] == 1.0 and np.all(np.diff(t) > 0)
+
+
+def test_nf4_dequantize_brute_force_and_groups():
+    # every code in every group: table[code] * scale of that group, a single fp32 product
+    N, K, G = 2, 64, 16
+    codes = np.tile(np.arange(16, dtype=np.uint8), (N, K // 16))
+    codes[1] = codes[1, ::-1]
+    scales = np.array([[0.5, 0.031, 3.0, 0.0123], [1.0, 0.07, 0.25, 9.0]], dtype=np.float32)
+    w = O.dequantize_woq_weight(O.pack_int4(codes), N, K, scales, None, O.WOQ_DTYPE_NF4, G)
+    for n in range(N):
+        for k in range(K):
+            exact = fractions.Fraction(float(O.NF4_DEQUANT_TABLE[codes[n, k]])) * fractions.Fraction(float(scales[n, k // G]))
+            assert w[n, k] == np.float32(float(exact)), (n, k)
+    # per-channel
+    w = O.dequantize_woq_weight(O.pack_int4(codes), N, K, np.array([2.0, 4.0], np.float32), None, O.WOQ_DTYPE_NF4, -1)
+    assert np.array_equal(w[0], 2 * O.NF4_DEQUANT_TABLE[codes[0]]) and np.array_equal(w[1], 4 * O.NF4_DEQUANT_TABLE[codes[1]])
+    with pytest.raises(AssertionError):
+        O.dequantize_woq_weight(O.pack_int4(codes), N, K, scales, scales, O.WOQ_DTYPE_NF4, G)
+
+
+def test_nf4_linear_paths_against_exact_rational_matmul():
+    rng = np.random.default_rng(5)
+    M, K, N, G = 3, 32, 4, 16
+    codes = rng.integers(0, 16, (N, K)).astype(np.uint8)
+    qw = O.pack_int4(codes)
+    scales = O.bf16_round(rng.uniform(0.02, 0.08, (N, K // G)).astype(np.float32))
+    x = O.bf16_round(rng.standard_normal((M, K)).astype(np.float32))
+    w = O.bf16_round(O.dequantize_woq_weight(qw, N, K, scales, None, O.WOQ_DTYPE_NF4, G))
+    exact = np.array(
+        [[float(sum(fractions.Fraction(float(x[m, k])) * fractions.Fraction(float(w[n, k])) for k in range(K)))
+          for n in range(N)] for m in range(M)]
+    )
+    acc, y = O.woq_linear_opt_bf16(x, "bf16", qw, N, K, scales, None, None, O.WOQ_DTYPE_NF4, G)
+    assert np.abs(acc - exact).max() <= 1e-12
+    assert np.array_equal(y, O.bf16_round(exact.astype(np.float32)))
+    # the fp16 chain rounds the table to fp16 and accumulates in fp16: close to, not equal to, exact
+    yh = O.woq_linear_opt_fp16(x, qw, N, K, scales, None, None, O.WOQ_DTYPE_NF4, G)
+    assert np.abs(yh - exact).max() <= 2e-2 * max(1.0, np.abs(exact).max())
+    # a zero scale row gives exact zeros whatever the codes (code 7 is 0, no implied offset)
+    s0 = scales.copy()
+    s0[2] = 0
+    assert np.all(O.woq_linear_opt_fp16(x, qw, N, K, s0, None, None, O.WOQ_DTYPE_NF4, G)[:, 2] == 0)
+
+
+def test_nf4_quantize_dequantize_roundtrip_error_bound():
+    # the package's quantizer picks the nearest table entry: error <= half the widest gap x scale
+    from ipex_amd.quantization._qconfig import WoqWeightDtype
+    from ipex_amd.quantization._quantize_utils import quantize_per_block
+
+    torch.manual_seed(3)
+    wt = torch.randn(8, 128) * 0.05
+    qw, sc, zp = quantize_per_block(wt, WoqWeightDtype.NF4, 32, sym_quant=True)
+    assert zp is None
+    w = O.dequantize_woq_weight(qw.numpy(), 8, 128, sc.numpy(), None, O.WOQ_DTYPE_NF4, 32)
+    half_gap = float(np.diff(O.NF4_DEQUANT_TABLE).max()) / 2
+    bound = half_gap * np.repeat(sc.numpy(), 32, axis=1)
+    assert np.all(np.abs(w - wt.numpy()) <= bound + 1e-7)
+    # the group's extreme element is reproduced exactly (code 0 or 15)
+    amax = wt.view(8, 4, 32).abs().max(dim=-1)[0].numpy()
+    assert np.allclose(np.abs(w).reshape(8, 4, 32).max(axis=-1), amax, rtol=0, atol=1e-7)
+
+
 def test_dequantize_group_indexing():
     # group g of row n must use scales[n, g]: make each group's scale identify it
     N, K, G = 3, 96, 32
