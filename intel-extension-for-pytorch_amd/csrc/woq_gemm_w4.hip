@@ -44,7 +44,8 @@ struct G4Shape {
   // block ahead of their first use needs a second set of MT fragment registers; with 16 row tiles
   // a block is long enough (256 cycles) to read them in the last block, each into the registers of
   // the fragment whose last MFMA has just been issued.
-  static constexpr int FETCH_T = MT >= 16 ? NTW - 1 : NTW - 2;
+  static constexpr int XA_SETS = MT >= 16 ? 1 : 2;
+  static constexpr int FETCH_T = XA_SETS == 1 ? NTW - 1 : NTW - 2;
 };
 
 template <int REGIME>
@@ -155,7 +156,7 @@ __global__ __launch_bounds__(256) void woq_gemm_w4_kernel(const FpArgs f, const 
   uint8_t zr[G4_NTW];
   G4Consts<REGIME> qc[G4_NTW];
   u4 bop[2];        // B operand in use / being dequantized
-  u4 xa[2][G4_MT];  // A fragments of the sub-step in use / of the next one
+  u4 xa[S::XA_SETS][G4_MT];  // A fragments of the sub-step in use (/ of the next one)
 
   // s_waitcnt immediates (vmcnt in bits 3:0 and 15:14; expcnt 6:4 and lgkmcnt 11:8 left at maximum)
   constexpr int kVmcnt0 = 0x0F70, kLgkmcnt0 = 0xC07F;
@@ -236,9 +237,9 @@ __global__ __launch_bounds__(256) void woq_gemm_w4_kernel(const FpArgs f, const 
         }
 #pragma unroll
         for (int mt = 0; mt < G4_MT; ++mt) {
-          acc[mt][t] = g4_mfma<REGIME>(xa[j & 1][mt], bop[cur], acc[mt][t]);
+          acc[mt][t] = g4_mfma<REGIME>(xa[(j & 1) % S::XA_SETS][mt], bop[cur], acc[mt][t]);
           if (fetch_t)
-            xa[(j & 1) ^ 1][mt] = j == 3 ? *(const u4*)(xsn + mt * 4096 + rd[0])
+            xa[((j & 1) ^ 1) % S::XA_SETS][mt] = j == 3 ? *(const u4*)(xsn + mt * 4096 + rd[0])
                                          : *(const u4*)(xs + mt * 4096 + rd[j + 1]);
         }
         if (j == 3) wr[t] = read_w((kt & 1) ^ 1, t);
@@ -363,15 +364,27 @@ int launch_gemm_w4(const FpArgs& f, int regime, hipStream_t st, int shape) {
   }
   // 128 rows x 448, 256 or 128 columns per workgroup: the widest shape does the most work per
   // activation fragment, the narrower ones make enough workgroups to fill the chip when M * N is
-  // small (e.g. N = 4096: 10 column blocks of 448 but 16 of 256).  A 256 x 256 shape (MT 16, NTW 4)
-  // would halve the dequantization work per MFMA, but its 256 accumulator registers leave the
-  // register allocator no spare tile and the generated loop copies accumulators through VGPRs and
-  // scratch; it measured slower and is not built.
+  // small (e.g. N = 4096: 10 column blocks of 448 but 16 of 256).
+  // 256 rows x 192 columns (MT 16, NTW 3: 192 accumulator registers) dequantizes half as much per
+  // MFMA but measured no faster per output (a workgroup takes 95-120 us for K = 4096 against 103 us
+  // for the 17 % larger 128 x 448 one); it is chosen only where it tiles the problem into whole
+  // generations of 256 workgroups and the others do not (N = 6144, M = 2048: 101 us against 138 us).
+  // A 256 x 256 shape would need all 256 accumulator registers; the register allocator then
+  // copies accumulators through VGPRs and scratch, it measured slower and is not built.
   using S7 = G4Shape<8, 7>;
   using S4 = G4Shape<8, 4>;
   using S2 = G4Shape<8, 2>;
+  using ST = G4Shape<16, 3>;
   const double c7 = shape_cost<S7>(f), c4 = shape_cost<S4>(f), c2 = shape_cost<S2>(f);
-  if (shape == 0) shape = (c7 <= c4 && c7 <= c2) ? 7 : (c4 <= c2 ? 4 : 2);
+  if (shape == 0) {
+    shape = (c7 <= c4 && c7 <= c2) ? 7 : (c4 <= c2 ? 4 : 2);
+    const int64_t wgs_t = ((f.NT * kTileN + ST::BN - 1) / ST::BN) * ((f.M + ST::BM - 1) / ST::BM);
+    const double ct = (double)(wgs_t / 256) * 7.4;
+    if (wgs_t % 256 == 0 && ct < c7 && ct < c4 && ct < c2) shape = 163;
+  }
+  if (shape == 163)
+    return regime == kRegimeF16 ? launch_shape<kRegimeF16, ST>(f, g_shift, st)
+                                : launch_shape<kRegimeBF16, ST>(f, g_shift, st);
   if (shape == 7)
     return regime == kRegimeF16 ? launch_shape<kRegimeF16, S7>(f, g_shift, st)
                                 : launch_shape<kRegimeBF16, S7>(f, g_shift, st);
