@@ -243,7 +243,7 @@ def main():
     import torch
 
     import ipex_amd  # noqa: F401
-    from ipex_amd import _lib, ops
+    from ipex_amd import _kernels, _lib, ops
     from ipex_amd.utils import synthetic
 
     assert torch.cuda.is_available(), "bench.py needs a GPU"
@@ -355,11 +355,29 @@ def main():
             _, ms = time_steps(torch, lib, [pp], steps_p, max(3, steps_p // 5), stream)
             us = ms * 1e3 / steps_p
             pre[name] = {"us_per_step": round(us, 2), "tflops": round(flops / (us * 1e-6) / 1e12, 1)}
+        # For scale: the vendor's dense bf16 GEMM (torch.matmul) on the same activations and the
+        # already dequantized weight.  It does no dequantization; its rate on random data is what
+        # this chip sustains for the shape (the clock drops under MFMA load with non-zero operands).
+        wd = _kernels.dequant_weight(keep[0].at_weight_, keep[0].weight_dtype_, N, K, keep[0].scales_list_[0],
+                                     keep[0].zeros_u8_, G, torch.bfloat16)
+        for _ in range(5):
+            torch.matmul(xp, wd.t())
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        e0.record()
+        for _ in range(steps_p):
+            torch.matmul(xp, wd.t())
+        e1.record()
+        torch.cuda.synchronize()
+        us_d = e0.elapsed_time(e1) * 1e3 / steps_p
+        del wd
         result["prefill_m2048"] = {
             "workload": f"INT4 g128 woq_linear prefill, M={Mp}, K={K}, N={N}",
             "flops_per_step": flops,
             "lowp_bf16": pre["bf16"],
             "lowp_int8_per_row": pre["int8"],
+            "dense_bf16_vendor_gemm_same_shape": {"us_per_step": round(us_d, 2),
+                                                  "tflops": round(flops / (us_d * 1e-6) / 1e12, 1)},
             "frac_of_bf16_mfma_peak": round(pre["bf16"]["tflops"] / MFMA_BF16_PEAK_TFLOPS, 4),
             "peak_tflops": MFMA_BF16_PEAK_TFLOPS,
         }
