@@ -1,1 +1,1 @@
-from . import quantization
+from . import modules, quantization

@@ -245,3 +245,95 @@ def test_fused_ops_through_torch_ops(cuda):
     assert torch.equal(torch.ops.torch_ipex.woq_linear_relu(x, h), torch.relu(base))
     got = torch.ops.torch_ipex.woq_linear_silu(x, h)
     assert torch.allclose(got.float(), torch.nn.functional.silu(base.float()), atol=2e-2, rtol=2e-2)
+
+
+# ---------------------------------------------------------------------------------------------
+# ipex.llm.modules linear fusions over WOQ linears
+# ---------------------------------------------------------------------------------------------
+def _woq_module(ipex, K, N, weight_dtype="INT4", group_size=128, lowp="BF16", bias=True, seed=0, device="cuda"):
+    q = ipex.quantization
+    torch.manual_seed(seed)
+    lin = torch.nn.Linear(K, N, bias=bias).to(torch.bfloat16)
+    qmap = q.get_weight_only_quant_qconfig_mapping(
+        weight_dtype=getattr(q.WoqWeightDtype, weight_dtype), lowp_mode=getattr(q.WoqLowpMode, lowp),
+        group_size=group_size,
+    )
+    model = torch.nn.Sequential(lin).eval().to(device)
+    return q.convert(q.prepare(model, qmap, inplace=True), inplace=True)[0]
+
+
+@pytest.mark.parametrize("M", [3, 40, 150])
+def test_llm_linear_fusion_modules_match_unfused_composition(cuda, M):
+    """Each fusion module against the same WOQ linear followed by the torch elementwise op
+    (the reference's fallback branch, fusions/linear_fusion.py:63-64 and siblings)."""
+    ipex = _ipex()
+    F = torch.nn.functional
+    mods = ipex.llm.modules
+    K, N = 512, 272
+    woq = _woq_module(ipex, K, N)
+    torch.manual_seed(M)
+    x = torch.randn(M, K).to(torch.bfloat16).to(cuda)
+    y = torch.randn(M, N).to(torch.bfloat16).to(cuda)
+    z = torch.randn(M, N).to(torch.bfloat16).to(cuda)
+    base = woq(x)
+
+    def close(a, b):
+        assert a.dtype == b.dtype and a.shape == b.shape
+        assert torch.allclose(a.float(), b.float(), atol=2e-2, rtol=2e-2), float((a.float() - b.float()).abs().max())
+
+    close(mods.LinearSilu(woq)(x), F.silu(base))
+    close(mods.LinearRelu(woq)(x), F.relu(base))
+    close(mods.LinearGelu(woq)(x), F.gelu(base))
+    close(mods.LinearNewGelu(woq)(x), F.gelu(base, approximate="tanh"))
+    close(mods.LinearMul(woq)(x, y), base * y)
+    close(mods.LinearAdd(woq)(x, y), base + y)
+    close(mods.LinearAddAdd(woq)(x, y, z), base + y + z)
+    close(mods.LinearSiluMul(woq)(x, y), F.silu(base) * y)
+    up = _woq_module(ipex, K, N, seed=1)
+    close(mods.Linear2SiluMul(woq, up)(x), F.silu(base) * up(x))
+    # a module that is not a WOQ linear takes the unfused path
+    plain = torch.nn.Linear(K, N).to(torch.bfloat16).to(cuda)
+    close(mods.LinearSilu(plain)(x), F.silu(plain(x)))
+    close(mods.Linear2SiluMul(plain, up)(x), F.silu(plain(x)) * up(x))
+
+
+@pytest.mark.parametrize("weight_dtype,group_size,lowp", [("INT4", 128, "BF16"), ("INT4", 32, "INT8"), ("INT8", -1, "BF16"), ("NF4", 64, "BF16")])
+@pytest.mark.parametrize("M", [1, 7, 70])
+def test_concat_linear_equals_the_separate_linears(cuda, weight_dtype, group_size, lowp, M):
+    ipex = _ipex()
+    K = 512
+    outs = (256, 64, 80)
+    lins = [_woq_module(ipex, K, n, weight_dtype, group_size, lowp, bias=(i != 1), seed=10 + i) for i, n in enumerate(outs)]
+    torch.manual_seed(M)
+    x = torch.randn(2, M, K).to(torch.bfloat16).to(cuda)
+    want = [lin(x) for lin in lins]
+    cat = ipex.llm.modules.ConcatLinear(lins)
+    assert cat.concat_linear is not None and cat.concat_linear.out_features == sum(outs)
+    assert not hasattr(cat, "linear_0")
+    got = cat(x)
+    assert len(got) == 3
+    for g, w in zip(got, want):
+        assert g.shape == w.shape
+        if lowp == "INT8":
+            # per-tensor activation statistics do not depend on N: same quantized activations, same sums
+            assert torch.allclose(g.float(), w.float(), atol=1e-2, rtol=1e-2)
+        else:
+            assert torch.equal(g, w)
+    # the merged context holds the concatenation of the stored codes and parameters
+    ctx = cat.concat_linear._op_context
+    assert torch.equal(ctx.to_public(ctx.get_weight()), torch.cat([l._op_context.to_public(l._op_context.get_weight()) for l in lins], 0))
+    assert torch.equal(ctx.get_scales(), torch.cat([l._op_context.get_scales() for l in lins], 0))
+
+
+def test_concat_linear_falls_back_when_the_linears_differ(cuda):
+    ipex = _ipex()
+    a = _woq_module(ipex, 256, 64, "INT4", 128)
+    b = _woq_module(ipex, 256, 32, "INT4", 64, seed=3)
+    cat = ipex.llm.modules.ConcatLinear([a, b])
+    assert cat.concat_linear is None
+    x = torch.randn(5, 256).to(torch.bfloat16).to(cuda)
+    ya, yb = cat(x)
+    assert torch.equal(ya, a(x)) and torch.equal(yb, b(x))
+    plain = torch.nn.Linear(256, 16).to(torch.bfloat16).to(cuda)
+    cat2 = ipex.llm.modules.ConcatLinear([a, plain])
+    assert cat2.concat_linear is None and len(cat2(x)) == 2
