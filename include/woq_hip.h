@@ -36,6 +36,10 @@
  *                               woq_shuffle_weight_back_by_group_idx, the channel shuffles of
  *                               GPTQ act-order (csrc/cpu/jit/cpu/kernels/LinearWoqPacked.cpp:407-421,
  *                               777-954)
+ *   woq_hip_moe_gather_rows, woq_hip_moe_scale_add_rows
+ *                            <- fuse_index_unsqueeze / fuse_index_mul_index_add, the token gather
+ *                               and weighted scatter around the expert linears of mixtral_moe_woq
+ *                               (csrc/cpu/aten/kernels/MoEKrnl.cpp:31-160, 254-284)
  */
 #ifndef WOQ_HIP_H_
 #define WOQ_HIP_H_
@@ -235,6 +239,19 @@ int woq_hip_shuffle_activations(const void* x, int x_dtype, int64_t M, int64_t K
                                 void* out, void* stream);
 int woq_hip_shuffle_int4_weight(const void* plain, int64_t N, int64_t K, const int32_t* src, void* out,
                                 void* stream);
+
+/* Mixture of experts over WOQ linears (csrc/cpu/aten/kernels/MoEKrnl.cpp:254-284): the rows of the
+ * tokens routed to one expert, and the weighted accumulation of the expert's output.
+ *   gather_rows:    out[i, :] = x[rows[i], :], x [T, H] and out [n, H] in x_dtype, rows int64 on the device.
+ *   scale_add_rows: out[top_x[i], :] += routing_weights[top_x[i], idx[i]] * expert_out[i, :] for i < n;
+ *                   out [T, H], expert_out [n, H], routing_weights [T, topk], all in `dtype`; bf16 and
+ *                   fp32 form product and sum in fp32 (one rounding), fp16 rounds the product first.
+ *                   The entries of top_x must be distinct (a token reaches an expert at most once). */
+int woq_hip_moe_gather_rows(const void* x, int x_dtype, int64_t T, int64_t H, const int64_t* rows, int64_t n,
+                            void* out, void* stream);
+int woq_hip_moe_scale_add_rows(void* out, int dtype, int64_t T, int64_t H, const void* expert_out,
+                               const void* routing_weights, int64_t topk, const int64_t* top_x, const int64_t* idx,
+                               int64_t n, void* stream);
 
 #ifdef __cplusplus
 }

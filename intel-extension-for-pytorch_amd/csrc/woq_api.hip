@@ -263,4 +263,26 @@ int woq_hip_shuffle_int4_weight(const void* plain, int64_t N, int64_t K, const i
   return launch_shuffle_int4_weight(plain, N, K, src, out, (hipStream_t)stream);
 }
 
+int woq_hip_moe_gather_rows(const void* x, int x_dtype, int64_t T, int64_t H, const int64_t* rows, int64_t n,
+                            void* out, void* stream) {
+  if (x_dtype < 0 || x_dtype > 2) return set_error("moe_gather_rows: bad x_dtype %d", x_dtype);
+  if (T < 0 || H < 0 || n < 0) return set_error("moe_gather_rows: negative size");
+  if (n > 0 && H > 0 && (!x || !rows || !out)) return set_error("moe_gather_rows: null pointer");
+  if (n > 0 && T == 0) return set_error("moe_gather_rows: rows requested from an empty tensor");
+  return launch_moe_gather_rows(x, x_dtype, H, rows, n, out, (hipStream_t)stream);
+}
+
+int woq_hip_moe_scale_add_rows(void* out, int dtype, int64_t T, int64_t H, const void* expert_out,
+                               const void* routing_weights, int64_t topk, const int64_t* top_x, const int64_t* idx,
+                               int64_t n, void* stream) {
+  if (dtype < 0 || dtype > 2) return set_error("moe_scale_add_rows: bad dtype %d", dtype);
+  if (T < 0 || H < 0 || n < 0 || topk <= 0) return set_error("moe_scale_add_rows: bad size");
+  if (n > 0 && H > 0 && (!out || !expert_out || !routing_weights || !top_x || !idx))
+    return set_error("moe_scale_add_rows: null pointer");
+  if (n > T) return set_error("moe_scale_add_rows: %lld rows for %lld tokens (a token may appear once)", (long long)n,
+                              (long long)T);
+  return launch_moe_scale_add_rows(out, dtype, H, expert_out, routing_weights, topk, top_x, idx, n,
+                                   (hipStream_t)stream);
+}
+
 }  // extern "C"

@@ -11,6 +11,12 @@
 #include "woq_common.h"
 #include "woq_internal.h"
 
+// The fp32 epilogue `C += (float(sum) * s_a) * s_w` keeps three separate roundings
+// (csrc/cpu/aten/utils/woq.h:2172-2186).  hipcc contracts a multiply feeding an add into one fused
+// multiply-add by default, also through the __fmul_rn / __fadd_rn helpers (header functions built
+// under the command line's mode), so contraction is switched off for the operators of this file.
+#pragma clang fp contract(off)
+
 namespace woq {
 
 __host__ __device__ inline bool quant_a_is_sym(int mode) { return mode >= WOQ_HIP_QUANT_A_PER_TENSOR_SYM; }
@@ -373,8 +379,8 @@ __global__ __launch_bounds__(1024) void woq_small_m_i8_kernel(const Int8KArgs p)
               for (int e = 0; e < 4; ++e) {
                 const int64_t n = nt * kTileN + 4 * (lane >> 4) + e;
                 const float sw = live ? a.scales[(nt * a.KG + g) * kTileN + 4 * (lane >> 4) + e] : 0.0f;
-                const float cterm = __fmul_rn(__fmul_rn((float)qc[mt][e], sa), sw);
-                acc[t][mt][e] = __fadd_rn(acc[t][mt][e], cterm);
+                const float cterm = ((float)qc[mt][e] * sa) * sw;
+                acc[t][mt][e] = acc[t][mt][e] + cterm;
                 if (a.debug_block_sums && live && m < a.M && n < a.N)
                   a.debug_block_sums[(m * a.N + n) * (p.Kpad / p.block_k) + kb] = qc[mt][e];
               }
@@ -626,8 +632,8 @@ __global__ __launch_bounds__(256) void woq_gemm_i8_kernel(const Int8KArgs p) {
 #pragma unroll
           for (int e = 0; e < 16; ++e) {
             const int qv = ASYM ? qc[i][j][e] - qcomp[j][e] * za_reg[i][e] : qc[i][j][e];
-            const float cterm = __fmul_rn(__fmul_rn((float)qv, sa_reg[i][e]), sw);
-            acc[i][j][e] = __fadd_rn(acc[i][j][e], cterm);
+            const float cterm = ((float)qv * sa_reg[i][e]) * sw;
+            acc[i][j][e] = acc[i][j][e] + cterm;
             if (DEBUG) {
               // the block sum as the reference defines it: unsigned activations times weights
               const int64_t m = mrow0 + i * 32 + 8 * (e >> 2) + (e & 3);

@@ -268,3 +268,49 @@ def shuffle_int4_weight(plain, N, K, src):
     with torch.cuda.device(plain.device):
         _lib.check(lib.woq_hip_shuffle_int4_weight(_ptr(plain), N, K, _ptr(src), _ptr(out), _stream()), "shuffle_int4_weight")
     return out
+
+
+def moe_gather_rows(x, rows):
+    """out[i, :] = x[rows[i], :]; x [T, H] on the GPU, rows int64 on the same device."""
+    lib = _lib.load()
+    _require_cuda(x, "hidden_states")
+    _require_cuda(rows, "top_x")
+    if x.dtype not in _ACT_CODE or x.dim() != 2:
+        raise RuntimeError(f"moe_gather_rows: expected a 2-D bf16 / fp16 / fp32 tensor, got {x.dtype} {tuple(x.shape)}")
+    x = x.contiguous()
+    rows = rows.to(torch.int64).contiguous()
+    out = torch.empty((rows.numel(), x.shape[1]), dtype=x.dtype, device=x.device)
+    with torch.cuda.device(x.device):
+        _lib.check(
+            lib.woq_hip_moe_gather_rows(_ptr(x), _ACT_CODE[x.dtype], x.shape[0], x.shape[1], _ptr(rows), rows.numel(),
+                                        _ptr(out), _stream()),
+            "moe_gather_rows",
+        )
+    return out
+
+
+def moe_scale_add_rows(output, expert_out, routing_weights, top_x, idx):
+    """output[top_x[i], :] += routing_weights[top_x[i], idx[i]] * expert_out[i, :], in place."""
+    lib = _lib.load()
+    for t, name in ((output, "output"), (expert_out, "expert output"), (routing_weights, "routing_weights"),
+                    (top_x, "top_x"), (idx, "idx")):
+        _require_cuda(t, name)
+    if output.dtype not in _ACT_CODE or expert_out.dtype != output.dtype or routing_weights.dtype != output.dtype:
+        raise RuntimeError("moe_scale_add_rows: output, expert output and routing_weights must share one float dtype")
+    if not output.is_contiguous() or output.dim() != 2:
+        raise RuntimeError("moe_scale_add_rows: output must be a contiguous [tokens, hidden] tensor")
+    n, H = top_x.numel(), output.shape[1]
+    expert_out = expert_out.reshape(-1, H).contiguous()
+    if expert_out.shape[0] != n or idx.numel() != n or routing_weights.dim() != 2 or routing_weights.shape[0] != output.shape[0]:
+        raise RuntimeError("moe_scale_add_rows: shape mismatch between top_x / idx / expert output / routing_weights")
+    routing_weights = routing_weights.contiguous()
+    top_x = top_x.to(torch.int64).contiguous()
+    idx = idx.to(torch.int64).contiguous()
+    with torch.cuda.device(output.device):
+        _lib.check(
+            lib.woq_hip_moe_scale_add_rows(_ptr(output), _ACT_CODE[output.dtype], output.shape[0], H, _ptr(expert_out),
+                                           _ptr(routing_weights), routing_weights.shape[1], _ptr(top_x), _ptr(idx), n,
+                                           _stream()),
+            "moe_scale_add_rows",
+        )
+    return output

@@ -35,6 +35,8 @@ EXPORTS = [
     "woq_hip_dequant_weight",
     "woq_hip_shuffle_activations",
     "woq_hip_shuffle_int4_weight",
+    "woq_hip_moe_gather_rows",
+    "woq_hip_moe_scale_add_rows",
 ]
 
 
@@ -122,6 +124,10 @@ def load():
         lib.woq_hip_shuffle_activations.argtypes = [vp, i32, i64, i64, vp, vp, vp]
         lib.woq_hip_shuffle_int4_weight.restype = i32
         lib.woq_hip_shuffle_int4_weight.argtypes = [vp, i64, i64, vp, vp, vp]
+        lib.woq_hip_moe_gather_rows.restype = i32
+        lib.woq_hip_moe_gather_rows.argtypes = [vp, i32, i64, i64, vp, i64, vp, vp]
+        lib.woq_hip_moe_scale_add_rows.restype = i32
+        lib.woq_hip_moe_scale_add_rows.argtypes = [vp, i32, i64, i64, vp, vp, i64, vp, vp, i64, vp]
         if lib.woq_hip_abi_version() != 1:
             raise RuntimeError("libwoq_hip.so has an unexpected ABI version")
         _lib = lib

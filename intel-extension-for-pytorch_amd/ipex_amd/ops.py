@@ -559,6 +559,67 @@ def woq_linear(
     )
 
 
+# ---- mixture of experts over WOQ linears ---------------------------------------------------------
+def _moe_expert(hidden_states, top_x, idx, gate, up, down, routing_weights, output):
+    """One expert: gather its tokens, down(up(x) * silu(gate(x))), weighted accumulation
+    (mixtral_moe_woq_kernl_impl, csrc/cpu/aten/kernels/MoEKrnl.cpp:254-284)."""
+    cur = _kernels.moe_gather_rows(hidden_states, top_x)
+    act = gate.run(cur, fusion=_lib.FUSE_SILU)
+    cur = down.run(up.run(cur, fusion=_lib.FUSE_MUL, others=(act,)))
+    return _kernels.moe_scale_add_rows(output, cur, routing_weights, top_x, idx)
+
+
+def _no_all_reduce(is_distributed, name):
+    if is_distributed:
+        raise RuntimeError(f"torch_ipex::{name}: is_distributed=True needs an all-reduce, which this one-GPU build does not have")
+
+
+def mixtral_moe_woq(hidden_states, top_x, idx, gate_wei, up_wei, down_wei, routing_weights, output, is_distributed):
+    """One expert of a Mixtral-style layer (csrc/cpu/aten/MoE.cpp:260-288): ``gate_wei`` / ``up_wei`` /
+    ``down_wei`` are context handles, ``top_x`` the tokens routed to the expert and ``idx`` their
+    slot in the top-k; accumulates into ``output`` and returns it."""
+    _require_gpu_input(hidden_states, "torch_ipex::mixtral_moe_woq")
+    _no_all_reduce(is_distributed, "mixtral_moe_woq")
+    if top_x.shape[0] == 0:
+        return output
+    dev = hidden_states.device
+    return _moe_expert(
+        hidden_states, top_x.to(dev), idx.to(dev), _context_from_handle(gate_wei), _context_from_handle(up_wei),
+        _context_from_handle(down_wei), routing_weights, output,
+    )
+
+
+def deepseek_moe_woq(hidden_states, topk_ids, gate_ctx, up_ctx, down_ctx, routing_weights, is_distributed):
+    """All experts of a layer (csrc/cpu/aten/MoE.cpp:290-328): ``topk_ids`` [tokens, top-k] names the
+    experts of every token, the three lists hold one WoqLinearOpContext per expert.  Experts are
+    visited in ascending order and, inside an expert, tokens in ascending order (get_expert_topx_idx,
+    MoE.cpp:64-81), which fixes the order of the additions into a token's row.
+    The routing table is read on the host (one synchronizing copy of [tokens, top-k] int64) to size
+    the per-expert launches."""
+    _require_gpu_input(hidden_states, "torch_ipex::deepseek_moe_woq")
+    _no_all_reduce(is_distributed, "deepseek_moe_woq")
+    num_experts = len(gate_ctx)
+    if len(up_ctx) != num_experts or len(down_ctx) != num_experts:
+        raise RuntimeError("torch_ipex::deepseek_moe_woq: gate / up / down lists differ in length")
+    output = torch.zeros_like(hidden_states)
+    ids = topk_ids.detach().to("cpu", torch.int64)
+    if ids.numel() == 0:
+        return output
+    if int(ids.min()) < 0 or int(ids.max()) >= num_experts:
+        raise RuntimeError(f"torch_ipex::deepseek_moe_woq: expert ids must lie in [0, {num_experts})")
+    topk = ids.shape[1]
+    order = torch.argsort(ids.reshape(-1), stable=True)  # by expert, then token, then slot
+    counts = torch.bincount(ids.reshape(-1), minlength=num_experts).tolist()
+    routed = torch.stack([order // topk, order % topk]).to(hidden_states.device)
+    start = 0
+    for e, n in enumerate(counts):
+        if n:
+            _moe_expert(hidden_states, routed[0, start:start + n], routed[1, start:start + n], gate_ctx[e], up_ctx[e],
+                        down_ctx[e], routing_weights, output)
+        start += n
+    return output
+
+
 _registered = False
 _libs = []
 
@@ -594,6 +655,13 @@ def register():
         "int group_size, int lowp_mode, int act_quant_mode, Tensor? compensation=None) -> Tensor"
     )
     tl.impl("woq_linear", woq_linear, key)
+    tl.define(
+        "mixtral_moe_woq(Tensor hidden_states, Tensor top_x, Tensor idx, Tensor gate_wei, Tensor up_wei, "
+        "Tensor down_wei, Tensor routing_weights, Tensor(a!) output, bool is_distributed) -> Tensor(a!)"
+    )
+    tl.impl("mixtral_moe_woq", mixtral_moe_woq, key)
+    # takes lists of context objects: attached like the prepack entry points below
+    setattr(torch.ops.torch_ipex, "deepseek_moe_woq", deepseek_moe_woq)
 
     pl = torch.library.Library("ipex_prepack", "FRAGMENT")
     _libs.append(pl)

@@ -19,6 +19,9 @@ It restates, in numpy, the arithmetic of intel/intel-extension-for-pytorch's WOQ
   dynamic_quantize_per_block         csrc/cpu/aten/utils/woq_dynamic_quant.h:1526-1750
   woq_linear_opt_int8                Dequantize<int8_t> + int8 BRGEMM + fp32 epilogue,
                                      woq.h:1664-1734, 2133-2199; driver woq.h:3298-3452
+  expert_token_lists                 get_expert_topx_idx, csrc/cpu/aten/MoE.cpp:64-81
+  moe_index_mul_index_add            fuse_index_mul_index_add, csrc/cpu/aten/kernels/MoEKrnl.cpp:31-121,
+                                     and the generic branch :277-280
   select_compute                     qlinear_woq_affine, kernels/WoqLinearKrnl.cpp:56-161
   int8_block_k                       get_block_k, csrc/cpu/aten/Linear.cpp:362-376
 
@@ -29,13 +32,18 @@ How each function is pinned (see tests/test_oracle.py):
   * GEMMs: exact rational / float64 brute force on tiny shapes;
   * dynamic quantization: properties the definition fixes (round-half-even at constructed ties,
     extreme element maps to +-127 / 0 / 255, |x - q*s| <= s/2) over all 65536 bf16 patterns;
-  * int8 block sums: exact integer arithmetic against a Python big-int loop.
+  * int8 block sums: exact integer arithmetic against a Python big-int loop;
+  * NF4 table: the published normal-quantile construction (scipy), codes by brute force;
+  * MoE token lists / weighted scatter: an independent formulation (nonzero per expert) and exact
+    rationals rounded once.
 PARITY UNPINNED (no fixture or invariant can fix them; they are below the stated tolerances):
   * the fp32 accumulation order inside libxsmm BRGEMM / oneDNN (third_party/libxsmm, an
     un-vendored submodule whose pinned commit is not recoverable from the mount) -- the
     oracle accumulates in float64 instead;
   * whether the compiler contracted `C += (qC * s_a) * s_w` (woq.h:2172-2186) into an FMA --
     the oracle uses separate roundings;
+  * whether the CPU compiler contracted `out + cs * rw` (MoEKrnl.cpp:107-108) into an FMA -- the
+    oracle multiplies and adds separately;
   * the k order and chain structure of the fp16 micro-kernel are restated from the source
     text (woq.h:919-940) and could only be confirmed by running an AVX512-FP16 build.
 """
@@ -394,3 +402,35 @@ def woq_linear(x, act_dtype, qw, N, K, scales, zps, bias, weight_dtype, group_si
         r = woq_linear_opt_int8(x, act_dtype, qw, N, K, scales, zps, bias, weight_dtype, group_size, act_quant_mode)
         return r["acc"], r["y"]
     raise NotImplementedError(cd)
+
+
+# ---------------------------------------------------------------------------------------------
+# mixture of experts around the WOQ linears
+# ---------------------------------------------------------------------------------------------
+def expert_token_lists(topk_ids, num_experts):
+    """Per expert: (tokens routed to it, their slot in the top-k), tokens ascending, slots ascending
+    inside a token -- the order get_expert_topx_idx builds by walking topk_ids row by row."""
+    ids = np.asarray(topk_ids)
+    top_x = [[] for _ in range(num_experts)]
+    idx = [[] for _ in range(num_experts)]
+    for i in range(ids.shape[0]):
+        for j in range(ids.shape[1]):
+            top_x[int(ids[i, j])].append(i)
+            idx[int(ids[i, j])].append(j)
+    return [np.asarray(t, dtype=np.int64) for t in top_x], [np.asarray(t, dtype=np.int64) for t in idx]
+
+
+def moe_index_mul_index_add(output, cur, routing_weights, top_x, idx, dtype):
+    """output[top_x[i], :] += routing_weights[top_x[i], idx[i]] * cur[i, :], sequentially in i.
+    All arrays float32 holding `dtype` values.  bf16 / fp32: product and sum in fp32, one rounding
+    to dtype; fp16: the product is rounded to fp16 before the add."""
+    out = np.array(output, dtype=np.float32, copy=True)
+    cur = np.asarray(cur, dtype=np.float32)
+    rw = np.asarray(routing_weights, dtype=np.float32)
+    for i in range(len(top_x)):
+        t = int(top_x[i])
+        p = (cur[i] * rw[t, int(idx[i])]).astype(np.float32)
+        if dtype == "fp16":
+            p = f16_round(p)
+        out[t] = _round_to((out[t] + p).astype(np.float32), dtype)
+    return out

@@ -337,3 +337,107 @@ def test_concat_linear_falls_back_when_the_linears_differ(cuda):
     plain = torch.nn.Linear(256, 16).to(torch.bfloat16).to(cuda)
     cat2 = ipex.llm.modules.ConcatLinear([a, plain])
     assert cat2.concat_linear is None and len(cat2(x)) == 2
+
+
+# ---------------------------------------------------------------------------------------------
+# mixture of experts over WOQ linears (torch_ipex::mixtral_moe_woq / deepseek_moe_woq)
+# ---------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("H", [128, 100])  # 16-byte chunks / element by element
+def test_moe_gather_and_weighted_scatter_bit_exact(cuda, dtype, H):
+    from ipex_amd import _kernels
+    from oracle import woq_oracle as O
+
+    name = {torch.bfloat16: "bf16", torch.float16: "fp16", torch.float32: "fp32"}[dtype]
+    g = torch.Generator().manual_seed(H)
+    T, topk = 37, 4
+    hidden = torch.randn(T, H, generator=g).to(dtype)
+    rw = torch.rand(T, topk, generator=g).to(dtype)
+    top_x = torch.randperm(T, generator=g)[:21].sort()[0]
+    idx = torch.randint(0, topk, (21,), generator=g)
+    cur = _kernels.moe_gather_rows(hidden.to(cuda), top_x.to(cuda))
+    assert torch.equal(cur.cpu(), hidden[top_x])
+    out0 = torch.randn(T, H, generator=g).to(dtype)
+    expert_out = torch.randn(21, H, generator=g).to(dtype)
+    got = _kernels.moe_scale_add_rows(out0.to(cuda).clone(), expert_out.to(cuda), rw.to(cuda), top_x.to(cuda), idx.to(cuda))
+    want = O.moe_index_mul_index_add(out0.float().numpy(), expert_out.float().numpy(), rw.float().numpy(),
+                                     top_x.numpy(), idx.numpy(), name)
+    assert np.array_equal(got.float().cpu().numpy(), want)
+
+
+def _moe_layer(ipex, E, H, I, seed):
+    gate = [_woq_module(ipex, H, I, "INT4", 64, "BF16", bias=False, seed=seed + 3 * e) for e in range(E)]
+    up = [_woq_module(ipex, H, I, "INT4", 64, "BF16", bias=False, seed=seed + 3 * e + 1) for e in range(E)]
+    down = [_woq_module(ipex, I, H, "INT4", 64, "BF16", bias=False, seed=seed + 3 * e + 2) for e in range(E)]
+    return gate, up, down
+
+
+@pytest.mark.parametrize("T,topk", [(12, 2), (1, 2), (70, 3)])
+def test_deepseek_moe_woq_matches_per_expert_composition(cuda, T, topk):
+    from oracle import woq_oracle as O
+
+    ipex = _ipex()
+    E, H, I = 5, 256, 384
+    gate, up, down = _moe_layer(ipex, E, H, I, 100)
+    g = torch.Generator().manual_seed(T)
+    hidden = torch.randn(T, H, generator=g).to(torch.bfloat16)
+    ids = torch.stack([torch.randperm(E, generator=g)[:topk] for _ in range(T)])
+    rw = torch.softmax(torch.randn(T, topk, generator=g), -1).to(torch.bfloat16)
+    ctxs = [[m._op_context for m in ms] for ms in (gate, up, down)]
+    got = torch.ops.torch_ipex.deepseek_moe_woq(hidden.to(cuda), ids.to(cuda), ctxs[0], ctxs[1], ctxs[2], rw.to(cuda), False)
+    assert got.shape == hidden.shape and got.dtype == torch.bfloat16
+
+    # the same experts one by one through the fusion modules, scatter by the oracle on the host
+    top_x, idx = O.expert_token_lists(ids.numpy(), E)
+    want = np.zeros((T, H), dtype=np.float32)
+    dense = torch.zeros(T, H)
+    mods = ipex.llm.modules
+    for e in range(E):
+        if len(top_x[e]) == 0:
+            continue
+        cur = hidden[torch.from_numpy(top_x[e])].to(cuda)
+        y = down[e](mods.Linear2SiluMul(gate[e], up[e])(cur))
+        want = O.moe_index_mul_index_add(want, y.float().cpu().numpy(), rw.float().numpy(), top_x[e], idx[e], "bf16")
+        # float reference on the dequantized weights
+        w = [c.get_scales() for c in (ctxs[0][e], ctxs[1][e], ctxs[2][e])]  # noqa: F841 (kept alive)
+        deq = lambda m: ipex.quantization.dequantize_per_block(
+            m._op_context.to_public(m._op_context.get_weight()).cpu(), m._op_context.get_scales().cpu(),
+            m._op_context.get_zero_points().cpu(), ipex.quantization.WoqWeightDtype.INT4, 64,
+            [m.out_features, m.in_features])
+        xc = cur.float().cpu()
+        ye = (torch.nn.functional.silu(xc @ deq(gate[e]).t()) * (xc @ deq(up[e]).t())) @ deq(down[e]).t()
+        sel = torch.from_numpy(top_x[e])
+        dense[sel] += ye * rw.float()[sel, torch.from_numpy(idx[e])].unsqueeze(-1)
+    assert np.array_equal(got.float().cpu().numpy(), want)
+    err = (got.float().cpu() - dense).abs().max() / dense.abs().max()
+    assert float(err) < 3e-2, float(err)
+
+
+def test_mixtral_moe_woq_single_expert_and_errors(cuda):
+    ipex = _ipex()
+    H, I, T = 128, 256, 6
+    gate, up, down = _moe_layer(ipex, 1, H, I, 200)
+    g = torch.Generator().manual_seed(5)
+    hidden = torch.randn(T, H, generator=g).to(torch.bfloat16).to(cuda)
+    rw = torch.rand(T, 2, generator=g).to(torch.bfloat16).to(cuda)
+    top_x = torch.tensor([0, 2, 5])
+    idx = torch.tensor([1, 0, 1])
+    out = torch.zeros_like(hidden)
+    handles = [m[0]._op_context.get_data_handle() for m in (gate, up, down)]
+    ret = torch.ops.torch_ipex.mixtral_moe_woq(hidden, top_x.to(cuda), idx.to(cuda), *handles, rw, out, False)
+    assert ret.data_ptr() == out.data_ptr()
+    y = down[0](ipex.llm.modules.Linear2SiluMul(gate[0], up[0])(hidden[top_x.to(cuda)]))
+    want = torch.zeros_like(hidden)
+    want[top_x.to(cuda)] = (y.float() * rw[top_x.to(cuda), idx.to(cuda)].float().unsqueeze(-1)).to(torch.bfloat16)
+    assert torch.equal(out, want)
+    assert bool((out[[1, 3, 4]] == 0).all())
+    # no tokens: output untouched
+    before = out.clone()
+    empty = torch.empty(0, dtype=torch.int64, device=cuda)
+    torch.ops.torch_ipex.mixtral_moe_woq(hidden, empty, empty, *handles, rw, out, False)
+    assert torch.equal(out, before)
+    with pytest.raises(RuntimeError, match="all-reduce"):
+        torch.ops.torch_ipex.mixtral_moe_woq(hidden, top_x.to(cuda), idx.to(cuda), *handles, rw, out, True)
+    ctxs = [[m[0]._op_context] for m in (gate, up, down)]
+    with pytest.raises(RuntimeError, match="expert ids"):
+        torch.ops.torch_ipex.deepseek_moe_woq(hidden, torch.full((T, 1), 3), ctxs[0], ctxs[1], ctxs[2], rw, False)

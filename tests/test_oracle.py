@@ -127,6 +127,37 @@ def test_nf4_quantize_dequantize_roundtrip_error_bound():
     assert np.allclose(np.abs(w).reshape(8, 4, 32).max(axis=-1), amax, rtol=0, atol=1e-7)
 
 
+def test_moe_token_lists_and_weighted_scatter():
+    rng = np.random.default_rng(11)
+    T, topk, E, H = 9, 3, 5, 6
+    ids = np.stack([rng.permutation(E)[:topk] for _ in range(T)])
+    top_x, idx = O.expert_token_lists(ids, E)
+    for e in range(E):  # independent formulation: row-major nonzero of the mask
+        r, c = np.nonzero(ids == e)
+        assert np.array_equal(top_x[e], r) and np.array_equal(idx[e], c)
+    assert sum(len(t) for t in top_x) == T * topk
+    # weighted scatter: exact rationals, rounded once (bf16 / fp32) or twice (fp16)
+    for dtype in ("bf16", "fp16", "fp32"):
+        rt = lambda a: O._round_to(np.asarray(a, dtype=np.float32), dtype)
+        out0, rw = rt(rng.standard_normal((T, H))), rt(rng.uniform(0, 1, (T, topk)))
+        e = int(np.argmax([len(t) for t in top_x]))
+        cur = rt(rng.standard_normal((len(top_x[e]), H)))
+        got = O.moe_index_mul_index_add(out0, cur, rw, top_x[e], idx[e], dtype)
+        want = out0.copy()
+        for i, (t, j) in enumerate(zip(top_x[e], idx[e])):
+            for h in range(H):
+                prod = fractions.Fraction(float(cur[i, h])) * fractions.Fraction(float(rw[t, j]))
+                if dtype == "fp16":
+                    prod = fractions.Fraction(float(np.float16(np.float32(float(prod)))))
+                    # (the fp32 product of two fp16 values is exact, so this is the fp16 rounding of it)
+                # fp32 rounding of the product, then of the sum, then the dtype
+                p32 = np.float32(float(prod))
+                want[t, h] = rt(np.float32(p32 + want[t, h]))
+        assert np.array_equal(got, want), dtype
+        untouched = np.setdiff1d(np.arange(T), top_x[e])
+        assert np.array_equal(got[untouched], out0[untouched])
+
+
 def test_dequantize_group_indexing():
     # group g of row n must use scales[n, g]: make each group's scale identify it
     N, K, G = 3, 96, 32
