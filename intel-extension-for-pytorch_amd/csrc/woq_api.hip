@@ -226,7 +226,16 @@ int woq_hip_linear(const woq_hip_linear_params* p) {
                        "power-of-two or per-channel group size and activations in the compute dtype");
     return launch_decode_dq(f, wbits, regime, st, kernel == 10 ? 4 : kernel - 7);
   }
-  if (kernel == 0) kernel = p->M <= 64 ? 1 : (gemm_w4_applies(f, wbits, regime) ? 3 : 2);
+  if (kernel == 0) {
+    // 33..64 rows: the streaming kernel re-reads the activations once per workgroup, which costs
+    // more than the prefill kernel's half-empty 128-row tiles once N is large (M = 64, 4096 -> 14336:
+    // 57 us against 37 us; 4096 -> 4096: 23 us against 35 us)
+    const bool w4 = gemm_w4_applies(f, wbits, regime);
+    if (p->M <= 64)
+      kernel = (p->M > 32 && w4 && p->N >= 8192) ? 3 : 1;
+    else
+      kernel = w4 ? 3 : 2;
+  }
   if (kernel == 1 && p->M > 64) return set_error("woq_linear: the small-M kernel takes M <= 64");
   const int w4_shape = kernel == 4 ? 7 : kernel == 5 ? 4 : kernel == 6 ? 2 : kernel == 11 ? 163 : 0;
   if ((kernel >= 4 && kernel <= 6) || kernel == 11) kernel = 3;
