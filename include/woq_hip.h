@@ -51,8 +51,8 @@ extern "C" {
 #endif
 
 /* weight dtype, csrc/cpu/aten/utils/woq_defines.h:6-9.  NF4: 4-bit codes into the NormalFloat4 table
- * (csrc/cpu/aten/utils/woq_utils.h:34-51), packed like INT4, symmetric only, floating-point
- * lowp modes only (woq_hip_linear returns an error for NF4 with WOQ_HIP_LOWP_INT8). */
+ * (csrc/cpu/aten/utils/woq_utils.h:34-51), packed like INT4, symmetric only; under
+ * WOQ_HIP_LOWP_INT8 the codes become the int8 table of csrc/cpu/aten/utils/woq.h:628-669. */
 #define WOQ_HIP_DTYPE_INT8 1
 #define WOQ_HIP_DTYPE_INT4 2
 #define WOQ_HIP_DTYPE_NF4 3

@@ -160,8 +160,6 @@ int woq_hip_linear(const woq_hip_linear_params* p) {
 
   const bool nf4 = p->weight_dtype == WOQ_HIP_DTYPE_NF4;
   if (nf4 && p->zeros_u8) return set_error("woq_linear: symmetric quantization is required for NF4 weights");
-  if (nf4 && p->lowp_mode == WOQ_HIP_LOWP_INT8)
-    return set_error("woq_linear: NF4 weights run in the floating-point regimes only (lowp_mode NONE, FP16 or BF16)");
   int lowp = p->lowp_mode;
   if (lowp == WOQ_HIP_LOWP_INT8) {
     const int64_t bk = woq_hip_int8_block_k(p->group_size, p->K);
@@ -185,6 +183,7 @@ int woq_hip_linear(const woq_hip_linear_params* p) {
       a.fusion = p->fusion; a.other0 = p->others[0]; a.other1 = p->others[1]; a.out = p->out;
       a.out_dtype = p->out_dtype; a.workspace = p->workspace; a.workspace_bytes = p->workspace_bytes;
       a.debug_block_sums = p->debug_block_sums;
+      a.nf4 = nf4 ? 1 : 0;
       return launch_int8_linear(a, st);
     }
   }

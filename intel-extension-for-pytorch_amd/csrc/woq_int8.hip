@@ -245,12 +245,30 @@ __device__ __forceinline__ uint32_t sub_bytes(uint32_t b, uint32_t z4) {
   return ((b | 0x80808080u) - z4) ^ 0x80808080u;
 }
 
+// NF4 under lowp_mode INT8: the code's table value times 127, rounded, as int8 (load_nf4_as_int8,
+// csrc/cpu/aten/utils/woq.h:628-669).  Four codes in the bytes of b: two byte permutes over the halves
+// of the table (codes 0..7 and 8..15), merged on bit 3 of each code.
+__device__ __forceinline__ uint32_t nf4_codes_to_i8(uint32_t b) {
+  // -127 -88 -67 -50 | -36 -23 -12 0 | 10 20 31 43 | 56 71 92 127, least significant byte first
+  const uint32_t t0 = 0xCEBDA881u, t1 = 0x00F4E9DCu, t2 = 0x2B1F140Au, t3 = 0x7F5C4738u;
+  const uint32_t sel = b & 0x07070707u;
+  const uint32_t lo = __builtin_amdgcn_perm(t1, t0, sel);
+  const uint32_t hi = __builtin_amdgcn_perm(t3, t2, sel);
+  const uint32_t m = ((b >> 3) & 0x01010101u) * 0xFFu;
+  return (hi & m) | (lo & ~m);
+}
+
 // 16 K elements of one lane for one 16x16x64 MFMA, from two packed dwords (4-bit) or four
 // dwords (8-bit); 4-bit yields the permuted order [e0 e4 e1 e5][e2 e6 e3 e7].
 template <int WBITS>
-__device__ __forceinline__ i4 decode16_i8(const uint32_t* d, uint32_t z4) {
+__device__ __forceinline__ i4 decode16_i8(const uint32_t* d, uint32_t z4, bool nf4 = false) {
   i4 r;
-  if (WBITS == 4) {
+  if (WBITS == 4 && nf4) {
+    r[0] = (int)nf4_codes_to_i8(d[0] & 0x0F0F0F0Fu);
+    r[1] = (int)nf4_codes_to_i8((d[0] >> 4) & 0x0F0F0F0Fu);
+    r[2] = (int)nf4_codes_to_i8(d[1] & 0x0F0F0F0Fu);
+    r[3] = (int)nf4_codes_to_i8((d[1] >> 4) & 0x0F0F0F0Fu);
+  } else if (WBITS == 4) {
     r[0] = (int)sub_bytes(d[0] & 0x0F0F0F0Fu, z4);
     r[1] = (int)sub_bytes((d[0] >> 4) & 0x0F0F0F0Fu, z4);
     r[2] = (int)sub_bytes(d[1] & 0x0F0F0F0Fu, z4);
@@ -324,7 +342,8 @@ __global__ __launch_bounds__(1024) void woq_small_m_i8_kernel(const Int8KArgs p)
           if (g >= a.KG) g = a.KG - 1;
           zb = a.zeros[(ntc * a.KG + g) * kTileN + r];
         }
-        const uint32_t dead = WBITS == 4 ? 0u : 0x80808080u;
+        // a tile past the end contributes zeros: q = z = 0, offset-binary 128, or NF4 code 7
+        const uint32_t dead = WBITS == 4 ? (a.nf4 ? 0x77777777u : 0u) : 0x80808080u;
         wreg[t][i] = live ? wv : u4{dead, dead, dead, dead};
         zreg[t][i] = live ? zb : (uint8_t)(WBITS == 4 ? 0 : 128);
       }
@@ -358,7 +377,7 @@ __global__ __launch_bounds__(1024) void woq_small_m_i8_kernel(const Int8KArgs p)
 #pragma unroll
         for (int j = 0; j < STEPS; ++j) {
           const uint32_t* d = (const uint32_t*)&wreg[t][i] + (WBITS == 4 ? 2 * j : 0);
-          const i4 aop = decode16_i8<WBITS>(d, z4);
+          const i4 aop = decode16_i8<WBITS>(d, z4, a.nf4 != 0);
 #pragma unroll
           for (int mt = 0; mt < MT; ++mt)
             qc[mt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(aop, xb[i][j][mt], qc[mt], 0, 0, 0);
@@ -378,7 +397,8 @@ __global__ __launch_bounds__(1024) void woq_small_m_i8_kernel(const Int8KArgs p)
 #pragma unroll
               for (int e = 0; e < 4; ++e) {
                 const int64_t n = nt * kTileN + 4 * (lane >> 4) + e;
-                const float sw = live ? a.scales[(nt * a.KG + g) * kTileN + 4 * (lane >> 4) + e] : 0.0f;
+                float sw = live ? a.scales[(nt * a.KG + g) * kTileN + 4 * (lane >> 4) + e] : 0.0f;
+                if (a.nf4) sw = sw * (1.0f / 127.0f);
                 const float cterm = ((float)qc[mt][e] * sa) * sw;
                 acc[t][mt][e] = acc[t][mt][e] + cterm;
                 if (a.debug_block_sums && live && m < a.M && n < a.N)
@@ -502,7 +522,8 @@ __global__ __launch_bounds__(256) void woq_gemm_i8_kernel(const Int8KArgs p) {
       wrow[q] = ntl * 16 + r;
       wcol[q] = WBITS == 4 ? c * 32 : kt_off * 64 + c * 16;
       const int64_t nt = nt0 + ntl, kt = k0 / TK + kt_off;
-      u4 wv = WBITS == 4 ? u4{0u, 0u, 0u, 0u} : u4{0x80808080u, 0x80808080u, 0x80808080u, 0x80808080u};
+      const uint32_t dead = WBITS == 4 ? (a.nf4 ? 0x77777777u : 0u) : 0x80808080u;
+      u4 wv = u4{dead, dead, dead, dead};
       uint32_t z = WBITS == 4 ? 8u : 128u;
       if (nt < a.NT && kt < a.KT) {
         wv = *(const u4*)(a.qweight + ((nt * a.KT + kt) * 64 + li) * 16);
@@ -516,8 +537,8 @@ __global__ __launch_bounds__(256) void woq_gemm_i8_kernel(const Int8KArgs p) {
       }
       const uint32_t z4 = z * 0x01010101u;
       if (WBITS == 4) {
-        const i4 lo = decode16_i8<4>((const uint32_t*)&wv, z4);
-        const i4 hi = decode16_i8<4>((const uint32_t*)&wv + 2, z4);
+        const i4 lo = decode16_i8<4>((const uint32_t*)&wv, z4, a.nf4 != 0);
+        const i4 hi = decode16_i8<4>((const uint32_t*)&wv + 2, z4, a.nf4 != 0);
         wo[q][0] = bitcast<u4>(lo);
         wo[q][WBITS == 4 ? 1 : 0] = bitcast<u4>(hi);
       } else {
@@ -626,7 +647,8 @@ __global__ __launch_bounds__(256) void woq_gemm_i8_kernel(const Int8KArgs p) {
       for (int j = 0; j < 2; ++j) {
         const int n = ncol0 + j * 32;  // < NT * 16 by construction of the grid? clamp below
         const int nc = n < (int)a.NT * kTileN ? n : (int)a.NT * kTileN - 1;
-        const float sw = a.scales[((nc >> 4) * (int)a.KG + g) * kTileN + (nc & 15)];
+        float sw = a.scales[((nc >> 4) * (int)a.KG + g) * kTileN + (nc & 15)];
+        if (a.nf4) sw = sw * (1.0f / 127.0f);
 #pragma unroll
         for (int i = 0; i < 2; ++i) {
 #pragma unroll

@@ -107,6 +107,7 @@ struct Int8Args {
   void* workspace;
   int64_t workspace_bytes;
   int32_t* debug_block_sums;
+  int nf4;  // 4-bit codes index the NF4 int8 table; the weight scale is multiplied by fp32(1 / 127)
 };
 
 int launch_dynamic_quant(const void* x, int x_dtype, int64_t M, int64_t K, int64_t ldq, int64_t qbk,

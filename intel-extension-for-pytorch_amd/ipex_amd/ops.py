@@ -90,8 +90,6 @@ class WoqLinearOpContext:
             raise RuntimeError(f"WOQ linear: unsupported weight dtype {weight_dtype}")
         if weight_dtype == _lib.DTYPE_NF4 and zero_points is not None:
             raise RuntimeError("WOQ: symmetric quantization is required for NF4 or INT8 with lowp-mode INT8")
-        if weight_dtype == _lib.DTYPE_NF4 and int(lowp_mode) == _lib.LOWP_INT8:
-            raise RuntimeError("WOQ linear: NF4 weights run with lowp_mode NONE, FP16 or BF16 (INT8 is not built)")
         N, K = int(weight_shape[0]), int(weight_shape[1])
         weight = _to_gpu(weight)
         dev = weight.device

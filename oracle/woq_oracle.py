@@ -305,9 +305,18 @@ def dynamic_quantize_per_block(x, quant_block_k, mode):
     return q, scales, (None if sym else zps)
 
 
+# NF4 codes as int8 for the lowp-INT8 kernels: round(127 * table) (the lookup table of
+# load_nf4_as_int8, csrc/cpu/aten/utils/woq.h:628-669); the weight scale is multiplied by
+# fp32(1 / 127) to make up for it (woq.h:1006-1009, 2174-2176).
+NF4_TO_INT8_TABLE = np.array([-127, -88, -67, -50, -36, -23, -12, 0, 10, 20, 31, 43, 56, 71, 92, 127], dtype=np.int64)
+
+
 def _int8_weights(qw, N, K, zps, weight_dtype, group_size):
     """B[n, k] = q - z as integers (the int8 operand of the lowp-INT8 kernels, woq.h:1701-1704,
-    614-625)."""
+    614-625); NF4: the int8 table value of the code."""
+    if weight_dtype == WOQ_DTYPE_NF4:
+        assert zps is None, "NF4 is symmetric"
+        return NF4_TO_INT8_TABLE[unpack_int4(qw)[:, :K]]
     if weight_dtype == WOQ_DTYPE_INT4:
         q = unpack_int4(qw)[:, :K].astype(np.int64)
         if zps is None:
@@ -327,16 +336,7 @@ def int8_weight_block_sums(qw, N, K, zps, weight_dtype, group_size, block_k):
 
 def int8_block_sums(xq, qw, N, K, zps, weight_dtype, group_size, block_k):
     """Exact int32 sums qC[m, n, kb] = sum_{k in block kb} xq[m, k] * (q[n, k] - z[n, g(k)])."""
-    if weight_dtype == WOQ_DTYPE_INT4:
-        q = unpack_int4(qw)[:, :K].astype(np.int64)
-        if zps is None:
-            B = q - 8
-        else:
-            z = np.asarray(zps).reshape(N, -1).astype(np.int64)
-            g = (np.arange(K) // group_size) if group_size > 0 else np.zeros(K, dtype=np.int64)
-            B = q - z[:, g]
-    else:
-        B = np.asarray(qw, dtype=np.int8).astype(np.int64)
+    B = _int8_weights(qw, N, K, zps, weight_dtype, group_size)
     A = np.asarray(xq).astype(np.int64)
     KB = K // block_k
     out = np.empty((A.shape[0], N, KB), dtype=np.int64)
@@ -360,6 +360,8 @@ def woq_linear_opt_int8(x, act_dtype, qw, N, K, scales, zps, bias, weight_dtype,
     xq, sa, za = dynamic_quantize_per_block(x, qbk, act_quant_mode)
     sums = int8_block_sums(xq, qw, N, K, zps, weight_dtype, group_size, bk)
     s = np.asarray(scales, dtype=np.float32).reshape(N, -1)
+    if weight_dtype == WOQ_DTYPE_NF4:
+        s = (s * (np.float32(1.0) / np.float32(127.0))).astype(np.float32)
     per_m = act_quant_mode in (2, 3, 6, 7)
     per_k = act_quant_mode in (1, 3, 5, 7)
     Kc = (K + qbk - 1) // qbk

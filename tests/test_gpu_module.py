@@ -23,7 +23,7 @@ def _ipex():
 @pytest.mark.parametrize("weight_dtype,group_size,lowp", [
     ("INT8", -1, "NONE"), ("INT8", -1, "BF16"), ("INT4", -1, "BF16"), ("INT4", 128, "BF16"), ("INT4", 32, "BF16"),
     ("INT4", 64, "FP16"), ("INT4", 128, "INT8"), ("INT8", -1, "INT8"),
-    ("NF4", 64, "BF16"), ("NF4", -1, "NONE"), ("NF4", 32, "FP16"),
+    ("NF4", 64, "BF16"), ("NF4", -1, "NONE"), ("NF4", 32, "FP16"), ("NF4", 128, "INT8"),
 ])
 @pytest.mark.parametrize("M", [1, 4, 33, 196])
 def test_prepare_convert_matches_dequantized_matmul(cuda, weight_dtype, group_size, lowp, M):

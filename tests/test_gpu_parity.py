@@ -433,8 +433,6 @@ def test_nf4_dequant_weight_bit_exact_and_pack_roundtrip(cuda, G):
 def test_nf4_rejections(cuda):
     syn = _synthetic()
     case = syn.make_nf4_case(25, 4, 256, 32, 64)
-    with pytest.raises(RuntimeError, match="NF4"):
-        make_context(case, O.LOWP_INT8, 6)
     bad = dict(case, zeros=torch.zeros(32, 4))
     with pytest.raises(RuntimeError, match="symmetric"):
         make_context(bad, O.LOWP_BF16)
@@ -443,6 +441,14 @@ def test_nf4_rejections(cuda):
         ctx.run(case["x"].cuda(), force_kernel=3)
     with pytest.raises(RuntimeError, match="NF4"):
         ctx.run(case["x"].cuda(), force_kernel=10)
+
+
+@pytest.mark.parametrize("mode", [6, 7, 2])
+@pytest.mark.parametrize("M,K,N,G", [(1, 1024, 272, 128), (40, 512, 144, 32), (150, 1024, 272, 128), (20, 768, 80, -1)])
+def test_nf4_lowp_int8(cuda, mode, M, K, N, G):
+    """NF4 codes as int8 table values, scale / 127: int32 block sums bit-exact, fp32 epilogue to the bar."""
+    case = _synthetic().make_nf4_case(28, M, K, N, G, bias=(M == 40))
+    _check_int8(case, mode, label=f"nf4 int8 lowp mode={mode} M={M} K={K} N={N} G={G}")
 
 
 def test_nf4_weight_cache_for_large_batch_matches_oracle(cuda):

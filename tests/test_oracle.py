@@ -109,6 +109,39 @@ def test_nf4_linear_paths_against_exact_rational_matmul():
     assert np.all(O.woq_linear_opt_fp16(x, qw, N, K, s0, None, None, O.WOQ_DTYPE_NF4, G)[:, 2] == 0)
 
 
+def test_nf4_int8_table_and_lowp_int8_linear():
+    # the int8 table is the float table times 127, rounded (closed form), and antisymmetric at the ends
+    assert np.array_equal(O.NF4_TO_INT8_TABLE, np.rint(O.NF4_DEQUANT_TABLE.astype(np.float64) * 127).astype(np.int64))
+    assert O.NF4_TO_INT8_TABLE[7] == 0 and O.NF4_TO_INT8_TABLE[0] == -127 and O.NF4_TO_INT8_TABLE[15] == 127
+    rng = np.random.default_rng(8)
+    M, K, N, G = 3, 256, 5, 128
+    codes = rng.integers(0, 16, (N, K)).astype(np.uint8)
+    qw = O.pack_int4(codes)
+    scales = rng.uniform(0.02, 0.08, (N, K // G)).astype(np.float32)
+    x = O.bf16_round(rng.standard_normal((M, K)).astype(np.float32))
+    r = O.woq_linear_opt_int8(x, "bf16", qw, N, K, scales, None, None, O.WOQ_DTYPE_NF4, G, 6)
+    # integer block sums: Python integers over the table values
+    B = [[int(O.NF4_TO_INT8_TABLE[c]) for c in row] for row in codes]
+    for m in range(M):
+        for n in range(N):
+            for kb in range(K // 128):
+                want = sum(int(r["xq"][m, k]) * B[n][k] for k in range(kb * 128, (kb + 1) * 128))
+                assert int(r["sums"][m, n, kb]) == want
+    # the epilogue undoes both quantizations: close to the float product with table * scale weights
+    w = O.dequantize_woq_weight(qw, N, K, scales, None, O.WOQ_DTYPE_NF4, G).astype(np.float64)
+    exact = x.astype(np.float64) @ w.T
+    assert np.abs(r["acc"] - exact).max() <= 0.02 * np.abs(exact).max() + 0.05
+    # and it is exactly sum_kb (float(sum) * s_a) * (s_w * fp32(1 / 127)) in fp32
+    f = np.float32
+    for m in range(M):
+        for n in range(N):
+            c = f(0)
+            for kb in range(K // 128):
+                sw = f(scales[n, kb] * (f(1.0) / f(127.0)))
+                c = f(c + f(f(f(r["sums"][m, n, kb]) * f(r["sa"][m])) * sw))
+            assert r["acc"][m, n] == c
+
+
 def test_nf4_quantize_dequantize_roundtrip_error_bound():
     # the package's quantizer picks the nearest table entry: error <= half the widest gap x scale
     from ipex_amd.quantization._qconfig import WoqWeightDtype
