@@ -212,24 +212,24 @@ int woq_hip_linear(const woq_hip_linear_params* p) {
   if (nf4) {
     // table lookups instead of the integer decode: the dequantizing decode kernel and the two
     // general kernels carry them
-    if (kernel == 0) kernel = decode_dq_applies(f, wbits, regime) ? 7 : (p->M <= 64 ? 1 : 2);
+    if (kernel == 0) kernel = (p->M <= 32 && decode_dq_applies(f, wbits, regime)) ? 7 : (p->M <= 64 ? 1 : 2);
     if (kernel != 1 && kernel != 2 && (kernel < 7 || kernel > 9))
       return set_error("woq_linear: NF4 weights run on kernels 1, 2 and 7..9 only");
   }
   if (kernel == 0 && decode_kernel_applies(f, wbits, regime, p->scale_zero_f16x2))
     return launch_decode(f, p->scale_zero_f16x2, st);
-  if (kernel == 0 && decode_dq_applies(f, wbits, regime)) kernel = 7;
+  // 33..64 rows: the decode kernel with four row tiles, except for very wide layers, where the
+  // prefill kernel's activation reuse wins (M = 64, 4096 -> 14336: 27 us against 37 us and 58 us for the
+  // small-M kernel; 4096 -> 28672: 51 us against 42 us)
+  const bool w4 = gemm_w4_applies(f, wbits, regime);
+  if (kernel == 0 && decode_dq_applies(f, wbits, regime) && !(p->M > 32 && w4 && p->N >= 16384)) kernel = 7;
   if (kernel >= 7 && kernel <= 10) {
     if (!decode_dq_applies(f, wbits, regime))
-      return set_error("woq_linear: the dequantizing decode kernel takes M <= 32, K a multiple of the weight tile, a "
+      return set_error("woq_linear: the dequantizing decode kernel takes M <= 64, K a multiple of the weight tile, a "
                        "power-of-two or per-channel group size and activations in the compute dtype");
     return launch_decode_dq(f, wbits, regime, st, kernel == 10 ? 4 : kernel - 7);
   }
   if (kernel == 0) {
-    // 33..64 rows: the streaming kernel re-reads the activations once per workgroup, which costs
-    // more than the prefill kernel's half-empty 128-row tiles once N is large (M = 64, 4096 -> 14336:
-    // 57 us against 37 us; 4096 -> 4096: 23 us against 35 us)
-    const bool w4 = gemm_w4_applies(f, wbits, regime);
     if (p->M <= 64)
       kernel = (p->M > 32 && w4 && p->N >= 8192) ? 3 : 1;
     else

@@ -234,24 +234,35 @@ __global__ __launch_bounds__(512, 4) void woq_decode_dq_kernel(const DecodeDqArg
 template <int REGIME, int WBITS, int MT, int NTW, bool NF4 = false>
 static int launch_dq_cfg(DecodeDqArgs a, hipStream_t st) {
   using Geo = DqGeom<WBITS, MT>;
-  // at most 64 KiB of activation buffers per workgroup, so that two workgroups share a CU
-  const int max_w = 65536 / (2 * Geo::SLICE);
+  // at most 64 KiB of activation buffers per workgroup, so that two workgroups share a CU; with
+  // four row tiles (33..64 rows) a wave's two buffers are 32 KiB and one workgroup of four waves
+  // takes 128 KiB
+  constexpr int kLdsCap = MT > 2 ? 131072 : 65536;
+  const int max_w = kLdsCap / (2 * Geo::SLICE);
   a.W = (int)(a.f.KT < max_w ? a.f.KT : max_w);
   if (a.W > 8) a.W = 8;
   size_t smem = (size_t)a.W * 2 * Geo::SLICE;
   const size_t red = (size_t)NTW * MT * a.W * 64 * sizeof(f4);
   if (red > smem) smem = red;
+  auto kern = woq_decode_dq_kernel<REGIME, WBITS, MT, NTW, NF4>;
+  if (MT > 2) {
+    // more than 64 KiB of LDS per workgroup needs an opt-in (once per kernel and process)
+    static const hipError_t lds_optin =
+        hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, kLdsCap);
+    if (lds_optin != hipSuccess)
+      return set_error("woq_decode_dq_kernel: LDS opt-in failed: %s", hipGetErrorString(lds_optin));
+  }
   const unsigned grid = (unsigned)(a.f.NT / NTW);
-  woq_decode_dq_kernel<REGIME, WBITS, MT, NTW, NF4><<<grid, a.W * 64, smem, st>>>(a);
+  kern<<<grid, a.W * 64, smem, st>>>(a);
   return check_launch("woq_decode_dq_kernel");
 }
 
-// At most 32 rows already in the compute dtype, whole K tiles, and (4-bit) a group size whose
+// At most 64 rows already in the compute dtype, whole K tiles, and (4-bit) a group size whose
 // boundaries never split a lane's 32 consecutive K values (8-bit: 16).
 bool decode_dq_applies(const FpArgs& f, int wbits, int regime) {
   const int want = regime == kRegimeF16 ? WOQ_HIP_ACT_FP16 : WOQ_HIP_ACT_BF16;
   const int tk = wbits == 4 ? kTileK4 : kTileK8;
-  if (f.M > 32 || f.x_dtype != want || ((uintptr_t)f.x & 15) != 0) return false;
+  if (f.M > 64 || f.x_dtype != want || ((uintptr_t)f.x & 15) != 0) return false;
   if (f.K % tk != 0 || f.M * f.K * 2 >= (int64_t)1 << 31) return false;
   if (f.G >= f.KT * tk) return true;
   return f.G >= (wbits == 4 ? 32 : 16) && (f.G & (f.G - 1)) == 0;
@@ -259,7 +270,13 @@ bool decode_dq_applies(const FpArgs& f, int wbits, int regime) {
 
 template <int REGIME, int WBITS>
 static int launch_dq_regime(const DecodeDqArgs& a, int ntw, hipStream_t st) {
-  const bool two_rows = a.f.M > 16;
+  const int mt = a.f.M > 32 ? 4 : a.f.M > 16 ? 2 : 1;
+  if (mt == 4) {
+    // 33..64 rows: one or two row-blocks per workgroup (four would leave too few workgroups)
+    if (ntw == 4) return set_error("woq_decode_dq_kernel: 33..64 rows take 1 or 2 row-blocks per workgroup");
+    return ntw == 2 ? launch_dq_cfg<REGIME, WBITS, 4, 2>(a, st) : launch_dq_cfg<REGIME, WBITS, 4, 1>(a, st);
+  }
+  const bool two_rows = mt == 2;
   if (ntw == 4) return two_rows ? launch_dq_cfg<REGIME, WBITS, 2, 4>(a, st) : launch_dq_cfg<REGIME, WBITS, 1, 4>(a, st);
   if (ntw == 2) return two_rows ? launch_dq_cfg<REGIME, WBITS, 2, 2>(a, st) : launch_dq_cfg<REGIME, WBITS, 1, 2>(a, st);
   return two_rows ? launch_dq_cfg<REGIME, WBITS, 2, 1>(a, st) : launch_dq_cfg<REGIME, WBITS, 1, 1>(a, st);
@@ -288,9 +305,11 @@ int launch_decode_dq(const FpArgs& f, int wbits, int regime, hipStream_t st, int
     return set_error("woq_decode_dq_kernel: %d row-blocks per workgroup do not divide %lld", ntw, (long long)f.NT);
   // Two row-blocks per workgroup re-read the activations half as often; with one there are twice
   // as many workgroups, which small N needs to fill the chip (two workgroups per CU are resident).
-  if (ntw == 0) ntw = (f.NT >= 512 && f.NT % 2 == 0) ? 2 : 1;
+  // (33..64 rows: the activations are four times the bytes, so two row-blocks pay off earlier)
+  if (ntw == 0) ntw = (f.NT >= (f.M > 32 ? 384 : 512) && f.NT % 2 == 0) ? 2 : 1;
   if (f.nf4) {
     if (wbits != 4 || f.zeros) return set_error("woq_decode_dq_kernel: NF4 weights are 4-bit and symmetric");
+    if (f.M > 32) return set_error("woq_decode_dq_kernel: NF4 weights take at most 32 rows");
     if (ntw == 4) return set_error("woq_decode_dq_kernel: NF4 weights take 1 or 2 row-blocks per workgroup");
     return regime == kRegimeF16 ? launch_dq_nf4<kRegimeF16>(a, ntw, st) : launch_dq_nf4<kRegimeBF16>(a, ntw, st);
   }

@@ -330,6 +330,27 @@ def test_dequantizing_decode_kernel_two_row_tiles_int4(cuda, M, K, N, G):
     _check_fp(case, O.LOWP_BF16, force_kernel=7, label=f"decode dq int4 M={M} K={K} N={N} G={G}")
 
 
+@pytest.mark.parametrize("M,K,N,G,bias", [(33, 1024, 96, 128, True), (64, 2048, 544, 32, False), (50, 384, 96, -1, True),
+                                          (64, 512, 768, 128, False)])
+@pytest.mark.parametrize("kernel", [0, 8, 9])  # automatic, then one / two row-blocks per workgroup
+def test_dequantizing_decode_kernel_four_row_tiles(cuda, M, K, N, G, bias, kernel):
+    """33..64 rows: four row tiles per wave, 128 KiB of activation buffers per workgroup."""
+    case = _synthetic().make_int4_case(35, M, K, N, G, bias=bias)
+    _check_fp(case, O.LOWP_BF16, force_kernel=kernel, label=f"decode dq int4 M={M} K={K} N={N} G={G} kernel={kernel}")
+
+
+def test_dequantizing_decode_kernel_four_row_tiles_int8_weights_and_rejections(cuda):
+    case = _synthetic().make_int8_case(36, 48, 704, 128)
+    _check_fp(case, O.LOWP_BF16, force_kernel=7, label="decode dq int8 weights M=48")
+    ctx = make_context(case, O.LOWP_BF16)
+    with pytest.raises(RuntimeError, match="row-blocks"):
+        ctx.run(case["x"].cuda(), force_kernel=10)
+    nf4 = _synthetic().make_nf4_case(37, 40, 512, 64, 128)
+    with pytest.raises(RuntimeError, match="NF4"):
+        make_context(nf4, O.LOWP_BF16).run(nf4["x"].cuda(), force_kernel=7)
+    _check_fp(nf4, O.LOWP_BF16, label="nf4 M=40 takes the small-M kernel")
+
+
 def test_dequantizing_decode_kernel_fp16_regime_and_symmetric(cuda):
     """fp16 regime with a group size the integer-weight decode kernel does not take, and weights
     without zero points."""
@@ -357,7 +378,7 @@ def test_dequantizing_decode_kernel_close_to_small_m_kernel(cuda):
     a, b = to_np_f32(ctx.run(x, force_kernel=7)), to_np_f32(ctx.run(x, force_kernel=1))
     assert bool(np.all((bf16_ulp_diff(a, b) <= 1) | (np.abs(a - b) <= 1e-4)))
     with pytest.raises(RuntimeError, match="dequantizing decode kernel"):
-        ctx.run(torch.randn(33, 2048, device=cuda).bfloat16(), force_kernel=7)
+        ctx.run(torch.randn(65, 2048, device=cuda).bfloat16(), force_kernel=7)
 
 
 def test_int8_weights_small_and_tiled(cuda):
