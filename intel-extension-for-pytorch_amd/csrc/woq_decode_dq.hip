@@ -1,4 +1,4 @@
-// Decode kernel with per-weight dequantization: 4- or 8-bit weights, M <= 32, HBM-bound weight
+// Decode kernel with per-weight dequantization: 4- or 8-bit weights, M <= 64, HBM-bound weight
 // streaming.
 //
 // Reference counterpart: the M >= 5 path of lowp_mode BF16 -- Dequantize<bfloat16> into a bf16
@@ -15,15 +15,15 @@
 // the weight stream itself, so the rounds are software pipelined: the requests of round r + 1
 // (tiles and parameters into registers, activations into the other LDS buffer) are issued before
 // round r is computed.
-// Activations: a wave copies the rows of its K tile (16 or 32 rows x 256 bytes for 4-bit weights,
+// Activations: a wave copies the rows of its K tile (16, 32 or 64 rows x 256 bytes for 4-bit weights,
 // x 128 bytes for 8-bit ones) straight into its private slice of LDS (global_load_lds_dwordx4:
 // fully coalesced, no registers) and reads the operand fragments from there; chunk p of row m sits
 // at p ^ m (p ^ (m / 2) for the 128-byte rows) so the fragment reads are conflict-free.  Reading
 // the fragments from global memory directly costs the same number of instructions but each one
 // gathers 64 separate 16-byte pieces, which made the texture addresser the bottleneck (M = 16:
 // 19.7 us against 13.9 us at M = 8 for the same weights).  Rows past M re-read row M - 1 and their
-// results are dropped.  The at most 64 KiB of slices are reused for the cross-wave sum, so two
-// workgroups fit on a CU.
+// results are dropped.  The at most 64 KiB of slices (up to 32 rows; 128 KiB and four waves for
+// 33..64 rows) are reused for the cross-wave sum; up to 32 rows two workgroups fit on a CU.
 #include "woq_common.h"
 #include "woq_internal.h"
 

@@ -74,7 +74,7 @@ struct DecodeArgs {
 bool decode_kernel_applies(const FpArgs& f, int wbits, int regime, const uint32_t* sz);
 int launch_decode(const FpArgs& f, const uint32_t* sz, hipStream_t st);
 
-// Decode kernel with per-weight dequantization (woq_decode_dq.hip): 4- or 8-bit weights, M <= 32.
+// Decode kernel with per-weight dequantization (woq_decode_dq.hip): 4- or 8-bit weights, M <= 64.
 // ntw: weight row-blocks per workgroup (1, 2 or 4), 0 = automatic
 bool decode_dq_applies(const FpArgs& f, int wbits, int regime);
 int launch_decode_dq(const FpArgs& f, int wbits, int regime, hipStream_t st, int ntw = 0);
