@@ -184,6 +184,7 @@ int woq_hip_linear(const woq_hip_linear_params* p) {
       a.out_dtype = p->out_dtype; a.workspace = p->workspace; a.workspace_bytes = p->workspace_bytes;
       a.debug_block_sums = p->debug_block_sums;
       a.nf4 = nf4 ? 1 : 0;
+      a.group_size = p->group_size;
       return launch_int8_linear(a, st);
     }
   }

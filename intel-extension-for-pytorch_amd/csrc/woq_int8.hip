@@ -659,7 +659,7 @@ __global__ __launch_bounds__(256) void woq_gemm_i8_kernel(const Int8KArgs p) {
             if (DEBUG) {
               // the block sum as the reference defines it: unsigned activations times weights
               const int64_t m = mrow0 + i * 32 + 8 * (e >> 2) + (e & 3);
-              if (m < a.M && n < a.N)
+              if (m < a.M && n < a.N && kq < (int)p.Kpad)  // (a K step may end past the padded K)
                 a.debug_block_sums[(m * a.N + n) * (p.Kpad / BLOCK_K) + kq / BLOCK_K] =
                     ASYM ? qc[i][j][e] + 128 * qcomp[j][e] : qc[i][j][e];
             }
@@ -731,8 +731,10 @@ int launch_int8_linear(const Int8Args& a, hipStream_t st) {
   p.a = a;
   p.Kpad = a.KT * TK;
   p.ldq = p.Kpad;
-  const int64_t G = a.G;  // per-channel callers pass G >= Kpad
-  const bool per_channel = G >= p.Kpad;
+  const int64_t G = a.G;
+  // Group-wise even when a single group covers all of K: the activation blocks then follow the
+  // group size, not the K block (quant_w_mode, csrc/cpu/aten/Linear.cpp:511-513).
+  const bool per_channel = a.group_size <= 0;
   p.block_k = woq_hip_int8_block_k(per_channel ? -1 : G, a.K);
   if (p.block_k % 32 != 0 || 128 % p.block_k != 0)
     return set_error("lowp_mode INT8: K block %lld (from group_size / K) must be 32, 64 or 128",

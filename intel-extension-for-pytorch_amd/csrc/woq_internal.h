@@ -97,6 +97,7 @@ struct Int8Args {
   const float* scales;   // fp32 [NT][KG][16]
   const uint8_t* zeros;  // [NT][KG][16] or nullptr
   int64_t G, KG;
+  int64_t group_size;    // as the caller gave it: <= 0 means one scale per output channel
   const float* bias;
   int act_quant_mode;
   int fusion;

@@ -727,3 +727,66 @@ def test_g_idx_validation(cuda):
         ops.WoqLinearOpContext(*args(torch.zeros(256, dtype=torch.int64)))
     with pytest.raises(RuntimeError, match="must lie in"):
         ops.WoqLinearOpContext(*args(torch.full((256,), 5, dtype=torch.int64)))
+
+
+# ---------------------------------------------------------------------------------------------
+# seeded random shapes through the automatic dispatch
+# ---------------------------------------------------------------------------------------------
+def _random_cases(n, seed):
+    rng = np.random.default_rng(seed)
+    out = []
+    for i in range(n):
+        kind = ["int4", "int4", "int4", "int8", "nf4"][int(rng.integers(0, 5))]
+        M = int(rng.choice([1, 2, 3, 4, 5, 7, 12, 16, 17, 29, 32, 33, 47, 64, 65, 90, 128, 150, 260]))
+        G = int(rng.choice([-1, 32, 64, 128, 256]))
+        if kind == "int8":
+            G = -1
+        kmul = 8 if rng.random() < 0.2 else (64 if kind == "int8" else 128)  # sometimes a ragged K
+        K = int(rng.integers(1, 9)) * kmul * (1 if kmul > 8 else int(rng.integers(4, 40)))
+        if G > 0:
+            K = max(G, (K // G) * G) if rng.random() < 0.8 else K  # mostly whole groups
+        K += K % 2  # two nibbles per byte
+        N = int(rng.choice([16, 17, 48, 64, 100, 272, 500, 1024]))
+        out.append((i, kind, M, K, N, G, bool(rng.random() < 0.5), bool(rng.random() < 0.3)))
+    return out
+
+
+@pytest.mark.parametrize("idx,kind,M,K,N,G,bias,sym", _random_cases(48, 2024))
+def test_random_shapes_float_regimes(cuda, idx, kind, M, K, N, G, bias, sym):
+    syn = _synthetic()
+    if kind == "int8":
+        case = syn.make_int8_case(100 + idx, M, K, N, bias=bias)
+    elif kind == "nf4":
+        case = syn.make_nf4_case(100 + idx, M, K, N, G, bias=bias)
+    else:
+        case = syn.make_int4_case(100 + idx, M, K, N, G, bias=bias)
+        if sym:
+            case["zeros"] = None
+    _check_fp(case, O.LOWP_BF16, label=f"random {idx}: {kind} M={M} K={K} N={N} G={G} bias={bias} sym={sym}")
+
+
+@pytest.mark.parametrize("idx,kind,M,K,N,G,bias,sym", [c for c in _random_cases(40, 777) if c[1] != "int8" or True][:32])
+def test_random_shapes_lowp_int8(cuda, idx, kind, M, K, N, G, bias, sym):
+    """lowp_mode INT8 with a random activation-quantization mode; shapes whose K blocks the int8
+    kernels do not take run unquantized, as the reference's fallback does, and are checked as such."""
+    syn = _synthetic()
+    mode = [6, 7, 4, 5, 2, 3, 0, 1][idx % 8]
+    if kind == "int8":
+        case = syn.make_int8_case(200 + idx, M, K, N, bias=bias)
+    elif kind == "nf4":
+        case = syn.make_nf4_case(200 + idx, M, K, N, G, bias=bias)
+    else:
+        case = syn.make_int4_case(200 + idx, M, K, N, G, bias=bias)
+        if sym:
+            case["zeros"] = None
+    bk = O.int8_block_k(G, K)
+    label = f"random int8 {idx}: {kind} mode={mode} M={M} K={K} N={N} G={G}"
+    if bk in (32, 64, 128):
+        _check_int8(case, mode, label=label)
+    else:
+        ctx = make_context(case, O.LOWP_INT8, mode)
+        y = to_np_f32(ctx.run(case["x"].cuda()))
+        c = case_np(case)
+        _, y_ref = O.woq_linear_ref(c["x"], "bf16", c["qw"], N, K, O.bf16_round(c["scales"]), c["zps"], c["bias"],
+                                    case["weight_dtype"], G, "bf16")
+        assert rel_l2(y, y_ref) <= (REL_L2_OUT if c["bias"] is None else 4e-3), label
