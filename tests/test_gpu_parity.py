@@ -790,3 +790,54 @@ def test_random_shapes_lowp_int8(cuda, idx, kind, M, K, N, G, bias, sym):
         _, y_ref = O.woq_linear_ref(c["x"], "bf16", c["qw"], N, K, O.bf16_round(c["scales"]), c["zps"], c["bias"],
                                     case["weight_dtype"], G, "bf16")
         assert rel_l2(y, y_ref) <= (REL_L2_OUT if c["bias"] is None else 4e-3), label
+
+
+def _activation_variants(n, seed):
+    rng = np.random.default_rng(seed)
+    out = []
+    for i in range(n):
+        act = ["bf16", "fp16", "fp32"][int(rng.integers(0, 3))]
+        lowp = int(rng.choice([O.LOWP_NONE, O.LOWP_FP16, O.LOWP_BF16]))
+        if act == "fp32" and lowp == O.LOWP_NONE:
+            lowp = O.LOWP_BF16
+        lead = [(1,), (3,), (2, 5), (1, 40), (4, 33), (2, 3, 7)][int(rng.integers(0, 6))]
+        K = int(rng.choice([128, 256, 320, 1000, 1024]))
+        G = int(rng.choice([-1, 32, 64, 128]))
+        if G > 0 and K % G:
+            G = -1
+        N = int(rng.choice([16, 48, 100, 272]))
+        layout = ["contiguous", "strided_rows", "transposed"][int(rng.integers(0, 3))]
+        out.append((i, act, lowp, lead, K, N, G, layout))
+    return out
+
+
+@pytest.mark.parametrize("idx,act,lowp,lead,K,N,G,layout", _activation_variants(36, 99))
+def test_activation_dtypes_shapes_and_layouts(cuda, idx, act, lowp, lead, K, N, G, layout):
+    """fp16 / fp32 activations (converted inside the kernels), leading dimensions, and inputs that
+    are views: the op takes what nn.Linear takes."""
+    tdt = {"bf16": torch.bfloat16, "fp16": torch.float16, "fp32": torch.float32}[act]
+    M = int(np.prod(lead))
+    case = _synthetic().make_int4_case(300 + idx, M, K, N, G, bias=(idx % 2 == 0))
+    x2 = case["x"].float().to(tdt)  # values representable in bf16 whatever the dtype
+    ctx = make_context(case, lowp)
+    xg = x2.cuda()
+    if layout == "strided_rows":
+        wide = torch.zeros(M, K + 8, dtype=tdt, device=cuda)
+        wide[:, :K] = xg
+        xin = wide[:, :K]
+    elif layout == "transposed":
+        xin = xg.t().contiguous().t()
+    else:
+        xin = xg
+    assert layout == "contiguous" or not xin.is_contiguous() or M == 1 or K == 1
+    y = torch.ops.torch_ipex.ipex_woq_linear(xin.reshape(*lead, K) if layout == "contiguous" else xin, ctx.get_data_handle())
+    assert y.dtype == tdt and tuple(y.shape) == ((*lead, N) if layout == "contiguous" else (M, N))
+    y = to_np_f32(y).reshape(M, N)
+    c = case_np(case)
+    xs = to_np_f32(x2)
+    cd = O.select_compute(lowp, act, M)
+    if cd == "bf16":
+        _, want = O.woq_linear_opt_bf16(xs, act, c["qw"], N, K, c["scales"], c["zps"], c["bias"], 2, G)
+    else:
+        _, want = O.woq_linear_ref(xs, act, c["qw"], N, K, O._round_to(c["scales"], cd), c["zps"], c["bias"], 2, G, cd)
+    assert rel_l2(y, want) <= REL_L2_OUT, (idx, act, lowp, lead, K, N, G, layout, rel_l2(y, want))
