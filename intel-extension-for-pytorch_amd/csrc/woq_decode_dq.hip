@@ -303,10 +303,17 @@ int launch_decode_dq(const FpArgs& f, int wbits, int regime, hipStream_t st, int
     return set_error("woq_decode_dq_kernel: 1, 2 or 4 row-blocks per workgroup, got %d", ntw);
   if (ntw != 0 && f.NT % ntw != 0)
     return set_error("woq_decode_dq_kernel: %d row-blocks per workgroup do not divide %lld", ntw, (long long)f.NT);
-  // Two row-blocks per workgroup re-read the activations half as often; with one there are twice
-  // as many workgroups, which small N needs to fill the chip (two workgroups per CU are resident).
-  // (33..64 rows: the activations are four times the bytes, so two row-blocks pay off earlier)
-  if (ntw == 0) ntw = (f.NT >= (f.M > 32 ? 384 : 512) && f.NT % 2 == 0) ? 2 : 1;
+  // More row-blocks per workgroup re-read the activations less often (every workgroup streams all
+  // of x through LDS); fewer make more workgroups, which small N needs to fill the chip.  Measured at
+  // M = 16 / 32: 4096 -> 14336 (896 row-blocks) 14.4 / 11.4 / 10.7 us with 1 / 2 / 4, 4096 -> 6144 (384)
+  // 8.5 / 7.0 / 9.7 us, 14336 -> 4096 (256) 12.9 / 15.5 / 24.5 us.  33..64 rows (four row tiles, no
+  // variant with four row-blocks) have four times the activation bytes per workgroup.
+  if (ntw == 0) {
+    if (f.M <= 32 && !f.nf4 && f.NT >= 640 && f.NT % 4 == 0)
+      ntw = 4;
+    else
+      ntw = (f.NT >= 384 && f.NT % 2 == 0) ? 2 : 1;
+  }
   if (f.nf4) {
     if (wbits != 4 || f.zeros) return set_error("woq_decode_dq_kernel: NF4 weights are 4-bit and symmetric");
     if (f.M > 32) return set_error("woq_decode_dq_kernel: NF4 weights take at most 32 rows");
