@@ -297,8 +297,9 @@ struct Int8KArgs {
 };
 
 // Small-M int8 kernel; same work decomposition as the floating-point small-M kernel.
-template <int WBITS, int MT, int KPW, int NTW>
+template <int WBITS, int MT, int KPW, int NTW, bool NF4>
 __global__ __launch_bounds__(1024) void woq_small_m_i8_kernel(const Int8KArgs p) {
+  static_assert(!NF4 || WBITS == 4, "NF4 codes are 4 bits wide");
   constexpr int TK = WBITS == 4 ? kTileK4 : kTileK8;
   constexpr int STEPS = WBITS == 4 ? 2 : 1;  // 16x16x64 MFMAs per tile
   constexpr int CK = TK / 4;
@@ -343,7 +344,7 @@ __global__ __launch_bounds__(1024) void woq_small_m_i8_kernel(const Int8KArgs p)
           zb = a.zeros[(ntc * a.KG + g) * kTileN + r];
         }
         // a tile past the end contributes zeros: q = z = 0, offset-binary 128, or NF4 code 7
-        const uint32_t dead = WBITS == 4 ? (a.nf4 ? 0x77777777u : 0u) : 0x80808080u;
+        const uint32_t dead = WBITS == 4 ? (NF4 ? 0x77777777u : 0u) : 0x80808080u;
         wreg[t][i] = live ? wv : u4{dead, dead, dead, dead};
         zreg[t][i] = live ? zb : (uint8_t)(WBITS == 4 ? 0 : 128);
       }
@@ -377,7 +378,7 @@ __global__ __launch_bounds__(1024) void woq_small_m_i8_kernel(const Int8KArgs p)
 #pragma unroll
         for (int j = 0; j < STEPS; ++j) {
           const uint32_t* d = (const uint32_t*)&wreg[t][i] + (WBITS == 4 ? 2 * j : 0);
-          const i4 aop = decode16_i8<WBITS>(d, z4, a.nf4 != 0);
+          const i4 aop = decode16_i8<WBITS>(d, z4, NF4);
 #pragma unroll
           for (int mt = 0; mt < MT; ++mt)
             qc[mt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(aop, xb[i][j][mt], qc[mt], 0, 0, 0);
@@ -398,7 +399,7 @@ __global__ __launch_bounds__(1024) void woq_small_m_i8_kernel(const Int8KArgs p)
               for (int e = 0; e < 4; ++e) {
                 const int64_t n = nt * kTileN + 4 * (lane >> 4) + e;
                 float sw = live ? a.scales[(nt * a.KG + g) * kTileN + 4 * (lane >> 4) + e] : 0.0f;
-                if (a.nf4) sw = sw * (1.0f / 127.0f);
+                if (NF4) sw = sw * (1.0f / 127.0f);
                 const float cterm = ((float)qc[mt][e] * sa) * sw;
                 acc[t][mt][e] = acc[t][mt][e] + cterm;
                 if (a.debug_block_sums && live && m < a.M && n < a.N)
@@ -450,8 +451,9 @@ constexpr int ILDS = IBK + 16;
 // The activations arrive as int8 q_a - 128, the zero points are used as zp_a - 128, and the weight
 // column sums of the K block ("compensation") come from one more MFMA against a row of ones:
 // (sum (q_a - 128) B) - (zp_a - 128) sum B = sum q_a B - zp_a sum B, exactly the reference's integer.
-template <int WBITS, int BLOCK_K, bool PER_K, bool DEBUG, bool ASYM>
+template <int WBITS, int BLOCK_K, bool PER_K, bool DEBUG, bool ASYM, bool NF4 = false>
 __global__ __launch_bounds__(256) void woq_gemm_i8_kernel(const Int8KArgs p) {
+  static_assert(!NF4 || WBITS == 4, "NF4 codes are 4 bits wide");
   static_assert(!ASYM || PER_K, "the asymmetric variant reloads scales and zero points per K block");
   constexpr int TK = WBITS == 4 ? kTileK4 : kTileK8;
   const Int8Args& a = p.a;
@@ -522,7 +524,7 @@ __global__ __launch_bounds__(256) void woq_gemm_i8_kernel(const Int8KArgs p) {
       wrow[q] = ntl * 16 + r;
       wcol[q] = WBITS == 4 ? c * 32 : kt_off * 64 + c * 16;
       const int64_t nt = nt0 + ntl, kt = k0 / TK + kt_off;
-      const uint32_t dead = WBITS == 4 ? (a.nf4 ? 0x77777777u : 0u) : 0x80808080u;
+      const uint32_t dead = WBITS == 4 ? (NF4 ? 0x77777777u : 0u) : 0x80808080u;
       u4 wv = u4{dead, dead, dead, dead};
       uint32_t z = WBITS == 4 ? 8u : 128u;
       if (nt < a.NT && kt < a.KT) {
@@ -537,8 +539,8 @@ __global__ __launch_bounds__(256) void woq_gemm_i8_kernel(const Int8KArgs p) {
       }
       const uint32_t z4 = z * 0x01010101u;
       if (WBITS == 4) {
-        const i4 lo = decode16_i8<4>((const uint32_t*)&wv, z4, a.nf4 != 0);
-        const i4 hi = decode16_i8<4>((const uint32_t*)&wv + 2, z4, a.nf4 != 0);
+        const i4 lo = decode16_i8<4>((const uint32_t*)&wv, z4, NF4);
+        const i4 hi = decode16_i8<4>((const uint32_t*)&wv + 2, z4, NF4);
         wo[q][0] = bitcast<u4>(lo);
         wo[q][WBITS == 4 ? 1 : 0] = bitcast<u4>(hi);
       } else {
@@ -648,7 +650,7 @@ __global__ __launch_bounds__(256) void woq_gemm_i8_kernel(const Int8KArgs p) {
         const int n = ncol0 + j * 32;  // < NT * 16 by construction of the grid? clamp below
         const int nc = n < (int)a.NT * kTileN ? n : (int)a.NT * kTileN - 1;
         float sw = a.scales[((nc >> 4) * (int)a.KG + g) * kTileN + (nc & 15)];
-        if (a.nf4) sw = sw * (1.0f / 127.0f);
+        if (NF4) sw = sw * (1.0f / 127.0f);
 #pragma unroll
         for (int i = 0; i < 2; ++i) {
 #pragma unroll
@@ -686,7 +688,10 @@ __global__ __launch_bounds__(256) void woq_gemm_i8_kernel(const Int8KArgs p) {
 template <int WBITS, int MT, int KPW, int NTW>
 static int launch_small_i8_cfg(Int8KArgs& p, hipStream_t st) {
   const size_t smem = (size_t)NTW * MT * p.W * 64 * sizeof(f4);
-  auto kern = woq_small_m_i8_kernel<WBITS, MT, KPW, NTW>;
+  auto kern = woq_small_m_i8_kernel<WBITS, MT, KPW, NTW, false>;
+  if constexpr (WBITS == 4) {
+    if (p.a.nf4) kern = woq_small_m_i8_kernel<WBITS, MT, KPW, NTW, true>;
+  }
   if (smem > 64 * 1024) {
     hipError_t err = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
     if (err != hipSuccess) return set_error("hipFuncSetAttribute: %s", hipGetErrorString(err));
@@ -790,11 +795,29 @@ int launch_int8_linear(const Int8Args& a, hipStream_t st) {
     case 64: { WOQ_I8_GEMM_B(WB, 64) } break;             \
     default: { WOQ_I8_GEMM_B(WB, 128) } break;            \
   }
-  if (a.wbits == 4) {
+  // NF4 codes: the same kernel with the table decode and the scale / 127 (no debug-less / per-K
+  // split: the per-K-block form covers every mode)
+#define WOQ_I8_GEMM_NF4(BK)                                                                   \
+  if (asym && dbg)                                                                            \
+    woq_gemm_i8_kernel<4, BK, true, true, true, true><<<grid, 256, 0, st>>>(p);               \
+  else if (asym)                                                                              \
+    woq_gemm_i8_kernel<4, BK, true, false, true, true><<<grid, 256, 0, st>>>(p);              \
+  else if (dbg)                                                                               \
+    woq_gemm_i8_kernel<4, BK, true, true, false, true><<<grid, 256, 0, st>>>(p);              \
+  else                                                                                        \
+    woq_gemm_i8_kernel<4, BK, true, false, false, true><<<grid, 256, 0, st>>>(p);
+  if (a.wbits == 4 && a.nf4) {
+    switch (p.block_k) {
+      case 32: { WOQ_I8_GEMM_NF4(32) } break;
+      case 64: { WOQ_I8_GEMM_NF4(64) } break;
+      default: { WOQ_I8_GEMM_NF4(128) } break;
+    }
+  } else if (a.wbits == 4) {
     WOQ_I8_GEMM(4)
   } else {
     WOQ_I8_GEMM(8)
   }
+#undef WOQ_I8_GEMM_NF4
 #undef WOQ_I8_GEMM
 #undef WOQ_I8_GEMM_B
   return check_launch("woq_gemm_i8_kernel");
