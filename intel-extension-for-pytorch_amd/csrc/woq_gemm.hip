@@ -38,8 +38,9 @@ struct GemmTraits<kRegimeBF16> {
 constexpr int BM = 128, BN = 128, BK = 64;
 constexpr int LDS_STRIDE = BK + 8;  // elements; 16-byte pad against bank conflicts
 
-template <int WBITS, int REGIME, bool CONV>
+template <int WBITS, int REGIME, bool CONV, bool NF4>
 __global__ __launch_bounds__(256) void woq_gemm_kernel(const FpArgs f) {
+  static_assert(!NF4 || WBITS == 4, "NF4 codes are 4 bits wide");
   using T = GemmTraits<REGIME>;
   using vec8 = typename T::vec8;
   constexpr int TK = WBITS == 4 ? kTileK4 : kTileK8;
@@ -56,7 +57,7 @@ __global__ __launch_bounds__(256) void woq_gemm_kernel(const FpArgs f) {
   const int64_t Kpad = f.KT * TK;
 
   __shared__ float sNf4[16];
-  const bool nf4 = WBITS == 4 && f.nf4 != 0;
+  constexpr bool nf4 = NF4;  // a template parameter: a runtime flag in the decode loop is not free
   if (nf4) {
     if (tid < 16) sNf4[tid] = kNf4Values[tid];
     __syncthreads();
@@ -215,10 +216,11 @@ __global__ __launch_bounds__(256) void woq_gemm_kernel(const FpArgs f) {
 template <int WBITS, int REGIME>
 static int launch_gemm_cfg(const FpArgs& f, bool conv, hipStream_t st) {
   dim3 grid((unsigned)((f.NT * kTileN + BN - 1) / BN), (unsigned)((f.M + BM - 1) / BM));
-  if (conv)
-    woq_gemm_kernel<WBITS, REGIME, true><<<grid, 256, 0, st>>>(f);
-  else
-    woq_gemm_kernel<WBITS, REGIME, false><<<grid, 256, 0, st>>>(f);
+  auto kern = conv ? woq_gemm_kernel<WBITS, REGIME, true, false> : woq_gemm_kernel<WBITS, REGIME, false, false>;
+  if constexpr (WBITS == 4) {
+    if (f.nf4) kern = conv ? woq_gemm_kernel<WBITS, REGIME, true, true> : woq_gemm_kernel<WBITS, REGIME, false, true>;
+  }
+  kern<<<grid, 256, 0, st>>>(f);
   return check_launch("woq_gemm_kernel");
 }
 

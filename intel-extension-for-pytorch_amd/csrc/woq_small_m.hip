@@ -99,8 +99,9 @@ struct SmallMArgs {
   int64_t Kpad;   // KT * tile_k
 };
 
-template <int WBITS, int REGIME, int MT, int KPW, int NTW, bool CONV>
+template <int WBITS, int REGIME, int MT, int KPW, int NTW, bool CONV, bool NF4>
 __global__ __launch_bounds__(1024) void woq_small_m_kernel(const SmallMArgs a) {
+  static_assert(!NF4 || WBITS == 4, "NF4 codes are 4 bits wide");
   using T = RegimeTraits<REGIME>;
   using vec8 = typename T::vec8;
   constexpr int TK = WBITS == 4 ? kTileK4 : kTileK8;
@@ -120,7 +121,7 @@ __global__ __launch_bounds__(1024) void woq_small_m_kernel(const SmallMArgs a) {
   const int rows = (int)(f.M < MT * 16 ? f.M : MT * 16);
 
   __shared__ float sNf4[16];
-  const bool nf4 = WBITS == 4 && f.nf4 != 0;
+  constexpr bool nf4 = NF4;  // a template parameter: a runtime flag in the decode loop is not free
   if (nf4) {
     if (threadIdx.x < 16) sNf4[threadIdx.x] = kNf4Values[threadIdx.x];
     __syncthreads();
@@ -268,7 +269,10 @@ static int launch_cfg(SmallMArgs& a, hipStream_t st) {
   while (a.W > 1 && smem_for(a.W) > 96 * 1024) a.W = (a.W + 1) / 2;
   const int W = a.W;
   const size_t smem = smem_for(W);
-  auto kern = woq_small_m_kernel<WBITS, REGIME, MT, KPW, NTW, CONV>;
+  auto kern = woq_small_m_kernel<WBITS, REGIME, MT, KPW, NTW, CONV, false>;
+  if constexpr (WBITS == 4) {
+    if (a.f.nf4) kern = woq_small_m_kernel<WBITS, REGIME, MT, KPW, NTW, CONV, true>;
+  }
   if (smem > 160 * 1024) return set_error("small-M kernel: LDS request %zu exceeds 160 KiB", smem);
   if (smem > 64 * 1024) {
     hipError_t err = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
