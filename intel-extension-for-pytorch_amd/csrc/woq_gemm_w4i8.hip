@@ -1,0 +1,337 @@
+// int8 MFMA GEMM for 4-bit weights and large M under lowp_mode INT8 (prefill): symmetric activation
+// quantization (per tensor, per row, per K block or per row and K block), K blocks of 128.
+//
+// Reference counterpart: Dequantize<int8_t> of a [128 x 32] weight block, int8 BRGEMM into int32,
+// then the fp32 epilogue C += (float(sum) * s_a[m]) * s_w[n, g] per K block
+// (csrc/cpu/aten/utils/woq.h:1664-1734, 2133-2199; driver woq.h:3298-3452).
+//
+// Same decomposition as the bf16 prefill kernel: v_mfma_i32_16x16x64_i8 with A = quantized
+// activations (row m = lane % 16, 16 K values per lane) and B = weights (column n = lane % 16);
+// the two packed dwords of a lane, decoded to sixteen int8 (q - z), ARE the B operand, so every
+// weight is decoded once per 64 rows by exactly one wave and never stored.  The activations
+// (already quantized, each group of eight in the order the nibble decode produces) and the packed
+// tiles go from global memory straight into LDS (global_load_lds_dwordx4), two K steps ahead; 16-byte
+// chunk p of activation row m sits at chunk p ^ ((m / 2) % 8), which makes the fragment reads
+// conflict-free for 128-byte rows.
+// The int32 sums of a K step (128 K values = the reference's K block) are scaled into fp32
+// accumulators right away: four VALU instructions per output element and step, which is what
+// bounds the kernel.  A workgroup is 64 rows x 128 columns so that three fit on a CU (152 registers,
+// 48 KiB of LDS): with 128 rows and one wave per SIMD the LDS reads, the barrier and the MFMAs of a
+// step all sat exposed between its VALU work (452 us for M = 2048, 4096 -> 14336, against 245 us).
+#include "woq_common.h"
+#include "woq_internal.h"
+
+// the three roundings of the epilogue stay separate (see woq_int8.hip)
+#pragma clang fp contract(off)
+
+namespace woq {
+
+constexpr int W8_WAVES = 4;
+constexpr int W8_MT = 4;    // 16-row tiles: 64 rows per workgroup
+constexpr int W8_NTW = 2;   // weight row-blocks per wave: 128 columns per workgroup
+constexpr int W8_BM = 16 * W8_MT;
+constexpr int W8_BN = W8_WAVES * W8_NTW * kTileN;
+constexpr int W8_XBYTES = W8_BM * kTileK4;                     // one activation buffer (int8)
+constexpr int W8_XLOADS = W8_XBYTES / (W8_WAVES * 1024);       // LDS loads per wave and buffer
+constexpr int W8_WSTAGE = W8_WAVES * W8_NTW * kTileBytes;      // one weight stage
+constexpr int W8_NBUF = 3;    // activation buffers and weight stages: requests run two K steps ahead
+constexpr int W8_LDS_BYTES = W8_NBUF * (W8_XBYTES + W8_WSTAGE + W8_BM * (int)sizeof(float));
+
+struct W4I8Args {
+  const uint8_t* xq;       // [M][ldq] int8, groups of eight in nibble-decode order
+  int64_t ldq;
+  const float* sa;         // activation scales: sa[m * sa_m_stride + (kt >> q_shift) * sa_k_stride]
+  int64_t sa_m_stride;     // per row: scales per row (1 or the K blocks per row), else 0
+  int64_t sa_k_stride;     // per K block: 1, else 0
+  int q_shift;             // K tile kt belongs to activation K block kt >> q_shift
+  int64_t M, N, NT, KT, KG;
+  const uint8_t* qweight;
+  const float* scales;     // fp32 [NT][KG][16]
+  const uint8_t* zeros;    // [NT][KG][16] or nullptr (symmetric: codes stand for code - 8)
+  int g_shift;             // K tile kt belongs to group kt >> g_shift
+  Epilogue ep;
+};
+
+typedef __attribute__((address_space(3))) void* w8_lds_ptr_t;
+typedef const __attribute__((address_space(1))) void* w8_global_ptr_t;
+
+// Four bytes at once: ((b | 0x80808080) - z4) ^ 0x80808080 never borrows across bytes for
+// |q - z| < 128 and leaves q - z in two's complement.
+__device__ __forceinline__ uint32_t w8_sub_bytes(uint32_t b, uint32_t z4) {
+  return ((b | 0x80808080u) - z4) ^ 0x80808080u;
+}
+// sixteen K values of one lane from two packed dwords, in the order [e0 e4 e1 e5][e2 e6 e3 e7] per dword
+__device__ __forceinline__ i4 w8_decode16(uint32_t d0, uint32_t d1, uint32_t z4) {
+  i4 r;
+  r[0] = (int)w8_sub_bytes(d0 & 0x0F0F0F0Fu, z4);
+  r[1] = (int)w8_sub_bytes((d0 >> 4) & 0x0F0F0F0Fu, z4);
+  r[2] = (int)w8_sub_bytes(d1 & 0x0F0F0F0Fu, z4);
+  r[3] = (int)w8_sub_bytes((d1 >> 4) & 0x0F0F0F0Fu, z4);
+  return r;
+}
+
+// PER_K: the activation scales change with the K block; they reach the lanes through LDS.
+template <bool PER_K>
+__global__ __launch_bounds__(256, 3) void woq_gemm_w4i8_kernel(const W4I8Args a) {
+  // the activation buffers, then the weight stages, then the activation scales of a step's rows
+  extern __shared__ __align__(1024) uint8_t sX[];
+  uint8_t* const sW = sX + W8_NBUF * W8_XBYTES;
+  float* const sSA = (float*)(sW + W8_NBUF * W8_WSTAGE);
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int r = lane & 15, c = lane >> 4;
+  const int M = (int)a.M, NT = (int)a.NT, KT = (int)a.KT, KG = (int)a.KG;
+  const int m0 = blockIdx.y * W8_BM;
+  const int nt0 = (blockIdx.x * W8_WAVES + wave) * W8_NTW;
+
+  f4 acc[W8_MT][W8_NTW];
+#pragma unroll
+  for (int mt = 0; mt < W8_MT; ++mt)
+#pragma unroll
+    for (int t = 0; t < W8_NTW; ++t) acc[mt][t] = f4{0.f, 0.f, 0.f, 0.f};
+
+  // activation scales of this lane's accumulator rows m = 16 mt + 4 c + e: constant over K, or
+  // (PER_K) read from LDS at the top of every step, where wave 0 put them a step earlier
+  f4 sa[W8_MT];
+  if (!PER_K) {
+#pragma unroll
+    for (int mt = 0; mt < W8_MT; ++mt)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const int m = m0 + mt * 16 + 4 * c + e;
+        sa[mt][e] = a.sa[(int64_t)(m < M ? m : M - 1) * a.sa_m_stride];
+      }
+  }
+  const int sa_row = m0 + tid < M ? m0 + tid : M - 1;  // wave 0: the row whose scale this thread fetches
+  const float* const sa_mine = a.sa + (int64_t)sa_row * a.sa_m_stride;
+  float sa_next = 0.0f;
+
+  // ---- activations: load i of wave w fills LDS KiB number w * XLOADS + i of a buffer: rows
+  // 8 (w * XLOADS + i) + lane / 8, physical chunk lane % 8 = logical chunk ^ ((row / 2) % 8).
+  // Rows past M re-read row M - 1; their results are never stored. ----
+  uint32_t xoff[W8_XLOADS];
+#pragma unroll
+  for (int i = 0; i < W8_XLOADS; ++i) {
+    const int rowl = (wave * W8_XLOADS + i) * 8 + (lane >> 3);
+    const int rowc = m0 + rowl < M ? rowl : M - 1 - m0;
+    const int chunk = (lane & 7) ^ ((rowl >> 1) & 7);
+    xoff[i] = (uint32_t)(rowc * (int)a.ldq + chunk * 16);
+  }
+  const uint8_t* xbase = a.xq + (int64_t)m0 * a.ldq;
+  auto load_x = [&](int kt, int buf) {
+    const uint32_t ko = (uint32_t)kt * kTileK4;
+#pragma unroll
+    for (int i = 0; i < W8_XLOADS; ++i)
+      __builtin_amdgcn_global_load_lds((w8_global_ptr_t)(xbase + (uint32_t)(xoff[i] + ko)),
+                                       (w8_lds_ptr_t)(sX + buf * W8_XBYTES + (wave * W8_XLOADS + i) * 1024), 16, 0,
+                                       0);
+  };
+  // A fragment of row tile mt, MFMA j: row 16 mt + r, logical chunk 2 c + j
+  uint32_t rd[2];
+#pragma unroll
+  for (int j = 0; j < 2; ++j) rd[j] = (uint32_t)(r * 128 + (((2 * c + j) ^ ((r >> 1) & 7)) << 4));
+
+  // ---- weights ----
+  const bool has_z = a.zeros != nullptr;
+  const uint8_t* wbase[W8_NTW];
+  const float* sbase[W8_NTW];
+  const uint8_t* zbase[W8_NTW];
+#pragma unroll
+  for (int t = 0; t < W8_NTW; ++t) {
+    const int nt = nt0 + t < NT ? nt0 + t : NT - 1;
+    wbase[t] = a.qweight + (size_t)nt * KT * kTileBytes;
+    sbase[t] = a.scales + (size_t)nt * KG * kTileN;
+    zbase[t] = has_z ? a.zeros + (size_t)nt * KG * kTileN : (const uint8_t*)sbase[t];
+  }
+  const uint32_t woff = (uint32_t)lane * 16u;
+  uint8_t* const wmine = sW + wave * (W8_NTW * kTileBytes);
+  auto dma_w = [&](int kt, int stage) {
+    const uint32_t wo = (uint32_t)kt * kTileBytes + woff;
+#pragma unroll
+    for (int t = 0; t < W8_NTW; ++t)
+      __builtin_amdgcn_global_load_lds((w8_global_ptr_t)(wbase[t] + wo),
+                                       (w8_lds_ptr_t)(wmine + stage * W8_WSTAGE + t * kTileBytes), 16, 0, 0);
+  };
+  // scale and zero point of this lane's accumulator column n = r... the D tile of an MFMA has column
+  // n = lane % 16 in every lane, so one scale per row-block and lane; the B operand's column is the
+  // same n, so the zero point is per lane too.
+  auto load_q = [&](int kt, float (&s)[W8_NTW], uint8_t (&z)[W8_NTW]) {
+    int g = kt >> a.g_shift;
+    g = g < KG ? g : KG - 1;
+    const uint32_t qoff = (uint32_t)(g * kTileN + r);
+#pragma unroll
+    for (int t = 0; t < W8_NTW; ++t) {
+      s[t] = sbase[t][qoff];
+      z[t] = *(zbase[t] + qoff);  // raw: any use here would wait for the load inside the request
+    }
+  };
+
+  constexpr int kVmcnt0 = 0x0F70;
+  // all but the youngest request of activations and tiles (one K step's worth) have landed
+  constexpr int kVmcntStep = 0x0F70 | (W8_XLOADS + W8_NTW);
+
+  u4 wr[W8_NTW];
+  float sw[W8_NTW], swn[W8_NTW];
+  uint8_t zq[W8_NTW], zqn[W8_NTW];
+
+  // A K step here is short (about 2000 cycles: 32 MFMAs and the fp32 epilogue of 64 sums per lane),
+  // shorter than the round trip of a request, so activations and tiles are requested two steps ahead
+  // into three buffers; the scales and zero points of the next step ride in registers.
+  load_x(0, 0);
+  dma_w(0, 0);
+  load_x(KT > 1 ? 1 : 0, 1);
+  dma_w(KT > 1 ? 1 : 0, 1);
+  load_q(0, sw, zq);
+  __builtin_amdgcn_s_waitcnt(kVmcnt0);
+  __syncthreads();
+#pragma unroll
+  for (int t = 0; t < W8_NTW; ++t) wr[t] = *(const u4*)(wmine + t * kTileBytes + woff);
+
+  if (PER_K && tid < W8_BM) sSA[tid] = sa_mine[0];
+  __syncthreads();
+
+  // Per K step: the MFMAs of row-block 0, then those of row-block 1 with the fp32 epilogue of
+  // row-block 0 between them, then the epilogue of row-block 1.  What stays exposed in one wave (the
+  // fragment reads, the first MFMAs, the barrier) is covered by the other two workgroups of the CU.
+  int b0 = 0, b1 = 1, b2 = 2;  // buffers of steps kt, kt + 1, kt + 2
+  for (int kt = 0; kt < KT; ++kt) {
+    const uint8_t* xs = sX + b0 * W8_XBYTES;
+    const int kt1 = kt + 1 < KT ? kt + 1 : KT - 1;
+    const int kt2 = kt + 2 < KT ? kt + 2 : KT - 1;
+    // requests, oldest first: parameters of step kt + 1, then activations and tiles of step kt + 2
+    // into the buffers of step kt - 1, which every wave left before the last barrier
+    load_q(kt1, swn, zqn);
+    if (PER_K && tid < W8_BM) sa_next = sa_mine[(int64_t)(kt1 >> a.q_shift) * a.sa_k_stride];
+    __builtin_amdgcn_sched_barrier(0);  // the parameter loads stay the oldest requests of the step
+    load_x(kt2, b2);
+    dma_w(kt2, b2);
+    __builtin_amdgcn_sched_barrier(0);
+
+    if (PER_K) {
+#pragma unroll
+      for (int mt = 0; mt < W8_MT; ++mt) sa[mt] = *(const f4*)(sSA + b0 * W8_BM + mt * 16 + 4 * c);
+    }
+    // A fragments of the step: 2 MFMAs x MT row tiles
+    i4 xa[2][W8_MT];
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int mt = 0; mt < W8_MT; ++mt) xa[j][mt] = *(const i4*)(xs + mt * 2048 + rd[j]);
+
+    i4 qc[W8_NTW][W8_MT];
+#pragma unroll
+    for (int t = 0; t < W8_NTW; ++t) {
+      const uint32_t z4 = (has_z ? (uint32_t)zq[t] : 8u) * 0x01010101u;
+      const i4 bq0 = w8_decode16(wr[t][0], wr[t][1], z4);
+      const i4 bq1 = w8_decode16(wr[t][2], wr[t][3], z4);
+      __builtin_amdgcn_sched_barrier(0);
+      // one MFMA, then (second row-block) the fp32 epilogue of two sums of the first:
+      // C += (float(sum) * s_a[m]) * s_w[n, g]; each pair is fenced so that the order stands
+#pragma unroll
+      for (int i = 0; i < 2 * W8_MT; ++i) {
+        const int mt = i % W8_MT;
+        if (i < W8_MT)
+          qc[t][mt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(xa[0][mt], bq0, i4{0, 0, 0, 0}, 0, 0, 0);
+        else
+          qc[t][mt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(xa[1][mt], bq1, qc[t][mt], 0, 0, 0);
+        if (t > 0) {
+#pragma unroll
+          for (int u = 0; u < 2; ++u) {
+            const int q = 2 * i + u, pm = q / 4, pe = q % 4;
+            const float cterm = ((float)qc[t - 1][pm][pe] * sa[pm][pe]) * sw[t - 1];
+            acc[pm][t - 1][pe] = acc[pm][t - 1][pe] + cterm;
+          }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+#pragma unroll
+    for (int mt = 0; mt < W8_MT; ++mt)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const float cterm = ((float)qc[W8_NTW - 1][mt][e] * sa[mt][e]) * sw[W8_NTW - 1];
+        acc[mt][W8_NTW - 1][e] = acc[mt][W8_NTW - 1][e] + cterm;
+      }
+
+    // Next step: its activations and tiles (requested a step ago) must have landed -- every wave
+    // waits for its own requests, the barrier covers the others' -- and every wave must be done
+    // reading this step's buffer.  Written as an instruction: before the barrier builtin the
+    // compiler waits for every outstanding load, the requests for step kt + 2 included.
+    if (PER_K) {
+      if (tid < W8_BM) sSA[b1 * W8_BM + tid] = sa_next;
+      __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): the LDS write is done before the barrier
+    }
+    __builtin_amdgcn_s_waitcnt(kVmcntStep);
+    asm volatile("s_barrier" ::: "memory");
+#pragma unroll
+    for (int t = 0; t < W8_NTW; ++t) {
+      wr[t] = *(const u4*)(wmine + b1 * W8_WSTAGE + t * kTileBytes + woff);
+      sw[t] = swn[t];
+      zq[t] = zqn[t];
+    }
+    const int b = b0;
+    b0 = b1;
+    b1 = b2;
+    b2 = b;
+  }
+  // the requests past the last step are still writing LDS: drain them before the workgroup can end
+  __builtin_amdgcn_s_waitcnt(kVmcnt0);
+
+  // ---- store: D[m][n], lane (n = r, c) holds rows m = 16 mt + 4 c + e ----
+#pragma unroll
+  for (int mt = 0; mt < W8_MT; ++mt)
+#pragma unroll
+    for (int t = 0; t < W8_NTW; ++t) {
+      const int64_t n = (int64_t)(nt0 + t) * kTileN + r;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const int64_t m = m0 + mt * 16 + 4 * c + e;
+        if (m < M && n < a.N && nt0 + t < NT) epilogue_store<kRegimeBF16>(a.ep, m, n, acc[mt][t][e]);
+      }
+    }
+}
+
+// 4-bit integer codes, symmetric activation scales per tensor or per row, K blocks of 128 that are
+// whole weight tiles, and a group size of 128 * 2^s (or one group), so that a K tile has one scale.
+bool gemm_w4i8_applies(const Int8Args& a, int64_t block_k, int64_t qbk, bool per_k, bool asym) {
+  if (a.wbits != 4 || a.nf4 || asym || a.debug_block_sums) return false;
+  if (block_k != 128 || a.K % 128 != 0 || a.M <= 64) return false;
+  if (a.group_size > 0 && (a.G % 128 != 0 || ((a.G / 128) & (a.G / 128 - 1)) != 0)) return false;
+  // activation K blocks of 128 * 2^s as well (they follow the group size, or the K block)
+  if (per_k && (qbk % 128 != 0 || ((qbk / 128) & (qbk / 128 - 1)) != 0)) return false;
+  return a.M * a.K < ((int64_t)1 << 31);
+}
+
+int launch_gemm_w4i8(const Int8Args& a, const uint8_t* xq, int64_t ldq, const float* sa, int64_t sa_m_stride,
+                     int64_t sa_k_stride, int64_t qbk, hipStream_t st) {
+  static const hipError_t lds_optin[2] = {
+      hipFuncSetAttribute(reinterpret_cast<const void*>(&woq_gemm_w4i8_kernel<false>),
+                          hipFuncAttributeMaxDynamicSharedMemorySize, W8_LDS_BYTES),
+      hipFuncSetAttribute(reinterpret_cast<const void*>(&woq_gemm_w4i8_kernel<true>),
+                          hipFuncAttributeMaxDynamicSharedMemorySize, W8_LDS_BYTES)};
+  if (lds_optin[0] != hipSuccess || lds_optin[1] != hipSuccess)
+    return set_error("woq_gemm_w4i8_kernel: LDS opt-in failed: %s",
+                     hipGetErrorString(lds_optin[0] != hipSuccess ? lds_optin[0] : lds_optin[1]));
+  W4I8Args k;
+  k.xq = xq; k.ldq = ldq; k.sa = sa; k.sa_m_stride = sa_m_stride; k.sa_k_stride = sa_k_stride;
+  k.q_shift = 0;
+  while (sa_k_stride != 0 && ((int64_t)128 << k.q_shift) < qbk) ++k.q_shift;
+  k.M = a.M; k.N = a.N; k.NT = a.NT; k.KT = a.KT; k.KG = a.KG;
+  k.qweight = a.qweight; k.scales = a.scales; k.zeros = a.zeros;
+  k.g_shift = 30;
+  if (a.group_size > 0) {
+    k.g_shift = 0;
+    while (((int64_t)128 << k.g_shift) < a.G) ++k.g_shift;
+  }
+  k.ep = Epilogue{a.bias, a.fusion, a.other0, a.other1, a.out, a.out_dtype, a.x_dtype, a.N};
+  dim3 grid((unsigned)((a.NT * kTileN + W8_BN - 1) / W8_BN), (unsigned)((a.M + W8_BM - 1) / W8_BM));
+  if (sa_k_stride != 0)
+    woq_gemm_w4i8_kernel<true><<<grid, 256, W8_LDS_BYTES, st>>>(k);
+  else
+    woq_gemm_w4i8_kernel<false><<<grid, 256, W8_LDS_BYTES, st>>>(k);
+  return check_launch("woq_gemm_w4i8_kernel");
+}
+
+}  // namespace woq

@@ -770,6 +770,11 @@ int launch_int8_linear(const Int8Args& a, hipStream_t st) {
                                  a.wbits == 4 ? 1 : 0, asym ? 1 : 0, st))
     return rc;
 
+  // Large M, 4-bit weights, one activation scale per row or tensor: the kernel that feeds the
+  // decoded dwords straight to the MFMA
+  if (gemm_w4i8_applies(a, p.block_k, qbk_quant, per_k, asym))
+    return launch_gemm_w4i8(a, xq, p.ldq, sa, p.sa_m_stride, p.sa_k_stride, qbk_quant, st);
+
   // The small-M kernel accumulates whole tiles per MFMA, so it needs K blocks that are whole
   // tiles; finer blocks (group_size 32 / 64 with 4-bit weights) go through the tiled kernel,
   // which re-lays the weights in LDS in plain K order.

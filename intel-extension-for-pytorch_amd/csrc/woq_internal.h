@@ -111,6 +111,11 @@ struct Int8Args {
   int nf4;  // 4-bit codes index the NF4 int8 table; the weight scale is multiplied by fp32(1 / 127)
 };
 
+// int8 MFMA prefill kernel for 4-bit weights (woq_gemm_w4i8.hip): symmetric activation scales, K
+// blocks of 128; sa[m * sa_m_stride + (k / qbk) * sa_k_stride] is the scale of row m at k.
+bool gemm_w4i8_applies(const Int8Args& a, int64_t block_k, int64_t qbk, bool per_k, bool asym);
+int launch_gemm_w4i8(const Int8Args& a, const uint8_t* xq, int64_t ldq, const float* sa, int64_t sa_m_stride,
+                     int64_t sa_k_stride, int64_t qbk, hipStream_t st);
 int launch_dynamic_quant(const void* x, int x_dtype, int64_t M, int64_t K, int64_t ldq, int64_t qbk,
                          int mode, void* q, float* scales, int32_t* zps, hipStream_t st);
 int launch_int8_linear(const Int8Args& a, hipStream_t st);
