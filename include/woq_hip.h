@@ -208,7 +208,7 @@ typedef struct woq_hip_linear_params {
    * workgroup shape by cost model; 4 / 5 / 6 = the same kernel with 448 / 256 / 128 columns per workgroup;
    * 7 = dequantizing decode kernel (M <= 64, K % 128 == 0 for 4-bit and K % 64 == 0 for 8-bit weights, x in the
    * compute dtype), 8 / 9 / 10 = the same with one / two / four weight row-blocks per workgroup;
-   * 11 = the 4-bit prefill GEMM with 256 rows x 192 columns per workgroup.
+   * 11 / 12 = the 4-bit prefill GEMM with 256 rows x 192 columns / 64 rows x 128 columns per workgroup.
    * NF4 weights: 0, 1, 2, 7, 8, 9 only */
   int32_t force_kernel;
 

@@ -237,8 +237,8 @@ int woq_hip_linear(const woq_hip_linear_params* p) {
       kernel = w4 ? 3 : 2;
   }
   if (kernel == 1 && p->M > 64) return set_error("woq_linear: the small-M kernel takes M <= 64");
-  const int w4_shape = kernel == 4 ? 7 : kernel == 5 ? 4 : kernel == 6 ? 2 : kernel == 11 ? 163 : 0;
-  if ((kernel >= 4 && kernel <= 6) || kernel == 11) kernel = 3;
+  const int w4_shape = kernel == 4 ? 7 : kernel == 5 ? 4 : kernel == 6 ? 2 : kernel == 11 ? 163 : kernel == 12 ? 42 : 0;
+  if ((kernel >= 4 && kernel <= 6) || kernel == 11 || kernel == 12) kernel = 3;
   if (kernel == 3 && !gemm_w4_applies(f, wbits, regime))
     return set_error("woq_linear: the 4-bit prefill kernel takes 4-bit weights, K %% 128 == 0, a power-of-two or "
                      "per-channel group size and activations in the compute dtype");

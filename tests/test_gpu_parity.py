@@ -240,7 +240,7 @@ def test_both_kernels_agree_on_mid_m(cuda, M):
         (150, 256, 450, 128, True),  # N not a multiple of 8: element-wise stores
     ],
 )
-@pytest.mark.parametrize("shape", [3, 4, 5, 6, 11])  # cost model, then 448 / 256 / 128 columns per workgroup, then 256 rows x 192
+@pytest.mark.parametrize("shape", [3, 4, 5, 6, 11, 12])  # cost model, then 448 / 256 / 128 columns per workgroup, then 256 rows x 192, 64 x 128
 def test_w4_prefill_kernel(cuda, M, K, N, G, bias, shape):
     case = _synthetic().make_int4_case(20, M, K, N, G, bias=bias)
     _check_fp(case, O.LOWP_BF16, force_kernel=shape, label=f"w4 prefill M={M} K={K} N={N} G={G} kernel={shape}")
@@ -252,7 +252,7 @@ def test_w4_prefill_kernel_shapes_agree_bit_for_bit(cuda):
     case = _synthetic().make_int4_case(22, 2048, 512, 6144, 32, bias=True)
     ctx = make_context(case, O.LOWP_BF16)
     x = case["x"].cuda()
-    ys = [ctx.run(x, force_kernel=code) for code in (0, 4, 5, 6, 11)]
+    ys = [ctx.run(x, force_kernel=code) for code in (0, 4, 5, 6, 11, 12)]
     for y in ys[1:]:
         assert torch.equal(y, ys[0])
     cols = np.r_[0:64, 3000:3064, 6080:6144]
