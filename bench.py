@@ -83,6 +83,39 @@ def time_steps(torch, lib, params, steps, warmup, stream):
     return t1 - t0, start.elapsed_time(stop)
 
 
+def _quantiles(vals):
+    v = sorted(vals)
+    pick = lambda q: v[min(len(v) - 1, int(q * len(v)))]
+    return {"median": round(pick(0.5), 3), "p10": round(pick(0.1), 3), "p90": round(pick(0.9), 3)}
+
+
+def launch_distribution(torch, lib, params, stream, batches=40, per_batch=100):
+    """Spread of the per-launch time: `batches` groups of back-to-back launches, each group between
+    its own pair of events (microseconds per launch), and the latency of a single launch on an idle
+    device (host clock from the call to the end of a synchronize)."""
+    n = len(params)
+    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(batches)]
+    torch.cuda.synchronize()
+    i = 0
+    for e0, e1 in evs:
+        e0.record(stream)
+        for _ in range(per_batch):
+            lib.woq_hip_linear(ctypes.byref(params[i % n]))
+            i += 1
+        e1.record(stream)
+    torch.cuda.synchronize()
+    per_launch = [e0.elapsed_time(e1) * 1e3 / per_batch for e0, e1 in evs]
+    single = []
+    for j in range(200):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        lib.woq_hip_linear(ctypes.byref(params[j % n]))
+        torch.cuda.synchronize()
+        single.append((time.perf_counter() - t0) * 1e6)
+    return ({**_quantiles(per_launch), "batches": batches, "launches_per_batch": per_batch},
+            {**_quantiles(single), "launches": len(single), "clock": "host, call to end of synchronize"})
+
+
 def time_graph(torch, lib, params, steps, warmup):
     """Same launches captured once into a HIP graph (one node per weight copy) and replayed."""
     n = len(params)
@@ -181,9 +214,22 @@ def config_sweep(torch, lib, lib_mod, ops_mod, synthetic, dev, stream, steps):
     return rows
 
 
-def cpu_baseline_decode(case, K, N, G, budget_s=12.0):
+def _cpu_model():
+    try:
+        with open("/proc/cpuinfo") as fh:
+            for line in fh:
+                if line.startswith("model name"):
+                    return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
+def cpu_baseline_decode(case, K, N, G, budget_s=12.0, gpu_out=None):
     """The oracle's C port (bf16-regime arithmetic, OpenMP over output channels) on the same
-    decode workload, timed on the host cores this process may use."""
+    decode workload, timed on the host cores this process may use.  With `gpu_out` (the GPU's
+    bf16 output for the same inputs, on the host) one more untimed pass in the arithmetic of
+    that batch size (weights rounded to fp16, fp32 accumulation) checks it."""
     import numpy as np
 
     so = os.path.join(ROOT, "oracle", "libwoq_oracle.so")
@@ -213,14 +259,32 @@ def cpu_baseline_decode(case, K, N, G, budget_s=12.0):
         run()
         times.append(time.perf_counter() - t0)
     med = sorted(times)[len(times) // 2]
-    return {
+    res = {
         "value": round(algorithmic_bytes(1, K, N, G) / med / 1e9, 3),
         "unit": "GB/s",
         "cores": cores,
         "kind": "port",
         "sample": f"full workload (M=1, K={K}, N={N}), median of {len(times)} passes of oracle/woq_ref.c",
         "ms_per_step": round(med * 1e3, 4),
+        "cpu_model": _cpu_model(),
+        "label": "CPU restatement of IPEX woq_linear (IPEX binary unavailable)",
     }
+    if gpu_out is not None:
+        lib.woq_ref_linear_int4(x.ctypes.data, 1, K, N, qw.ctypes.data, sc.ctypes.data, zp.ctypes.data, G, None, 0,
+                                0, N, acc.ctypes.data)
+        got = gpu_out.float().numpy().reshape(-1).astype(np.float64)
+        torch = __import__("torch")
+        # the reference rounds the fp32 sum to fp16 and then to the activation dtype
+        want = torch.from_numpy(acc.reshape(-1).copy()).half().bfloat16().double().numpy()
+        rel_l2 = float(np.linalg.norm(got - want) / np.linalg.norm(want))
+        res["parity_of_gpu_output"] = {
+            "max_abs": round(float(np.abs(got - want).max()), 6),
+            "rel_l2": round(rel_l2, 7),
+            "rel_l2_gate": 2e-3,
+            "ok": bool(rel_l2 <= 2e-3),
+            "against": "this port with fp16-rounded weights and fp32 accumulation, sum rounded to fp16 then bf16",
+        }
+    return res
 
 
 def main():
@@ -298,6 +362,8 @@ def main():
         p.stream = stream.cuda_stream
     # cache-resident figure: the same weight every launch
     _, hot_ms = time_steps(torch, lib, params[:1], args.steps, args.warmup, stream)
+    spread, single = launch_distribution(torch, lib, params, stream)
+    out_host = out.cpu()
 
     us_launch = ev_ms * 1e3 / args.steps
     us_graph = g_ev_ms * 1e3 / g_steps
@@ -334,6 +400,8 @@ def main():
             "us_per_launch_stream": round(us_launch, 3),
             "us_per_launch_graph": round(us_graph, 3),
             "us_per_launch_cache_resident": round(hot_ms * 1e3 / args.steps, 3),
+            "us_per_launch_spread": spread,
+            "single_launch_latency_us": single,
         },
     }
 
@@ -389,7 +457,8 @@ def main():
                                                max(50, min(400, args.steps // 10)))
 
     if not args.no_cpu:
-        result["cpu_baseline"] = cpu_baseline_decode(synthetic.make_int4_case(2, 1, K, N, G), K, N, G)
+        result["cpu_baseline"] = cpu_baseline_decode(synthetic.make_int4_case(2, 1, K, N, G), K, N, G,
+                                                     gpu_out=out_host if M == 1 else None)
     else:
         result["cpu_baseline"] = None
     print(json.dumps(result))
