@@ -29,6 +29,8 @@
 
 namespace woq {
 
+constexpr int kDqMaxWaves = 8;
+
 struct DecodeDqArgs {
   FpArgs f;
   int W;        // waves per workgroup
@@ -218,12 +220,12 @@ __global__ __launch_bounds__(512, 4) void woq_decode_dq_kernel(const DecodeDqArg
     const int64_t n = (nt0 + t) * kTileN + col;
     if (m >= M || n >= f.N) continue;
     const int slot = (col + 16 * (m16 >> 2)) * 4 + (m16 & 3);
-    float part[8];
+    float part[kDqMaxWaves];
 #pragma unroll
-    for (int w = 0; w < 8; ++w) part[w] = w < W ? redf[(tm * W + w) * 256 + slot] : 0.0f;
+    for (int w = 0; w < kDqMaxWaves; ++w) part[w] = w < W ? redf[(tm * W + w) * 256 + slot] : 0.0f;
     float s = part[0];
 #pragma unroll
-    for (int w = 1; w < 8; ++w) s += part[w];
+    for (int w = 1; w < kDqMaxWaves; ++w) s += part[w];
     if (plain)
       ((uint16_t*)f.out)[(int64_t)m * f.N + n] = f32_to_bf16_bits(s);
     else
@@ -234,25 +236,30 @@ __global__ __launch_bounds__(512, 4) void woq_decode_dq_kernel(const DecodeDqArg
 template <int REGIME, int WBITS, int MT, int NTW, bool NF4 = false>
 static int launch_dq_cfg(DecodeDqArgs a, hipStream_t st) {
   using Geo = DqGeom<WBITS, MT>;
-  // at most 64 KiB of activation buffers per workgroup, so that two workgroups share a CU; with
-  // four row tiles (33..64 rows) a wave's two buffers are 32 KiB and one workgroup of four waves
-  // takes 128 KiB
-  constexpr int kLdsCap = MT > 2 ? 131072 : 65536;
-  const int max_w = kLdsCap / (2 * Geo::SLICE);
+  // At most 64 KiB of activation buffers per workgroup, so that two workgroups share a CU -- unless
+  // there is at most one workgroup per CU anyway: then two row tiles (17..32 rows, 16 KiB per wave for
+  // 4-bit weights) take 128 KiB and keep eight waves instead of four (M = 32, 4096 -> 14336, four
+  // row-blocks per workgroup: 13.9 us against 15.7 us; 14336 -> 4096: 19.1 us against 25.1 us).  With
+  // four row tiles (33..64 rows) a wave's two buffers are 32 KiB and one workgroup of four waves takes
+  // 128 KiB.  Sixteen waves of one row tile measured no faster than eight.
+  constexpr int kLdsMax = 131072;
+  const unsigned grid = (unsigned)(a.f.NT / NTW);
+  const bool alone = MT == 2 && grid <= 256;
+  const int lds_cap = (MT > 2 || alone) ? kLdsMax : 65536;
+  const int max_w = lds_cap / (2 * Geo::SLICE);
   a.W = (int)(a.f.KT < max_w ? a.f.KT : max_w);
-  if (a.W > 8) a.W = 8;
+  if (a.W > kDqMaxWaves) a.W = kDqMaxWaves;
   size_t smem = (size_t)a.W * 2 * Geo::SLICE;
   const size_t red = (size_t)NTW * MT * a.W * 64 * sizeof(f4);
   if (red > smem) smem = red;
   auto kern = woq_decode_dq_kernel<REGIME, WBITS, MT, NTW, NF4>;
-  if (MT > 2) {
+  if (MT >= 2) {
     // more than 64 KiB of LDS per workgroup needs an opt-in (once per kernel and process)
     static const hipError_t lds_optin =
-        hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, kLdsCap);
+        hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, kLdsMax);
     if (lds_optin != hipSuccess)
       return set_error("woq_decode_dq_kernel: LDS opt-in failed: %s", hipGetErrorString(lds_optin));
   }
-  const unsigned grid = (unsigned)(a.f.NT / NTW);
   kern<<<grid, a.W * 64, smem, st>>>(a);
   return check_launch("woq_decode_dq_kernel");
 }
