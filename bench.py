@@ -31,6 +31,9 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
 MEASURED_HBM_BYTES_PER_LAUNCH = {(1, 4096, 14336, 128): 31384678}
 
 
+_SPLIT_K_SCRATCH = {}
+
+
 def algorithmic_bytes(M, K, N, G):
     """INT4 weights 1/2 B, bf16 scales 2 B and packed uint4 zeros 1/2 B per (n, group),
     bf16 activations and outputs."""
@@ -58,6 +61,20 @@ def build_params(lib_mod, x, ctx, out, lowp_mode, act_quant_mode=-1, workspace=N
     p.fusion = 0
     p.out = out.data_ptr()
     p.out_dtype = lib_mod.ACT_BF16
+    if workspace is None and lowp_mode != 3:
+        # what the op layer passes for small batches: scratch that lets the decode kernel split K
+        # across workgroups, and the zeroed counters that go with it.  One block for all launches of
+        # this stream, as the op layer gets from torch's caching allocator call after call.
+        nbytes = lib_mod.load().woq_hip_linear_split_k_workspace_bytes(p.M, p.N)
+        if nbytes:
+            import torch
+
+            if "counters" not in _SPLIT_K_SCRATCH:
+                _SPLIT_K_SCRATCH["counters"] = torch.zeros(512, dtype=torch.int32, device=x.device)
+            if nbytes not in _SPLIT_K_SCRATCH:
+                _SPLIT_K_SCRATCH[nbytes] = torch.empty(nbytes, dtype=torch.uint8, device=x.device)
+            workspace = _SPLIT_K_SCRATCH[nbytes]
+            p.split_k_counters = _SPLIT_K_SCRATCH["counters"].data_ptr()
     if workspace is not None:
         p.workspace = workspace.data_ptr()
         p.workspace_bytes = workspace.numel()
@@ -189,13 +206,19 @@ def config_sweep(torch, lib, lib_mod, ops_mod, synthetic, dev, stream, steps):
     def run(name, case):
         M, K, N, G = case["M"], case["K"], case["N"], case["group_size"]
         params, keep = _rotating_params(torch, lib_mod, ops_mod, case, 2, dev, stream)
-        _, ms = time_steps(torch, lib, params, steps, max(10, steps // 10), stream)
-        us = ms * 1e3 / steps
+        # Each configuration starts after an idle period (its inputs are generated on the host) and
+        # the first few thousand launches after one run up to 10 % slower; single groups of a few
+        # hundred launches also scatter by +-5 %.  So: a warm-up as long as one group, then nine
+        # groups, and the median group is reported.
+        time_steps(torch, lib, params, steps, max(200, steps), stream)
+        groups = sorted(time_steps(torch, lib, params, steps, 0, stream)[1] * 1e3 / steps for _ in range(9))
+        us = groups[4]
         if case["weight_dtype"] == 2:
             nbytes = algorithmic_bytes(M, K, N, G)
         else:
             nbytes = N * K + N * 4 + M * K * 2 + M * N * 2 + (N * 2 if case["bias"] is not None else 0)
         rows.append({"config": name, "M": M, "K": K, "N": N, "group_size": G, "us_per_launch": round(us, 2),
+                     "us_p10_p90": [round(groups[1], 2), round(groups[7], 2)],
                      "GB_per_s": round(nbytes / us / 1e3, 1), "frac_of_hbm_peak": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 3)})
         del params, keep
         torch.cuda.empty_cache()
@@ -291,7 +314,9 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=4000)
-    ap.add_argument("--warmup", type=int, default=400)
+    ap.add_argument("--warmup", type=int, default=2000,
+                    help="untimed launches before the timed ones (the first few milliseconds after an idle "
+                         "period run 3-10 %% slower: clocks and translation caches are still warming up)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-prefill", action="store_true", help="skip the M=2048 measurement")
     ap.add_argument("--no-sweep", action="store_true", help="skip the other named configurations")
@@ -420,7 +445,7 @@ def main():
             pp = build_params(_lib, xp, keep[0], outp, lowp, aq, ws)
             pp.stream = stream.cuda_stream
             steps_p = max(10, min(200, args.steps // 20))
-            _, ms = time_steps(torch, lib, [pp], steps_p, max(3, steps_p // 5), stream)
+            _, ms = time_steps(torch, lib, [pp], steps_p, max(3, steps_p // 2), stream)
             us = ms * 1e3 / steps_p
             pre[name] = {"us_per_step": round(us, 2), "tflops": round(flops / (us * 1e-6) / 1e12, 1)}
         # For scale: the vendor's dense bf16 GEMM (torch.matmul) on the same activations and the

@@ -195,9 +195,18 @@ typedef struct woq_hip_linear_params {
   void* out;
   int32_t out_dtype;
 
-  /* workspace for lowp_mode == INT8 (size from woq_hip_linear_workspace_bytes) */
+  /* workspace: for lowp_mode == INT8 the quantized activations (size from
+   * woq_hip_linear_workspace_bytes); for the other modes, optional scratch for the split-K form of
+   * the dequantizing decode kernel (size from woq_hip_linear_split_k_workspace_bytes; contents
+   * undefined before and after the call) */
   void* workspace;
   int64_t workspace_bytes;
+
+  /* optional, with the split-K scratch: 512 int32 counters that are zero when the call is enqueued
+   * and are zero again when its work has finished (allocate and zero them once; calls that may run
+   * at the same time, e.g. on different streams, need arrays of their own).  NULL: K is never split
+   * across workgroups.  No counterpart in the reference, whose threads share the activations in cache. */
+  int32_t* split_k_counters;
 
   /* optional, lowp_mode == INT8 only: receives the exact int32 sum of every
    * (m, n, K-block) as int32 [M, N, Kp/block_k] (tests only, small shapes) */
@@ -208,8 +217,10 @@ typedef struct woq_hip_linear_params {
    * workgroup shape by cost model; 4 / 5 / 6 = the same kernel with 448 / 256 / 128 columns per workgroup;
    * 7 = dequantizing decode kernel (M <= 64, K % 128 == 0 for 4-bit and K % 64 == 0 for 8-bit weights, x in the
    * compute dtype), 8 / 9 / 10 = the same with one / two / four weight row-blocks per workgroup;
-   * 11 / 12 = the 4-bit prefill GEMM with 256 rows x 192 columns / 64 rows x 128 columns per workgroup.
-   * NF4 weights: 0, 1, 2, 7, 8, 9 only */
+   * 11 / 12 = the 4-bit prefill GEMM with 256 rows x 192 columns / 64 rows x 128 columns per workgroup;
+   * 13..17 = the dequantizing decode kernel (M <= 32) with (row-blocks per workgroup, K splits) =
+   * (1, 2), (2, 2), (4, 2), (2, 4), (4, 4): needs workspace and split_k_counters.
+   * NF4 weights: 0, 1, 2, 7, 8, 9, 13, 14, 16 only */
   int32_t force_kernel;
 
   void* stream;
@@ -217,6 +228,10 @@ typedef struct woq_hip_linear_params {
 
 int64_t woq_hip_linear_workspace_bytes(int64_t M, int64_t K, int32_t lowp_mode,
                                        int32_t act_quant_mode, int64_t group_size);
+
+/* Scratch bytes that let woq_hip_linear split K across workgroups for M rows and N output columns
+ * in the floating-point modes; 0 where it never does (M > 32).  No counterpart in the reference. */
+int64_t woq_hip_linear_split_k_workspace_bytes(int64_t M, int64_t N);
 
 /* K-block of the int8 path: min(group_size, 128), per-channel -> 128
  * (get_block_k, csrc/cpu/aten/Linear.cpp:362-376). */

@@ -114,6 +114,13 @@ int64_t woq_hip_linear_workspace_bytes(int64_t M, int64_t K, int32_t lowp_mode, 
   return qbytes + (M * Kc + 64) * 8;
 }
 
+int64_t woq_hip_linear_split_k_workspace_bytes(int64_t M, int64_t N) {
+  if (M <= 0 || M > 32 || N <= 0) return 0;
+  const int64_t NT = woq_hip_padded_n(N) / kTileN;
+  if (NT > 4 * kSplitKCounters) return 0;
+  return decode_dq_splitk_bytes(M, NT, kSplitKMax);
+}
+
 int woq_hip_linear(const woq_hip_linear_params* p) {
   if (!p) return set_error("woq_linear: null params");
   if (p->struct_size != sizeof(woq_hip_linear_params))
@@ -208,14 +215,20 @@ int woq_hip_linear(const woq_hip_linear_params* p) {
   f.zeros = p->zeros_u8; f.G = G; f.KG = KG; f.bias = p->bias; f.fusion = p->fusion;
   f.other0 = p->others[0]; f.other1 = p->others[1]; f.out = p->out; f.out_dtype = p->out_dtype;
   f.nf4 = nf4 ? 1 : 0;
+  SplitKScratch scratch;
+  if (p->split_k_counters && p->workspace && p->workspace_bytes > 0) {
+    scratch.partial = (float*)p->workspace;
+    scratch.bytes = p->workspace_bytes;
+    scratch.counters = p->split_k_counters;
+  }
 
   int kernel = p->force_kernel;
   if (nf4) {
     // table lookups instead of the integer decode: the dequantizing decode kernel and the two
     // general kernels carry them
     if (kernel == 0) kernel = (p->M <= 32 && decode_dq_applies(f, wbits, regime)) ? 7 : (p->M <= 64 ? 1 : 2);
-    if (kernel != 1 && kernel != 2 && (kernel < 7 || kernel > 9))
-      return set_error("woq_linear: NF4 weights run on kernels 1, 2 and 7..9 only");
+    if (kernel != 1 && kernel != 2 && (kernel < 7 || kernel > 9) && kernel != 13 && kernel != 14 && kernel != 16)
+      return set_error("woq_linear: NF4 weights run on kernels 1, 2, 7..9, 13, 14 and 16 only");
   }
   if (kernel == 0 && decode_kernel_applies(f, wbits, regime, p->scale_zero_f16x2))
     return launch_decode(f, p->scale_zero_f16x2, st);
@@ -228,7 +241,14 @@ int woq_hip_linear(const woq_hip_linear_params* p) {
     if (!decode_dq_applies(f, wbits, regime))
       return set_error("woq_linear: the dequantizing decode kernel takes M <= 64, K a multiple of the weight tile, a "
                        "power-of-two or per-channel group size and activations in the compute dtype");
-    return launch_decode_dq(f, wbits, regime, st, kernel == 10 ? 4 : kernel - 7);
+    // 7: row-blocks per workgroup and K splits by shape; 8..10: that many row-blocks, K not split
+    return launch_decode_dq(f, wbits, regime, st, kernel == 10 ? 4 : kernel - 7, kernel == 7 ? 0 : 1, &scratch);
+  }
+  if (kernel >= 13 && kernel <= 17) {
+    static const int kNtw[5] = {1, 2, 4, 2, 4}, kSplits[5] = {2, 2, 2, 4, 4};
+    if (!decode_dq_applies(f, wbits, regime))
+      return set_error("woq_linear: the dequantizing decode kernel does not take this problem");
+    return launch_decode_dq(f, wbits, regime, st, kNtw[kernel - 13], kSplits[kernel - 13], &scratch);
   }
   if (kernel == 0) {
     if (p->M <= 64)

@@ -24,6 +24,13 @@
 // 19.7 us against 13.9 us at M = 8 for the same weights).  Rows past M re-read row M - 1 and their
 // results are dropped.  The at most 64 KiB of slices (up to 32 rows; 128 KiB and four waves for
 // 33..64 rows) are reused for the cross-wave sum; up to 32 rows two workgroups fit on a CU.
+// Split K: every workgroup streams the activations of all the K tiles it owns, so a layer with few
+// output columns (few row-blocks, hence one row-block per workgroup to fill the chip) reads the
+// activations once per 16 columns -- M = 32, 14336 -> 4096: 235 MB through LDS against 29 MB of
+// weights.  With gridDim.y = S > 1 a workgroup owns more row-blocks and 1 / S of the K tiles; it
+// writes its fp32 partial tile to scratch memory, and the workgroup that arrives last at the
+// row-block set's counter (no workgroup ever waits) adds the S partial tiles in split order and runs
+// the epilogue.  The sum order is fixed, so the result does not depend on the arrival order.
 #include "woq_common.h"
 #include "woq_internal.h"
 
@@ -35,6 +42,9 @@ struct DecodeDqArgs {
   FpArgs f;
   int W;        // waves per workgroup
   int g_shift;  // log2(group size); 30 for per-channel
+  int KTs;      // K tiles per workgroup row (gridDim.y workgroups share the K tiles of a row-block set)
+  float* partial;  // split K: [gridDim.y][gridDim.x] fp32 partial tiles
+  int* counters;   // split K: [gridDim.x], zero between launches
 };
 
 template <int REGIME>
@@ -152,10 +162,13 @@ __global__ __launch_bounds__(512, 4) void woq_decode_dq_kernel(const DecodeDqArg
     }
   };
 
-  // Rounds: wave w takes K tiles w, w + W, ...; a wave with no tile left idles until the sum.
-  if (wave < KT) request(wave, 0);
+  // Rounds: wave w takes K tiles kt0 + w, kt0 + w + W, ... of this workgroup's range [kt0, kt1); a
+  // wave with no tile left idles until the sum.
+  const int kt0 = (int)blockIdx.y * a.KTs;
+  const int kt1 = kt0 + a.KTs < KT ? kt0 + a.KTs : KT;
+  if (kt0 + wave < kt1) request(kt0 + wave, 0);
 #pragma unroll 1
-  for (int kt = wave, buf = 0; kt < KT; kt += W, buf ^= 1) {
+  for (int kt = kt0 + wave, buf = 0; kt < kt1; kt += W, buf ^= 1) {
     u4 wreg[NTW];
     G4Consts<REGIME> qc4[WBITS == 4 ? NTW : 1];
     G8Consts qc8[WBITS == 8 || NF4 ? NTW : 1];
@@ -173,7 +186,7 @@ __global__ __launch_bounds__(512, 4) void woq_decode_dq_kernel(const DecodeDqArg
     }
     // The compiler does not order LDS reads after the LDS-writing loads: wait for them here.
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
-    if (kt + W < KT) request(kt + W, buf ^ 1);
+    if (kt + W < kt1) request(kt + W, buf ^ 1);
     __builtin_amdgcn_sched_barrier(0);
 
 #pragma unroll
@@ -213,12 +226,9 @@ __global__ __launch_bounds__(512, 4) void woq_decode_dq_kernel(const DecodeDqArg
                      f.out_dtype == WOQ_HIP_ACT_BF16;
   // one thread per output element, consecutive threads on consecutive columns; D[m][n] of a row
   // tile sits in lane n + 16 (m / 4), register m % 4
-  for (int idx = threadIdx.x; idx < NTW * MT * 256; idx += blockDim.x) {
+  constexpr int kTileElems = NTW * MT * 256;
+  auto wave_sum = [&](int idx) {
     const int col = idx & 15, m16 = (idx >> 4) & 15, tm = idx >> 8;
-    const int t = tm / MT, mt = tm - t * MT;
-    const int m = mt * 16 + m16;
-    const int64_t n = (nt0 + t) * kTileN + col;
-    if (m >= M || n >= f.N) continue;
     const int slot = (col + 16 * (m16 >> 2)) * 4 + (m16 & 3);
     float part[kDqMaxWaves];
 #pragma unroll
@@ -226,16 +236,56 @@ __global__ __launch_bounds__(512, 4) void woq_decode_dq_kernel(const DecodeDqArg
     float s = part[0];
 #pragma unroll
     for (int w = 1; w < kDqMaxWaves; ++w) s += part[w];
+    return s;
+  };
+  auto store = [&](int idx, float s) {
+    const int col = idx & 15, m16 = (idx >> 4) & 15, tm = idx >> 8;
+    const int t = tm / MT, mt = tm - t * MT;
+    const int m = mt * 16 + m16;
+    const int64_t n = (nt0 + t) * kTileN + col;
+    if (m >= M || n >= f.N) return;
     if (plain)
       ((uint16_t*)f.out)[(int64_t)m * f.N + n] = f32_to_bf16_bits(s);
     else
       epilogue_store<REGIME>(ep, m, n, s);
+  };
+  const int S = (int)gridDim.y;
+  if (S == 1) {
+    for (int idx = threadIdx.x; idx < kTileElems; idx += blockDim.x) store(idx, wave_sum(idx));
+    return;
   }
+  // ---- split K: partial tile to scratch, then the last workgroup of this row-block set sums ----
+  // Every access to the scratch is a relaxed atomic at device scope: such stores write through to
+  // the point where the other XCDs see them and such loads do not hit a stale cache line, so no
+  // cache-wide write-back or invalidation (what a device-scope fence costs) is needed.  Order: a
+  // thread's stores have completed at its vmcnt(0), the barrier collects all threads, then thread 0
+  // moves the counter; the last workgroup reads only after it has seen the final count.
+  float* const mine = a.partial + ((size_t)blockIdx.y * gridDim.x + blockIdx.x) * kTileElems;
+  for (int idx = threadIdx.x; idx < kTileElems; idx += blockDim.x)
+    __hip_atomic_store(mine + idx, wave_sum(idx), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+  __syncthreads();
+  __shared__ int s_last;
+  if (threadIdx.x == 0)
+    s_last = __hip_atomic_fetch_add(a.counters + blockIdx.x, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == S - 1;
+  __syncthreads();
+  if (!s_last) return;
+  const float* const all = a.partial + (size_t)blockIdx.x * kTileElems;
+  for (int idx = threadIdx.x; idx < kTileElems; idx += blockDim.x) {
+    float s = __hip_atomic_load(all + idx, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    for (int k = 1; k < S; ++k)
+      s += __hip_atomic_load(all + (size_t)k * gridDim.x * kTileElems + idx, __ATOMIC_RELAXED,
+                             __HIP_MEMORY_SCOPE_AGENT);
+    store(idx, s);
+  }
+  // the counter is back at zero for the next launch that uses it
+  if (threadIdx.x == 0) __hip_atomic_store(a.counters + blockIdx.x, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 template <int REGIME, int WBITS, int MT, int NTW, bool NF4 = false>
-static int launch_dq_cfg(DecodeDqArgs a, hipStream_t st) {
+static int launch_dq_cfg(DecodeDqArgs a, int splits, hipStream_t st) {
   using Geo = DqGeom<WBITS, MT>;
+  if (MT > 2 && splits > 1) return set_error("woq_decode_dq_kernel: split K takes at most 32 rows");
   // At most 64 KiB of activation buffers per workgroup, so that two workgroups share a CU -- unless
   // there is at most one workgroup per CU anyway: then two row tiles (17..32 rows, 16 KiB per wave for
   // 4-bit weights) take 128 KiB and keep eight waves instead of four (M = 32, 4096 -> 14336, four
@@ -243,11 +293,12 @@ static int launch_dq_cfg(DecodeDqArgs a, hipStream_t st) {
   // four row tiles (33..64 rows) a wave's two buffers are 32 KiB and one workgroup of four waves takes
   // 128 KiB.  Sixteen waves of one row tile measured no faster than eight.
   constexpr int kLdsMax = 131072;
-  const unsigned grid = (unsigned)(a.f.NT / NTW);
-  const bool alone = MT == 2 && grid <= 256;
+  const dim3 grid((unsigned)(a.f.NT / NTW), (unsigned)splits);
+  const bool alone = MT == 2 && grid.x * grid.y <= 256;
   const int lds_cap = (MT > 2 || alone) ? kLdsMax : 65536;
   const int max_w = lds_cap / (2 * Geo::SLICE);
-  a.W = (int)(a.f.KT < max_w ? a.f.KT : max_w);
+  a.KTs = (int)((a.f.KT + splits - 1) / splits);
+  a.W = a.KTs < max_w ? a.KTs : max_w;
   if (a.W > kDqMaxWaves) a.W = kDqMaxWaves;
   size_t smem = (size_t)a.W * 2 * Geo::SLICE;
   const size_t red = (size_t)NTW * MT * a.W * 64 * sizeof(f4);
@@ -276,31 +327,39 @@ bool decode_dq_applies(const FpArgs& f, int wbits, int regime) {
 }
 
 template <int REGIME, int WBITS>
-static int launch_dq_regime(const DecodeDqArgs& a, int ntw, hipStream_t st) {
+static int launch_dq_regime(const DecodeDqArgs& a, int ntw, int splits, hipStream_t st) {
   const int mt = a.f.M > 32 ? 4 : a.f.M > 16 ? 2 : 1;
   if (mt == 4) {
     // 33..64 rows: one or two row-blocks per workgroup (four would leave too few workgroups)
     if (ntw == 4) return set_error("woq_decode_dq_kernel: 33..64 rows take 1 or 2 row-blocks per workgroup");
-    return ntw == 2 ? launch_dq_cfg<REGIME, WBITS, 4, 2>(a, st) : launch_dq_cfg<REGIME, WBITS, 4, 1>(a, st);
+    return ntw == 2 ? launch_dq_cfg<REGIME, WBITS, 4, 2>(a, splits, st) : launch_dq_cfg<REGIME, WBITS, 4, 1>(a, splits, st);
   }
   const bool two_rows = mt == 2;
-  if (ntw == 4) return two_rows ? launch_dq_cfg<REGIME, WBITS, 2, 4>(a, st) : launch_dq_cfg<REGIME, WBITS, 1, 4>(a, st);
-  if (ntw == 2) return two_rows ? launch_dq_cfg<REGIME, WBITS, 2, 2>(a, st) : launch_dq_cfg<REGIME, WBITS, 1, 2>(a, st);
-  return two_rows ? launch_dq_cfg<REGIME, WBITS, 2, 1>(a, st) : launch_dq_cfg<REGIME, WBITS, 1, 1>(a, st);
+  if (ntw == 4) return two_rows ? launch_dq_cfg<REGIME, WBITS, 2, 4>(a, splits, st) : launch_dq_cfg<REGIME, WBITS, 1, 4>(a, splits, st);
+  if (ntw == 2) return two_rows ? launch_dq_cfg<REGIME, WBITS, 2, 2>(a, splits, st) : launch_dq_cfg<REGIME, WBITS, 1, 2>(a, splits, st);
+  return two_rows ? launch_dq_cfg<REGIME, WBITS, 2, 1>(a, splits, st) : launch_dq_cfg<REGIME, WBITS, 1, 1>(a, splits, st);
 }
 
 // NF4: one or two row-blocks per workgroup.
 template <int REGIME>
-static int launch_dq_nf4(const DecodeDqArgs& a, int ntw, hipStream_t st) {
+static int launch_dq_nf4(const DecodeDqArgs& a, int ntw, int splits, hipStream_t st) {
   const bool two_rows = a.f.M > 16;
-  if (ntw == 2) return two_rows ? launch_dq_cfg<REGIME, 4, 2, 2, true>(a, st) : launch_dq_cfg<REGIME, 4, 1, 2, true>(a, st);
-  return two_rows ? launch_dq_cfg<REGIME, 4, 2, 1, true>(a, st) : launch_dq_cfg<REGIME, 4, 1, 1, true>(a, st);
+  if (ntw == 2) return two_rows ? launch_dq_cfg<REGIME, 4, 2, 2, true>(a, splits, st) : launch_dq_cfg<REGIME, 4, 1, 2, true>(a, splits, st);
+  return two_rows ? launch_dq_cfg<REGIME, 4, 2, 1, true>(a, splits, st) : launch_dq_cfg<REGIME, 4, 1, 1, true>(a, splits, st);
 }
 
-int launch_decode_dq(const FpArgs& f, int wbits, int regime, hipStream_t st, int ntw) {
+int64_t decode_dq_splitk_bytes(int64_t M, int64_t NT, int splits) {
+  return (int64_t)splits * NT * (M > 16 ? 2 : 1) * 256 * (int64_t)sizeof(float);
+}
+
+int launch_decode_dq(const FpArgs& f, int wbits, int regime, hipStream_t st, int ntw, int splits,
+                     const SplitKScratch* scratch) {
   DecodeDqArgs a;
   a.f = f;
+  a.partial = scratch ? scratch->partial : nullptr;
+  a.counters = scratch ? scratch->counters : nullptr;
   a.W = 1;
+  a.KTs = (int)f.KT;
   a.g_shift = 30;
   if (f.G < f.KT * (wbits == 4 ? kTileK4 : kTileK8)) {
     a.g_shift = 0;
@@ -315,23 +374,52 @@ int launch_decode_dq(const FpArgs& f, int wbits, int regime, hipStream_t st, int
   // M = 16 / 32: 4096 -> 14336 (896 row-blocks) 14.4 / 11.4 / 10.7 us with 1 / 2 / 4, 4096 -> 6144 (384)
   // 8.5 / 7.0 / 9.7 us, 14336 -> 4096 (256) 12.9 / 15.5 / 24.5 us.  33..64 rows (four row tiles, no
   // variant with four row-blocks) have four times the activation bytes per workgroup.
+  const bool auto_ntw = ntw == 0;
   if (ntw == 0) {
     if (f.M <= 32 && !f.nf4 && f.NT >= 640 && f.NT % 4 == 0)
       ntw = 4;
     else
       ntw = (f.NT >= 384 && f.NT % 2 == 0) ? 2 : 1;
   }
+  // Few output columns and a long K: one row-block per workgroup fills the chip but re-reads the
+  // activations once per 16 columns.  Two workgroups per row-block set, each with half of the K tiles
+  // and twice the row-blocks, halve that traffic: 14336 -> 4096 (256 row-blocks), G = 128, takes
+  // 10.8 / 11.2 / 15.1 us at M = 8 / 16 / 32 against 12.7 / 13.6 / 19.1 us unsplit (four splits of four
+  // row-blocks: 13.3 / 13.4 / 17.1 us); at K = 4096 the unsplit form stays faster (4096 -> 4096, M = 16:
+  // 6.0 against 7.0 us).
+  if (splits == 0) {
+    splits = 1;
+    const bool have = scratch && scratch->partial && scratch->counters &&
+                      scratch->bytes >= decode_dq_splitk_bytes(f.M, f.NT, 2);
+    if (have && auto_ntw && f.M >= 5 && f.M <= 32 && f.K >= 8192 && f.NT <= 256) {
+      splits = 2;
+      ntw = (f.NT > 128 && f.NT % 2 == 0) ? 2 : 1;
+    }
+  }
+  if (splits != 1 && splits != 2 && splits != 4)
+    return set_error("woq_decode_dq_kernel: 1, 2 or 4 K splits, got %d", splits);
+  if (splits > 1) {
+    if (f.M > 32) return set_error("woq_decode_dq_kernel: split K takes at most 32 rows");
+    if (!a.partial || !a.counters)
+      return set_error("woq_decode_dq_kernel: split K needs the partial-tile workspace and the counter array");
+    if (scratch->bytes < decode_dq_splitk_bytes(f.M, f.NT, splits))
+      return set_error("woq_decode_dq_kernel: split K needs %lld bytes of workspace, got %lld",
+                       (long long)decode_dq_splitk_bytes(f.M, f.NT, splits), (long long)scratch->bytes);
+    if (f.NT / ntw > kSplitKCounters)
+      return set_error("woq_decode_dq_kernel: split K takes at most %d row-block sets", kSplitKCounters);
+  }
   if (f.nf4) {
     if (wbits != 4 || f.zeros) return set_error("woq_decode_dq_kernel: NF4 weights are 4-bit and symmetric");
     if (f.M > 32) return set_error("woq_decode_dq_kernel: NF4 weights take at most 32 rows");
     if (ntw == 4) return set_error("woq_decode_dq_kernel: NF4 weights take 1 or 2 row-blocks per workgroup");
-    return regime == kRegimeF16 ? launch_dq_nf4<kRegimeF16>(a, ntw, st) : launch_dq_nf4<kRegimeBF16>(a, ntw, st);
+    return regime == kRegimeF16 ? launch_dq_nf4<kRegimeF16>(a, ntw, splits, st)
+                                : launch_dq_nf4<kRegimeBF16>(a, ntw, splits, st);
   }
   if (wbits == 4)
-    return regime == kRegimeF16 ? launch_dq_regime<kRegimeF16, 4>(a, ntw, st)
-                                : launch_dq_regime<kRegimeBF16, 4>(a, ntw, st);
-  return regime == kRegimeF16 ? launch_dq_regime<kRegimeF16, 8>(a, ntw, st)
-                              : launch_dq_regime<kRegimeBF16, 8>(a, ntw, st);
+    return regime == kRegimeF16 ? launch_dq_regime<kRegimeF16, 4>(a, ntw, splits, st)
+                                : launch_dq_regime<kRegimeBF16, 4>(a, ntw, splits, st);
+  return regime == kRegimeF16 ? launch_dq_regime<kRegimeF16, 8>(a, ntw, splits, st)
+                              : launch_dq_regime<kRegimeBF16, 8>(a, ntw, splits, st);
 }
 
 }  // namespace woq

@@ -35,6 +35,17 @@ struct FpArgs {
   int nf4;  // 4-bit codes index the NF4 table instead of standing for integers (zeros == nullptr)
 };
 
+// Split-K scratch of the dequantizing decode kernel: fp32 partial tiles, and one counter per
+// row-block set that is zero between launches.
+struct SplitKScratch {
+  float* partial = nullptr;
+  int64_t bytes = 0;
+  int* counters = nullptr;
+};
+// Entries the caller's split-K counter array must have, and the largest number of K splits.
+constexpr int kSplitKCounters = 512;
+constexpr int kSplitKMax = 4;
+
 int launch_pack_weight(const void* plain, int weight_dtype, int64_t N, int64_t K, void* packed,
                        hipStream_t st);
 int launch_unpack_weight(const void* packed, int weight_dtype, int64_t N, int64_t K, void* plain,
@@ -75,9 +86,14 @@ bool decode_kernel_applies(const FpArgs& f, int wbits, int regime, const uint32_
 int launch_decode(const FpArgs& f, const uint32_t* sz, hipStream_t st);
 
 // Decode kernel with per-weight dequantization (woq_decode_dq.hip): 4- or 8-bit weights, M <= 64.
-// ntw: weight row-blocks per workgroup (1, 2 or 4), 0 = automatic
+// ntw: weight row-blocks per workgroup (1, 2 or 4), 0 = automatic;
+// splits: workgroups that share the K tiles of a row-block set (1, 2 or 4; more than 1 needs the
+// scratch and at most 32 rows), 0 = automatic (only together with ntw = 0)
 bool decode_dq_applies(const FpArgs& f, int wbits, int regime);
-int launch_decode_dq(const FpArgs& f, int wbits, int regime, hipStream_t st, int ntw = 0);
+int launch_decode_dq(const FpArgs& f, int wbits, int regime, hipStream_t st, int ntw = 0, int splits = 1,
+                     const SplitKScratch* scratch = nullptr);
+// Bytes of partial-tile scratch that `splits` workgroups per row-block set need.
+int64_t decode_dq_splitk_bytes(int64_t M, int64_t NT, int splits);
 
 // regime: 0 = fp16, 1 = bf16 (woq::Regime)
 int launch_small_m(const FpArgs& a, int wbits, int regime, hipStream_t st);

@@ -141,6 +141,21 @@ def int8_block_k(group_size, K):
     return _lib.load().woq_hip_int8_block_k(group_size, K)
 
 
+_counter_cache = {}
+
+
+def _split_k_counters(device):
+    """The zeroed counter array the split-K decode kernel needs, one per (device, stream): launches
+    on one stream run in order and every launch leaves the counters at zero."""
+    with torch.cuda.device(device):
+        key = (torch.cuda.current_device(), torch.cuda.current_stream().cuda_stream)
+    buf = _counter_cache.get(key)
+    if buf is None:
+        buf = torch.zeros(512, dtype=torch.int32, device=device)
+        _counter_cache[key] = buf
+    return buf
+
+
 def linear(
     x,
     qweight,
@@ -208,6 +223,13 @@ def linear(
     p.out_dtype = _ACT_CODE[out_dtype]
     ws = None
     wbytes = lib.woq_hip_linear_workspace_bytes(M, K, lowp_mode, act_quant_mode, group_size)
+    counters = None
+    if wbytes == 0 and lowp_mode != 3:
+        # scratch that lets the decode kernel split K across workgroups (small M, few output columns)
+        wbytes = lib.woq_hip_linear_split_k_workspace_bytes(M, N)
+        if wbytes > 0:
+            counters = _split_k_counters(x.device)
+            p.split_k_counters = counters.data_ptr()
     if wbytes > 0:
         ws = torch.empty((wbytes,), dtype=torch.uint8, device=x.device)
         p.workspace = ws.data_ptr()

@@ -30,6 +30,7 @@ EXPORTS = [
     "woq_hip_unpack_int4_zeros",
     "woq_hip_dynamic_quant",
     "woq_hip_linear_workspace_bytes",
+    "woq_hip_linear_split_k_workspace_bytes",
     "woq_hip_int8_block_k",
     "woq_hip_linear",
     "woq_hip_dequant_weight",
@@ -67,6 +68,7 @@ class LinearParams(ctypes.Structure):
         ("out_dtype", ctypes.c_int32),
         ("workspace", ctypes.c_void_p),
         ("workspace_bytes", ctypes.c_int64),
+        ("split_k_counters", ctypes.c_void_p),
         ("debug_block_sums", ctypes.c_void_p),
         ("force_kernel", ctypes.c_int32),
         ("stream", ctypes.c_void_p),
@@ -114,6 +116,8 @@ def load():
         lib.woq_hip_dynamic_quant.argtypes = [vp, i32, i64, i64, i64, i32, vp, vp, vp, vp]
         lib.woq_hip_linear_workspace_bytes.restype = i64
         lib.woq_hip_linear_workspace_bytes.argtypes = [i64, i64, ctypes.c_int32, ctypes.c_int32, i64]
+        lib.woq_hip_linear_split_k_workspace_bytes.restype = i64
+        lib.woq_hip_linear_split_k_workspace_bytes.argtypes = [i64, i64]
         lib.woq_hip_int8_block_k.restype = i64
         lib.woq_hip_int8_block_k.argtypes = [i64, i64]
         lib.woq_hip_linear.restype = i32

@@ -17,6 +17,7 @@ The context is a Python object here (the reference's is a TorchScript custom cla
 (csrc/cpu/jit/cpu/kernels/OpContext.cpp:396-400), and the ops resolve it through a registry
 of live contexts, so a stale handle raises instead of dereferencing freed memory.
 """
+import contextlib
 import ctypes
 import os
 import threading
@@ -281,13 +282,18 @@ class WoqLinearOpContext:
             else:
                 p.others[i] = None
         lib = _lib.load()
-        if x.device.index == torch.cuda.current_device():
+        with contextlib.nullcontext() if x.device.index == torch.cuda.current_device() else torch.cuda.device(x.device):
             p.stream = torch.cuda.current_stream().cuda_stream
+            ws = None
+            if M <= 32 and K >= 8192 and N <= 4096:
+                # long K, few output columns: scratch with which the decode kernel may share K between
+                # workgroups (the library decides), and the zeroed counters of this stream
+                ws = torch.empty(lib.woq_hip_linear_split_k_workspace_bytes(M, N), dtype=torch.uint8, device=x.device)
+                p.workspace, p.workspace_bytes = ws.data_ptr(), ws.numel()
+                p.split_k_counters = _kernels._split_k_counters(x.device).data_ptr()
+            else:
+                p.workspace, p.workspace_bytes, p.split_k_counters = None, 0, None
             rc = lib.woq_hip_linear(ctypes.byref(p))
-        else:
-            with torch.cuda.device(x.device):
-                p.stream = torch.cuda.current_stream().cuda_stream
-                rc = lib.woq_hip_linear(ctypes.byref(p))
         _lib.check(rc, "woq_linear")
         return out
 

@@ -351,6 +351,116 @@ def test_dequantizing_decode_kernel_four_row_tiles_int8_weights_and_rejections(c
     _check_fp(nf4, O.LOWP_BF16, label="nf4 M=40 takes the small-M kernel")
 
 
+SPLIT_K_CODES = {13: (1, 2), 14: (2, 2), 15: (4, 2), 16: (2, 4), 17: (4, 4)}  # (row-blocks per workgroup, K splits)
+
+
+@pytest.mark.parametrize(
+    "M,K,N,G,bias",
+    [
+        (5, 1024, 64, 128, False),  # eight K tiles: two per workgroup with four splits
+        (16, 4096, 1024, 32, True),
+        (13, 1152, 96, -1, False),  # nine K tiles: with four splits the last workgroup has none
+        (16, 128, 64, 128, False),  # a single K tile: every split but the first is empty
+        (32, 2048, 64, 32, True),  # two row tiles
+        (20, 1024, 96, 128, True),
+        (3, 256, 128, 256, True),  # bf16 compute forced by lowp NONE
+    ],
+)
+@pytest.mark.parametrize("kernel", sorted(SPLIT_K_CODES))
+def test_dequantizing_decode_kernel_split_k(cuda, M, K, N, G, bias, kernel):
+    """K shared between 2 or 4 workgroups; the one that finishes last adds the partial tiles."""
+    if (N // 16) % SPLIT_K_CODES[kernel][0]:
+        pytest.skip("row-blocks per workgroup must divide N / 16")
+    case = _synthetic().make_int4_case(44, M, K, N, G, bias=bias)
+    lowp = O.LOWP_NONE if M < 5 else O.LOWP_BF16
+    _check_fp(case, lowp, force_kernel=kernel, label=f"decode dq split K M={M} K={K} N={N} G={G} kernel={kernel}")
+
+
+@pytest.mark.parametrize("M", [2, 16, 27])
+@pytest.mark.parametrize("kernel", [13, 14, 17])
+def test_dequantizing_decode_kernel_split_k_int8_weights(cuda, M, kernel):
+    case = _synthetic().make_int8_case(45, M, 704, 128)  # 11 K tiles
+    lowp = O.LOWP_NONE if M < 5 else O.LOWP_BF16
+    _check_fp(case, lowp, force_kernel=kernel, label=f"decode dq split K int8 weights M={M} kernel={kernel}")
+
+
+def test_dequantizing_decode_kernel_split_k_nf4_and_fp16(cuda):
+    syn = _synthetic()
+    nf4 = syn.make_nf4_case(46, 12, 1024, 96, 64)
+    for kernel in (13, 14, 16):
+        _check_fp(nf4, O.LOWP_BF16, force_kernel=kernel, label=f"nf4 split K kernel={kernel}")
+    with pytest.raises(RuntimeError, match="NF4"):
+        make_context(nf4, O.LOWP_BF16).run(nf4["x"].cuda(), force_kernel=15)
+    case = syn.make_int4_case(47, 11, 1024, 96, 32, bias=True, scale_dtype=torch.float16)
+    case["x"] = case["x"].to(torch.float16)
+    ctx = make_context(case, O.LOWP_FP16)
+    want = to_np_f32(ctx.run(case["x"].cuda(), force_kernel=8))
+    for kernel in (13, 14, 16):
+        got = to_np_f32(ctx.run(case["x"].cuda(), force_kernel=kernel))
+        assert rel_l2(got, want) <= 1e-3, kernel
+
+
+@pytest.mark.parametrize("M,K,N,G", [(16, 8192, 4096, 128), (8, 14336, 512, 128), (32, 8192, 2048, 32)])
+def test_dequantizing_decode_kernel_splits_k_by_itself_for_long_k(cuda, M, K, N, G):
+    """Few output columns and K >= 8192: the automatic choice shares K between two workgroups.  The
+    result must not depend on which workgroup finishes last (the partial tiles are added in split
+    order), the counters are zero again after every call, and a side stream has counters of its own."""
+    case = _synthetic().make_int4_case(48, M, K, N, G, bias=True)
+    cols = list(range(0, N, 37))
+    _check_fp(case, O.LOWP_BF16, cols=cols, label=f"decode dq automatic split K M={M} K={K} N={N} G={G}")
+    ctx = make_context(case, O.LOWP_BF16)
+    x = case["x"].cuda()
+    first = ctx.run(x)
+    # another summation order shows in the fp32 sums: the split form ran
+    assert not torch.equal(ctx.run(x, out_fp32=True), ctx.run(x, out_fp32=True, force_kernel=8))
+    assert rel_l2(to_np_f32(first), to_np_f32(ctx.run(x, force_kernel=8))) <= 1e-3
+    for _ in range(5):
+        assert torch.equal(ctx.run(x), first)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        other = ctx.run(x)
+    side.synchronize()
+    assert torch.equal(other, first)
+    torch.cuda.synchronize()
+    from ipex_amd import _kernels as kmod
+
+    assert len(kmod._counter_cache) >= 2
+    assert all(int(buf.abs().sum()) == 0 for buf in kmod._counter_cache.values())
+
+
+def test_dequantizing_decode_kernel_split_k_needs_scratch(cuda):
+    """Through the C ABI without the scratch: forced split-K codes are refused, code 0 runs unsplit."""
+    import ctypes
+
+    from ipex_amd import _lib
+
+    lib = _lib.load()
+    case = _synthetic().make_int4_case(49, 16, 8192, 256, 128)
+    ctx = make_context(case, O.LOWP_BF16)
+    x = case["x"].cuda()
+    out = torch.empty(16, 256, dtype=torch.bfloat16, device="cuda")
+    p = _lib.LinearParams()
+    p.struct_size = ctypes.sizeof(_lib.LinearParams)
+    p.x, p.x_dtype, p.M, p.K, p.N = x.data_ptr(), _lib.ACT_BF16, 16, 8192, 256
+    p.qweight, p.weight_dtype = ctx.at_weight_.data_ptr(), 2
+    p.scales_f32, p.scales_f16, p.scales_bf16 = (t.data_ptr() for t in ctx.scales_list_)
+    p.zeros_u8 = ctx.zeros_u8_.data_ptr()
+    p.group_size, p.lowp_mode, p.act_quant_mode = 128, 2, -1
+    p.out, p.out_dtype = out.data_ptr(), _lib.ACT_BF16
+    p.stream = torch.cuda.current_stream().cuda_stream
+    p.force_kernel = 14
+    assert lib.woq_hip_linear(ctypes.byref(p)) != 0
+    assert b"split K needs" in lib.woq_hip_last_error()
+    p.force_kernel = 0
+    assert lib.woq_hip_linear(ctypes.byref(p)) == 0
+    torch.cuda.synchronize()
+    assert torch.equal(out, ctx.run(x, force_kernel=8))
+    assert lib.woq_hip_linear_split_k_workspace_bytes(16, 256) == 4 * 16 * 1024
+    assert lib.woq_hip_linear_split_k_workspace_bytes(17, 256) == 4 * 16 * 2048
+    assert lib.woq_hip_linear_split_k_workspace_bytes(33, 256) == 0
+
+
 def test_dequantizing_decode_kernel_fp16_regime_and_symmetric(cuda):
     """fp16 regime with a group size the integer-weight decode kernel does not take, and weights
     without zero points."""
