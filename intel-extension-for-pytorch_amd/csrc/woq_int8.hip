@@ -211,6 +211,10 @@ static int launch_quant_impl(const void* x, int x_dtype, int64_t M, int64_t K, i
   if (qbk <= 0) qbk = K;
   const int64_t Kc = (K + qbk - 1) / qbk;
   const int64_t groups = num_quant_groups(M, Kc, mode);
+  // one pass over whole rows where a row fits a wave's registers; otherwise statistics, then quantization
+  if (act_quant_rows_applies(x, x_dtype, K, q, ldq, qbk, quant_a_per_m(mode), quant_a_per_k(mode)))
+    return launch_act_quant_rows(x, x_dtype, M, K, ldq, qbk, Kc, quant_a_per_k(mode), quant_a_is_sym(mode), q, scales,
+                                 zps, permute, offset128, st);
   if (quant_a_per_m(mode)) {
     act_stats_kernel<<<(unsigned)groups, 256, 0, st>>>(x, x_dtype, M, K, qbk, Kc, mode, scales, zps);
     if (int rc = check_launch("act_stats_kernel")) return rc;

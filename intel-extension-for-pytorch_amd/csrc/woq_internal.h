@@ -132,6 +132,13 @@ struct Int8Args {
 bool gemm_w4i8_applies(const Int8Args& a, int64_t block_k, int64_t qbk, bool per_k, bool asym);
 int launch_gemm_w4i8(const Int8Args& a, const uint8_t* xq, int64_t ldq, const float* sa, int64_t sa_m_stride,
                      int64_t sa_k_stride, int64_t qbk, hipStream_t st);
+// One-pass quantization of whole rows (woq_act_quant.hip): 16-bit activations, one scale per row or per
+// (row, K block), padded rows of at most 16384 elements.  Same bytes and scales as the two-kernel form.
+bool act_quant_rows_applies(const void* x, int x_dtype, int64_t K, const void* q, int64_t ldq, int64_t qbk,
+                            bool per_m, bool per_k);
+int launch_act_quant_rows(const void* x, int x_dtype, int64_t M, int64_t K, int64_t ldq, int64_t qbk, int64_t Kc,
+                          bool per_k, bool sym, void* q, float* scales, int32_t* zps, int permute, int offset128,
+                          hipStream_t st);
 int launch_dynamic_quant(const void* x, int x_dtype, int64_t M, int64_t K, int64_t ldq, int64_t qbk,
                          int mode, void* q, float* scales, int32_t* zps, hipStream_t st);
 int launch_int8_linear(const Int8Args& a, hipStream_t st);

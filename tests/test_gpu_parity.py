@@ -618,6 +618,35 @@ def test_dynamic_quant_bit_exact(cuda, mode, M, K):
         assert np.array_equal(zp.cpu().numpy().reshape(-1), zp_ref.reshape(-1))
 
 
+@pytest.mark.parametrize("mode", [2, 3, 6, 7])
+@pytest.mark.parametrize(
+    "M,K,block,dtype",
+    [
+        (9, 8192, 64, torch.bfloat16),  # sixteen 512-element chunks per row
+        (5, 14336, 512, torch.bfloat16),  # thirty-two chunks, a block per chunk
+        (6, 1000, 32, torch.float16),  # K not a multiple of the block: a partial last block
+        (3, 4096, 256, torch.float16),
+        (4, 2048, 1024, torch.bfloat16),  # blocks wider than a chunk: the two-kernel form
+        (4, 24576, 128, torch.bfloat16),  # rows too long for a wave's registers: the two-kernel form
+        (7, 768, 128, torch.float32),  # fp32 activations: the two-kernel form
+    ],
+)
+def test_dynamic_quant_rows_bit_exact(cuda, mode, M, K, block, dtype):
+    """Per-row and per-(row, K block) scales over the row lengths, block sizes and activation types
+    that select the one-pass kernel or the two-kernel form; one row is all zeros (scale 0)."""
+    k = _kernels()
+    x = torch.randn(M, K, generator=torch.Generator().manual_seed(M * 7 + K + mode)) * 3.0
+    x[1] = 0.0
+    x[0, :5] = torch.tensor([0.5, -0.5, 1.5, 2.5, 1e-3])
+    x = x.to(dtype)
+    q, s, zp = k.dynamic_quant(x.to(cuda), block, mode)
+    q_ref, s_ref, zp_ref = O.dynamic_quantize_per_block(x.float().numpy(), block, mode)
+    assert np.array_equal(s.cpu().numpy().reshape(-1), s_ref.reshape(-1))
+    assert np.array_equal(q.cpu().numpy(), q_ref)
+    if mode < 4:
+        assert np.array_equal(zp.cpu().numpy().reshape(-1), zp_ref.reshape(-1))
+
+
 def test_dynamic_quant_all_bf16_patterns(cuda):
     k = _kernels()
     bits = torch.arange(65536, dtype=torch.int32).to(torch.int16)
