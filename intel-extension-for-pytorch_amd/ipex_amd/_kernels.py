@@ -146,13 +146,17 @@ _counter_cache = {}
 
 def _split_k_counters(device):
     """The zeroed counter array the split-K decode kernel needs, one per (device, stream): launches
-    on one stream run in order and every launch leaves the counters at zero."""
+    on one stream run in order and every launch leaves the counters at zero.  None while a HIP graph
+    is being captured on a stream that has no array yet (an allocation made during capture belongs to
+    the graph's memory pool and must not outlive it): the call then runs without splitting K."""
     with torch.cuda.device(device):
         key = (torch.cuda.current_device(), torch.cuda.current_stream().cuda_stream)
-    buf = _counter_cache.get(key)
-    if buf is None:
-        buf = torch.zeros(512, dtype=torch.int32, device=device)
-        _counter_cache[key] = buf
+        buf = _counter_cache.get(key)
+        if buf is None:
+            if torch.cuda.is_current_stream_capturing():
+                return None
+            buf = torch.zeros(512, dtype=torch.int32, device=device)
+            _counter_cache[key] = buf
     return buf
 
 
@@ -227,9 +231,11 @@ def linear(
     if wbytes == 0 and lowp_mode != 3:
         # scratch that lets the decode kernel split K across workgroups (small M, few output columns)
         wbytes = lib.woq_hip_linear_split_k_workspace_bytes(M, N)
-        if wbytes > 0:
-            counters = _split_k_counters(x.device)
+        counters = _split_k_counters(x.device) if wbytes > 0 else None
+        if counters is not None:
             p.split_k_counters = counters.data_ptr()
+        else:
+            wbytes = 0
     if wbytes > 0:
         ws = torch.empty((wbytes,), dtype=torch.uint8, device=x.device)
         p.workspace = ws.data_ptr()

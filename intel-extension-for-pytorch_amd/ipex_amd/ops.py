@@ -284,13 +284,15 @@ class WoqLinearOpContext:
         lib = _lib.load()
         with contextlib.nullcontext() if x.device.index == torch.cuda.current_device() else torch.cuda.device(x.device):
             p.stream = torch.cuda.current_stream().cuda_stream
-            ws = None
+            ws = counters = None
             if M <= 32 and K >= 8192 and N <= 4096:
                 # long K, few output columns: scratch with which the decode kernel may share K between
                 # workgroups (the library decides), and the zeroed counters of this stream
+                counters = _kernels._split_k_counters(x.device)
+            if counters is not None:
                 ws = torch.empty(lib.woq_hip_linear_split_k_workspace_bytes(M, N), dtype=torch.uint8, device=x.device)
                 p.workspace, p.workspace_bytes = ws.data_ptr(), ws.numel()
-                p.split_k_counters = _kernels._split_k_counters(x.device).data_ptr()
+                p.split_k_counters = counters.data_ptr()
             else:
                 p.workspace, p.workspace_bytes, p.split_k_counters = None, 0, None
             rc = lib.woq_hip_linear(ctypes.byref(p))
