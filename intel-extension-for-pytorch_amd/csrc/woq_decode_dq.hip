@@ -79,8 +79,13 @@ struct G8Consts {
 };
 
 // NF4: the 4-bit codes index the NormalFloat4 table (a copy in LDS) and there are no zero points.
-template <int REGIME, int WBITS, int MT, int NTW, bool NF4>
+// XCONV (fp16 regime, one row tile): the activations are bf16 and become fp16 on the way in, as the
+// reference's fp16 kernel converts them per K block (csrc/cpu/aten/utils/woq.h:3076-3079) -- the common
+// case of a bf16 model under lowp_mode BF16 with fewer than five rows.  The rows then travel through
+// registers (16-byte loads, conversion, ds_write to the same swizzled places) instead of the LDS DMA.
+template <int REGIME, int WBITS, int MT, int NTW, bool NF4, bool XCONV>
 __global__ __launch_bounds__(512, 4) void woq_decode_dq_kernel(const DecodeDqArgs a) {
+  static_assert(!XCONV || (REGIME == kRegimeF16 && MT == 1), "bf16 -> fp16 rows: fp16 regime, one row tile");
   using Geo = DqGeom<WBITS, MT>;
   constexpr int TK = Geo::TK, NJ = Geo::NJ, NX = Geo::NX, SLICE = Geo::SLICE;
   static_assert(!NF4 || WBITS == 4, "NF4 codes are 4 bits wide");
@@ -140,6 +145,7 @@ __global__ __launch_bounds__(512, 4) void woq_decode_dq_kernel(const DecodeDqArg
   u4 wnext[NTW];
   uint16_t snext[NTW];
   uint8_t znext[NTW];
+  u4 xnext[XCONV ? NX : 1];  // XCONV: the next round's activation rows, still bf16
   // every request of one round: activations into LDS buffer `buf`, tiles and parameters into registers
   auto request = [&](int kt, int buf) {
     // uniform base + 32-bit offset; instructions whose rows lie entirely past M are skipped
@@ -147,9 +153,13 @@ __global__ __launch_bounds__(512, 4) void woq_decode_dq_kernel(const DecodeDqArg
     const uint32_t ko = (uint32_t)kt * Geo::ROWB;
 #pragma unroll
     for (int i = 0; i < NX; ++i)
-      if (Geo::RPI * i < M)
-        __builtin_amdgcn_global_load_lds((dq_global_ptr_t)((const uint8_t*)f.x + (uint32_t)(xoff[i] + ko)),
-                                         (dq_lds_ptr_t)(sx + buf * SLICE + i * 1024), 16, 0, 0);
+      if (Geo::RPI * i < M) {
+        if constexpr (XCONV)
+          xnext[i] = *(const u4*)((const uint8_t*)f.x + (uint32_t)(xoff[i] + ko));
+        else
+          __builtin_amdgcn_global_load_lds((dq_global_ptr_t)((const uint8_t*)f.x + (uint32_t)(xoff[i] + ko)),
+                                           (dq_lds_ptr_t)(sx + buf * SLICE + i * 1024), 16, 0, 0);
+      }
     int g = (kt * TK + c * (TK / 4)) >> a.g_shift;
     g = g < KG ? g : KG - 1;
     const uint32_t qoff = (uint32_t)(g * kTileN + r);
@@ -186,6 +196,21 @@ __global__ __launch_bounds__(512, 4) void woq_decode_dq_kernel(const DecodeDqArg
     }
     // The compiler does not order LDS reads after the LDS-writing loads: wait for them here.
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+    if constexpr (XCONV) {
+      // bf16 -> fp16 (exact inside the fp16 range, round to nearest even below it) into this wave's
+      // slice; a wave's LDS accesses complete in order, so the fragment reads below see the rows
+#pragma unroll
+      for (int i = 0; i < NX; ++i)
+        if (Geo::RPI * i < M) {
+          u4 h;
+#pragma unroll
+          for (int v = 0; v < 4; ++v) {
+            const float lo = bitcast<float>(xnext[i][v] << 16), hi = bitcast<float>(xnext[i][v] & 0xFFFF0000u);
+            h[v] = (uint32_t)f32_to_f16_bits(lo) | ((uint32_t)f32_to_f16_bits(hi) << 16);
+          }
+          *(u4*)(sx + buf * SLICE + i * 1024 + lane * 16) = h;
+        }
+    }
     if (kt + W < kt1) request(kt + W, buf ^ 1);
     __builtin_amdgcn_sched_barrier(0);
 
@@ -282,7 +307,7 @@ __global__ __launch_bounds__(512, 4) void woq_decode_dq_kernel(const DecodeDqArg
   if (threadIdx.x == 0) __hip_atomic_store(a.counters + blockIdx.x, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-template <int REGIME, int WBITS, int MT, int NTW, bool NF4 = false>
+template <int REGIME, int WBITS, int MT, int NTW, bool NF4 = false, bool XCONV = false>
 static int launch_dq_cfg(DecodeDqArgs a, int splits, hipStream_t st) {
   using Geo = DqGeom<WBITS, MT>;
   if (MT > 2 && splits > 1) return set_error("woq_decode_dq_kernel: split K takes at most 32 rows");
@@ -303,7 +328,7 @@ static int launch_dq_cfg(DecodeDqArgs a, int splits, hipStream_t st) {
   size_t smem = (size_t)a.W * 2 * Geo::SLICE;
   const size_t red = (size_t)NTW * MT * a.W * 64 * sizeof(f4);
   if (red > smem) smem = red;
-  auto kern = woq_decode_dq_kernel<REGIME, WBITS, MT, NTW, NF4>;
+  auto kern = woq_decode_dq_kernel<REGIME, WBITS, MT, NTW, NF4, XCONV>;
   if (MT >= 2) {
     // more than 64 KiB of LDS per workgroup needs an opt-in (once per kernel and process)
     static const hipError_t lds_optin =
@@ -315,12 +340,14 @@ static int launch_dq_cfg(DecodeDqArgs a, int splits, hipStream_t st) {
   return check_launch("woq_decode_dq_kernel");
 }
 
-// At most 64 rows already in the compute dtype, whole K tiles, and (4-bit) a group size whose
+// At most 64 rows already in the compute dtype (or up to 16 bf16 rows for fp16 compute), whole K tiles, and (4-bit) a group size whose
 // boundaries never split a lane's 32 consecutive K values (8-bit: 16).
 bool decode_dq_applies(const FpArgs& f, int wbits, int regime) {
   const int want = regime == kRegimeF16 ? WOQ_HIP_ACT_FP16 : WOQ_HIP_ACT_BF16;
   const int tk = wbits == 4 ? kTileK4 : kTileK8;
-  if (f.M > 64 || f.x_dtype != want || ((uintptr_t)f.x & 15) != 0) return false;
+  // bf16 rows under the fp16 regime are converted on the way in, up to one row tile
+  const bool converts = regime == kRegimeF16 && f.x_dtype == WOQ_HIP_ACT_BF16 && f.M <= 16;
+  if (f.M > 64 || (f.x_dtype != want && !converts) || ((uintptr_t)f.x & 15) != 0) return false;
   if (f.K % tk != 0 || f.M * f.K * 2 >= (int64_t)1 << 31) return false;
   if (f.G >= f.KT * tk) return true;
   return f.G >= (wbits == 4 ? 32 : 16) && (f.G & (f.G - 1)) == 0;
@@ -329,6 +356,13 @@ bool decode_dq_applies(const FpArgs& f, int wbits, int regime) {
 template <int REGIME, int WBITS>
 static int launch_dq_regime(const DecodeDqArgs& a, int ntw, int splits, hipStream_t st) {
   const int mt = a.f.M > 32 ? 4 : a.f.M > 16 ? 2 : 1;
+  if constexpr (REGIME == kRegimeF16) {
+    if (a.f.x_dtype == WOQ_HIP_ACT_BF16) {  // one row tile, rows converted to fp16 on the way in
+      if (ntw == 4) return launch_dq_cfg<REGIME, WBITS, 1, 4, false, true>(a, splits, st);
+      if (ntw == 2) return launch_dq_cfg<REGIME, WBITS, 1, 2, false, true>(a, splits, st);
+      return launch_dq_cfg<REGIME, WBITS, 1, 1, false, true>(a, splits, st);
+    }
+  }
   if (mt == 4) {
     // 33..64 rows: one or two row-blocks per workgroup (four would leave too few workgroups)
     if (ntw == 4) return set_error("woq_decode_dq_kernel: 33..64 rows take 1 or 2 row-blocks per workgroup");
@@ -343,6 +377,11 @@ static int launch_dq_regime(const DecodeDqArgs& a, int ntw, int splits, hipStrea
 // NF4: one or two row-blocks per workgroup.
 template <int REGIME>
 static int launch_dq_nf4(const DecodeDqArgs& a, int ntw, int splits, hipStream_t st) {
+  if constexpr (REGIME == kRegimeF16) {
+    if (a.f.x_dtype == WOQ_HIP_ACT_BF16)
+      return ntw == 2 ? launch_dq_cfg<REGIME, 4, 1, 2, true, true>(a, splits, st)
+                      : launch_dq_cfg<REGIME, 4, 1, 1, true, true>(a, splits, st);
+  }
   const bool two_rows = a.f.M > 16;
   if (ntw == 2) return two_rows ? launch_dq_cfg<REGIME, 4, 2, 2, true>(a, splits, st) : launch_dq_cfg<REGIME, 4, 1, 2, true>(a, splits, st);
   return two_rows ? launch_dq_cfg<REGIME, 4, 2, 1, true>(a, splits, st) : launch_dq_cfg<REGIME, 4, 1, 1, true>(a, splits, st);

@@ -351,6 +351,36 @@ def test_dequantizing_decode_kernel_four_row_tiles_int8_weights_and_rejections(c
     _check_fp(nf4, O.LOWP_BF16, label="nf4 M=40 takes the small-M kernel")
 
 
+@pytest.mark.parametrize(
+    "M,K,N,G,bias",
+    [(1, 1024, 64, 32, False), (2, 4096, 1024, 64, True), (4, 1152, 96, -1, True), (3, 512, 128, 32, False),
+     (4, 256, 64, 256, True)],
+)
+@pytest.mark.parametrize("kernel", [0, 8, 9, 10, 13, 14])
+def test_dequantizing_decode_kernel_bf16_rows_under_fp16_compute(cuda, M, K, N, G, bias, kernel):
+    """lowp_mode BF16 with fewer than five bf16 rows computes in fp16 (the reference converts the rows
+    per K block): group sizes the integer-weight decode kernel does not take go through this kernel,
+    which converts the rows on the way into LDS."""
+    ntw = {0: 1, 8: 1, 9: 2, 10: 4, 13: 1, 14: 2}[kernel]
+    if (N // 16) % ntw:
+        pytest.skip("row-blocks per workgroup must divide N / 16")
+    case = _synthetic().make_int4_case(54, M, K, N, G, bias=bias)
+    _check_fp(case, O.LOWP_BF16, force_kernel=kernel, label=f"decode dq bf16 rows, fp16 compute M={M} K={K} N={N} G={G} kernel={kernel}")
+
+
+def test_dequantizing_decode_kernel_bf16_rows_under_fp16_compute_other_weights(cuda):
+    syn = _synthetic()
+    for M in (1, 4):
+        _check_fp(syn.make_int8_case(55, M, 704, 128), O.LOWP_BF16, force_kernel=7, label=f"int8 weights M={M}")
+        _check_fp(syn.make_nf4_case(56, M, 1024, 96, 64), O.LOWP_BF16, force_kernel=7, label=f"nf4 M={M}")
+    # lowp_mode FP16 with bf16 activations: fp16 compute at any M; one row tile converts in the kernel
+    case = syn.make_int4_case(57, 13, 1024, 96, 32, bias=True)
+    _check_fp(case, O.LOWP_FP16, force_kernel=7, label="lowp FP16, bf16 rows, M=13")
+    with pytest.raises(RuntimeError, match="dequantizing decode kernel"):
+        big = syn.make_int4_case(58, 20, 1024, 96, 32)
+        make_context(big, O.LOWP_FP16).run(big["x"].cuda(), force_kernel=7)
+
+
 SPLIT_K_CODES = {13: (1, 2), 14: (2, 2), 15: (4, 2), 16: (2, 4), 17: (4, 4)}  # (row-blocks per workgroup, K splits)
 
 
