@@ -310,9 +310,12 @@ __global__ __launch_bounds__(256, 3) void woq_gemm_w4i8_kernel(const W4I8Args a)
 
 // 4-bit integer codes, symmetric activation scales per tensor or per row, K blocks of 128 that are
 // whole weight tiles, and a group size of 128 * 2^s (or one group), so that a K tile has one scale.
+// More than 16 rows: with a single 64-row tile the kernel still beats the small-M one (4096 -> 14336,
+// per-row scales, M = 32 / 48 / 64: 31 / 34 / 36 us against 50 / 157 / 162 us); up to 16 rows that one
+// is faster (27-29 us).
 bool gemm_w4i8_applies(const Int8Args& a, int64_t block_k, int64_t qbk, bool per_k, bool asym) {
   if (a.wbits != 4 || a.nf4 || asym || a.debug_block_sums) return false;
-  if (block_k != 128 || a.K % 128 != 0 || a.M <= 64) return false;
+  if (block_k != 128 || a.K % 128 != 0 || a.M <= 16) return false;
   if (a.group_size > 0 && (a.G % 128 != 0 || ((a.G / 128) & (a.G / 128 - 1)) != 0)) return false;
   // activation K blocks of 128 * 2^s as well (they follow the group size, or the K block)
   if (per_k && (qbk % 128 != 0 || ((qbk / 128) & (qbk / 128 - 1)) != 0)) return false;
