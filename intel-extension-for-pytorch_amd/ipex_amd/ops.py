@@ -332,6 +332,18 @@ class WoqLinearOpContext:
             w = self._cached_bf16_weight()
             b = self.at_bias_.to(torch.bfloat16) if self.at_bias_ is not None else None
             return torch.nn.functional.linear(x.to(torch.bfloat16), w, b).to(x.dtype)
+        if (
+            self.lowp_mode_ == _lib.LOWP_FP16
+            and x.dtype == torch.bfloat16
+            and M > 16
+            and fusion == _lib.FUSE_NONE
+            and not kw
+        ):
+            # fp16 compute on bf16 activations beyond one row tile: the reference converts the rows to
+            # fp16 and casts the fp16 result back (csrc/cpu/aten/utils/woq.h:3076-3085); doing the two
+            # casts around the call reaches the kernels that want rows in the compute dtype
+            # (M = 2048, 4096 -> 14336: 430 us through the converting general kernel otherwise)
+            return self.run(x.to(torch.float16)).to(torch.bfloat16)
         if not kw and self.lowp_mode_ != _lib.LOWP_INT8 and x.dtype in _kernels._ACT_CODE and x.is_cuda:
             return self._run_planned(x, M, fusion, others)
         return _kernels.linear(

@@ -535,6 +535,22 @@ def test_lowp_none_and_fp16_modes(cuda):
     _check_fp(case, O.LOWP_FP16, label="lowp FP16 tiled")
 
 
+@pytest.mark.parametrize("M,bias", [(20, True), (70, False), (200, True)])
+def test_lowp_fp16_with_bf16_rows_beyond_one_row_tile(cuda, M, bias):
+    """The op layer casts the rows to fp16 and the fp16 result back, as the reference's fp16 kernel does;
+    the converting general kernel (reached through force_kernel) must agree."""
+    case = _synthetic().make_int4_case(19, M, 1024, 272, 128, bias=bias)
+    ctx = make_context(case, O.LOWP_FP16)
+    x = case["x"].cuda()
+    y = ctx.run(x)
+    assert y.dtype == torch.bfloat16
+    c = case_np(case)
+    _, y_ref = O.woq_linear_ref(c["x"], "bf16", c["qw"], 272, 1024, O._round_to(c["scales"], "fp16"), c["zps"],
+                                c["bias"], 2, 128, "fp16")
+    assert rel_l2(to_np_f32(y), y_ref) <= REL_L2_OUT
+    assert rel_l2(to_np_f32(y), to_np_f32(ctx.run(x, force_kernel=0))) <= 1e-3
+
+
 def test_symmetric_int4(cuda):
     case = _synthetic().make_int4_case(18, 7, 512, 96, 128)
     case["zeros"] = None
