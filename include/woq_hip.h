@@ -213,11 +213,13 @@ typedef struct woq_hip_linear_params {
   int32_t* debug_block_sums;
 
   /* force_kernel: 0 = automatic; 1 = small-M streaming kernel; 2 = tiled MFMA GEMM (any shape);
-   * 3 = 4-bit prefill GEMM (K % 128 == 0, power-of-two or per-channel groups, x in the compute dtype),
+   * 3 = prefill GEMM with register-resident dequantization (4-bit integer weights, or 8-bit weights with
+   * groups of at least 128; K % 128 == 0, power-of-two or per-channel groups, x in the compute dtype),
    * workgroup shape by cost model; 4 / 5 / 6 = the same kernel with 448 / 256 / 128 columns per workgroup;
    * 7 = dequantizing decode kernel (M <= 64, K % 128 == 0 for 4-bit and K % 64 == 0 for 8-bit weights, x in the
    * compute dtype), 8 / 9 / 10 = the same with one / two / four weight row-blocks per workgroup;
-   * 11 / 12 = the 4-bit prefill GEMM with 256 rows x 192 columns / 64 rows x 128 columns per workgroup;
+   * 11 / 12 = the same prefill GEMM with 256 rows x 192 columns / 64 rows x 128 columns per workgroup
+   * (8-bit weights: 5, 6 and 12 only);
    * 13..17 = the dequantizing decode kernel (M <= 32) with (row-blocks per workgroup, K splits) =
    * (1, 2), (2, 2), (4, 2), (2, 4), (4, 4): needs workspace and split_k_counters.
    * NF4 weights: 0, 1, 2, 7, 8, 9, 13, 14, 16 only */

@@ -260,10 +260,11 @@ int woq_hip_linear(const woq_hip_linear_params* p) {
   const int w4_shape = kernel == 4 ? 7 : kernel == 5 ? 4 : kernel == 6 ? 2 : kernel == 11 ? 163 : kernel == 12 ? 42 : 0;
   if ((kernel >= 4 && kernel <= 6) || kernel == 11 || kernel == 12) kernel = 3;
   if (kernel == 3 && !gemm_w4_applies(f, wbits, regime))
-    return set_error("woq_linear: the 4-bit prefill kernel takes 4-bit weights, K %% 128 == 0, a power-of-two or "
-                     "per-channel group size and activations in the compute dtype");
+    return set_error("woq_linear: the prefill kernel takes 4-bit integer weights (or 8-bit ones with groups of at "
+                     "least 128), K %% 128 == 0, a power-of-two or per-channel group size and activations in the "
+                     "compute dtype");
   if (kernel == 1) return launch_small_m(f, wbits, regime, st);
-  return kernel == 3 ? launch_gemm_w4(f, regime, st, w4_shape) : launch_gemm(f, wbits, regime, st);
+  return kernel == 3 ? launch_gemm_w4(f, wbits, regime, st, w4_shape) : launch_gemm(f, wbits, regime, st);
 }
 
 int woq_hip_dequant_weight(const void* qweight, int weight_dtype, int64_t N, int64_t K, const float* scales_f32,

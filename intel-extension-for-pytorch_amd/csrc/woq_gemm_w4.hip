@@ -22,7 +22,12 @@
 //     into a per-wave LDS stage two steps ahead and are read into registers during the last K
 //     sub-step of the step before;
 //   * the step is software pipelined over its 4 K sub-steps and NTW row-blocks: while the MT MFMAs
-//     of one (sub-step, row-block) run, the VALU dequantizes the dword of the next one.
+//     of one (sub-step, row-block) run, the VALU dequantizes the dword of the next one;
+//   * 8-bit weights (WBITS 8; per-channel or groups of at least 128) run through the same loop: a K
+//     step of 128 is then two packed tiles per row-block (a tile is 16 rows x 64 bytes), sub-step j
+//     takes dwords 2 (j % 2), 2 (j % 2) + 1 of tile j / 2 -- the K offsets 64 (j / 2) + 16 c + 8 (j % 2)
+//     of lane column c -- and the A fragment is read from the matching 16-byte chunk; 20 VALU
+//     instructions per B operand (byte -> float, fma, pack) against 17.
 #include "woq_common.h"
 #include "woq_internal.h"
 
@@ -37,8 +42,8 @@ struct G4Shape {
   static constexpr int BN = G4_WAVES * NTW * kTileN;    // columns per workgroup
   static constexpr int XBYTES = BM * kTileK4 * 2;       // one activation buffer
   static constexpr int XLOADS = XBYTES / (G4_WAVES * 1024);  // LDS loads per wave and buffer
-  static constexpr int WSTAGE = G4_WAVES * NTW * kTileBytes;  // one weight stage
-  static constexpr int LDS_BYTES = 2 * XBYTES + 2 * WSTAGE;
+  static constexpr int WSTAGE = G4_WAVES * NTW * kTileBytes;  // one weight stage of 4-bit tiles (8-bit: two)
+  static constexpr int LDS_BYTES = 2 * XBYTES + 2 * WSTAGE;   // 4-bit weights; lds_bytes() below
   static constexpr int SSTRIDE = NTW * kTileN + 4;      // fp32 row stride of the epilogue staging tile
   // Row-block during whose MFMAs the A fragments of the next K sub-step are read from LDS.  One
   // block ahead of their first use needs a second set of MT fragment registers; with 16 row tiles
@@ -47,6 +52,11 @@ struct G4Shape {
   static constexpr int XA_SETS = MT >= 16 ? 1 : 2;
   static constexpr int FETCH_T = XA_SETS == 1 ? NTW - 1 : NTW - 2;
 };
+
+template <class S, int WBITS>
+constexpr int g4_lds_bytes() {
+  return 2 * S::XBYTES + 2 * S::WSTAGE * (WBITS / 4);
+}
 
 template <int REGIME>
 __device__ __forceinline__ f4 g4_mfma(u4 a, u4 b, f4 c) {
@@ -59,10 +69,11 @@ __device__ __forceinline__ f4 g4_mfma(u4 a, u4 b, f4 c) {
 typedef __attribute__((address_space(3))) void* lds_ptr_t;
 typedef const __attribute__((address_space(1))) void* global_ptr_t;
 
-template <int REGIME, class S>
+template <int REGIME, class S, int WBITS>
 __global__ __launch_bounds__(256) void woq_gemm_w4_kernel(const FpArgs f, const int g_shift) {
+  constexpr int TPS = WBITS / 4;  // packed tiles per row-block and K step of 128
   constexpr int G4_MT = S::MT, G4_NTW = S::NTW, G4_BM = S::BM, G4_XBYTES = S::XBYTES, G4_XLOADS = S::XLOADS,
-                G4_WSTAGE = S::WSTAGE, G4_SSTRIDE = S::SSTRIDE;
+                G4_WSTAGE = S::WSTAGE * TPS, G4_SSTRIDE = S::SSTRIDE;
   // two activation buffers, then two weight stages of 4 waves x NTW tiles x 1 KiB
   extern __shared__ __align__(1024) uint8_t sX[];
   uint8_t* const sW = sX + 2 * G4_XBYTES;
@@ -71,7 +82,9 @@ __global__ __launch_bounds__(256) void woq_gemm_w4_kernel(const FpArgs f, const 
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int r = lane & 15, c = lane >> 4;
-  const int M = (int)f.M, K = (int)f.K, NT = (int)f.NT, KT = (int)f.KT, KG = (int)f.KG;
+  const int M = (int)f.M, K = (int)f.K, NT = (int)f.NT, KG = (int)f.KG;
+  const int KTW = (int)f.KT;   // packed tiles along K of a row-block
+  const int KT = KTW / TPS;    // K steps of 128
   const int m0 = blockIdx.y * G4_BM;
   const int nt0 = (blockIdx.x * G4_WAVES + wave) * G4_NTW;  // first row-block of this wave
 
@@ -108,10 +121,14 @@ __global__ __launch_bounds__(256) void woq_gemm_w4_kernel(const FpArgs f, const 
                                        (lds_ptr_t)(sX + buf * G4_XBYTES + (wave * G4_XLOADS + i) * 1024), 16, 0,
                                        0);
   };
-  // A fragment of row tile mt, sub-step j: row 16 mt + r, logical chunk 4 c + j
+  // A fragment of row tile mt, sub-step j: row 16 mt + r, logical chunk 4 c + j (8-bit weights:
+  // 8 (j / 2) + 2 c + j % 2, the K offsets of the lane column's bytes in tile j / 2)
   uint32_t rd[4];
 #pragma unroll
-  for (int j = 0; j < 4; ++j) rd[j] = (uint32_t)(r * 256 + (((c * 4 + j) ^ r) << 4));
+  for (int j = 0; j < 4; ++j) {
+    const int chunk = WBITS == 4 ? c * 4 + j : 8 * (j / 2) + 2 * c + (j % 2);
+    rd[j] = (uint32_t)(r * 256 + ((chunk ^ r) << 4));
+  }
 
   // ---- weights of one K tile: one dwordx4 + one (scale, zero) per row-block and lane.  Symmetric
   // weights carry no zero points: scale bytes are read (and ignored) instead of branching. ----
@@ -122,7 +139,7 @@ __global__ __launch_bounds__(256) void woq_gemm_w4_kernel(const FpArgs f, const 
 #pragma unroll
   for (int t = 0; t < G4_NTW; ++t) {
     const int nt = nt0 + t < NT ? nt0 + t : NT - 1;
-    wbase[t] = f.qweight + (size_t)nt * KT * kTileBytes;
+    wbase[t] = f.qweight + (size_t)nt * KTW * kTileBytes;
     sbase[t] = (const uint8_t*)(f.scales + (size_t)nt * KG * kTileN);
     zbase[t] = has_z ? f.zeros + (size_t)nt * KG * kTileN : sbase[t];
   }
@@ -135,35 +152,61 @@ __global__ __launch_bounds__(256) void woq_gemm_w4_kernel(const FpArgs f, const 
     for (int t = 0; t < G4_NTW; ++t) {
       s[t] = *(const uint16_t*)(sbase[t] + (uint32_t)(qoff * 2u));
       const uint8_t zb = *(zbase[t] + qoff);
-      z[t] = has_z ? zb : (uint8_t)8;
+      z[t] = has_z ? zb : (uint8_t)(WBITS == 4 ? 8 : 128);  // symmetric: the stored code of zero
     }
   };
   // The packed tiles of a K step travel global -> LDS -> registers: the LDS stage costs no
   // registers while the load is in flight, which lets the tiles be requested two steps ahead.
   // Each wave fills and reads only its own NTW KiB of a stage.
-  uint8_t* const wmine = sW + wave * (G4_NTW * kTileBytes);
+  uint8_t* const wmine = sW + wave * (G4_NTW * TPS * kTileBytes);
   auto dma_w = [&](int kt, int stage) {
-    const uint32_t wo = (uint32_t)kt * kTileBytes + woff;
+    const uint32_t wo = (uint32_t)kt * (TPS * kTileBytes) + woff;
 #pragma unroll
     for (int t = 0; t < G4_NTW; ++t)
-      __builtin_amdgcn_global_load_lds((global_ptr_t)(wbase[t] + wo),
-                                       (lds_ptr_t)(wmine + stage * G4_WSTAGE + t * kTileBytes), 16, 0, 0);
+#pragma unroll
+      for (int u = 0; u < TPS; ++u)
+        __builtin_amdgcn_global_load_lds((global_ptr_t)(wbase[t] + (uint32_t)(wo + u * kTileBytes)),
+                                         (lds_ptr_t)(wmine + stage * G4_WSTAGE + (t * TPS + u) * kTileBytes), 16, 0,
+                                         0);
   };
-  auto read_w = [&](int stage, int t) { return *(const u4*)(wmine + stage * G4_WSTAGE + t * kTileBytes + woff); };
+  auto read_w = [&](int stage, int t, int u) {
+    return *(const u4*)(wmine + stage * G4_WSTAGE + (t * TPS + u) * kTileBytes + woff);
+  };
 
-  u4 wr[G4_NTW];
+  u4 wr[G4_NTW][TPS];
   uint16_t sr[G4_NTW];
   uint8_t zr[G4_NTW];
-  G4Consts<REGIME> qc[G4_NTW];
+  G4Consts<REGIME> qc[WBITS == 4 ? G4_NTW : 1];
+  float q8s[WBITS == 8 ? G4_NTW : 1], q8c[WBITS == 8 ? G4_NTW : 1];  // 8-bit: scale, -(128 + z) * scale
+  auto set_q = [&](int t, uint16_t sbits, float z) {
+    if constexpr (WBITS == 4) {
+      qc[t].set(sbits, z);
+    } else {
+      q8s[t] = REGIME == kRegimeF16 ? f16_bits_to_f32(sbits) : bf16_bits_to_f32(sbits);
+      q8c[t] = -(z * q8s[t]);
+    }
+  };
+  // B operand of row-block t, K sub-step j
+  auto deq = [&](int t, int j) -> u4 {
+    if constexpr (WBITS == 4) {
+      return g4_dequant(wr[t][0][j], km, qc[t]);
+    } else {
+      const uint32_t d0 = wr[t][j / 2][2 * (j % 2)], d1 = wr[t][j / 2][2 * (j % 2) + 1];
+      if constexpr (REGIME == kRegimeF16)
+        return bitcast<u4>(dequant8_f16_w8(d0, d1, q8s[t], q8c[t]));
+      else
+        return bitcast<u4>(dequant8_bf16_w8(d0, d1, q8s[t], q8c[t]));
+    }
+  };
   u4 bop[2];        // B operand in use / being dequantized
   u4 xa[S::XA_SETS][G4_MT];  // A fragments of the sub-step in use (/ of the next one)
 
   // s_waitcnt immediates (vmcnt in bits 3:0 and 15:14; expcnt 6:4 and lgkmcnt 11:8 left at maximum)
   constexpr int kVmcnt0 = 0x0F70, kLgkmcnt0 = 0xC07F;
-  constexpr int kVmcntW = 0x0F70 | G4_NTW;  // all but the last NTW loads (one weight stage) have landed
-  // everything older than one whole step of loads (2 NTW parameter loads, XLOADS + NTW LDS loads)
-  constexpr int kStepLoads = 3 * G4_NTW + G4_XLOADS;
-  static_assert(kStepLoads < 64 && G4_NTW < 16, "s_waitcnt vmcnt is a 6-bit field");
+  constexpr int kVmcntW = 0x0F70 | (G4_NTW * TPS);  // all but the last loads (one weight stage) have landed
+  // everything older than one whole step of loads (2 NTW parameter loads, XLOADS + NTW * TPS LDS loads)
+  constexpr int kStepLoads = (2 + TPS) * G4_NTW + G4_XLOADS;
+  static_assert(kStepLoads < 64 && G4_NTW * TPS < 16, "s_waitcnt vmcnt is a 6-bit field");
   constexpr int kVmcntStep = 0x0F70 | (kStepLoads & 15) | ((kStepLoads >> 4) << 14);
 
   load_x(0, 0);
@@ -174,10 +217,11 @@ __global__ __launch_bounds__(256) void woq_gemm_w4_kernel(const FpArgs f, const 
   __syncthreads();
 #pragma unroll
   for (int t = 0; t < G4_NTW; ++t) {
-    wr[t] = read_w(0, t);
-    qc[t].set(sr[t], (float)zr[t]);
+#pragma unroll
+    for (int u = 0; u < TPS; ++u) wr[t][u] = read_w(0, t, u);
+    set_q(t, sr[t], (float)zr[t]);
   }
-  bop[0] = g4_dequant(wr[0][0], km, qc[0]);
+  bop[0] = deq(0, 0);
 #pragma unroll
   for (int mt = 0; mt < G4_MT; ++mt) xa[0][mt] = *(const u4*)(sX + mt * 4096 + rd[0]);
 
@@ -228,12 +272,12 @@ __global__ __launch_bounds__(256) void woq_gemm_w4_kernel(const FpArgs f, const 
         }
         if (last_t && j == 3) {
 #pragma unroll
-          for (int u = 0; u < G4_NTW; ++u) qc[u].set(sr[u], (float)zr[u]);
-          bop[cur ^ 1] = g4_dequant(wr[0][0], km, qc[0]);
+          for (int u = 0; u < G4_NTW; ++u) set_q(u, sr[u], (float)zr[u]);
+          bop[cur ^ 1] = deq(0, 0);
         } else if (last_t) {
-          bop[cur ^ 1] = g4_dequant(wr[0][j + 1], km, qc[0]);
+          bop[cur ^ 1] = deq(0, j + 1);
         } else {
-          bop[cur ^ 1] = g4_dequant(wr[t + 1][j], km, qc[t + 1]);
+          bop[cur ^ 1] = deq(t + 1, j);
         }
 #pragma unroll
         for (int mt = 0; mt < G4_MT; ++mt) {
@@ -242,7 +286,10 @@ __global__ __launch_bounds__(256) void woq_gemm_w4_kernel(const FpArgs f, const 
             xa[((j & 1) ^ 1) % S::XA_SETS][mt] = j == 3 ? *(const u4*)(xsn + mt * 4096 + rd[0])
                                          : *(const u4*)(xs + mt * 4096 + rd[j + 1]);
         }
-        if (j == 3) wr[t] = read_w((kt & 1) ^ 1, t);
+        if (j == 3) {
+#pragma unroll
+          for (int u = 0; u < TPS; ++u) wr[t][u] = read_w((kt & 1) ^ 1, t, u);
+        }
 #pragma unroll
         for (int mt = 0; mt < G4_MT; ++mt) {
           __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
@@ -325,26 +372,29 @@ __global__ __launch_bounds__(256) void woq_gemm_w4_kernel(const FpArgs f, const 
   }
 }
 
-// The kernel needs whole K tiles, activations already in the regime's dtype, and a group size whose
-// boundaries never split a lane's 32 consecutive K values.
+// The kernel needs whole K steps of 128, activations already in the regime's dtype, and a group size
+// whose boundaries never split a lane's 32 consecutive K values (8-bit weights: a K step, so groups of
+// at least 128 or one scale per channel).  NF4 codes are not taken.
 bool gemm_w4_applies(const FpArgs& f, int wbits, int regime) {
   const int want = regime == kRegimeF16 ? WOQ_HIP_ACT_FP16 : WOQ_HIP_ACT_BF16;
-  if (wbits != 4 || f.x_dtype != want || ((uintptr_t)f.x & 15) != 0) return false;
+  if ((wbits != 4 && wbits != 8) || f.nf4 || f.x_dtype != want || ((uintptr_t)f.x & 15) != 0) return false;
   if (f.K % kTileK4 != 0 || f.K * 256 * 2 >= (int64_t)1 << 31) return false;
-  if (f.G >= f.KT * kTileK4) return true;                 // per-channel: one group
-  return f.G >= 32 && (f.G & (f.G - 1)) == 0;
+  if (f.G >= f.KT * (wbits == 4 ? kTileK4 : kTileK8)) return true;  // per-channel: one group
+  return f.G >= (wbits == 4 ? 32 : 128) && (f.G & (f.G - 1)) == 0;
 }
 
-template <int REGIME, class S>
+template <int REGIME, class S, int WBITS = 4>
 static int launch_shape(const FpArgs& f, int g_shift, hipStream_t st) {
+  constexpr int kLds = g4_lds_bytes<S, WBITS>();
+  static_assert(kLds <= 160 * 1024, "a workgroup's LDS");
   // more than 64 KiB of LDS per workgroup needs an opt-in (once per kernel and process)
   static const hipError_t lds_optin =
-      hipFuncSetAttribute(reinterpret_cast<const void*>(&woq_gemm_w4_kernel<REGIME, S>),
-                          hipFuncAttributeMaxDynamicSharedMemorySize, S::LDS_BYTES);
+      hipFuncSetAttribute(reinterpret_cast<const void*>(&woq_gemm_w4_kernel<REGIME, S, WBITS>),
+                          hipFuncAttributeMaxDynamicSharedMemorySize, kLds);
   if (lds_optin != hipSuccess)
     return set_error("woq_gemm_w4_kernel: LDS opt-in failed: %s", hipGetErrorString(lds_optin));
   dim3 grid((unsigned)((f.NT * kTileN + S::BN - 1) / S::BN), (unsigned)((f.M + S::BM - 1) / S::BM));
-  woq_gemm_w4_kernel<REGIME, S><<<grid, 256, S::LDS_BYTES, st>>>(f, g_shift);
+  woq_gemm_w4_kernel<REGIME, S, WBITS><<<grid, 256, kLds, st>>>(f, g_shift);
   return check_launch("woq_gemm_w4_kernel");
 }
 
@@ -356,9 +406,9 @@ static double shape_cost(const FpArgs& f) {
   return (double)(int64_t)((wgs + 255) / 256) * (S::NTW + 1.0);
 }
 
-int launch_gemm_w4(const FpArgs& f, int regime, hipStream_t st, int shape) {
+int launch_gemm_w4(const FpArgs& f, int wbits, int regime, hipStream_t st, int shape) {
   int g_shift = 30;
-  if (f.G < f.KT * kTileK4) {
+  if (f.G < f.KT * (wbits == 4 ? kTileK4 : kTileK8)) {
     g_shift = 0;
     while (((int64_t)1 << g_shift) < f.G) ++g_shift;
   }
@@ -376,6 +426,24 @@ int launch_gemm_w4(const FpArgs& f, int regime, hipStream_t st, int shape) {
   using S2 = G4Shape<8, 2>;
   using ST = G4Shape<16, 3>;
   using S42 = G4Shape<4, 2>;
+  if (wbits == 8) {
+    // 8-bit weights: twice the tile bytes per K step, so at most four row-blocks per wave fit the LDS
+    // (128 x 256, 128 x 128 and 64 x 128 workgroup tiles), chosen like the 4-bit ones
+    if (shape != 0 && shape != 4 && shape != 2 && shape != 42)
+      return set_error("woq_gemm_w4_kernel: 8-bit weights take the 128 x 256, 128 x 128 and 64 x 128 shapes");
+    if (shape == 0) {
+      const int64_t wgs42 = ((f.NT * kTileN + S42::BN - 1) / S42::BN) * ((f.M + S42::BM - 1) / S42::BM);
+      shape = wgs42 <= 256 ? 42 : (shape_cost<S4>(f) <= shape_cost<S2>(f) ? 4 : 2);
+    }
+    if (shape == 42)
+      return regime == kRegimeF16 ? launch_shape<kRegimeF16, S42, 8>(f, g_shift, st)
+                                  : launch_shape<kRegimeBF16, S42, 8>(f, g_shift, st);
+    if (shape == 4)
+      return regime == kRegimeF16 ? launch_shape<kRegimeF16, S4, 8>(f, g_shift, st)
+                                  : launch_shape<kRegimeBF16, S4, 8>(f, g_shift, st);
+    return regime == kRegimeF16 ? launch_shape<kRegimeF16, S2, 8>(f, g_shift, st)
+                                : launch_shape<kRegimeBF16, S2, 8>(f, g_shift, st);
+  }
   if (shape == 0) {
     // Small M x N: 64 x 128 tiles at four waves per SIMD (79 + 32 registers, 48 KiB of LDS).  While
     // every workgroup has a CU to itself the K loop is one memory round trip per step whatever the

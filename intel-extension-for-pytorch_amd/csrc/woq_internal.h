@@ -98,10 +98,12 @@ int64_t decode_dq_splitk_bytes(int64_t M, int64_t NT, int splits);
 // regime: 0 = fp16, 1 = bf16 (woq::Regime)
 int launch_small_m(const FpArgs& a, int wbits, int regime, hipStream_t st);
 int launch_gemm(const FpArgs& a, int wbits, int regime, hipStream_t st);
-// 4-bit prefill GEMM with register-resident dequantization (woq_gemm_w4.hip)
+// Prefill GEMM with register-resident dequantization (woq_gemm_w4.hip): 4-bit integer weights, or
+// 8-bit weights with one scale per channel or per group of at least 128
 bool gemm_w4_applies(const FpArgs& f, int wbits, int regime);
-// shape: row-blocks per wave (7, 4 or 2: 448, 256 or 128 columns per workgroup), 0 = by cost model
-int launch_gemm_w4(const FpArgs& f, int regime, hipStream_t st, int shape = 0);
+// shape: row-blocks per wave (7, 4 or 2: 448, 256 or 128 columns per workgroup), 163 / 42 = 256 x 192 /
+// 64 x 128 tiles, 0 = by cost model; 8-bit weights: 4, 2, 42 or 0
+int launch_gemm_w4(const FpArgs& f, int wbits, int regime, hipStream_t st, int shape = 0);
 
 struct Int8Args {
   const void* x;

@@ -41,12 +41,13 @@ def make_nf4_case(cfg, M, K, N, group_size, bias=False, scale_dtype=torch.bfloat
     return case
 
 
-def make_int8_case(cfg, M, K, N, bias=True):
-    """Per-output-channel symmetric int8 weights uniform in -127..127, fp32 scales uniform in
-    [0.001, 0.01], bf16 bias ~ N(0, 0.02)."""
+def make_int8_case(cfg, M, K, N, bias=True, group_size=-1):
+    """Symmetric int8 weights uniform in -127..127, fp32 scales uniform in [0.001, 0.01] per output
+    channel (or per group of ``group_size`` input channels), bf16 bias ~ N(0, 0.02)."""
     x = torch.randn(M, K, generator=_gen(cfg, 0)).to(torch.bfloat16)
     qweight = torch.randint(-127, 128, (N, K), dtype=torch.int8, generator=_gen(cfg, 1))
-    scales = 0.001 + 0.009 * torch.rand(N, generator=_gen(cfg, 2))
+    shape = (N,) if group_size <= 0 else (N, (K + group_size - 1) // group_size)
+    scales = 0.001 + 0.009 * torch.rand(shape, generator=_gen(cfg, 2))
     b = (0.02 * torch.randn(N, generator=_gen(cfg, 4))).to(torch.bfloat16) if bias else None
     return dict(x=x, qweight=qweight, scales=scales, zeros=None, bias=b, M=M, K=K, N=N,
-                group_size=-1, weight_dtype=1)
+                group_size=group_size, weight_dtype=1)

@@ -287,10 +287,44 @@ def test_w4_prefill_kernel_fp16_regime(cuda):
     assert rel_l2(y, to_np_f32(ctx.run(x, force_kernel=2))) <= 1e-3
 
 
+@pytest.mark.parametrize(
+    "M,K,N,G,bias",
+    [
+        (65, 1024, 272, -1, True),
+        (200, 384, 464, -1, False),  # three K steps, ragged M and N
+        (300, 2048, 128, 128, True),  # one scale per 128 input channels
+        (129, 512, 1040, 256, False),
+        (2048, 256, 256, -1, True),
+    ],
+)
+@pytest.mark.parametrize("kernel", [0, 5, 6, 12])  # automatic, 128 x 256, 128 x 128, 64 x 128 tiles
+def test_prefill_kernel_int8_weights(cuda, M, K, N, G, bias, kernel):
+    """8-bit weights through the prefill GEMM: two packed tiles per row-block and K step."""
+    case = _synthetic().make_int8_case(26, M, K, N, bias=bias, group_size=G)
+    _check_fp(case, O.LOWP_BF16, force_kernel=kernel, label=f"int8-weight prefill M={M} K={K} N={N} G={G} kernel={kernel}")
+
+
+def test_prefill_kernel_int8_weights_fp16_and_rejections(cuda):
+    syn = _synthetic()
+    case = syn.make_int8_case(27, 150, 512, 272)
+    case["x"] = case["x"].to(torch.float16)
+    ctx = make_context(case, O.LOWP_FP16)
+    x = case["x"].cuda()
+    want = to_np_f32(ctx.run(x, force_kernel=2))
+    for kernel in (3, 5, 6, 12):
+        assert rel_l2(to_np_f32(ctx.run(x, force_kernel=kernel)), want) <= 1e-3, kernel
+    with pytest.raises(RuntimeError, match="8-bit weights take"):
+        ctx.run(x, force_kernel=4)  # 448 columns per workgroup: the tiles of a step would not fit the LDS
+    small_groups = syn.make_int8_case(28, 100, 512, 64, group_size=64)
+    with pytest.raises(RuntimeError, match="prefill kernel takes"):
+        make_context(small_groups, O.LOWP_BF16).run(small_groups["x"].cuda(), force_kernel=3)
+    _check_fp(small_groups, O.LOWP_BF16, label="int8 weights, groups of 64: general kernel")
+
+
 def test_w4_prefill_kernel_rejects_other_shapes(cuda):
     case = _synthetic().make_int4_case(23, 70, 1000, 64, -1)  # K is not a multiple of 128
     ctx = make_context(case, O.LOWP_BF16)
-    with pytest.raises(RuntimeError, match="4-bit prefill kernel"):
+    with pytest.raises(RuntimeError, match="prefill kernel takes"):
         ctx.run(case["x"].cuda(), force_kernel=3)
 
 
