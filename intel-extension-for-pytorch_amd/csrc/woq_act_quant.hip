@@ -72,12 +72,17 @@ struct AqArgs {
   int permute, offset128;
 };
 
-// NCH: 512-element chunks of a (padded) row
-template <int NCH>
+// NCH: 512-element chunks of a (padded) row that one wave holds.  SPLIT: the four waves of a
+// workgroup share one row (wave w takes chunks w, w + 4, ...), for the few rows of a decode step,
+// where a single wave per row would be one long dependent chain (M = 1, K = 4096: 6.5 us).
+template <int NCH, bool SPLIT>
 __global__ __launch_bounds__(256) void act_quant_rows_kernel(const AqArgs a) {
   const int lane = threadIdx.x & 63;
-  const int64_t m = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int wave = threadIdx.x >> 6;
+  const int64_t m = SPLIT ? (int64_t)blockIdx.x : (int64_t)blockIdx.x * 4 + wave;
   if (m >= a.M) return;
+  // chunk held in register slot c
+  auto chunk_of = [&](int c) { return SPLIT ? wave + 4 * c : c; };
   const uint16_t* const row = a.x + m * a.K;
   const bool bf16 = a.bf16 != 0, sym = a.sym != 0, per_k = a.block_lanes_log2 >= 0;
 
@@ -85,7 +90,7 @@ __global__ __launch_bounds__(256) void act_quant_rows_kernel(const AqArgs a) {
   u4 raw[NCH];
 #pragma unroll
   for (int c = 0; c < NCH; ++c) {
-    const int64_t k0 = (int64_t)c * 512 + lane * 8;
+    const int64_t k0 = (int64_t)chunk_of(c) * 512 + lane * 8;
     raw[c] = k0 < a.K ? *(const u4*)(row + k0) : u4{0u, 0u, 0u, 0u};
   }
 
@@ -94,7 +99,7 @@ __global__ __launch_bounds__(256) void act_quant_rows_kernel(const AqArgs a) {
   for (int c = 0; c < NCH; ++c) {
     mn[c] = __builtin_inff();
     mx[c] = -__builtin_inff();
-    if ((int64_t)c * 512 + lane * 8 < a.K) {
+    if ((int64_t)chunk_of(c) * 512 + lane * 8 < a.K) {
       float v[8];
       aq_unpack(raw[c], bf16, v);
 #pragma unroll
@@ -115,6 +120,20 @@ __global__ __launch_bounds__(256) void act_quant_rows_kernel(const AqArgs a) {
       mn[0] = fminf(mn[0], __shfl_xor(mn[0], off));
       mx[0] = fmaxf(mx[0], __shfl_xor(mx[0], off));
     }
+    if constexpr (SPLIT) {
+      // the four waves' extremes meet in LDS (every wave of the workgroup is here: same row)
+      __shared__ float smn[4], smx[4];
+      if (lane == 0) {
+        smn[wave] = mn[0];
+        smx[wave] = mx[0];
+      }
+      __syncthreads();
+#pragma unroll
+      for (int w = 0; w < 4; ++w) {
+        mn[0] = fminf(mn[0], smn[w]);
+        mx[0] = fmaxf(mx[0], smx[w]);
+      }
+    }
   } else {
     // the lanes of one K block are 2^block_lanes_log2 consecutive lanes, aligned
 #pragma unroll
@@ -129,7 +148,7 @@ __global__ __launch_bounds__(256) void act_quant_rows_kernel(const AqArgs a) {
   if (!per_k) {
     int32_t z = 0;
     row_p = aq_params(mn[0], mx[0], sym, &z);
-    if (lane == 0) {
+    if (lane == 0 && (!SPLIT || wave == 0)) {
       a.scales[m] = row_p.s;
       if (!sym) a.zps[m] = z;
     }
@@ -137,7 +156,7 @@ __global__ __launch_bounds__(256) void act_quant_rows_kernel(const AqArgs a) {
   uint8_t* const qrow = a.q + m * a.ldq;
 #pragma unroll
   for (int c = 0; c < NCH; ++c) {
-    const int64_t k0 = (int64_t)c * 512 + lane * 8;
+    const int64_t k0 = (int64_t)chunk_of(c) * 512 + lane * 8;
     if (k0 >= a.ldq) continue;
     u2 out = u2{0u, 0u};  // the tail of a padded row is zero
     if (k0 < a.K) {
@@ -199,14 +218,24 @@ int launch_act_quant_rows(const void* x, int x_dtype, int64_t M, int64_t K, int6
   a.sym = sym;
   a.scales = scales; a.zps = zps; a.q = (uint8_t*)q;
   a.permute = permute; a.offset128 = offset128;
-  const unsigned grid = (unsigned)((M + 3) / 4);
   const int64_t chunks = (ldq + 511) / 512;
+  if (M <= 64) {
+    // few rows: a workgroup per row, a quarter of the chunks per wave
+    if (chunks <= 8)
+      act_quant_rows_kernel<2, true><<<(unsigned)M, 256, 0, st>>>(a);
+    else if (chunks <= 16)
+      act_quant_rows_kernel<4, true><<<(unsigned)M, 256, 0, st>>>(a);
+    else
+      act_quant_rows_kernel<8, true><<<(unsigned)M, 256, 0, st>>>(a);
+    return check_launch("act_quant_rows_kernel");
+  }
+  const unsigned grid = (unsigned)((M + 3) / 4);
   if (chunks <= 8)
-    act_quant_rows_kernel<8><<<grid, 256, 0, st>>>(a);
+    act_quant_rows_kernel<8, false><<<grid, 256, 0, st>>>(a);
   else if (chunks <= 16)
-    act_quant_rows_kernel<16><<<grid, 256, 0, st>>>(a);
+    act_quant_rows_kernel<16, false><<<grid, 256, 0, st>>>(a);
   else
-    act_quant_rows_kernel<32><<<grid, 256, 0, st>>>(a);
+    act_quant_rows_kernel<32, false><<<grid, 256, 0, st>>>(a);
   return check_launch("act_quant_rows_kernel");
 }
 

@@ -308,14 +308,166 @@ __global__ __launch_bounds__(256, 3) void woq_gemm_w4i8_kernel(const W4I8Args a)
     }
 }
 
+// ---- at most 16 rows (decode): the weight stream bounds the kernel -------------------------------
+// Same work decomposition as the floating-point decode kernels: a workgroup owns NTW weight
+// row-blocks and all of K, its W <= 8 waves take one K tile (= one K block of 128) each per round,
+// the fp32 partial sums meet in LDS and are added in wave order.  Per tile and row-block: two
+// v_mfma_i32_16x16x64_i8 on the decoded dwords, then the four sums of a lane go into its fp32
+// accumulators as in the prefill kernel.  The quantized rows of a tile (16 x 128 bytes) are copied
+// into the wave's own LDS slice (global_load_lds, swizzled as in the prefill kernel); requests run
+// one round ahead.
+struct DecodeW4I8Args {
+  W4I8Args k;
+  int W;  // waves per workgroup
+};
+
+template <bool PER_K, int NTW>
+__global__ __launch_bounds__(512, 4) void woq_decode_w4i8_kernel(const DecodeW4I8Args a) {
+  constexpr int SLICE = 16 * kTileK4;  // one buffer of one wave: 16 rows x 128 bytes
+  extern __shared__ __align__(1024) uint8_t smem[];
+  const W4I8Args& k = a.k;
+  const int W = a.W;
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+  const int r = lane & 15, c = lane >> 4;
+  const int M = (int)k.M, KT = (int)k.KT, KG = (int)k.KG;
+  const int64_t nt0 = (int64_t)blockIdx.x * NTW;
+  uint8_t* const sx = smem + wave * (2 * SLICE);
+  f4* const red = (f4*)smem;  // [NTW][W][64], after the K loop
+
+  f4 acc[NTW];
+#pragma unroll
+  for (int t = 0; t < NTW; ++t) acc[t] = f4{0.f, 0.f, 0.f, 0.f};
+
+  // activation load i (two per tile) fills LDS bytes [1024 i, +1024) of a buffer: rows 8 i + lane / 8,
+  // physical chunk lane % 8 = logical chunk ^ ((row / 2) % 8); rows past M re-read row M - 1
+  uint32_t xoff[2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int row = 8 * i + (lane >> 3);
+    const int rowc = row < M ? row : M - 1;
+    const int chunk = (lane & 7) ^ ((row >> 1) & 7);
+    xoff[i] = (uint32_t)(rowc * (int)k.ldq + chunk * 16);
+  }
+  uint32_t rd[2];  // A fragment of MFMA j: row r, logical chunk 2 c + j
+#pragma unroll
+  for (int j = 0; j < 2; ++j) rd[j] = (uint32_t)(r * 128 + (((2 * c + j) ^ ((r >> 1) & 7)) << 4));
+
+  const bool has_z = k.zeros != nullptr;
+  const uint8_t* wbase[NTW];
+  const float* sbase[NTW];
+  const uint8_t* zbase[NTW];
+#pragma unroll
+  for (int t = 0; t < NTW; ++t) {
+    wbase[t] = k.qweight + (size_t)(nt0 + t) * KT * kTileBytes;
+    sbase[t] = k.scales + (size_t)(nt0 + t) * KG * kTileN;
+    zbase[t] = has_z ? k.zeros + (size_t)(nt0 + t) * KG * kTileN : (const uint8_t*)sbase[t];
+  }
+  const uint32_t woff = (uint32_t)lane * 16u;
+
+  // activation scales of this lane's accumulator rows m = 4 c + e: one per row for the whole K, or
+  // (PER_K) one per row and K block, requested with the tile
+  f4 sa_row;
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    const int m = 4 * c + e;
+    sa_row[e] = PER_K ? 0.0f : k.sa[(int64_t)(m < M ? m : M - 1) * k.sa_m_stride];
+  }
+
+  u4 wnext[NTW];
+  float snext[NTW];
+  uint8_t znext[NTW];
+  f4 sanext;
+  auto request = [&](int kt, int buf) {
+    const uint32_t ko = (uint32_t)kt * kTileK4;
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+      if (8 * i < M)
+        __builtin_amdgcn_global_load_lds((w8_global_ptr_t)(k.xq + (uint32_t)(xoff[i] + ko)),
+                                         (w8_lds_ptr_t)(sx + buf * SLICE + i * 1024), 16, 0, 0);
+    int g = kt >> k.g_shift;
+    g = g < KG ? g : KG - 1;
+    const uint32_t qoff = (uint32_t)(g * kTileN + r);
+    const uint32_t wo = (uint32_t)kt * kTileBytes + woff;
+#pragma unroll
+    for (int t = 0; t < NTW; ++t) {
+      wnext[t] = __builtin_nontemporal_load((const u4*)(wbase[t] + wo));
+      snext[t] = sbase[t][qoff];
+      znext[t] = *(zbase[t] + qoff);  // raw: any use here would wait for the load inside the request
+    }
+    if (PER_K) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const int m = 4 * c + e;
+        sanext[e] = k.sa[(int64_t)(m < M ? m : M - 1) * k.sa_m_stride + (int64_t)(kt >> k.q_shift) * k.sa_k_stride];
+      }
+    }
+  };
+
+  if (wave < KT) request(wave, 0);
+#pragma unroll 1
+  for (int kt = wave, buf = 0; kt < KT; kt += W, buf ^= 1) {
+    u4 wreg[NTW];
+    float sw[NTW];
+    uint32_t z4[NTW];
+    f4 sa = sa_row;
+#pragma unroll
+    for (int t = 0; t < NTW; ++t) {
+      wreg[t] = wnext[t];
+      sw[t] = snext[t];
+      z4[t] = (has_z ? (uint32_t)znext[t] : 8u) * 0x01010101u;
+    }
+    if (PER_K) sa = sanext;
+    // the compiler does not order LDS reads after the LDS-writing loads: wait for them here
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+    if (kt + W < KT) request(kt + W, buf ^ 1);
+    __builtin_amdgcn_sched_barrier(0);
+
+    const i4 xa0 = *(const i4*)(sx + buf * SLICE + rd[0]);
+    const i4 xa1 = *(const i4*)(sx + buf * SLICE + rd[1]);
+#pragma unroll
+    for (int t = 0; t < NTW; ++t) {
+      const i4 bq0 = w8_decode16(wreg[t][0], wreg[t][1], z4[t]);
+      const i4 bq1 = w8_decode16(wreg[t][2], wreg[t][3], z4[t]);
+      i4 qc = __builtin_amdgcn_mfma_i32_16x16x64_i8(xa0, bq0, i4{0, 0, 0, 0}, 0, 0, 0);
+      qc = __builtin_amdgcn_mfma_i32_16x16x64_i8(xa1, bq1, qc, 0, 0, 0);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) acc[t][e] = w8_accumulate<PER_K>(qc[e], sa[e], sw[t], acc[t][e]);
+    }
+  }
+
+  // ---- combine the waves' partial sums in wave order, then scale / bias / rounding / store ----
+  __syncthreads();  // every wave is done with its activation slices: the region becomes `red`
+#pragma unroll
+  for (int t = 0; t < NTW; ++t) red[(t * W + wave) * 64 + lane] = acc[t];
+  __syncthreads();
+  const float* redf = (const float*)red;
+  // one thread per output element, consecutive threads on consecutive columns; D[m][n] of a row
+  // tile sits in lane n + 16 (m / 4), register m % 4
+  for (int idx = threadIdx.x; idx < NTW * 256; idx += blockDim.x) {
+    const int col = idx & 15, m = (idx >> 4) & 15, t = idx >> 8;
+    const int64_t n = (nt0 + t) * kTileN + col;
+    if (m >= M || n >= k.N) continue;
+    const int slot = (col + 16 * (m >> 2)) * 4 + (m & 3);
+    float part[8];
+#pragma unroll
+    for (int w = 0; w < 8; ++w) part[w] = w < W ? redf[(t * W + w) * 256 + slot] : 0.0f;
+    float s = part[0];
+#pragma unroll
+    for (int w = 1; w < 8; ++w) s = s + part[w];
+    if (!PER_K) s = s * k.sa[(int64_t)m * k.sa_m_stride];
+    epilogue_store<kRegimeBF16>(k.ep, m, n, s);
+  }
+}
+
 // 4-bit integer codes, symmetric activation scales per tensor or per row, K blocks of 128 that are
 // whole weight tiles, and a group size of 128 * 2^s (or one group), so that a K tile has one scale.
-// More than 16 rows: with a single 64-row tile the kernel still beats the small-M one (4096 -> 14336,
-// per-row scales, M = 32 / 48 / 64: 31 / 34 / 36 us against 50 / 157 / 162 us); up to 16 rows that one
-// is faster (27-29 us).
+// Up to 16 rows run on the decode form (woq_decode_w4i8_kernel); from 17 rows the 64-row tiles of the
+// MFMA GEMM, which with a single row tile still beats the general small-M kernel (4096 -> 14336, per-row
+// scales, M = 32 / 48 / 64: 31 / 34 / 36 us against 50 / 157 / 162 us).
 bool gemm_w4i8_applies(const Int8Args& a, int64_t block_k, int64_t qbk, bool per_k, bool asym) {
   if (a.wbits != 4 || a.nf4 || asym || a.debug_block_sums) return false;
-  if (block_k != 128 || a.K % 128 != 0 || a.M <= 16) return false;
+  if (block_k != 128 || a.K % 128 != 0) return false;
   if (a.group_size > 0 && (a.G % 128 != 0 || ((a.G / 128) & (a.G / 128 - 1)) != 0)) return false;
   // activation K blocks of 128 * 2^s as well (they follow the group size, or the K block)
   if (per_k && (qbk % 128 != 0 || ((qbk / 128) & (qbk / 128 - 1)) != 0)) return false;
@@ -344,6 +496,30 @@ int launch_gemm_w4i8(const Int8Args& a, const uint8_t* xq, int64_t ldq, const fl
     while (((int64_t)128 << k.g_shift) < a.G) ++k.g_shift;
   }
   k.ep = Epilogue{a.bias, a.fusion, a.other0, a.other1, a.out, a.out_dtype, a.x_dtype, a.N};
+  if (a.M <= 16) {
+    // decode form: 2 row-blocks per workgroup while that leaves at least 256 workgroups, else 1
+    DecodeW4I8Args d;
+    d.k = k;
+    d.W = (int)(a.KT < 8 ? a.KT : 8);
+    const int ntw = (a.NT >= 512 && a.NT % 2 == 0) ? 2 : 1;
+    size_t smem = (size_t)d.W * 2 * 16 * kTileK4;
+    const size_t red = (size_t)ntw * d.W * 64 * sizeof(f4);
+    if (red > smem) smem = red;
+    const unsigned dgrid = (unsigned)(a.NT / ntw);
+    const bool per_k = sa_k_stride != 0;
+    if (ntw == 2) {
+      if (per_k)
+        woq_decode_w4i8_kernel<true, 2><<<dgrid, d.W * 64, smem, st>>>(d);
+      else
+        woq_decode_w4i8_kernel<false, 2><<<dgrid, d.W * 64, smem, st>>>(d);
+    } else {
+      if (per_k)
+        woq_decode_w4i8_kernel<true, 1><<<dgrid, d.W * 64, smem, st>>>(d);
+      else
+        woq_decode_w4i8_kernel<false, 1><<<dgrid, d.W * 64, smem, st>>>(d);
+    }
+    return check_launch("woq_decode_w4i8_kernel");
+  }
   dim3 grid((unsigned)((a.NT * kTileN + W8_BN - 1) / W8_BN), (unsigned)((a.M + W8_BM - 1) / W8_BM));
   if (sa_k_stride != 0)
     woq_gemm_w4i8_kernel<true><<<grid, 256, W8_LDS_BYTES, st>>>(k);
