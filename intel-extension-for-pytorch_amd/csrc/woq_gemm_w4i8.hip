@@ -316,12 +316,17 @@ __global__ __launch_bounds__(256, 3) void woq_gemm_w4i8_kernel(const W4I8Args a)
 // accumulators as in the prefill kernel.  The quantized rows of a tile (16 x 128 bytes) are copied
 // into the wave's own LDS slice (global_load_lds, swizzled as in the prefill kernel); requests run
 // one round ahead.
+// GSUB > 1: groups of 64 or 32 input channels, i.e. 2 or 4 K blocks per tile.  A lane column c holds
+// the K values 32 c .. 32 c + 31 of the tile, all of one group, but an MFMA sums over the four lane
+// columns; block g is therefore computed with the activation fragments of the other blocks' lane
+// columns zeroed (GSUB times the MFMAs, which a decode step has to spare), and scaled with its own
+// weight and activation scales.
 struct DecodeW4I8Args {
   W4I8Args k;
   int W;  // waves per workgroup
 };
 
-template <bool PER_K, int NTW>
+template <bool PER_K, int NTW, int GSUB>
 __global__ __launch_bounds__(512, 4) void woq_decode_w4i8_kernel(const DecodeW4I8Args a) {
   constexpr int SLICE = 16 * kTileK4;  // one buffer of one wave: 16 rows x 128 bytes
   extern __shared__ __align__(1024) uint8_t smem[];
@@ -375,9 +380,10 @@ __global__ __launch_bounds__(512, 4) void woq_decode_w4i8_kernel(const DecodeW4I
   }
 
   u4 wnext[NTW];
-  float snext[NTW];
+  float snext[NTW][GSUB];
   uint8_t znext[NTW];
-  f4 sanext;
+  f4 sanext[GSUB];
+  const int my_block = c / (4 / GSUB);  // K block of the tile this lane column's weights belong to
   auto request = [&](int kt, int buf) {
     const uint32_t ko = (uint32_t)kt * kTileK4;
 #pragma unroll
@@ -385,22 +391,27 @@ __global__ __launch_bounds__(512, 4) void woq_decode_w4i8_kernel(const DecodeW4I
       if (8 * i < M)
         __builtin_amdgcn_global_load_lds((w8_global_ptr_t)(k.xq + (uint32_t)(xoff[i] + ko)),
                                          (w8_lds_ptr_t)(sx + buf * SLICE + i * 1024), 16, 0, 0);
-    int g = kt >> k.g_shift;
-    g = g < KG ? g : KG - 1;
-    const uint32_t qoff = (uint32_t)(g * kTileN + r);
+    // first group of the tile (GSUB == 1: the tile's only one, shared by 2^g_shift tiles)
+    int g0 = GSUB == 1 ? (kt >> k.g_shift) : kt * GSUB;
+    g0 = g0 < KG ? g0 : KG - 1;
     const uint32_t wo = (uint32_t)kt * kTileBytes + woff;
 #pragma unroll
     for (int t = 0; t < NTW; ++t) {
       wnext[t] = __builtin_nontemporal_load((const u4*)(wbase[t] + wo));
-      snext[t] = sbase[t][qoff];
-      znext[t] = *(zbase[t] + qoff);  // raw: any use here would wait for the load inside the request
+#pragma unroll
+      for (int g = 0; g < GSUB; ++g) snext[t][g] = sbase[t][(uint32_t)((g0 + g) * kTileN + r)];
+      // raw: any use here would wait for the load inside the request
+      znext[t] = *(zbase[t] + (uint32_t)((g0 + (GSUB == 1 ? 0 : my_block)) * kTileN + r));
     }
     if (PER_K) {
 #pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        const int m = 4 * c + e;
-        sanext[e] = k.sa[(int64_t)(m < M ? m : M - 1) * k.sa_m_stride + (int64_t)(kt >> k.q_shift) * k.sa_k_stride];
-      }
+      for (int g = 0; g < GSUB; ++g)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const int m = 4 * c + e;
+          const int64_t kb = GSUB == 1 ? (int64_t)(kt >> k.q_shift) : (int64_t)kt * GSUB + g;
+          sanext[g][e] = k.sa[(int64_t)(m < M ? m : M - 1) * k.sa_m_stride + kb * k.sa_k_stride];
+        }
     }
   };
 
@@ -408,16 +419,18 @@ __global__ __launch_bounds__(512, 4) void woq_decode_w4i8_kernel(const DecodeW4I
 #pragma unroll 1
   for (int kt = wave, buf = 0; kt < KT; kt += W, buf ^= 1) {
     u4 wreg[NTW];
-    float sw[NTW];
+    float sw[NTW][GSUB];
     uint32_t z4[NTW];
-    f4 sa = sa_row;
+    f4 sa[GSUB];
 #pragma unroll
     for (int t = 0; t < NTW; ++t) {
       wreg[t] = wnext[t];
-      sw[t] = snext[t];
+#pragma unroll
+      for (int g = 0; g < GSUB; ++g) sw[t][g] = snext[t][g];
       z4[t] = (has_z ? (uint32_t)znext[t] : 8u) * 0x01010101u;
     }
-    if (PER_K) sa = sanext;
+#pragma unroll
+    for (int g = 0; g < GSUB; ++g) sa[g] = PER_K ? sanext[g] : sa_row;
     // the compiler does not order LDS reads after the LDS-writing loads: wait for them here
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
     if (kt + W < KT) request(kt + W, buf ^ 1);
@@ -429,10 +442,19 @@ __global__ __launch_bounds__(512, 4) void woq_decode_w4i8_kernel(const DecodeW4I
     for (int t = 0; t < NTW; ++t) {
       const i4 bq0 = w8_decode16(wreg[t][0], wreg[t][1], z4[t]);
       const i4 bq1 = w8_decode16(wreg[t][2], wreg[t][3], z4[t]);
-      i4 qc = __builtin_amdgcn_mfma_i32_16x16x64_i8(xa0, bq0, i4{0, 0, 0, 0}, 0, 0, 0);
-      qc = __builtin_amdgcn_mfma_i32_16x16x64_i8(xa1, bq1, qc, 0, 0, 0);
 #pragma unroll
-      for (int e = 0; e < 4; ++e) acc[t][e] = w8_accumulate<PER_K>(qc[e], sa[e], sw[t], acc[t][e]);
+      for (int g = 0; g < GSUB; ++g) {
+        // activation fragments of K block g: the lane columns of the other blocks contribute zeros
+        // (masked again for every row-block: holding GSUB masked copies costs more registers than
+        // the selects cost time)
+        const bool mine = GSUB == 1 || my_block == g;
+        const i4 xg0 = mine ? xa0 : i4{0, 0, 0, 0};
+        const i4 xg1 = mine ? xa1 : i4{0, 0, 0, 0};
+        i4 qc = __builtin_amdgcn_mfma_i32_16x16x64_i8(xg0, bq0, i4{0, 0, 0, 0}, 0, 0, 0);
+        qc = __builtin_amdgcn_mfma_i32_16x16x64_i8(xg1, bq1, qc, 0, 0, 0);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) acc[t][e] = w8_accumulate<PER_K>(qc[e], sa[g][e], sw[t][g], acc[t][e]);
+      }
     }
   }
 
@@ -467,7 +489,12 @@ __global__ __launch_bounds__(512, 4) void woq_decode_w4i8_kernel(const DecodeW4I
 // scales, M = 32 / 48 / 64: 31 / 34 / 36 us against 50 / 157 / 162 us).
 bool gemm_w4i8_applies(const Int8Args& a, int64_t block_k, int64_t qbk, bool per_k, bool asym) {
   if (a.wbits != 4 || a.nf4 || asym || a.debug_block_sums) return false;
-  if (block_k != 128 || a.K % 128 != 0) return false;
+  if (a.K % 128 != 0) return false;
+  if (block_k == 32 || block_k == 64) {
+    // groups of 32 / 64: the decode form only (K blocks inside a tile), activation blocks = groups
+    return a.M <= 16 && a.group_size == block_k && (!per_k || qbk == block_k) && a.M * a.K < ((int64_t)1 << 31);
+  }
+  if (block_k != 128) return false;
   if (a.group_size > 0 && (a.G % 128 != 0 || ((a.G / 128) & (a.G / 128 - 1)) != 0)) return false;
   // activation K blocks of 128 * 2^s as well (they follow the group size, or the K block)
   if (per_k && (qbk % 128 != 0 || ((qbk / 128) & (qbk / 128 - 1)) != 0)) return false;
@@ -501,23 +528,37 @@ int launch_gemm_w4i8(const Int8Args& a, const uint8_t* xq, int64_t ldq, const fl
     DecodeW4I8Args d;
     d.k = k;
     d.W = (int)(a.KT < 8 ? a.KT : 8);
-    const int ntw = (a.NT >= 512 && a.NT % 2 == 0) ? 2 : 1;
+    // (groups of 32: one, the four sets of scales do not fit the registers of two)
+    const int gsub = a.group_size == 32 ? 4 : a.group_size == 64 ? 2 : 1;
+    const int ntw = (gsub < 4 && a.NT >= 512 && a.NT % 2 == 0) ? 2 : 1;
     size_t smem = (size_t)d.W * 2 * 16 * kTileK4;
     const size_t red = (size_t)ntw * d.W * 64 * sizeof(f4);
     if (red > smem) smem = red;
     const unsigned dgrid = (unsigned)(a.NT / ntw);
     const bool per_k = sa_k_stride != 0;
-    if (ntw == 2) {
+#define WOQ_DECODE_W4I8(GS)                                                    \
+  if (ntw == 2) {                                                              \
+    if (per_k)                                                                 \
+      woq_decode_w4i8_kernel<true, 2, GS><<<dgrid, d.W * 64, smem, st>>>(d);   \
+    else                                                                       \
+      woq_decode_w4i8_kernel<false, 2, GS><<<dgrid, d.W * 64, smem, st>>>(d);  \
+  } else {                                                                     \
+    if (per_k)                                                                 \
+      woq_decode_w4i8_kernel<true, 1, GS><<<dgrid, d.W * 64, smem, st>>>(d);   \
+    else                                                                       \
+      woq_decode_w4i8_kernel<false, 1, GS><<<dgrid, d.W * 64, smem, st>>>(d);  \
+  }
+    if (gsub == 4) {
       if (per_k)
-        woq_decode_w4i8_kernel<true, 2><<<dgrid, d.W * 64, smem, st>>>(d);
+        woq_decode_w4i8_kernel<true, 1, 4><<<dgrid, d.W * 64, smem, st>>>(d);
       else
-        woq_decode_w4i8_kernel<false, 2><<<dgrid, d.W * 64, smem, st>>>(d);
+        woq_decode_w4i8_kernel<false, 1, 4><<<dgrid, d.W * 64, smem, st>>>(d);
+    } else if (gsub == 2) {
+      WOQ_DECODE_W4I8(2)
     } else {
-      if (per_k)
-        woq_decode_w4i8_kernel<true, 1><<<dgrid, d.W * 64, smem, st>>>(d);
-      else
-        woq_decode_w4i8_kernel<false, 1><<<dgrid, d.W * 64, smem, st>>>(d);
+      WOQ_DECODE_W4I8(1)
     }
+#undef WOQ_DECODE_W4I8
     return check_launch("woq_decode_w4i8_kernel");
   }
   dim3 grid((unsigned)((a.NT * kTileN + W8_BN - 1) / W8_BN), (unsigned)((a.M + W8_BM - 1) / W8_BM));
