@@ -326,9 +326,11 @@ struct DecodeW4I8Args {
   int W;  // waves per workgroup
 };
 
-template <bool PER_K, int NTW, int GSUB>
+// MT: 16-row tiles (one or two)
+template <bool PER_K, int MT, int NTW, int GSUB>
 __global__ __launch_bounds__(512, 4) void woq_decode_w4i8_kernel(const DecodeW4I8Args a) {
-  constexpr int SLICE = 16 * kTileK4;  // one buffer of one wave: 16 rows x 128 bytes
+  constexpr int SLICE = MT * 16 * kTileK4;  // one buffer of one wave: 16 MT rows x 128 bytes
+  constexpr int NX = 2 * MT;                // activation loads per tile (eight rows each)
   extern __shared__ __align__(1024) uint8_t smem[];
   const W4I8Args& k = a.k;
   const int W = a.W;
@@ -338,23 +340,25 @@ __global__ __launch_bounds__(512, 4) void woq_decode_w4i8_kernel(const DecodeW4I
   const int M = (int)k.M, KT = (int)k.KT, KG = (int)k.KG;
   const int64_t nt0 = (int64_t)blockIdx.x * NTW;
   uint8_t* const sx = smem + wave * (2 * SLICE);
-  f4* const red = (f4*)smem;  // [NTW][W][64], after the K loop
+  f4* const red = (f4*)smem;  // [NTW * MT][W][64], after the K loop
 
-  f4 acc[NTW];
+  f4 acc[NTW][MT];
 #pragma unroll
-  for (int t = 0; t < NTW; ++t) acc[t] = f4{0.f, 0.f, 0.f, 0.f};
+  for (int t = 0; t < NTW; ++t)
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) acc[t][mt] = f4{0.f, 0.f, 0.f, 0.f};
 
-  // activation load i (two per tile) fills LDS bytes [1024 i, +1024) of a buffer: rows 8 i + lane / 8,
-  // physical chunk lane % 8 = logical chunk ^ ((row / 2) % 8); rows past M re-read row M - 1
-  uint32_t xoff[2];
+  // activation load i fills LDS bytes [1024 i, +1024) of a buffer: rows 8 i + lane / 8, physical
+  // chunk lane % 8 = logical chunk ^ ((row / 2) % 8); rows past M re-read row M - 1
+  uint32_t xoff[NX];
 #pragma unroll
-  for (int i = 0; i < 2; ++i) {
+  for (int i = 0; i < NX; ++i) {
     const int row = 8 * i + (lane >> 3);
     const int rowc = row < M ? row : M - 1;
     const int chunk = (lane & 7) ^ ((row >> 1) & 7);
     xoff[i] = (uint32_t)(rowc * (int)k.ldq + chunk * 16);
   }
-  uint32_t rd[2];  // A fragment of MFMA j: row r, logical chunk 2 c + j
+  uint32_t rd[2];  // A fragment of MFMA j in row tile 0: row r, logical chunk 2 c + j
 #pragma unroll
   for (int j = 0; j < 2; ++j) rd[j] = (uint32_t)(r * 128 + (((2 * c + j) ^ ((r >> 1) & 7)) << 4));
 
@@ -370,24 +374,17 @@ __global__ __launch_bounds__(512, 4) void woq_decode_w4i8_kernel(const DecodeW4I
   }
   const uint32_t woff = (uint32_t)lane * 16u;
 
-  // activation scales of this lane's accumulator rows m = 4 c + e: one per row for the whole K, or
-  // (PER_K) one per row and K block, requested with the tile
-  f4 sa_row;
-#pragma unroll
-  for (int e = 0; e < 4; ++e) {
-    const int m = 4 * c + e;
-    sa_row[e] = PER_K ? 0.0f : k.sa[(int64_t)(m < M ? m : M - 1) * k.sa_m_stride];
-  }
-
+  // activation scales of this lane's accumulator rows m = 16 mt + 4 c + e: one per row for the whole
+  // K (applied after the sum over the waves), or (PER_K) one per row and K block, requested with the tile
   u4 wnext[NTW];
   float snext[NTW][GSUB];
   uint8_t znext[NTW];
-  f4 sanext[GSUB];
+  f4 sanext[PER_K ? GSUB : 1][PER_K ? MT : 1];
   const int my_block = c / (4 / GSUB);  // K block of the tile this lane column's weights belong to
   auto request = [&](int kt, int buf) {
     const uint32_t ko = (uint32_t)kt * kTileK4;
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < NX; ++i)
       if (8 * i < M)
         __builtin_amdgcn_global_load_lds((w8_global_ptr_t)(k.xq + (uint32_t)(xoff[i] + ko)),
                                          (w8_lds_ptr_t)(sx + buf * SLICE + i * 1024), 16, 0, 0);
@@ -403,15 +400,17 @@ __global__ __launch_bounds__(512, 4) void woq_decode_w4i8_kernel(const DecodeW4I
       // raw: any use here would wait for the load inside the request
       znext[t] = *(zbase[t] + (uint32_t)((g0 + (GSUB == 1 ? 0 : my_block)) * kTileN + r));
     }
-    if (PER_K) {
+    if constexpr (PER_K) {
 #pragma unroll
       for (int g = 0; g < GSUB; ++g)
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          const int m = 4 * c + e;
-          const int64_t kb = GSUB == 1 ? (int64_t)(kt >> k.q_shift) : (int64_t)kt * GSUB + g;
-          sanext[g][e] = k.sa[(int64_t)(m < M ? m : M - 1) * k.sa_m_stride + kb * k.sa_k_stride];
-        }
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const int m = 16 * mt + 4 * c + e;
+            const int64_t kb = GSUB == 1 ? (int64_t)(kt >> k.q_shift) : (int64_t)kt * GSUB + g;
+            sanext[g][mt][e] = k.sa[(int64_t)(m < M ? m : M - 1) * k.sa_m_stride + kb * k.sa_k_stride];
+          }
     }
   };
 
@@ -421,7 +420,7 @@ __global__ __launch_bounds__(512, 4) void woq_decode_w4i8_kernel(const DecodeW4I
     u4 wreg[NTW];
     float sw[NTW][GSUB];
     uint32_t z4[NTW];
-    f4 sa[GSUB];
+    f4 sa[PER_K ? GSUB : 1][PER_K ? MT : 1];
 #pragma unroll
     for (int t = 0; t < NTW; ++t) {
       wreg[t] = wnext[t];
@@ -429,15 +428,22 @@ __global__ __launch_bounds__(512, 4) void woq_decode_w4i8_kernel(const DecodeW4I
       for (int g = 0; g < GSUB; ++g) sw[t][g] = snext[t][g];
       z4[t] = (has_z ? (uint32_t)znext[t] : 8u) * 0x01010101u;
     }
+    if constexpr (PER_K) {
 #pragma unroll
-    for (int g = 0; g < GSUB; ++g) sa[g] = PER_K ? sanext[g] : sa_row;
+      for (int g = 0; g < GSUB; ++g)
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) sa[g][mt] = sanext[g][mt];
+    }
     // the compiler does not order LDS reads after the LDS-writing loads: wait for them here
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
     if (kt + W < KT) request(kt + W, buf ^ 1);
     __builtin_amdgcn_sched_barrier(0);
 
-    const i4 xa0 = *(const i4*)(sx + buf * SLICE + rd[0]);
-    const i4 xa1 = *(const i4*)(sx + buf * SLICE + rd[1]);
+    i4 xa[MT][2];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int j = 0; j < 2; ++j) xa[mt][j] = *(const i4*)(sx + buf * SLICE + mt * 2048 + rd[j]);
 #pragma unroll
     for (int t = 0; t < NTW; ++t) {
       const i4 bq0 = w8_decode16(wreg[t][0], wreg[t][1], z4[t]);
@@ -448,12 +454,16 @@ __global__ __launch_bounds__(512, 4) void woq_decode_w4i8_kernel(const DecodeW4I
         // (masked again for every row-block: holding GSUB masked copies costs more registers than
         // the selects cost time)
         const bool mine = GSUB == 1 || my_block == g;
-        const i4 xg0 = mine ? xa0 : i4{0, 0, 0, 0};
-        const i4 xg1 = mine ? xa1 : i4{0, 0, 0, 0};
-        i4 qc = __builtin_amdgcn_mfma_i32_16x16x64_i8(xg0, bq0, i4{0, 0, 0, 0}, 0, 0, 0);
-        qc = __builtin_amdgcn_mfma_i32_16x16x64_i8(xg1, bq1, qc, 0, 0, 0);
 #pragma unroll
-        for (int e = 0; e < 4; ++e) acc[t][e] = w8_accumulate<PER_K>(qc[e], sa[g][e], sw[t][g], acc[t][e]);
+        for (int mt = 0; mt < MT; ++mt) {
+          const i4 xg0 = mine ? xa[mt][0] : i4{0, 0, 0, 0};
+          const i4 xg1 = mine ? xa[mt][1] : i4{0, 0, 0, 0};
+          i4 qc = __builtin_amdgcn_mfma_i32_16x16x64_i8(xg0, bq0, i4{0, 0, 0, 0}, 0, 0, 0);
+          qc = __builtin_amdgcn_mfma_i32_16x16x64_i8(xg1, bq1, qc, 0, 0, 0);
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            acc[t][mt][e] = w8_accumulate<PER_K>(qc[e], PER_K ? sa[g][mt][e] : 0.0f, sw[t][g], acc[t][mt][e]);
+        }
       }
     }
   }
@@ -461,19 +471,23 @@ __global__ __launch_bounds__(512, 4) void woq_decode_w4i8_kernel(const DecodeW4I
   // ---- combine the waves' partial sums in wave order, then scale / bias / rounding / store ----
   __syncthreads();  // every wave is done with its activation slices: the region becomes `red`
 #pragma unroll
-  for (int t = 0; t < NTW; ++t) red[(t * W + wave) * 64 + lane] = acc[t];
+  for (int t = 0; t < NTW; ++t)
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) red[((t * MT + mt) * W + wave) * 64 + lane] = acc[t][mt];
   __syncthreads();
   const float* redf = (const float*)red;
   // one thread per output element, consecutive threads on consecutive columns; D[m][n] of a row
   // tile sits in lane n + 16 (m / 4), register m % 4
-  for (int idx = threadIdx.x; idx < NTW * 256; idx += blockDim.x) {
-    const int col = idx & 15, m = (idx >> 4) & 15, t = idx >> 8;
+  for (int idx = threadIdx.x; idx < NTW * MT * 256; idx += blockDim.x) {
+    const int col = idx & 15, m16 = (idx >> 4) & 15, tm = idx >> 8;
+    const int t = tm / MT, mt = tm - t * MT;
+    const int m = 16 * mt + m16;
     const int64_t n = (nt0 + t) * kTileN + col;
     if (m >= M || n >= k.N) continue;
-    const int slot = (col + 16 * (m >> 2)) * 4 + (m & 3);
+    const int slot = (col + 16 * (m16 >> 2)) * 4 + (m16 & 3);
     float part[8];
 #pragma unroll
-    for (int w = 0; w < 8; ++w) part[w] = w < W ? redf[(t * W + w) * 256 + slot] : 0.0f;
+    for (int w = 0; w < 8; ++w) part[w] = w < W ? redf[(tm * W + w) * 256 + slot] : 0.0f;
     float s = part[0];
 #pragma unroll
     for (int w = 1; w < 8; ++w) s = s + part[w];
@@ -481,6 +495,11 @@ __global__ __launch_bounds__(512, 4) void woq_decode_w4i8_kernel(const DecodeW4I
     epilogue_store<kRegimeBF16>(k.ep, m, n, s);
   }
 }
+
+// Rows the decode form is built for: one row tile with groups of 32 (four K blocks per tile), two
+// otherwise -- the per-block activation scales of more would not fit the registers, and from 33 rows
+// the 64-row tiles of the GEMM form are as fast.
+static int decode_w4i8_max_rows(int64_t group_size) { return group_size == 32 ? 16 : 32; }
 
 // 4-bit integer codes, symmetric activation scales per tensor or per row, K blocks of 128 that are
 // whole weight tiles, and a group size of 128 * 2^s (or one group), so that a K tile has one scale.
@@ -492,7 +511,8 @@ bool gemm_w4i8_applies(const Int8Args& a, int64_t block_k, int64_t qbk, bool per
   if (a.K % 128 != 0) return false;
   if (block_k == 32 || block_k == 64) {
     // groups of 32 / 64: the decode form only (K blocks inside a tile), activation blocks = groups
-    return a.M <= 16 && a.group_size == block_k && (!per_k || qbk == block_k) && a.M * a.K < ((int64_t)1 << 31);
+    return a.M <= decode_w4i8_max_rows(a.group_size) && a.group_size == block_k && (!per_k || qbk == block_k) &&
+           a.M * a.K < ((int64_t)1 << 31);
   }
   if (block_k != 128) return false;
   if (a.group_size > 0 && (a.G % 128 != 0 || ((a.G / 128) & (a.G / 128 - 1)) != 0)) return false;
@@ -523,40 +543,41 @@ int launch_gemm_w4i8(const Int8Args& a, const uint8_t* xq, int64_t ldq, const fl
     while (((int64_t)128 << k.g_shift) < a.G) ++k.g_shift;
   }
   k.ep = Epilogue{a.bias, a.fusion, a.other0, a.other1, a.out, a.out_dtype, a.x_dtype, a.N};
-  if (a.M <= 16) {
-    // decode form: 2 row-blocks per workgroup while that leaves at least 256 workgroups, else 1
+  if (a.M <= decode_w4i8_max_rows(a.group_size)) {
+    // decode form; 2 row-blocks per workgroup while that leaves at least 256 workgroups and the
+    // registers allow it, else 1
     DecodeW4I8Args d;
     d.k = k;
-    d.W = (int)(a.KT < 8 ? a.KT : 8);
-    // (groups of 32: one, the four sets of scales do not fit the registers of two)
     const int gsub = a.group_size == 32 ? 4 : a.group_size == 64 ? 2 : 1;
-    const int ntw = (gsub < 4 && a.NT >= 512 && a.NT % 2 == 0) ? 2 : 1;
-    size_t smem = (size_t)d.W * 2 * 16 * kTileK4;
-    const size_t red = (size_t)ntw * d.W * 64 * sizeof(f4);
+    const int mt = a.M > 16 ? 2 : 1;
+    const int ntw = (gsub * mt <= 2 && a.NT >= 512 && a.NT % 2 == 0) ? 2 : 1;
+    const int slice = mt * 16 * kTileK4;
+    int w = 65536 / (2 * slice);  // at most 64 KiB of activation slices
+    if (w > 8) w = 8;
+    d.W = (int)(a.KT < w ? a.KT : w);
+    size_t smem = (size_t)d.W * 2 * slice;
+    const size_t red = (size_t)ntw * mt * d.W * 64 * sizeof(f4);
     if (red > smem) smem = red;
     const unsigned dgrid = (unsigned)(a.NT / ntw);
     const bool per_k = sa_k_stride != 0;
-#define WOQ_DECODE_W4I8(GS)                                                    \
-  if (ntw == 2) {                                                              \
-    if (per_k)                                                                 \
-      woq_decode_w4i8_kernel<true, 2, GS><<<dgrid, d.W * 64, smem, st>>>(d);   \
-    else                                                                       \
-      woq_decode_w4i8_kernel<false, 2, GS><<<dgrid, d.W * 64, smem, st>>>(d);  \
-  } else {                                                                     \
-    if (per_k)                                                                 \
-      woq_decode_w4i8_kernel<true, 1, GS><<<dgrid, d.W * 64, smem, st>>>(d);   \
-    else                                                                       \
-      woq_decode_w4i8_kernel<false, 1, GS><<<dgrid, d.W * 64, smem, st>>>(d);  \
-  }
+#define WOQ_DECODE_W4I8(MTV, NTWV, GS)                                                  \
+  do {                                                                                  \
+    if (per_k)                                                                          \
+      woq_decode_w4i8_kernel<true, MTV, NTWV, GS><<<dgrid, d.W * 64, smem, st>>>(d);    \
+    else                                                                                \
+      woq_decode_w4i8_kernel<false, MTV, NTWV, GS><<<dgrid, d.W * 64, smem, st>>>(d);   \
+  } while (0)
     if (gsub == 4) {
-      if (per_k)
-        woq_decode_w4i8_kernel<true, 1, 4><<<dgrid, d.W * 64, smem, st>>>(d);
-      else
-        woq_decode_w4i8_kernel<false, 1, 4><<<dgrid, d.W * 64, smem, st>>>(d);
+      WOQ_DECODE_W4I8(1, 1, 4);
     } else if (gsub == 2) {
-      WOQ_DECODE_W4I8(2)
+      if (mt == 2) WOQ_DECODE_W4I8(2, 1, 2);
+      else if (ntw == 2) WOQ_DECODE_W4I8(1, 2, 2);
+      else WOQ_DECODE_W4I8(1, 1, 2);
     } else {
-      WOQ_DECODE_W4I8(1)
+      if (mt == 2 && ntw == 2) WOQ_DECODE_W4I8(2, 2, 1);
+      else if (mt == 2) WOQ_DECODE_W4I8(2, 1, 1);
+      else if (ntw == 2) WOQ_DECODE_W4I8(1, 2, 1);
+      else WOQ_DECODE_W4I8(1, 1, 1);
     }
 #undef WOQ_DECODE_W4I8
     return check_launch("woq_decode_w4i8_kernel");

@@ -800,6 +800,18 @@ def test_int8_lowp_other_groups(cuda, G, M):
     _check_int8(case, 6, label=f"int8 lowp G={G} M={M} per-M")
 
 
+@pytest.mark.parametrize("mode", [4, 5, 6, 7])
+@pytest.mark.parametrize("M,K,N,G", [(17, 1024, 272, 128), (32, 2048, 1040, 64), (9, 512, 144, 32), (16, 1152, 96, -1),
+                                     (25, 1024, 8208, 256), (2, 384, 48, 64)])
+def test_int8_lowp_decode_kernel(cuda, mode, M, K, N, G):
+    """The int8 MFMA decode kernel: one or two row tiles, groups of 32 / 64 as K blocks inside a tile,
+    two row-blocks per workgroup for wide layers; the general kernel (debug run) supplies the bit-exact
+    block sums, this one the outputs."""
+    case = _synthetic().make_int4_case(22, M, K, N, G, bias=True, outliers=True)
+    cols = None if N < 4096 else list(range(0, N, 53)) + [N - 1]
+    _check_int8(case, mode, cols=cols, debug=N < 4096, label=f"int8 lowp decode mode={mode} M={M} K={K} N={N} G={G}")
+
+
 def test_int8_lowp_int8_weights(cuda):
     for M in (2, 20, 140):
         case = _synthetic().make_int8_case(22, M, 512, 80)
