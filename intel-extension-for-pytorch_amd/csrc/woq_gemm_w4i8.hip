@@ -1,5 +1,6 @@
-// int8 MFMA GEMM for 4-bit weights and large M under lowp_mode INT8 (prefill): symmetric activation
-// quantization (per tensor, per row, per K block or per row and K block), K blocks of 128.
+// int8 MFMA kernels for 4-bit weights under lowp_mode INT8: the GEMM form for large M (prefill,
+// below) and the decode form for up to 32 rows (further down); symmetric activation quantization
+// (per tensor, per row, per K block or per row and K block), K blocks of 128.
 //
 // Reference counterpart: Dequantize<int8_t> of a [128 x 32] weight block, int8 BRGEMM into int32,
 // then the fp32 epilogue C += (float(sum) * s_a[m]) * s_w[n, g] per K block
@@ -503,9 +504,9 @@ static int decode_w4i8_max_rows(int64_t group_size) { return group_size == 32 ? 
 
 // 4-bit integer codes, symmetric activation scales per tensor or per row, K blocks of 128 that are
 // whole weight tiles, and a group size of 128 * 2^s (or one group), so that a K tile has one scale.
-// Up to 16 rows run on the decode form (woq_decode_w4i8_kernel); from 17 rows the 64-row tiles of the
-// MFMA GEMM, which with a single row tile still beats the general small-M kernel (4096 -> 14336, per-row
-// scales, M = 32 / 48 / 64: 31 / 34 / 36 us against 50 / 157 / 162 us).
+// Up to 32 rows run on the decode form (woq_decode_w4i8_kernel; M = 32: 14 us), from 33 rows on the
+// 64-row tiles of the MFMA GEMM, which with a single row tile still beats the general small-M kernel
+// (4096 -> 14336, per-row scales, M = 48 / 64: 34 / 36 us against 157 / 162 us).
 bool gemm_w4i8_applies(const Int8Args& a, int64_t block_k, int64_t qbk, bool per_k, bool asym) {
   if (a.wbits != 4 || a.nf4 || asym || a.debug_block_sums) return false;
   if (a.K % 128 != 0) return false;
