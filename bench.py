@@ -164,15 +164,19 @@ def time_graph(torch, lib, params, steps, warmup):
     return reps * n, t1 - t0, start.elapsed_time(stop)
 
 
-def _rotating_params(torch, lib_mod, ops_mod, case, lowp_mode, dev, stream, min_bytes=640e6):
+def _rotating_params(torch, lib_mod, ops_mod, case, lowp_mode, dev, stream, min_bytes=640e6, act_quant_mode=-1):
     """One op context per weight copy (enough copies that the working set exceeds the Infinity
     Cache), the launch parameters of each, and the objects that keep the memory alive."""
     M, K, N, G = case["M"], case["K"], case["N"], case["group_size"]
     ctx0 = ops_mod.WoqLinearOpContext(
         case["qweight"].to(dev), case["weight_dtype"], [N, K], case["scales"].to(dev),
         None if case["zeros"] is None else case["zeros"].to(dev),
-        None if case["bias"] is None else case["bias"].to(dev), None, None, G, lowp_mode, -1,
+        None if case["bias"] is None else case["bias"].to(dev), None, None, G, lowp_mode, act_quant_mode,
     )
+    ws = None
+    if lowp_mode == 3:  # the quantized activations; one block for every launch of this stream
+        ws = torch.empty(lib_mod.load().woq_hip_linear_workspace_bytes(M, K, 3, act_quant_mode, G), dtype=torch.uint8,
+                         device=dev)
     copies = int(min_bytes // ctx0.at_weight_.numel()) + 1
     x = case["x"].to(dev)
     out = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
@@ -190,9 +194,10 @@ def _rotating_params(torch, lib_mod, ops_mod, case, lowp_mode, dev, stream, min_
             c.zeros_u8_ = None if ctx0.zeros_u8_ is None else ctx0.zeros_u8_.clone()
             c.scale_zero_f16x2_ = None if ctx0.scale_zero_f16x2_ is None else ctx0.scale_zero_f16x2_.clone()
         keep.append(c)
-        p = build_params(lib_mod, x, c, out, lowp_mode)
+        p = build_params(lib_mod, x, c, out, lowp_mode, act_quant_mode, ws)
         p.stream = stream.cuda_stream
         params.append(p)
+    keep.append(ws)
     return params, keep
 
 
@@ -203,9 +208,9 @@ def config_sweep(torch, lib, lib_mod, ops_mod, synthetic, dev, stream, steps):
     and outputs."""
     rows = []
 
-    def run(name, case):
+    def run(name, case, lowp=2, aq=-1):
         M, K, N, G = case["M"], case["K"], case["N"], case["group_size"]
-        params, keep = _rotating_params(torch, lib_mod, ops_mod, case, 2, dev, stream)
+        params, keep = _rotating_params(torch, lib_mod, ops_mod, case, lowp, dev, stream, act_quant_mode=aq)
         # Each configuration starts after an idle period (its inputs are generated on the host) and
         # the first few thousand launches after one run up to 10 % slower; single groups of a few
         # hundred launches also scatter by +-5 %.  So: a warm-up as long as one group, then nine
@@ -217,9 +222,15 @@ def config_sweep(torch, lib, lib_mod, ops_mod, synthetic, dev, stream, steps):
             nbytes = algorithmic_bytes(M, K, N, G)
         else:
             nbytes = N * K + N * 4 + M * K * 2 + M * N * 2 + (N * 2 if case["bias"] is not None else 0)
-        rows.append({"config": name, "M": M, "K": K, "N": N, "group_size": G, "us_per_launch": round(us, 2),
-                     "us_p10_p90": [round(groups[1], 2), round(groups[7], 2)],
-                     "GB_per_s": round(nbytes / us / 1e3, 1), "frac_of_hbm_peak": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 3)})
+        row = {"config": name, "M": M, "K": K, "N": N, "group_size": G, "us_per_launch": round(us, 2),
+               "us_p10_p90": [round(groups[1], 2), round(groups[7], 2)]}
+        if M >= 256:  # MFMA-bound: a rate in flops, not in bytes
+            row["tflops"] = round(2.0 * M * K * N / us / 1e6, 1)
+            row["frac_of_bf16_mfma_peak"] = round(2.0 * M * K * N / us / 1e6 / MFMA_BF16_PEAK_TFLOPS, 3)
+        else:
+            row["GB_per_s"] = round(nbytes / us / 1e3, 1)
+            row["frac_of_hbm_peak"] = round(nbytes / us / 1e3 / HBM_PEAK_GBS, 3)
+        rows.append(row)
         del params, keep
         torch.cuda.empty_cache()
 
@@ -234,6 +245,14 @@ def config_sweep(torch, lib, lib_mod, ops_mod, synthetic, dev, stream, steps):
         run(f"C4 int4 g32 M=16 {what} {K}->{N}", synthetic.make_int4_case(4, 16, K, N, 32))
         block += rows[-1]["us_per_launch"]
     rows.append({"config": "C4 decoder block, summed WOQ-linear time per token step", "us": round(block, 2)})
+    # Beyond the named configurations: what the same layers cost in the neighbouring settings a user of
+    # the reference may run (single-stream decode of a group-32 model, lowp_mode INT8 decode with
+    # per-row and per-(row, K block) activation scales, INT8 weights at prefill size).
+    run("extra: int4 g32 M=1 4096->14336 (lowp BF16)", synthetic.make_int4_case(5, 1, 4096, 14336, 32))
+    run("extra: int4 g128 M=1 4096->14336 lowp INT8 per-row", synthetic.make_int4_case(5, 1, 4096, 14336, 128), 3, 6)
+    run("extra: int4 g128 M=16 4096->14336 lowp INT8 per-row-and-K-block", synthetic.make_int4_case(5, 16, 4096, 14336, 128), 3, 7)
+    run("extra: int4 g32 M=1 4096->14336 lowp INT8 per-row-and-K-block", synthetic.make_int4_case(5, 1, 4096, 14336, 32), 3, 7)
+    run("extra: int8 per-channel M=2048 4096->11008 +bias (lowp BF16)", synthetic.make_int8_case(5, 2048, 4096, 11008))
     return rows
 
 
