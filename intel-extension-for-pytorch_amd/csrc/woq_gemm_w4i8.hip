@@ -327,9 +327,10 @@ struct DecodeW4I8Args {
   int W;  // waves per workgroup
 };
 
-// MT: 16-row tiles (one or two)
+// MT: 16-row tiles (one, two or four).  The forms with many K blocks and row tiles keep GSUB x MT sets of
+// activation scales in flight and get the registers of two waves per SIMD instead of four.
 template <bool PER_K, int MT, int NTW, int GSUB>
-__global__ __launch_bounds__(512, 4) void woq_decode_w4i8_kernel(const DecodeW4I8Args a) {
+__global__ __launch_bounds__(512, (GSUB * MT > 4 ? 2 : 4)) void woq_decode_w4i8_kernel(const DecodeW4I8Args a) {
   constexpr int SLICE = MT * 16 * kTileK4;  // one buffer of one wave: 16 MT rows x 128 bytes
   constexpr int NX = 2 * MT;                // activation loads per tile (eight rows each)
   extern __shared__ __align__(1024) uint8_t smem[];
@@ -497,10 +498,10 @@ __global__ __launch_bounds__(512, 4) void woq_decode_w4i8_kernel(const DecodeW4I
   }
 }
 
-// Rows the decode form is built for: one row tile with groups of 32 (four K blocks per tile), two
-// otherwise -- the per-block activation scales of more would not fit the registers, and from 33 rows
-// the 64-row tiles of the GEMM form are as fast.
-static int decode_w4i8_max_rows(int64_t group_size) { return group_size == 32 ? 16 : 32; }
+// Rows the decode form takes: up to 32 for groups of at least 128 (from 33 rows the 64-row tiles of the
+// GEMM form are as fast), and for groups of 64 / 32, which the GEMM form does not take, up to 64 / 32
+// (four row tiles times four K blocks of activation scales do not fit the registers).
+static int decode_w4i8_max_rows(int64_t group_size) { return group_size == 64 ? 64 : 32; }
 
 // 4-bit integer codes, symmetric activation scales per tensor or per row, K blocks of 128 that are
 // whole weight tiles, and a group size of 128 * 2^s (or one group), so that a K tile has one scale.
@@ -550,7 +551,7 @@ int launch_gemm_w4i8(const Int8Args& a, const uint8_t* xq, int64_t ldq, const fl
     DecodeW4I8Args d;
     d.k = k;
     const int gsub = a.group_size == 32 ? 4 : a.group_size == 64 ? 2 : 1;
-    const int mt = a.M > 16 ? 2 : 1;
+    const int mt = a.M > 32 ? 4 : a.M > 16 ? 2 : 1;
     const int ntw = (gsub * mt <= 2 && a.NT >= 512 && a.NT % 2 == 0) ? 2 : 1;
     const int slice = mt * 16 * kTileK4;
     int w = 65536 / (2 * slice);  // at most 64 KiB of activation slices
@@ -569,9 +570,11 @@ int launch_gemm_w4i8(const Int8Args& a, const uint8_t* xq, int64_t ldq, const fl
       woq_decode_w4i8_kernel<false, MTV, NTWV, GS><<<dgrid, d.W * 64, smem, st>>>(d);   \
   } while (0)
     if (gsub == 4) {
-      WOQ_DECODE_W4I8(1, 1, 4);
+      if (mt == 2) WOQ_DECODE_W4I8(2, 1, 4);
+      else WOQ_DECODE_W4I8(1, 1, 4);
     } else if (gsub == 2) {
-      if (mt == 2) WOQ_DECODE_W4I8(2, 1, 2);
+      if (mt == 4) WOQ_DECODE_W4I8(4, 1, 2);
+      else if (mt == 2) WOQ_DECODE_W4I8(2, 1, 2);
       else if (ntw == 2) WOQ_DECODE_W4I8(1, 2, 2);
       else WOQ_DECODE_W4I8(1, 1, 2);
     } else {
