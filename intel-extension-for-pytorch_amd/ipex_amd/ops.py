@@ -28,6 +28,12 @@ import torch
 
 from . import _kernels, _lib
 
+_NO_GUARD = contextlib.nullcontext()
+_current_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None) or (
+    lambda index: torch.cuda.current_stream(index).cuda_stream
+)
+_current_device = getattr(torch._C, "_cuda_getDevice", None) or torch.cuda.current_device
+
 WOQ_DTYPE_MAP = {"int8": _lib.DTYPE_INT8, "int4": _lib.DTYPE_INT4, "nf4": _lib.DTYPE_NF4}
 PLAIN_WEIGHT_FORMAT, GPTQ_WEIGHT_FORMAT, AWQ_WEIGHT_FORMAT = 0, 1, 2
 
@@ -282,8 +288,11 @@ class WoqLinearOpContext:
             else:
                 p.others[i] = None
         lib = _lib.load()
-        with contextlib.nullcontext() if x.device.index == torch.cuda.current_device() else torch.cuda.device(x.device):
-            p.stream = torch.cuda.current_stream().cuda_stream
+        dev_index = x.device.index
+        with _NO_GUARD if dev_index == _current_device() else torch.cuda.device(x.device):
+            # the raw handle of the current stream: torch.cuda.current_stream() builds a Stream object
+            # around it, 2.8 us of a call whose kernel takes 5-8 us
+            p.stream = _current_raw_stream(dev_index)
             ws = counters = None
             if M <= 32 and K >= 8192 and N <= 4096:
                 # long K, few output columns: scratch with which the decode kernel may share K between
