@@ -464,7 +464,10 @@ def test_dequantizing_decode_kernel_split_k_nf4_and_fp16(cuda):
         assert rel_l2(got, want) <= 1e-3, kernel
 
 
-@pytest.mark.parametrize("M,K,N,G", [(16, 8192, 4096, 128), (8, 14336, 512, 128), (32, 8192, 2048, 32)])
+# (16 x 125 and 2 x 61 row-block sets: the two workgroups of a set sit 125 / 61 places apart in the launch
+# order, i.e. on different XCDs, whose L2 caches are not coherent with each other)
+@pytest.mark.parametrize("M,K,N,G", [(16, 8192, 4096, 128), (8, 14336, 512, 128), (32, 8192, 2048, 32),
+                                     (16, 8192, 2000, 128), (12, 16384, 1952, 64)])
 def test_dequantizing_decode_kernel_splits_k_by_itself_for_long_k(cuda, M, K, N, G):
     """Few output columns and K >= 8192: the automatic choice shares K between two workgroups.  The
     result must not depend on which workgroup finishes last (the partial tiles are added in split
