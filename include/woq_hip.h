@@ -221,7 +221,8 @@ typedef struct woq_hip_linear_params {
    * 11 / 12 = the same prefill GEMM with 256 rows x 192 columns / 64 rows x 128 columns per workgroup
    * (8-bit weights: 5, 6 and 12 only);
    * 13..17 = the dequantizing decode kernel (M <= 32) with (row-blocks per workgroup, K splits) =
-   * (1, 2), (2, 2), (4, 2), (2, 4), (4, 4): needs workspace and split_k_counters.
+   * (1, 2), (2, 2), (4, 2), (2, 4), (4, 4): needs workspace and split_k_counters;
+   * 19 / 20 = the prefill GEMM with 64 x 128 tiles and K shared by two / four workgroups per tile (same needs).
    * NF4 weights: 0, 1, 2, 7, 8, 9, 13, 14, 16 only */
   int32_t force_kernel;
 
@@ -232,7 +233,8 @@ int64_t woq_hip_linear_workspace_bytes(int64_t M, int64_t K, int32_t lowp_mode,
                                        int32_t act_quant_mode, int64_t group_size);
 
 /* Scratch bytes that let woq_hip_linear split K across workgroups for M rows and N output columns
- * in the floating-point modes; 0 where it never does (M > 32).  No counterpart in the reference. */
+ * in the floating-point modes (decode kernel up to 32 rows; prefill GEMM when its 64 x 128 tiles are
+ * at most 128); 0 where it never does.  No counterpart in the reference. */
 int64_t woq_hip_linear_split_k_workspace_bytes(int64_t M, int64_t N);
 
 /* K-block of the int8 path: min(group_size, 128), per-channel -> 128

@@ -115,7 +115,14 @@ int64_t woq_hip_linear_workspace_bytes(int64_t M, int64_t K, int32_t lowp_mode, 
 }
 
 int64_t woq_hip_linear_split_k_workspace_bytes(int64_t M, int64_t N) {
-  if (M <= 0 || M > 32 || N <= 0) return 0;
+  if (M <= 0 || N <= 0) return 0;
+  if (M > 64) {
+    // prefill GEMM, 64 x 128 tiles, up to four workgroups per tile while the tiles alone fill less than
+    // half of the chip
+    const int64_t tiles = ((M + 63) / 64) * ((woq_hip_padded_n(N) + 127) / 128);
+    return tiles <= 128 ? 4 * tiles * 64 * 128 * (int64_t)sizeof(float) : 0;
+  }
+  if (M > 32) return 0;
   const int64_t NT = woq_hip_padded_n(N) / kTileN;
   if (NT > 4 * kSplitKCounters) return 0;
   return decode_dq_splitk_bytes(M, NT, kSplitKMax);
@@ -257,14 +264,18 @@ int woq_hip_linear(const woq_hip_linear_params* p) {
       kernel = w4 ? 3 : 2;
   }
   if (kernel == 1 && p->M > 64) return set_error("woq_linear: the small-M kernel takes M <= 64");
-  const int w4_shape = kernel == 4 ? 7 : kernel == 5 ? 4 : kernel == 6 ? 2 : kernel == 11 ? 163 : kernel == 12 ? 42 : 0;
-  if ((kernel >= 4 && kernel <= 6) || kernel == 11 || kernel == 12) kernel = 3;
+  const int w4_shape = kernel == 4 ? 7 : kernel == 5 ? 4 : kernel == 6 ? 2 : kernel == 11 ? 163
+                       : (kernel == 12 || kernel == 19 || kernel == 20) ? 42 : 0;
+  // forced shapes run unsplit, 19 / 20 split K in two / four; the automatic choice may split
+  const int w4_splits = kernel == 19 ? 2 : kernel == 20 ? 4 : kernel == 3 || kernel == 0 ? 0 : 1;
+  if ((kernel >= 4 && kernel <= 6) || kernel == 11 || kernel == 12 || kernel == 19 || kernel == 20) kernel = 3;
   if (kernel == 3 && !gemm_w4_applies(f, wbits, regime))
     return set_error("woq_linear: the prefill kernel takes 4-bit integer weights (or 8-bit ones with groups of at "
                      "least 128), K %% 128 == 0, a power-of-two or per-channel group size and activations in the "
                      "compute dtype");
   if (kernel == 1) return launch_small_m(f, wbits, regime, st);
-  return kernel == 3 ? launch_gemm_w4(f, wbits, regime, st, w4_shape) : launch_gemm(f, wbits, regime, st);
+  return kernel == 3 ? launch_gemm_w4(f, wbits, regime, st, w4_shape, w4_splits, &scratch)
+                     : launch_gemm(f, wbits, regime, st);
 }
 
 int woq_hip_dequant_weight(const void* qweight, int weight_dtype, int64_t N, int64_t K, const float* scales_f32,

@@ -69,8 +69,14 @@ __device__ __forceinline__ f4 g4_mfma(u4 a, u4 b, f4 c) {
 typedef __attribute__((address_space(3))) void* lds_ptr_t;
 typedef const __attribute__((address_space(1))) void* global_ptr_t;
 
+// gridDim.z > 1 (small M x N with a long K, where the tiles alone leave most CUs idle): workgroup z
+// of a tile takes the K steps [z * kts, (z + 1) * kts), writes its accumulators to scratch memory as they
+// lie in the registers, and the workgroup that arrives last at the tile's counter adds the partial
+// tiles in z order (its own from the registers) and runs the epilogue.  Nobody waits; the order of
+// the sum is fixed.  All scratch accesses are relaxed device-scope atomics, as in the decode kernel.
 template <int REGIME, class S, int WBITS>
-__global__ __launch_bounds__(256) void woq_gemm_w4_kernel(const FpArgs f, const int g_shift) {
+__global__ __launch_bounds__(256) void woq_gemm_w4_kernel(const FpArgs f, const int g_shift, float* const sk_partial,
+                                                          int* const sk_counters, const int kts) {
   constexpr int TPS = WBITS / 4;  // packed tiles per row-block and K step of 128
   constexpr int G4_MT = S::MT, G4_NTW = S::NTW, G4_BM = S::BM, G4_XBYTES = S::XBYTES, G4_XLOADS = S::XLOADS,
                 G4_WSTAGE = S::WSTAGE * TPS, G4_SSTRIDE = S::SSTRIDE;
@@ -84,7 +90,10 @@ __global__ __launch_bounds__(256) void woq_gemm_w4_kernel(const FpArgs f, const 
   const int r = lane & 15, c = lane >> 4;
   const int M = (int)f.M, K = (int)f.K, NT = (int)f.NT, KG = (int)f.KG;
   const int KTW = (int)f.KT;   // packed tiles along K of a row-block
-  const int KT = KTW / TPS;    // K steps of 128
+  // K steps of 128 of this workgroup: [kt_lo, KT); kts is even, so the buffer parity of a step is
+  // that of its number whatever the split
+  const int kt_lo = (int)blockIdx.z * kts;
+  const int KT = KTW / TPS < kt_lo + kts ? KTW / TPS : kt_lo + kts;
   const int m0 = blockIdx.y * G4_BM;
   const int nt0 = (blockIdx.x * G4_WAVES + wave) * G4_NTW;  // first row-block of this wave
 
@@ -209,10 +218,10 @@ __global__ __launch_bounds__(256) void woq_gemm_w4_kernel(const FpArgs f, const 
   static_assert(kStepLoads < 64 && G4_NTW * TPS < 16, "s_waitcnt vmcnt is a 6-bit field");
   constexpr int kVmcntStep = 0x0F70 | (kStepLoads & 15) | ((kStepLoads >> 4) << 14);
 
-  load_x(0, 0);
-  dma_w(0, 0);
-  dma_w(KT > 1 ? 1 : 0, 1);
-  load_q(0, sr, zr);
+  load_x(kt_lo, 0);
+  dma_w(kt_lo, 0);
+  dma_w(KT > kt_lo + 1 ? kt_lo + 1 : kt_lo, 1);
+  load_q(kt_lo, sr, zr);
   __builtin_amdgcn_s_waitcnt(kVmcnt0);
   __syncthreads();
 #pragma unroll
@@ -233,7 +242,7 @@ __global__ __launch_bounds__(256) void woq_gemm_w4_kernel(const FpArgs f, const 
 #pragma unroll
     for (int t = 0; t < G4_NTW; ++t) asm volatile("" : "+a"(acc[mt][t]));
 
-  for (int kt = 0; kt < KT; ++kt) {
+  for (int kt = kt_lo; kt < KT; ++kt) {
     const uint8_t* xs = sX + (kt & 1) * G4_XBYTES;
     const uint8_t* xsn = sX + ((kt & 1) ^ 1) * G4_XBYTES;
     // ---- requests, in this order (s_waitcnt vmcnt counts from the youngest): parameters and
@@ -307,6 +316,53 @@ __global__ __launch_bounds__(256) void woq_gemm_w4_kernel(const FpArgs f, const 
   for (int mt = 0; mt < G4_MT; ++mt)
 #pragma unroll
     for (int t = 0; t < G4_NTW; ++t) asm volatile("" : "+a"(acc[mt][t]));
+
+  if (gridDim.z > 1) {
+    const int nsplit = (int)gridDim.z, z = (int)blockIdx.z;
+    const int tiles = (int)(gridDim.x * gridDim.y), tile = (int)(blockIdx.y * gridDim.x + blockIdx.x);
+    constexpr int kWaveFloats = G4_MT * G4_NTW * 256;
+    float* const mine = sk_partial + ((size_t)(z * tiles + tile) * G4_WAVES + wave) * kWaveFloats + lane * 4;
+#pragma unroll
+    for (int mt = 0; mt < G4_MT; ++mt)
+#pragma unroll
+      for (int t = 0; t < G4_NTW; ++t)
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          __hip_atomic_store(mine + (mt * G4_NTW + t) * 256 + e, acc[mt][t][e], __ATOMIC_RELAXED,
+                             __HIP_MEMORY_SCOPE_AGENT);
+    __builtin_amdgcn_s_waitcnt(kVmcnt0);  // this thread's stores have completed
+    __syncthreads();
+    __shared__ int s_last;
+    if (tid == 0)
+      s_last = __hip_atomic_fetch_add(sk_counters + tile, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == nsplit - 1;
+    __syncthreads();
+    if (!s_last) return;
+#pragma unroll
+    for (int mt = 0; mt < G4_MT; ++mt)
+#pragma unroll
+      for (int t = 0; t < G4_NTW; ++t) {
+        f4 sum = f4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll 1
+        for (int zz = 0; zz < nsplit; ++zz) {
+          f4 v = acc[mt][t];
+          if (zz != z) {
+            const float* const other = sk_partial + ((size_t)(zz * tiles + tile) * G4_WAVES + wave) * kWaveFloats +
+                                       lane * 4 + (mt * G4_NTW + t) * 256;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) v[e] = __hip_atomic_load(other + e, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          }
+          if (zz == 0) {
+            sum = v;
+          } else {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) sum[e] = sum[e] + v[e];
+          }
+        }
+        acc[mt][t] = sum;
+      }
+    // the counter is back at zero for the next launch that uses it
+    if (tid == 0) __hip_atomic_store(sk_counters + tile, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
 
   // ---- epilogue: D[m][n], lane (n = r, c) holds rows m = 16 mt + 4 c + e.  Each wave transposes
   // one 16 x (16 NTW) accumulator tile at a time through its own LDS region (the activation buffers are
@@ -384,7 +440,8 @@ bool gemm_w4_applies(const FpArgs& f, int wbits, int regime) {
 }
 
 template <int REGIME, class S, int WBITS = 4>
-static int launch_shape(const FpArgs& f, int g_shift, hipStream_t st) {
+static int launch_shape(const FpArgs& f, int g_shift, hipStream_t st, int splits = 1,
+                        const SplitKScratch* scratch = nullptr) {
   constexpr int kLds = g4_lds_bytes<S, WBITS>();
   static_assert(kLds <= 160 * 1024, "a workgroup's LDS");
   // more than 64 KiB of LDS per workgroup needs an opt-in (once per kernel and process)
@@ -393,8 +450,22 @@ static int launch_shape(const FpArgs& f, int g_shift, hipStream_t st) {
                           hipFuncAttributeMaxDynamicSharedMemorySize, kLds);
   if (lds_optin != hipSuccess)
     return set_error("woq_gemm_w4_kernel: LDS opt-in failed: %s", hipGetErrorString(lds_optin));
-  dim3 grid((unsigned)((f.NT * kTileN + S::BN - 1) / S::BN), (unsigned)((f.M + S::BM - 1) / S::BM));
-  woq_gemm_w4_kernel<REGIME, S, WBITS><<<grid, 256, kLds, st>>>(f, g_shift);
+  dim3 grid((unsigned)((f.NT * kTileN + S::BN - 1) / S::BN), (unsigned)((f.M + S::BM - 1) / S::BM),
+            (unsigned)splits);
+  const int ksteps = (int)(f.KT / (WBITS / 4));
+  int kts = ksteps;
+  if (splits > 1) {
+    kts = ((ksteps + splits - 1) / splits + 1) & ~1;  // even, so that every workgroup starts on buffer 0
+    const int64_t tiles = (int64_t)grid.x * grid.y;
+    const int64_t need = (int64_t)splits * tiles * S::BM * S::BN * (int64_t)sizeof(float);
+    if ((int64_t)(splits - 1) * kts >= ksteps)
+      return set_error("woq_gemm_w4_kernel: %d K steps are too few for %d splits", ksteps, splits);
+    if (!scratch || !scratch->partial || !scratch->counters || scratch->bytes < need || tiles > kSplitKCounters)
+      return set_error("woq_gemm_w4_kernel: split K needs %lld bytes of workspace, the counter array and at most %d "
+                       "tiles", (long long)need, kSplitKCounters);
+  }
+  woq_gemm_w4_kernel<REGIME, S, WBITS><<<grid, 256, kLds, st>>>(f, g_shift, splits > 1 ? scratch->partial : nullptr,
+                                                                 splits > 1 ? scratch->counters : nullptr, kts);
   return check_launch("woq_gemm_w4_kernel");
 }
 
@@ -406,7 +477,20 @@ static double shape_cost(const FpArgs& f) {
   return (double)(int64_t)((wgs + 255) / 256) * (S::NTW + 1.0);
 }
 
-int launch_gemm_w4(const FpArgs& f, int wbits, int regime, hipStream_t st, int shape) {
+// K splits of the 64 x 128 shape: 4 or 2 workgroups per tile while that stays within 256 workgroups,
+// leaves each at least 16 K steps and the caller's scratch suffices (14336 -> 4096, M = 128: 64 tiles).
+static int pick_splits(const FpArgs& f, int wbits, int64_t tiles, const SplitKScratch* scratch) {
+  if (!scratch || !scratch->partial || !scratch->counters || tiles > kSplitKCounters) return 1;
+  const int64_t ksteps = f.KT / (wbits / 4);
+  for (int s = 4; s >= 2; s -= 2) {
+    const int64_t need = (int64_t)s * tiles * 64 * 128 * (int64_t)sizeof(float);
+    if (tiles * s <= 256 && ksteps / s >= 16 && scratch->bytes >= need) return s;
+  }
+  return 1;
+}
+
+int launch_gemm_w4(const FpArgs& f, int wbits, int regime, hipStream_t st, int shape, int splits,
+                   const SplitKScratch* scratch) {
   int g_shift = 30;
   if (f.G < f.KT * (wbits == 4 ? kTileK4 : kTileK8)) {
     g_shift = 0;
@@ -431,13 +515,14 @@ int launch_gemm_w4(const FpArgs& f, int wbits, int regime, hipStream_t st, int s
     // (128 x 256, 128 x 128 and 64 x 128 workgroup tiles), chosen like the 4-bit ones
     if (shape != 0 && shape != 4 && shape != 2 && shape != 42)
       return set_error("woq_gemm_w4_kernel: 8-bit weights take the 128 x 256, 128 x 128 and 64 x 128 shapes");
-    if (shape == 0) {
-      const int64_t wgs42 = ((f.NT * kTileN + S42::BN - 1) / S42::BN) * ((f.M + S42::BM - 1) / S42::BM);
-      shape = wgs42 <= 256 ? 42 : (shape_cost<S4>(f) <= shape_cost<S2>(f) ? 4 : 2);
+    const int64_t wgs42 = ((f.NT * kTileN + S42::BN - 1) / S42::BN) * ((f.M + S42::BM - 1) / S42::BM);
+    if (shape == 0) shape = wgs42 <= 256 ? 42 : (shape_cost<S4>(f) <= shape_cost<S2>(f) ? 4 : 2);
+    if (shape == 42) {
+      if (splits == 0) splits = pick_splits(f, 8, wgs42, scratch);
+      return regime == kRegimeF16 ? launch_shape<kRegimeF16, S42, 8>(f, g_shift, st, splits, scratch)
+                                  : launch_shape<kRegimeBF16, S42, 8>(f, g_shift, st, splits, scratch);
     }
-    if (shape == 42)
-      return regime == kRegimeF16 ? launch_shape<kRegimeF16, S42, 8>(f, g_shift, st)
-                                  : launch_shape<kRegimeBF16, S42, 8>(f, g_shift, st);
+    if (splits > 1) return set_error("woq_gemm_w4_kernel: K is split for the 64 x 128 shape only");
     if (shape == 4)
       return regime == kRegimeF16 ? launch_shape<kRegimeF16, S4, 8>(f, g_shift, st)
                                   : launch_shape<kRegimeBF16, S4, 8>(f, g_shift, st);
@@ -452,9 +537,13 @@ int launch_gemm_w4(const FpArgs& f, int wbits, int regime, hipStream_t st, int s
     const int64_t wgs42 = ((f.NT * kTileN + S42::BN - 1) / S42::BN) * ((f.M + S42::BM - 1) / S42::BM);
     if (wgs42 <= 256) shape = 42;
   }
-  if (shape == 42)
-    return regime == kRegimeF16 ? launch_shape<kRegimeF16, S42>(f, g_shift, st)
-                                : launch_shape<kRegimeBF16, S42>(f, g_shift, st);
+  if (shape == 42) {
+    const int64_t wgs42 = ((f.NT * kTileN + S42::BN - 1) / S42::BN) * ((f.M + S42::BM - 1) / S42::BM);
+    if (splits == 0) splits = pick_splits(f, 4, wgs42, scratch);
+    return regime == kRegimeF16 ? launch_shape<kRegimeF16, S42>(f, g_shift, st, splits, scratch)
+                                : launch_shape<kRegimeBF16, S42>(f, g_shift, st, splits, scratch);
+  }
+  if (splits > 1) return set_error("woq_gemm_w4_kernel: K is split for the 64 x 128 shape only");
   const double c7 = shape_cost<S7>(f), c4 = shape_cost<S4>(f), c2 = shape_cost<S2>(f);
   if (shape == 0) {
     shape = (c7 <= c4 && c7 <= c2) ? 7 : (c4 <= c2 ? 4 : 2);

@@ -103,7 +103,10 @@ int launch_gemm(const FpArgs& a, int wbits, int regime, hipStream_t st);
 bool gemm_w4_applies(const FpArgs& f, int wbits, int regime);
 // shape: row-blocks per wave (7, 4 or 2: 448, 256 or 128 columns per workgroup), 163 / 42 = 256 x 192 /
 // 64 x 128 tiles, 0 = by cost model; 8-bit weights: 4, 2, 42 or 0
-int launch_gemm_w4(const FpArgs& f, int wbits, int regime, hipStream_t st, int shape = 0);
+// splits: workgroups that share the K steps of a tile (64 x 128 shape only; 2 or 4 need the scratch),
+// 0 = by problem size, 1 = none
+int launch_gemm_w4(const FpArgs& f, int wbits, int regime, hipStream_t st, int shape = 0, int splits = 0,
+                   const SplitKScratch* scratch = nullptr);
 
 struct Int8Args {
   const void* x;

@@ -294,13 +294,16 @@ class WoqLinearOpContext:
             # around it, 2.8 us of a call whose kernel takes 5-8 us
             p.stream = _current_raw_stream(dev_index)
             ws = counters = None
-            if M <= 32 and K >= 8192 and N <= 4096:
-                # long K, few output columns: scratch with which the decode kernel may share K between
-                # workgroups (the library decides), and the zeroed counters of this stream
-                counters = _kernels._split_k_counters(x.device)
+            wbytes = 0
+            if (M <= 32 and K >= 8192 and N <= 4096) or (M > 64 and K >= 4096 and M * N <= 1048576):
+                # long K and few output tiles: scratch with which the decode kernel or the prefill GEMM may
+                # share K between workgroups (the library decides), and the zeroed counters of this stream
+                wbytes = lib.woq_hip_linear_split_k_workspace_bytes(M, N)
+                if wbytes > 0:
+                    counters = _kernels._split_k_counters(x.device)
             if counters is not None:
-                ws = torch.empty(lib.woq_hip_linear_split_k_workspace_bytes(M, N), dtype=torch.uint8, device=x.device)
-                p.workspace, p.workspace_bytes = ws.data_ptr(), ws.numel()
+                ws = torch.empty(wbytes, dtype=torch.uint8, device=x.device)
+                p.workspace, p.workspace_bytes = ws.data_ptr(), wbytes
                 p.split_k_counters = counters.data_ptr()
             else:
                 p.workspace, p.workspace_bytes, p.split_k_counters = None, 0, None

@@ -321,6 +321,36 @@ def test_prefill_kernel_int8_weights_fp16_and_rejections(cuda):
     _check_fp(small_groups, O.LOWP_BF16, label="int8 weights, groups of 64: general kernel")
 
 
+@pytest.mark.parametrize("kind,M,K,N,G,bias", [("int4", 128, 4096, 512, 128, True), ("int4", 70, 2560, 272, 32, False),
+                                               ("int8", 200, 4096, 256, -1, True), ("int4", 65, 8192, 1040, -1, False)])
+@pytest.mark.parametrize("kernel", [0, 19, 20])  # automatic, K shared by two / four workgroups per tile
+def test_prefill_kernel_split_k(cuda, kind, M, K, N, G, bias, kernel):
+    """Few 64 x 128 tiles and a long K: the workgroups of a tile each take part of K, the last one to
+    finish adds the partial tiles in order."""
+    syn = _synthetic()
+    case = syn.make_int8_case(29, M, K, N, bias=bias) if kind == "int8" else syn.make_int4_case(29, M, K, N, G, bias=bias)
+    _check_fp(case, O.LOWP_BF16, force_kernel=kernel, label=f"prefill split K {kind} M={M} K={K} N={N} G={G} kernel={kernel}")
+    ctx = make_context(case, O.LOWP_BF16)
+    x = case["x"].cuda()
+    first = ctx.run(x, force_kernel=kernel)
+    runs = [ctx.run(x, force_kernel=kernel) for _ in range(100)]
+    torch.cuda.synchronize()
+    assert all(torch.equal(y, first) for y in runs)
+    assert rel_l2(to_np_f32(first), to_np_f32(ctx.run(x, force_kernel=12))) <= 1e-3
+    from ipex_amd import _kernels as kmod
+
+    assert all(int(buf.abs().sum()) == 0 for buf in kmod._counter_cache.values())
+
+
+def test_prefill_kernel_split_k_rejections(cuda):
+    case = _synthetic().make_int4_case(30, 128, 512, 256, 128)  # four K steps: too few to share
+    with pytest.raises(RuntimeError, match="too few"):
+        make_context(case, O.LOWP_BF16).run(case["x"].cuda(), force_kernel=20)
+    big = _synthetic().make_int4_case(31, 2048, 512, 2048, 128)  # 512 tiles: no scratch is offered
+    with pytest.raises(RuntimeError, match="split K needs"):
+        make_context(big, O.LOWP_BF16).run(big["x"].cuda(), force_kernel=19)
+
+
 def test_w4_prefill_kernel_rejects_other_shapes(cuda):
     case = _synthetic().make_int4_case(23, 70, 1000, 64, -1)  # K is not a multiple of 128
     ctx = make_context(case, O.LOWP_BF16)
