@@ -196,9 +196,10 @@ typedef struct woq_hip_linear_params {
   int32_t out_dtype;
 
   /* workspace: for lowp_mode == INT8 the quantized activations (size from
-   * woq_hip_linear_workspace_bytes); for the other modes, optional scratch for the split-K form of
-   * the dequantizing decode kernel (size from woq_hip_linear_split_k_workspace_bytes; contents
-   * undefined before and after the call) */
+   * woq_hip_linear_workspace_bytes), optionally followed by split-K scratch (round that size up to a
+   * multiple of 256 and add woq_hip_linear_split_k_workspace_bytes); for the other modes, optional
+   * split-K scratch alone (size from woq_hip_linear_split_k_workspace_bytes).  Contents undefined
+   * before and after the call */
   void* workspace;
   int64_t workspace_bytes;
 

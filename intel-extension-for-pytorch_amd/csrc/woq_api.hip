@@ -196,6 +196,7 @@ int woq_hip_linear(const woq_hip_linear_params* p) {
       a.zeros = p->zeros_u8; a.G = G; a.KG = KG; a.bias = p->bias; a.act_quant_mode = p->act_quant_mode;
       a.fusion = p->fusion; a.other0 = p->others[0]; a.other1 = p->others[1]; a.out = p->out;
       a.out_dtype = p->out_dtype; a.workspace = p->workspace; a.workspace_bytes = p->workspace_bytes;
+      a.split_k_counters = p->split_k_counters;
       a.debug_block_sums = p->debug_block_sums;
       a.nf4 = nf4 ? 1 : 0;
       a.group_size = p->group_size;

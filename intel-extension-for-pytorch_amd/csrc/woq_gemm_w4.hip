@@ -317,7 +317,9 @@ __global__ __launch_bounds__(256) void woq_gemm_w4_kernel(const FpArgs f, const 
 #pragma unroll
     for (int t = 0; t < G4_NTW; ++t) asm volatile("" : "+a"(acc[mt][t]));
 
-  if (gridDim.z > 1) {
+  // (built for the 64 x 128 shape only, the one that is ever launched with gridDim.z > 1: with more
+  // accumulator tiles the second copy of them would not fit the registers)
+  if constexpr (G4_MT * G4_NTW <= 8) if (gridDim.z > 1) {
     const int nsplit = (int)gridDim.z, z = (int)blockIdx.z;
     const int tiles = (int)(gridDim.x * gridDim.y), tile = (int)(blockIdx.y * gridDim.x + blockIdx.x);
     constexpr int kWaveFloats = G4_MT * G4_NTW * 256;
@@ -337,29 +339,41 @@ __global__ __launch_bounds__(256) void woq_gemm_w4_kernel(const FpArgs f, const 
       s_last = __hip_atomic_fetch_add(sk_counters + tile, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == nsplit - 1;
     __syncthreads();
     if (!s_last) return;
+    // the other workgroups' partial tiles, one after the other in z order: all loads of one in flight
+    // together, then the additions (this workgroup's own tile comes from its registers, in its turn)
+    f4 total[G4_MT][G4_NTW];
+#pragma unroll 1
+    for (int zz = 0; zz < nsplit; ++zz) {
+      f4 v[G4_MT][G4_NTW];
+      const float* const other = sk_partial + ((size_t)(zz * tiles + tile) * G4_WAVES + wave) * kWaveFloats + lane * 4;
+#pragma unroll
+      for (int mt = 0; mt < G4_MT; ++mt)
+#pragma unroll
+        for (int t = 0; t < G4_NTW; ++t) {
+          v[mt][t] = acc[mt][t];
+          if (zz != z) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+              v[mt][t][e] = __hip_atomic_load(other + (mt * G4_NTW + t) * 256 + e, __ATOMIC_RELAXED,
+                                              __HIP_MEMORY_SCOPE_AGENT);
+          }
+        }
+#pragma unroll
+      for (int mt = 0; mt < G4_MT; ++mt)
+#pragma unroll
+        for (int t = 0; t < G4_NTW; ++t) {
+          if (zz == 0) {
+            total[mt][t] = v[mt][t];
+          } else {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) total[mt][t][e] = total[mt][t][e] + v[mt][t][e];
+          }
+        }
+    }
 #pragma unroll
     for (int mt = 0; mt < G4_MT; ++mt)
 #pragma unroll
-      for (int t = 0; t < G4_NTW; ++t) {
-        f4 sum = f4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll 1
-        for (int zz = 0; zz < nsplit; ++zz) {
-          f4 v = acc[mt][t];
-          if (zz != z) {
-            const float* const other = sk_partial + ((size_t)(zz * tiles + tile) * G4_WAVES + wave) * kWaveFloats +
-                                       lane * 4 + (mt * G4_NTW + t) * 256;
-#pragma unroll
-            for (int e = 0; e < 4; ++e) v[e] = __hip_atomic_load(other + e, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-          }
-          if (zz == 0) {
-            sum = v;
-          } else {
-#pragma unroll
-            for (int e = 0; e < 4; ++e) sum[e] = sum[e] + v[e];
-          }
-        }
-        acc[mt][t] = sum;
-      }
+      for (int t = 0; t < G4_NTW; ++t) acc[mt][t] = total[mt][t];
     // the counter is back at zero for the next launch that uses it
     if (tid == 0) __hip_atomic_store(sk_counters + tile, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
@@ -455,6 +469,7 @@ static int launch_shape(const FpArgs& f, int g_shift, hipStream_t st, int splits
   const int ksteps = (int)(f.KT / (WBITS / 4));
   int kts = ksteps;
   if (splits > 1) {
+    if (S::MT * S::NTW > 8) return set_error("woq_gemm_w4_kernel: K is split for the 64 x 128 shape only");
     kts = ((ksteps + splits - 1) / splits + 1) & ~1;  // even, so that every workgroup starts on buffer 0
     const int64_t tiles = (int64_t)grid.x * grid.y;
     const int64_t need = (int64_t)splits * tiles * S::BM * S::BN * (int64_t)sizeof(float);

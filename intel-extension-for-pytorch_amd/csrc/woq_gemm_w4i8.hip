@@ -51,6 +51,10 @@ struct W4I8Args {
   const uint8_t* zeros;    // [NT][KG][16] or nullptr (symmetric: codes stand for code - 8)
   int g_shift;             // K tile kt belongs to group kt >> g_shift
   Epilogue ep;
+  // GEMM form with gridDim.z > 1: K steps per workgroup, fp32 partial tiles, one counter per tile
+  int kts;
+  float* sk_partial;
+  int* sk_counters;
 };
 
 typedef __attribute__((address_space(3))) void* w8_lds_ptr_t;
@@ -98,7 +102,12 @@ __global__ __launch_bounds__(256, 3) void woq_gemm_w4i8_kernel(const W4I8Args a)
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int r = lane & 15, c = lane >> 4;
-  const int M = (int)a.M, NT = (int)a.NT, KT = (int)a.KT, KG = (int)a.KG;
+  const int M = (int)a.M, NT = (int)a.NT, KTW = (int)a.KT, KG = (int)a.KG;
+  // K steps of this workgroup: [kt_lo, KT).  gridDim.z > 1 (few tiles, long K): the workgroups of a tile
+  // share K; each writes its fp32 accumulators to scratch and the one that arrives last at the tile's
+  // counter adds the partial tiles in z order and stores -- the scheme of the bf16 prefill kernel.
+  const int kt_lo = (int)blockIdx.z * a.kts;
+  const int KT = KTW < kt_lo + a.kts ? KTW : kt_lo + a.kts;
   const int m0 = blockIdx.y * W8_BM;
   const int nt0 = (blockIdx.x * W8_WAVES + wave) * W8_NTW;
 
@@ -157,7 +166,7 @@ __global__ __launch_bounds__(256, 3) void woq_gemm_w4i8_kernel(const W4I8Args a)
 #pragma unroll
   for (int t = 0; t < W8_NTW; ++t) {
     const int nt = nt0 + t < NT ? nt0 + t : NT - 1;
-    wbase[t] = a.qweight + (size_t)nt * KT * kTileBytes;
+    wbase[t] = a.qweight + (size_t)nt * KTW * kTileBytes;
     sbase[t] = a.scales + (size_t)nt * KG * kTileN;
     zbase[t] = has_z ? a.zeros + (size_t)nt * KG * kTileN : (const uint8_t*)sbase[t];
   }
@@ -195,24 +204,24 @@ __global__ __launch_bounds__(256, 3) void woq_gemm_w4i8_kernel(const W4I8Args a)
   // A K step here is short (about 2000 cycles: 32 MFMAs and the fp32 epilogue of 64 sums per lane),
   // shorter than the round trip of a request, so activations and tiles are requested two steps ahead
   // into three buffers; the scales and zero points of the next step ride in registers.
-  load_x(0, 0);
-  dma_w(0, 0);
-  load_x(KT > 1 ? 1 : 0, 1);
-  dma_w(KT > 1 ? 1 : 0, 1);
-  load_q(0, sw, zq);
+  load_x(kt_lo, 0);
+  dma_w(kt_lo, 0);
+  load_x(KT > kt_lo + 1 ? kt_lo + 1 : kt_lo, 1);
+  dma_w(KT > kt_lo + 1 ? kt_lo + 1 : kt_lo, 1);
+  load_q(kt_lo, sw, zq);
   __builtin_amdgcn_s_waitcnt(kVmcnt0);
   __syncthreads();
 #pragma unroll
   for (int t = 0; t < W8_NTW; ++t) wr[t] = *(const u4*)(wmine + t * kTileBytes + woff);
 
-  if (PER_K && tid < W8_BM) sSA[tid] = sa_mine[0];
+  if (PER_K && tid < W8_BM) sSA[tid] = sa_mine[(int64_t)(kt_lo >> a.q_shift) * a.sa_k_stride];
   __syncthreads();
 
   // Per K step: the MFMAs of row-block 0, then those of row-block 1 with the fp32 epilogue of
   // row-block 0 between them, then the epilogue of row-block 1.  What stays exposed in one wave (the
   // fragment reads, the first MFMAs, the barrier) is covered by the other two workgroups of the CU.
   int b0 = 0, b1 = 1, b2 = 2;  // buffers of steps kt, kt + 1, kt + 2
-  for (int kt = 0; kt < KT; ++kt) {
+  for (int kt = kt_lo; kt < KT; ++kt) {
     const uint8_t* xs = sX + b0 * W8_XBYTES;
     const int kt1 = kt + 1 < KT ? kt + 1 : KT - 1;
     const int kt2 = kt + 2 < KT ? kt + 2 : KT - 1;
@@ -293,6 +302,65 @@ __global__ __launch_bounds__(256, 3) void woq_gemm_w4i8_kernel(const W4I8Args a)
   }
   // the requests past the last step are still writing LDS: drain them before the workgroup can end
   __builtin_amdgcn_s_waitcnt(kVmcnt0);
+
+  if (gridDim.z > 1) {
+    const int nsplit = (int)gridDim.z, z = (int)blockIdx.z;
+    const int tiles = (int)(gridDim.x * gridDim.y), tile = (int)(blockIdx.y * gridDim.x + blockIdx.x);
+    constexpr int kWaveFloats = W8_MT * W8_NTW * 256;
+    float* const mine = a.sk_partial + ((size_t)(z * tiles + tile) * W8_WAVES + wave) * kWaveFloats + lane * 4;
+#pragma unroll
+    for (int mt = 0; mt < W8_MT; ++mt)
+#pragma unroll
+      for (int t = 0; t < W8_NTW; ++t)
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          __hip_atomic_store(mine + (mt * W8_NTW + t) * 256 + e, acc[mt][t][e], __ATOMIC_RELAXED,
+                             __HIP_MEMORY_SCOPE_AGENT);
+    __builtin_amdgcn_s_waitcnt(kVmcnt0);  // this thread's stores have completed
+    __syncthreads();
+    __shared__ int s_last;
+    if (tid == 0)
+      s_last = __hip_atomic_fetch_add(a.sk_counters + tile, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == nsplit - 1;
+    __syncthreads();
+    if (!s_last) return;
+    // the other workgroups' partial tiles, one after the other in z order: all loads of one in flight
+    // together, then the additions (this workgroup's own tile comes from its registers, in its turn)
+    f4 total[W8_MT][W8_NTW];
+#pragma unroll 1
+    for (int zz = 0; zz < nsplit; ++zz) {
+      f4 v[W8_MT][W8_NTW];
+      const float* const other = a.sk_partial + ((size_t)(zz * tiles + tile) * W8_WAVES + wave) * kWaveFloats + lane * 4;
+#pragma unroll
+      for (int mt = 0; mt < W8_MT; ++mt)
+#pragma unroll
+        for (int t = 0; t < W8_NTW; ++t) {
+          v[mt][t] = acc[mt][t];
+          if (zz != z) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+              v[mt][t][e] = __hip_atomic_load(other + (mt * W8_NTW + t) * 256 + e, __ATOMIC_RELAXED,
+                                              __HIP_MEMORY_SCOPE_AGENT);
+          }
+        }
+#pragma unroll
+      for (int mt = 0; mt < W8_MT; ++mt)
+#pragma unroll
+        for (int t = 0; t < W8_NTW; ++t) {
+          if (zz == 0) {
+            total[mt][t] = v[mt][t];
+          } else {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) total[mt][t][e] = total[mt][t][e] + v[mt][t][e];
+          }
+        }
+    }
+#pragma unroll
+    for (int mt = 0; mt < W8_MT; ++mt)
+#pragma unroll
+      for (int t = 0; t < W8_NTW; ++t) acc[mt][t] = total[mt][t];
+    // the counter is back at zero for the next launch that uses it
+    if (tid == 0) __hip_atomic_store(a.sk_counters + tile, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
 
   // ---- store: D[m][n], lane (n = r, c) holds rows m = 16 mt + 4 c + e ----
 #pragma unroll
@@ -524,7 +592,7 @@ bool gemm_w4i8_applies(const Int8Args& a, int64_t block_k, int64_t qbk, bool per
 }
 
 int launch_gemm_w4i8(const Int8Args& a, const uint8_t* xq, int64_t ldq, const float* sa, int64_t sa_m_stride,
-                     int64_t sa_k_stride, int64_t qbk, hipStream_t st) {
+                     int64_t sa_k_stride, int64_t qbk, hipStream_t st, const SplitKScratch* scratch) {
   static const hipError_t lds_optin[2] = {
       hipFuncSetAttribute(reinterpret_cast<const void*>(&woq_gemm_w4i8_kernel<false>),
                           hipFuncAttributeMaxDynamicSharedMemorySize, W8_LDS_BYTES),
@@ -545,6 +613,9 @@ int launch_gemm_w4i8(const Int8Args& a, const uint8_t* xq, int64_t ldq, const fl
     while (((int64_t)128 << k.g_shift) < a.G) ++k.g_shift;
   }
   k.ep = Epilogue{a.bias, a.fusion, a.other0, a.other1, a.out, a.out_dtype, a.x_dtype, a.N};
+  k.kts = (int)a.KT;
+  k.sk_partial = nullptr;
+  k.sk_counters = nullptr;
   if (a.M <= decode_w4i8_max_rows(a.group_size)) {
     // decode form; 2 row-blocks per workgroup while that leaves at least 256 workgroups and the
     // registers allow it, else 1
@@ -587,6 +658,22 @@ int launch_gemm_w4i8(const Int8Args& a, const uint8_t* xq, int64_t ldq, const fl
     return check_launch("woq_decode_w4i8_kernel");
   }
   dim3 grid((unsigned)((a.NT * kTileN + W8_BN - 1) / W8_BN), (unsigned)((a.M + W8_BM - 1) / W8_BM));
+  // few tiles and a long K: 4 or 2 workgroups per tile while that stays within 256 workgroups, leaves
+  // each at least 16 K steps and the caller's scratch suffices
+  const int64_t tiles = (int64_t)grid.x * grid.y;
+  if (scratch && scratch->partial && scratch->counters && tiles <= kSplitKCounters) {
+    for (int s = 4; s >= 2; s -= 2) {
+      const int64_t need = (int64_t)s * tiles * W8_BM * W8_BN * (int64_t)sizeof(float);
+      const int kts = (int)((a.KT + s - 1) / s);
+      if (tiles * s <= 256 && a.KT / s >= 16 && scratch->bytes >= need && (int64_t)(s - 1) * kts < a.KT) {
+        grid.z = (unsigned)s;
+        k.kts = kts;
+        k.sk_partial = scratch->partial;
+        k.sk_counters = scratch->counters;
+        break;
+      }
+    }
+  }
   if (sa_k_stride != 0)
     woq_gemm_w4i8_kernel<true><<<grid, 256, W8_LDS_BYTES, st>>>(k);
   else

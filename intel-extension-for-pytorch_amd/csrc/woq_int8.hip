@@ -776,8 +776,18 @@ int launch_int8_linear(const Int8Args& a, hipStream_t st) {
 
   // Large M, 4-bit weights, one activation scale per row or tensor: the kernel that feeds the
   // decoded dwords straight to the MFMA
-  if (gemm_w4i8_applies(a, p.block_k, qbk_quant, per_k, asym))
-    return launch_gemm_w4i8(a, xq, p.ldq, sa, p.sa_m_stride, p.sa_k_stride, qbk_quant, st);
+  if (gemm_w4i8_applies(a, p.block_k, qbk_quant, per_k, asym)) {
+    // what the caller gave beyond the quantized activations and their parameters serves as scratch for
+    // sharing K between workgroups (with the caller's counters)
+    SplitKScratch scratch;
+    const int64_t used = (need + 255) / 256 * 256;
+    if (a.split_k_counters && a.workspace_bytes > used) {
+      scratch.partial = (float*)((uint8_t*)a.workspace + used);
+      scratch.bytes = a.workspace_bytes - used;
+      scratch.counters = a.split_k_counters;
+    }
+    return launch_gemm_w4i8(a, xq, p.ldq, sa, p.sa_m_stride, p.sa_k_stride, qbk_quant, st, &scratch);
+  }
 
   // The small-M kernel accumulates whole tiles per MFMA, so it needs K blocks that are whole
   // tiles; finer blocks (group_size 32 / 64 with 4-bit weights) go through the tiled kernel,

@@ -128,6 +128,7 @@ struct Int8Args {
   int out_dtype;
   void* workspace;
   int64_t workspace_bytes;
+  int32_t* split_k_counters;  // optional; with workspace bytes beyond the quantized activations: split K
   int32_t* debug_block_sums;
   int nf4;  // 4-bit codes index the NF4 int8 table; the weight scale is multiplied by fp32(1 / 127)
 };
@@ -136,7 +137,7 @@ struct Int8Args {
 // blocks of 128; sa[m * sa_m_stride + (k / qbk) * sa_k_stride] is the scale of row m at k.
 bool gemm_w4i8_applies(const Int8Args& a, int64_t block_k, int64_t qbk, bool per_k, bool asym);
 int launch_gemm_w4i8(const Int8Args& a, const uint8_t* xq, int64_t ldq, const float* sa, int64_t sa_m_stride,
-                     int64_t sa_k_stride, int64_t qbk, hipStream_t st);
+                     int64_t sa_k_stride, int64_t qbk, hipStream_t st, const SplitKScratch* scratch = nullptr);
 // One-pass quantization of whole rows (woq_act_quant.hip): 16-bit activations, one scale per row or per
 // (row, K block), padded rows of at most 16384 elements.  Same bytes and scales as the two-kernel form.
 bool act_quant_rows_applies(const void* x, int x_dtype, int64_t K, const void* q, int64_t ldq, int64_t qbk,

@@ -228,6 +228,14 @@ def linear(
     ws = None
     wbytes = lib.woq_hip_linear_workspace_bytes(M, K, lowp_mode, act_quant_mode, group_size)
     counters = None
+    if wbytes > 0 and lowp_mode == 3 and M > 64:
+        # lowp INT8 at prefill sizes: room behind the quantized activations lets the int8 GEMM share a
+        # long K between the workgroups of its few tiles
+        extra = lib.woq_hip_linear_split_k_workspace_bytes(M, N)
+        counters = _split_k_counters(x.device) if extra > 0 else None
+        if counters is not None:
+            p.split_k_counters = counters.data_ptr()
+            wbytes = (wbytes + 255) // 256 * 256 + extra
     if wbytes == 0 and lowp_mode != 3:
         # scratch that lets the decode kernel split K across workgroups (small M, few output columns)
         wbytes = lib.woq_hip_linear_split_k_workspace_bytes(M, N)

@@ -849,6 +849,24 @@ def test_int8_lowp_decode_kernel(cuda, mode, M, K, N, G):
     _check_int8(case, mode, cols=cols, debug=N < 4096, label=f"int8 lowp decode mode={mode} M={M} K={K} N={N} G={G}")
 
 
+@pytest.mark.parametrize("mode", [6, 7])
+@pytest.mark.parametrize("M,K,N,G", [(100, 4096, 256, 128), (200, 8192, 144, 256), (65, 14336, 512, -1)])
+def test_int8_lowp_prefill_split_k(cuda, mode, M, K, N, G):
+    """Few 64 x 128 tiles and a long K under lowp INT8: the workgroups of a tile share K (scratch behind
+    the quantized activations); repeated launches must agree bit for bit."""
+    case = _synthetic().make_int4_case(32, M, K, N, G, bias=True, outliers=True)
+    _check_int8(case, mode, debug=False, label=f"int8 lowp split K mode={mode} M={M} K={K} N={N} G={G}")
+    ctx = make_context(case, O.LOWP_INT8, mode)
+    x = case["x"].cuda()
+    first = ctx.run(x)
+    runs = [ctx.run(x) for _ in range(100)]
+    torch.cuda.synchronize()
+    assert all(torch.equal(y, first) for y in runs)
+    from ipex_amd import _kernels as kmod
+
+    assert all(int(buf.abs().sum()) == 0 for buf in kmod._counter_cache.values())
+
+
 def test_int8_lowp_int8_weights(cuda):
     for M in (2, 20, 140):
         case = _synthetic().make_int8_case(22, M, 512, 80)
