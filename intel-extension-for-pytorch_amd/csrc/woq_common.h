@@ -298,19 +298,27 @@ static __constant__ const float kNf4Values[16] = {
     0.07958029955625534f, 0.16093020141124725f, 0.24611230194568634f, 0.33791524171829224f,
     0.44070982933044434f, 0.5626170039176941f, 0.7229568362236023f, 1.0f};
 
-// One packed dword (8 codes of one row) -> 8 compute-dtype weights in K order.  `lut` is a copy
-// of the table in LDS: the 64 lanes read at most 16 distinct words, one per bank.
+// One packed dword (8 codes of one row) -> 8 compute-dtype weights in K order.  `lut` is the pair
+// table in LDS (nf4_fill_lut): entry b holds the table values of the two codes in byte b, so a dword
+// takes four 8-byte reads instead of eight 4-byte ones and half the address arithmetic.  Byte b of the
+// dword carries the codes of nibble positions 2 b and 2 b + 1; output dword v pairs the positions v and
+// v + 4 (K elements 2 v and 2 v + 1).
+constexpr int kNf4LutEntries = 256;
+__device__ __forceinline__ void nf4_fill_lut(f2* lut, int tid, int nthreads) {
+  for (int i = tid; i < kNf4LutEntries; i += nthreads) lut[i] = f2{kNf4Values[i & 15], kNf4Values[i >> 4]};
+}
 template <int REGIME>
-__device__ __forceinline__ u4 nf4_dequant(uint32_t d, const float* lut, float s) {
+__device__ __forceinline__ u4 nf4_dequant(uint32_t d, const f2* lut, float s) {
+  const f2 p0 = lut[d & 0xFFu], p1 = lut[(d >> 8) & 0xFFu], p2 = lut[(d >> 16) & 0xFFu], p3 = lut[d >> 24];
+  const float lo[4] = {__fmul_rn(p0[0], s), __fmul_rn(p0[1], s), __fmul_rn(p1[0], s), __fmul_rn(p1[1], s)};
+  const float hi[4] = {__fmul_rn(p2[0], s), __fmul_rn(p2[1], s), __fmul_rn(p3[0], s), __fmul_rn(p3[1], s)};
   u4 r;
 #pragma unroll
   for (int v = 0; v < 4; ++v) {
-    const float lo = __fmul_rn(lut[(d >> (4 * v)) & 15u], s);
-    const float hi = __fmul_rn(lut[(d >> (16 + 4 * v)) & 15u], s);
     if constexpr (REGIME == kRegimeF16)
-      r[v] = (uint32_t)f32_to_f16_bits(lo) | ((uint32_t)f32_to_f16_bits(hi) << 16);
+      r[v] = (uint32_t)f32_to_f16_bits(lo[v]) | ((uint32_t)f32_to_f16_bits(hi[v]) << 16);
     else
-      r[v] = g4_cvt_pair(f2{lo, hi});
+      r[v] = g4_cvt_pair(f2{lo[v], hi[v]});
   }
   return r;
 }

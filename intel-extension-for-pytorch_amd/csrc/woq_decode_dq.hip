@@ -90,9 +90,9 @@ __global__ __launch_bounds__(512, 4) void woq_decode_dq_kernel(const DecodeDqArg
   constexpr int TK = Geo::TK, NJ = Geo::NJ, NX = Geo::NX, SLICE = Geo::SLICE;
   static_assert(!NF4 || WBITS == 4, "NF4 codes are 4 bits wide");
   extern __shared__ __align__(1024) uint8_t smem[];
-  __shared__ float sNf4[16];
+  __shared__ f2 sNf4[NF4 ? kNf4LutEntries : 1];
   if constexpr (NF4) {
-    if (threadIdx.x < 16) sNf4[threadIdx.x] = kNf4Values[threadIdx.x];
+    nf4_fill_lut(sNf4, (int)threadIdx.x, (int)blockDim.x);
     __syncthreads();
   }
   const FpArgs& f = a.f;

@@ -56,10 +56,10 @@ __global__ __launch_bounds__(256) void woq_gemm_kernel(const FpArgs f) {
   const int64_t nt0 = n0 / kTileN;
   const int64_t Kpad = f.KT * TK;
 
-  __shared__ float sNf4[16];
+  __shared__ f2 sNf4[NF4 ? kNf4LutEntries : 1];
   constexpr bool nf4 = NF4;  // a template parameter: a runtime flag in the decode loop is not free
   if (nf4) {
-    if (tid < 16) sNf4[tid] = kNf4Values[tid];
+    nf4_fill_lut(sNf4, (int)tid, (int)blockDim.x);
     __syncthreads();
   }
 

@@ -120,10 +120,10 @@ __global__ __launch_bounds__(1024) void woq_small_m_kernel(const SmallMArgs a) {
   uint16_t* sx = (uint16_t*)(smem + (size_t)NTW * MT * W * 64 * sizeof(f4));  // [rows][KC]
   const int rows = (int)(f.M < MT * 16 ? f.M : MT * 16);
 
-  __shared__ float sNf4[16];
+  __shared__ f2 sNf4[NF4 ? kNf4LutEntries : 1];
   constexpr bool nf4 = NF4;  // a template parameter: a runtime flag in the decode loop is not free
   if (nf4) {
-    if (threadIdx.x < 16) sNf4[threadIdx.x] = kNf4Values[threadIdx.x];
+    nf4_fill_lut(sNf4, (int)threadIdx.x, (int)blockDim.x);
     __syncthreads();
   }
 
