@@ -234,7 +234,7 @@ int woq_hip_linear(const woq_hip_linear_params* p) {
   if (nf4) {
     // table lookups instead of the integer decode: the dequantizing decode kernel and the two
     // general kernels carry them
-    if (kernel == 0) kernel = (p->M <= 32 && decode_dq_applies(f, wbits, regime)) ? 7 : (p->M <= 64 ? 1 : 2);
+    if (kernel == 0) kernel = decode_dq_applies(f, wbits, regime) ? 7 : (p->M <= 64 ? 1 : 2);
     if (kernel != 1 && kernel != 2 && (kernel < 7 || kernel > 9) && kernel != 13 && kernel != 14 && kernel != 16)
       return set_error("woq_linear: NF4 weights run on kernels 1, 2, 7..9, 13, 14 and 16 only");
   }

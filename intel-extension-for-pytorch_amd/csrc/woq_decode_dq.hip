@@ -382,6 +382,8 @@ static int launch_dq_nf4(const DecodeDqArgs& a, int ntw, int splits, hipStream_t
       return ntw == 2 ? launch_dq_cfg<REGIME, 4, 1, 2, true, true>(a, splits, st)
                       : launch_dq_cfg<REGIME, 4, 1, 1, true, true>(a, splits, st);
   }
+  if (a.f.M > 32)  // four row tiles
+    return ntw == 2 ? launch_dq_cfg<REGIME, 4, 4, 2, true>(a, splits, st) : launch_dq_cfg<REGIME, 4, 4, 1, true>(a, splits, st);
   const bool two_rows = a.f.M > 16;
   if (ntw == 2) return two_rows ? launch_dq_cfg<REGIME, 4, 2, 2, true>(a, splits, st) : launch_dq_cfg<REGIME, 4, 1, 2, true>(a, splits, st);
   return two_rows ? launch_dq_cfg<REGIME, 4, 2, 1, true>(a, splits, st) : launch_dq_cfg<REGIME, 4, 1, 1, true>(a, splits, st);
@@ -449,7 +451,7 @@ int launch_decode_dq(const FpArgs& f, int wbits, int regime, hipStream_t st, int
   }
   if (f.nf4) {
     if (wbits != 4 || f.zeros) return set_error("woq_decode_dq_kernel: NF4 weights are 4-bit and symmetric");
-    if (f.M > 32) return set_error("woq_decode_dq_kernel: NF4 weights take at most 32 rows");
+
     if (ntw == 4) return set_error("woq_decode_dq_kernel: NF4 weights take 1 or 2 row-blocks per workgroup");
     return regime == kRegimeF16 ? launch_dq_nf4<kRegimeF16>(a, ntw, splits, st)
                                 : launch_dq_nf4<kRegimeBF16>(a, ntw, splits, st);

@@ -410,9 +410,11 @@ def test_dequantizing_decode_kernel_four_row_tiles_int8_weights_and_rejections(c
     with pytest.raises(RuntimeError, match="row-blocks"):
         ctx.run(case["x"].cuda(), force_kernel=10)
     nf4 = _synthetic().make_nf4_case(37, 40, 512, 64, 128)
+    for kernel in (0, 7, 8, 9, 1):  # four row tiles of NF4 codes, then the small-M kernel
+        _check_fp(nf4, O.LOWP_BF16, force_kernel=kernel, label=f"nf4 M=40 kernel={kernel}")
     with pytest.raises(RuntimeError, match="NF4"):
-        make_context(nf4, O.LOWP_BF16).run(nf4["x"].cuda(), force_kernel=7)
-    _check_fp(nf4, O.LOWP_BF16, label="nf4 M=40 takes the small-M kernel")
+        make_context(nf4, O.LOWP_BF16).run(nf4["x"].cuda(), force_kernel=10)
+    _check_fp(_synthetic().make_nf4_case(38, 64, 1024, 272, 64, bias=True), O.LOWP_BF16, label="nf4 M=64")
 
 
 @pytest.mark.parametrize(
