@@ -90,6 +90,27 @@ __device__ __forceinline__ float w8_accumulate(int sum, float s_a, float s_w, fl
     return __builtin_fmaf((float)sum, s_w, acc);
 }
 
+// NF4 codes under lowp_mode INT8: the code's table value times 127, rounded, as int8
+// (load_nf4_as_int8, csrc/cpu/aten/utils/woq.h:628-669): two byte permutes over the halves of the
+// table (codes 0..7 and 8..15), merged on bit 3 of each code; the weight scale carries the 1 / 127.
+__device__ __forceinline__ uint32_t w8_nf4_codes_to_i8(uint32_t b) {
+  // -127 -88 -67 -50 | -36 -23 -12 0 | 10 20 31 43 | 56 71 92 127, least significant byte first
+  const uint32_t t0 = 0xCEBDA881u, t1 = 0x00F4E9DCu, t2 = 0x2B1F140Au, t3 = 0x7F5C4738u;
+  const uint32_t sel = b & 0x07070707u;
+  const uint32_t lo = __builtin_amdgcn_perm(t1, t0, sel);
+  const uint32_t hi = __builtin_amdgcn_perm(t3, t2, sel);
+  const uint32_t m = ((b >> 3) & 0x01010101u) * 0xFFu;
+  return (hi & m) | (lo & ~m);
+}
+__device__ __forceinline__ i4 w8_decode16_nf4(uint32_t d0, uint32_t d1) {
+  i4 r;
+  r[0] = (int)w8_nf4_codes_to_i8(d0 & 0x0F0F0F0Fu);
+  r[1] = (int)w8_nf4_codes_to_i8((d0 >> 4) & 0x0F0F0F0Fu);
+  r[2] = (int)w8_nf4_codes_to_i8(d1 & 0x0F0F0F0Fu);
+  r[3] = (int)w8_nf4_codes_to_i8((d1 >> 4) & 0x0F0F0F0Fu);
+  return r;
+}
+
 // PER_K: the activation scales change with the K block; they reach the lanes through LDS.
 template <bool PER_K>
 __global__ __launch_bounds__(256, 3) void woq_gemm_w4i8_kernel(const W4I8Args a) {
@@ -397,7 +418,8 @@ struct DecodeW4I8Args {
 
 // MT: 16-row tiles (one, two or four).  The forms with many K blocks and row tiles keep GSUB x MT sets of
 // activation scales in flight and get the registers of two waves per SIMD instead of four.
-template <bool PER_K, int MT, int NTW, int GSUB>
+// NF4: the codes index the int8 NormalFloat4 table (no zero points; scale / 127).
+template <bool PER_K, int MT, int NTW, int GSUB, bool NF4>
 __global__ __launch_bounds__(512, (GSUB * MT > 4 ? 2 : 4)) void woq_decode_w4i8_kernel(const DecodeW4I8Args a) {
   constexpr int SLICE = MT * 16 * kTileK4;  // one buffer of one wave: 16 MT rows x 128 bytes
   constexpr int NX = 2 * MT;                // activation loads per tile (eight rows each)
@@ -495,7 +517,7 @@ __global__ __launch_bounds__(512, (GSUB * MT > 4 ? 2 : 4)) void woq_decode_w4i8_
     for (int t = 0; t < NTW; ++t) {
       wreg[t] = wnext[t];
 #pragma unroll
-      for (int g = 0; g < GSUB; ++g) sw[t][g] = snext[t][g];
+      for (int g = 0; g < GSUB; ++g) sw[t][g] = NF4 ? snext[t][g] * (1.0f / 127.0f) : snext[t][g];
       z4[t] = (has_z ? (uint32_t)znext[t] : 8u) * 0x01010101u;
     }
     if constexpr (PER_K) {
@@ -516,8 +538,8 @@ __global__ __launch_bounds__(512, (GSUB * MT > 4 ? 2 : 4)) void woq_decode_w4i8_
       for (int j = 0; j < 2; ++j) xa[mt][j] = *(const i4*)(sx + buf * SLICE + mt * 2048 + rd[j]);
 #pragma unroll
     for (int t = 0; t < NTW; ++t) {
-      const i4 bq0 = w8_decode16(wreg[t][0], wreg[t][1], z4[t]);
-      const i4 bq1 = w8_decode16(wreg[t][2], wreg[t][3], z4[t]);
+      const i4 bq0 = NF4 ? w8_decode16_nf4(wreg[t][0], wreg[t][1]) : w8_decode16(wreg[t][0], wreg[t][1], z4[t]);
+      const i4 bq1 = NF4 ? w8_decode16_nf4(wreg[t][2], wreg[t][3]) : w8_decode16(wreg[t][2], wreg[t][3], z4[t]);
 #pragma unroll
       for (int g = 0; g < GSUB; ++g) {
         // activation fragments of K block g: the lane columns of the other blocks contribute zeros
@@ -577,8 +599,10 @@ static int decode_w4i8_max_rows(int64_t group_size) { return group_size == 64 ? 
 // 64-row tiles of the MFMA GEMM, which with a single row tile still beats the general small-M kernel
 // (4096 -> 14336, per-row scales, M = 48 / 64: 34 / 36 us against 157 / 162 us).
 bool gemm_w4i8_applies(const Int8Args& a, int64_t block_k, int64_t qbk, bool per_k, bool asym) {
-  if (a.wbits != 4 || a.nf4 || asym || a.debug_block_sums) return false;
+  if (a.wbits != 4 || asym || a.debug_block_sums) return false;
   if (a.K % 128 != 0) return false;
+  // NF4 codes: the decode form only (up to two row tiles)
+  if (a.nf4 && (a.M > 32 || a.zeros)) return false;
   if (block_k == 32 || block_k == 64) {
     // groups of 32 / 64: the decode form only (K blocks inside a tile), activation blocks = groups
     return a.M <= decode_w4i8_max_rows(a.group_size) && a.group_size == block_k && (!per_k || qbk == block_k) &&
@@ -633,13 +657,35 @@ int launch_gemm_w4i8(const Int8Args& a, const uint8_t* xq, int64_t ldq, const fl
     if (red > smem) smem = red;
     const unsigned dgrid = (unsigned)(a.NT / ntw);
     const bool per_k = sa_k_stride != 0;
-#define WOQ_DECODE_W4I8(MTV, NTWV, GS)                                                  \
-  do {                                                                                  \
-    if (per_k)                                                                          \
-      woq_decode_w4i8_kernel<true, MTV, NTWV, GS><<<dgrid, d.W * 64, smem, st>>>(d);    \
-    else                                                                                \
-      woq_decode_w4i8_kernel<false, MTV, NTWV, GS><<<dgrid, d.W * 64, smem, st>>>(d);   \
+#define WOQ_DECODE_W4I8(MTV, NTWV, GS)                                                         \
+  do {                                                                                         \
+    if (per_k)                                                                                 \
+      woq_decode_w4i8_kernel<true, MTV, NTWV, GS, false><<<dgrid, d.W * 64, smem, st>>>(d);    \
+    else                                                                                       \
+      woq_decode_w4i8_kernel<false, MTV, NTWV, GS, false><<<dgrid, d.W * 64, smem, st>>>(d);   \
   } while (0)
+#define WOQ_DECODE_W4I8_NF4(MTV, NTWV, GS)                                                     \
+  do {                                                                                         \
+    if (per_k)                                                                                 \
+      woq_decode_w4i8_kernel<true, MTV, NTWV, GS, true><<<dgrid, d.W * 64, smem, st>>>(d);     \
+    else                                                                                       \
+      woq_decode_w4i8_kernel<false, MTV, NTWV, GS, true><<<dgrid, d.W * 64, smem, st>>>(d);    \
+  } while (0)
+    if (a.nf4) {  // at most two row tiles (gemm_w4i8_applies)
+      if (mt == 2) {
+        if (gsub == 4) WOQ_DECODE_W4I8_NF4(2, 1, 4);
+        else if (gsub == 2) WOQ_DECODE_W4I8_NF4(2, 1, 2);
+        else if (ntw == 2) WOQ_DECODE_W4I8_NF4(2, 2, 1);
+        else WOQ_DECODE_W4I8_NF4(2, 1, 1);
+      } else {
+        if (gsub == 4) WOQ_DECODE_W4I8_NF4(1, 1, 4);
+        else if (gsub == 2 && ntw == 2) WOQ_DECODE_W4I8_NF4(1, 2, 2);
+        else if (gsub == 2) WOQ_DECODE_W4I8_NF4(1, 1, 2);
+        else if (ntw == 2) WOQ_DECODE_W4I8_NF4(1, 2, 1);
+        else WOQ_DECODE_W4I8_NF4(1, 1, 1);
+      }
+      return check_launch("woq_decode_w4i8_kernel");
+    }
     if (gsub == 4) {
       if (mt == 2) WOQ_DECODE_W4I8(2, 1, 4);
       else WOQ_DECODE_W4I8(1, 1, 4);
@@ -655,6 +701,7 @@ int launch_gemm_w4i8(const Int8Args& a, const uint8_t* xq, int64_t ldq, const fl
       else WOQ_DECODE_W4I8(1, 1, 1);
     }
 #undef WOQ_DECODE_W4I8
+#undef WOQ_DECODE_W4I8_NF4
     return check_launch("woq_decode_w4i8_kernel");
   }
   dim3 grid((unsigned)((a.NT * kTileN + W8_BN - 1) / W8_BN), (unsigned)((a.M + W8_BM - 1) / W8_BM));

@@ -693,7 +693,8 @@ def test_nf4_rejections(cuda):
 
 
 @pytest.mark.parametrize("mode", [6, 7, 2])
-@pytest.mark.parametrize("M,K,N,G", [(1, 1024, 272, 128), (40, 512, 144, 32), (150, 1024, 272, 128), (20, 768, 80, -1)])
+@pytest.mark.parametrize("M,K,N,G", [(1, 1024, 272, 128), (40, 512, 144, 32), (150, 1024, 272, 128), (20, 768, 80, -1),
+                                     (16, 1024, 8208, 64), (9, 512, 144, 32), (4, 1152, 96, -1), (30, 1024, 272, 32), (32, 512, 1040, 128)])
 def test_nf4_lowp_int8(cuda, mode, M, K, N, G):
     """NF4 codes as int8 table values, scale / 127: int32 block sums bit-exact, fp32 epilogue to the bar."""
     case = _synthetic().make_nf4_case(28, M, K, N, G, bias=(M == 40))
