@@ -246,9 +246,9 @@ class WoqLinearOpContext:
 
     # ---- execution ----
     def _run_planned(self, x, M, fusion, others):
-        """The common call (floating-point regimes, no debugging options) through a parameter
-        block that is filled once per context and thread: per call only the activation / output
-        pointers, M, the post-op and the stream change."""
+        """The common call (no debugging options) through a parameter block that is filled once per
+        context and thread: per call only the activation / output pointers, M, the post-op, the
+        workspace and the stream change."""
         N, K = self.weight_shape_
         tl = self.__dict__.setdefault("_tls", threading.local())
         p = getattr(tl, "plan", None)
@@ -295,18 +295,23 @@ class WoqLinearOpContext:
             p.stream = _current_raw_stream(dev_index)
             ws = counters = None
             wbytes = 0
-            if (M <= 32 and K >= 8192 and N <= 4096) or (M > 64 and K >= 4096 and M * N <= 1048576):
-                # long K and few output tiles: scratch with which the decode kernel or the prefill GEMM may
+            int8 = self.lowp_mode_ == _lib.LOWP_INT8
+            if int8:  # the quantized activations and their scales
+                wbytes = lib.woq_hip_linear_workspace_bytes(M, K, _lib.LOWP_INT8, self.act_quant_mode_, self.group_size_)
+            if ((M <= 32 and K >= 8192 and N <= 4096) and not int8) or (M > 64 and K >= 4096 and M * N <= 1048576):
+                # long K and few output tiles: scratch with which the decode kernel or the prefill GEMMs may
                 # share K between workgroups (the library decides), and the zeroed counters of this stream
-                wbytes = lib.woq_hip_linear_split_k_workspace_bytes(M, N)
-                if wbytes > 0:
+                extra = lib.woq_hip_linear_split_k_workspace_bytes(M, N)
+                if extra > 0:
                     counters = _kernels._split_k_counters(x.device)
-            if counters is not None:
+                if counters is not None:
+                    wbytes = (wbytes + 255) // 256 * 256 + extra
+            if wbytes > 0:
                 ws = torch.empty(wbytes, dtype=torch.uint8, device=x.device)
                 p.workspace, p.workspace_bytes = ws.data_ptr(), wbytes
-                p.split_k_counters = counters.data_ptr()
             else:
-                p.workspace, p.workspace_bytes, p.split_k_counters = None, 0, None
+                p.workspace, p.workspace_bytes = None, 0
+            p.split_k_counters = counters.data_ptr() if counters is not None else None
             rc = lib.woq_hip_linear(ctypes.byref(p))
         _lib.check(rc, "woq_linear")
         return out
@@ -356,7 +361,7 @@ class WoqLinearOpContext:
             # casts around the call reaches the kernels that want rows in the compute dtype
             # (M = 2048, 4096 -> 14336: 430 us through the converting general kernel otherwise)
             return self.run(x.to(torch.float16)).to(torch.bfloat16)
-        if not kw and self.lowp_mode_ != _lib.LOWP_INT8 and x.dtype in _kernels._ACT_CODE and x.is_cuda:
+        if not kw and x.dtype in _kernels._ACT_CODE and x.is_cuda:
             return self._run_planned(x, M, fusion, others)
         return _kernels.linear(
             x,
