@@ -250,7 +250,9 @@ class WoqLinearOpContext:
         context and thread: per call only the activation / output pointers, M, the post-op, the
         workspace and the stream change."""
         N, K = self.weight_shape_
-        tl = self.__dict__.setdefault("_tls", threading.local())
+        tl = self.__dict__.get("_tls")
+        if tl is None:
+            tl = self.__dict__.setdefault("_tls", threading.local())
         p = getattr(tl, "plan", None)
         if p is None:
             p = _lib.LinearParams()
@@ -267,7 +269,10 @@ class WoqLinearOpContext:
             p.bias = self.bias_f32_.data_ptr() if self.bias_f32_ is not None else None
             p.lowp_mode = self.lowp_mode_
             p.act_quant_mode = self.act_quant_mode_
+            p.others[0] = p.others[1] = None
             tl.plan = p
+            tl.plan_ref = ctypes.byref(p)
+            tl.had_others = tl.had_scratch = False
         x2 = x if x.is_contiguous() else x.contiguous()
         if x2.data_ptr() % 16:
             x2 = x2.clone()  # the kernels read activation rows with 16-byte loads
@@ -277,17 +282,19 @@ class WoqLinearOpContext:
         p.out, p.out_dtype = out.data_ptr(), code
         p.fusion = fusion
         keep = []
-        for i in range(2):
-            if i < len(others):
-                o = others[i]
-                if o.numel() != M * N:
-                    raise RuntimeError("woq_linear: post-op operand must have the output's shape")
-                o = o.to(x.dtype).contiguous()
-                keep.append(o)
-                p.others[i] = o.data_ptr()
-            else:
-                p.others[i] = None
-        lib = _lib.load()
+        if others or tl.had_others:
+            for i in range(2):
+                if i < len(others):
+                    o = others[i]
+                    if o.numel() != M * N:
+                        raise RuntimeError("woq_linear: post-op operand must have the output's shape")
+                    o = o.to(x.dtype).contiguous()
+                    keep.append(o)
+                    p.others[i] = o.data_ptr()
+                else:
+                    p.others[i] = None
+            tl.had_others = bool(others)
+        lib = _lib._lib or _lib.load()
         dev_index = x.device.index
         with _NO_GUARD if dev_index == _current_device() else torch.cuda.device(x.device):
             # the raw handle of the current stream: torch.cuda.current_stream() builds a Stream object
@@ -309,11 +316,14 @@ class WoqLinearOpContext:
             if wbytes > 0:
                 ws = torch.empty(wbytes, dtype=torch.uint8, device=x.device)
                 p.workspace, p.workspace_bytes = ws.data_ptr(), wbytes
-            else:
-                p.workspace, p.workspace_bytes = None, 0
-            p.split_k_counters = counters.data_ptr() if counters is not None else None
-            rc = lib.woq_hip_linear(ctypes.byref(p))
-        _lib.check(rc, "woq_linear")
+                p.split_k_counters = counters.data_ptr() if counters is not None else None
+                tl.had_scratch = True
+            elif tl.had_scratch:
+                p.workspace, p.workspace_bytes, p.split_k_counters = None, 0, None
+                tl.had_scratch = False
+            rc = lib.woq_hip_linear(tl.plan_ref)
+        if rc:
+            _lib.check(rc, "woq_linear")
         return out
 
     def _cached_bf16_weight(self):
