@@ -397,9 +397,8 @@ class WoqLinearOpContext:
 def _context_from_handle(handle):
     if handle.dtype != torch.int64 or handle.numel() != 1:
         raise RuntimeError("ipex_woq_linear: W_prepack must be the 1-element int64 tensor of get_data_handle()")
-    key = int(handle.reshape(-1)[0])
-    with _contexts_lock:
-        ref = _contexts.get(key)
+    key = handle.item()
+    ref = _contexts.get(key)  # a single dict read: atomic under the interpreter lock
     ctx = ref() if ref is not None else None
     if ctx is None:
         raise RuntimeError("ipex_woq_linear: the prepack context behind this handle no longer exists")
