@@ -419,8 +419,13 @@ struct DecodeW4I8Args {
 // MT: 16-row tiles (one, two or four).  The forms with many K blocks and row tiles keep GSUB x MT sets of
 // activation scales in flight and get the registers of two waves per SIMD instead of four.
 // NF4: the codes index the int8 NormalFloat4 table (no zero points; scale / 127).
-template <bool PER_K, int MT, int NTW, int GSUB, bool NF4>
+// WBITS 8: symmetric 8-bit weights, stored offset-binary; a packed tile is 16 rows x 64 K values, so a
+// round takes two tiles per row-block (one MFMA each) and the lane's 16 bytes are the B operand as they
+// are, sign bit flipped; the A fragment of tile u is chunk 4 u + c of the 128-byte row.
+template <bool PER_K, int MT, int NTW, int GSUB, bool NF4, int WBITS = 4>
 __global__ __launch_bounds__(512, (GSUB * MT > 4 ? 2 : 4)) void woq_decode_w4i8_kernel(const DecodeW4I8Args a) {
+  static_assert(WBITS == 4 || (WBITS == 8 && GSUB == 1 && !NF4), "8-bit weights: one K block per round");
+  constexpr int TPR = WBITS / 4;  // packed tiles per row-block and round of 128 K values
   constexpr int SLICE = MT * 16 * kTileK4;  // one buffer of one wave: 16 MT rows x 128 bytes
   constexpr int NX = 2 * MT;                // activation loads per tile (eight rows each)
   extern __shared__ __align__(1024) uint8_t smem[];
@@ -429,7 +434,8 @@ __global__ __launch_bounds__(512, (GSUB * MT > 4 ? 2 : 4)) void woq_decode_w4i8_
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
   const int r = lane & 15, c = lane >> 4;
-  const int M = (int)k.M, KT = (int)k.KT, KG = (int)k.KG;
+  const int M = (int)k.M, KTW = (int)k.KT, KG = (int)k.KG;
+  const int KT = KTW / TPR;  // rounds of 128 K values
   const int64_t nt0 = (int64_t)blockIdx.x * NTW;
   uint8_t* const sx = smem + wave * (2 * SLICE);
   f4* const red = (f4*)smem;  // [NTW * MT][W][64], after the K loop
@@ -450,9 +456,10 @@ __global__ __launch_bounds__(512, (GSUB * MT > 4 ? 2 : 4)) void woq_decode_w4i8_
     const int chunk = (lane & 7) ^ ((row >> 1) & 7);
     xoff[i] = (uint32_t)(rowc * (int)k.ldq + chunk * 16);
   }
-  uint32_t rd[2];  // A fragment of MFMA j in row tile 0: row r, logical chunk 2 c + j
+  uint32_t rd[2];  // A fragment of MFMA j in row tile 0: row r, logical chunk 2 c + j (8-bit weights: 4 j + c)
 #pragma unroll
-  for (int j = 0; j < 2; ++j) rd[j] = (uint32_t)(r * 128 + (((2 * c + j) ^ ((r >> 1) & 7)) << 4));
+  for (int j = 0; j < 2; ++j)
+    rd[j] = (uint32_t)(r * 128 + ((((WBITS == 4 ? 2 * c + j : 4 * j + c)) ^ ((r >> 1) & 7)) << 4));
 
   const bool has_z = k.zeros != nullptr;
   const uint8_t* wbase[NTW];
@@ -460,7 +467,7 @@ __global__ __launch_bounds__(512, (GSUB * MT > 4 ? 2 : 4)) void woq_decode_w4i8_
   const uint8_t* zbase[NTW];
 #pragma unroll
   for (int t = 0; t < NTW; ++t) {
-    wbase[t] = k.qweight + (size_t)(nt0 + t) * KT * kTileBytes;
+    wbase[t] = k.qweight + (size_t)(nt0 + t) * KTW * kTileBytes;
     sbase[t] = k.scales + (size_t)(nt0 + t) * KG * kTileN;
     zbase[t] = has_z ? k.zeros + (size_t)(nt0 + t) * KG * kTileN : (const uint8_t*)sbase[t];
   }
@@ -468,7 +475,7 @@ __global__ __launch_bounds__(512, (GSUB * MT > 4 ? 2 : 4)) void woq_decode_w4i8_
 
   // activation scales of this lane's accumulator rows m = 16 mt + 4 c + e: one per row for the whole
   // K (applied after the sum over the waves), or (PER_K) one per row and K block, requested with the tile
-  u4 wnext[NTW];
+  u4 wnext[NTW][TPR];
   float snext[NTW][GSUB];
   uint8_t znext[NTW];
   f4 sanext[PER_K ? GSUB : 1][PER_K ? MT : 1];
@@ -483,10 +490,12 @@ __global__ __launch_bounds__(512, (GSUB * MT > 4 ? 2 : 4)) void woq_decode_w4i8_
     // first group of the tile (GSUB == 1: the tile's only one, shared by 2^g_shift tiles)
     int g0 = GSUB == 1 ? (kt >> k.g_shift) : kt * GSUB;
     g0 = g0 < KG ? g0 : KG - 1;
-    const uint32_t wo = (uint32_t)kt * kTileBytes + woff;
+    const uint32_t wo = (uint32_t)kt * (TPR * kTileBytes) + woff;
 #pragma unroll
     for (int t = 0; t < NTW; ++t) {
-      wnext[t] = __builtin_nontemporal_load((const u4*)(wbase[t] + wo));
+#pragma unroll
+      for (int u = 0; u < TPR; ++u)
+        wnext[t][u] = __builtin_nontemporal_load((const u4*)(wbase[t] + (uint32_t)(wo + u * kTileBytes)));
 #pragma unroll
       for (int g = 0; g < GSUB; ++g) snext[t][g] = sbase[t][(uint32_t)((g0 + g) * kTileN + r)];
       // raw: any use here would wait for the load inside the request
@@ -509,13 +518,14 @@ __global__ __launch_bounds__(512, (GSUB * MT > 4 ? 2 : 4)) void woq_decode_w4i8_
   if (wave < KT) request(wave, 0);
 #pragma unroll 1
   for (int kt = wave, buf = 0; kt < KT; kt += W, buf ^= 1) {
-    u4 wreg[NTW];
+    u4 wreg[NTW][TPR];
     float sw[NTW][GSUB];
     uint32_t z4[NTW];
     f4 sa[PER_K ? GSUB : 1][PER_K ? MT : 1];
 #pragma unroll
     for (int t = 0; t < NTW; ++t) {
-      wreg[t] = wnext[t];
+#pragma unroll
+      for (int u = 0; u < TPR; ++u) wreg[t][u] = wnext[t][u];
 #pragma unroll
       for (int g = 0; g < GSUB; ++g) sw[t][g] = NF4 ? snext[t][g] * (1.0f / 127.0f) : snext[t][g];
       z4[t] = (has_z ? (uint32_t)znext[t] : 8u) * 0x01010101u;
@@ -538,8 +548,18 @@ __global__ __launch_bounds__(512, (GSUB * MT > 4 ? 2 : 4)) void woq_decode_w4i8_
       for (int j = 0; j < 2; ++j) xa[mt][j] = *(const i4*)(sx + buf * SLICE + mt * 2048 + rd[j]);
 #pragma unroll
     for (int t = 0; t < NTW; ++t) {
-      const i4 bq0 = NF4 ? w8_decode16_nf4(wreg[t][0], wreg[t][1]) : w8_decode16(wreg[t][0], wreg[t][1], z4[t]);
-      const i4 bq1 = NF4 ? w8_decode16_nf4(wreg[t][2], wreg[t][3]) : w8_decode16(wreg[t][2], wreg[t][3], z4[t]);
+      i4 bq0, bq1;
+      if constexpr (WBITS == 8) {
+        // offset-binary bytes: flipping the sign bit leaves the two's complement weight
+        bq0 = bitcast<i4>(wreg[t][0] ^ u4{0x80808080u, 0x80808080u, 0x80808080u, 0x80808080u});
+        bq1 = bitcast<i4>(wreg[t][TPR - 1] ^ u4{0x80808080u, 0x80808080u, 0x80808080u, 0x80808080u});
+      } else if constexpr (NF4) {
+        bq0 = w8_decode16_nf4(wreg[t][0][0], wreg[t][0][1]);
+        bq1 = w8_decode16_nf4(wreg[t][0][2], wreg[t][0][3]);
+      } else {
+        bq0 = w8_decode16(wreg[t][0][0], wreg[t][0][1], z4[t]);
+        bq1 = w8_decode16(wreg[t][0][2], wreg[t][0][3], z4[t]);
+      }
 #pragma unroll
       for (int g = 0; g < GSUB; ++g) {
         // activation fragments of K block g: the lane columns of the other blocks contribute zeros
@@ -599,8 +619,16 @@ static int decode_w4i8_max_rows(int64_t group_size) { return group_size == 64 ? 
 // 64-row tiles of the MFMA GEMM, which with a single row tile still beats the general small-M kernel
 // (4096 -> 14336, per-row scales, M = 48 / 64: 34 / 36 us against 157 / 162 us).
 bool gemm_w4i8_applies(const Int8Args& a, int64_t block_k, int64_t qbk, bool per_k, bool asym) {
-  if (a.wbits != 4 || asym || a.debug_block_sums) return false;
+  if (asym || a.debug_block_sums) return false;
   if (a.K % 128 != 0) return false;
+  if (a.wbits == 8) {
+    // symmetric 8-bit weights: the decode form only, one scale per channel or per 128 * 2^s input channels
+    if (a.zeros || a.M > 32 || block_k != 128) return false;
+    if (a.group_size > 0 && (a.G % 128 != 0 || ((a.G / 128) & (a.G / 128 - 1)) != 0)) return false;
+    if (per_k && (qbk % 128 != 0 || ((qbk / 128) & (qbk / 128 - 1)) != 0)) return false;
+    return a.M * a.K < ((int64_t)1 << 31);
+  }
+  if (a.wbits != 4) return false;
   // NF4 codes: the decode form only (up to two row tiles)
   if (a.nf4 && (a.M > 32 || a.zeros)) return false;
   if (block_k == 32 || block_k == 64) {
@@ -651,7 +679,8 @@ int launch_gemm_w4i8(const Int8Args& a, const uint8_t* xq, int64_t ldq, const fl
     const int slice = mt * 16 * kTileK4;
     int w = 65536 / (2 * slice);  // at most 64 KiB of activation slices
     if (w > 8) w = 8;
-    d.W = (int)(a.KT < w ? a.KT : w);
+    const int64_t rounds = a.KT / (a.wbits / 4);
+    d.W = (int)(rounds < w ? rounds : w);
     size_t smem = (size_t)d.W * 2 * slice;
     const size_t red = (size_t)ntw * mt * d.W * 64 * sizeof(f4);
     if (red > smem) smem = red;
@@ -671,6 +700,21 @@ int launch_gemm_w4i8(const Int8Args& a, const uint8_t* xq, int64_t ldq, const fl
     else                                                                                       \
       woq_decode_w4i8_kernel<false, MTV, NTWV, GS, true><<<dgrid, d.W * 64, smem, st>>>(d);    \
   } while (0)
+    if (a.wbits == 8) {  // at most two row tiles, one K block per round (gemm_w4i8_applies)
+#define WOQ_DECODE_W8I8(MTV, NTWV)                                                                  \
+  do {                                                                                              \
+    if (per_k)                                                                                      \
+      woq_decode_w4i8_kernel<true, MTV, NTWV, 1, false, 8><<<dgrid, d.W * 64, smem, st>>>(d);       \
+    else                                                                                            \
+      woq_decode_w4i8_kernel<false, MTV, NTWV, 1, false, 8><<<dgrid, d.W * 64, smem, st>>>(d);      \
+  } while (0)
+      if (mt == 2 && ntw == 2) WOQ_DECODE_W8I8(2, 2);
+      else if (mt == 2) WOQ_DECODE_W8I8(2, 1);
+      else if (ntw == 2) WOQ_DECODE_W8I8(1, 2);
+      else WOQ_DECODE_W8I8(1, 1);
+#undef WOQ_DECODE_W8I8
+      return check_launch("woq_decode_w4i8_kernel");
+    }
     if (a.nf4) {  // at most two row tiles (gemm_w4i8_applies)
       if (mt == 2) {
         if (gsub == 4) WOQ_DECODE_W4I8_NF4(2, 1, 4);

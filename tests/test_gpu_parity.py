@@ -876,6 +876,16 @@ def test_int8_lowp_int8_weights(cuda):
         _check_int8(case, 6, label=f"int8 lowp int8 weights M={M}")
 
 
+@pytest.mark.parametrize("mode", [4, 6, 7])
+@pytest.mark.parametrize("M,K,N,G", [(1, 1024, 272, -1), (16, 4096, 8208, -1), (17, 1152, 96, 128), (32, 2048, 1040, 256)])
+def test_int8_lowp_int8_weights_decode_kernel(cuda, mode, M, K, N, G):
+    """Symmetric 8-bit weights in the int8 MFMA decode kernel: two packed tiles per round, the lane's
+    bytes are the B operand as they are."""
+    case = _synthetic().make_int8_case(23, M, K, N, group_size=G)
+    cols = None if N < 4096 else list(range(0, N, 53)) + [N - 1]
+    _check_int8(case, mode, cols=cols, debug=N < 4096, label=f"int8 lowp int8 weights decode mode={mode} M={M} K={K} N={N} G={G}")
+
+
 def test_c3_prefill_int8(cuda):
     case = _synthetic().make_int4_case(3, 2048, 4096, 14336, 128, outliers=True)
     _check_int8(case, 6, cols=np.arange(0, 14336, 61), debug=False, label="C3 int8 per-M")
