@@ -45,6 +45,7 @@ struct W4I8Args {
   int64_t sa_m_stride;     // per row: scales per row (1 or the K blocks per row), else 0
   int64_t sa_k_stride;     // per K block: 1, else 0
   int q_shift;             // K tile kt belongs to activation K block kt >> q_shift
+  const int32_t* za;       // asymmetric activations: zero points, indexed like sa; xq then holds q_a - 128
   int64_t M, N, NT, KT, KG;
   const uint8_t* qweight;
   const float* scales;     // fp32 [NT][KG][16]
@@ -90,6 +91,18 @@ __device__ __forceinline__ float w8_accumulate(int sum, float s_a, float s_w, fl
     return __builtin_fmaf((float)sum, s_w, acc);
 }
 
+// Asymmetric activations (uint8 q_a with zero point z_a; csrc/cpu/aten/utils/woq.h:2172-2186): the
+// reference's block integer is sum q_a B - z_a sum B.  The activations arrive as the int8 numbers
+// q_a - 128, so it equals (sum (q_a - 128) B) + (128 - z_a) sum B, with the column sums of the block's
+// weights ("compensation") from one more pair of MFMAs against rows of ones: every row of that D tile
+// is the same, so register 0 of a lane is the sum of its column n = lane % 16.
+__device__ __forceinline__ int w8_column_sums(i4 bq0, i4 bq1) {
+  const i4 ones = i4{0x01010101, 0x01010101, 0x01010101, 0x01010101};
+  i4 cv = __builtin_amdgcn_mfma_i32_16x16x64_i8(ones, bq0, i4{0, 0, 0, 0}, 0, 0, 0);
+  cv = __builtin_amdgcn_mfma_i32_16x16x64_i8(ones, bq1, cv, 0, 0, 0);
+  return cv[0];
+}
+
 // NF4 codes under lowp_mode INT8: the code's table value times 127, rounded, as int8
 // (load_nf4_as_int8, csrc/cpu/aten/utils/woq.h:628-669): two byte permutes over the halves of the
 // table (codes 0..7 and 8..15), merged on bit 3 of each code; the weight scale carries the 1 / 127.
@@ -112,12 +125,15 @@ __device__ __forceinline__ i4 w8_decode16_nf4(uint32_t d0, uint32_t d1) {
 }
 
 // PER_K: the activation scales change with the K block; they reach the lanes through LDS.
-template <bool PER_K>
+// ASYM: asymmetric activations (w8_column_sums); the zero points travel like the scales.
+template <bool PER_K, bool ASYM = false>
 __global__ __launch_bounds__(256, 3) void woq_gemm_w4i8_kernel(const W4I8Args a) {
-  // the activation buffers, then the weight stages, then the activation scales of a step's rows
+  // the activation buffers, then the weight stages, then the activation scales (and, ASYM, zero points)
+  // of a step's rows
   extern __shared__ __align__(1024) uint8_t sX[];
   uint8_t* const sW = sX + W8_NBUF * W8_XBYTES;
   float* const sSA = (float*)(sW + W8_NBUF * W8_WSTAGE);
+  int32_t* const sZA = (int32_t*)(sSA + W8_NBUF * W8_BM);
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -153,6 +169,19 @@ __global__ __launch_bounds__(256, 3) void woq_gemm_w4i8_kernel(const W4I8Args a)
   const int sa_row = m0 + tid < M ? m0 + tid : M - 1;  // wave 0: the row whose scale this thread fetches
   const float* const sa_mine = a.sa + (int64_t)sa_row * a.sa_m_stride;
   float sa_next = 0.0f;
+  // 128 - z_a of the same rows
+  i4 zoff[ASYM ? W8_MT : 1];
+  if (ASYM && !PER_K) {
+#pragma unroll
+    for (int mt = 0; mt < (ASYM ? W8_MT : 1); ++mt)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const int m = m0 + mt * 16 + 4 * c + e;
+        zoff[mt][e] = 128 - a.za[(int64_t)(m < M ? m : M - 1) * a.sa_m_stride];
+      }
+  }
+  const int32_t* const za_mine = ASYM ? a.za + (int64_t)sa_row * a.sa_m_stride : nullptr;
+  int32_t za_next = 0;
 
   // ---- activations: load i of wave w fills LDS KiB number w * XLOADS + i of a buffer: rows
   // 8 (w * XLOADS + i) + lane / 8, physical chunk lane % 8 = logical chunk ^ ((row / 2) % 8).
@@ -236,6 +265,7 @@ __global__ __launch_bounds__(256, 3) void woq_gemm_w4i8_kernel(const W4I8Args a)
   for (int t = 0; t < W8_NTW; ++t) wr[t] = *(const u4*)(wmine + t * kTileBytes + woff);
 
   if (PER_K && tid < W8_BM) sSA[tid] = sa_mine[(int64_t)(kt_lo >> a.q_shift) * a.sa_k_stride];
+  if (PER_K && ASYM && tid < W8_BM) sZA[tid] = za_mine[(int64_t)(kt_lo >> a.q_shift) * a.sa_k_stride];
   __syncthreads();
 
   // Per K step: the MFMAs of row-block 0, then those of row-block 1 with the fp32 epilogue of
@@ -250,6 +280,7 @@ __global__ __launch_bounds__(256, 3) void woq_gemm_w4i8_kernel(const W4I8Args a)
     // into the buffers of step kt - 1, which every wave left before the last barrier
     load_q(kt1, swn, zqn);
     if (PER_K && tid < W8_BM) sa_next = sa_mine[(int64_t)(kt1 >> a.q_shift) * a.sa_k_stride];
+    if (PER_K && ASYM && tid < W8_BM) za_next = za_mine[(int64_t)(kt1 >> a.q_shift) * a.sa_k_stride];
     __builtin_amdgcn_sched_barrier(0);  // the parameter loads stay the oldest requests of the step
     load_x(kt2, b2);
     dma_w(kt2, b2);
@@ -258,6 +289,11 @@ __global__ __launch_bounds__(256, 3) void woq_gemm_w4i8_kernel(const W4I8Args a)
     if (PER_K) {
 #pragma unroll
       for (int mt = 0; mt < W8_MT; ++mt) sa[mt] = *(const f4*)(sSA + b0 * W8_BM + mt * 16 + 4 * c);
+      if constexpr (ASYM) {
+#pragma unroll
+        for (int mt = 0; mt < W8_MT; ++mt)
+          zoff[mt] = i4{128, 128, 128, 128} - *(const i4*)(sZA + b0 * W8_BM + mt * 16 + 4 * c);
+      }
     }
     // A fragments of the step: 2 MFMAs x MT row tiles
     i4 xa[2][W8_MT];
@@ -267,11 +303,13 @@ __global__ __launch_bounds__(256, 3) void woq_gemm_w4i8_kernel(const W4I8Args a)
       for (int mt = 0; mt < W8_MT; ++mt) xa[j][mt] = *(const i4*)(xs + mt * 2048 + rd[j]);
 
     i4 qc[W8_NTW][W8_MT];
+    int cm[W8_NTW];  // ASYM: column sum of the block's weights, row-block t
 #pragma unroll
     for (int t = 0; t < W8_NTW; ++t) {
       const uint32_t z4 = (has_z ? (uint32_t)zq[t] : 8u) * 0x01010101u;
       const i4 bq0 = w8_decode16(wr[t][0], wr[t][1], z4);
       const i4 bq1 = w8_decode16(wr[t][2], wr[t][3], z4);
+      cm[t] = ASYM ? w8_column_sums(bq0, bq1) : 0;
       __builtin_amdgcn_sched_barrier(0);
       // one MFMA, then (second row-block) the fp32 epilogue of two sums of the first:
       // C += (float(sum) * s_a[m]) * s_w[n, g]; each pair is fenced so that the order stands
@@ -286,7 +324,8 @@ __global__ __launch_bounds__(256, 3) void woq_gemm_w4i8_kernel(const W4I8Args a)
 #pragma unroll
           for (int u = 0; u < 2; ++u) {
             const int q = 2 * i + u, pm = q / 4, pe = q % 4;
-            acc[pm][t - 1][pe] = w8_accumulate<PER_K>(qc[t - 1][pm][pe], sa[pm][pe], sw[t - 1], acc[pm][t - 1][pe]);
+            const int qv = ASYM ? qc[t - 1][pm][pe] + cm[t - 1] * zoff[ASYM ? pm : 0][pe] : qc[t - 1][pm][pe];
+            acc[pm][t - 1][pe] = w8_accumulate<PER_K>(qv, sa[pm][pe], sw[t - 1], acc[pm][t - 1][pe]);
           }
         }
         __builtin_amdgcn_sched_barrier(0);
@@ -296,8 +335,8 @@ __global__ __launch_bounds__(256, 3) void woq_gemm_w4i8_kernel(const W4I8Args a)
     for (int mt = 0; mt < W8_MT; ++mt)
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
-        acc[mt][W8_NTW - 1][e] = w8_accumulate<PER_K>(qc[W8_NTW - 1][mt][e], sa[mt][e], sw[W8_NTW - 1],
-                                                      acc[mt][W8_NTW - 1][e]);
+        const int qv = ASYM ? qc[W8_NTW - 1][mt][e] + cm[W8_NTW - 1] * zoff[ASYM ? mt : 0][e] : qc[W8_NTW - 1][mt][e];
+        acc[mt][W8_NTW - 1][e] = w8_accumulate<PER_K>(qv, sa[mt][e], sw[W8_NTW - 1], acc[mt][W8_NTW - 1][e]);
       }
 
     // Next step: its activations and tiles (requested a step ago) must have landed -- every wave
@@ -306,6 +345,7 @@ __global__ __launch_bounds__(256, 3) void woq_gemm_w4i8_kernel(const W4I8Args a)
     // compiler waits for every outstanding load, the requests for step kt + 2 included.
     if (PER_K) {
       if (tid < W8_BM) sSA[b1 * W8_BM + tid] = sa_next;
+      if (ASYM && tid < W8_BM) sZA[b1 * W8_BM + tid] = za_next;
       __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): the LDS write is done before the barrier
     }
     __builtin_amdgcn_s_waitcnt(kVmcntStep);
@@ -422,9 +462,11 @@ struct DecodeW4I8Args {
 // WBITS 8: symmetric 8-bit weights, stored offset-binary; a packed tile is 16 rows x 64 K values, so a
 // round takes two tiles per row-block (one MFMA each) and the lane's 16 bytes are the B operand as they
 // are, sign bit flipped; the A fragment of tile u is chunk 4 u + c of the 128-byte row.
-template <bool PER_K, int MT, int NTW, int GSUB, bool NF4, int WBITS = 4>
+// ASYM: asymmetric activations (w8_column_sums), for 4-bit integer codes with one K block per tile.
+template <bool PER_K, int MT, int NTW, int GSUB, bool NF4, int WBITS = 4, bool ASYM = false>
 __global__ __launch_bounds__(512, (GSUB * MT > 4 ? 2 : 4)) void woq_decode_w4i8_kernel(const DecodeW4I8Args a) {
   static_assert(WBITS == 4 || (WBITS == 8 && GSUB == 1 && !NF4), "8-bit weights: one K block per round");
+  static_assert(!ASYM || (WBITS == 4 && GSUB == 1 && !NF4), "asymmetric activations: 4-bit codes, one K block per tile");
   constexpr int TPR = WBITS / 4;  // packed tiles per row-block and round of 128 K values
   constexpr int SLICE = MT * 16 * kTileK4;  // one buffer of one wave: 16 MT rows x 128 bytes
   constexpr int NX = 2 * MT;                // activation loads per tile (eight rows each)
@@ -479,6 +521,18 @@ __global__ __launch_bounds__(512, (GSUB * MT > 4 ? 2 : 4)) void woq_decode_w4i8_
   float snext[NTW][GSUB];
   uint8_t znext[NTW];
   f4 sanext[PER_K ? GSUB : 1][PER_K ? MT : 1];
+  i4 zanext[PER_K && ASYM ? MT : 1];
+  // 128 - z_a of the accumulator rows: fixed (one zero point per row or tensor) or per K block
+  i4 zoff[ASYM ? MT : 1];
+  if constexpr (ASYM && !PER_K) {
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const int m = 16 * mt + 4 * c + e;
+        zoff[mt][e] = 128 - k.za[(int64_t)(m < M ? m : M - 1) * k.sa_m_stride];
+      }
+  }
   const int my_block = c / (4 / GSUB);  // K block of the tile this lane column's weights belong to
   auto request = [&](int kt, int buf) {
     const uint32_t ko = (uint32_t)kt * kTileK4;
@@ -511,6 +565,8 @@ __global__ __launch_bounds__(512, (GSUB * MT > 4 ? 2 : 4)) void woq_decode_w4i8_
             const int m = 16 * mt + 4 * c + e;
             const int64_t kb = GSUB == 1 ? (int64_t)(kt >> k.q_shift) : (int64_t)kt * GSUB + g;
             sanext[g][mt][e] = k.sa[(int64_t)(m < M ? m : M - 1) * k.sa_m_stride + kb * k.sa_k_stride];
+            if constexpr (ASYM)
+              zanext[mt][e] = k.za[(int64_t)(m < M ? m : M - 1) * k.sa_m_stride + kb * k.sa_k_stride];
           }
     }
   };
@@ -535,6 +591,10 @@ __global__ __launch_bounds__(512, (GSUB * MT > 4 ? 2 : 4)) void woq_decode_w4i8_
       for (int g = 0; g < GSUB; ++g)
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) sa[g][mt] = sanext[g][mt];
+      if constexpr (ASYM) {
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) zoff[mt] = i4{128, 128, 128, 128} - zanext[mt];
+      }
     }
     // the compiler does not order LDS reads after the LDS-writing loads: wait for them here
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
@@ -560,6 +620,7 @@ __global__ __launch_bounds__(512, (GSUB * MT > 4 ? 2 : 4)) void woq_decode_w4i8_
         bq0 = w8_decode16(wreg[t][0][0], wreg[t][0][1], z4[t]);
         bq1 = w8_decode16(wreg[t][0][2], wreg[t][0][3], z4[t]);
       }
+      const int cm = ASYM ? w8_column_sums(bq0, bq1) : 0;
 #pragma unroll
       for (int g = 0; g < GSUB; ++g) {
         // activation fragments of K block g: the lane columns of the other blocks contribute zeros
@@ -573,8 +634,10 @@ __global__ __launch_bounds__(512, (GSUB * MT > 4 ? 2 : 4)) void woq_decode_w4i8_
           i4 qc = __builtin_amdgcn_mfma_i32_16x16x64_i8(xg0, bq0, i4{0, 0, 0, 0}, 0, 0, 0);
           qc = __builtin_amdgcn_mfma_i32_16x16x64_i8(xg1, bq1, qc, 0, 0, 0);
 #pragma unroll
-          for (int e = 0; e < 4; ++e)
-            acc[t][mt][e] = w8_accumulate<PER_K>(qc[e], PER_K ? sa[g][mt][e] : 0.0f, sw[t][g], acc[t][mt][e]);
+          for (int e = 0; e < 4; ++e) {
+            const int qv = ASYM ? qc[e] + cm * zoff[ASYM ? mt : 0][e] : qc[e];
+            acc[t][mt][e] = w8_accumulate<PER_K>(qv, PER_K ? sa[g][mt][e] : 0.0f, sw[t][g], acc[t][mt][e]);
+          }
         }
       }
     }
@@ -619,8 +682,10 @@ static int decode_w4i8_max_rows(int64_t group_size) { return group_size == 64 ? 
 // 64-row tiles of the MFMA GEMM, which with a single row tile still beats the general small-M kernel
 // (4096 -> 14336, per-row scales, M = 48 / 64: 34 / 36 us against 157 / 162 us).
 bool gemm_w4i8_applies(const Int8Args& a, int64_t block_k, int64_t qbk, bool per_k, bool asym) {
-  if (asym || a.debug_block_sums) return false;
+  if (a.debug_block_sums) return false;
   if (a.K % 128 != 0) return false;
+  // asymmetric activations: 4-bit integer codes with groups of at least 128
+  if (asym && (a.wbits != 4 || a.nf4 || block_k != 128)) return false;
   if (a.wbits == 8) {
     // symmetric 8-bit weights: the decode form only, one scale per channel or per 128 * 2^s input channels
     if (a.zeros || a.M > 32 || block_k != 128) return false;
@@ -644,17 +709,25 @@ bool gemm_w4i8_applies(const Int8Args& a, int64_t block_k, int64_t qbk, bool per
 }
 
 int launch_gemm_w4i8(const Int8Args& a, const uint8_t* xq, int64_t ldq, const float* sa, int64_t sa_m_stride,
-                     int64_t sa_k_stride, int64_t qbk, hipStream_t st, const SplitKScratch* scratch) {
-  static const hipError_t lds_optin[2] = {
-      hipFuncSetAttribute(reinterpret_cast<const void*>(&woq_gemm_w4i8_kernel<false>),
+                     int64_t sa_k_stride, int64_t qbk, hipStream_t st, const SplitKScratch* scratch,
+                     const int32_t* za) {
+  constexpr int kLdsAsym = W8_LDS_BYTES + W8_NBUF * W8_BM * (int)sizeof(int32_t);
+  static const hipError_t lds_optin[4] = {
+      hipFuncSetAttribute(reinterpret_cast<const void*>(&woq_gemm_w4i8_kernel<false, false>),
                           hipFuncAttributeMaxDynamicSharedMemorySize, W8_LDS_BYTES),
-      hipFuncSetAttribute(reinterpret_cast<const void*>(&woq_gemm_w4i8_kernel<true>),
-                          hipFuncAttributeMaxDynamicSharedMemorySize, W8_LDS_BYTES)};
-  if (lds_optin[0] != hipSuccess || lds_optin[1] != hipSuccess)
-    return set_error("woq_gemm_w4i8_kernel: LDS opt-in failed: %s",
-                     hipGetErrorString(lds_optin[0] != hipSuccess ? lds_optin[0] : lds_optin[1]));
+      hipFuncSetAttribute(reinterpret_cast<const void*>(&woq_gemm_w4i8_kernel<true, false>),
+                          hipFuncAttributeMaxDynamicSharedMemorySize, W8_LDS_BYTES),
+      hipFuncSetAttribute(reinterpret_cast<const void*>(&woq_gemm_w4i8_kernel<false, true>),
+                          hipFuncAttributeMaxDynamicSharedMemorySize, kLdsAsym),
+      hipFuncSetAttribute(reinterpret_cast<const void*>(&woq_gemm_w4i8_kernel<true, true>),
+                          hipFuncAttributeMaxDynamicSharedMemorySize, kLdsAsym)};
+  for (int i = 0; i < 4; ++i)
+    if (lds_optin[i] != hipSuccess)
+      return set_error("woq_gemm_w4i8_kernel: LDS opt-in failed: %s", hipGetErrorString(lds_optin[i]));
+  const bool asym = za != nullptr;
   W4I8Args k;
   k.xq = xq; k.ldq = ldq; k.sa = sa; k.sa_m_stride = sa_m_stride; k.sa_k_stride = sa_k_stride;
+  k.za = za;
   k.q_shift = 0;
   while (sa_k_stride != 0 && ((int64_t)128 << k.q_shift) < qbk) ++k.q_shift;
   k.M = a.M; k.N = a.N; k.NT = a.NT; k.KT = a.KT; k.KG = a.KG;
@@ -700,6 +773,21 @@ int launch_gemm_w4i8(const Int8Args& a, const uint8_t* xq, int64_t ldq, const fl
     else                                                                                       \
       woq_decode_w4i8_kernel<false, MTV, NTWV, GS, true><<<dgrid, d.W * 64, smem, st>>>(d);    \
   } while (0)
+    if (asym) {  // 4-bit integer codes, one K block per tile, at most two row tiles (gemm_w4i8_applies)
+#define WOQ_DECODE_W4I8_ASYM(MTV, NTWV)                                                                  \
+  do {                                                                                                   \
+    if (per_k)                                                                                           \
+      woq_decode_w4i8_kernel<true, MTV, NTWV, 1, false, 4, true><<<dgrid, d.W * 64, smem, st>>>(d);      \
+    else                                                                                                 \
+      woq_decode_w4i8_kernel<false, MTV, NTWV, 1, false, 4, true><<<dgrid, d.W * 64, smem, st>>>(d);     \
+  } while (0)
+      if (mt == 2 && ntw == 2) WOQ_DECODE_W4I8_ASYM(2, 2);
+      else if (mt == 2) WOQ_DECODE_W4I8_ASYM(2, 1);
+      else if (ntw == 2) WOQ_DECODE_W4I8_ASYM(1, 2);
+      else WOQ_DECODE_W4I8_ASYM(1, 1);
+#undef WOQ_DECODE_W4I8_ASYM
+      return check_launch("woq_decode_w4i8_kernel");
+    }
     if (a.wbits == 8) {  // at most two row tiles, one K block per round (gemm_w4i8_applies)
 #define WOQ_DECODE_W8I8(MTV, NTWV)                                                                  \
   do {                                                                                              \
@@ -765,7 +853,11 @@ int launch_gemm_w4i8(const Int8Args& a, const uint8_t* xq, int64_t ldq, const fl
       }
     }
   }
-  if (sa_k_stride != 0)
+  if (asym && sa_k_stride != 0)
+    woq_gemm_w4i8_kernel<true, true><<<grid, 256, kLdsAsym, st>>>(k);
+  else if (asym)
+    woq_gemm_w4i8_kernel<false, true><<<grid, 256, kLdsAsym, st>>>(k);
+  else if (sa_k_stride != 0)
     woq_gemm_w4i8_kernel<true><<<grid, 256, W8_LDS_BYTES, st>>>(k);
   else
     woq_gemm_w4i8_kernel<false><<<grid, 256, W8_LDS_BYTES, st>>>(k);

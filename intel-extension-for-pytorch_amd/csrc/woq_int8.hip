@@ -211,10 +211,10 @@ static int launch_quant_impl(const void* x, int x_dtype, int64_t M, int64_t K, i
   if (qbk <= 0) qbk = K;
   const int64_t Kc = (K + qbk - 1) / qbk;
   const int64_t groups = num_quant_groups(M, Kc, mode);
-  // one pass over whole rows where a row fits a wave's registers; otherwise statistics, then quantization
+  // whole rows from a wave's registers where a row fits them; otherwise the general statistics and quantization
   if (act_quant_rows_applies(x, x_dtype, K, q, ldq, qbk, quant_a_per_m(mode), quant_a_per_k(mode)))
-    return launch_act_quant_rows(x, x_dtype, M, K, ldq, qbk, Kc, quant_a_per_k(mode), quant_a_is_sym(mode), q, scales,
-                                 zps, permute, offset128, st);
+    return launch_act_quant_rows(x, x_dtype, M, K, ldq, qbk, Kc, quant_a_per_m(mode), quant_a_per_k(mode),
+                                 quant_a_is_sym(mode), q, scales, zps, permute, offset128, st);
   if (quant_a_per_m(mode)) {
     act_stats_kernel<<<(unsigned)groups, 256, 0, st>>>(x, x_dtype, M, K, qbk, Kc, mode, scales, zps);
     if (int rc = check_launch("act_stats_kernel")) return rc;
@@ -786,13 +786,14 @@ int launch_int8_linear(const Int8Args& a, hipStream_t st) {
       scratch.bytes = a.workspace_bytes - used;
       scratch.counters = a.split_k_counters;
     }
-    return launch_gemm_w4i8(a, xq, p.ldq, sa, p.sa_m_stride, p.sa_k_stride, qbk_quant, st, &scratch);
+    return launch_gemm_w4i8(a, xq, p.ldq, sa, p.sa_m_stride, p.sa_k_stride, qbk_quant, st, &scratch, za);
   }
 
   // The small-M kernel accumulates whole tiles per MFMA, so it needs K blocks that are whole
   // tiles; finer blocks (group_size 32 / 64 with 4-bit weights) go through the tiled kernel,
   // which re-lays the weights in LDS in plain K order.
-  // Asymmetric activations (rare: the reference's default is symmetric) always take the tiled kernel.
+  // Asymmetric activations that the kernels above do not take (8-bit or NF4 weights, groups below 128)
+  // take the tiled kernel.
   if (!asym && a.M <= 64 && p.block_k % TK == 0)
     return a.wbits == 4 ? dispatch_small_i8<4>(p, st) : dispatch_small_i8<8>(p, st);
   dim3 grid((unsigned)((a.NT * kTileN + IBN - 1) / IBN), (unsigned)((a.M + IBM - 1) / IBM));

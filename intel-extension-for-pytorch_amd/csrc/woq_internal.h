@@ -133,18 +133,22 @@ struct Int8Args {
   int nf4;  // 4-bit codes index the NF4 int8 table; the weight scale is multiplied by fp32(1 / 127)
 };
 
-// int8 MFMA prefill kernel for 4-bit weights (woq_gemm_w4i8.hip): symmetric activation scales, K
-// blocks of 128; sa[m * sa_m_stride + (k / qbk) * sa_k_stride] is the scale of row m at k.
+// int8 MFMA kernels that feed the stored codes to the MFMA (woq_gemm_w4i8.hip);
+// sa[m * sa_m_stride + (k / qbk) * sa_k_stride] is the activation scale of row m at k, za (asymmetric
+// modes, else nullptr) the zero point at the same index, the quantized activations then being q_a - 128.
 bool gemm_w4i8_applies(const Int8Args& a, int64_t block_k, int64_t qbk, bool per_k, bool asym);
 int launch_gemm_w4i8(const Int8Args& a, const uint8_t* xq, int64_t ldq, const float* sa, int64_t sa_m_stride,
-                     int64_t sa_k_stride, int64_t qbk, hipStream_t st, const SplitKScratch* scratch = nullptr);
-// One-pass quantization of whole rows (woq_act_quant.hip): 16-bit activations, one scale per row or per
-// (row, K block), padded rows of at most 16384 elements.  Same bytes and scales as the two-kernel form.
+                     int64_t sa_k_stride, int64_t qbk, hipStream_t st, const SplitKScratch* scratch = nullptr,
+                     const int32_t* za = nullptr);
+// Quantization of whole rows from registers (woq_act_quant.hip): 16-bit activations, padded rows of at
+// most 16384 elements.  per_m (one scale per row or per (row, K block)): one pass; scales shared by all
+// rows: a statistics pass, then the same kernel with the scales given.  Same bytes and scales as the
+// general form in woq_int8.hip.
 bool act_quant_rows_applies(const void* x, int x_dtype, int64_t K, const void* q, int64_t ldq, int64_t qbk,
                             bool per_m, bool per_k);
 int launch_act_quant_rows(const void* x, int x_dtype, int64_t M, int64_t K, int64_t ldq, int64_t qbk, int64_t Kc,
-                          bool per_k, bool sym, void* q, float* scales, int32_t* zps, int permute, int offset128,
-                          hipStream_t st);
+                          bool per_m, bool per_k, bool sym, void* q, float* scales, int32_t* zps, int permute,
+                          int offset128, hipStream_t st);
 int launch_dynamic_quant(const void* x, int x_dtype, int64_t M, int64_t K, int64_t ldq, int64_t qbk,
                          int mode, void* q, float* scales, int32_t* zps, hipStream_t st);
 int launch_int8_linear(const Int8Args& a, hipStream_t st);

@@ -766,6 +766,35 @@ def test_dynamic_quant_rows_bit_exact(cuda, mode, M, K, block, dtype):
         assert np.array_equal(zp.cpu().numpy().reshape(-1), zp_ref.reshape(-1))
 
 
+@pytest.mark.parametrize("mode", [0, 1, 4, 5])
+@pytest.mark.parametrize(
+    "M,K,block,dtype",
+    [
+        (2100, 4096, 128, torch.bfloat16),  # eight rows per workgroup, the last workgroup partly empty
+        (9, 8192, 64, torch.bfloat16),
+        (70, 14336, 512, torch.bfloat16),  # thirty-two chunks; more than 64 rows: a wave per row
+        (6, 1000, 32, torch.float16),  # a partial last block
+        (1, 4096, 128, torch.float16),  # one row: its statistics are the tensor's
+        (4, 24576, 128, torch.bfloat16),  # rows too long for a wave's registers: the general form
+    ],
+)
+def test_dynamic_quant_shared_scales_bit_exact(cuda, mode, M, K, block, dtype):
+    """One scale per tensor or per K block (shared by all rows): statistics merged over workgroups,
+    then quantization with the scales given; one K block is all zeros (scale 0 in the per-block modes)."""
+    k = _kernels()
+    x = torch.randn(M, K, generator=torch.Generator().manual_seed(M * 5 + K + mode)) * 2.0
+    x[:, block : 2 * block] = 0.0
+    x[0, :5] = torch.tensor([0.5, -0.5, 1.5, 2.5, 1e-3])
+    x[M // 2, K - 1] = 9.0
+    x = x.to(dtype)
+    q, s, zp = k.dynamic_quant(x.to(cuda), block, mode)
+    q_ref, s_ref, zp_ref = O.dynamic_quantize_per_block(x.float().numpy(), block, mode)
+    assert np.array_equal(s.cpu().numpy().reshape(-1), s_ref.reshape(-1))
+    assert np.array_equal(q.cpu().numpy(), q_ref)
+    if mode < 4:
+        assert np.array_equal(zp.cpu().numpy().reshape(-1), zp_ref.reshape(-1))
+
+
 def test_dynamic_quant_all_bf16_patterns(cuda):
     k = _kernels()
     bits = torch.arange(65536, dtype=torch.int32).to(torch.int16)
@@ -786,12 +815,13 @@ def _check_int8(case, mode, cols=None, debug=True, label=""):
     N, K, G = case["N"], case["K"], case["group_size"]
     c = case_np(case)
     y = to_np_f32(ctx.run(x))
+    # the accumulators of the kernel that serves the call, and (debug) those of the general kernel with
+    # its block sums
+    acc = ctx.run(x, out_fp32=True).cpu().numpy()
+    acc_dbg, sums = None, None
     if debug:
-        acc, sums = ctx.run(x, out_fp32=True, debug_block_sums=True)
-        sums = sums.cpu().numpy()
-    else:
-        acc, sums = ctx.run(x, out_fp32=True), None
-    acc = acc.cpu().numpy()
+        acc_dbg, sums = ctx.run(x, out_fp32=True, debug_block_sums=True)
+        acc_dbg, sums = acc_dbg.cpu().numpy(), sums.cpu().numpy()
     qw, sc, zp, b = c["qw"], c["scales"], c["zps"], c["bias"]
     if cols is not None:
         qw, sc = qw[cols], sc[cols]
@@ -799,11 +829,14 @@ def _check_int8(case, mode, cols=None, debug=True, label=""):
         b = None if b is None else b[cols]
         y, acc = y[:, cols], acc[:, cols]
         sums = None if sums is None else sums[:, cols]
+        acc_dbg = None if acc_dbg is None else acc_dbg[:, cols]
         N = len(cols)
     r = O.woq_linear_opt_int8(c["x"], "bf16", qw, N, K, sc, zp, b, case["weight_dtype"], G, mode)
     if sums is not None:
         assert np.array_equal(sums[:, :, : r["sums"].shape[2]], r["sums"]), label  # int32, bit-exact
     stats = {"max_abs_acc": max_abs(acc, r["acc"]), "rel_l2_out": rel_l2(y, r["y"])}
+    if acc_dbg is not None:
+        stats["max_abs_acc"] = max(stats["max_abs_acc"], max_abs(acc_dbg, r["acc"]))
     print(label, stats)
     assert stats["max_abs_acc"] <= MAX_ABS_ACC and stats["rel_l2_out"] <= REL_L2_OUT, (label, stats)
     return stats
@@ -824,6 +857,38 @@ def test_int8_lowp_asymmetric_activations(cuda, mode, M, K, N, G):
     case = _synthetic().make_int4_case(28, M, K, N, G, bias=True, outliers=True)
     case["x"] = (case["x"].float() + 0.5).to(torch.bfloat16)  # off-centre: zero points far from 128
     _check_int8(case, mode, label=f"int8 lowp asym mode={mode} M={M} K={K} N={N} G={G}")
+
+
+@pytest.mark.parametrize("mode", [0, 1, 2, 3])
+@pytest.mark.parametrize(
+    "M,K,N,G",
+    [
+        (1, 1024, 272, 128),
+        (16, 4096, 1024, 128),
+        (32, 2048, 1040, 256),  # two row tiles
+        (25, 1024, 8208, -1),  # per channel; two row-blocks per workgroup
+        (70, 2048, 528, -1),  # the 64-row tiles, ragged in both directions
+        (150, 1024, 272, 128),
+        (300, 4096, 256, 512),  # activation blocks of four tiles
+    ],
+)
+def test_int8_lowp_asymmetric_activations_mfma_kernels(cuda, mode, M, K, N, G):
+    """Asymmetric activations through the kernels that feed the stored codes to the int8 MFMA (groups
+    of at least 128): the column sums of the weights come from MFMAs against rows of ones, the zero
+    points enter in integers.  The general kernel (debug run) supplies the bit-exact block sums."""
+    case = _synthetic().make_int4_case(33, M, K, N, G, bias=True, outliers=True)
+    case["x"] = (case["x"].float() + 0.5).to(torch.bfloat16)  # off-centre: zero points far from 128
+    cols = None if N < 4096 else list(range(0, N, 53)) + [N - 1]
+    _check_int8(case, mode, cols=cols, debug=N < 4096 and M * N * (K // 128) < 1 << 24,
+                label=f"int8 lowp asym mfma mode={mode} M={M} K={K} N={N} G={G}")
+
+
+@pytest.mark.parametrize("mode", [2, 3])
+def test_int8_lowp_asymmetric_activations_split_k(cuda, mode):
+    """Asymmetric activations with the workgroups of a tile sharing K."""
+    case = _synthetic().make_int4_case(34, 100, 4096, 256, 128, bias=True, outliers=True)
+    case["x"] = (case["x"].float() - 0.7).to(torch.bfloat16)
+    _check_int8(case, mode, debug=False, label=f"int8 lowp asym split K mode={mode}")
 
 
 def test_int8_lowp_asymmetric_activations_int8_weights(cuda):
