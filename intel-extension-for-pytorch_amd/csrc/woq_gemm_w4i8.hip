@@ -34,9 +34,11 @@ constexpr int W8_BM = 16 * W8_MT;
 constexpr int W8_BN = W8_WAVES * W8_NTW * kTileN;
 constexpr int W8_XBYTES = W8_BM * kTileK4;                     // one activation buffer (int8)
 constexpr int W8_XLOADS = W8_XBYTES / (W8_WAVES * 1024);       // LDS loads per wave and buffer
-constexpr int W8_WSTAGE = W8_WAVES * W8_NTW * kTileBytes;      // one weight stage
+constexpr int W8_WSTAGE = W8_WAVES * W8_NTW * kTileBytes;      // one weight stage (4-bit codes)
 constexpr int W8_NBUF = 3;    // activation buffers and weight stages: requests run two K steps ahead
 constexpr int W8_LDS_BYTES = W8_NBUF * (W8_XBYTES + W8_WSTAGE + W8_BM * (int)sizeof(float));
+// 8-bit weights: two packed tiles (64 K values each) per row-block and K step
+constexpr int W8_LDS_BYTES_W8 = W8_NBUF * (W8_XBYTES + 2 * W8_WSTAGE + W8_BM * (int)sizeof(float));
 
 struct W4I8Args {
   const uint8_t* xq;       // [M][ldq] int8, groups of eight in nibble-decode order
@@ -126,21 +128,30 @@ __device__ __forceinline__ i4 w8_decode16_nf4(uint32_t d0, uint32_t d1) {
 
 // PER_K: the activation scales change with the K block; they reach the lanes through LDS.
 // ASYM: asymmetric activations (w8_column_sums); the zero points travel like the scales.
-template <bool PER_K, bool ASYM = false>
+// WBITS 8: symmetric 8-bit weights, stored offset-binary: a K step of 128 takes two packed tiles per
+// row-block (one MFMA each), the lane's 16 bytes with the sign bit flipped are the B operand, and the A
+// fragment of tile u is chunk 4 u + c of the 128-byte row (the activations keep their plain byte order).
+// The doubled weight stages leave two workgroups per CU instead of three.
+// NF4: the codes index the int8 NormalFloat4 table (no zero points; scale / 127).
+template <bool PER_K, bool ASYM = false, int WBITS = 4, bool NF4 = false>
 __global__ __launch_bounds__(256, 3) void woq_gemm_w4i8_kernel(const W4I8Args a) {
+  static_assert(WBITS == 4 || (WBITS == 8 && !ASYM), "8-bit weights: symmetric activations only");
+  static_assert(!NF4 || (WBITS == 4 && !ASYM), "NF4 codes: 4 bits wide, symmetric activations only");
+  constexpr int TPS = WBITS / 4;  // packed tiles per row-block and K step
+  constexpr int WSTAGE = TPS * W8_WSTAGE;
   // the activation buffers, then the weight stages, then the activation scales (and, ASYM, zero points)
   // of a step's rows
   extern __shared__ __align__(1024) uint8_t sX[];
   uint8_t* const sW = sX + W8_NBUF * W8_XBYTES;
-  float* const sSA = (float*)(sW + W8_NBUF * W8_WSTAGE);
+  float* const sSA = (float*)(sW + W8_NBUF * WSTAGE);
   int32_t* const sZA = (int32_t*)(sSA + W8_NBUF * W8_BM);
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int r = lane & 15, c = lane >> 4;
-  const int M = (int)a.M, NT = (int)a.NT, KTW = (int)a.KT, KG = (int)a.KG;
-  // K steps of this workgroup: [kt_lo, KT).  gridDim.z > 1 (few tiles, long K): the workgroups of a tile
+  const int M = (int)a.M, NT = (int)a.NT, KTW = (int)a.KT / TPS, KG = (int)a.KG;
+  // K steps (of 128 values) of this workgroup: [kt_lo, KT).  gridDim.z > 1 (few tiles, long K): the workgroups of a tile
   // share K; each writes its fp32 accumulators to scratch and the one that arrives last at the tile's
   // counter adds the partial tiles in z order and stores -- the scheme of the bf16 prefill kernel.
   const int kt_lo = (int)blockIdx.z * a.kts;
@@ -206,7 +217,8 @@ __global__ __launch_bounds__(256, 3) void woq_gemm_w4i8_kernel(const W4I8Args a)
   // A fragment of row tile mt, MFMA j: row 16 mt + r, logical chunk 2 c + j
   uint32_t rd[2];
 #pragma unroll
-  for (int j = 0; j < 2; ++j) rd[j] = (uint32_t)(r * 128 + (((2 * c + j) ^ ((r >> 1) & 7)) << 4));
+  for (int j = 0; j < 2; ++j)
+    rd[j] = (uint32_t)(r * 128 + (((WBITS == 4 ? 2 * c + j : 4 * j + c) ^ ((r >> 1) & 7)) << 4));
 
   // ---- weights ----
   const bool has_z = a.zeros != nullptr;
@@ -216,18 +228,21 @@ __global__ __launch_bounds__(256, 3) void woq_gemm_w4i8_kernel(const W4I8Args a)
 #pragma unroll
   for (int t = 0; t < W8_NTW; ++t) {
     const int nt = nt0 + t < NT ? nt0 + t : NT - 1;
-    wbase[t] = a.qweight + (size_t)nt * KTW * kTileBytes;
+    wbase[t] = a.qweight + (size_t)nt * KTW * (TPS * kTileBytes);
     sbase[t] = a.scales + (size_t)nt * KG * kTileN;
     zbase[t] = has_z ? a.zeros + (size_t)nt * KG * kTileN : (const uint8_t*)sbase[t];
   }
   const uint32_t woff = (uint32_t)lane * 16u;
-  uint8_t* const wmine = sW + wave * (W8_NTW * kTileBytes);
+  uint8_t* const wmine = sW + wave * (W8_NTW * TPS * kTileBytes);
   auto dma_w = [&](int kt, int stage) {
-    const uint32_t wo = (uint32_t)kt * kTileBytes + woff;
+    const uint32_t wo = (uint32_t)kt * (TPS * kTileBytes) + woff;
 #pragma unroll
     for (int t = 0; t < W8_NTW; ++t)
-      __builtin_amdgcn_global_load_lds((w8_global_ptr_t)(wbase[t] + wo),
-                                       (w8_lds_ptr_t)(wmine + stage * W8_WSTAGE + t * kTileBytes), 16, 0, 0);
+#pragma unroll
+      for (int u = 0; u < TPS; ++u)
+        __builtin_amdgcn_global_load_lds((w8_global_ptr_t)(wbase[t] + (uint32_t)(wo + u * kTileBytes)),
+                                         (w8_lds_ptr_t)(wmine + stage * WSTAGE + (t * TPS + u) * kTileBytes), 16,
+                                         0, 0);
   };
   // scale and zero point of this lane's accumulator column n = r... the D tile of an MFMA has column
   // n = lane % 16 in every lane, so one scale per row-block and lane; the B operand's column is the
@@ -242,12 +257,15 @@ __global__ __launch_bounds__(256, 3) void woq_gemm_w4i8_kernel(const W4I8Args a)
       z[t] = *(zbase[t] + qoff);  // raw: any use here would wait for the load inside the request
     }
   };
+  // NF4: the table holds round(127 value), the scale carries the 1 / 127 (applied where a step's scales
+  // become current, after their load has landed)
+  auto current = [&](float v) { return NF4 ? v * (1.0f / 127.0f) : v; };
 
   constexpr int kVmcnt0 = 0x0F70;
   // all but the youngest request of activations and tiles (one K step's worth) have landed
-  constexpr int kVmcntStep = 0x0F70 | (W8_XLOADS + W8_NTW);
+  constexpr int kVmcntStep = 0x0F70 | (W8_XLOADS + W8_NTW * TPS);
 
-  u4 wr[W8_NTW];
+  u4 wr[W8_NTW][TPS];
   float sw[W8_NTW], swn[W8_NTW];
   uint8_t zq[W8_NTW], zqn[W8_NTW];
 
@@ -260,9 +278,13 @@ __global__ __launch_bounds__(256, 3) void woq_gemm_w4i8_kernel(const W4I8Args a)
   dma_w(KT > kt_lo + 1 ? kt_lo + 1 : kt_lo, 1);
   load_q(kt_lo, sw, zq);
   __builtin_amdgcn_s_waitcnt(kVmcnt0);
+#pragma unroll
+  for (int t = 0; t < W8_NTW; ++t) sw[t] = current(sw[t]);
   __syncthreads();
 #pragma unroll
-  for (int t = 0; t < W8_NTW; ++t) wr[t] = *(const u4*)(wmine + t * kTileBytes + woff);
+  for (int t = 0; t < W8_NTW; ++t)
+#pragma unroll
+    for (int u = 0; u < TPS; ++u) wr[t][u] = *(const u4*)(wmine + (t * TPS + u) * kTileBytes + woff);
 
   if (PER_K && tid < W8_BM) sSA[tid] = sa_mine[(int64_t)(kt_lo >> a.q_shift) * a.sa_k_stride];
   if (PER_K && ASYM && tid < W8_BM) sZA[tid] = za_mine[(int64_t)(kt_lo >> a.q_shift) * a.sa_k_stride];
@@ -306,9 +328,19 @@ __global__ __launch_bounds__(256, 3) void woq_gemm_w4i8_kernel(const W4I8Args a)
     int cm[W8_NTW];  // ASYM: column sum of the block's weights, row-block t
 #pragma unroll
     for (int t = 0; t < W8_NTW; ++t) {
-      const uint32_t z4 = (has_z ? (uint32_t)zq[t] : 8u) * 0x01010101u;
-      const i4 bq0 = w8_decode16(wr[t][0], wr[t][1], z4);
-      const i4 bq1 = w8_decode16(wr[t][2], wr[t][3], z4);
+      i4 bq0, bq1;
+      if constexpr (WBITS == 8) {
+        // offset-binary bytes: flipping the sign bit leaves the two's complement weight
+        bq0 = bitcast<i4>(wr[t][0] ^ u4{0x80808080u, 0x80808080u, 0x80808080u, 0x80808080u});
+        bq1 = bitcast<i4>(wr[t][TPS - 1] ^ u4{0x80808080u, 0x80808080u, 0x80808080u, 0x80808080u});
+      } else if constexpr (NF4) {
+        bq0 = w8_decode16_nf4(wr[t][0][0], wr[t][0][1]);
+        bq1 = w8_decode16_nf4(wr[t][0][2], wr[t][0][3]);
+      } else {
+        const uint32_t z4 = (has_z ? (uint32_t)zq[t] : 8u) * 0x01010101u;
+        bq0 = w8_decode16(wr[t][0][0], wr[t][0][1], z4);
+        bq1 = w8_decode16(wr[t][0][2], wr[t][0][3], z4);
+      }
       cm[t] = ASYM ? w8_column_sums(bq0, bq1) : 0;
       __builtin_amdgcn_sched_barrier(0);
       // one MFMA, then (second row-block) the fp32 epilogue of two sums of the first:
@@ -352,8 +384,10 @@ __global__ __launch_bounds__(256, 3) void woq_gemm_w4i8_kernel(const W4I8Args a)
     asm volatile("s_barrier" ::: "memory");
 #pragma unroll
     for (int t = 0; t < W8_NTW; ++t) {
-      wr[t] = *(const u4*)(wmine + b1 * W8_WSTAGE + t * kTileBytes + woff);
-      sw[t] = swn[t];
+#pragma unroll
+      for (int u = 0; u < TPS; ++u)
+        wr[t][u] = *(const u4*)(wmine + b1 * WSTAGE + (t * TPS + u) * kTileBytes + woff);
+      sw[t] = current(swn[t]);
       zq[t] = zqn[t];
     }
     const int b = b0;
@@ -676,8 +710,9 @@ __global__ __launch_bounds__(512, (GSUB * MT > 4 ? 2 : 4)) void woq_decode_w4i8_
 // (four row tiles times four K blocks of activation scales do not fit the registers).
 static int decode_w4i8_max_rows(int64_t group_size) { return group_size == 64 ? 64 : 32; }
 
-// 4-bit integer codes, symmetric activation scales per tensor or per row, K blocks of 128 that are
-// whole weight tiles, and a group size of 128 * 2^s (or one group), so that a K tile has one scale.
+// K blocks of 128 that are whole weight tiles and a group size of 128 * 2^s (or one group), so that a K
+// tile has one scale: 4-bit integer codes (any activation mode), NF4 codes and symmetric 8-bit weights
+// (symmetric activation modes).  Groups of 32 / 64: the decode form only.
 // Up to 32 rows run on the decode form (woq_decode_w4i8_kernel; M = 32: 14 us), from 33 rows on the
 // 64-row tiles of the MFMA GEMM, which with a single row tile still beats the general small-M kernel
 // (4096 -> 14336, per-row scales, M = 48 / 64: 34 / 36 us against 157 / 162 us).
@@ -687,15 +722,18 @@ bool gemm_w4i8_applies(const Int8Args& a, int64_t block_k, int64_t qbk, bool per
   // asymmetric activations: 4-bit integer codes with groups of at least 128
   if (asym && (a.wbits != 4 || a.nf4 || block_k != 128)) return false;
   if (a.wbits == 8) {
-    // symmetric 8-bit weights: the decode form only, one scale per channel or per 128 * 2^s input channels
-    if (a.zeros || a.M > 32 || block_k != 128) return false;
+    // symmetric 8-bit weights, symmetric activations, one scale per channel or per 128 * 2^s input channels
+    if (a.zeros || asym || block_k != 128) return false;
+    // two workgroups per CU: from 512 rows on, with one scale per row, the general tiled kernel is level
+    // or ahead (4096 -> 11008, M = 2048: 249 us against 260 us here; per (row, K block): 268 against 252)
+    if (a.M > 512 && !per_k) return false;
     if (a.group_size > 0 && (a.G % 128 != 0 || ((a.G / 128) & (a.G / 128 - 1)) != 0)) return false;
     if (per_k && (qbk % 128 != 0 || ((qbk / 128) & (qbk / 128 - 1)) != 0)) return false;
     return a.M * a.K < ((int64_t)1 << 31);
   }
   if (a.wbits != 4) return false;
-  // NF4 codes: the decode form only (up to two row tiles)
-  if (a.nf4 && (a.M > 32 || a.zeros)) return false;
+  // NF4 codes: no zero points; above two row tiles the 64 x 128 tiles, which take K blocks of 128 only
+  if (a.nf4 && (a.zeros || (a.M > 32 && block_k != 128))) return false;
   if (block_k == 32 || block_k == 64) {
     // groups of 32 / 64: the decode form only (K blocks inside a tile), activation blocks = groups
     return a.M <= decode_w4i8_max_rows(a.group_size) && a.group_size == block_k && (!per_k || qbk == block_k) &&
@@ -724,6 +762,18 @@ int launch_gemm_w4i8(const Int8Args& a, const uint8_t* xq, int64_t ldq, const fl
   for (int i = 0; i < 4; ++i)
     if (lds_optin[i] != hipSuccess)
       return set_error("woq_gemm_w4i8_kernel: LDS opt-in failed: %s", hipGetErrorString(lds_optin[i]));
+  static const hipError_t lds_optin_w8[4] = {
+      hipFuncSetAttribute(reinterpret_cast<const void*>(&woq_gemm_w4i8_kernel<false, false, 8>),
+                          hipFuncAttributeMaxDynamicSharedMemorySize, W8_LDS_BYTES_W8),
+      hipFuncSetAttribute(reinterpret_cast<const void*>(&woq_gemm_w4i8_kernel<true, false, 8>),
+                          hipFuncAttributeMaxDynamicSharedMemorySize, W8_LDS_BYTES_W8),
+      hipFuncSetAttribute(reinterpret_cast<const void*>(&woq_gemm_w4i8_kernel<false, false, 4, true>),
+                          hipFuncAttributeMaxDynamicSharedMemorySize, W8_LDS_BYTES),
+      hipFuncSetAttribute(reinterpret_cast<const void*>(&woq_gemm_w4i8_kernel<true, false, 4, true>),
+                          hipFuncAttributeMaxDynamicSharedMemorySize, W8_LDS_BYTES)};
+  for (int i = 0; i < 4; ++i)
+    if (lds_optin_w8[i] != hipSuccess)
+      return set_error("woq_gemm_w4i8_kernel: LDS opt-in failed: %s", hipGetErrorString(lds_optin_w8[i]));
   const bool asym = za != nullptr;
   W4I8Args k;
   k.xq = xq; k.ldq = ldq; k.sa = sa; k.sa_m_stride = sa_m_stride; k.sa_k_stride = sa_k_stride;
@@ -738,7 +788,8 @@ int launch_gemm_w4i8(const Int8Args& a, const uint8_t* xq, int64_t ldq, const fl
     while (((int64_t)128 << k.g_shift) < a.G) ++k.g_shift;
   }
   k.ep = Epilogue{a.bias, a.fusion, a.other0, a.other1, a.out, a.out_dtype, a.x_dtype, a.N};
-  k.kts = (int)a.KT;
+  const int64_t ksteps = a.KT / (a.wbits / 4);  // K steps of 128 values
+  k.kts = (int)ksteps;
   k.sk_partial = nullptr;
   k.sk_counters = nullptr;
   if (a.M <= decode_w4i8_max_rows(a.group_size)) {
@@ -843,8 +894,8 @@ int launch_gemm_w4i8(const Int8Args& a, const uint8_t* xq, int64_t ldq, const fl
   if (scratch && scratch->partial && scratch->counters && tiles <= kSplitKCounters) {
     for (int s = 4; s >= 2; s -= 2) {
       const int64_t need = (int64_t)s * tiles * W8_BM * W8_BN * (int64_t)sizeof(float);
-      const int kts = (int)((a.KT + s - 1) / s);
-      if (tiles * s <= 256 && a.KT / s >= 16 && scratch->bytes >= need && (int64_t)(s - 1) * kts < a.KT) {
+      const int kts = (int)((ksteps + s - 1) / s);
+      if (tiles * s <= 256 && ksteps / s >= 16 && scratch->bytes >= need && (int64_t)(s - 1) * kts < ksteps) {
         grid.z = (unsigned)s;
         k.kts = kts;
         k.sk_partial = scratch->partial;
@@ -853,7 +904,15 @@ int launch_gemm_w4i8(const Int8Args& a, const uint8_t* xq, int64_t ldq, const fl
       }
     }
   }
-  if (asym && sa_k_stride != 0)
+  if (a.wbits == 8 && sa_k_stride != 0)
+    woq_gemm_w4i8_kernel<true, false, 8><<<grid, 256, W8_LDS_BYTES_W8, st>>>(k);
+  else if (a.wbits == 8)
+    woq_gemm_w4i8_kernel<false, false, 8><<<grid, 256, W8_LDS_BYTES_W8, st>>>(k);
+  else if (a.nf4 && sa_k_stride != 0)
+    woq_gemm_w4i8_kernel<true, false, 4, true><<<grid, 256, W8_LDS_BYTES, st>>>(k);
+  else if (a.nf4)
+    woq_gemm_w4i8_kernel<false, false, 4, true><<<grid, 256, W8_LDS_BYTES, st>>>(k);
+  else if (asym && sa_k_stride != 0)
     woq_gemm_w4i8_kernel<true, true><<<grid, 256, kLdsAsym, st>>>(k);
   else if (asym)
     woq_gemm_w4i8_kernel<false, true><<<grid, 256, kLdsAsym, st>>>(k);

@@ -694,7 +694,8 @@ def test_nf4_rejections(cuda):
 
 @pytest.mark.parametrize("mode", [6, 7, 2])
 @pytest.mark.parametrize("M,K,N,G", [(1, 1024, 272, 128), (40, 512, 144, 32), (150, 1024, 272, 128), (20, 768, 80, -1),
-                                     (16, 1024, 8208, 64), (9, 512, 144, 32), (4, 1152, 96, -1), (30, 1024, 272, 32), (32, 512, 1040, 128)])
+                                     (16, 1024, 8208, 64), (9, 512, 144, 32), (4, 1152, 96, -1), (30, 1024, 272, 32), (32, 512, 1040, 128),
+                                     (70, 2048, 528, 256), (100, 4096, 256, 128), (48, 1024, 144, 64)])
 def test_nf4_lowp_int8(cuda, mode, M, K, N, G):
     """NF4 codes as int8 table values, scale / 127: int32 block sums bit-exact, fp32 epilogue to the bar."""
     case = _synthetic().make_nf4_case(28, M, K, N, G, bias=(M == 40))
@@ -949,6 +950,28 @@ def test_int8_lowp_int8_weights_decode_kernel(cuda, mode, M, K, N, G):
     case = _synthetic().make_int8_case(23, M, K, N, group_size=G)
     cols = None if N < 4096 else list(range(0, N, 53)) + [N - 1]
     _check_int8(case, mode, cols=cols, debug=N < 4096, label=f"int8 lowp int8 weights decode mode={mode} M={M} K={K} N={N} G={G}")
+
+
+@pytest.mark.parametrize("mode", [4, 5, 6, 7])
+@pytest.mark.parametrize("M,K,N,G", [(33, 1024, 272, -1), (70, 2048, 528, 128), (150, 1152, 96, -1), (300, 1024, 1040, 256)])
+def test_int8_lowp_int8_weights_mfma_tiles(cuda, mode, M, K, N, G):
+    """Symmetric 8-bit weights above 32 rows: the 64 x 128 tiles of the int8 MFMA kernel with two packed
+    tiles per row-block and K step; the general kernel (debug run) supplies the bit-exact block sums."""
+    case = _synthetic().make_int8_case(24, M, K, N, group_size=G)
+    _check_int8(case, mode, label=f"int8 lowp int8 weights tiles mode={mode} M={M} K={K} N={N} G={G}")
+
+
+@pytest.mark.parametrize("mode", [6, 7])
+def test_int8_lowp_int8_weights_split_k(cuda, mode):
+    """8-bit weights with the workgroups of a tile sharing K; repeated launches agree bit for bit."""
+    case = _synthetic().make_int8_case(25, 100, 4096, 256)
+    _check_int8(case, mode, debug=False, label=f"int8 lowp int8 weights split K mode={mode}")
+    ctx = make_context(case, O.LOWP_INT8, mode)
+    x = case["x"].cuda()
+    first = ctx.run(x)
+    runs = [ctx.run(x) for _ in range(50)]
+    torch.cuda.synchronize()
+    assert all(torch.equal(y, first) for y in runs)
 
 
 def test_c3_prefill_int8(cuda):
