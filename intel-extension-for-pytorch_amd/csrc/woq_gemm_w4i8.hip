@@ -133,8 +133,14 @@ __device__ __forceinline__ i4 w8_decode16_nf4(uint32_t d0, uint32_t d1) {
 // fragment of tile u is chunk 4 u + c of the 128-byte row (the activations keep their plain byte order).
 // The doubled weight stages leave two workgroups per CU instead of three.
 // NF4: the codes index the int8 NormalFloat4 table (no zero points; scale / 127).
-template <bool PER_K, bool ASYM = false, int WBITS = 4, bool NF4 = false>
-__global__ __launch_bounds__(256, 3) void woq_gemm_w4i8_kernel(const W4I8Args a) {
+// GSUB > 1: groups of 64 or 32 input channels, i.e. 2 or 4 K blocks per packed tile, each computed with
+// the other blocks' lane columns of the B operand zeroed (see woq_decode_w4i8_kernel) and scaled on its
+// own: GSUB times the MFMAs and the fp32 scalings of a step.
+// (their extra scales and the second set of int32 sums do not fit the registers of three workgroups per
+// CU: two).
+template <bool PER_K, bool ASYM = false, int WBITS = 4, bool NF4 = false, int GSUB = 1>
+__global__ __launch_bounds__(256, (GSUB > 1 ? 2 : 3)) void woq_gemm_w4i8_kernel(const W4I8Args a) {
+  static_assert(GSUB == 1 || (WBITS == 4 && !ASYM && !NF4), "K blocks inside a tile: 4-bit integer codes, symmetric activations");
   static_assert(WBITS == 4 || (WBITS == 8 && !ASYM), "8-bit weights: symmetric activations only");
   static_assert(!NF4 || (WBITS == 4 && !ASYM), "NF4 codes: 4 bits wide, symmetric activations only");
   constexpr int TPS = WBITS / 4;  // packed tiles per row-block and K step
@@ -144,7 +150,7 @@ __global__ __launch_bounds__(256, 3) void woq_gemm_w4i8_kernel(const W4I8Args a)
   extern __shared__ __align__(1024) uint8_t sX[];
   uint8_t* const sW = sX + W8_NBUF * W8_XBYTES;
   float* const sSA = (float*)(sW + W8_NBUF * WSTAGE);
-  int32_t* const sZA = (int32_t*)(sSA + W8_NBUF * W8_BM);
+  int32_t* const sZA = (int32_t*)(sSA + W8_NBUF * GSUB * W8_BM);
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -179,7 +185,10 @@ __global__ __launch_bounds__(256, 3) void woq_gemm_w4i8_kernel(const W4I8Args a)
   }
   const int sa_row = m0 + tid < M ? m0 + tid : M - 1;  // wave 0: the row whose scale this thread fetches
   const float* const sa_mine = a.sa + (int64_t)sa_row * a.sa_m_stride;
-  float sa_next = 0.0f;
+  float sa_next[GSUB];
+  // activation K block of scale g of K step kt
+  auto sa_block = [&](int kt, int g) { return GSUB == 1 ? (int64_t)(kt >> a.q_shift) : (int64_t)kt * GSUB + g; };
+  const int my_block = c / (4 / GSUB);  // K block of the tile this lane column's weights belong to
   // 128 - z_a of the same rows
   i4 zoff[ASYM ? W8_MT : 1];
   if (ASYM && !PER_K) {
@@ -247,14 +256,17 @@ __global__ __launch_bounds__(256, 3) void woq_gemm_w4i8_kernel(const W4I8Args a)
   // scale and zero point of this lane's accumulator column n = r... the D tile of an MFMA has column
   // n = lane % 16 in every lane, so one scale per row-block and lane; the B operand's column is the
   // same n, so the zero point is per lane too.
-  auto load_q = [&](int kt, float (&s)[W8_NTW], uint8_t (&z)[W8_NTW]) {
-    int g = kt >> a.g_shift;
+  auto load_q = [&](int kt, float (&s)[W8_NTW][GSUB], uint8_t (&z)[W8_NTW]) {
+    // first group of the tile (GSUB == 1: the tile's only one, shared by 2^g_shift tiles)
+    int g = GSUB == 1 ? (kt >> a.g_shift) : kt * GSUB;
     g = g < KG ? g : KG - 1;
     const uint32_t qoff = (uint32_t)(g * kTileN + r);
 #pragma unroll
     for (int t = 0; t < W8_NTW; ++t) {
-      s[t] = sbase[t][qoff];
-      z[t] = *(zbase[t] + qoff);  // raw: any use here would wait for the load inside the request
+#pragma unroll
+      for (int gg = 0; gg < GSUB; ++gg) s[t][gg] = sbase[t][qoff + gg * kTileN];
+      // raw: any use here would wait for the load inside the request
+      z[t] = *(zbase[t] + qoff + (GSUB == 1 ? 0 : my_block) * kTileN);
     }
   };
   // NF4: the table holds round(127 value), the scale carries the 1 / 127 (applied where a step's scales
@@ -266,7 +278,7 @@ __global__ __launch_bounds__(256, 3) void woq_gemm_w4i8_kernel(const W4I8Args a)
   constexpr int kVmcntStep = 0x0F70 | (W8_XLOADS + W8_NTW * TPS);
 
   u4 wr[W8_NTW][TPS];
-  float sw[W8_NTW], swn[W8_NTW];
+  float sw[W8_NTW][GSUB], swn[W8_NTW][GSUB];
   uint8_t zq[W8_NTW], zqn[W8_NTW];
 
   // A K step here is short (about 2000 cycles: 32 MFMAs and the fp32 epilogue of 64 sums per lane),
@@ -279,14 +291,19 @@ __global__ __launch_bounds__(256, 3) void woq_gemm_w4i8_kernel(const W4I8Args a)
   load_q(kt_lo, sw, zq);
   __builtin_amdgcn_s_waitcnt(kVmcnt0);
 #pragma unroll
-  for (int t = 0; t < W8_NTW; ++t) sw[t] = current(sw[t]);
+  for (int t = 0; t < W8_NTW; ++t)
+#pragma unroll
+    for (int g = 0; g < GSUB; ++g) sw[t][g] = current(sw[t][g]);
   __syncthreads();
 #pragma unroll
   for (int t = 0; t < W8_NTW; ++t)
 #pragma unroll
     for (int u = 0; u < TPS; ++u) wr[t][u] = *(const u4*)(wmine + (t * TPS + u) * kTileBytes + woff);
 
-  if (PER_K && tid < W8_BM) sSA[tid] = sa_mine[(int64_t)(kt_lo >> a.q_shift) * a.sa_k_stride];
+  if (PER_K && tid < W8_BM) {
+#pragma unroll
+    for (int g = 0; g < GSUB; ++g) sSA[g * W8_BM + tid] = sa_mine[sa_block(kt_lo, g) * a.sa_k_stride];
+  }
   if (PER_K && ASYM && tid < W8_BM) sZA[tid] = za_mine[(int64_t)(kt_lo >> a.q_shift) * a.sa_k_stride];
   __syncthreads();
 
@@ -301,14 +318,17 @@ __global__ __launch_bounds__(256, 3) void woq_gemm_w4i8_kernel(const W4I8Args a)
     // requests, oldest first: parameters of step kt + 1, then activations and tiles of step kt + 2
     // into the buffers of step kt - 1, which every wave left before the last barrier
     load_q(kt1, swn, zqn);
-    if (PER_K && tid < W8_BM) sa_next = sa_mine[(int64_t)(kt1 >> a.q_shift) * a.sa_k_stride];
+    if (PER_K && tid < W8_BM) {
+#pragma unroll
+      for (int g = 0; g < GSUB; ++g) sa_next[g] = sa_mine[sa_block(kt1, g) * a.sa_k_stride];
+    }
     if (PER_K && ASYM && tid < W8_BM) za_next = za_mine[(int64_t)(kt1 >> a.q_shift) * a.sa_k_stride];
     __builtin_amdgcn_sched_barrier(0);  // the parameter loads stay the oldest requests of the step
     load_x(kt2, b2);
     dma_w(kt2, b2);
     __builtin_amdgcn_sched_barrier(0);
 
-    if (PER_K) {
+    if (PER_K && GSUB == 1) {
 #pragma unroll
       for (int mt = 0; mt < W8_MT; ++mt) sa[mt] = *(const f4*)(sSA + b0 * W8_BM + mt * 16 + 4 * c);
       if constexpr (ASYM) {
@@ -324,59 +344,119 @@ __global__ __launch_bounds__(256, 3) void woq_gemm_w4i8_kernel(const W4I8Args a)
 #pragma unroll
       for (int mt = 0; mt < W8_MT; ++mt) xa[j][mt] = *(const i4*)(xs + mt * 2048 + rd[j]);
 
-    i4 qc[W8_NTW][W8_MT];
-    int cm[W8_NTW];  // ASYM: column sum of the block's weights, row-block t
+    if constexpr (GSUB > 1) {
+      // units (row-block t, K block g): the MFMAs of a unit with the fp32 scaling of the unit before
+      // between them, the B operand masked to the lane columns of block g
+      constexpr int NU = W8_NTW * GSUB;
+      i4 qcu[2][W8_MT];
+      i4 bqt0 = i4{0, 0, 0, 0}, bqt1 = i4{0, 0, 0, 0};
+      f4 sap[W8_MT];  // PER_K: activation scales of the previous unit's K block
 #pragma unroll
-    for (int t = 0; t < W8_NTW; ++t) {
-      i4 bq0, bq1;
-      if constexpr (WBITS == 8) {
-        // offset-binary bytes: flipping the sign bit leaves the two's complement weight
-        bq0 = bitcast<i4>(wr[t][0] ^ u4{0x80808080u, 0x80808080u, 0x80808080u, 0x80808080u});
-        bq1 = bitcast<i4>(wr[t][TPS - 1] ^ u4{0x80808080u, 0x80808080u, 0x80808080u, 0x80808080u});
-      } else if constexpr (NF4) {
-        bq0 = w8_decode16_nf4(wr[t][0][0], wr[t][0][1]);
-        bq1 = w8_decode16_nf4(wr[t][0][2], wr[t][0][3]);
-      } else {
-        const uint32_t z4 = (has_z ? (uint32_t)zq[t] : 8u) * 0x01010101u;
-        bq0 = w8_decode16(wr[t][0][0], wr[t][0][1], z4);
-        bq1 = w8_decode16(wr[t][0][2], wr[t][0][3], z4);
-      }
-      cm[t] = ASYM ? w8_column_sums(bq0, bq1) : 0;
-      __builtin_amdgcn_sched_barrier(0);
-      // one MFMA, then (second row-block) the fp32 epilogue of two sums of the first:
-      // C += (float(sum) * s_a[m]) * s_w[n, g]; each pair is fenced so that the order stands
+      for (int u = 0; u < NU; ++u) {
+        const int t = u / GSUB, g = u % GSUB;
+        if (g == 0) {
+          const uint32_t z4 = (has_z ? (uint32_t)zq[t] : 8u) * 0x01010101u;
+          bqt0 = w8_decode16(wr[t][0][0], wr[t][0][1], z4);
+          bqt1 = w8_decode16(wr[t][0][2], wr[t][0][3], z4);
+        }
+        const bool mine = my_block == g;
+        const i4 bm0 = mine ? bqt0 : i4{0, 0, 0, 0};
+        const i4 bm1 = mine ? bqt1 : i4{0, 0, 0, 0};
+        if (PER_K && u > 0) {
 #pragma unroll
-      for (int i = 0; i < 2 * W8_MT; ++i) {
-        const int mt = i % W8_MT;
-        if (i < W8_MT)
-          qc[t][mt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(xa[0][mt], bq0, i4{0, 0, 0, 0}, 0, 0, 0);
-        else
-          qc[t][mt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(xa[1][mt], bq1, qc[t][mt], 0, 0, 0);
-        if (t > 0) {
-#pragma unroll
-          for (int u = 0; u < 2; ++u) {
-            const int q = 2 * i + u, pm = q / 4, pe = q % 4;
-            const int qv = ASYM ? qc[t - 1][pm][pe] + cm[t - 1] * zoff[ASYM ? pm : 0][pe] : qc[t - 1][pm][pe];
-            acc[pm][t - 1][pe] = w8_accumulate<PER_K>(qv, sa[pm][pe], sw[t - 1], acc[pm][t - 1][pe]);
-          }
+          for (int mt = 0; mt < W8_MT; ++mt)
+            sap[mt] = *(const f4*)(sSA + (b0 * GSUB + (u - 1) % GSUB) * W8_BM + mt * 16 + 4 * c);
         }
         __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int i = 0; i < 2 * W8_MT; ++i) {
+          const int mt = i % W8_MT;
+          if (i < W8_MT)
+            qcu[u & 1][mt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(xa[0][mt], bm0, i4{0, 0, 0, 0}, 0, 0, 0);
+          else
+            qcu[u & 1][mt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(xa[1][mt], bm1, qcu[u & 1][mt], 0, 0, 0);
+          if (u > 0) {
+            const int tp = (u - 1) / GSUB, gp = (u - 1) % GSUB;
+#pragma unroll
+            for (int w = 0; w < 2; ++w) {
+              const int q = 2 * i + w, pm = q / 4, pe = q % 4;
+              acc[pm][tp][pe] = w8_accumulate<PER_K>(qcu[(u - 1) & 1][pm][pe], PER_K ? sap[pm][pe] : 0.0f, sw[tp][gp],
+                                                     acc[pm][tp][pe]);
+            }
+          }
+          __builtin_amdgcn_sched_barrier(0);
+        }
       }
+      if (PER_K) {
+#pragma unroll
+        for (int mt = 0; mt < W8_MT; ++mt)
+          sap[mt] = *(const f4*)(sSA + (b0 * GSUB + GSUB - 1) * W8_BM + mt * 16 + 4 * c);
+      }
+#pragma unroll
+      for (int mt = 0; mt < W8_MT; ++mt)
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          acc[mt][W8_NTW - 1][e] = w8_accumulate<PER_K>(qcu[(NU - 1) & 1][mt][e], PER_K ? sap[mt][e] : 0.0f,
+                                                        sw[W8_NTW - 1][GSUB - 1], acc[mt][W8_NTW - 1][e]);
+    } else {
+      i4 qc[W8_NTW][W8_MT];
+      int cm[W8_NTW];  // ASYM: column sum of the block's weights, row-block t
+  #pragma unroll
+      for (int t = 0; t < W8_NTW; ++t) {
+        i4 bq0, bq1;
+        if constexpr (WBITS == 8) {
+          // offset-binary bytes: flipping the sign bit leaves the two's complement weight
+          bq0 = bitcast<i4>(wr[t][0] ^ u4{0x80808080u, 0x80808080u, 0x80808080u, 0x80808080u});
+          bq1 = bitcast<i4>(wr[t][TPS - 1] ^ u4{0x80808080u, 0x80808080u, 0x80808080u, 0x80808080u});
+        } else if constexpr (NF4) {
+          bq0 = w8_decode16_nf4(wr[t][0][0], wr[t][0][1]);
+          bq1 = w8_decode16_nf4(wr[t][0][2], wr[t][0][3]);
+        } else {
+          const uint32_t z4 = (has_z ? (uint32_t)zq[t] : 8u) * 0x01010101u;
+          bq0 = w8_decode16(wr[t][0][0], wr[t][0][1], z4);
+          bq1 = w8_decode16(wr[t][0][2], wr[t][0][3], z4);
+        }
+        cm[t] = ASYM ? w8_column_sums(bq0, bq1) : 0;
+        __builtin_amdgcn_sched_barrier(0);
+        // one MFMA, then (second row-block) the fp32 epilogue of two sums of the first:
+        // C += (float(sum) * s_a[m]) * s_w[n, g]; each pair is fenced so that the order stands
+  #pragma unroll
+        for (int i = 0; i < 2 * W8_MT; ++i) {
+          const int mt = i % W8_MT;
+          if (i < W8_MT)
+            qc[t][mt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(xa[0][mt], bq0, i4{0, 0, 0, 0}, 0, 0, 0);
+          else
+            qc[t][mt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(xa[1][mt], bq1, qc[t][mt], 0, 0, 0);
+          if (t > 0) {
+  #pragma unroll
+            for (int u = 0; u < 2; ++u) {
+              const int q = 2 * i + u, pm = q / 4, pe = q % 4;
+              const int qv = ASYM ? qc[t - 1][pm][pe] + cm[t - 1] * zoff[ASYM ? pm : 0][pe] : qc[t - 1][pm][pe];
+              acc[pm][t - 1][pe] = w8_accumulate<PER_K>(qv, sa[pm][pe], sw[t - 1][0], acc[pm][t - 1][pe]);
+            }
+          }
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      }
+  #pragma unroll
+      for (int mt = 0; mt < W8_MT; ++mt)
+  #pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const int qv = ASYM ? qc[W8_NTW - 1][mt][e] + cm[W8_NTW - 1] * zoff[ASYM ? mt : 0][e] : qc[W8_NTW - 1][mt][e];
+          acc[mt][W8_NTW - 1][e] = w8_accumulate<PER_K>(qv, sa[mt][e], sw[W8_NTW - 1][0], acc[mt][W8_NTW - 1][e]);
+        }
+
     }
-#pragma unroll
-    for (int mt = 0; mt < W8_MT; ++mt)
-#pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        const int qv = ASYM ? qc[W8_NTW - 1][mt][e] + cm[W8_NTW - 1] * zoff[ASYM ? mt : 0][e] : qc[W8_NTW - 1][mt][e];
-        acc[mt][W8_NTW - 1][e] = w8_accumulate<PER_K>(qv, sa[mt][e], sw[W8_NTW - 1], acc[mt][W8_NTW - 1][e]);
-      }
 
     // Next step: its activations and tiles (requested a step ago) must have landed -- every wave
     // waits for its own requests, the barrier covers the others' -- and every wave must be done
     // reading this step's buffer.  Written as an instruction: before the barrier builtin the
     // compiler waits for every outstanding load, the requests for step kt + 2 included.
     if (PER_K) {
-      if (tid < W8_BM) sSA[b1 * W8_BM + tid] = sa_next;
+      if (tid < W8_BM) {
+#pragma unroll
+        for (int g = 0; g < GSUB; ++g) sSA[(b1 * GSUB + g) * W8_BM + tid] = sa_next[g];
+      }
       if (ASYM && tid < W8_BM) sZA[b1 * W8_BM + tid] = za_next;
       __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): the LDS write is done before the barrier
     }
@@ -387,7 +467,8 @@ __global__ __launch_bounds__(256, 3) void woq_gemm_w4i8_kernel(const W4I8Args a)
 #pragma unroll
       for (int u = 0; u < TPS; ++u)
         wr[t][u] = *(const u4*)(wmine + b1 * WSTAGE + (t * TPS + u) * kTileBytes + woff);
-      sw[t] = current(swn[t]);
+#pragma unroll
+      for (int g = 0; g < GSUB; ++g) sw[t][g] = current(swn[t][g]);
       zq[t] = zqn[t];
     }
     const int b = b0;
@@ -735,9 +816,13 @@ bool gemm_w4i8_applies(const Int8Args& a, int64_t block_k, int64_t qbk, bool per
   // NF4 codes: no zero points; above two row tiles the 64 x 128 tiles, which take K blocks of 128 only
   if (a.nf4 && (a.zeros || (a.M > 32 && block_k != 128))) return false;
   if (block_k == 32 || block_k == 64) {
-    // groups of 32 / 64: the decode form only (K blocks inside a tile), activation blocks = groups
-    return a.M <= decode_w4i8_max_rows(a.group_size) && a.group_size == block_k && (!per_k || qbk == block_k) &&
-           a.M * a.K < ((int64_t)1 << 31);
+    // groups of 32 / 64 (K blocks inside a tile), activation blocks = groups; above the rows of the decode
+    // form: the 64 x 128 tiles, for 4-bit integer codes and symmetric activations
+    // (not groups of 32 with per-(row, K block) scales: four sets of activation scales on top of the
+    // second set of sums spill, and a reload waits behind the requests of two steps -- 4096 -> 14336,
+    // M = 128: 257 us against 62 us with per-row scales; the general kernel keeps that case)
+    if (a.M > decode_w4i8_max_rows(a.group_size) && (a.nf4 || asym || (block_k == 32 && per_k))) return false;
+    return a.group_size == block_k && (!per_k || qbk == block_k) && a.M * a.K < ((int64_t)1 << 31);
   }
   if (block_k != 128) return false;
   if (a.group_size > 0 && (a.G % 128 != 0 || ((a.G / 128) & (a.G / 128 - 1)) != 0)) return false;
@@ -774,6 +859,16 @@ int launch_gemm_w4i8(const Int8Args& a, const uint8_t* xq, int64_t ldq, const fl
   for (int i = 0; i < 4; ++i)
     if (lds_optin_w8[i] != hipSuccess)
       return set_error("woq_gemm_w4i8_kernel: LDS opt-in failed: %s", hipGetErrorString(lds_optin_w8[i]));
+  static const hipError_t lds_optin_gsub[3] = {
+      hipFuncSetAttribute(reinterpret_cast<const void*>(&woq_gemm_w4i8_kernel<false, false, 4, false, 2>),
+                          hipFuncAttributeMaxDynamicSharedMemorySize, W8_LDS_BYTES + W8_NBUF * W8_BM * 4),
+      hipFuncSetAttribute(reinterpret_cast<const void*>(&woq_gemm_w4i8_kernel<true, false, 4, false, 2>),
+                          hipFuncAttributeMaxDynamicSharedMemorySize, W8_LDS_BYTES + W8_NBUF * W8_BM * 4),
+      hipFuncSetAttribute(reinterpret_cast<const void*>(&woq_gemm_w4i8_kernel<false, false, 4, false, 4>),
+                          hipFuncAttributeMaxDynamicSharedMemorySize, W8_LDS_BYTES + W8_NBUF * 3 * W8_BM * 4)};
+  for (int i = 0; i < 3; ++i)
+    if (lds_optin_gsub[i] != hipSuccess)
+      return set_error("woq_gemm_w4i8_kernel: LDS opt-in failed: %s", hipGetErrorString(lds_optin_gsub[i]));
   const bool asym = za != nullptr;
   W4I8Args k;
   k.xq = xq; k.ldq = ldq; k.sa = sa; k.sa_m_stride = sa_m_stride; k.sa_k_stride = sa_k_stride;
@@ -904,7 +999,15 @@ int launch_gemm_w4i8(const Int8Args& a, const uint8_t* xq, int64_t ldq, const fl
       }
     }
   }
-  if (a.wbits == 8 && sa_k_stride != 0)
+  if (a.group_size == 64 && sa_k_stride != 0)
+    woq_gemm_w4i8_kernel<true, false, 4, false, 2><<<grid, 256, W8_LDS_BYTES + W8_NBUF * W8_BM * 4, st>>>(k);
+  else if (a.group_size == 64)
+    woq_gemm_w4i8_kernel<false, false, 4, false, 2><<<grid, 256, W8_LDS_BYTES + W8_NBUF * W8_BM * 4, st>>>(k);
+  else if (a.group_size == 32 && sa_k_stride != 0)
+    return set_error("woq_gemm_w4i8_kernel: groups of 32 with per-(row, K block) scales are not taken here");
+  else if (a.group_size == 32)
+    woq_gemm_w4i8_kernel<false, false, 4, false, 4><<<grid, 256, W8_LDS_BYTES + W8_NBUF * 3 * W8_BM * 4, st>>>(k);
+  else if (a.wbits == 8 && sa_k_stride != 0)
     woq_gemm_w4i8_kernel<true, false, 8><<<grid, 256, W8_LDS_BYTES_W8, st>>>(k);
   else if (a.wbits == 8)
     woq_gemm_w4i8_kernel<false, false, 8><<<grid, 256, W8_LDS_BYTES_W8, st>>>(k);

@@ -918,6 +918,18 @@ def test_int8_lowp_decode_kernel(cuda, mode, M, K, N, G):
     _check_int8(case, mode, cols=cols, debug=N < 4096, label=f"int8 lowp decode mode={mode} M={M} K={K} N={N} G={G}")
 
 
+@pytest.mark.parametrize("mode", [4, 5, 6, 7])
+@pytest.mark.parametrize("M,K,N,G", [(33, 1024, 272, 32), (65, 1024, 272, 64), (150, 2048, 528, 32), (300, 1024, 1040, 64),
+                                     (100, 4096, 256, 32)])
+def test_int8_lowp_small_groups_mfma_tiles(cuda, mode, M, K, N, G):
+    """Groups of 32 / 64 above the rows of the decode form: the 64 x 128 tiles with the K blocks of a
+    packed tile computed one by one (B operand masked to the block's lane columns); the last shape shares
+    K between workgroups.  The general kernel (debug run) supplies the bit-exact block sums."""
+    case = _synthetic().make_int4_case(35, M, K, N, G, bias=True, outliers=True)
+    _check_int8(case, mode, debug=M * N * (K // G) < 1 << 24,
+                label=f"int8 lowp small groups tiles mode={mode} M={M} K={K} N={N} G={G}")
+
+
 @pytest.mark.parametrize("mode", [6, 7])
 @pytest.mark.parametrize("M,K,N,G", [(100, 4096, 256, 128), (200, 8192, 144, 256), (65, 14336, 512, -1)])
 def test_int8_lowp_prefill_split_k(cuda, mode, M, K, N, G):
