@@ -247,12 +247,16 @@ def config_sweep(torch, lib, lib_mod, ops_mod, synthetic, dev, stream, steps):
     rows.append({"config": "C4 decoder block, summed WOQ-linear time per token step", "us": round(block, 2)})
     # Beyond the named configurations: what the same layers cost in the neighbouring settings a user of
     # the reference may run (single-stream decode of a group-32 model, lowp_mode INT8 decode with
-    # per-row and per-(row, K block) activation scales, INT8 weights at prefill size).
+    # per-row and per-(row, K block) activation scales, INT8 weights at prefill size, asymmetric
+    # activations, a group-64 model and INT8 weights at a serving batch under lowp_mode INT8).
     run("extra: int4 g32 M=1 4096->14336 (lowp BF16)", synthetic.make_int4_case(5, 1, 4096, 14336, 32))
     run("extra: int4 g128 M=1 4096->14336 lowp INT8 per-row", synthetic.make_int4_case(5, 1, 4096, 14336, 128), 3, 6)
     run("extra: int4 g128 M=16 4096->14336 lowp INT8 per-row-and-K-block", synthetic.make_int4_case(5, 16, 4096, 14336, 128), 3, 7)
     run("extra: int4 g32 M=1 4096->14336 lowp INT8 per-row-and-K-block", synthetic.make_int4_case(5, 1, 4096, 14336, 32), 3, 7)
     run("extra: int8 per-channel M=2048 4096->11008 +bias (lowp BF16)", synthetic.make_int8_case(5, 2048, 4096, 11008))
+    run("extra: int4 g128 M=16 4096->14336 lowp INT8 asymmetric per-row", synthetic.make_int4_case(5, 16, 4096, 14336, 128), 3, 2)
+    run("extra: int4 g64 M=128 4096->14336 lowp INT8 per-row", synthetic.make_int4_case(5, 128, 4096, 14336, 64), 3, 6)
+    run("extra: int8 per-channel M=128 4096->11008 +bias lowp INT8 per-row", synthetic.make_int8_case(5, 128, 4096, 11008), 3, 6)
     return rows
 
 
