@@ -212,8 +212,17 @@ int woq_hip_linear(const woq_hip_linear_params* p) {
     regime = kRegimeF16;
   } else if ((lowp == WOQ_HIP_LOWP_NONE && p->x_dtype == WOQ_HIP_ACT_BF16) || lowp == WOQ_HIP_LOWP_BF16) {
     regime = kRegimeBF16;
+  } else if (lowp == WOQ_HIP_LOWP_NONE && p->x_dtype == WOQ_HIP_ACT_FP32) {
+    // fp32 compute (csrc/cpu/aten/kernels/WoqLinearKrnl.cpp:142-158)
+    if (p->force_kernel != 0) return set_error("woq_linear: fp32 compute has one kernel; force_kernel must be 0");
+    Fp32Args a;
+    a.x = (const float*)p->x; a.M = p->M; a.K = p->K; a.N = p->N; a.NT = NT; a.KT = KT;
+    a.qweight = (const uint8_t*)p->qweight; a.scales = p->scales_f32; a.zeros = p->zeros_u8;
+    a.G = G; a.KG = KG; a.bias = p->bias; a.fusion = p->fusion;
+    a.other0 = p->others[0]; a.other1 = p->others[1]; a.out = p->out; a.nf4 = nf4 ? 1 : 0;
+    return launch_fp32(a, wbits, st);
   } else {
-    return set_error("woq_linear: fp32 compute (lowp_mode NONE with fp32 activations) is not supported");
+    return set_error("woq_linear: lowp_mode %d does not take x_dtype %d", lowp, p->x_dtype);
   }
 
   FpArgs f;

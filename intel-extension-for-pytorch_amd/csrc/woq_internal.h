@@ -85,6 +85,24 @@ struct DecodeArgs {
 bool decode_kernel_applies(const FpArgs& f, int wbits, int regime, const uint32_t* sz);
 int launch_decode(const FpArgs& f, const uint32_t* sz, hipStream_t st);
 
+// fp32 compute (woq_fp32.hip): lowp_mode NONE with fp32 activations; fp32 scales, one-byte zero
+// points, fp32 output.
+struct Fp32Args {
+  const float* x;
+  int64_t M, K, N, NT, KT;
+  const uint8_t* qweight;
+  const float* scales;   // [NT][KG][16]
+  const uint8_t* zeros;  // [NT][KG][16] or null (symmetric)
+  int64_t G, KG;
+  const float* bias;
+  int fusion;
+  const void* other0;
+  const void* other1;
+  void* out;
+  int nf4;
+};
+int launch_fp32(const Fp32Args& f, int wbits, hipStream_t st);
+
 // Decode kernel with per-weight dequantization (woq_decode_dq.hip): 4- or 8-bit weights, M <= 64.
 // ntw: weight row-blocks per workgroup (1, 2 or 4), 0 = automatic;
 // splits: workgroups that share the K tiles of a row-block set (1, 2 or 4; more than 1 needs the

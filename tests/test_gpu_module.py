@@ -67,6 +67,40 @@ def test_prepare_convert_matches_dequantized_matmul(cuda, weight_dtype, group_si
         assert torch.equal(ctx.get_zero_points().cpu(), z.float())
 
 
+@pytest.mark.parametrize("weight_dtype,group_size", [(None, -1), ("INT4", 128), ("NF4", 64)])
+@pytest.mark.parametrize("M", [1, 70])
+def test_default_qconfig_on_an_fp32_model_computes_in_fp32(cuda, weight_dtype, group_size, M):
+    """get_weight_only_quant_qconfig_mapping() defaults to INT8 weights and lowp_mode NONE
+    (quantization/_qconfig.py:188-196); on an fp32 model that is fp32 compute."""
+    ipex = _ipex()
+    q = ipex.quantization
+    torch.manual_seed(1)
+    K, N = 384, 100
+    lin = torch.nn.Linear(K, N, bias=True)
+    model = torch.nn.Sequential(lin).eval()
+    if weight_dtype is None:
+        qmap = q.get_weight_only_quant_qconfig_mapping()
+        dt = q.WoqWeightDtype.INT8
+    else:
+        dt = getattr(q.WoqWeightDtype, weight_dtype)
+        qmap = q.get_weight_only_quant_qconfig_mapping(weight_dtype=dt, group_size=group_size)
+    assert qmap.global_qconfig.lowp_mode == q.WoqLowpMode.NONE
+    w_float = lin.weight.detach().clone()
+    qmodel = q.convert(q.prepare(copy.deepcopy(model).to(cuda), qmap, inplace=True), inplace=True)
+    x = torch.randn(2, M, K)
+    y = qmodel(x.to(cuda))
+    assert y.dtype == torch.float32 and tuple(y.shape) == (2, M, N)
+    sym = qmap.global_qconfig.weight_qscheme == q.WoqWeightQScheme.SYMMETRIC
+    if group_size == -1:
+        qw, s, z = q.quantize_per_channel(w_float, dt, None, None, sym)
+        dq = q.dequantize_per_channel(qw, s, z, dt, [N, K])
+    else:
+        qw, s, z = q.quantize_per_block(w_float, dt, group_size, None, None, sym)
+        dq = q.dequantize_per_block(qw, s, z, dt, group_size, [N, K])
+    ref = (x.double() @ dq.double().t() + lin.bias.double()).float()
+    assert torch.allclose(y.cpu(), ref, atol=1e-5, rtol=1e-5), float((y.cpu() - ref).abs().max())
+
+
 def test_all_zero_bias_is_dropped_and_weight_emptied(cuda):
     ipex = _ipex()
     q = ipex.quantization

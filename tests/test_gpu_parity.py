@@ -1240,3 +1240,67 @@ def test_activation_dtypes_shapes_and_layouts(cuda, idx, act, lowp, lead, K, N, 
     else:
         _, want = O.woq_linear_ref(xs, act, c["qw"], N, K, O._round_to(c["scales"], cd), c["zps"], c["bias"], 2, G, cd)
     assert rel_l2(y, want) <= REL_L2_OUT, (idx, act, lowp, lead, K, N, G, layout, rel_l2(y, want))
+
+
+# ---- fp32 compute: lowp_mode NONE with fp32 activations (WoqLinearKrnl.cpp:142-158) -----------
+@pytest.mark.parametrize(
+    "kind,M,K,N,G,bias",
+    [
+        ("int4", 1, 4096, 512, 128, False),
+        ("int4", 130, 1000, 272, -1, True),   # ragged K, N and M; K % 4 == 0
+        ("int4", 7, 250, 48, -1, False),      # K % 4 != 0: element-wise activation loads
+        ("int4", 33, 640, 100, 32, True),
+        ("int4sym", 5, 512, 80, 64, False),
+        ("int8", 33, 512, 100, -1, True),
+        ("int8", 3, 320, 272, 64, False),
+        ("nf4", 40, 512, 80, 64, True),
+    ],
+)
+def test_fp32_compute(cuda, kind, M, K, N, G, bias):
+    """fp32 scales kept unrounded, w = (q - z) * s in fp32, fp32 products and sums, fp32 output:
+    against the fallback oracle in fp32 (float64 sums), to fp32 summation accuracy."""
+    syn = _synthetic()
+    if kind == "int8":
+        case = syn.make_int8_case(410, M, K, N, bias=bias, group_size=G)
+    elif kind == "nf4":
+        case = syn.make_nf4_case(411, M, K, N, G, bias=bias, scale_dtype=torch.float32)
+    else:
+        case = syn.make_int4_case(412, M, K, N, G, bias=bias, scale_dtype=torch.float32)
+        if kind == "int4sym":
+            case["zeros"] = None
+    gen = torch.Generator().manual_seed(413)
+    x = torch.randn(M, K, generator=gen)  # genuine fp32 values, not bf16-representable ones
+    ctx = make_context(case, O.LOWP_NONE)
+    y = torch.ops.torch_ipex.ipex_woq_linear(x.cuda(), ctx.get_data_handle())
+    assert y.dtype == torch.float32 and tuple(y.shape) == (M, N)
+    c = case_np(case)
+    assert O.select_compute(O.LOWP_NONE, "fp32", M) == "fp32"
+    acc, want = O.woq_linear_ref(x.numpy(), "fp32", c["qw"], N, K, c["scales"], c["zps"], c["bias"],
+                                 case["weight_dtype"], G, "fp32")
+    got = y.cpu().numpy()
+    assert rel_l2(got, acc) <= 1e-5, (kind, M, K, N, G, rel_l2(got, acc))
+    assert max_abs(got, acc) <= 2e-4 * max(1.0, float(np.abs(acc).max())), (kind, M, K, N, G, max_abs(got, acc))
+    # lowp_mode INT8 on fp32 activations runs unquantized in fp32 as well
+    # (WoqInt8GemmAPerMKrnl.cpp:143-169): same kernel, same bits
+    if kind in ("int4sym", "int8", "nf4"):
+        ctx8 = make_context(case, O.LOWP_INT8, 6)
+        assert torch.equal(ctx8.run(x.cuda()), y)
+
+
+def test_fp32_compute_post_ops(cuda):
+    from ipex_amd import _lib
+    import torch.nn.functional as F
+
+    case = _synthetic().make_int4_case(420, 9, 256, 64, 128, bias=True, scale_dtype=torch.float32)
+    gen = torch.Generator().manual_seed(421)
+    x = torch.randn(9, 256, generator=gen).cuda()
+    o1, o2 = torch.randn(9, 64, generator=gen).cuda(), torch.randn(9, 64, generator=gen).cuda()
+    ctx = make_context(case, O.LOWP_NONE)
+    base = ctx.run(x)
+    assert base.dtype == torch.float32
+    assert torch.allclose(ctx.run(x, fusion=_lib.FUSE_SILU), F.silu(base), atol=1e-4, rtol=1e-4)
+    assert torch.allclose(ctx.run(x, fusion=_lib.FUSE_GELU_ERF), F.gelu(base), atol=1e-4, rtol=1e-4)
+    assert torch.equal(ctx.run(x, fusion=_lib.FUSE_RELU), F.relu(base))
+    assert torch.equal(ctx.run(x, fusion=_lib.FUSE_ADD, others=(o1,)), base + o1)
+    assert torch.equal(ctx.run(x, fusion=_lib.FUSE_MUL, others=(o1,)), base * o1)
+    assert torch.equal(ctx.run(x, fusion=_lib.FUSE_ADD_ADD, others=(o1, o2)), base + o1 + o2)
