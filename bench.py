@@ -23,6 +23,7 @@ for _p in (ROOT, os.path.join(ROOT, "intel-extension-for-pytorch_amd")):
 
 HBM_PEAK_GBS = 8000.0       # MI355X HBM3E, published
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
+MFMA_FP32_PEAK_TFLOPS = 157.3   # MI355X dense fp32 matrix, published
 
 
 # HBM bytes per launch of the dominant kernel, from two rocprofv3 --pmc runs of `bench.py --traffic-probe`
@@ -45,7 +46,7 @@ def build_params(lib_mod, x, ctx, out, lowp_mode, act_quant_mode=-1, workspace=N
     p = lib_mod.LinearParams()
     p.struct_size = ctypes.sizeof(lib_mod.LinearParams)
     p.x = x.data_ptr()
-    p.x_dtype = lib_mod.ACT_BF16
+    p.x_dtype = lib_mod.ACT_FP32 if x.element_size() == 4 else lib_mod.ACT_BF16
     p.M, p.K, p.N = x.shape[0], ctx.weight_shape_[1], ctx.weight_shape_[0]
     p.qweight = ctx.at_weight_.data_ptr()
     p.weight_dtype = ctx.weight_dtype_
@@ -60,7 +61,7 @@ def build_params(lib_mod, x, ctx, out, lowp_mode, act_quant_mode=-1, workspace=N
     p.act_quant_mode = act_quant_mode
     p.fusion = 0
     p.out = out.data_ptr()
-    p.out_dtype = lib_mod.ACT_BF16
+    p.out_dtype = lib_mod.ACT_FP32 if out.element_size() == 4 else lib_mod.ACT_BF16
     if workspace is None and lowp_mode != 3:
         # what the op layer passes for small batches: scratch that lets the decode kernel split K
         # across workgroups, and the zeroed counters that go with it.  One block for all launches of
@@ -179,7 +180,9 @@ def _rotating_params(torch, lib_mod, ops_mod, case, lowp_mode, dev, stream, min_
                          device=dev)
     copies = int(min_bytes // ctx0.at_weight_.numel()) + 1
     x = case["x"].to(dev)
-    out = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
+    if case.get("fp32_activations"):  # fp32 compute: lowp_mode NONE on fp32 rows, fp32 output
+        x = x.float()
+    out = torch.empty(M, N, dtype=x.dtype, device=dev)
 
     class Copy:
         pass
@@ -226,7 +229,10 @@ def config_sweep(torch, lib, lib_mod, ops_mod, synthetic, dev, stream, steps):
                "us_p10_p90": [round(groups[1], 2), round(groups[7], 2)]}
         if M >= 256:  # MFMA-bound: a rate in flops, not in bytes
             row["tflops"] = round(2.0 * M * K * N / us / 1e6, 1)
-            row["frac_of_bf16_mfma_peak"] = round(2.0 * M * K * N / us / 1e6 / MFMA_BF16_PEAK_TFLOPS, 3)
+            if case.get("fp32_activations"):
+                row["frac_of_fp32_mfma_peak"] = round(2.0 * M * K * N / us / 1e6 / MFMA_FP32_PEAK_TFLOPS, 3)
+            else:
+                row["frac_of_bf16_mfma_peak"] = round(2.0 * M * K * N / us / 1e6 / MFMA_BF16_PEAK_TFLOPS, 3)
         else:
             row["GB_per_s"] = round(nbytes / us / 1e3, 1)
             row["frac_of_hbm_peak"] = round(nbytes / us / 1e3 / HBM_PEAK_GBS, 3)
@@ -257,6 +263,10 @@ def config_sweep(torch, lib, lib_mod, ops_mod, synthetic, dev, stream, steps):
     run("extra: int4 g128 M=16 4096->14336 lowp INT8 asymmetric per-row", synthetic.make_int4_case(5, 16, 4096, 14336, 128), 3, 2)
     run("extra: int4 g64 M=128 4096->14336 lowp INT8 per-row", synthetic.make_int4_case(5, 128, 4096, 14336, 64), 3, 6)
     run("extra: int8 per-channel M=128 4096->11008 +bias lowp INT8 per-row", synthetic.make_int8_case(5, 128, 4096, 11008), 3, 6)
+    # fp32 compute: the reference's default qconfig (INT8 weights, lowp_mode NONE) on an fp32 model
+    case = synthetic.make_int8_case(5, 2048, 4096, 11008)
+    case["fp32_activations"] = True
+    run("extra: int8 per-channel M=2048 4096->11008 +bias, fp32 activations, lowp NONE (fp32 MFMA)", case, 0)
     return rows
 
 
