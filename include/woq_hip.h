@@ -100,6 +100,12 @@ const char* woq_hip_last_error(void);
 /* ABI version; bumped whenever a struct or a layout below changes. */
 int woq_hip_abi_version(void);
 
+/* Name of the kernel the calling thread enqueued last through any entry point below ("" before the
+ * first launch), e.g. "woq_gemm_w4i8_kernel": lets a test or a profile script state which kernel served
+ * a call.  No counterpart in the reference, whose kernel choice is visible only in its dispatch code
+ * (csrc/cpu/aten/kernels/WoqLinearKrnl.cpp:56-161). */
+const char* woq_hip_last_kernel(void);
+
 /* Padded extents of the packed layout: N up to a multiple of 16, K up to a multiple of
  * the tile K extent.  packed bytes = Np/16 * Kp/tile_k * 1024. */
 int64_t woq_hip_padded_n(int64_t N);

@@ -1,6 +1,8 @@
 """Builds libwoq_hip.so (gfx950) from the .hip sources in this directory.
 
-Usage: python build.py [--jobs N]
+Usage: python build.py [--jobs N] [--incremental]
+--incremental recompiles only the sources that are newer than their object file (or older than a
+header); the default compiles everything.
 The library is written to ../lib/libwoq_hip.so, in-tree, so that a copy of the
 repository carries it to a machine that has no compiler cache.
 """
@@ -29,8 +31,19 @@ def lib_path():
     return os.path.join(LIB_DIR, "libwoq_hip.so")
 
 
-def _compile(src):
+def _stale(src, obj):
+    if not os.path.exists(obj):
+        return True
+    t = os.path.getmtime(obj)
+    deps = [os.path.join(HERE, src)] + [os.path.join(HERE, h) for h in os.listdir(HERE) if h.endswith(".h")]
+    deps.append(os.path.join(os.path.dirname(os.path.dirname(HERE)), "include", "woq_hip.h"))
+    return any(os.path.getmtime(d) > t for d in deps)
+
+
+def _compile(src, incremental=False):
     obj = os.path.join(OBJ_DIR, src.replace(".hip", ".o"))
+    if incremental and not _stale(src, obj):
+        return obj
     cmd = [HIPCC, *FLAGS, "-c", os.path.join(HERE, src), "-o", obj]
     res = subprocess.run(cmd, capture_output=True, text=True)
     err = "\n".join(l for l in res.stderr.splitlines() if "packed-fp32-ops" not in l)
@@ -41,11 +54,11 @@ def _compile(src):
     return obj
 
 
-def build(jobs=4, verbose=True):
+def build(jobs=4, verbose=True, incremental=False):
     os.makedirs(LIB_DIR, exist_ok=True)
     os.makedirs(OBJ_DIR, exist_ok=True)
     with ThreadPoolExecutor(max_workers=jobs) as ex:
-        objs = list(ex.map(_compile, SOURCES))
+        objs = list(ex.map(lambda src: _compile(src, incremental), SOURCES))
     cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", lib_path(), *objs]
     res = subprocess.run(cmd, capture_output=True, text=True)
     if res.returncode != 0:
@@ -58,4 +71,6 @@ def build(jobs=4, verbose=True):
 if __name__ == "__main__":
     ap = argparse.ArgumentParser()
     ap.add_argument("--jobs", type=int, default=4)
-    build(ap.parse_args().jobs)
+    ap.add_argument("--incremental", action="store_true")
+    args = ap.parse_args()
+    build(args.jobs, incremental=args.incremental)

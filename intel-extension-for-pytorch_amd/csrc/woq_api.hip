@@ -9,6 +9,8 @@
 namespace woq {
 
 static thread_local char g_err[512] = "";
+// name of the kernel this thread launched last (check_launch is called once per launch with it)
+static thread_local const char* g_last_kernel = "";
 
 int set_error(const char* fmt, ...) {
   va_list ap;
@@ -19,6 +21,7 @@ int set_error(const char* fmt, ...) {
 }
 
 int check_launch(const char* what) {
+  g_last_kernel = what;
   hipError_t err = hipGetLastError();
   if (err != hipSuccess) return set_error("%s: %s", what, hipGetErrorString(err));
   return 0;
@@ -37,6 +40,8 @@ extern "C" {
 const char* woq_hip_last_error(void) { return g_err; }
 
 int woq_hip_abi_version(void) { return 1; }
+
+const char* woq_hip_last_kernel(void) { return g_last_kernel; }
 
 int64_t woq_hip_padded_n(int64_t N) { return (N + kTileN - 1) / kTileN * kTileN; }
 

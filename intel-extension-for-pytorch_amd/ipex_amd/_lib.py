@@ -21,6 +21,7 @@ TILE_N, TILE_BYTES, TILE_K_INT4, TILE_K_INT8 = 16, 1024, 128, 64
 EXPORTS = [
     "woq_hip_last_error",
     "woq_hip_abi_version",
+    "woq_hip_last_kernel",
     "woq_hip_padded_n",
     "woq_hip_padded_k",
     "woq_hip_packed_weight_bytes",
@@ -98,6 +99,8 @@ def load():
         lib.woq_hip_last_error.restype = ctypes.c_char_p
         lib.woq_hip_last_error.argtypes = []
         lib.woq_hip_abi_version.restype = i32
+        lib.woq_hip_last_kernel.restype = ctypes.c_char_p
+        lib.woq_hip_last_kernel.argtypes = []
         lib.woq_hip_padded_n.restype = i64
         lib.woq_hip_padded_n.argtypes = [i64]
         lib.woq_hip_padded_k.restype = i64
@@ -136,6 +139,11 @@ def load():
             raise RuntimeError("libwoq_hip.so has an unexpected ABI version")
         _lib = lib
     return _lib
+
+
+def last_kernel():
+    """Name of the kernel this thread launched last through the library."""
+    return load().woq_hip_last_kernel().decode("ascii")
 
 
 def check(rc, what):

@@ -347,6 +347,12 @@ class WoqLinearOpContext:
             return x.new_empty(*x.shape[:-1], N)
         if self.g_src_ is not None:
             x = _kernels.shuffle_activations(x, self.g_src_)
+        return self._run_sorted(x, M, fusion, others, kw)
+
+    def _run_sorted(self, x, M, fusion, others, kw):
+        """``run`` behind the act-order shuffle: the input channels of ``x`` are already in the order of
+        the stored weight."""
+        N, K = self.weight_shape_
         if (
             self.cache_weight_for_large_batch_
             and self.lowp_mode_ == _lib.LOWP_BF16
@@ -370,7 +376,7 @@ class WoqLinearOpContext:
             # fp16 and casts the fp16 result back (csrc/cpu/aten/utils/woq.h:3076-3085); doing the two
             # casts around the call reaches the kernels that want rows in the compute dtype
             # (M = 2048, 4096 -> 14336: 430 us through the converting general kernel otherwise)
-            return self.run(x.to(torch.float16)).to(torch.bfloat16)
+            return self._run_sorted(x.to(torch.float16), M, fusion, others, kw).to(torch.bfloat16)
         if not kw and x.dtype in _kernels._ACT_CODE and x.is_cuda:
             return self._run_planned(x, M, fusion, others)
         return _kernels.linear(

@@ -351,8 +351,9 @@ def woq_linear_opt_int8(x, act_dtype, qw, N, K, scales, zps, bias, weight_dtype,
     """lowp_mode INT8.  C = fp32 bias or 0; for each K block kb ascending:
     C += (float(qC[kb]) * s_a) * s_w[n, g(kb)] for the symmetric activation modes 4..7, and
     C += (float(qC[kb] - compensation[n, kb] * zp_a) * s_a) * s_w[n, g(kb)] for the asymmetric
-    modes 0..3 (integer subtraction first, woq.h:2172-2186).  Returns dict(xq, sa, za, sums, acc
-    (fp32), y)."""
+    modes 0..3 (integer subtraction first, woq.h:2172-2186).  Returns dict(xq, sa, za, sums, ints
+    (the integer that is converted to fp32 per block: sums, minus the compensation term for the
+    asymmetric modes), acc (fp32), y)."""
     M = x.shape[0]
     asym = act_quant_mode < 4
     bk = int8_block_k(group_size, K)
@@ -372,6 +373,7 @@ def woq_linear_opt_int8(x, act_dtype, qw, N, K, scales, zps, bias, weight_dtype,
     C = np.zeros((M, N), dtype=np.float32)
     if bias is not None:
         C[:] = np.asarray(bias, dtype=np.float32)[None, :]
+    ints = sums if not asym else np.empty_like(sums)
     for kb in range(K // bk):
         g = (kb * bk) // group_size if group_size > 0 else 0
         kc = (kb * bk) // qbk if per_k else 0
@@ -380,10 +382,11 @@ def woq_linear_opt_int8(x, act_dtype, qw, N, K, scales, zps, bias, weight_dtype,
         if asym:
             qv = qv - comp[:, kb][None, :] * za2[:, kc].reshape(-1, 1)
             assert np.abs(qv).max() < 2**31
+            ints[:, :, kb] = qv
         c = (qv.astype(np.float32) * sa_col).astype(np.float32)
         c = (c * s[:, g][None, :]).astype(np.float32)
         C = (C + c).astype(np.float32)
-    return {"xq": xq, "sa": sa, "za": za, "sums": sums, "acc": C, "y": _round_to(C, act_dtype)}
+    return {"xq": xq, "sa": sa, "za": za, "sums": sums, "ints": ints, "acc": C, "y": _round_to(C, act_dtype)}
 
 
 def woq_linear(x, act_dtype, qw, N, K, scales, zps, bias, weight_dtype, group_size, lowp_mode, act_quant_mode=-1,

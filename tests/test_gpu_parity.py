@@ -998,6 +998,241 @@ def test_c3_prefill_int8(cuda):
 
 
 # ---------------------------------------------------------------------------------------------
+# lowp INT8: the int32 block sums of the kernels that serve the calls (no debug path)
+# ---------------------------------------------------------------------------------------------
+# The debug_block_sums run above is served by the general int8 kernels.  The two checks below read the
+# integers out of the kernels that serve a plain call, through their ordinary fp32 output:
+#  * one K block at a time: with the activations of every other K block set to zero, the accumulator of
+#    (m, n) is the block's integer times s_a[m] times s_w[n, g] with two or three fp32 roundings, so
+#    rint(acc / (s_a s_w)) in float64 is the integer itself while |integer| * 3 * 2^-24 < 1/2
+#    (|integer| <= 128 * 255 * 127 < 2^22);
+#  * all K blocks at once: with weight scales that are powers of two (2^-7 or 2^-6) and activations laid
+#    out so that every activation scale is a power of two, every product and every partial sum of the
+#    epilogue is exact in fp32 in any order, so the fp32 accumulator must EQUAL the oracle's.
+def _pow2_weight_scales(case, seed):
+    out = dict(case)
+    g = torch.Generator().manual_seed(seed)
+    e = torch.randint(6, 8, case["scales"].shape, generator=g).float()
+    out["scales"] = torch.pow(2.0, -e)
+    out["bias"] = None
+    return out
+
+
+def _isolate_k_block(x, kb, bk):
+    out = torch.zeros_like(x)
+    out[:, kb * bk:(kb + 1) * bk] = x[:, kb * bk:(kb + 1) * bk]
+    return out
+
+
+def _plant_pow2_activation_scales(x, mode, qbk, seed):
+    """Clamps every quantization group of x (bf16 [M, K]) into a range whose ends are planted in it, so
+    that its scale is a power of two: symmetric modes max|x| = 127 * 2^e; asymmetric modes
+    min = -a * 2^e, max = (255 - a) * 2^e (max - min = 255 * 2^e, zero point a)."""
+    M, K = x.shape
+    sym, per_m, per_k = mode >= 4, mode in (2, 3, 6, 7), mode in (1, 3, 5, 7)
+    rng = np.random.default_rng(seed)
+    xf = x.float().clone()
+    row_groups = [slice(m, m + 1) for m in range(M)] if per_m else [slice(0, M)]
+    col_groups = [slice(k, min(k + qbk, K)) for k in range(0, K, qbk)] if per_k else [slice(0, K)]
+    for rs in row_groups:
+        for cs in col_groups:
+            e = float(2.0 ** int(rng.integers(-5, -2)))
+            if sym:
+                lo, hi = -127 * e, 127 * e
+            else:
+                a = int(rng.integers(40, 216))
+                lo, hi = -a * e, (255 - a) * e
+            blk = xf[rs, cs].clamp(lo, hi)
+            flat = blk.reshape(-1).clone()
+            i, j = rng.choice(flat.numel(), size=2, replace=False) if flat.numel() > 1 else (0, 0)
+            if sym:
+                flat[i] = hi if rng.integers(2) else lo
+            else:
+                flat[i], flat[j] = lo, hi
+            xf[rs, cs] = flat.reshape(blk.shape)
+    out = xf.to(torch.bfloat16)
+    # the planted ends are bf16 values (integers below 256 times a power of two); rounding the rest to
+    # bf16 cannot leave the range they span
+    return out
+
+
+def _served_by(want_kernel, label):
+    from ipex_amd import _lib
+
+    got = _lib.last_kernel()
+    assert want_kernel is None or got == want_kernel, (label, got, want_kernel)
+    return got
+
+
+def _check_int8_block_integers(case, mode, blocks=None, rows=None, cols=None, want_kernel=None, label=""):
+    """Bit-exact int32 block sums (after the zero-point compensation for the asymmetric modes) of the
+    kernel that serves the call, one K block at a time (see above)."""
+    case = _pow2_weight_scales(case, 7)
+    ctx = make_context(case, O.LOWP_INT8, mode)
+    N, K, G, wd = case["N"], case["K"], case["group_size"], case["weight_dtype"]
+    c = case_np(case)
+    bk = O.int8_block_k(G, K)
+    qbk = G if G > 0 else bk
+    M = case["x"].shape[0]
+    rows = np.arange(M) if rows is None or mode in (0, 1, 4, 5) else np.asarray(rows)
+    cols = np.arange(N) if cols is None else np.asarray(cols)
+    qw, sc = c["qw"][cols], c["scales"].reshape(N, -1)[cols]
+    zp = None if c["zps"] is None else c["zps"].reshape(N, -1)[cols]
+    s_eff = (sc * (np.float32(1.0) / np.float32(127.0))).astype(np.float32) if wd == O.WOQ_DTYPE_NF4 else sc
+    per_m, per_k, asym = mode in (2, 3, 6, 7), mode in (1, 3, 5, 7), mode < 4
+    cols_t = torch.as_tensor(cols).cuda()
+    rows_t = torch.as_tensor(rows).cuda()
+    for kb in (range(K // bk) if blocks is None else blocks):
+        xk = _isolate_k_block(case["x"], kb, bk)
+        acc = ctx.run(xk.cuda(), out_fp32=True)
+        kernel = _served_by(want_kernel, label)
+        acc = acc[rows_t][:, cols_t].double().cpu().numpy()
+        xs = to_np_f32(xk)[rows]
+        xq, sa, za = O.dynamic_quantize_per_block(xs if per_m else to_np_f32(xk), qbk, mode)
+        if not per_m:
+            xq = xq[rows]
+        Mr, Kc = len(rows), (K + qbk - 1) // qbk
+        sa2 = np.asarray(sa, dtype=np.float32).reshape(Mr if per_m else 1, Kc if per_k else 1)
+        kc = (kb * bk) // qbk if per_k else 0
+        want = O.int8_block_sums(xq, qw, len(cols), K, zp, wd, G, bk)[:, :, kb].astype(np.int64)
+        if asym:
+            comp = O.int8_weight_block_sums(qw, len(cols), K, zp, wd, G, bk).astype(np.int64)
+            za2 = np.asarray(za, dtype=np.int64).reshape(Mr if per_m else 1, Kc if per_k else 1)
+            want = want - comp[:, kb][None, :] * za2[:, kc].reshape(-1, 1)
+        assert np.abs(want).max() * 3 * 2.0 ** -24 < 0.5
+        g = (kb * bk) // G if G > 0 else 0
+        denom = sa2[:, kc].reshape(-1, 1).astype(np.float64) * s_eff[:, g][None, :].astype(np.float64)
+        with np.errstate(divide="ignore", invalid="ignore"):
+            got = np.rint(acc / denom)
+        got = np.where(denom == 0, 0, got)  # an all-zero row: scale 0, accumulator 0
+        want = np.where(denom == 0, 0, want)
+        assert np.array_equal(got, want), (label, kernel, kb, int(np.abs(got - want).max()))
+    return kernel
+
+
+def _check_int8_exact_accumulator(case, mode, want_kernel=None, cols=None, label=""):
+    """Power-of-two scales on both sides: the fp32 accumulator of the serving kernel equals the oracle's."""
+    case = _pow2_weight_scales(case, 11)
+    N, K, G, wd = case["N"], case["K"], case["group_size"], case["weight_dtype"]
+    M = case["x"].shape[0]
+    assert wd != O.WOQ_DTYPE_NF4  # its weight scale carries fp32(1 / 127): not a power of two
+    bk = O.int8_block_k(G, K)
+    case["x"] = _plant_pow2_activation_scales(case["x"], mode, G if G > 0 else bk, 5)
+    ctx = make_context(case, O.LOWP_INT8, mode)
+    acc = ctx.run(case["x"].cuda(), out_fp32=True)
+    kernel = _served_by(want_kernel, label)
+    c = case_np(case)
+    cols = np.arange(N) if cols is None else np.asarray(cols)
+    acc = acc[:, torch.as_tensor(cols).cuda()].cpu().numpy()
+    sc = c["scales"].reshape(N, -1)[cols]
+    zp = None if c["zps"] is None else c["zps"].reshape(N, -1)[cols]
+    r = O.woq_linear_opt_int8(c["x"], "bf16", c["qw"][cols], len(cols), K, sc if G > 0 else sc.reshape(-1), zp, None, wd, G, mode)
+    sa = np.asarray(r["sa"], dtype=np.float64)
+    assert np.all(np.log2(sa) == np.rint(np.log2(sa))), "the planted activation scales are powers of two"
+    # every term of the epilogue is an integer multiple of `unit`; while the sum of the terms' magnitudes
+    # stays below 2^24 units every partial sum is exact in fp32, in any order
+    per_m, per_k = mode in (2, 3, 6, 7), mode in (1, 3, 5, 7)
+    qbk = G if G > 0 else bk
+    KB, Kc = K // bk, (K + qbk - 1) // qbk
+    sa2 = sa.reshape(M if per_m else 1, Kc if per_k else 1)
+    sa_kb = sa2[:, [(kb * bk) // qbk if per_k else 0 for kb in range(KB)]]  # [M or 1, KB]
+    sw_kb = sc.astype(np.float64)[:, [(kb * bk) // G if G > 0 else 0 for kb in range(KB)]]  # [cols, KB]
+    unit = sa.min() * 2.0 ** -7
+    mags = np.einsum("mnk,mk,nk->mn", np.abs(r["ints"]).astype(np.float64), np.broadcast_to(sa_kb, (M, KB)), sw_kb)
+    assert mags.max() / unit < 2 ** 24, (label, mags.max() / unit)
+    assert np.array_equal(acc, r["acc"]), (label, kernel, float(np.abs(acc - r["acc"]).max()))
+    return kernel
+
+
+@pytest.mark.parametrize("mode", [0, 1, 2, 3, 4, 5, 6, 7])
+@pytest.mark.parametrize(
+    "M,K,N,G,kernel",
+    [
+        (1, 1024, 272, 128, "woq_decode_w4i8_kernel"),
+        (16, 2048, 1040, 256, "woq_decode_w4i8_kernel"),
+        (32, 1024, 8208, -1, "woq_decode_w4i8_kernel"),  # two row tiles, two row-blocks per workgroup
+        (64, 1024, 272, 128, "woq_gemm_w4i8_kernel"),
+        (150, 1024, 272, 128, "woq_gemm_w4i8_kernel"),
+        (100, 4096, 256, 128, "woq_gemm_w4i8_kernel"),  # K shared between the workgroups of a tile
+        (300, 2048, 528, 512, "woq_gemm_w4i8_kernel"),  # activation blocks of four tiles
+    ],
+)
+def test_int8_mfma_kernels_block_integers_bit_exact(cuda, mode, M, K, N, G, kernel):
+    case = _synthetic().make_int4_case(41, M, K, N, G, outliers=True)
+    if mode < 4:
+        case["x"] = (case["x"].float() + 0.5).to(torch.bfloat16)
+    cols = None if N < 4096 else list(range(0, N, 53)) + [N - 1]
+    label = f"int8 block integers mode={mode} M={M} K={K} N={N} G={G}"
+    blocks = None if K <= 2048 else [0, 1, 13, K // 128 - 1]
+    _check_int8_block_integers(case, mode, blocks=blocks, cols=cols, want_kernel=kernel, label=label)
+    _check_int8_exact_accumulator(case, mode, want_kernel=kernel, cols=cols, label=label)
+
+
+@pytest.mark.parametrize("mode", [4, 5, 6, 7])
+@pytest.mark.parametrize(
+    "M,K,N,G,kernel",
+    [
+        (9, 512, 144, 32, "woq_decode_w4i8_kernel"),  # K blocks inside a packed tile: lane-column masking
+        (32, 1024, 272, 32, "woq_decode_w4i8_kernel"),
+        (2, 384, 48, 64, "woq_decode_w4i8_kernel"),
+        (64, 512, 144, 64, "woq_decode_w4i8_kernel"),  # four row tiles
+        (65, 1024, 272, 64, "woq_gemm_w4i8_kernel"),
+        (150, 2048, 528, 32, None),  # per-(row, K block) scales stay on the general kernel, the others do not
+        (100, 4096, 256, 32, None),
+    ],
+)
+def test_int8_mfma_kernels_small_groups_block_integers_bit_exact(cuda, mode, M, K, N, G, kernel):
+    case = _synthetic().make_int4_case(42, M, K, N, G, outliers=True)
+    label = f"int8 block integers small groups mode={mode} M={M} K={K} N={N} G={G}"
+    if kernel is None:
+        kernel = "woq_gemm_i8_kernel" if (G == 32 and mode in (5, 7)) else "woq_gemm_w4i8_kernel"
+    blocks = None if K // G <= 16 else sorted({0, 1, 2, 3, 4, 37 % (K // G), K // G - 1})
+    _check_int8_block_integers(case, mode, blocks=blocks, want_kernel=kernel, label=label)
+    _check_int8_exact_accumulator(case, mode, want_kernel=kernel, label=label)
+
+
+@pytest.mark.parametrize("mode", [4, 6, 7])
+@pytest.mark.parametrize(
+    "M,K,N,G,kernel",
+    [
+        (1, 1024, 272, -1, "woq_decode_w4i8_kernel"),
+        (17, 1152, 96, 128, "woq_decode_w4i8_kernel"),
+        (70, 2048, 528, 128, "woq_gemm_w4i8_kernel"),
+        (300, 1024, 1040, 256, "woq_gemm_w4i8_kernel"),
+    ],
+)
+def test_int8_mfma_kernels_int8_weights_block_integers_bit_exact(cuda, mode, M, K, N, G, kernel):
+    """Symmetric 8-bit weights: the stored bytes with the sign bit flipped are the MFMA operand."""
+    case = _synthetic().make_int8_case(43, M, K, N, bias=False, group_size=G)
+    label = f"int8 block integers int8 weights mode={mode} M={M} K={K} N={N} G={G}"
+    _check_int8_block_integers(case, mode, want_kernel=kernel, label=label)
+    _check_int8_exact_accumulator(case, mode, want_kernel=kernel, label=label)
+
+
+@pytest.mark.parametrize("mode", [6, 7])
+@pytest.mark.parametrize("M,K,N,G,kernel", [(1, 1024, 272, 128, "woq_decode_w4i8_kernel"), (40, 512, 144, 32, None),
+                                            (150, 1024, 272, 128, "woq_gemm_w4i8_kernel")])
+def test_int8_mfma_kernels_nf4_block_integers_bit_exact(cuda, mode, M, K, N, G, kernel):
+    """NF4 codes as int8 table values through two byte permutes."""
+    case = _synthetic().make_nf4_case(44, M, K, N, G)
+    _check_int8_block_integers(case, mode, want_kernel=kernel,
+                               label=f"int8 block integers nf4 mode={mode} M={M} K={K} N={N} G={G}")
+
+
+@pytest.mark.parametrize("mode", [6, 7])
+def test_c3_prefill_int8_block_integers_bit_exact(cuda, mode):
+    """The named prefill configuration at full size (M = 2048, 4096 -> 14336, G = 128, 1 % outliers) on the
+    kernel that serves it: K blocks 0, 1, 13 and 31 alone (every 61st column, every 8th row against the
+    oracle), then all blocks with power-of-two scales: accumulators equal to the oracle's."""
+    case = _synthetic().make_int4_case(3, 2048, 4096, 14336, 128, outliers=True)
+    cols = np.arange(0, 14336, 61)
+    _check_int8_block_integers(case, mode, blocks=[0, 1, 13, 31], rows=np.arange(0, 2048, 8), cols=cols,
+                               want_kernel="woq_gemm_w4i8_kernel", label=f"C3 int8 block integers mode={mode}")
+    _check_int8_exact_accumulator(case, mode, want_kernel="woq_gemm_w4i8_kernel", cols=cols,
+                                  label=f"C3 int8 exact accumulator mode={mode}")
+
+
+# ---------------------------------------------------------------------------------------------
 # post-ops and size-independent properties
 # ---------------------------------------------------------------------------------------------
 def test_fused_post_ops(cuda):
@@ -1112,6 +1347,35 @@ def test_g_idx_matches_the_group_sorted_problem(cuda, M):
         )
         ref_i8 = make_context(sorted_case, O.LOWP_INT8, 6)
         assert torch.equal(ctx_i8.run(x), ref_i8.run(sorted_case["x"].cuda()))
+
+
+@pytest.mark.parametrize("M", [17, 200])
+def test_g_idx_under_lowp_fp16_with_bf16_rows(cuda, M):
+    """fp16 compute on bf16 rows beyond one row tile casts the rows around the call: the act-order
+    shuffle must be applied once, not once per cast level.  Checked against the oracle on the
+    group-sorted problem and bit for bit against the context of the sorted problem."""
+    from ipex_amd import ops
+
+    K, N, G = 512, 96, 128
+    for name, g_idx in _g_idx_cases(K, G):
+        case = _synthetic().make_int4_case(36, M, K, N, G, bias=True)
+        src = np.argsort(g_idx.numpy(), kind="stable")
+        dst = torch.from_numpy(np.argsort(src))
+        q = O.unpack_int4(case["qweight"].numpy())[:, :K]
+        sorted_case = dict(case)
+        sorted_case["x"] = case["x"][:, torch.from_numpy(src)].contiguous()
+        sorted_case["qweight"] = torch.from_numpy(O.pack_int4(np.ascontiguousarray(q[:, src])))
+        ctx = ops.WoqLinearOpContext(
+            case["qweight"].cuda(), 2, [N, K], case["scales"].cuda(), case["zeros"].cuda(), case["bias"].cuda(),
+            g_idx, None, G, O.LOWP_FP16, -1,
+        )
+        ref = make_context(sorted_case, O.LOWP_FP16)
+        y = ctx.run(case["x"].cuda())
+        assert torch.equal(y, ref.run(sorted_case["x"].cuda())), name
+        c = case_np(sorted_case)
+        _, want = O.woq_linear_ref(c["x"], "bf16", c["qw"], N, K, O._round_to(c["scales"], "fp16"), c["zps"], c["bias"],
+                                   2, G, "fp16")
+        assert rel_l2(to_np_f32(y), want) <= REL_L2_OUT, name
 
 
 def test_g_idx_validation(cuda):
