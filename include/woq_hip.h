@@ -252,6 +252,20 @@ int64_t woq_hip_int8_block_k(int64_t group_size, int64_t K);
 
 int woq_hip_linear(const woq_hip_linear_params* p);
 
+/* woq_hip_linear for callers that cannot allocate and hold no workspace: code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc.  No counterpart in the reference, whose kernels
+ * take their temporaries from the CPU heap.  Same arguments and results as woq_hip_linear, except that
+ * workspace, workspace_bytes and split_k_counters must be NULL / 0: the quantized activations of
+ * lowp_mode INT8 and the split-K scratch live in an array that the library keeps resident on every GPU it
+ * runs on (WOQ_HIP_NOALLOC_MAX_WORKSPACE_BYTES plus 2 KiB of counters, until the process ends).  A call
+ * whose workspace need (woq_hip_linear_workspace_bytes) exceeds that maximum is rejected with an error
+ * before anything is launched; K is shared between workgroups only while that scratch fits as well.
+ * Allocates nothing, on the device or through any library.  All calls on one GPU share the array: calls
+ * that may overlap in time on one GPU (different streams, concurrent graph launches) race and must be
+ * serialised by the caller. */
+#define WOQ_HIP_NOALLOC_MAX_WORKSPACE_BYTES (12 * 1024 * 1024)
+int woq_hip_linear_noalloc(const woq_hip_linear_params* p);
+
 /* Packed weight -> dense [N, K] in out_dtype (fp32: (q - z) * s exactly; fp16 / bf16: that
  * value rounded to nearest even).  Used by the weight cache and by tests. */
 int woq_hip_dequant_weight(const void* qweight, int weight_dtype, int64_t N, int64_t K,

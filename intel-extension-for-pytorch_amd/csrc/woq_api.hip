@@ -3,6 +3,8 @@
 #include <stdio.h>
 #include <string.h>
 
+#include <mutex>
+
 #include "woq_common.h"
 #include "woq_internal.h"
 
@@ -339,6 +341,87 @@ int woq_hip_moe_scale_add_rows(void* out, int dtype, int64_t T, int64_t H, const
                               (long long)T);
   return launch_moe_scale_add_rows(out, dtype, H, expert_out, routing_weights, topk, top_x, idx, n,
                                    (hipStream_t)stream);
+}
+
+// ---- woq_hip_linear for callers that cannot allocate ----------------------------------------------
+// One array per GPU, resident until the process ends: 512 split-K counters, then the workspace.
+constexpr int64_t kNoAllocCounterBytes = kSplitKCounters * (int64_t)sizeof(int32_t);
+constexpr int64_t kNoAllocWorkspaceBytes = WOQ_HIP_NOALLOC_MAX_WORKSPACE_BYTES;
+static __device__ __align__(256) unsigned char scratch[kNoAllocCounterBytes + kNoAllocWorkspaceBytes];
+
+// `scratch` above is a host-side stand-in, not a device address: the address of each GPU's copy comes
+// from hipGetSymbolAddress with that GPU current, once per device.
+constexpr int kMaxDevices = 64;
+static std::mutex g_scratch_mutex;
+static unsigned char* g_scratch_ptr[kMaxDevices] = {};
+
+static int scratch_of_current_device(unsigned char** out) {
+  int dev = -1;
+  hipError_t err = hipGetDevice(&dev);
+  if (err != hipSuccess) return set_error("woq_linear_noalloc: hipGetDevice: %s", hipGetErrorString(err));
+  if (dev < 0 || dev >= kMaxDevices) return set_error("woq_linear_noalloc: device index %d out of range", dev);
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_ptr[dev]) {
+    void* ptr = nullptr;
+    err = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (err != hipSuccess || !ptr)
+      return set_error("woq_linear_noalloc: hipGetSymbolAddress: %s", hipGetErrorString(err));
+    g_scratch_ptr[dev] = (unsigned char*)ptr;
+  }
+  *out = g_scratch_ptr[dev];
+  return 0;
+}
+
+__global__ void zero_counters_kernel(int32_t* p, int n) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) p[i] = 0;
+}
+
+int woq_hip_linear_noalloc(const woq_hip_linear_params* p) {
+  if (!p) return set_error("woq_linear_noalloc: null params");
+  if (p->struct_size != sizeof(woq_hip_linear_params))
+    return set_error("woq_linear_noalloc: struct_size %u does not match this library (%zu)", p->struct_size,
+                     sizeof(woq_hip_linear_params));
+  if (p->workspace || p->workspace_bytes != 0 || p->split_k_counters)
+    return set_error("woq_linear_noalloc: workspace and split_k_counters must be null; the library's resident "
+                     "scratch takes their place");
+  if (p->M < 0 || p->K <= 0 || p->N <= 0)
+    return set_error("woq_linear_noalloc: bad shape M=%lld K=%lld N=%lld", (long long)p->M, (long long)p->K,
+                     (long long)p->N);
+  if (p->M == 0) return woq_hip_linear(p);
+  const bool int8 = p->lowp_mode == WOQ_HIP_LOWP_INT8;
+  int64_t need = woq_hip_linear_workspace_bytes(p->M, p->K, p->lowp_mode, p->act_quant_mode, p->group_size);
+  if (need > kNoAllocWorkspaceBytes)
+    return set_error("woq_linear_noalloc: M=%lld K=%lld under lowp_mode INT8 needs %lld bytes of workspace, the "
+                     "resident scratch holds %lld; use woq_hip_linear with a workspace of your own",
+                     (long long)p->M, (long long)p->K, (long long)need, (long long)kNoAllocWorkspaceBytes);
+  // Sharing K between workgroups is an option, not a need: offered for the problems it pays for (few
+  // output tiles and a long K) while its scratch fits behind the quantized activations.
+  bool split = false;
+  if ((!int8 && p->M <= 32 && p->K >= 8192 && p->N <= 4096) || (p->M > 64 && p->K >= 4096 && p->M * p->N <= 1048576)) {
+    const int64_t extra = woq_hip_linear_split_k_workspace_bytes(p->M, p->N);
+    const int64_t base = (need + 255) / 256 * 256;
+    if (extra > 0 && base + extra <= kNoAllocWorkspaceBytes) {
+      need = base + extra;
+      split = true;
+    }
+  }
+  woq_hip_linear_params q = *p;
+  if (need > 0) {
+    unsigned char* ptr = nullptr;
+    if (int rc = scratch_of_current_device(&ptr)) return rc;
+    q.workspace = ptr + kNoAllocCounterBytes;
+    q.workspace_bytes = need;
+    if (split) {
+      // every finished launch leaves the counters at zero; a fill kernel (not a memset node, so that the
+      // call can be captured into a HIP graph) makes that hold whatever ran before
+      q.split_k_counters = (int32_t*)ptr;
+      zero_counters_kernel<<<(kSplitKCounters + 255) / 256, 256, 0, (hipStream_t)p->stream>>>(q.split_k_counters,
+                                                                                              kSplitKCounters);
+      if (int rc = check_launch("zero_counters_kernel")) return rc;
+    }
+  }
+  return woq_hip_linear(&q);
 }
 
 }  // extern "C"

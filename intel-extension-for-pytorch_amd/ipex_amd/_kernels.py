@@ -180,10 +180,12 @@ def linear(
     out_fp32=False,
     force_kernel=0,
     debug_block_sums=False,
+    noalloc=False,
 ):
     """y = x @ dequant(W)^T (+ bias, post-op).  x: [..., K]; returns [..., N] in x.dtype, or the
     fp32 accumulator when ``out_fp32``.  With ``debug_block_sums`` also returns the int32 sum of
-    every (m, n, K block) of the int8 path."""
+    every (m, n, K block) of the int8 path.  ``noalloc``: through ``woq_hip_linear_noalloc``, which
+    takes no workspace (the output tensor is still made here)."""
     lib = _lib.load()
     _require_cuda(x, "input")
     if x.dtype not in _ACT_CODE:
@@ -226,7 +228,7 @@ def linear(
     p.out = out.data_ptr()
     p.out_dtype = _ACT_CODE[out_dtype]
     ws = None
-    wbytes = lib.woq_hip_linear_workspace_bytes(M, K, lowp_mode, act_quant_mode, group_size)
+    wbytes = 0 if noalloc else lib.woq_hip_linear_workspace_bytes(M, K, lowp_mode, act_quant_mode, group_size)
     counters = None
     if wbytes > 0 and lowp_mode == 3 and M > 64:
         # lowp INT8 at prefill sizes: room behind the quantized activations lets the int8 GEMM share a
@@ -236,7 +238,7 @@ def linear(
         if counters is not None:
             p.split_k_counters = counters.data_ptr()
             wbytes = (wbytes + 255) // 256 * 256 + extra
-    if wbytes == 0 and lowp_mode != 3:
+    if wbytes == 0 and lowp_mode != 3 and not noalloc:
         # scratch that lets the decode kernel split K across workgroups (small M, few output columns)
         wbytes = lib.woq_hip_linear_split_k_workspace_bytes(M, N)
         counters = _split_k_counters(x.device) if wbytes > 0 else None
@@ -257,7 +259,8 @@ def linear(
     p.force_kernel = force_kernel
     with torch.cuda.device(x.device):
         p.stream = torch.cuda.current_stream().cuda_stream
-        _lib.check(lib.woq_hip_linear(ctypes.byref(p)), "woq_linear")
+        entry = lib.woq_hip_linear_noalloc if noalloc else lib.woq_hip_linear
+        _lib.check(entry(ctypes.byref(p)), "woq_linear")
     out = out.reshape(*x.shape[:-1], N)
     if debug_block_sums:
         return out, sums

@@ -34,6 +34,7 @@ EXPORTS = [
     "woq_hip_linear_split_k_workspace_bytes",
     "woq_hip_int8_block_k",
     "woq_hip_linear",
+    "woq_hip_linear_noalloc",
     "woq_hip_dequant_weight",
     "woq_hip_shuffle_activations",
     "woq_hip_shuffle_int4_weight",
@@ -125,6 +126,8 @@ def load():
         lib.woq_hip_int8_block_k.argtypes = [i64, i64]
         lib.woq_hip_linear.restype = i32
         lib.woq_hip_linear.argtypes = [ctypes.POINTER(LinearParams)]
+        lib.woq_hip_linear_noalloc.restype = i32
+        lib.woq_hip_linear_noalloc.argtypes = [ctypes.POINTER(LinearParams)]
         lib.woq_hip_dequant_weight.restype = i32
         lib.woq_hip_dequant_weight.argtypes = [vp, i32, i64, i64, vp, vp, i64, vp, i32, vp]
         lib.woq_hip_shuffle_activations.restype = i32
