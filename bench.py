@@ -26,10 +26,15 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
 MFMA_FP32_PEAK_TFLOPS = 157.3   # MI355X dense fp32 matrix, published
 
 
-# HBM bytes per launch of the dominant kernel, from two rocprofv3 --pmc runs of `bench.py --traffic-probe`
-# (FETCH_SIZE 15310.55 KiB and WRITE_SIZE 28.00 KiB per dispatch, scaled by what the same counters read for a
-# 256 MiB copy: x2.000 and x1.000); keyed by (M, K, N, group size).  Other shapes have not been measured.
-MEASURED_HBM_BYTES_PER_LAUNCH = {(1, 4096, 14336, 128): 31384678}
+# HBM bytes per launch of the dominant kernel.  Hardware counters cannot be read from inside this process:
+# the figure comes from two rocprofv3 --pmc runs of `bench.py --probe decode` (FETCH_SIZE 15310.55 KiB and
+# WRITE_SIZE 28.00 KiB per dispatch, scaled by what the same counters read for a 256 MiB copy: x2.000 and
+# x1.000), whose summary is the file named beside it; keyed by (M, K, N, group size).  Other shapes: null.
+PROFILED_HBM_BYTES_PER_LAUNCH = {(1, 4096, 14336, 128): 31384678}
+PROFILED_HBM_BYTES_SOURCE = "profiles/woq_decode_kernel_M1_4096x14336_g128.hbm_traffic.txt"
+# Launches that precede every timed region whatever --warmup says: the first milliseconds after an idle
+# period run 3-10 % slower (clocks, translation caches).
+MIN_WARMUP_LAUNCHES = 2000
 
 
 _SPLIT_K_SCRATCH = {}
@@ -101,6 +106,13 @@ def time_steps(torch, lib, params, steps, warmup, stream):
     return t1 - t0, start.elapsed_time(stop)
 
 
+def time_groups(torch, lib, params, steps, stream, groups=9):
+    """`groups` timed regions of exactly `steps` launches each (synchronize on both sides, HIP events on
+    the launch stream inside); returns the (host wall seconds, event milliseconds) of the median group."""
+    runs = sorted((time_steps(torch, lib, params, steps, 0, stream) for _ in range(groups)), key=lambda r: r[1])
+    return runs[len(runs) // 2]
+
+
 def _quantiles(vals):
     v = sorted(vals)
     pick = lambda q: v[min(len(v) - 1, int(q * len(v)))]
@@ -153,16 +165,19 @@ def time_graph(torch, lib, params, steps, warmup):
     reps = max(1, steps // n)
     for _ in range(max(1, warmup // n)):
         g.replay()
-    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    start.record()
-    for _ in range(reps):
-        g.replay()
-    stop.record()
-    torch.cuda.synchronize()
-    t1 = time.perf_counter()
-    return reps * n, t1 - t0, start.elapsed_time(stop)
+    runs = []
+    for _ in range(9):
+        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        start.record()
+        for _ in range(reps):
+            g.replay()
+        stop.record()
+        torch.cuda.synchronize()
+        runs.append((time.perf_counter() - t0, start.elapsed_time(stop)))
+    runs.sort(key=lambda r: r[1])
+    return (reps * n,) + runs[len(runs) // 2]
 
 
 def _rotating_params(torch, lib_mod, ops_mod, case, lowp_mode, dev, stream, min_bytes=640e6, act_quant_mode=-1):
@@ -343,24 +358,127 @@ def cpu_baseline_decode(case, K, N, G, budget_s=12.0, gpu_out=None):
     return res
 
 
+def _calibration_copy(torch, dev):
+    """One 256 MiB device-to-device copy: FETCH_SIZE / WRITE_SIZE of this dispatch against its known size
+    give the factors that turn the counters of the other dispatches into bytes."""
+    src = torch.empty(256 << 20, dtype=torch.uint8, device=dev)
+    dst = torch.empty_like(src)
+    torch.cuda.synchronize()
+    dst.copy_(src)
+    torch.cuda.synchronize()
+    return 256 << 20
+
+
+def run_probe(name, torch, lib, lib_mod, ops_mod, synthetic, dev, stream):
+    """Short fixed workloads for `rocprofv3 --pmc ... -- python3 bench.py --probe NAME` (one counter set per
+    run) and for `rocprofv3 --kernel-trace --stats`: a few launches of one kernel family over rotating
+    weight copies (every launch reads its weights from HBM), then a device copy of known size that
+    calibrates the byte counters.  Prints one JSON line saying what was launched."""
+    info = {"probe": name}
+    if name == "decode_dq":
+        # the bf16-regime decode kernel at the named M = 16 shapes (both layers of a gated MLP)
+        info["launches"] = []
+        for K, N in ((4096, 14336), (14336, 4096)):
+            case = synthetic.make_int4_case(2, 16, K, N, 128)
+            params, keep = _rotating_params(torch, lib_mod, ops_mod, case, 2, dev, stream)
+            for i in range(66):
+                assert lib.woq_hip_linear(ctypes.byref(params[i % len(params)])) == 0, lib.woq_hip_last_error()
+            torch.cuda.synchronize()
+            info["launches"].append({"M": 16, "K": K, "N": N, "G": 128, "count": 66, "kernel": lib_mod.last_kernel(),
+                                     "algorithmic_bytes_per_launch": algorithmic_bytes(16, K, N, 128)})
+            del params, keep
+    elif name == "prefill":
+        # the named prefill configuration under lowp_mode BF16 and INT8 (per-row activation scales)
+        K, N, G, Mp = 4096, 14336, 128, 2048
+        case = synthetic.make_int4_case(3, Mp, K, N, G, outliers=True)
+        info["launches"] = []
+        for lowp, aq in ((2, -1), (3, 6)):
+            params, keep = _rotating_params(torch, lib_mod, ops_mod, case, lowp, dev, stream, min_bytes=1, act_quant_mode=aq)
+            for _ in range(20):
+                assert lib.woq_hip_linear(ctypes.byref(params[0])) == 0, lib.woq_hip_last_error()
+            torch.cuda.synchronize()
+            info["launches"].append({"M": Mp, "K": K, "N": N, "G": G, "lowp_mode": lowp, "count": 20,
+                                     "kernel": lib_mod.last_kernel(), "flops_per_launch": 2.0 * Mp * K * N})
+            del params, keep
+    elif name == "floor":
+        info.update(floor_probe(torch, lib, dev, stream))
+        print(json.dumps(info))
+        return
+    else:
+        raise SystemExit(f"unknown probe {name!r}")
+    info["calibration_copy_bytes"] = _calibration_copy(torch, dev)
+    print(json.dumps(info))
+
+
+def floor_probe(torch, lib, dev, stream, groups=9, per_group=200):
+    """What a launch of the headline decode kernel's shape costs without its arithmetic: an empty kernel
+    of the same grid (448 workgroups of 16 waves) and pure streaming reads of the same 28 MiB of packed
+    weights (rotating over 23 distinct buffers, 675 MB, so that every launch reads HBM) in several
+    launch shapes; microseconds per launch, median of `groups` groups of `per_group` back-to-back launches."""
+    nbytes = 14336 * 4096 // 2
+    bufs = [torch.empty(nbytes, dtype=torch.uint8, device=dev).random_(0, 256) for _ in range(23)]
+    sink = torch.zeros(4, dtype=torch.int32, device=dev)
+    st = ctypes.c_void_p(stream.cuda_stream)
+
+    def timed(launch):
+        for i in range(per_group):
+            launch(i)
+        vals = []
+        for _ in range(groups):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            torch.cuda.synchronize()
+            e0.record(stream)
+            for i in range(per_group):
+                launch(i)
+            e1.record(stream)
+            torch.cuda.synchronize()
+            vals.append(e0.elapsed_time(e1) * 1e3 / per_group)
+        return round(sorted(vals)[len(vals) // 2], 3)
+
+    out = {"bytes_per_launch": nbytes, "rotating_buffers": len(bufs)}
+
+    def empty(i):
+        assert lib.woq_hip_probe_empty(448, 16, st) == 0
+
+    out["empty_kernel_448x16_waves_us"] = timed(empty)
+    reads = {}
+    for waves, kib in ((16, 4), (16, 2), (8, 4), (8, 8), (4, 8), (16, 1)):
+        def read(i, waves=waves, kib=kib):
+            rc = lib.woq_hip_probe_stream_read(ctypes.c_void_p(bufs[i % len(bufs)].data_ptr()), nbytes, waves, kib,
+                                               ctypes.c_void_p(sink.data_ptr()), st)
+            assert rc == 0, lib.woq_hip_last_error()
+
+        us = timed(read)
+        reads[f"{waves}_waves_x_{kib}_KiB"] = {"us": us, "GB_per_s": round(nbytes / us / 1e3, 1),
+                                               "frac_of_hbm_peak": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 3)}
+    out["stream_read_us"] = reads
+    best = min(v["us"] for v in reads.values())
+    out["best_stream_read_us"] = best
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=4000)
     ap.add_argument("--warmup", type=int, default=2000,
-                    help="untimed launches before the timed ones (the first few milliseconds after an idle "
-                         "period run 3-10 %% slower: clocks and translation caches are still warming up)")
+                    help="untimed launches before the timed ones; at least %d are run whatever is asked "
+                         "(the first few milliseconds after an idle period run 3-10 %%%% slower: clocks and "
+                         "translation caches are still warming up)" % MIN_WARMUP_LAUNCHES)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-prefill", action="store_true", help="skip the M=2048 measurement")
     ap.add_argument("--no-sweep", action="store_true", help="skip the other named configurations")
+    ap.add_argument("--no-floor", action="store_true", help="skip the streaming-read / empty-kernel floor")
     ap.add_argument("--M", type=int, default=1, help="decode batch (1..16)")
-    ap.add_argument("--traffic-probe", action="store_true",
-                    help="short run for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE: a few decode launches plus a "
-                         "plain device copy of known size that calibrates the counter")
+    ap.add_argument("--probe", choices=["decode", "decode_dq", "prefill", "floor"],
+                    help="short fixed workload for a rocprofv3 run (counters or kernel trace) instead of the benchmark")
+    ap.add_argument("--traffic-probe", action="store_true", help="same as --probe decode")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path; run with --gpus 1", file=sys.stderr)
         sys.exit(2)
+    if args.traffic_probe:
+        args.probe = "decode"
 
     import torch
 
@@ -373,6 +491,10 @@ def main():
     dev = torch.device("cuda", 0)
     stream = torch.cuda.current_stream()
     K, N, G, M = 4096, 14336, 128, args.M
+
+    if args.probe and args.probe != "decode":
+        run_probe(args.probe, torch, lib, _lib, ops, synthetic, dev, stream)
+        return _finish()
 
     case = synthetic.make_int4_case(2, M, K, N, G)
     ctx0 = ops.WoqLinearOpContext(
@@ -402,32 +524,38 @@ def main():
         params.append(p)
 
     nbytes = algorithmic_bytes(M, K, N, G)
-    if args.traffic_probe:
+    if args.probe == "decode":
         # 64 launches over distinct weight copies, then one 256 MiB device-to-device copy kernel
         for i in range(64):
             lib.woq_hip_linear(ctypes.byref(params[i % len(params)]))
-        src = torch.empty(256 << 20, dtype=torch.uint8, device=dev)
-        dst = torch.empty_like(src)
         torch.cuda.synchronize()
-        dst.copy_(src)
-        torch.cuda.synchronize()
-        print(json.dumps({"traffic_probe": True, "decode_launches": 64, "copy_bytes": 256 << 20,
+        print(json.dumps({"probe": "decode", "decode_launches": 64, "kernel": _lib.last_kernel(),
+                          "calibration_copy_bytes": _calibration_copy(torch, dev),
                           "algorithmic_bytes_per_launch": nbytes}))
-        return
-    wall, ev_ms = time_steps(torch, lib, params, args.steps, args.warmup, stream)
-    g_steps, g_wall, g_ev_ms = time_graph(torch, lib, params, args.steps, args.warmup)
+        return _finish()
+
+    # Whatever --steps / --warmup ask for, the device is warmed up first and the timed region of exactly
+    # `steps` launches is repeated nine times, the median region being reported.
+    warm = max(args.warmup, MIN_WARMUP_LAUNCHES)
+    time_steps(torch, lib, params, 1, warm, stream)
+    wall, ev_ms = time_groups(torch, lib, params, args.steps, stream)
+    kernel_name = _lib.last_kernel()
+    g_steps, g_wall, g_ev_ms = time_graph(torch, lib, params, args.steps, warm)
     for p in params:
         p.stream = stream.cuda_stream
     # cache-resident figure: the same weight every launch
-    _, hot_ms = time_steps(torch, lib, params[:1], args.steps, args.warmup, stream)
+    time_steps(torch, lib, params[:1], 1, 200, stream)
+    _, hot_ms = time_groups(torch, lib, params[:1], args.steps, stream)
     spread, single = launch_distribution(torch, lib, params, stream)
     out_host = out.cpu()
 
     us_launch = ev_ms * 1e3 / args.steps
     us_graph = g_ev_ms * 1e3 / g_steps
     best_us = min(us_launch, us_graph)
-    value = nbytes / (min(wall / args.steps, g_wall / g_steps)) / 1e9
-    achieved = nbytes / (best_us * 1e-6) / 1e9
+    # throughput of the timed region on the device clock (HIP events on the launch stream, inputs resident);
+    # the host's wall clock around the same region is reported beside it: with few steps it is dominated
+    # by the latency of the closing synchronize
+    value = nbytes / (best_us * 1e-6) / 1e9
 
     result = {
         "metric": "INT4 WOQ linear: GB/s (% of HBM peak) at M=1; TFLOPS at M=2048",
@@ -436,25 +564,31 @@ def main():
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
-        "ms_per_step": round(min(wall / args.steps, g_wall / g_steps) * 1e3, 6),
+        "ms_per_step": round(best_us * 1e-3, 6),
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "fp16 x int4 -> fp32 accumulate (lowp_mode BF16, M < 5)" if M < 5 else "bf16 x int4 -> fp32 accumulate",
+        "dtype": ("bf16 activations x int4 weights -> fp32 accumulate (v_mfma_f32_16x16x32_bf16 on exact integer "
+                  "weights, group scale applied to the group sum in fp32; the reference's M < 5 arithmetic)") if M < 5
+                 else "bf16 x bf16-rounded dequantized int4 -> fp32 accumulate (v_mfma_f32_16x16x32_bf16)",
         "data": "synthetic",
         "config": {
             "workload": f"INT4 g128 woq_linear decode, M={M}, K={K}, N={N}, lowp_mode=BF16, "
                         f"{copies} rotating weight copies ({copies * per_copy / 1e6:.0f} MB)",
             "algorithmic_bytes_per_step": nbytes,
+            "timing": f"{warm} warm-up launches, then 9 regions of {args.steps} back-to-back launches each between "
+                      "HIP events on the launch stream; median region",
+            "ms_per_step_host_wall": round(min(wall / args.steps, g_wall / g_steps) * 1e3, 6),
         },
         "roofline": {
             "bound": "hbm",
-            "achieved": round(achieved, 1),
+            "achieved": round(value, 1),
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
-            "frac": round(achieved / HBM_PEAK_GBS, 4),
-            "traffic": MEASURED_HBM_BYTES_PER_LAUNCH.get((M, K, N, G)),
-            "kernel": "woq_decode_kernel",
+            "frac": round(value / HBM_PEAK_GBS, 4),
+            "traffic": PROFILED_HBM_BYTES_PER_LAUNCH.get((M, K, N, G)),
+            "traffic_source": PROFILED_HBM_BYTES_SOURCE if (M, K, N, G) in PROFILED_HBM_BYTES_PER_LAUNCH else None,
+            "kernel": kernel_name,
             "us_per_launch_stream": round(us_launch, 3),
             "us_per_launch_graph": round(us_graph, 3),
             "us_per_launch_cache_resident": round(hot_ms * 1e3 / args.steps, 3),
@@ -470,6 +604,8 @@ def main():
         outp = torch.empty(Mp, N, dtype=torch.bfloat16, device=dev)
         flops = 2.0 * Mp * K * N
         pre = {}
+        # its own fixed counts, whatever --steps says: 60 warm-up launches, then five regions of 40
+        warm_p, steps_p, groups_p = 60, 40, 5
         for name, lowp, aq in (("bf16", 2, -1), ("int8", 3, 6)):
             ws = None
             wbytes = lib.woq_hip_linear_workspace_bytes(Mp, K, lowp, aq, G)
@@ -477,28 +613,33 @@ def main():
                 ws = torch.empty(wbytes, dtype=torch.uint8, device=dev)
             pp = build_params(_lib, xp, keep[0], outp, lowp, aq, ws)
             pp.stream = stream.cuda_stream
-            steps_p = max(10, min(200, args.steps // 20))
-            _, ms = time_steps(torch, lib, [pp], steps_p, max(3, steps_p // 2), stream)
+            time_steps(torch, lib, [pp], 1, warm_p, stream)
+            _, ms = time_groups(torch, lib, [pp], steps_p, stream, groups=groups_p)
             us = ms * 1e3 / steps_p
-            pre[name] = {"us_per_step": round(us, 2), "tflops": round(flops / (us * 1e-6) / 1e12, 1)}
+            pre[name] = {"us_per_step": round(us, 2), "tflops": round(flops / (us * 1e-6) / 1e12, 1),
+                         "kernel": _lib.last_kernel()}
         # For scale: the vendor's dense bf16 GEMM (torch.matmul) on the same activations and the
         # already dequantized weight.  It does no dequantization; its rate on random data is what
         # this chip sustains for the shape (the clock drops under MFMA load with non-zero operands).
         wd = _kernels.dequant_weight(keep[0].at_weight_, keep[0].weight_dtype_, N, K, keep[0].scales_list_[0],
                                      keep[0].zeros_u8_, G, torch.bfloat16)
-        for _ in range(5):
+        for _ in range(warm_p):
             torch.matmul(xp, wd.t())
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        torch.cuda.synchronize()
-        e0.record()
-        for _ in range(steps_p):
-            torch.matmul(xp, wd.t())
-        e1.record()
-        torch.cuda.synchronize()
-        us_d = e0.elapsed_time(e1) * 1e3 / steps_p
+        dense = []
+        for _ in range(groups_p):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            torch.cuda.synchronize()
+            e0.record()
+            for _ in range(steps_p):
+                torch.matmul(xp, wd.t())
+            e1.record()
+            torch.cuda.synchronize()
+            dense.append(e0.elapsed_time(e1) * 1e3 / steps_p)
+        us_d = sorted(dense)[len(dense) // 2]
         del wd
         result["prefill_m2048"] = {
             "workload": f"INT4 g128 woq_linear prefill, M={Mp}, K={K}, N={N}",
+            "timing": f"{warm_p} warm-up launches, then {groups_p} regions of {steps_p} launches; median region",
             "flops_per_step": flops,
             "lowp_bf16": pre["bf16"],
             "lowp_int8_per_row": pre["int8"],
@@ -508,9 +649,14 @@ def main():
             "peak_tflops": MFMA_BF16_PEAK_TFLOPS,
         }
 
-    if not args.no_sweep and M == 1:
-        del params, keep
+    del params, keep
+    torch.cuda.empty_cache()
+    if not args.no_floor and M == 1:
+        # the floor of a launch of this size on this GPU, measured in the same process
+        result["roofline"]["launch_floor"] = floor_probe(torch, lib, dev, stream)
         torch.cuda.empty_cache()
+
+    if not args.no_sweep and M == 1:
         result["other_configs"] = config_sweep(torch, lib, _lib, ops, synthetic, dev, stream,
                                                max(50, min(400, args.steps // 10)))
 
@@ -520,6 +666,18 @@ def main():
     else:
         result["cpu_baseline"] = None
     print(json.dumps(result))
+    _finish()
+
+
+def _finish():
+    """Leaves at once: everything is printed, and the runtime's teardown (worker threads of the CPU leg,
+    the HIP context) has nothing left to do that a result depends on."""
+    import torch
+
+    torch.cuda.synchronize()
+    sys.stdout.flush()
+    sys.stderr.flush()
+    os._exit(0)
 
 
 if __name__ == "__main__":

@@ -295,6 +295,16 @@ int woq_hip_moe_scale_add_rows(void* out, int dtype, int64_t T, int64_t H, const
                                const void* routing_weights, int64_t topk, const int64_t* top_x, const int64_t* idx,
                                int64_t n, void* stream);
 
+/* Measurement probes (no counterpart in the reference): the floor of an HBM-bound launch on this GPU.
+ *   probe_stream_read: reads `bytes` from src once, `kib_per_wave` (1, 2, 4 or 8) KiB per wave as one
+ *                      non-temporal dwordx4 load per lane and KiB, `waves_per_wg` (1..16) waves per
+ *                      workgroup, no arithmetic, nothing written (sink, one dword, may be NULL);
+ *                      bytes must be whole workgroups.
+ *   probe_empty:       an empty kernel of the given grid. */
+int woq_hip_probe_stream_read(const void* src, int64_t bytes, int waves_per_wg, int kib_per_wave, void* sink,
+                              void* stream);
+int woq_hip_probe_empty(int64_t workgroups, int waves_per_wg, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -40,6 +40,8 @@ EXPORTS = [
     "woq_hip_shuffle_int4_weight",
     "woq_hip_moe_gather_rows",
     "woq_hip_moe_scale_add_rows",
+    "woq_hip_probe_stream_read",
+    "woq_hip_probe_empty",
 ]
 
 
@@ -138,6 +140,10 @@ def load():
         lib.woq_hip_moe_gather_rows.argtypes = [vp, i32, i64, i64, vp, i64, vp, vp]
         lib.woq_hip_moe_scale_add_rows.restype = i32
         lib.woq_hip_moe_scale_add_rows.argtypes = [vp, i32, i64, i64, vp, vp, i64, vp, vp, i64, vp]
+        lib.woq_hip_probe_stream_read.restype = i32
+        lib.woq_hip_probe_stream_read.argtypes = [vp, i64, i32, i32, vp, vp]
+        lib.woq_hip_probe_empty.restype = i32
+        lib.woq_hip_probe_empty.argtypes = [i64, i32, vp]
         if lib.woq_hip_abi_version() != 1:
             raise RuntimeError("libwoq_hip.so has an unexpected ABI version")
         _lib = lib
