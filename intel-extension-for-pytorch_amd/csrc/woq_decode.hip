@@ -196,6 +196,183 @@ __global__ __launch_bounds__(1024, 8) void woq_decode_kernel(const DecodeArgs a)
   }
 }
 
+// One row (M = 1), the single-stream decode step: the same decomposition with fewer VALU instructions
+// per weight, which is what the kernel above spends its time on once the data has arrived (every wave of
+// a SIMD gets its tiles at about the same time, and their decode then queues on the one VALU).
+//   * the row is converted to fp16 on its way into LDS (the reference's M < 5 path computes in fp16 and
+//     converts bf16 rows the same way, csrc/cpu/aten/utils/woq.h:3076-3079, 3369-3375) and the MFMA is
+//     the fp16 one: the 10-bit fp16 mantissa holds a nibble in place at bits 0..3 AND at bits 4..7 --
+//     0x6400 | q is 1024 + q and 0x5400 | (q << 4) is 64 + q -- so a packed dword becomes the four
+//     operand dwords with one shift and four v_and_or_b32 (5 instructions instead of 7 for 8 weights);
+//   * sum_k x (q - z) = sum_k x (c_k + q) - sum_k (c_k - 128) x - (128 + z) sum_k x with c_k = 1024 or 64
+//     by position: the middle sum is one more MFMA per K chunk against the constants (-896, +64), whose
+//     result is the C input of the weight MFMAs (no VALU instruction at all); the last is the MFMA
+//     against -1 as above;
+//   * every row of the A operand is the one activation row, so every row of D is the result: a lane
+//     scales and accumulates one element per tile instead of four.
+template <bool XBF16, int NTW, bool ONE_ROUND>
+__global__ __launch_bounds__(1024, 8) void woq_decode_m1_kernel(const DecodeArgs a) {
+  constexpr int KPW = kDecodeKPW;
+  constexpr int SLICE = KPW * kTileK4;  // K elements of one wave per round
+  extern __shared__ __align__(16) uint8_t smem[];
+  const int W = a.W;
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+  const int r = lane & 15, c = lane >> 4;
+  const int64_t nt0 = (int64_t)blockIdx.x * NTW;
+
+  uint16_t* sx = (uint16_t*)smem + (size_t)wave * SLICE;                // this wave's fp16 slice of the row
+  float* red = (float*)(smem + (size_t)W * SLICE * sizeof(uint16_t));  // [NTW][16 columns][16 waves]
+
+  // buffer resources over the packed weight and its parameters: a load then takes the resource, one
+  // VGPR offset shared by all loads, a wave-uniform offset in a scalar register and an immediate, so
+  // the address arithmetic of the whole kernel runs on the scalar unit (offsets are 32 bits wide: the
+  // launcher sends larger weights elsewhere); reads past the end return zero
+  const __amdgpu_buffer_rsrc_t wrs = __builtin_amdgcn_make_buffer_rsrc((void*)a.qweight, 0, (int)a.wbytes, 0x00020000);
+  const __amdgpu_buffer_rsrc_t srs = __builtin_amdgcn_make_buffer_rsrc((void*)a.sz, 0, (int)a.szbytes, 0x00020000);
+
+  uint32_t mask_lo, mask_hi, magic_a, magic_b;
+  asm volatile("s_mov_b32 %0, 0x000F000F" : "=s"(mask_lo));
+  asm volatile("s_mov_b32 %0, 0x00F000F0" : "=s"(mask_hi));
+  asm volatile("v_mov_b32 %0, 0x64006400" : "=v"(magic_a));
+  asm volatile("v_mov_b32 %0, 0x54005400" : "=v"(magic_b));
+  // One MFMA chain gives both correction sums: output columns 0..7 see the constant -1 (their D is
+  // -sum x), columns 8..15 the constants -(1024 - 128), -(64 - 128) (their D is -sum (c - 128) x); a lane
+  // takes the sum it does not hold from the lane eight columns over (a rotation inside its row of 16).
+  const bool low_cols = r < 8;
+  const u4 kcorr = low_cols ? u4{0xBC00BC00u, 0xBC00BC00u, 0xBC00BC00u, 0xBC00BC00u}
+                            : u4{0xE300E300u, 0x54005400u, 0xE300E300u, 0x54005400u};
+
+  float acc[NTW];
+#pragma unroll
+  for (int t = 0; t < NTW; ++t) acc[t] = 0.f;
+
+  const int KT = (int)a.KT, KG = (int)a.KG;
+  const int tpg_shift = a.tpg_shift;
+  static_assert(KPW == 2, "two K tiles per wave and round");
+  const int xlane = lane & (KPW * 16 - 1);  // lanes 32..63 mirror 0..31
+  // What the last instructions of the kernel need from the argument block, loaded with the rest of it
+  // and kept in scalar registers: left to itself the compiler reads them behind the barrier, one
+  // dependent scalar load after the other in the only part of the kernel that nothing overlaps.
+  // (pinned behind the first round's requests, so that their own loads do not delay those)
+  uint32_t out_lo = 0, out_hi = 0;
+  int n_cols = 0, plain = 0;
+  const int rounds = ONE_ROUND ? 1 : (KT + W * KPW - 1) / (W * KPW);
+#pragma unroll 1
+  for (int rd = 0; rd < rounds; ++rd) {
+    const int ktw = (rd * W + wave) * KPW;
+    if (!ONE_ROUND && ktw >= KT) break;
+
+    const uint8_t* xbase = (const uint8_t*)a.x + (uint32_t)ktw * (kTileK4 * 2);  // uniform
+    const u4 xs = *(const u4*)(xbase + (uint32_t)xlane * 16u);
+
+    u4 wreg[NTW][KPW];
+    uint32_t szreg[NTW][KPW];
+    const int lane16 = lane * 16, r4 = r * 4;
+    // requested in the order of use: K tile by K tile, row-block by row-block, each tile with its parameters
+#pragma unroll
+    for (int i = 0; i < KPW; ++i) {
+#pragma unroll
+      for (int t = 0; t < NTW; ++t) {
+        const uint32_t nt = (uint32_t)nt0 + t;
+        const int woff = (int)((nt * (uint32_t)KT + (uint32_t)(ktw + i)) * (uint32_t)kTileBytes);
+        const int soff = (int)((nt * (uint32_t)KG + ((uint32_t)(ktw + i) >> tpg_shift)) * (uint32_t)(kTileN * sizeof(uint32_t)));
+        wreg[t][i] = __builtin_amdgcn_raw_buffer_load_b128(wrs, lane16, woff, 2);  // non-temporal
+        szreg[t][i] = __builtin_amdgcn_raw_buffer_load_b32(srs, r4, soff, 0);
+      }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    if (ONE_ROUND || rd == 0) {
+      out_lo = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)a.out);
+      out_hi = __builtin_amdgcn_readfirstlane((uint32_t)((uintptr_t)a.out >> 32));
+      n_cols = __builtin_amdgcn_readfirstlane((int)a.N);
+      plain = __builtin_amdgcn_readfirstlane(
+          (int)(a.fusion == WOQ_HIP_FUSE_NONE && a.bias == nullptr && a.out_dtype == WOQ_HIP_ACT_BF16));
+      asm volatile("" : "+s"(out_lo), "+s"(out_hi), "+s"(n_cols), "+s"(plain));
+    }
+    __builtin_amdgcn_sched_barrier(0);
+
+    u4 xh = xs;
+    if constexpr (XBF16) {
+#pragma unroll
+      for (int v = 0; v < 4; ++v) {
+        const float lo = bitcast<float>(xs[v] << 16), hi = bitcast<float>(xs[v] & 0xFFFF0000u);
+        xh[v] = bitcast<uint32_t>(__builtin_amdgcn_cvt_pkrtz(lo, hi));  // exact for every fp16-normal value
+      }
+    }
+    *(u4*)(sx + xlane * 8) = xh;
+
+#pragma unroll
+    for (int i = 0; i < KPW; ++i) {
+      u4 xa[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) xa[j] = *(const u4*)(sx + i * kTileK4 + c * 32 + j * 8);
+      f4 dk = f4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int j = 0; j < 4; ++j) dk = mfma16<true>(xa[j], kcorr, dk);
+      const float mine = dk[0];
+      const float theirs = bitcast<float>(__builtin_amdgcn_mov_dpp(bitcast<int>(mine), 0x128, 0xf, 0xf, true));  // row_ror:8
+      const float d1 = low_cols ? mine : theirs;                    // -sum x
+      const f4 dc = f4{low_cols ? theirs : mine, 0.f, 0.f, 0.f};   // -sum (c - 128) x; rows 1..3 are not used
+#pragma unroll
+      for (int t = 0; t < NTW; ++t) {
+        f4 dw = dc;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const uint32_t d = wreg[t][i][j], d8 = d >> 8;
+          u4 bop;
+          bop[0] = v_and_or(d, mask_lo, magic_a);
+          bop[1] = v_and_or(d, mask_hi, magic_b);
+          bop[2] = v_and_or(d8, mask_lo, magic_a);
+          bop[3] = v_and_or(d8, mask_hi, magic_b);
+          dw = mfma16<true>(xa[j], bop, dw);
+        }
+        // dw = sum x (c + q) - sum (c - 128) x, d1 = -sum x;  group term = s * (dw + (128 + z) * d1)
+        const float tsum = fma_f16hi(d1, szreg[t][i], dw[0]);
+        acc[t] = fma_f16lo(tsum, szreg[t][i], acc[t]);
+      }
+    }
+  }
+
+  // the partial sums of waves that do not exist read as zero
+  if (W < 16 && threadIdx.x < NTW * 16) {
+    for (int w = W; w < 16; ++w) red[threadIdx.x * 16 + w] = 0.f;
+  }
+  // every lane column holds the same sums; column 0 publishes them
+  if (c == 0) {
+#pragma unroll
+    for (int t = 0; t < NTW; ++t) red[(t * 16 + r) * 16 + wave] = acc[t];
+  }
+  __syncthreads();
+
+  if (threadIdx.x < NTW * 16) {
+    const int col = threadIdx.x & 15, t = threadIdx.x >> 4;
+    const int n = ((int)nt0 + t) * kTileN + col;
+    // the 16 partial sums of this output in four reads, added pairwise in a fixed order
+    const f4* mine = (const f4*)(red + threadIdx.x * 16);
+    const f4 p0 = mine[0], p1 = mine[1], p2 = mine[2], p3 = mine[3];
+    const float s = (((p0[0] + p0[1]) + (p0[2] + p0[3])) + ((p1[0] + p1[1]) + (p1[2] + p1[3]))) +
+                    (((p2[0] + p2[1]) + (p2[2] + p2[3])) + ((p3[0] + p3[1]) + (p3[2] + p3[3])));
+    if (n < n_cols) {
+      if (plain) {
+        typedef __attribute__((address_space(1))) uint16_t* global_u16_ptr;  // a global store, not a flat one
+        global_u16_ptr out = (global_u16_ptr)(((uintptr_t)out_hi << 32) | out_lo);
+        out[n] = f32_to_bf16_bits((float)(_Float16)s);
+      } else {
+        Epilogue ep{a.bias, a.fusion, a.other0, a.other1, a.out, a.out_dtype, a.x_dtype, a.N};
+        epilogue_store<kRegimeF16>(ep, 0, n, s);
+      }
+    }
+  }
+}
+
+template <bool XBF16, int NTW, bool ONE_ROUND>
+static int launch_decode_m1_cfg(const DecodeArgs& a, hipStream_t st) {
+  const size_t smem = (size_t)NTW * 16 * 16 * sizeof(float) + (size_t)a.W * kDecodeKPW * kTileK4 * sizeof(uint16_t);
+  woq_decode_m1_kernel<XBF16, NTW, ONE_ROUND><<<(unsigned)((a.NT + NTW - 1) / NTW), a.W * 64, smem, st>>>(a);
+  return check_launch("woq_decode_m1_kernel");
+}
+
 template <bool XF16, int NTW, int MAXM, bool ONE_ROUND>
 static int launch_decode_cfg(const DecodeArgs& a, hipStream_t st) {
   const size_t smem = (size_t)NTW * a.W * 16 * sizeof(f4) +
@@ -238,11 +415,21 @@ int launch_decode(const FpArgs& f, const uint32_t* sz, hipStream_t st) {
   a.W = (int)w;
   const bool xf16 = f.x_dtype == WOQ_HIP_ACT_FP16;
   const bool two = f.NT >= 512 && f.NT % 2 == 0;
-  const bool one_row = f.M == 1;
+  // the single-row kernel addresses the weight and its parameters with 32-bit offsets
+  const int64_t wbytes = f.NT * f.KT * kTileBytes, szbytes = f.NT * f.KG * kTileN * (int64_t)sizeof(uint32_t);
+  const bool one_row = f.M == 1 && wbytes < ((int64_t)1 << 32) && szbytes < ((int64_t)1 << 32);
+  a.wbytes = (uint32_t)wbytes;
+  a.szbytes = (uint32_t)szbytes;
   const bool one_round = f.KT == (int64_t)a.W * kDecodeKPW;
-#define WOQ_DECODE(XF, NTW)                                                                             \
-  (one_row ? (one_round ? launch_decode_cfg<XF, NTW, 1, true>(a, st) : launch_decode_cfg<XF, NTW, 1, false>(a, st)) \
-           : (one_round ? launch_decode_cfg<XF, NTW, 4, true>(a, st) : launch_decode_cfg<XF, NTW, 4, false>(a, st)))
+  if (one_row) {
+#define WOQ_DECODE_M1(XB, NTW) \
+  (one_round ? launch_decode_m1_cfg<XB, NTW, true>(a, st) : launch_decode_m1_cfg<XB, NTW, false>(a, st))
+    if (xf16) return two ? WOQ_DECODE_M1(false, 2) : WOQ_DECODE_M1(false, 1);
+    return two ? WOQ_DECODE_M1(true, 2) : WOQ_DECODE_M1(true, 1);
+#undef WOQ_DECODE_M1
+  }
+#define WOQ_DECODE(XF, NTW) \
+  (one_round ? launch_decode_cfg<XF, NTW, 4, true>(a, st) : launch_decode_cfg<XF, NTW, 4, false>(a, st))
   if (xf16) return two ? WOQ_DECODE(true, 2) : WOQ_DECODE(true, 1);
   return two ? WOQ_DECODE(false, 2) : WOQ_DECODE(false, 1);
 #undef WOQ_DECODE

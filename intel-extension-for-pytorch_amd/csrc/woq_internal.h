@@ -81,6 +81,7 @@ struct DecodeArgs {
   int out_dtype;
   int W;
   int tpg_shift;  // log2(G / 128)
+  uint32_t wbytes, szbytes;  // extents of qweight and sz: the single-row kernel addresses them with 32-bit offsets
 };
 bool decode_kernel_applies(const FpArgs& f, int wbits, int regime, const uint32_t* sz);
 int launch_decode(const FpArgs& f, const uint32_t* sz, hipStream_t st);
