@@ -77,11 +77,12 @@ __global__ __launch_bounds__(1024, 8) void woq_decode_kernel(const DecodeArgs a)
 #pragma unroll
   for (int t = 0; t < NTW; ++t) acc[t] = f4{0.f, 0.f, 0.f, 0.f};
 
-  const int NT = (int)a.NT, KT = (int)a.KT, KG = (int)a.KG;
+  const int KT = (int)a.KT, KG = (int)a.KG;
   const int tpg_shift = a.tpg_shift;  // log2(tiles per group)
   const int xlane = lane & (KPW * 16 - 1);  // lanes 32..63 mirror 0..31
-  (void)NT;
   const int xrow = r < MAXM ? r : 0;
+  const __amdgpu_buffer_rsrc_t wrs = __builtin_amdgcn_make_buffer_rsrc((void*)a.qweight, 0, (int)a.wbytes, 0x00020000);
+  const __amdgpu_buffer_rsrc_t srs = __builtin_amdgcn_make_buffer_rsrc((void*)a.sz, 0, (int)a.szbytes, 0x00020000);
 
   // 32-bit offsets from uniform base pointers keep the per-lane address state in one VGPR each
   // (the packed weight, its parameters and the activations are each far below 4 GiB)
@@ -105,21 +106,21 @@ __global__ __launch_bounds__(1024, 8) void woq_decode_kernel(const DecodeArgs a)
     }
 
     // ---- the weight stream of this round, in the order it is consumed: one KiB tile per load,
-    // all in flight together; uniform bases + one per-lane offset ----
+    // all in flight together.  Buffer loads: the resource, one VGPR offset shared by every load and a
+    // wave-uniform 32-bit offset in a scalar register, so the address arithmetic runs on the scalar
+    // unit (decode_kernel_applies keeps weights of 4 GiB and more away) ----
     u4 wreg[NTW][KPW];
     uint32_t szreg[NTW][KPW];
+    const int lane16 = lane * 16, r4 = r * 4;
 #pragma unroll
     for (int i = 0; i < KPW; ++i) {
-      const int kt = ktw + i;
-      int g = kt >> tpg_shift;
-      g = g < KG ? g : KG - 1;
 #pragma unroll
       for (int t = 0; t < NTW; ++t) {
-        const size_t nt = (size_t)nt0 + t;
-        const uint8_t* wb = a.qweight + (nt * KT + kt) * kTileBytes;                      // uniform
-        const uint8_t* sb = (const uint8_t*)a.sz + (nt * KG + g) * (kTileN * sizeof(uint32_t));  // uniform
-        wreg[t][i] = __builtin_nontemporal_load((const u4*)(wb + (uint32_t)lane * 16u));
-        szreg[t][i] = *(const uint32_t*)(sb + (uint32_t)r * 4u);
+        const uint32_t nt = (uint32_t)nt0 + t;
+        const int woff = (int)((nt * (uint32_t)KT + (uint32_t)(ktw + i)) * (uint32_t)kTileBytes);
+        const int soff = (int)((nt * (uint32_t)KG + ((uint32_t)(ktw + i) >> tpg_shift)) * (uint32_t)(kTileN * sizeof(uint32_t)));
+        wreg[t][i] = __builtin_amdgcn_raw_buffer_load_b128(wrs, lane16, woff, 2);  // non-temporal
+        szreg[t][i] = __builtin_amdgcn_raw_buffer_load_b32(srs, r4, soff, 0);
       }
     }
 
@@ -389,6 +390,8 @@ static int launch_decode_cfg(const DecodeArgs& a, hipStream_t st) {
 
 bool decode_kernel_applies(const FpArgs& f, int wbits, int regime, const uint32_t* sz) {
   const int64_t tpg = f.G / kTileK4;
+  // the kernels address the packed weight and its parameters with 32-bit offsets
+  if (f.NT * f.KT * kTileBytes >= ((int64_t)1 << 32) || f.NT * f.KG * kTileN * 4 >= ((int64_t)1 << 32)) return false;
   return sz != nullptr && wbits == 4 && regime == kRegimeF16 && f.M <= 4 && (f.G % kTileK4) == 0 &&
          (tpg & (tpg - 1)) == 0 && (f.K % (kDecodeKPW * kTileK4)) == 0 && (f.x_dtype == WOQ_HIP_ACT_BF16 || f.x_dtype == WOQ_HIP_ACT_FP16);
 }
@@ -415,11 +418,9 @@ int launch_decode(const FpArgs& f, const uint32_t* sz, hipStream_t st) {
   a.W = (int)w;
   const bool xf16 = f.x_dtype == WOQ_HIP_ACT_FP16;
   const bool two = f.NT >= 512 && f.NT % 2 == 0;
-  // the single-row kernel addresses the weight and its parameters with 32-bit offsets
-  const int64_t wbytes = f.NT * f.KT * kTileBytes, szbytes = f.NT * f.KG * kTileN * (int64_t)sizeof(uint32_t);
-  const bool one_row = f.M == 1 && wbytes < ((int64_t)1 << 32) && szbytes < ((int64_t)1 << 32);
-  a.wbytes = (uint32_t)wbytes;
-  a.szbytes = (uint32_t)szbytes;
+  a.wbytes = (uint32_t)(f.NT * f.KT * kTileBytes);  // below 4 GiB (decode_kernel_applies)
+  a.szbytes = (uint32_t)(f.NT * f.KG * kTileN * (int64_t)sizeof(uint32_t));
+  const bool one_row = f.M == 1;
   const bool one_round = f.KT == (int64_t)a.W * kDecodeKPW;
   if (one_row) {
 #define WOQ_DECODE_M1(XB, NTW) \
