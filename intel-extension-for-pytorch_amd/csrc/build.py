@@ -31,6 +31,37 @@ def lib_path():
     return os.path.join(LIB_DIR, "libwoq_hip.so")
 
 
+def torch_lib_path():
+    return os.path.join(LIB_DIR, "libwoq_torch.so")
+
+
+def build_torch_binding(verbose=True, incremental=False):
+    """g++ on torch_binding.cpp (host code only: the operator / custom-class registrations over the C ABI)
+    -> ../lib/libwoq_torch.so, linked against libwoq_hip.so beside it and the libraries of the installed
+    PyTorch (ROCm build).  No hipify step: the source is written against the HIP headers of PyTorch."""
+    import torch
+    from torch.utils import cpp_extension
+
+    src = os.path.join(HERE, "torch_binding.cpp")
+    out = torch_lib_path()
+    if incremental and os.path.exists(out) and os.path.getmtime(out) > max(
+            os.path.getmtime(src), os.path.getmtime(os.path.join(os.path.dirname(os.path.dirname(HERE)), "include", "woq_hip.h"))):
+        return out
+    tlib = os.path.join(os.path.dirname(torch.__file__), "lib")
+    cmd = ["g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-D__HIP_PLATFORM_AMD__=1", "-DUSE_ROCM=1",
+           f"-D_GLIBCXX_USE_CXX11_ABI={int(torch._C._GLIBCXX_USE_CXX11_ABI)}", "-Wno-deprecated-declarations"]
+    for inc in cpp_extension.include_paths() + ["/opt/rocm/include"]:
+        cmd += ["-isystem", inc]
+    cmd += [src, "-o", out, f"-L{LIB_DIR}", "-lwoq_hip", f"-L{tlib}", "-lc10", "-lc10_hip", "-ltorch_cpu", "-ltorch",
+            "-lamdhip64", "-Wl,-rpath,$ORIGIN", f"-Wl,-rpath,{tlib}"]
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    if res.returncode != 0:
+        raise RuntimeError("g++ failed for torch_binding.cpp:\n" + res.stderr[-6000:])
+    if verbose:
+        print("built", out)
+    return out
+
+
 def _stale(src, obj):
     if not os.path.exists(obj):
         return True
@@ -65,6 +96,7 @@ def build(jobs=4, verbose=True, incremental=False):
         raise RuntimeError("link failed:\n" + res.stderr)
     if verbose:
         print("built", lib_path())
+    build_torch_binding(verbose, incremental)
     return lib_path()
 
 

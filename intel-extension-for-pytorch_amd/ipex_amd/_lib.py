@@ -150,6 +150,32 @@ def load():
     return _lib
 
 
+TORCH_LIB_PATH = os.path.join(os.path.dirname(_HERE), "lib", "libwoq_torch.so")
+_torch_binding_loaded = False
+
+
+def load_torch_binding():
+    """Loads libwoq_torch.so, whose static initialisers register the ``torch_ipex`` / ``ipex_prepack``
+    operators and the ``ipex_prepack.WoqLinearOpContext`` custom class; raises if it has not been built."""
+    global _torch_binding_loaded
+    if _torch_binding_loaded:
+        return
+    load()  # libwoq_hip.so first: the binding links against it
+    with _lock:
+        if _torch_binding_loaded:
+            return
+        if not os.path.exists(TORCH_LIB_PATH):
+            raise RuntimeError(
+                f"{TORCH_LIB_PATH} is missing: build it with "
+                "`python intel-extension-for-pytorch_amd/csrc/build.py` (needs hipcc and g++); "
+                "there is no Python or CPU fallback for the WOQ linear operators."
+            )
+        import torch
+
+        torch.ops.load_library(TORCH_LIB_PATH)
+        _torch_binding_loaded = True
+
+
 def last_kernel():
     """Name of the kernel this thread launched last through the library."""
     return load().woq_hip_last_kernel().decode("ascii")

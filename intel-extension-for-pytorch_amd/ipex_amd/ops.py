@@ -1,8 +1,10 @@
 """Operator boundary: the ``torch_ipex`` / ``ipex_prepack`` ops and the prepack context.
 
-Same op names, argument order and error behaviour as the reference
+The operators and the TorchScript custom class ``torch.classes.ipex_prepack.WoqLinearOpContext`` are
+registered by the C++ binding (csrc/torch_binding.cpp -> lib/libwoq_torch.so), loaded by ``register()``:
+same op names, argument order and error behaviour as the reference
 (csrc/cpu/aten/Linear.cpp:1013-1112, csrc/cpu/jit/cpu/kernels/RegisterOpContextClass.cpp:127-223),
-registered for tensors that live on the GPU:
+for tensors that live on the GPU:
 
     torch.ops.torch_ipex.ipex_woq_linear(x, ctx.get_data_handle())
     torch.ops.torch_ipex.woq_linear_{gelu,new_gelu,relu,silu}(x, handle)
@@ -12,10 +14,11 @@ registered for tensors that live on the GPU:
     torch.ops.ipex_prepack.weight_only_qlinear_prepack_int4(...) -> WoqLinearOpContext
     torch.ops.ipex_prepack.woq_linear_pack_weight(...) / woq_linear_unpack_weight(...)
 
-The context is a Python object here (the reference's is a TorchScript custom class); its
-``get_data_handle()`` returns a 1-element CPU int64 tensor, as the reference's does
-(csrc/cpu/jit/cpu/kernels/OpContext.cpp:396-400), and the ops resolve it through a registry
-of live contexts, so a stale handle raises instead of dereferencing freed memory.
+This module adds the mixture-of-experts ops on top of them, and keeps ``WoqLinearOpContext``, a
+Python twin of the custom class over the same C ABI through ctypes: the vehicle of the C-ABI tests
+(``run`` takes the library's debugging options: fp32 accumulators, forced kernels, block sums).  Its
+handles name Python objects and are understood by the functions of this module only, not by
+``torch.ops``.
 """
 import contextlib
 import ctypes
@@ -610,12 +613,31 @@ def woq_linear(
 
 
 # ---- mixture of experts over WOQ linears ---------------------------------------------------------
+def _is_python_context(ctx):
+    return isinstance(ctx, WoqLinearOpContext)
+
+
+def _run_context(ctx, x, fusion=_lib.FUSE_NONE, others=()):
+    """One linear of an expert: ``ctx`` is a ``torch.classes.ipex_prepack.WoqLinearOpContext`` (the
+    registered operators, by handle) or the ctypes twin of this module."""
+    if _is_python_context(ctx):
+        return ctx.run(x, fusion=fusion, others=others)
+    h = ctx if isinstance(ctx, torch.Tensor) else ctx.get_data_handle()
+    if fusion == _lib.FUSE_NONE:
+        return torch.ops.torch_ipex.ipex_woq_linear(x, h)
+    if fusion == _lib.FUSE_SILU:
+        return torch.ops.torch_ipex.woq_linear_silu(x, h)
+    if fusion == _lib.FUSE_MUL:
+        return torch.ops.torch_ipex.woq_linear_mul(x, h, list(others))
+    raise RuntimeError(f"unexpected post-op 0x{fusion:x} in an expert")
+
+
 def _moe_expert(hidden_states, top_x, idx, gate, up, down, routing_weights, output):
     """One expert: gather its tokens, down(up(x) * silu(gate(x))), weighted accumulation
     (mixtral_moe_woq_kernl_impl, csrc/cpu/aten/kernels/MoEKrnl.cpp:254-284)."""
     cur = _kernels.moe_gather_rows(hidden_states, top_x)
-    act = gate.run(cur, fusion=_lib.FUSE_SILU)
-    cur = down.run(up.run(cur, fusion=_lib.FUSE_MUL, others=(act,)))
+    act = _run_context(gate, cur, _lib.FUSE_SILU)
+    cur = _run_context(down, _run_context(up, cur, _lib.FUSE_MUL, (act,)))
     return _kernels.moe_scale_add_rows(output, cur, routing_weights, top_x, idx)
 
 
@@ -633,10 +655,7 @@ def mixtral_moe_woq(hidden_states, top_x, idx, gate_wei, up_wei, down_wei, routi
     if top_x.shape[0] == 0:
         return output
     dev = hidden_states.device
-    return _moe_expert(
-        hidden_states, top_x.to(dev), idx.to(dev), _context_from_handle(gate_wei), _context_from_handle(up_wei),
-        _context_from_handle(down_wei), routing_weights, output,
-    )
+    return _moe_expert(hidden_states, top_x.to(dev), idx.to(dev), gate_wei, up_wei, down_wei, routing_weights, output)
 
 
 def deepseek_moe_woq(hidden_states, topk_ids, gate_ctx, up_ctx, down_ctx, routing_weights, is_distributed):
@@ -675,57 +694,20 @@ _libs = []
 
 
 def register():
-    """Registers the ops under ``torch.ops.torch_ipex`` / ``torch.ops.ipex_prepack`` (idempotent)."""
+    """Loads the C++ binding, which registers the operators and the custom class under
+    ``torch.ops.torch_ipex`` / ``torch.ops.ipex_prepack`` / ``torch.classes.ipex_prepack``, and adds the
+    mixture-of-experts ops (idempotent).  Raises if the binding has not been built."""
     global _registered
     if _registered:
         return
+    _lib.load_torch_binding()
     tl = torch.library.Library("torch_ipex", "FRAGMENT")
     _libs.append(tl)
-    key = "CompositeExplicitAutograd"
-    tl.define("ipex_woq_linear(Tensor input, Tensor W_prepack) -> Tensor")
-    tl.impl("ipex_woq_linear", ipex_woq_linear, key)
-    for name, fn in (
-        ("woq_linear_gelu", woq_linear_gelu),
-        ("woq_linear_new_gelu", woq_linear_new_gelu),
-        ("woq_linear_relu", woq_linear_relu),
-        ("woq_linear_silu", woq_linear_silu),
-    ):
-        tl.define(f"{name}(Tensor input, Tensor W_prepack) -> Tensor")
-        tl.impl(name, fn, key)
-    for name, fn in (
-        ("woq_linear_add", woq_linear_add),
-        ("woq_linear_add_add", woq_linear_add_add),
-        ("woq_linear_mul", woq_linear_mul),
-    ):
-        tl.define(f"{name}(Tensor input, Tensor W_prepack, Tensor[] others) -> Tensor")
-        tl.impl(name, fn, key)
-    tl.define(
-        "woq_linear(Tensor input, Tensor qweight, str weight_dtype, int[] weight_shape, "
-        "Tensor[] weight_scales, Tensor[]? weight_zeros, Tensor[]? bias, Tensor? g_idx, "
-        "int group_size, int lowp_mode, int act_quant_mode, Tensor? compensation=None) -> Tensor"
-    )
-    tl.impl("woq_linear", woq_linear, key)
     tl.define(
         "mixtral_moe_woq(Tensor hidden_states, Tensor top_x, Tensor idx, Tensor gate_wei, Tensor up_wei, "
         "Tensor down_wei, Tensor routing_weights, Tensor(a!) output, bool is_distributed) -> Tensor(a!)"
     )
-    tl.impl("mixtral_moe_woq", mixtral_moe_woq, key)
-    # takes lists of context objects: attached like the prepack entry points below
+    tl.impl("mixtral_moe_woq", mixtral_moe_woq, "CompositeExplicitAutograd")
+    # takes lists of context objects, which no operator schema can name
     setattr(torch.ops.torch_ipex, "deepseek_moe_woq", deepseek_moe_woq)
-
-    pl = torch.library.Library("ipex_prepack", "FRAGMENT")
-    _libs.append(pl)
-    pl.define(
-        "woq_linear_pack_weight(Tensor W, str W_dtype, int[] W_shape, Tensor scales, Tensor? zero_points, "
-        "Tensor? B, Tensor? g_idx, int group_size, int lowp_mode) -> (Tensor, Tensor[], Tensor[]?, Tensor[]?, Tensor?)"
-    )
-    pl.impl("woq_linear_pack_weight", woq_linear_pack_weight, key)
-    pl.define("woq_linear_unpack_weight(Tensor W, str W_dtype, int[] W_shape, int lowp_mode) -> Tensor")
-    pl.impl("woq_linear_unpack_weight", woq_linear_unpack_weight, key)
-    # The two context-returning entry points cannot be torch.library ops (their result is a
-    # Python object); they are attached to the same namespace so that the reference call sites
-    # `torch.ops.ipex_prepack.weight_only_qlinear_prepack[_int4](...)` work unchanged.
-    ns = torch.ops.ipex_prepack
-    setattr(ns, "weight_only_qlinear_prepack", weight_only_qlinear_prepack)
-    setattr(ns, "weight_only_qlinear_prepack_int4", weight_only_qlinear_prepack_int4)
     _registered = True

@@ -55,3 +55,25 @@ def make_context(case, lowp_mode, act_quant_mode=-1, device="cuda", cache=False)
         act_quant_mode,
         cache,
     )
+
+
+def make_torch_context(case, lowp_mode, act_quant_mode=-1, device="cuda", cache=False, g_idx=None):
+    """The registered custom class (torch.classes.ipex_prepack.WoqLinearOpContext) for a synthetic case,
+    made by the registered prepack operator."""
+    import torch
+    import ipex_amd  # noqa: F401
+
+    return torch.ops.ipex_prepack.weight_only_qlinear_prepack(
+        case["qweight"].to(device),
+        case["weight_dtype"],
+        [case["N"], case["K"]],
+        case["scales"].to(device),
+        None if case["zeros"] is None else case["zeros"].to(device),
+        None if case["bias"] is None else case["bias"].to(device),
+        g_idx,
+        None,
+        case["group_size"],
+        lowp_mode,
+        act_quant_mode,
+        cache,
+    )

@@ -185,10 +185,10 @@ def test_context_pickle_roundtrip(cuda):
 
 def test_stale_handle_raises(cuda):
     from ipex_amd.utils import synthetic
-    from helpers import make_context
+    from helpers import make_torch_context
 
     case = synthetic.make_int4_case(31, 1, 256, 32, 128)
-    ctx = make_context(case, 2)
+    ctx = make_torch_context(case, 2)
     handle = ctx.get_data_handle()
     x = case["x"].to(cuda)
     torch.ops.torch_ipex.ipex_woq_linear(x, handle)
@@ -266,10 +266,10 @@ def test_weight_cache_for_large_batch(cuda):
 
 def test_fused_ops_through_torch_ops(cuda):
     from ipex_amd.utils import synthetic
-    from helpers import make_context
+    from helpers import make_torch_context
 
     case = synthetic.make_int4_case(35, 6, 256, 48, 128, bias=True)
-    ctx = make_context(case, 2)
+    ctx = make_torch_context(case, 2)
     h = ctx.get_data_handle()
     x = case["x"].to(cuda)
     base = torch.ops.torch_ipex.ipex_woq_linear(x, h)
@@ -475,3 +475,131 @@ def test_mixtral_moe_woq_single_expert_and_errors(cuda):
     ctxs = [[m[0]._op_context] for m in (gate, up, down)]
     with pytest.raises(RuntimeError, match="expert ids"):
         torch.ops.torch_ipex.deepseek_moe_woq(hidden, torch.full((T, 1), 3), ctxs[0], ctxs[1], ctxs[2], rw, False)
+
+
+# ---------------------------------------------------------------------------------------------
+# the C++ binding: registered operators and the TorchScript custom class
+# ---------------------------------------------------------------------------------------------
+def test_custom_class_method_surface_and_pickle(cuda):
+    """torch.classes.ipex_prepack.WoqLinearOpContext: the twelve methods of the reference's class
+    (RegisterOpContextClass.cpp:127-173) and its pickle (plain format out, re-prepacked on load)."""
+    from ipex_amd.utils import synthetic
+    from helpers import make_context, make_torch_context
+
+    case = synthetic.make_int4_case(60, 5, 512, 80, 128, bias=True)
+    ctx = make_torch_context(case, 2)
+    assert "WoqLinearOpContext" in str(type(ctx)) or "ScriptObject" in str(type(ctx))
+    assert ctx.get_weight_shape() == [80, 512]
+    assert torch.equal(ctx.to_public(ctx.get_weight()).cpu(), case["qweight"])
+    assert torch.equal(ctx.pack(case["qweight"].to(cuda)), ctx.get_weight())
+    assert torch.equal(ctx.get_scales().cpu(), case["scales"]) and ctx.get_scales().shape == (80, 4)
+    assert torch.equal(ctx.get_zero_points().cpu(), case["zeros"])
+    assert torch.equal(ctx.get_bias().cpu(), case["bias"])
+    assert ctx.get_g_idx() is None and ctx.get_cached_weight() is None and ctx.get_cached_compensation() is None
+    h = ctx.get_data_handle()
+    assert h.dtype == torch.int64 and h.numel() == 1 and h.device.type == "cpu"
+    x = case["x"].to(cuda)
+    y0 = torch.ops.torch_ipex.ipex_woq_linear(x, h)
+    # same kernels as the ctypes twin: bit-identical
+    assert torch.equal(y0, make_context(case, 2).run(x))
+    ctx2 = pickle.loads(pickle.dumps(ctx))
+    assert ctx2.get_data_handle().item() != h.item()
+    assert torch.equal(torch.ops.torch_ipex.ipex_woq_linear(x, ctx2.get_data_handle()), y0)
+    # load_from_ctx: the state of another context under the old handle
+    other = make_torch_context(synthetic.make_int4_case(61, 5, 512, 80, 128, bias=True), 2)
+    y_other = torch.ops.torch_ipex.ipex_woq_linear(x, other.get_data_handle())
+    ctx.load_from_ctx(other)
+    assert ctx.get_data_handle().item() == h.item()
+    assert torch.equal(torch.ops.torch_ipex.ipex_woq_linear(x, h), y_other)
+
+
+@pytest.mark.parametrize("weight_dtype,bias", [("INT8", True), ("INT4", False)])
+@pytest.mark.parametrize("M,K,N", [(3, 31 * 8, 31), (4, 4096, 4080), (70, 1024, 512)])
+def test_jit_trace_save_load(cuda, tmp_path, weight_dtype, bias, M, K, N):
+    """As the reference's test_weight_only_quantization_jit_save_load
+    (tests/cpu/test_quantization_default_recipe.py:453-502): trace the converted model, freeze, save,
+    load, compare.  The loaded module owns a context re-made from the pickled plain format."""
+    import ipex_amd as ipex
+
+    q = ipex.quantization
+    torch.manual_seed(5)
+    model = torch.nn.Sequential(torch.nn.Linear(K, N, bias=bias)).to(torch.bfloat16).eval().to(cuda)
+    x = torch.rand(M, K, device=cuda).to(torch.bfloat16)
+    qmap = q.get_weight_only_quant_qconfig_mapping(weight_dtype=getattr(q.WoqWeightDtype, weight_dtype),
+                                                   lowp_mode=q.WoqLowpMode.BF16)
+    with torch.no_grad():
+        converted = q.convert(q.prepare(model, qmap, inplace=False), inplace=False)
+        want = converted(x)
+        traced = torch.jit.freeze(torch.jit.trace(converted, x))
+        path = str(tmp_path / "woq.pt")
+        traced.save(path)
+        loaded = torch.jit.load(path)
+        assert torch.equal(traced(x), want)
+        assert torch.equal(loaded(x), want)
+        # the loaded graph calls the operator with a handle taken at run time, not a baked-in one
+        assert "ipex_woq_linear" in str(loaded.graph) or "ipex_woq_linear" in str(loaded.inlined_graph)
+        del converted, traced
+        assert torch.equal(loaded(x), want)
+
+
+def test_autocast_casts_the_input_only(cuda):
+    """AutocastCUDA (csrc/cpu/aten/Linear.cpp:874-883): fp32 rows under autocast(bf16) run as bf16 rows."""
+    from ipex_amd.utils import synthetic
+    from helpers import make_torch_context
+
+    case = synthetic.make_int4_case(62, 9, 512, 96, 128, bias=True)
+    ctx = make_torch_context(case, 2)
+    h = ctx.get_data_handle()
+    x32 = case["x"].to(cuda).float()
+    with torch.autocast("cuda", dtype=torch.bfloat16):
+        y = torch.ops.torch_ipex.ipex_woq_linear(x32, h)
+        ys = torch.ops.torch_ipex.woq_linear_silu(x32, h)
+    assert y.dtype == torch.bfloat16
+    assert torch.equal(y, torch.ops.torch_ipex.ipex_woq_linear(x32.bfloat16(), h))
+    assert torch.equal(ys, torch.ops.torch_ipex.woq_linear_silu(x32.bfloat16(), h))
+    # without autocast the fp32 rows are computed in fp32
+    assert torch.ops.torch_ipex.ipex_woq_linear(x32, make_torch_context(case, 0).get_data_handle()).dtype == torch.float32
+
+
+@pytest.mark.parametrize("N,K,G", [(64, 256, 64), (33, 512, 128), (16, 128, -1), (80, 1024, 32)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+def test_dequantize_nf4_op(cuda, N, K, G, dtype):
+    """torch_ipex::dequantize_nf4 (csrc/cpu/aten/Linear.cpp:804-811, test
+    tests/cpu/test_quantization_default_recipe.py:2230-2261): table[code] * scale against the oracle's
+    table, bit-exact in fp32 and after one rounding in the 16-bit types."""
+    import numpy as np
+
+    from oracle import woq_oracle as O
+
+    g = torch.Generator().manual_seed(N + K)
+    codes = torch.randint(0, 256, (N, K // 2), dtype=torch.uint8, generator=g)
+    KG = (K + G - 1) // G if G > 0 else 1
+    scales = (0.02 + torch.rand(N, KG, generator=g)).float()
+    got = torch.ops.torch_ipex.dequantize_nf4(codes.to(cuda), scales.to(cuda) if G > 0 else scales.reshape(N).to(cuda), G, dtype)
+    assert got.dtype == dtype and tuple(got.shape) == (N, K)
+    want = O.dequantize_woq_weight(codes.numpy(), N, K, scales.numpy(), None, O.WOQ_DTYPE_NF4, G)
+    if dtype == torch.float32:
+        assert np.array_equal(got.cpu().numpy(), want)
+    else:
+        assert torch.equal(got.cpu(), torch.from_numpy(want).to(dtype))
+    with pytest.raises(RuntimeError, match="GPU"):
+        torch.ops.torch_ipex.dequantize_nf4(codes, scales, G, dtype)
+
+
+def test_moe_over_registered_contexts(cuda):
+    """deepseek_moe_woq over lists of the registered custom class equals the same layer over the ctypes twins."""
+    from ipex_amd.utils import synthetic
+    from helpers import make_context, make_torch_context
+
+    T, H, I, E, topk = 12, 256, 512, 4, 2
+    g = torch.Generator().manual_seed(9)
+    hidden = torch.randn(T, H, generator=g).bfloat16().to(cuda)
+    ids = torch.stack([torch.randperm(E, generator=g)[:topk] for _ in range(T)]).to(cuda)
+    rw = torch.rand(T, topk, generator=g).bfloat16().to(cuda)
+    cases = [[synthetic.make_int4_case(70 + 3 * e + j, 1, H if j < 2 else I, I if j < 2 else H, 128) for e in range(E)]
+             for j in range(3)]
+    py = [[make_context(c, 2) for c in row] for row in cases]
+    cc = [[make_torch_context(c, 2) for c in row] for row in cases]
+    want = torch.ops.torch_ipex.deepseek_moe_woq(hidden, ids, py[0], py[1], py[2], rw, False)
+    got = torch.ops.torch_ipex.deepseek_moe_woq(hidden, ids, cc[0], cc[1], cc[2], rw, False)
+    assert torch.equal(got, want)

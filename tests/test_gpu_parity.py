@@ -11,7 +11,7 @@ import numpy as np
 import pytest
 import torch
 
-from helpers import bf16_ulp_diff, case_np, make_context, max_abs, rel_l2, to_np_f32
+from helpers import bf16_ulp_diff, case_np, make_context, make_torch_context, max_abs, rel_l2, to_np_f32
 from oracle import woq_oracle as O
 
 pytestmark = pytest.mark.gpu
@@ -1482,7 +1482,7 @@ def test_activation_dtypes_shapes_and_layouts(cuda, idx, act, lowp, lead, K, N, 
     M = int(np.prod(lead))
     case = _synthetic().make_int4_case(300 + idx, M, K, N, G, bias=(idx % 2 == 0))
     x2 = case["x"].float().to(tdt)  # values representable in bf16 whatever the dtype
-    ctx = make_context(case, lowp)
+    ctx = make_torch_context(case, lowp)
     xg = x2.cuda()
     if layout == "strided_rows":
         wide = torch.zeros(M, K + 8, dtype=tdt, device=cuda)
@@ -1534,7 +1534,7 @@ def test_fp32_compute(cuda, kind, M, K, N, G, bias):
             case["zeros"] = None
     gen = torch.Generator().manual_seed(413)
     x = torch.randn(M, K, generator=gen)  # genuine fp32 values, not bf16-representable ones
-    ctx = make_context(case, O.LOWP_NONE)
+    ctx = make_torch_context(case, O.LOWP_NONE)
     y = torch.ops.torch_ipex.ipex_woq_linear(x.cuda(), ctx.get_data_handle())
     assert y.dtype == torch.float32 and tuple(y.shape) == (M, N)
     c = case_np(case)

@@ -238,6 +238,14 @@ def test_ops_are_registered_with_reference_schemas():
             getattr(torch.ops.torch_ipex, name).default._schema
         )
     assert hasattr(torch.ops.torch_ipex, "woq_linear")
+    assert "dequantize_nf4(Tensor t, Tensor scales, int group_size, ScalarType out_dtype) -> Tensor" in str(
+        torch.ops.torch_ipex.dequantize_nf4.default._schema)
+    # registered by the C++ binding, with the custom class the prepack operators return
+    assert "__torch__.torch.classes.ipex_prepack.WoqLinearOpContext" in str(
+        torch.ops.ipex_prepack.weight_only_qlinear_prepack.default._schema)
+    assert torch.classes.ipex_prepack.WoqLinearOpContext is not None
+    assert torch._C._dispatch_has_kernel_for_dispatch_key("torch_ipex::ipex_woq_linear", "CUDA")
+    assert torch._C._dispatch_has_kernel_for_dispatch_key("torch_ipex::ipex_woq_linear", "AutocastCUDA")
     for name in ("weight_only_qlinear_prepack", "weight_only_qlinear_prepack_int4", "woq_linear_pack_weight",
                  "woq_linear_unpack_weight"):
         assert hasattr(torch.ops.ipex_prepack, name)

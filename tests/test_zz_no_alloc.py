@@ -68,7 +68,7 @@ def test_noalloc_plain_calls_and_rejections(cuda):
     case = _synthetic().make_int4_case(54, 4, 1024, 512, 128)
     ctx = make_context(case, O.LOWP_BF16)
     assert _run_both(ctx, case["x"].cuda()) == "woq_decode_kernel"
-    assert _run_both(ctx, case["x"][:1].cuda()) == "woq_decode_kernel"
+    assert _run_both(ctx, case["x"][:1].cuda()) == "woq_decode_m1_kernel"
     # beyond the resident scratch: rejected before anything is launched
     N, K = 64, 4096
     big = _synthetic().make_int4_case(55, 1, K, N, 128)
