@@ -1260,6 +1260,41 @@ def test_fused_post_ops(cuda):
     assert torch.equal(ctx.run(x, fusion=_lib.FUSE_ADD_ADD, others=(o1, o2)), want)
 
 
+@pytest.mark.parametrize("K", [256, 384, 4096])
+def test_output_rounding_chain_with_bias(cuda, K):
+    """Hand-built sums (every weight is (q - z) * s = 1, so the GEMM result is the sum of the row) on which
+    the number of roundings shows: the fp16 regime rounds the sum to fp16, adds the fp16 bias in fp16 and
+    casts (as the fallback does, woq.h:3569-3576); the bf16 regime adds the fp32 bias before its single
+    rounding (woq.h:3298-3310, 3452).  K = 256 / 4096: the integer-weight decode kernels, 384: the others."""
+    from ipex_amd import ops
+
+    N = 32
+    qw = torch.full((N, K // 2), 0x99, dtype=torch.uint8)
+    scales, zeros = torch.ones(N, 1), torch.full((N, 1), 8.0)
+    # fp16 regime, fp16 rows: 1 + 2^-11 + 2^-13 -> fp16 1 + 2^-10; + 2^-11 -> tie -> 1 + 2^-9
+    for M in (1, 3):
+        x = torch.zeros(M, K, dtype=torch.float16)
+        x[:, 0], x[:, K // 2], x[:, K - 1] = 1.0, 2.0 ** -11, 2.0 ** -13
+        ctx = ops.WoqLinearOpContext(qw.cuda(), 2, [N, K], scales.cuda(), zeros.cuda(),
+                                     torch.full((N,), 2.0 ** -11).cuda(), None, None, -1, O.LOWP_FP16, -1)
+        y = ctx.run(x.cuda())
+        assert torch.all(y.float() == 1 + 2.0 ** -9), (M, y.float().unique())
+    # bf16 regime (M >= 5): 1 + 2^-8 + 2^-10 + bias 2^-8 = 1 + 2^-7 + 2^-10 -> 1 + 2^-7 in one rounding
+    for M in (5, 70):
+        x = torch.zeros(M, K, dtype=torch.bfloat16)
+        x[:, 0], x[:, K // 2], x[:, K - 1] = 1.0, 2.0 ** -8, 2.0 ** -10
+        ctx = ops.WoqLinearOpContext(qw.cuda(), 2, [N, K], scales.cuda(), zeros.cuda(),
+                                     torch.full((N,), 2.0 ** -8).cuda(), None, None, -1, O.LOWP_BF16, -1)
+        y = ctx.run(x.cuda())
+        assert torch.all(y.float() == 1.0078125), (M, y.float().unique())
+    # lowp_mode BF16 below five rows computes in fp16 on bf16 rows: fp16(1 + 2^-8 + 2^-10) is exact, the fp16 bias
+    # 2^-8 gives 1 + 2^-7 + 2^-10 (exact in fp16), and the cast to bf16 rounds it to 1 + 2^-7
+    x = torch.zeros(2, K, dtype=torch.bfloat16)
+    x[:, 0], x[:, K // 2], x[:, K - 1] = 1.0, 2.0 ** -8, 2.0 ** -10
+    y = ctx.run(x.cuda())
+    assert torch.all(y.float() == 1.0078125)
+
+
 def test_linearity_in_scales_at_full_size(cuda):
     # doubling every scale doubles the fp32 accumulator exactly (powers of two commute with
     # every rounding on the path); run at the full decode shape

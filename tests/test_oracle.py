@@ -277,6 +277,35 @@ def test_gemm_paths_against_exact_rational_matmul():
     assert np.max(np.abs(y_h - exact[:2])) < 0.08
 
 
+def test_ref_rounding_chain_with_bias_rounds_twice():
+    """woq_gemm_ref_impl rounds the GEMM result to the compute dtype, adds the bias in that dtype (a second
+    rounding) and casts to the activation dtype (csrc/cpu/aten/utils/woq.h:3569-3576, 3612).  Hand-built
+    case where two roundings and one rounding of the exact sum differ: every weight is (q - z) * s = 1, so
+    the exact GEMM result is the sum of the activations.
+      bf16: sum = 1 + 2^-8 + 2^-10 -> bf16 1 + 2^-7 (above the tie); + bias 2^-8 = 1 + 2^-7 + 2^-8, a tie ->
+            even mantissa 1 + 2^-6 = 1.015625.  One rounding of 1 + 2^-7 + 2^-10 would give 1.0078125.
+      fp16: the same eight binades further down: 1 + 2^-11 + 2^-13 -> 1 + 2^-10; + 2^-11 -> tie -> 1 + 2^-9."""
+    qw = O.pack_int4(np.full((1, 4), 9, dtype=np.uint8))
+    scales, zps = np.ones((1, 1), dtype=np.float32), np.full((1, 1), 8, dtype=np.float32)
+    x = np.array([[1.0, 2.0 ** -8, 2.0 ** -10, 0.0]], dtype=np.float32)
+    acc, y = O.woq_linear_ref(x, "bf16", qw, 1, 4, scales, zps, np.array([2.0 ** -8], dtype=np.float32), 2, 4, "bf16")
+    assert float(acc[0, 0]) == 1 + 2.0 ** -7 + 2.0 ** -10
+    assert float(y[0, 0]) == 1.015625
+    _, y_nobias = O.woq_linear_ref(x, "bf16", qw, 1, 4, scales, zps, None, 2, 4, "bf16")
+    assert float(y_nobias[0, 0]) == 1.0078125
+    x = np.array([[1.0, 2.0 ** -11, 2.0 ** -13, 0.0]], dtype=np.float32)
+    _, y = O.woq_linear_ref(x, "fp16", qw, 1, 4, scales, zps, np.array([2.0 ** -11], dtype=np.float32), 2, 4, "fp16")
+    assert float(y[0, 0]) == 1 + 2.0 ** -9
+    # bf16 activations under fp16 compute (lowp_mode BF16 with M < 5): the fp16 result 1 + 2^-9 is then cast to
+    # bf16, where it rounds to 1
+    _, y = O.woq_linear_ref(x, "bf16", qw, 1, 4, scales, zps, np.array([2.0 ** -11], dtype=np.float32), 2, 4, "fp16")
+    assert float(y[0, 0]) == 1.0
+    # the optimized bf16 kernel adds the fp32 bias before its single rounding
+    x = np.array([[1.0, 2.0 ** -8, 2.0 ** -10, 0.0]], dtype=np.float32)
+    _, y = O.woq_linear_opt_bf16(x, "bf16", qw, 1, 4, scales, zps, np.array([2.0 ** -8], dtype=np.float32), 2, 4)
+    assert float(y[0, 0]) == 1.0078125
+
+
 def test_fp16_chain_order_matters_and_is_sequential():
     # one output, K = 4: ((x0*w0 + x1*w1) + x2*w2) + x3*w3 in fp16, chosen so that another order differs
     x = np.array([[1024.0, 0.25, 0.25, -1024.0]], dtype=np.float32)
@@ -312,7 +341,7 @@ def _all_bf16_values():
     return v[np.isfinite(v)]
 
 
-@pytest.mark.parametrize("mode", [4, 6, 7, 0, 2])
+@pytest.mark.parametrize("mode", [4, 5, 6, 7, 0, 1, 2, 3])
 def test_dynamic_quant_invariants_over_all_bf16_patterns(mode):
     vals = _all_bf16_values()
     vals = vals[np.abs(vals) < 1e4]
