@@ -288,7 +288,10 @@ int woq_hip_shuffle_int4_weight(const void* plain, int64_t N, int64_t K, const i
  *   scale_add_rows: out[top_x[i], :] += routing_weights[top_x[i], idx[i]] * expert_out[i, :] for i < n;
  *                   out [T, H], expert_out [n, H], routing_weights [T, topk], all in `dtype`; bf16 and
  *                   fp32 form product and sum in fp32 (one rounding), fp16 rounds the product first.
- *                   The entries of top_x must be distinct (a token reaches an expert at most once). */
+ *                   The entries of top_x must be distinct (a token reaches an expert at most once: two rows
+ *                   for one token would race on its output row).
+ * Indices outside [0, T) (rows, top_x) or [0, topk) (idx) are not an error the kernels can report: such a
+ * row is skipped -- gather_rows leaves zeros, scale_add_rows adds nothing -- instead of faulting. */
 int woq_hip_moe_gather_rows(const void* x, int x_dtype, int64_t T, int64_t H, const int64_t* rows, int64_t n,
                             void* out, void* stream);
 int woq_hip_moe_scale_add_rows(void* out, int dtype, int64_t T, int64_t H, const void* expert_out,

@@ -210,7 +210,6 @@ class WoqLinearOpContext : public torch::CustomClassHolder {
     unregister_context(handle_);
     packed_ = Tensor();
     q_ = PackedQParams();
-    cached_weight_ = Tensor();
     bias_f32_ = Tensor();
   }
 
@@ -221,12 +220,12 @@ class WoqLinearOpContext : public torch::CustomClassHolder {
   optional<Tensor> get_zero_points() { return zeros_plain_; }
   std::vector<int64_t> get_weight_shape() { return {N_, K_}; }
   optional<Tensor> get_g_idx() { return g_idx_; }
-  // A bf16 copy of the dequantized weight, kept from the first call on that asks for it: with
-  // cache_weight_for_large_batch under lowp_mode BF16 large batches run on it
-  // (csrc/cpu/jit/cpu/kernels/LinearWoqPacked.cpp:430-533).
-  optional<Tensor> get_cached_weight() {
-    return cached_weight_.defined() ? optional<Tensor>(cached_weight_) : c10::nullopt;
-  }
+  // The reference keeps a dequantized bf16 copy of the weight for batches of 64 rows and more when
+  // cache_weight_for_large_batch is set (csrc/cpu/jit/cpu/kernels/LinearWoqPacked.cpp:430-533), because
+  // its kernel dequantizes a weight block again for every 64 rows.  The prefill kernels here dequantize
+  // in registers once per 128 rows and run within 15 % of a dense bf16 GEMM on the same shape, so the
+  // flag is accepted, kept and pickled, and no copy (four times the packed weight's memory) is made.
+  optional<Tensor> get_cached_weight() { return c10::nullopt; }
   // The reference caches the column sums of an int8 copy of the weight for lowp_mode INT8
   // (LinearWoqPacked.cpp:485-508); here the int8 MFMA kernels read the stored codes and form those sums
   // on the fly, so there is nothing to cache.
@@ -361,13 +360,12 @@ class WoqLinearOpContext : public torch::CustomClassHolder {
     q_ = pack_qparams(scales, zps, weight_dtype);
     scales_plain_ = group_size > 0 ? scales : scales.reshape({N});
     zeros_plain_ = zps.has_value() ? optional<Tensor>(group_size > 0 ? *zps : zps->reshape({N})) : c10::nullopt;
-    cached_weight_ = Tensor();
   }
 
   void copy_state(const WoqLinearOpContext& o) {
     packed_ = o.packed_; q_ = o.q_; bias_ = o.bias_; bias_f32_ = o.bias_f32_; scales_plain_ = o.scales_plain_;
     zeros_plain_ = o.zeros_plain_; g_idx_ = o.g_idx_; g_src_ = o.g_src_; g_dst_ = o.g_dst_;
-    cached_weight_ = o.cached_weight_; N_ = o.N_; K_ = o.K_; group_size_ = o.group_size_;
+    N_ = o.N_; K_ = o.K_; group_size_ = o.group_size_;
     weight_dtype_ = o.weight_dtype_; lowp_mode_ = o.lowp_mode_; act_quant_mode_ = o.act_quant_mode_;
     batch_size_ = o.batch_size_; cache_weight_ = o.cache_weight_;
   }
@@ -375,21 +373,6 @@ class WoqLinearOpContext : public torch::CustomClassHolder {
   // `run` behind the act-order shuffle: the input channels of x are in the order of the stored weight
   Tensor run_sorted(const Tensor& x, int64_t M, int64_t fusion, const std::vector<Tensor>& others,
                     const std::vector<int64_t>& out_sizes) {
-    static const int64_t cache_threshold = [] {
-      const char* e = getenv("IPEX_WOQ_WEIGHT_CACHE_BATCH_THRESHOLD");  // LinearWoqPacked.cpp:17-18
-      return e ? (int64_t)atoll(e) : (int64_t)64;
-    }();
-    if (cache_weight_ && lowp_mode_ == WOQ_HIP_LOWP_BF16 && M >= cache_threshold && fusion == WOQ_HIP_FUSE_NONE &&
-        weight_dtype_ == WOQ_HIP_DTYPE_NF4) {
-      // NF4 above 64 rows has no kernel with register-resident dequantization: the cached bf16 weight
-      // and the prefill GEMM's dense counterpart serve it (csrc/cpu/jit/cpu/kernels/LinearWoqPacked.cpp:517-526).
-      // Integer weights stay on woq_gemm_w4_kernel, which needs no copy of the weight.
-      if (!cached_weight_.defined())
-        cached_weight_ = dequant_weight(packed_, weight_dtype_, N_, K_, q_.sb16.to(at::kFloat), q_.z8, group_size_,
-                                        at::kBFloat16);
-      optional<Tensor> b = bias_.has_value() ? optional<Tensor>(bias_->to(at::kBFloat16)) : c10::nullopt;
-      return at::linear(x.to(at::kBFloat16), cached_weight_, b).to(x.scalar_type());
-    }
     if (lowp_mode_ == WOQ_HIP_LOWP_FP16 && x.scalar_type() == at::kBFloat16 && M > 16 && fusion == WOQ_HIP_FUSE_NONE) {
       // fp16 compute on bf16 rows beyond one row tile: the reference converts the rows to fp16 and casts
       // the fp16 result back (csrc/cpu/aten/utils/woq.h:3076-3085)
@@ -455,7 +438,6 @@ class WoqLinearOpContext : public torch::CustomClassHolder {
   optional<Tensor> zeros_plain_;
   optional<Tensor> g_idx_;
   Tensor g_src_, g_dst_;
-  Tensor cached_weight_;
   int64_t N_ = 0, K_ = 0, group_size_ = -1, weight_dtype_ = 0, lowp_mode_ = 0, act_quant_mode_ = 0;
   optional<int64_t> batch_size_;
   bool cache_weight_ = false;

@@ -327,7 +327,7 @@ int woq_hip_moe_gather_rows(const void* x, int x_dtype, int64_t T, int64_t H, co
   if (T < 0 || H < 0 || n < 0) return set_error("moe_gather_rows: negative size");
   if (n > 0 && H > 0 && (!x || !rows || !out)) return set_error("moe_gather_rows: null pointer");
   if (n > 0 && T == 0) return set_error("moe_gather_rows: rows requested from an empty tensor");
-  return launch_moe_gather_rows(x, x_dtype, H, rows, n, out, (hipStream_t)stream);
+  return launch_moe_gather_rows(x, x_dtype, T, H, rows, n, out, (hipStream_t)stream);
 }
 
 int woq_hip_moe_scale_add_rows(void* out, int dtype, int64_t T, int64_t H, const void* expert_out,
@@ -339,7 +339,7 @@ int woq_hip_moe_scale_add_rows(void* out, int dtype, int64_t T, int64_t H, const
     return set_error("moe_scale_add_rows: null pointer");
   if (n > T) return set_error("moe_scale_add_rows: %lld rows for %lld tokens (a token may appear once)", (long long)n,
                               (long long)T);
-  return launch_moe_scale_add_rows(out, dtype, H, expert_out, routing_weights, topk, top_x, idx, n,
+  return launch_moe_scale_add_rows(out, dtype, T, H, expert_out, routing_weights, topk, top_x, idx, n,
                                    (hipStream_t)stream);
 }
 

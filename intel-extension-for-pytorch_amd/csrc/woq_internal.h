@@ -58,9 +58,9 @@ int launch_shuffle_activations(const void* x, int x_dtype, int64_t M, int64_t K,
                                hipStream_t st);
 int launch_shuffle_int4_weight(const void* plain, int64_t N, int64_t K, const int32_t* src, void* out,
                                hipStream_t st);
-int launch_moe_gather_rows(const void* x, int x_dtype, int64_t H, const int64_t* rows, int64_t n, void* out,
+int launch_moe_gather_rows(const void* x, int x_dtype, int64_t T, int64_t H, const int64_t* rows, int64_t n, void* out,
                            hipStream_t st);
-int launch_moe_scale_add_rows(void* out, int dtype, int64_t H, const void* cur, const void* rw, int64_t topk,
+int launch_moe_scale_add_rows(void* out, int dtype, int64_t T, int64_t H, const void* cur, const void* rw, int64_t topk,
                               const int64_t* top_x, const int64_t* idx, int64_t n, hipStream_t st);
 int launch_dequant_weight(const void* qweight, int weight_dtype, int64_t N, int64_t K, const float* s32,
                           const uint8_t* z8, int64_t G, void* out, int out_dtype, hipStream_t st);

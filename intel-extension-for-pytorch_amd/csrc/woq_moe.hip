@@ -19,14 +19,17 @@
 
 namespace woq {
 
-// out[i, :] = x[rows[i], :]; a row is `chunks` units of T.
+// out[i, :] = x[rows[i], :]; a row is `chunks` units of T.  The indices come from the caller's routing
+// tensors: a row outside [0, tokens) reads nothing and leaves zeros (an out-of-bounds access would be a
+// device fault, not an error the host can report).
 template <typename T>
 __global__ void moe_gather_rows_kernel(const T* __restrict__ x, const int64_t* __restrict__ rows, int64_t n,
-                                       int64_t chunks, T* __restrict__ out) {
+                                       int64_t chunks, int64_t tokens, T* __restrict__ out) {
   const int64_t g = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (g >= n * chunks) return;
   const int64_t i = g / chunks, c = g - i * chunks;
-  out[g] = x[rows[i] * chunks + c];
+  const int64_t row = rows[i];
+  out[g] = (uint64_t)row < (uint64_t)tokens ? x[row * chunks + c] : T{};
 }
 
 template <int DTYPE>
@@ -44,14 +47,17 @@ __device__ __forceinline__ float moe_accumulate(float o, float v, float w) {
 template <int DTYPE>
 __global__ void moe_scale_add_rows_kernel(void* __restrict__ out, const void* __restrict__ cur,
                                           const void* __restrict__ rw, int64_t topk, const int64_t* __restrict__ top_x,
-                                          const int64_t* __restrict__ idx, int64_t n, int64_t H, bool vec) {
+                                          const int64_t* __restrict__ idx, int64_t n, int64_t H, int64_t tokens,
+                                          bool vec) {
   constexpr int PER = DTYPE == WOQ_HIP_ACT_FP32 ? 4 : 8;
   const int64_t chunks = (H + PER - 1) / PER;
   const int64_t g = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (g >= n * chunks) return;
   const int64_t i = g / chunks, j0 = (g - i * chunks) * PER;
-  const int64_t t = top_x[i];
-  const float w = load_act(rw, DTYPE, t * topk + idx[i]);
+  const int64_t t = top_x[i], slot = idx[i];
+  // a token or a top-k slot out of range is skipped: nothing is read or written for it
+  if ((uint64_t)t >= (uint64_t)tokens || (uint64_t)slot >= (uint64_t)topk) return;
+  const float w = load_act(rw, DTYPE, t * topk + slot);
   const int64_t ob = t * H + j0, cb = i * H + j0;
   if (vec) {
     if constexpr (DTYPE == WOQ_HIP_ACT_FP32) {
@@ -86,33 +92,33 @@ __global__ void moe_scale_add_rows_kernel(void* __restrict__ out, const void* __
 
 static inline unsigned moe_blocks(int64_t n) { return (unsigned)((n + 255) / 256); }
 
-int launch_moe_gather_rows(const void* x, int x_dtype, int64_t H, const int64_t* rows, int64_t n, void* out,
+int launch_moe_gather_rows(const void* x, int x_dtype, int64_t T, int64_t H, const int64_t* rows, int64_t n, void* out,
                            hipStream_t st) {
   if (n == 0 || H == 0) return 0;
   const int64_t row_bytes = H * (x_dtype == WOQ_HIP_ACT_FP32 ? 4 : 2);
   if (row_bytes % 16 == 0 && (((uintptr_t)x | (uintptr_t)out) & 15) == 0) {
     const int64_t chunks = row_bytes / 16;
-    moe_gather_rows_kernel<u4><<<moe_blocks(n * chunks), 256, 0, st>>>((const u4*)x, rows, n, chunks, (u4*)out);
+    moe_gather_rows_kernel<u4><<<moe_blocks(n * chunks), 256, 0, st>>>((const u4*)x, rows, n, chunks, T, (u4*)out);
   } else if (x_dtype == WOQ_HIP_ACT_FP32) {
-    moe_gather_rows_kernel<uint32_t><<<moe_blocks(n * H), 256, 0, st>>>((const uint32_t*)x, rows, n, H, (uint32_t*)out);
+    moe_gather_rows_kernel<uint32_t><<<moe_blocks(n * H), 256, 0, st>>>((const uint32_t*)x, rows, n, H, T, (uint32_t*)out);
   } else {
-    moe_gather_rows_kernel<uint16_t><<<moe_blocks(n * H), 256, 0, st>>>((const uint16_t*)x, rows, n, H, (uint16_t*)out);
+    moe_gather_rows_kernel<uint16_t><<<moe_blocks(n * H), 256, 0, st>>>((const uint16_t*)x, rows, n, H, T, (uint16_t*)out);
   }
   return check_launch("moe_gather_rows");
 }
 
-int launch_moe_scale_add_rows(void* out, int dtype, int64_t H, const void* cur, const void* rw, int64_t topk,
+int launch_moe_scale_add_rows(void* out, int dtype, int64_t T, int64_t H, const void* cur, const void* rw, int64_t topk,
                               const int64_t* top_x, const int64_t* idx, int64_t n, hipStream_t st) {
   if (n == 0 || H == 0) return 0;
   const int per = dtype == WOQ_HIP_ACT_FP32 ? 4 : 8;
   const bool vec = H % per == 0 && (((uintptr_t)out | (uintptr_t)cur) & 15) == 0;
   const unsigned blocks = moe_blocks(n * ((H + per - 1) / per));
   if (dtype == WOQ_HIP_ACT_BF16)
-    moe_scale_add_rows_kernel<WOQ_HIP_ACT_BF16><<<blocks, 256, 0, st>>>(out, cur, rw, topk, top_x, idx, n, H, vec);
+    moe_scale_add_rows_kernel<WOQ_HIP_ACT_BF16><<<blocks, 256, 0, st>>>(out, cur, rw, topk, top_x, idx, n, H, T, vec);
   else if (dtype == WOQ_HIP_ACT_FP16)
-    moe_scale_add_rows_kernel<WOQ_HIP_ACT_FP16><<<blocks, 256, 0, st>>>(out, cur, rw, topk, top_x, idx, n, H, vec);
+    moe_scale_add_rows_kernel<WOQ_HIP_ACT_FP16><<<blocks, 256, 0, st>>>(out, cur, rw, topk, top_x, idx, n, H, T, vec);
   else
-    moe_scale_add_rows_kernel<WOQ_HIP_ACT_FP32><<<blocks, 256, 0, st>>>(out, cur, rw, topk, top_x, idx, n, H, vec);
+    moe_scale_add_rows_kernel<WOQ_HIP_ACT_FP32><<<blocks, 256, 0, st>>>(out, cur, rw, topk, top_x, idx, n, H, T, vec);
   return check_launch("moe_scale_add_rows");
 }
 

@@ -22,7 +22,6 @@ handles name Python objects and are understood by the functions of this module o
 """
 import contextlib
 import ctypes
-import os
 import threading
 import weakref
 from typing import List, Optional
@@ -39,10 +38,6 @@ _current_device = getattr(torch._C, "_cuda_getDevice", None) or torch.cuda.curre
 
 WOQ_DTYPE_MAP = {"int8": _lib.DTYPE_INT8, "int4": _lib.DTYPE_INT4, "nf4": _lib.DTYPE_NF4}
 PLAIN_WEIGHT_FORMAT, GPTQ_WEIGHT_FORMAT, AWQ_WEIGHT_FORMAT = 0, 1, 2
-
-# M at and above which a cached dequantized weight is used (IPEX_WOQ_WEIGHT_CACHE_BATCH_THRESHOLD,
-# csrc/cpu/jit/cpu/kernels/LinearWoqPacked.cpp:17-18).
-WEIGHT_CACHE_BATCH_THRESHOLD = int(os.environ.get("IPEX_WOQ_WEIGHT_CACHE_BATCH_THRESHOLD", "64"))
 
 _contexts = {}
 _contexts_lock = threading.Lock()
@@ -169,7 +164,6 @@ class WoqLinearOpContext:
         self.zero_points_plain_ = (
             None if zero_points is None else (zero_points if group_size > 0 else zero_points.reshape(N))
         )
-        self.cached_weight_ = None
         self.cached_compensation_ = None
         with _contexts_lock:
             self._handle = _next_handle[0]
@@ -203,7 +197,11 @@ class WoqLinearOpContext:
         return self.g_idx_
 
     def get_cached_weight(self):
-        return self.cached_weight_
+        """Always None: ``cache_weight_for_large_batch`` is accepted, kept and pickled, but no dequantized
+        copy of the weight is made.  The reference caches one for batches of 64 rows and more because its
+        kernel dequantizes a block again for every 64 rows (LinearWoqPacked.cpp:430-533); the prefill
+        kernels here dequantize in registers once per 128 rows."""
+        return None
 
     def get_cached_compensation(self):
         return self.cached_compensation_
@@ -329,16 +327,6 @@ class WoqLinearOpContext:
             _lib.check(rc, "woq_linear")
         return out
 
-    def _cached_bf16_weight(self):
-        if self.cached_weight_ is None:
-            N, K = self.weight_shape_
-            # the bf16-rounded scales are what the bf16 kernel dequantizes with
-            s = self.scales_list_[2].to(torch.float32)
-            self.cached_weight_ = _kernels.dequant_weight(
-                self.at_weight_, self.weight_dtype_, N, K, s, self.zeros_u8_, self.group_size_, torch.bfloat16
-            )
-        return self.cached_weight_
-
     def run(self, x, fusion=_lib.FUSE_NONE, others=(), **kw):
         N, K = self.weight_shape_
         if x.shape[-1] != K:
@@ -356,18 +344,6 @@ class WoqLinearOpContext:
         """``run`` behind the act-order shuffle: the input channels of ``x`` are already in the order of
         the stored weight."""
         N, K = self.weight_shape_
-        if (
-            self.cache_weight_for_large_batch_
-            and self.lowp_mode_ == _lib.LOWP_BF16
-            and M >= WEIGHT_CACHE_BATCH_THRESHOLD
-            and fusion == _lib.FUSE_NONE
-            and not kw
-        ):
-            # first-token path on a cached dequantized weight: a plain bf16 GEMM
-            # (csrc/cpu/jit/cpu/kernels/LinearWoqPacked.cpp:517-526)
-            w = self._cached_bf16_weight()
-            b = self.at_bias_.to(torch.bfloat16) if self.at_bias_ is not None else None
-            return torch.nn.functional.linear(x.to(torch.bfloat16), w, b).to(x.dtype)
         if (
             self.lowp_mode_ == _lib.LOWP_FP16
             and x.dtype == torch.bfloat16
