@@ -211,9 +211,8 @@ __global__ __launch_bounds__(1024, 8) void woq_decode_kernel(const DecodeArgs a)
 //     against -1 as above;
 //   * every row of the A operand is the one activation row, so every row of D is the result: a lane
 //     scales and accumulates one element per tile instead of four.
-template <bool XBF16, int NTW, bool ONE_ROUND>
-__global__ __launch_bounds__(1024, 8) void woq_decode_m1_kernel(const DecodeArgs a) {
-  constexpr int KPW = kDecodeKPW;
+template <bool XBF16, int NTW, int KPW, bool ONE_ROUND>
+__global__ __launch_bounds__(KPW == 2 ? 1024 : 512, KPW == 2 ? 8 : 4) void woq_decode_m1_kernel(const DecodeArgs a) {
   constexpr int SLICE = KPW * kTileK4;  // K elements of one wave per round
   extern __shared__ __align__(16) uint8_t smem[];
   const int W = a.W;
@@ -250,7 +249,7 @@ __global__ __launch_bounds__(1024, 8) void woq_decode_m1_kernel(const DecodeArgs
 
   const int KT = (int)a.KT, KG = (int)a.KG;
   const int tpg_shift = a.tpg_shift;
-  static_assert(KPW == 2, "two K tiles per wave and round");
+  static_assert(KPW == 2 || KPW == 4, "two or four K tiles per wave and round");
   const int xlane = lane & (KPW * 16 - 1);  // lanes 32..63 mirror 0..31
   // What the last instructions of the kernel need from the argument block, loaded with the rest of it
   // and kept in scalar registers: left to itself the compiler reads them behind the barrier, one
@@ -367,10 +366,10 @@ __global__ __launch_bounds__(1024, 8) void woq_decode_m1_kernel(const DecodeArgs
   }
 }
 
-template <bool XBF16, int NTW, bool ONE_ROUND>
+template <bool XBF16, int NTW, int KPW, bool ONE_ROUND>
 static int launch_decode_m1_cfg(const DecodeArgs& a, hipStream_t st) {
-  const size_t smem = (size_t)NTW * 16 * 16 * sizeof(float) + (size_t)a.W * kDecodeKPW * kTileK4 * sizeof(uint16_t);
-  woq_decode_m1_kernel<XBF16, NTW, ONE_ROUND><<<(unsigned)((a.NT + NTW - 1) / NTW), a.W * 64, smem, st>>>(a);
+  const size_t smem = (size_t)NTW * 16 * 16 * sizeof(float) + (size_t)a.W * KPW * kTileK4 * sizeof(uint16_t);
+  woq_decode_m1_kernel<XBF16, NTW, KPW, ONE_ROUND><<<(unsigned)((a.NT + NTW - 1) / NTW), a.W * 64, smem, st>>>(a);
   return check_launch("woq_decode_m1_kernel");
 }
 
@@ -423,8 +422,18 @@ int launch_decode(const FpArgs& f, const uint32_t* sz, hipStream_t st) {
   const bool one_row = f.M == 1;
   const bool one_round = f.KT == (int64_t)a.W * kDecodeKPW;
   if (one_row) {
+    // Four K tiles per wave (half the waves, each with twice the bytes in flight) where two tiles per
+    // wave would leave at most two waves per SIMD anyway: the per-wave overhead then weighs more than
+    // the occupancy (M = 1, 2048 -> 8192: 3.8 us against 4.6 us; 4096 -> 14336, seven waves per SIMD:
+    // 7.4 us against 7.1 us the other way round).
+    const int64_t waves2 = (f.NT / (two ? 2 : 1)) * ((f.KT + 1) / 2);
+    if (waves2 <= 2048 && f.KT % 4 == 0 && f.KT / 4 <= 8) {
+      a.W = (int)(f.KT / 4);
+      if (xf16) return two ? launch_decode_m1_cfg<false, 2, 4, true>(a, st) : launch_decode_m1_cfg<false, 1, 4, true>(a, st);
+      return two ? launch_decode_m1_cfg<true, 2, 4, true>(a, st) : launch_decode_m1_cfg<true, 1, 4, true>(a, st);
+    }
 #define WOQ_DECODE_M1(XB, NTW) \
-  (one_round ? launch_decode_m1_cfg<XB, NTW, true>(a, st) : launch_decode_m1_cfg<XB, NTW, false>(a, st))
+  (one_round ? launch_decode_m1_cfg<XB, NTW, 2, true>(a, st) : launch_decode_m1_cfg<XB, NTW, 2, false>(a, st))
     if (xf16) return two ? WOQ_DECODE_M1(false, 2) : WOQ_DECODE_M1(false, 1);
     return two ? WOQ_DECODE_M1(true, 2) : WOQ_DECODE_M1(true, 1);
 #undef WOQ_DECODE_M1

@@ -1603,3 +1603,20 @@ def test_fp32_compute_post_ops(cuda):
     assert torch.equal(ctx.run(x, fusion=_lib.FUSE_ADD, others=(o1,)), base + o1)
     assert torch.equal(ctx.run(x, fusion=_lib.FUSE_MUL, others=(o1,)), base * o1)
     assert torch.equal(ctx.run(x, fusion=_lib.FUSE_ADD_ADD, others=(o1, o2)), base + o1 + o2)
+
+
+@pytest.mark.parametrize("K,N", [(2048, 8192), (1024, 512), (512, 272), (4096, 512)])
+def test_single_row_decode_with_four_k_tiles_per_wave(cuda, K, N):
+    """M = 1 on layers small enough that the kernel gives every wave four K tiles instead of two."""
+    from ipex_amd import _lib
+
+    case = _synthetic().make_int4_case(77, 1, K, N, 128, bias=(N % 32 == 16))
+    _check_fp(case, O.LOWP_BF16, label=f"M=1 K={K} N={N}")
+    assert _lib.last_kernel() == "woq_decode_m1_kernel"
+    case16 = dict(case)
+    case16["x"] = case["x"].to(torch.float16)
+    ctx = make_context(case16, O.LOWP_FP16)
+    c = case_np(case16)
+    y = to_np_f32(ctx.run(case16["x"].cuda()))
+    _, want = O.woq_linear_ref(c["x"], "fp16", c["qw"], N, K, O._round_to(c["scales"], "fp16"), c["zps"], c["bias"], 2, 128, "fp16")
+    assert rel_l2(y, want) <= REL_L2_OUT
