@@ -30,8 +30,8 @@ MFMA_FP32_PEAK_TFLOPS = 157.3   # MI355X dense fp32 matrix, published
 # the figure comes from two rocprofv3 --pmc runs of `bench.py --probe decode` (FETCH_SIZE 15310.55 KiB and
 # WRITE_SIZE 28.00 KiB per dispatch, scaled by what the same counters read for a 256 MiB copy: x2.000 and
 # x1.000), whose summary is the file named beside it; keyed by (M, K, N, group size).  Other shapes: null.
-PROFILED_HBM_BYTES_PER_LAUNCH = {(1, 4096, 14336, 128): 31384678}
-PROFILED_HBM_BYTES_SOURCE = "profiles/woq_decode_kernel_M1_4096x14336_g128.hbm_traffic.txt"
+PROFILED_HBM_BYTES_PER_LAUNCH = {(1, 4096, 14336, 128): 31339412}
+PROFILED_HBM_BYTES_SOURCE = "profiles/woq_decode_m1_kernel_M1_4096x14336_g128.hbm_traffic_and_counters.txt"
 # Launches that precede every timed region whatever --warmup says: the first milliseconds after an idle
 # period run 3-10 % slower (clocks, translation caches).
 MIN_WARMUP_LAUNCHES = 2000
