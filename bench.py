@@ -270,6 +270,7 @@ def config_sweep(torch, lib, lib_mod, ops_mod, synthetic, dev, stream, steps):
     # the reference may run (single-stream decode of a group-32 model, lowp_mode INT8 decode with
     # per-row and per-(row, K block) activation scales, INT8 weights at prefill size, asymmetric
     # activations, a group-64 model and INT8 weights at a serving batch under lowp_mode INT8).
+    run("extra: int4 g128 M=1 4096->28672 (gate+up in one launch, lowp BF16)", synthetic.make_int4_case(5, 1, 4096, 28672, 128))
     run("extra: int4 g32 M=1 4096->14336 (lowp BF16)", synthetic.make_int4_case(5, 1, 4096, 14336, 32))
     run("extra: int4 g128 M=1 4096->14336 lowp INT8 per-row", synthetic.make_int4_case(5, 1, 4096, 14336, 128), 3, 6)
     run("extra: int4 g128 M=16 4096->14336 lowp INT8 per-row-and-K-block", synthetic.make_int4_case(5, 16, 4096, 14336, 128), 3, 7)
