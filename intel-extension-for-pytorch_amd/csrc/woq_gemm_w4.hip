@@ -290,7 +290,7 @@ __global__ __launch_bounds__(256) void woq_gemm_w4_kernel(const FpArgs f, const 
         }
 #pragma unroll
         for (int mt = 0; mt < G4_MT; ++mt) {
-          acc[mt][t] = g4_mfma<REGIME>(xa[(j & 1) % S::XA_SETS][mt], bop[cur], acc[mt][t]);
+          acc[mt][t] = g4_mfma<REGIME>(bop[cur], xa[(j & 1) % S::XA_SETS][mt], acc[mt][t]);
           if (fetch_t)
             xa[((j & 1) ^ 1) % S::XA_SETS][mt] = j == 3 ? *(const u4*)(xsn + mt * 4096 + rd[0])
                                          : *(const u4*)(xs + mt * 4096 + rd[j + 1]);
@@ -378,66 +378,61 @@ __global__ __launch_bounds__(256) void woq_gemm_w4_kernel(const FpArgs f, const 
     if (tid == 0) __hip_atomic_store(sk_counters + tile, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
 
-  // ---- epilogue: D[m][n], lane (n = r, c) holds rows m = 16 mt + 4 c + e.  Each wave transposes
-  // one 16 x (16 NTW) accumulator tile at a time through its own LDS region (the activation buffers are
-  // idle after the last barrier), so that consecutive lanes store consecutive columns. ----
-  float* stage = (float*)sX + wave * (16 * G4_SSTRIDE);
+  // ---- epilogue.  The weights are the first MFMA operand and the activations the second, so the
+  // accumulator tile is D[n][m]: lane (r, c) holds row m = 16 mt + r and the four consecutive columns
+  // n = 16 t + 4 c + e.  In the plain case (no post-op, output in the activation dtype) a lane rounds
+  // its four values and stores them as 8 bytes straight from the registers: the four lane columns of a
+  // row write 32 contiguous bytes, the NTW row-blocks of a wave follow each other in the row, and
+  // nothing waits on LDS.  Post-ops go through a per-wave LDS tile (the activation buffers are idle
+  // after the last barrier) so that the element-wise tail sees consecutive columns in consecutive lanes. ----
   const int64_t ncol0 = (int64_t)nt0 * kTileN;
   const int act = REGIME == kRegimeF16 ? WOQ_HIP_ACT_FP16 : WOQ_HIP_ACT_BF16;
-  const bool fast = f.fusion == WOQ_HIP_FUSE_NONE && f.out_dtype == act && (f.N % 8) == 0 &&
-                    ncol0 + G4_NTW * kTileN <= f.N && (((uintptr_t)f.out | (uintptr_t)f.bias) & 15) == 0;
+  const bool fast = f.fusion == WOQ_HIP_FUSE_NONE && f.out_dtype == act && (f.N % 4) == 0 &&
+                    ncol0 + G4_NTW * kTileN <= f.N && (((uintptr_t)f.out & 7) | ((uintptr_t)f.bias & 15)) == 0;
   const bool hb = f.bias != nullptr;
+  if (fast) {
+    f4 bias4[G4_NTW];
+#pragma unroll
+    for (int t = 0; t < G4_NTW; ++t)
+      bias4[t] = hb ? *(const f4*)(f.bias + ncol0 + t * kTileN + 4 * c) : f4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int mt = 0; mt < G4_MT; ++mt) {
+      const int m = m0 + mt * 16 + r;
+      if (m < M) {
+        uint16_t* const row = (uint16_t*)f.out + (int64_t)m * f.N + ncol0 + 4 * c;
+#pragma unroll
+        for (int t = 0; t < G4_NTW; ++t) {
+          const float y0 = finalize_acc<REGIME>(acc[mt][t][0], hb, bias4[t][0]);
+          const float y1 = finalize_acc<REGIME>(acc[mt][t][1], hb, bias4[t][1]);
+          const float y2 = finalize_acc<REGIME>(acc[mt][t][2], hb, bias4[t][2]);
+          const float y3 = finalize_acc<REGIME>(acc[mt][t][3], hb, bias4[t][3]);
+          u2 o;
+          if constexpr (REGIME == kRegimeF16) {
+            o[0] = (uint32_t)f32_to_f16_bits(y0) | ((uint32_t)f32_to_f16_bits(y1) << 16);
+            o[1] = (uint32_t)f32_to_f16_bits(y2) | ((uint32_t)f32_to_f16_bits(y3) << 16);
+          } else {
+            o[0] = bitcast<uint32_t>(__builtin_convertvector(f2{y0, y1}, b2));
+            o[1] = bitcast<uint32_t>(__builtin_convertvector(f2{y2, y3}, b2));
+          }
+          *(u2*)(row + t * kTileN) = o;
+        }
+      }
+    }
+    return;
+  }
+  float* stage = (float*)sX + wave * (16 * G4_SSTRIDE);
   Epilogue ep{f.bias, f.fusion, f.other0, f.other1, f.out, f.out_dtype, f.x_dtype, f.N};
 #pragma unroll
   for (int mt = 0; mt < G4_MT; ++mt) {
 #pragma unroll
-    for (int t = 0; t < G4_NTW; ++t)
-#pragma unroll
-      for (int e = 0; e < 4; ++e) stage[(4 * c + e) * G4_SSTRIDE + t * kTileN + r] = acc[mt][t][e];
-    if (fast) {
-      // 16 rows x 2 NTW chunks of 8 columns: one 16-byte store per chunk
-      constexpr int CH = 2 * G4_NTW;
-#pragma unroll
-      for (int it = 0; it < (16 * CH + 63) / 64; ++it) {
-        const int idx = it * 64 + lane;
-        const int row = idx / CH, ch = idx - row * CH;
-        const int m = m0 + mt * 16 + row;
-        if (idx < 16 * CH && m < M) {
-          const f4 v0 = *(const f4*)(stage + row * G4_SSTRIDE + ch * 8);
-          const f4 v1 = *(const f4*)(stage + row * G4_SSTRIDE + ch * 8 + 4);
-          const int64_t n = ncol0 + ch * 8;
-          f4 b0 = f4{0.f, 0.f, 0.f, 0.f}, b1 = b0;
-          if (hb) {
-            b0 = *(const f4*)(f.bias + n);
-            b1 = *(const f4*)(f.bias + n + 4);
-          }
-          u4 o;
-#pragma unroll
-          for (int i = 0; i < 2; ++i) {
-            const float y0 = finalize_acc<REGIME>(v0[2 * i], hb, b0[2 * i]);
-            const float y1 = finalize_acc<REGIME>(v0[2 * i + 1], hb, b0[2 * i + 1]);
-            const float y2 = finalize_acc<REGIME>(v1[2 * i], hb, b1[2 * i]);
-            const float y3 = finalize_acc<REGIME>(v1[2 * i + 1], hb, b1[2 * i + 1]);
-            if constexpr (REGIME == kRegimeF16) {
-              o[i] = (uint32_t)f32_to_f16_bits(y0) | ((uint32_t)f32_to_f16_bits(y1) << 16);
-              o[i + 2] = (uint32_t)f32_to_f16_bits(y2) | ((uint32_t)f32_to_f16_bits(y3) << 16);
-            } else {
-              o[i] = bitcast<uint32_t>(__builtin_convertvector(f2{y0, y1}, b2));
-              o[i + 2] = bitcast<uint32_t>(__builtin_convertvector(f2{y2, y3}, b2));
-            }
-          }
-          *(u4*)((uint16_t*)f.out + (int64_t)m * f.N + n) = o;
-        }
-      }
-    } else {
+    for (int t = 0; t < G4_NTW; ++t) *(f4*)(stage + r * G4_SSTRIDE + t * kTileN + 4 * c) = acc[mt][t];
 #pragma unroll 1
-      for (int it = 0; it < 16 * G4_NTW * kTileN / 64; ++it) {
-        const int idx = it * 64 + lane;
-        const int row = idx / (G4_NTW * kTileN), col = idx - row * (G4_NTW * kTileN);
-        const int m = m0 + mt * 16 + row;
-        const int64_t n = ncol0 + col;
-        if (m < M && n < f.N) epilogue_store<REGIME>(ep, m, n, stage[row * G4_SSTRIDE + col]);
-      }
+    for (int it = 0; it < 16 * G4_NTW * kTileN / 64; ++it) {
+      const int idx = it * 64 + lane;
+      const int row = idx / (G4_NTW * kTileN), col = idx - row * (G4_NTW * kTileN);
+      const int m = m0 + mt * 16 + row;
+      const int64_t n = ncol0 + col;
+      if (m < M && n < f.N) epilogue_store<REGIME>(ep, m, n, stage[row * G4_SSTRIDE + col]);
     }
   }
 }
