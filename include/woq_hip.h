@@ -31,6 +31,8 @@
  *                               fused post-ops of woq_linear_unary_kernel /
  *                               woq_linear_binary_kernel (csrc/cpu/aten/Linear.cpp:619-801)
  *   woq_hip_dequant_weight   <- dequantize_woq_weight (csrc/cpu/aten/utils/woq_utils.h:79-163)
+ *   woq_hip_convert_activations<- the conversion of bf16 activation rows to the fp16 compute type in front
+ *                               of the fp16 kernels (csrc/cpu/aten/utils/woq.h:3076-3079)
  *   woq_hip_shuffle_activations, woq_hip_shuffle_int4_weight
  *                            <- woq_shuffle_tensor_by_group_idx /
  *                               woq_shuffle_weight_back_by_group_idx, the channel shuffles of
@@ -197,7 +199,9 @@ typedef struct woq_hip_linear_params {
   const void* others[2];
 
   /* output [M, N]; out_dtype = x_dtype, or WOQ_HIP_ACT_FP32 to receive the fp32
-   * accumulator (bias added, no output rounding, no post-op) for parity checks */
+   * accumulator (bias added, no output rounding, no post-op) for parity checks, or -- without a
+   * post-op -- the other 16-bit type: the result in the compute type's rounding, cast to it (fp16 rows
+   * made by woq_hip_convert_activations from a bf16 tensor under lowp_mode FP16, bf16 output) */
   void* out;
   int32_t out_dtype;
 
@@ -271,6 +275,13 @@ int woq_hip_linear_noalloc(const woq_hip_linear_params* p);
 int woq_hip_dequant_weight(const void* qweight, int weight_dtype, int64_t N, int64_t K,
                            const float* scales_f32, const uint8_t* zeros_u8,
                            int64_t group_size, void* out, int out_dtype, void* stream);
+
+/* dst[i] = src[i] converted, round to nearest even; dtypes WOQ_HIP_ACT_*; count elements.  With it a
+ * caller runs lowp_mode FP16 on a bf16 tensor of any number of rows through the fp16 kernels: convert
+ * the rows once, call woq_hip_linear with x_dtype FP16 and out_dtype BF16 (up to 16 rows woq_hip_linear
+ * converts on the way into LDS by itself). */
+int woq_hip_convert_activations(const void* src, int src_dtype, void* dst, int dst_dtype, int64_t count,
+                                void* stream);
 
 /* GPTQ act-order.  src[p] (int32, K entries, a permutation of 0..K-1) is the input channel that
  * belongs at position p once the channels are sorted by group (stable in the channel index).

@@ -373,19 +373,25 @@ class WoqLinearOpContext : public torch::CustomClassHolder {
   // `run` behind the act-order shuffle: the input channels of x are in the order of the stored weight
   Tensor run_sorted(const Tensor& x, int64_t M, int64_t fusion, const std::vector<Tensor>& others,
                     const std::vector<int64_t>& out_sizes) {
-    if (lowp_mode_ == WOQ_HIP_LOWP_FP16 && x.scalar_type() == at::kBFloat16 && M > 16 && fusion == WOQ_HIP_FUSE_NONE) {
-      // fp16 compute on bf16 rows beyond one row tile: the reference converts the rows to fp16 and casts
-      // the fp16 result back (csrc/cpu/aten/utils/woq.h:3076-3085)
-      return run_sorted(x.to(at::kHalf), M, fusion, others, out_sizes).to(at::kBFloat16);
-    }
     Tensor x2 = x.is_contiguous() ? x : x.contiguous();
     if ((uintptr_t)x2.data_ptr() % 16) x2 = x2.clone();  // the kernels read activation rows with 16-byte loads
     Tensor out = at::empty(out_sizes, x.options());
+    if (lowp_mode_ == WOQ_HIP_LOWP_FP16 && x.scalar_type() == at::kBFloat16 && M > 16 && fusion == WOQ_HIP_FUSE_NONE) {
+      // fp16 compute on bf16 rows beyond one row tile: the reference converts the rows to fp16 and casts
+      // the fp16 result to bf16 (csrc/cpu/aten/utils/woq.h:3076-3085).  The library converts the rows once;
+      // its fp16 kernels then write the bf16 output themselves.
+      Tensor xh = at::empty(x2.sizes(), x2.options().dtype(at::kHalf));
+      DeviceScope scope(x2);
+      check_rc(woq_hip_convert_activations(x2.data_ptr(), WOQ_HIP_ACT_BF16, xh.data_ptr(), WOQ_HIP_ACT_FP16,
+                                           x2.numel(), current_stream(x2)),
+               "woq_linear");
+      x2 = xh;
+    }
     woq_hip_linear_params p;
     memset(&p, 0, sizeof(p));
     p.struct_size = sizeof(p);
     p.x = x2.data_ptr();
-    p.x_dtype = act_code(x.scalar_type());
+    p.x_dtype = act_code(x2.scalar_type());
     p.M = M; p.K = K_; p.N = N_;
     p.qweight = packed_.data_ptr();
     p.weight_dtype = (int32_t)weight_dtype_;
@@ -406,7 +412,7 @@ class WoqLinearOpContext : public torch::CustomClassHolder {
       p.others[i] = keep.back().data_ptr();
     }
     p.out = out.data_ptr();
-    p.out_dtype = p.x_dtype;
+    p.out_dtype = act_code(x.scalar_type());
     DeviceScope scope(x2);
     p.stream = current_stream(x2);
     const bool int8 = lowp_mode_ == WOQ_HIP_LOWP_INT8;

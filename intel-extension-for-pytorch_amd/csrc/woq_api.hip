@@ -145,8 +145,13 @@ int woq_hip_linear(const woq_hip_linear_params* p) {
     return set_error("woq_linear: bad shape M=%lld K=%lld N=%lld", (long long)p->M, (long long)p->K, (long long)p->N);
   if (p->x_dtype != WOQ_HIP_ACT_BF16 && p->x_dtype != WOQ_HIP_ACT_FP16 && p->x_dtype != WOQ_HIP_ACT_FP32)
     return set_error("woq_linear: bad x_dtype %d", p->x_dtype);
-  if (p->out_dtype != p->x_dtype && p->out_dtype != WOQ_HIP_ACT_FP32)
-    return set_error("woq_linear: out_dtype must equal x_dtype or be fp32");
+  if (p->out_dtype != p->x_dtype && p->out_dtype != WOQ_HIP_ACT_FP32) {
+    const bool both16 = p->x_dtype != WOQ_HIP_ACT_FP32 &&
+                        (p->out_dtype == WOQ_HIP_ACT_FP16 || p->out_dtype == WOQ_HIP_ACT_BF16);
+    if (!both16 || p->fusion != WOQ_HIP_FUSE_NONE)
+      return set_error("woq_linear: out_dtype must equal x_dtype or be fp32 (without a post-op it may be the "
+                       "other 16-bit type)");
+  }
   if (p->lowp_mode < 0 || p->lowp_mode > 3) return set_error("woq_linear: bad lowp_mode %d", p->lowp_mode);
   if (p->M == 0) return 0;
   if (!p->x || !p->qweight || !p->out || !p->scales_f32 || !p->scales_f16 || !p->scales_bf16)
@@ -302,6 +307,16 @@ int woq_hip_dequant_weight(const void* qweight, int weight_dtype, int64_t N, int
   if (N > 0 && K > 0 && (!qweight || !scales_f32 || !out)) return set_error("dequant_weight: null pointer");
   return launch_dequant_weight(qweight, weight_dtype, N, K, scales_f32, zeros_u8, group_size, out, out_dtype,
                                (hipStream_t)stream);
+}
+
+int woq_hip_convert_activations(const void* src, int src_dtype, void* dst, int dst_dtype, int64_t count,
+                                void* stream) {
+  if (src_dtype < 0 || src_dtype > 2 || dst_dtype < 0 || dst_dtype > 2)
+    return set_error("convert_activations: bad dtype %d -> %d", src_dtype, dst_dtype);
+  if (count < 0) return set_error("convert_activations: bad count %lld", (long long)count);
+  if (count == 0) return 0;
+  if (!src || !dst) return set_error("convert_activations: null pointer argument");
+  return launch_convert_activations(src, src_dtype, dst, dst_dtype, count, (hipStream_t)stream);
 }
 
 int woq_hip_shuffle_activations(const void* x, int x_dtype, int64_t M, int64_t K, const int32_t* src, void* out,

@@ -386,8 +386,9 @@ __global__ __launch_bounds__(256) void woq_gemm_w4_kernel(const FpArgs f, const 
   // nothing waits on LDS.  Post-ops go through a per-wave LDS tile (the activation buffers are idle
   // after the last barrier) so that the element-wise tail sees consecutive columns in consecutive lanes. ----
   const int64_t ncol0 = (int64_t)nt0 * kTileN;
-  const int act = REGIME == kRegimeF16 ? WOQ_HIP_ACT_FP16 : WOQ_HIP_ACT_BF16;
-  const bool fast = f.fusion == WOQ_HIP_FUSE_NONE && f.out_dtype == act && (f.N % 4) == 0 &&
+  // (the output may be the other 16-bit type than the activations: fp16 rows converted from a bf16 tensor)
+  const bool out_f16 = f.out_dtype == WOQ_HIP_ACT_FP16;
+  const bool fast = f.fusion == WOQ_HIP_FUSE_NONE && (out_f16 || f.out_dtype == WOQ_HIP_ACT_BF16) && (f.N % 4) == 0 &&
                     ncol0 + G4_NTW * kTileN <= f.N && (((uintptr_t)f.out & 7) | ((uintptr_t)f.bias & 15)) == 0;
   const bool hb = f.bias != nullptr;
   if (fast) {
@@ -407,7 +408,7 @@ __global__ __launch_bounds__(256) void woq_gemm_w4_kernel(const FpArgs f, const 
           const float y2 = finalize_acc<REGIME>(acc[mt][t][2], hb, bias4[t][2]);
           const float y3 = finalize_acc<REGIME>(acc[mt][t][3], hb, bias4[t][3]);
           u2 o;
-          if constexpr (REGIME == kRegimeF16) {
+          if (out_f16) {
             o[0] = (uint32_t)f32_to_f16_bits(y0) | ((uint32_t)f32_to_f16_bits(y1) << 16);
             o[1] = (uint32_t)f32_to_f16_bits(y2) | ((uint32_t)f32_to_f16_bits(y3) << 16);
           } else {

@@ -54,6 +54,7 @@ int launch_pack_qparams(const float* scales, const float* zeros, int weight_dtyp
                         float* s32, void* s16, void* sb16, uint8_t* z8, uint32_t* sz, hipStream_t st);
 int launch_unpack_int4_zeros(const int32_t* zp32, int64_t rows, int64_t cols, int64_t cols_zp32,
                              float* out, hipStream_t st);
+int launch_convert_activations(const void* src, int src_dtype, void* dst, int dst_dtype, int64_t count, hipStream_t st);
 int launch_shuffle_activations(const void* x, int x_dtype, int64_t M, int64_t K, const int32_t* src, void* out,
                                hipStream_t st);
 int launch_shuffle_int4_weight(const void* plain, int64_t N, int64_t K, const int32_t* src, void* out,

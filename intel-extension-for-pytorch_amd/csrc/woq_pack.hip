@@ -279,6 +279,43 @@ __global__ void shuffle_int4_weight_kernel(const uint8_t* __restrict__ plain, in
   out[i] = v;
 }
 
+// Element-wise conversion between the activation dtypes, eight elements per thread where both
+// pointers allow 16-byte accesses of the narrower type.
+__global__ void convert_activations_kernel(const void* __restrict__ src, int src_dtype, void* __restrict__ dst,
+                                           int dst_dtype, int64_t count) {
+  const int64_t i0 = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * 8;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    const int64_t i = i0 + e;
+    if (i < count) store_act(dst, dst_dtype, i, load_act(src, src_dtype, i));
+  }
+}
+__global__ void convert_bf16_to_f16_kernel(const u4* __restrict__ src, u4* __restrict__ dst, int64_t chunks) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= chunks) return;
+  const u4 v = __builtin_nontemporal_load(src + i);
+  u4 o;
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    const float lo = bitcast<float>(v[e] << 16), hi = bitcast<float>(v[e] & 0xFFFF0000u);
+    o[e] = (uint32_t)f32_to_f16_bits(lo) | ((uint32_t)f32_to_f16_bits(hi) << 16);
+  }
+  dst[i] = o;
+}
+
+int launch_convert_activations(const void* src, int src_dtype, void* dst, int dst_dtype, int64_t count,
+                               hipStream_t st) {
+  if (count == 0) return 0;
+  if (src_dtype == WOQ_HIP_ACT_BF16 && dst_dtype == WOQ_HIP_ACT_FP16 && count % 8 == 0 &&
+      (((uintptr_t)src | (uintptr_t)dst) & 15) == 0) {
+    convert_bf16_to_f16_kernel<<<blocks_for(count / 8, 256), 256, 0, st>>>((const u4*)src, (u4*)dst, count / 8);
+  } else {
+    convert_activations_kernel<<<blocks_for((count + 7) / 8, 256), 256, 0, st>>>(src, src_dtype, dst, dst_dtype,
+                                                                                 count);
+  }
+  return check_launch("convert_activations");
+}
+
 int launch_shuffle_activations(const void* x, int x_dtype, int64_t M, int64_t K, const int32_t* src, void* out,
                                hipStream_t st) {
   const int64_t total = M * K;

@@ -181,11 +181,13 @@ def linear(
     force_kernel=0,
     debug_block_sums=False,
     noalloc=False,
+    out_dtype=None,
 ):
     """y = x @ dequant(W)^T (+ bias, post-op).  x: [..., K]; returns [..., N] in x.dtype, or the
     fp32 accumulator when ``out_fp32``.  With ``debug_block_sums`` also returns the int32 sum of
     every (m, n, K block) of the int8 path.  ``noalloc``: through ``woq_hip_linear_noalloc``, which
-    takes no workspace (the output tensor is still made here)."""
+    takes no workspace (the output tensor is still made here).  ``out_dtype``: without a post-op, the other
+    16-bit type than x's (fp16 rows converted from a bf16 tensor, bf16 output)."""
     lib = _lib.load()
     _require_cuda(x, "input")
     if x.dtype not in _ACT_CODE:
@@ -198,7 +200,7 @@ def linear(
     if x2.data_ptr() % 16:
         x2 = x2.clone()  # the kernels read activation rows with 16-byte loads
     M = x2.shape[0]
-    out_dtype = torch.float32 if out_fp32 else x.dtype
+    out_dtype = torch.float32 if out_fp32 else (out_dtype or x.dtype)
     out = torch.empty((M, N), dtype=out_dtype, device=x.device)
     p = _lib.LinearParams()
     p.struct_size = ctypes.sizeof(_lib.LinearParams)
@@ -277,6 +279,22 @@ def dequant_weight(qweight, weight_dtype, N, K, scales_f32, zeros_u8, group_size
                 _ACT_CODE[dtype], _stream()
             ),
             "dequant_weight",
+        )
+    return out
+
+
+def convert_activations(x, dtype):
+    """x converted to ``dtype`` (round to nearest even) by the library's own kernel."""
+    lib = _lib.load()
+    _require_cuda(x, "input")
+    if x.dtype not in _ACT_CODE or dtype not in _ACT_CODE:
+        raise RuntimeError(f"convert_activations: unsupported dtype {x.dtype} -> {dtype}")
+    x2 = x.contiguous()
+    out = torch.empty(x2.shape, dtype=dtype, device=x.device)
+    with torch.cuda.device(x.device):
+        _lib.check(
+            lib.woq_hip_convert_activations(_ptr(x2), _ACT_CODE[x.dtype], _ptr(out), _ACT_CODE[dtype], x2.numel(), _stream()),
+            "convert_activations",
         )
     return out
 

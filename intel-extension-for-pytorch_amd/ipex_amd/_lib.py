@@ -36,6 +36,7 @@ EXPORTS = [
     "woq_hip_linear",
     "woq_hip_linear_noalloc",
     "woq_hip_dequant_weight",
+    "woq_hip_convert_activations",
     "woq_hip_shuffle_activations",
     "woq_hip_shuffle_int4_weight",
     "woq_hip_moe_gather_rows",
@@ -132,6 +133,8 @@ def load():
         lib.woq_hip_linear_noalloc.argtypes = [ctypes.POINTER(LinearParams)]
         lib.woq_hip_dequant_weight.restype = i32
         lib.woq_hip_dequant_weight.argtypes = [vp, i32, i64, i64, vp, vp, i64, vp, i32, vp]
+        lib.woq_hip_convert_activations.restype = i32
+        lib.woq_hip_convert_activations.argtypes = [vp, i32, vp, i32, i64, vp]
         lib.woq_hip_shuffle_activations.restype = i32
         lib.woq_hip_shuffle_activations.argtypes = [vp, i32, i64, i64, vp, vp, vp]
         lib.woq_hip_shuffle_int4_weight.restype = i32

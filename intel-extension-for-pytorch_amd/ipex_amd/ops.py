@@ -352,10 +352,11 @@ class WoqLinearOpContext:
             and not kw
         ):
             # fp16 compute on bf16 activations beyond one row tile: the reference converts the rows to
-            # fp16 and casts the fp16 result back (csrc/cpu/aten/utils/woq.h:3076-3085); doing the two
-            # casts around the call reaches the kernels that want rows in the compute dtype
+            # fp16 and casts the fp16 result to bf16 (csrc/cpu/aten/utils/woq.h:3076-3085).  The library
+            # converts the rows once and its fp16 kernels write the bf16 output themselves
             # (M = 2048, 4096 -> 14336: 430 us through the converting general kernel otherwise)
-            return self._run_sorted(x.to(torch.float16), M, fusion, others, kw).to(torch.bfloat16)
+            x = _kernels.convert_activations(x, torch.float16)
+            kw = {"out_dtype": torch.bfloat16}
         if not kw and x.dtype in _kernels._ACT_CODE and x.is_cuda:
             return self._run_planned(x, M, fusion, others)
         return _kernels.linear(

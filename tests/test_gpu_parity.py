@@ -1413,6 +1413,69 @@ def test_g_idx_under_lowp_fp16_with_bf16_rows(cuda, M):
         assert rel_l2(to_np_f32(y), want) <= REL_L2_OUT, name
 
 
+@pytest.mark.parametrize("M,K,N,G,bias", [(17, 512, 96, 128, True), (64, 1024, 272, 128, False), (200, 512, 96, 128, True),
+                                          (300, 1024, 528, 64, False)])
+def test_lowp_fp16_on_bf16_rows_beyond_one_tile(cuda, M, K, N, G, bias):
+    """fp16 compute on a bf16 tensor of more than 16 rows: the library converts the rows to fp16 with its own
+    kernel and the fp16 kernels write the bf16 output (no casts around the call).  Equal, bit for bit, to the
+    same call on rows converted by torch with the fp16 result cast by torch; within the output gate of the
+    fallback in fp16 arithmetic; the same through the C++ operator."""
+    from ipex_amd import _kernels
+
+    case = _synthetic().make_int4_case(61, M, K, N, G, bias=bias)
+    ctx = make_context(case, O.LOWP_FP16)
+    x = case["x"].cuda()
+    xh = _kernels.convert_activations(x, torch.float16)
+    assert torch.equal(xh, x.to(torch.float16))
+    y = ctx.run(x)
+    assert y.dtype == torch.bfloat16
+    assert torch.equal(y, ctx.run(x.to(torch.float16)).to(torch.bfloat16))
+    c = case_np(case)
+    _, want = O.woq_linear_ref(c["x"], "bf16", c["qw"], N, K, O._round_to(c["scales"], "fp16"), c["zps"], c["bias"],
+                               2, G, "fp16")
+    assert rel_l2(to_np_f32(y), want) <= REL_L2_OUT
+    tc = make_torch_context(case, O.LOWP_FP16)
+    assert torch.equal(torch.ops.torch_ipex.ipex_woq_linear(x, tc.get_data_handle()), y)
+
+
+def test_convert_activations_rounds_to_nearest_even(cuda):
+    """Every dtype pair against torch's conversion, on every finite bf16 / fp16 bit pattern and on fp32 values
+    that sit on and beside rounding ties; ragged counts and a pointer that is not 16-byte aligned."""
+    from ipex_amd import _kernels
+
+    bits = torch.arange(0, 65536, dtype=torch.int32).to(torch.int16)
+    for src in (torch.bfloat16, torch.float16):
+        v = bits.view(src)
+        v = v[torch.isfinite(v.float())].cuda()
+        for dst in (torch.float16, torch.bfloat16, torch.float32):
+            got = _kernels.convert_activations(v, dst)
+            want = v.to(dst)
+            assert torch.equal(got.view(torch.int16 if dst != torch.float32 else torch.int32),
+                               want.view(torch.int16 if dst != torch.float32 else torch.int32)), (src, dst)
+    g = torch.Generator().manual_seed(5)
+    f = torch.randn(100003, generator=g) * 3.0
+    ties = (torch.arange(0, 4096, dtype=torch.int32) << 12 | 0x3F800000).view(torch.float32)  # fp16 / bf16 ties
+    f = torch.cat([f, ties, -ties, ties * (1 + 2.0 ** -20)]).cuda()
+    for dst in (torch.float16, torch.bfloat16):
+        assert torch.equal(_kernels.convert_activations(f, dst), f.to(dst)), dst
+    odd = torch.randn(4099, generator=g).bfloat16().cuda()[3:]  # 4096 elements, 6 bytes past an aligned address
+    assert torch.equal(_kernels.convert_activations(odd, torch.float16), odd.to(torch.float16))
+
+
+def test_other_16_bit_output_type_rejections(cuda):
+    """The other 16-bit output type is for plain calls only."""
+    from ipex_amd import _kernels, _lib
+
+    case = _synthetic().make_int4_case(62, 20, 256, 48, 128)
+    ctx = make_context(case, O.LOWP_FP16)
+    xh = case["x"].cuda().to(torch.float16)
+    other = torch.zeros(20, 48, dtype=torch.float16, device="cuda")
+    with pytest.raises(RuntimeError, match="other 16-bit type"):
+        ctx.run(xh, fusion=_lib.FUSE_ADD, others=(other,), out_dtype=torch.bfloat16)
+    with pytest.raises(RuntimeError, match="other 16-bit type"):
+        ctx.run(case["x"].cuda().float(), out_dtype=torch.bfloat16)
+
+
 def test_g_idx_validation(cuda):
     from ipex_amd import ops
 
