@@ -30,7 +30,7 @@ MFMA_FP32_PEAK_TFLOPS = 157.3   # MI355X dense fp32 matrix, published
 # the figure comes from two rocprofv3 --pmc runs of `bench.py --probe decode` (FETCH_SIZE 15310.55 KiB and
 # WRITE_SIZE 28.00 KiB per dispatch, scaled by what the same counters read for a 256 MiB copy: x2.000 and
 # x1.000), whose summary is the file named beside it; keyed by (M, K, N, group size).  Other shapes: null.
-PROFILED_HBM_BYTES_PER_LAUNCH = {(1, 4096, 14336, 128): 31339412}
+PROFILED_HBM_BYTES_PER_LAUNCH = {(1, 4096, 14336, 128): 31339793}
 PROFILED_HBM_BYTES_SOURCE = "profiles/woq_decode_m1_kernel_M1_4096x14336_g128.hbm_traffic_and_counters.txt"
 # Launches that precede every timed region whatever --warmup says: the first milliseconds after an idle
 # period run 3-10 % slower (clocks, translation caches).
@@ -568,10 +568,24 @@ def main():
     handle = tctx.get_data_handle()
     op = torch.ops.torch_ipex.ipex_woq_linear
     p0 = ctypes.byref(params[0])
+    sp = ctypes.c_void_p(stream.cuda_stream)
+    pz = _lib.LinearParams.from_buffer_copy(params[0])
+    pz.M = 0
+    pz_ref = ctypes.byref(pz)
+    probe_buf = torch.empty(K * N // 2, dtype=torch.uint8, device=dev)
+    probe_sink = torch.zeros(64, dtype=torch.int32, device=dev)
     host = {"c_abi_woq_hip_linear": host_us(lambda: lib.woq_hip_linear(p0)),
             "torch_ops_ipex_woq_linear": host_us(lambda: op(x, handle)),
+            # what the library adds to a launch: its argument checks alone (a call with M = 0 returns behind
+            # them); and what the runtime's launch path costs for a kernel of this duration and for an empty
+            # one, through the same library (with kernels longer than the host's time per call the launch
+            # queue grows during a burst, and the runtime's bookkeeping with it)
+            "c_abi_checks_only_M0": host_us(lambda: lib.woq_hip_linear(pz_ref)),
+            "c_abi_stream_read_probe_launch": host_us(
+                lambda: lib.woq_hip_probe_stream_read(probe_buf.data_ptr(), probe_buf.numel(), 16, 4, probe_sink.data_ptr(), sp)),
+            "c_abi_empty_kernel_launch": host_us(lambda: lib.woq_hip_probe_empty(448, 16, sp)),
             "what": "host microseconds per call, bursts of 200 calls on an idle device, no synchronization inside a burst"}
-    del tctx
+    del tctx, probe_buf
 
     us_launch = ev_ms * 1e3 / args.steps
     us_graph = g_ev_ms * 1e3 / g_steps
