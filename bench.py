@@ -606,8 +606,11 @@ def main():
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": ("bf16 activations x int4 weights -> fp32 accumulate (v_mfma_f32_16x16x32_bf16 on exact integer "
-                  "weights, group scale applied to the group sum in fp32; the reference's M < 5 arithmetic)") if M < 5
+        "dtype": ("bf16 activations (as fp16: exact in fp16's normal range) x int4 weights held as exact fp16 integers "
+                  "-> fp32 accumulate (v_mfma_f32_16x16x32_f16; the group scale is applied to the group sum in fp32; "
+                  "the reference's M < 5 kernel computes the same algebra with fp16 accumulators)") if M == 1
+                 else ("bf16 activations x int4 weights held as exact bf16 integers -> fp32 accumulate "
+                       "(v_mfma_f32_16x16x32_bf16; group scale applied to the group sum in fp32)") if M < 5
                  else "bf16 x bf16-rounded dequantized int4 -> fp32 accumulate (v_mfma_f32_16x16x32_bf16)",
         "data": "synthetic",
         "config": {
