@@ -58,6 +58,11 @@ extern "C" {
 #define WOQ_HIP_DTYPE_INT8 1
 #define WOQ_HIP_DTYPE_INT4 2
 #define WOQ_HIP_DTYPE_NF4 3
+/* FP8: float8 e4m3fn bytes, no zero points, not under WOQ_HIP_LOWP_INT8: w = conv(byte) * scale rounded once to
+ * the compute type (load_dequant_fp8, csrc/cpu/aten/utils/woq.h:728-741).  conv is the reference kernels'
+ * conversion (convert_fp8_e4m3_to_fp32, woq.h:465-485): the float8 value on +-0 and every normal code,
+ * (8 + m) * 2^-10 on the subnormal codes 0x01..0x07 (float8: m * 2^-9), +-480 on the NaN codes 0x7F / 0xFF. */
+#define WOQ_HIP_DTYPE_FP8 4
 
 /* lowp_mode, csrc/cpu/aten/utils/woq_defines.h:21-24 */
 #define WOQ_HIP_LOWP_NONE 0
@@ -120,6 +125,7 @@ int64_t woq_hip_packed_weight_bytes(int weight_dtype, int64_t N, int64_t K);
  *               low nibble and 2j+1 in the high nibble
  *               (intel_extension_for_pytorch/quantization/_quantize_utils.py:1184).
  *   INT8:       plain is int8 [N, K].
+ *   FP8:        plain is the float8 e4m3fn bytes [N, K].
  * Packed layout (the same bytes serve the small-M kernel, the MFMA GEMM and the int8 path):
  *   tiles [Np/16][Kp/tile_k], 1024 bytes each, K-tiles of one row block contiguous.
  *   Lane l = r + 16*c of a wave64 owns bytes [16*l, 16*l+16) of a tile: output row
@@ -128,6 +134,7 @@ int64_t woq_hip_packed_weight_bytes(int weight_dtype, int64_t N, int64_t K);
  *           element e stored in nibble position (e even ? e/2 : 4 + e/2), so that
  *           (dword >> 4*v) & 0x000F000F yields elements (2v, 2v+1) in the two 16-bit halves;
  *     INT8: K offsets 16*c .. 16*c+15, one per byte, stored offset-binary (value + 128).
+ *     FP8:  the same places, the bytes as they are.
  *   Padding rows / columns hold zero-weight encodings and never contribute.
  */
 int woq_hip_pack_weight(const void* plain, int weight_dtype, int64_t N, int64_t K,

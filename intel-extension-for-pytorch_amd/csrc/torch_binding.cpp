@@ -44,6 +44,7 @@ static int64_t weight_dtype_of(c10::string_view name) {
   if (name == "int8") return WOQ_HIP_DTYPE_INT8;
   if (name == "int4") return WOQ_HIP_DTYPE_INT4;
   if (name == "nf4") return WOQ_HIP_DTYPE_NF4;
+  if (name == "fp8") return WOQ_HIP_DTYPE_FP8;
   TORCH_CHECK(false, "Unsupported weight dtype: ", name);
   return 0;
 }
@@ -83,9 +84,11 @@ static void require_gpu_input(const Tensor& x, const char* name) {
 }
 
 // ---- C ABI wrappers on tensors ---------------------------------------------------------------------
+static bool is_8bit(int64_t wd) { return wd == WOQ_HIP_DTYPE_INT8 || wd == WOQ_HIP_DTYPE_FP8; }
+
 static Tensor pack_weight(const Tensor& plain_in, int64_t wd, int64_t N, int64_t K) {
   const Tensor plain = plain_in.contiguous();
-  const int64_t tk = wd == WOQ_HIP_DTYPE_INT8 ? WOQ_HIP_TILE_K_INT8 : WOQ_HIP_TILE_K_INT4;
+  const int64_t tk = is_8bit(wd) ? WOQ_HIP_TILE_K_INT8 : WOQ_HIP_TILE_K_INT4;
   const int64_t nt = woq_hip_padded_n(N) / WOQ_HIP_TILE_N, kt = woq_hip_padded_k((int)wd, K) / tk;
   Tensor packed = at::empty({nt, kt, WOQ_HIP_TILE_BYTES}, plain.options().dtype(at::kByte));
   DeviceScope scope(plain);
@@ -96,8 +99,9 @@ static Tensor pack_weight(const Tensor& plain_in, int64_t wd, int64_t N, int64_t
 
 static Tensor unpack_weight(const Tensor& packed, int64_t wd, int64_t N, int64_t K) {
   TORCH_CHECK(packed.is_cuda(), "packed weight must live on the GPU");
-  Tensor plain = wd == WOQ_HIP_DTYPE_INT8 ? at::empty({N, K}, packed.options().dtype(at::kChar))
-                                          : at::empty({N, (K + 1) / 2}, packed.options().dtype(at::kByte));
+  Tensor plain = wd == WOQ_HIP_DTYPE_FP8    ? at::empty({N, K}, packed.options().dtype(at::kFloat8_e4m3fn))
+                 : wd == WOQ_HIP_DTYPE_INT8 ? at::empty({N, K}, packed.options().dtype(at::kChar))
+                                            : at::empty({N, (K + 1) / 2}, packed.options().dtype(at::kByte));
   DeviceScope scope(packed);
   check_rc(woq_hip_unpack_weight(packed.data_ptr(), (int)wd, N, K, plain.data_ptr(), current_stream(packed)),
            "unpack_weight");
@@ -155,7 +159,7 @@ static PackedQParams pack_qparams(const Tensor& scales_in, const optional<Tensor
     zeros = zeros_in->to(at::kFloat).contiguous();
     q.z8 = at::empty({nt, KG, WOQ_HIP_TILE_N}, opt.dtype(at::kByte));
   }
-  if (wd != WOQ_HIP_DTYPE_INT8) q.sz = at::empty({nt, KG, WOQ_HIP_TILE_N}, opt.dtype(at::kInt));
+  if (!is_8bit(wd)) q.sz = at::empty({nt, KG, WOQ_HIP_TILE_N}, opt.dtype(at::kInt));
   DeviceScope scope(scales);
   check_rc(woq_hip_pack_qparams(scales.data_ptr<float>(), zeros.defined() ? zeros.data_ptr<float>() : nullptr, (int)wd,
                                 N, KG, q.s32.data_ptr<float>(), q.s16.data_ptr(), q.sb16.data_ptr(),
@@ -214,7 +218,9 @@ class WoqLinearOpContext : public torch::CustomClassHolder {
   }
 
   // ---- the reference's method surface ----
-  Tensor get_weight() { return packed_; }
+  // The packed bytes; for FP8 weights seen as float8 e4m3fn, the dtype the reference's packed weight keeps
+  // (tests/cpu/test_quantization_default_recipe.py:2211-2214).
+  Tensor get_weight() { return weight_dtype_ == WOQ_HIP_DTYPE_FP8 ? packed_.view(at::kFloat8_e4m3fn) : packed_; }
   optional<Tensor> get_bias() { return bias_; }
   Tensor get_scales() { return scales_plain_; }
   optional<Tensor> get_zero_points() { return zeros_plain_; }
@@ -264,7 +270,11 @@ class WoqLinearOpContext : public torch::CustomClassHolder {
     auto cpu = [](const optional<Tensor>& t) -> optional<Tensor> {
       return t.has_value() ? optional<Tensor>(t->detach().cpu()) : c10::nullopt;
     };
-    return State(to_public(packed_).cpu(), weight_dtype_, {N_, K_}, scales_plain_.detach().cpu(), cpu(zeros_plain_),
+    // float8 tensors do not pickle with every torch version: the state carries their bytes, which the
+    // constructor takes as well
+    Tensor w = to_public(packed_).cpu();
+    if (w.scalar_type() == at::kFloat8_e4m3fn) w = w.view(at::kByte);
+    return State(w, weight_dtype_, {N_, K_}, scales_plain_.detach().cpu(), cpu(zeros_plain_),
                  cpu(bias_), cpu(g_idx_), batch_size_, group_size_, lowp_mode_, act_quant_mode_, cache_weight_);
   }
 
@@ -288,15 +298,24 @@ class WoqLinearOpContext : public torch::CustomClassHolder {
             optional<Tensor> zero_points, optional<Tensor> bias, optional<Tensor> g_idx, optional<int64_t> batch_size,
             int64_t group_size, int64_t lowp_mode, int64_t act_quant_mode, bool cache_weight) {
     TORCH_CHECK(weight_dtype == WOQ_HIP_DTYPE_INT8 || weight_dtype == WOQ_HIP_DTYPE_INT4 ||
-                    weight_dtype == WOQ_HIP_DTYPE_NF4,
+                    weight_dtype == WOQ_HIP_DTYPE_NF4 || weight_dtype == WOQ_HIP_DTYPE_FP8,
                 "WOQ linear: unsupported weight dtype ", weight_dtype);
     TORCH_CHECK(!(weight_dtype == WOQ_HIP_DTYPE_NF4 && zero_points.has_value()),
                 "WOQ: symmetric quantization is required for NF4 or INT8 with lowp-mode INT8");
+    TORCH_CHECK(!(weight_dtype == WOQ_HIP_DTYPE_FP8 && zero_points.has_value()), "WOQ: FP8 weights take no zero points");
+    TORCH_CHECK(!(weight_dtype == WOQ_HIP_DTYPE_FP8 && lowp_mode == WOQ_HIP_LOWP_INT8),
+                "WOQ: lowp-mode INT8 does not take FP8 weights");
     TORCH_CHECK(weight_shape.size() == 2, "WOQ linear: weight shape must be [N, K]");
     const int64_t N = weight_shape[0], K = weight_shape[1];
     weight = to_gpu(weight);
     const auto dev = weight.device();
-    if (weight_dtype != WOQ_HIP_DTYPE_INT8) {
+    if (weight_dtype == WOQ_HIP_DTYPE_FP8) {
+      // float8 e4m3fn values, or their bytes
+      TORCH_CHECK((weight.scalar_type() == at::kFloat8_e4m3fn || weight.scalar_type() == at::kByte) && weight.dim() == 2 &&
+                      weight.size(0) == N && weight.size(1) == K,
+                  "WOQ linear: fp8 weight must be float8_e4m3fn [", N, ", ", K, "]");
+      weight = weight.contiguous().view(at::kByte);
+    } else if (weight_dtype != WOQ_HIP_DTYPE_INT8) {
       if (weight.scalar_type() != at::kByte) weight = weight.contiguous().view(at::kByte);
       TORCH_CHECK(weight.dim() == 2 && weight.size(0) == N && weight.size(1) == (K + 1) / 2,
                   "WOQ linear: 4-bit weight has shape ", weight.sizes(), ", expected [", N, ", ", (K + 1) / 2, "]");

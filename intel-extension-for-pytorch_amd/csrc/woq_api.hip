@@ -30,8 +30,9 @@ int check_launch(const char* what) {
 }
 
 static bool valid_wdtype(int d) {
-  return d == WOQ_HIP_DTYPE_INT8 || d == WOQ_HIP_DTYPE_INT4 || d == WOQ_HIP_DTYPE_NF4;
+  return d == WOQ_HIP_DTYPE_INT8 || d == WOQ_HIP_DTYPE_INT4 || d == WOQ_HIP_DTYPE_NF4 || d == WOQ_HIP_DTYPE_FP8;
 }
+static bool wdtype_is_8bit(int d) { return d == WOQ_HIP_DTYPE_INT8 || d == WOQ_HIP_DTYPE_FP8; }
 
 }  // namespace woq
 
@@ -48,12 +49,12 @@ const char* woq_hip_last_kernel(void) { return g_last_kernel; }
 int64_t woq_hip_padded_n(int64_t N) { return (N + kTileN - 1) / kTileN * kTileN; }
 
 int64_t woq_hip_padded_k(int weight_dtype, int64_t K) {
-  const int tk = weight_dtype == WOQ_HIP_DTYPE_INT8 ? kTileK8 : kTileK4;
+  const int tk = wdtype_is_8bit(weight_dtype) ? kTileK8 : kTileK4;
   return (K + tk - 1) / tk * tk;
 }
 
 int64_t woq_hip_packed_weight_bytes(int weight_dtype, int64_t N, int64_t K) {
-  const int tk = weight_dtype == WOQ_HIP_DTYPE_INT8 ? kTileK8 : kTileK4;
+  const int tk = wdtype_is_8bit(weight_dtype) ? kTileK8 : kTileK4;
   return woq_hip_padded_n(N) / kTileN * (woq_hip_padded_k(weight_dtype, K) / tk) * kTileBytes;
 }
 
@@ -175,7 +176,7 @@ int woq_hip_linear(const woq_hip_linear_params* p) {
   if (p->out_dtype == WOQ_HIP_ACT_FP32 && p->x_dtype != WOQ_HIP_ACT_FP32 && p->fusion != WOQ_HIP_FUSE_NONE)
     return set_error("woq_linear: the fp32 accumulator output does not take a post-op");
 
-  const int wbits = p->weight_dtype == WOQ_HIP_DTYPE_INT8 ? 8 : 4;
+  const int wbits = wdtype_is_8bit(p->weight_dtype) ? 8 : 4;
   const int tk = wbits == 4 ? kTileK4 : kTileK8;
   const int64_t NT = woq_hip_padded_n(p->N) / kTileN;
   const int64_t KT = woq_hip_padded_k(p->weight_dtype, p->K) / tk;
@@ -186,6 +187,10 @@ int woq_hip_linear(const woq_hip_linear_params* p) {
 
   const bool nf4 = p->weight_dtype == WOQ_HIP_DTYPE_NF4;
   if (nf4 && p->zeros_u8) return set_error("woq_linear: symmetric quantization is required for NF4 weights");
+  const bool fp8 = p->weight_dtype == WOQ_HIP_DTYPE_FP8;
+  if (fp8 && p->zeros_u8) return set_error("woq_linear: FP8 weights take no zero points");
+  if (fp8 && p->lowp_mode == WOQ_HIP_LOWP_INT8)
+    return set_error("woq_linear: lowp_mode INT8 does not take FP8 weights");
   int lowp = p->lowp_mode;
   if (lowp == WOQ_HIP_LOWP_INT8) {
     const int64_t bk = woq_hip_int8_block_k(p->group_size, p->K);
@@ -232,6 +237,7 @@ int woq_hip_linear(const woq_hip_linear_params* p) {
     a.qweight = (const uint8_t*)p->qweight; a.scales = p->scales_f32; a.zeros = p->zeros_u8;
     a.G = G; a.KG = KG; a.bias = p->bias; a.fusion = p->fusion;
     a.other0 = p->others[0]; a.other1 = p->others[1]; a.out = p->out; a.nf4 = nf4 ? 1 : 0;
+    a.fp8 = fp8 ? 1 : 0;
     return launch_fp32(a, wbits, st);
   } else {
     return set_error("woq_linear: lowp_mode %d does not take x_dtype %d", lowp, p->x_dtype);
@@ -244,6 +250,7 @@ int woq_hip_linear(const woq_hip_linear_params* p) {
   f.zeros = p->zeros_u8; f.G = G; f.KG = KG; f.bias = p->bias; f.fusion = p->fusion;
   f.other0 = p->others[0]; f.other1 = p->others[1]; f.out = p->out; f.out_dtype = p->out_dtype;
   f.nf4 = nf4 ? 1 : 0;
+  f.fp8 = fp8 ? 1 : 0;
   SplitKScratch scratch;
   if (p->split_k_counters && p->workspace && p->workspace_bytes > 0) {
     scratch.partial = (float*)p->workspace;

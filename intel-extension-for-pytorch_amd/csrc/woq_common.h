@@ -107,6 +107,57 @@ __device__ __forceinline__ b8 dequant8_bf16(uint32_t d, float s, float c) {
 
 // ---- 8-bit decode (bytes are offset-binary: stored = q + 128) ---------------------------
 // 8 consecutive K elements live in two dwords.
+// float8 e4m3fn byte (1 sign, 4 exponent bits with bias 7, 3 mantissa bits) -> fp32 the way the reference's
+// weight-only kernels convert it (convert_fp8_e4m3_to_fp32, csrc/cpu/aten/utils/woq.h:465-485): the 7 low bits
+// shifted to the fp32 exponent / mantissa boundary plus the bias difference (127 - 7) << 23, zero when those
+// bits are zero, then the sign.  Every code is read as a normal number: that is the float8 value for
+// exponents 1..15 and for +-0; the subnormal codes 0x01..0x07 give (8 + m) * 2^-10 where float8 means
+// m * 2^-9, and the NaN codes 0x7F / 0xFF give +-480.  Kept, so that a checkpoint gives the reference's numbers.
+__device__ __forceinline__ float fp8_e4m3fn_to_f32(uint32_t byte) {
+  const uint32_t mag = byte & 0x7Fu;
+  const uint32_t bits = mag ? (mag << 20) + (120u << 23) : 0u;
+  return bitcast<float>(bits | ((byte & 0x80u) << 24));
+}
+
+// The same conversion for two bytes at once, to fp16, where every one of its values is exact: v holds the bytes in
+// bits 15..8 and 31..24; the 7 low bits of each land on fp16's exponent / mantissa boundary (>> 1), the bias
+// difference (15 - 7) << 10 is added unless they are zero, the sign bit stays where it is.
+// (min(t, 1) * 0x2000 + t on 16-bit halves; written as the two packed instructions because the compiler turns the
+// same expression into a compare and a select per half.)
+__device__ __forceinline__ h2 fp8x2_to_f16x2(uint32_t v) {
+  const uint32_t t = (v & 0x7F007F00u) >> 1;
+  uint32_t nz, r;
+  asm("v_pk_min_u16 %0, %1, %2" : "=v"(nz) : "v"(t), "v"(0x00010001u));
+  asm("v_pk_mad_u16 %0, %1, %2, %3" : "=v"(r) : "v"(nz), "v"(0x20002000u), "v"(t));
+  return bitcast<h2>(r | (v & 0x80008000u));
+}
+
+// 8-bit weights as fp8: w = cd(fp8(byte) * s), one rounding (load_dequant_fp8, csrc/cpu/aten/utils/woq.h:728-741:
+// the converted value times the scale in the compute type).  fp16: the fp16 product of two fp16 numbers is that
+// rounding.  bf16: the product is exact in fp32 (4 x 8 significant bits) and rounded once.
+__device__ __forceinline__ h8 dequant8_f16_fp8(uint32_t d0, uint32_t d1, float s) {
+  const h2 sh = {(_Float16)s, (_Float16)s};  // exact: the fp16 regime reads fp16 scales
+  const h2 p0 = fp8x2_to_f16x2(__builtin_amdgcn_perm(0u, d0, 0x010c000cu)) * sh;
+  const h2 p1 = fp8x2_to_f16x2(__builtin_amdgcn_perm(0u, d0, 0x030c020cu)) * sh;
+  const h2 p2 = fp8x2_to_f16x2(__builtin_amdgcn_perm(0u, d1, 0x010c000cu)) * sh;
+  const h2 p3 = fp8x2_to_f16x2(__builtin_amdgcn_perm(0u, d1, 0x030c020cu)) * sh;
+  return h8{p0[0], p0[1], p1[0], p1[1], p2[0], p2[1], p3[0], p3[1]};
+}
+// fp32(fp16 half of v) * s in one mixed-precision instruction (a zero product comes out as +0)
+__device__ __forceinline__ f2 f16x2_times_f32(h2 v, float s) {
+  f2 r;
+  asm("v_fma_mix_f32 %0, %1, %2, 0 op_sel_hi:[1,0,0]" : "=v"(r[0]) : "v"(bitcast<uint32_t>(v)), "v"(s));
+  asm("v_fma_mix_f32 %0, %1, %2, 0 op_sel:[1,0,0] op_sel_hi:[1,0,0]" : "=v"(r[1]) : "v"(bitcast<uint32_t>(v)), "v"(s));
+  return r;
+}
+__device__ __forceinline__ b8 dequant8_bf16_fp8(uint32_t d0, uint32_t d1, float s) {
+  const b2 p0 = __builtin_convertvector(f16x2_times_f32(fp8x2_to_f16x2(__builtin_amdgcn_perm(0u, d0, 0x010c000cu)), s), b2);
+  const b2 p1 = __builtin_convertvector(f16x2_times_f32(fp8x2_to_f16x2(__builtin_amdgcn_perm(0u, d0, 0x030c020cu)), s), b2);
+  const b2 p2 = __builtin_convertvector(f16x2_times_f32(fp8x2_to_f16x2(__builtin_amdgcn_perm(0u, d1, 0x010c000cu)), s), b2);
+  const b2 p3 = __builtin_convertvector(f16x2_times_f32(fp8x2_to_f16x2(__builtin_amdgcn_perm(0u, d1, 0x030c020cu)), s), b2);
+  return b8{p0[0], p0[1], p1[0], p1[1], p2[0], p2[1], p3[0], p3[1]};
+}
+
 __device__ __forceinline__ h8 dequant8_f16_w8(uint32_t d0, uint32_t d1, float s, float c) {
   // w = fp16((u - uz) * s), computed as fma(u, s, -uz * s) in fp32 (exact for fp16/bf16-valued
   // scales: 8 bits x 11 bits) and rounded once to fp16.

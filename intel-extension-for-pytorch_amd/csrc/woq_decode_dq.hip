@@ -83,12 +83,13 @@ struct G8Consts {
 // reference's fp16 kernel converts them per K block (csrc/cpu/aten/utils/woq.h:3076-3079) -- the common
 // case of a bf16 model under lowp_mode BF16 with fewer than five rows.  The rows then travel through
 // registers (16-byte loads, conversion, ds_write to the same swizzled places) instead of the LDS DMA.
-template <int REGIME, int WBITS, int MT, int NTW, bool NF4, bool XCONV>
+template <int REGIME, int WBITS, int MT, int NTW, bool NF4, bool XCONV, bool FP8>
 __global__ __launch_bounds__(512, 4) void woq_decode_dq_kernel(const DecodeDqArgs a) {
   static_assert(!XCONV || (REGIME == kRegimeF16 && MT == 1), "bf16 -> fp16 rows: fp16 regime, one row tile");
   using Geo = DqGeom<WBITS, MT>;
   constexpr int TK = Geo::TK, NJ = Geo::NJ, NX = Geo::NX, SLICE = Geo::SLICE;
   static_assert(!NF4 || WBITS == 4, "NF4 codes are 4 bits wide");
+  static_assert(!FP8 || WBITS == 8, "float8 weights are bytes");
   extern __shared__ __align__(1024) uint8_t smem[];
   __shared__ f2 sNf4[NF4 ? kNf4LutEntries : 1];
   if constexpr (NF4) {
@@ -226,6 +227,11 @@ __global__ __launch_bounds__(512, 4) void woq_decode_dq_kernel(const DecodeDqArg
           bop = nf4_dequant<REGIME>(wreg[t][j], sNf4, qc8[t].s);
         } else if constexpr (WBITS == 4) {
           bop = g4_dequant(wreg[t][j], km, qc4[t]);
+        } else if constexpr (FP8) {
+          if constexpr (REGIME == kRegimeF16)
+            bop = bitcast<u4>(dequant8_f16_fp8(wreg[t][2 * j], wreg[t][2 * j + 1], qc8[t].s));
+          else
+            bop = bitcast<u4>(dequant8_bf16_fp8(wreg[t][2 * j], wreg[t][2 * j + 1], qc8[t].s));
         } else if constexpr (REGIME == kRegimeF16) {
           bop = bitcast<u4>(dequant8_f16_w8(wreg[t][2 * j], wreg[t][2 * j + 1], qc8[t].s, qc8[t].c));
         } else {
@@ -307,7 +313,7 @@ __global__ __launch_bounds__(512, 4) void woq_decode_dq_kernel(const DecodeDqArg
   if (threadIdx.x == 0) __hip_atomic_store(a.counters + blockIdx.x, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-template <int REGIME, int WBITS, int MT, int NTW, bool NF4 = false, bool XCONV = false>
+template <int REGIME, int WBITS, int MT, int NTW, bool NF4 = false, bool XCONV = false, bool FP8 = false>
 static int launch_dq_cfg(DecodeDqArgs a, int splits, hipStream_t st) {
   using Geo = DqGeom<WBITS, MT>;
   if (MT > 2 && splits > 1) return set_error("woq_decode_dq_kernel: split K takes at most 32 rows");
@@ -328,7 +334,7 @@ static int launch_dq_cfg(DecodeDqArgs a, int splits, hipStream_t st) {
   size_t smem = (size_t)a.W * 2 * Geo::SLICE;
   const size_t red = (size_t)NTW * MT * a.W * 64 * sizeof(f4);
   if (red > smem) smem = red;
-  auto kern = woq_decode_dq_kernel<REGIME, WBITS, MT, NTW, NF4, XCONV>;
+  auto kern = woq_decode_dq_kernel<REGIME, WBITS, MT, NTW, NF4, XCONV, FP8>;
   if (MT >= 2) {
     // more than 64 KiB of LDS per workgroup needs an opt-in (once per kernel and process)
     static const hipError_t lds_optin =
@@ -353,25 +359,25 @@ bool decode_dq_applies(const FpArgs& f, int wbits, int regime) {
   return f.G >= (wbits == 4 ? 32 : 16) && (f.G & (f.G - 1)) == 0;
 }
 
-template <int REGIME, int WBITS>
+template <int REGIME, int WBITS, bool FP8 = false>
 static int launch_dq_regime(const DecodeDqArgs& a, int ntw, int splits, hipStream_t st) {
   const int mt = a.f.M > 32 ? 4 : a.f.M > 16 ? 2 : 1;
   if constexpr (REGIME == kRegimeF16) {
     if (a.f.x_dtype == WOQ_HIP_ACT_BF16) {  // one row tile, rows converted to fp16 on the way in
-      if (ntw == 4) return launch_dq_cfg<REGIME, WBITS, 1, 4, false, true>(a, splits, st);
-      if (ntw == 2) return launch_dq_cfg<REGIME, WBITS, 1, 2, false, true>(a, splits, st);
-      return launch_dq_cfg<REGIME, WBITS, 1, 1, false, true>(a, splits, st);
+      if (ntw == 4) return launch_dq_cfg<REGIME, WBITS, 1, 4, false, true, FP8>(a, splits, st);
+      if (ntw == 2) return launch_dq_cfg<REGIME, WBITS, 1, 2, false, true, FP8>(a, splits, st);
+      return launch_dq_cfg<REGIME, WBITS, 1, 1, false, true, FP8>(a, splits, st);
     }
   }
   if (mt == 4) {
     // 33..64 rows: one or two row-blocks per workgroup (four would leave too few workgroups)
     if (ntw == 4) return set_error("woq_decode_dq_kernel: 33..64 rows take 1 or 2 row-blocks per workgroup");
-    return ntw == 2 ? launch_dq_cfg<REGIME, WBITS, 4, 2>(a, splits, st) : launch_dq_cfg<REGIME, WBITS, 4, 1>(a, splits, st);
+    return ntw == 2 ? launch_dq_cfg<REGIME, WBITS, 4, 2, false, false, FP8>(a, splits, st) : launch_dq_cfg<REGIME, WBITS, 4, 1, false, false, FP8>(a, splits, st);
   }
   const bool two_rows = mt == 2;
-  if (ntw == 4) return two_rows ? launch_dq_cfg<REGIME, WBITS, 2, 4>(a, splits, st) : launch_dq_cfg<REGIME, WBITS, 1, 4>(a, splits, st);
-  if (ntw == 2) return two_rows ? launch_dq_cfg<REGIME, WBITS, 2, 2>(a, splits, st) : launch_dq_cfg<REGIME, WBITS, 1, 2>(a, splits, st);
-  return two_rows ? launch_dq_cfg<REGIME, WBITS, 2, 1>(a, splits, st) : launch_dq_cfg<REGIME, WBITS, 1, 1>(a, splits, st);
+  if (ntw == 4) return two_rows ? launch_dq_cfg<REGIME, WBITS, 2, 4, false, false, FP8>(a, splits, st) : launch_dq_cfg<REGIME, WBITS, 1, 4, false, false, FP8>(a, splits, st);
+  if (ntw == 2) return two_rows ? launch_dq_cfg<REGIME, WBITS, 2, 2, false, false, FP8>(a, splits, st) : launch_dq_cfg<REGIME, WBITS, 1, 2, false, false, FP8>(a, splits, st);
+  return two_rows ? launch_dq_cfg<REGIME, WBITS, 2, 1, false, false, FP8>(a, splits, st) : launch_dq_cfg<REGIME, WBITS, 1, 1, false, false, FP8>(a, splits, st);
 }
 
 // NF4: one or two row-blocks per workgroup.
@@ -459,6 +465,11 @@ int launch_decode_dq(const FpArgs& f, int wbits, int regime, hipStream_t st, int
   if (wbits == 4)
     return regime == kRegimeF16 ? launch_dq_regime<kRegimeF16, 4>(a, ntw, splits, st)
                                 : launch_dq_regime<kRegimeBF16, 4>(a, ntw, splits, st);
+  if (f.fp8) {  // float8 bytes: own instances, so that the integer ones keep their registers
+    if (wbits != 8 || f.zeros) return set_error("woq_decode_dq_kernel: FP8 weights are bytes without zero points");
+    return regime == kRegimeF16 ? launch_dq_regime<kRegimeF16, 8, true>(a, ntw, splits, st)
+                                : launch_dq_regime<kRegimeBF16, 8, true>(a, ntw, splits, st);
+  }
   return regime == kRegimeF16 ? launch_dq_regime<kRegimeF16, 8>(a, ntw, splits, st)
                               : launch_dq_regime<kRegimeBF16, 8>(a, ntw, splits, st);
 }

@@ -122,6 +122,8 @@ __global__ __launch_bounds__(256) void woq_fp32_kernel(const Fp32Args f) {
         q = (float)((d[e >> 2] >> (8 * (e & 3))) & 0xFFu);
       if (NF4)
         w[e] = wvalid ? __fmul_rn(sTab[(int)q], s) : 0.0f;
+      else if (WBITS == 8 && f.fp8)  // float8 e4m3fn bytes: w = fp8(byte) * s (woq.h:728-741)
+        w[e] = wvalid ? __fmul_rn(fp8_e4m3fn_to_f32((d[e >> 2] >> (8 * (e & 3))) & 0xFFu), s) : 0.0f;
       else
         w[e] = wvalid ? __fmul_rn(__fsub_rn(q, z), s) : 0.0f;
     }

@@ -151,12 +151,22 @@ __global__ __launch_bounds__(256) void woq_gemm_kernel(const FpArgs f) {
       } else {
         const float s = REGIME == kRegimeF16 ? f16_bits_to_f32(sbits) : bf16_bits_to_f32(sbits);
         const float cc = -(z * s);
+        if (f.fp8) {  // (uniform) float8 e4m3fn bytes
 #pragma unroll
-        for (int j = 0; j < 2; ++j) {
-          if constexpr (REGIME == kRegimeF16)
-            wd[2 * q + j] = dequant8_f16_w8(wv[q][2 * j], wv[q][2 * j + 1], s, cc);
-          else
-            wd[2 * q + j] = dequant8_bf16_w8(wv[q][2 * j], wv[q][2 * j + 1], s, cc);
+          for (int j = 0; j < 2; ++j) {
+            if constexpr (REGIME == kRegimeF16)
+              wd[2 * q + j] = dequant8_f16_fp8(wv[q][2 * j], wv[q][2 * j + 1], s);
+            else
+              wd[2 * q + j] = dequant8_bf16_fp8(wv[q][2 * j], wv[q][2 * j + 1], s);
+          }
+        } else {
+#pragma unroll
+          for (int j = 0; j < 2; ++j) {
+            if constexpr (REGIME == kRegimeF16)
+              wd[2 * q + j] = dequant8_f16_w8(wv[q][2 * j], wv[q][2 * j + 1], s, cc);
+            else
+              wd[2 * q + j] = dequant8_bf16_w8(wv[q][2 * j], wv[q][2 * j + 1], s, cc);
+          }
         }
       }
     }

@@ -74,7 +74,7 @@ typedef const __attribute__((address_space(1))) void* global_ptr_t;
 // lie in the registers, and the workgroup that arrives last at the tile's counter adds the partial
 // tiles in z order (its own from the registers) and runs the epilogue.  Nobody waits; the order of
 // the sum is fixed.  All scratch accesses are relaxed device-scope atomics, as in the decode kernel.
-template <int REGIME, class S, int WBITS>
+template <int REGIME, class S, int WBITS, bool FP8>
 __global__ __launch_bounds__(256) void woq_gemm_w4_kernel(const FpArgs f, const int g_shift, float* const sk_partial,
                                                           int* const sk_counters, const int kts) {
   constexpr int TPS = WBITS / 4;  // packed tiles per row-block and K step of 128
@@ -201,7 +201,11 @@ __global__ __launch_bounds__(256) void woq_gemm_w4_kernel(const FpArgs f, const 
       return g4_dequant(wr[t][0][j], km, qc[t]);
     } else {
       const uint32_t d0 = wr[t][j / 2][2 * (j % 2)], d1 = wr[t][j / 2][2 * (j % 2) + 1];
-      if constexpr (REGIME == kRegimeF16)
+      if constexpr (FP8 && REGIME == kRegimeF16)  // float8 e4m3fn bytes
+        return bitcast<u4>(dequant8_f16_fp8(d0, d1, q8s[t]));
+      else if constexpr (FP8)
+        return bitcast<u4>(dequant8_bf16_fp8(d0, d1, q8s[t]));
+      else if constexpr (REGIME == kRegimeF16)
         return bitcast<u4>(dequant8_f16_w8(d0, d1, q8s[t], q8c[t]));
       else
         return bitcast<u4>(dequant8_bf16_w8(d0, d1, q8s[t], q8c[t]));
@@ -449,14 +453,14 @@ bool gemm_w4_applies(const FpArgs& f, int wbits, int regime) {
   return f.G >= (wbits == 4 ? 32 : 128) && (f.G & (f.G - 1)) == 0;
 }
 
-template <int REGIME, class S, int WBITS = 4>
+template <int REGIME, class S, int WBITS = 4, bool FP8 = false>
 static int launch_shape(const FpArgs& f, int g_shift, hipStream_t st, int splits = 1,
                         const SplitKScratch* scratch = nullptr) {
   constexpr int kLds = g4_lds_bytes<S, WBITS>();
   static_assert(kLds <= 160 * 1024, "a workgroup's LDS");
   // more than 64 KiB of LDS per workgroup needs an opt-in (once per kernel and process)
   static const hipError_t lds_optin =
-      hipFuncSetAttribute(reinterpret_cast<const void*>(&woq_gemm_w4_kernel<REGIME, S, WBITS>),
+      hipFuncSetAttribute(reinterpret_cast<const void*>(&woq_gemm_w4_kernel<REGIME, S, WBITS, FP8>),
                           hipFuncAttributeMaxDynamicSharedMemorySize, kLds);
   if (lds_optin != hipSuccess)
     return set_error("woq_gemm_w4_kernel: LDS opt-in failed: %s", hipGetErrorString(lds_optin));
@@ -475,7 +479,7 @@ static int launch_shape(const FpArgs& f, int g_shift, hipStream_t st, int splits
       return set_error("woq_gemm_w4_kernel: split K needs %lld bytes of workspace, the counter array and at most %d "
                        "tiles", (long long)need, kSplitKCounters);
   }
-  woq_gemm_w4_kernel<REGIME, S, WBITS><<<grid, 256, kLds, st>>>(f, g_shift, splits > 1 ? scratch->partial : nullptr,
+  woq_gemm_w4_kernel<REGIME, S, WBITS, FP8><<<grid, 256, kLds, st>>>(f, g_shift, splits > 1 ? scratch->partial : nullptr,
                                                                  splits > 1 ? scratch->counters : nullptr, kts);
   return check_launch("woq_gemm_w4_kernel");
 }
@@ -498,6 +502,17 @@ static int pick_splits(const FpArgs& f, int wbits, int64_t tiles, const SplitKSc
     if (tiles * s <= 256 && ksteps / s >= 16 && scratch->bytes >= need) return s;
   }
   return 1;
+}
+
+// 8-bit weights of one shape: integers or float8 bytes, fp16 or bf16 compute
+template <class S>
+static int launch8(const FpArgs& f, int regime, int g_shift, hipStream_t st, int splits = 1,
+                   const SplitKScratch* scratch = nullptr) {
+  if (f.fp8)
+    return regime == kRegimeF16 ? launch_shape<kRegimeF16, S, 8, true>(f, g_shift, st, splits, scratch)
+                                : launch_shape<kRegimeBF16, S, 8, true>(f, g_shift, st, splits, scratch);
+  return regime == kRegimeF16 ? launch_shape<kRegimeF16, S, 8>(f, g_shift, st, splits, scratch)
+                              : launch_shape<kRegimeBF16, S, 8>(f, g_shift, st, splits, scratch);
 }
 
 int launch_gemm_w4(const FpArgs& f, int wbits, int regime, hipStream_t st, int shape, int splits,
@@ -530,15 +545,12 @@ int launch_gemm_w4(const FpArgs& f, int wbits, int regime, hipStream_t st, int s
     if (shape == 0) shape = wgs42 <= 256 ? 42 : (shape_cost<S4>(f) <= shape_cost<S2>(f) ? 4 : 2);
     if (shape == 42) {
       if (splits == 0) splits = pick_splits(f, 8, wgs42, scratch);
-      return regime == kRegimeF16 ? launch_shape<kRegimeF16, S42, 8>(f, g_shift, st, splits, scratch)
-                                  : launch_shape<kRegimeBF16, S42, 8>(f, g_shift, st, splits, scratch);
+      return launch8<S42>(f, regime, g_shift, st, splits, scratch);
     }
     if (splits > 1) return set_error("woq_gemm_w4_kernel: K is split for the 64 x 128 shape only");
     if (shape == 4)
-      return regime == kRegimeF16 ? launch_shape<kRegimeF16, S4, 8>(f, g_shift, st)
-                                  : launch_shape<kRegimeBF16, S4, 8>(f, g_shift, st);
-    return regime == kRegimeF16 ? launch_shape<kRegimeF16, S2, 8>(f, g_shift, st)
-                                : launch_shape<kRegimeBF16, S2, 8>(f, g_shift, st);
+      return launch8<S4>(f, regime, g_shift, st);
+    return launch8<S2>(f, regime, g_shift, st);
   }
   if (shape == 0) {
     // Small M x N: 64 x 128 tiles at four waves per SIMD (79 + 32 registers, 48 KiB of LDS).  While

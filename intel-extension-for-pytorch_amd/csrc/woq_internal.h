@@ -33,6 +33,7 @@ struct FpArgs {
   void* out;
   int out_dtype;
   int nf4;  // 4-bit codes index the NF4 table instead of standing for integers (zeros == nullptr)
+  int fp8;  // 8-bit weights are float8 e4m3fn bytes, not offset-binary integers (zeros == nullptr)
 };
 
 // Split-K scratch of the dequantizing decode kernel: fp32 partial tiles, and one counter per
@@ -102,6 +103,7 @@ struct Fp32Args {
   const void* other1;
   void* out;
   int nf4;
+  int fp8;  // 8-bit weights are float8 e4m3fn bytes (symmetric)
 };
 int launch_fp32(const Fp32Args& f, int wbits, hipStream_t st);
 

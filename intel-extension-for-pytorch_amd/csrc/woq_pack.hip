@@ -57,8 +57,10 @@ __global__ void unpack_int4_kernel(const uint32_t* __restrict__ packed, uint8_t*
 }
 
 // One thread per packed dword (4 K elements of one row).
+// flip = 0x80: int8 values become offset-binary bytes (q + 128), padding is the byte of zero; flip = 0: float8
+// bytes are stored as they are, padding is +0.
 __global__ void pack_int8_kernel(const int8_t* __restrict__ plain, uint32_t* __restrict__ packed,
-                                 int64_t N, int64_t K, int64_t KT, int64_t total_dwords) {
+                                 int64_t N, int64_t K, int64_t KT, int64_t total_dwords, uint32_t flip) {
   const int64_t gid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (gid >= total_dwords) return;
   const int j = gid & 3;
@@ -68,13 +70,13 @@ __global__ void pack_int8_kernel(const int8_t* __restrict__ plain, uint32_t* __r
   const int r = lane & 15, c = lane >> 4;
   const int64_t n = nt * kTileN + r;
   const int64_t kbase = kt * kTileK8 + c * 16 + j * 4;
-  uint32_t out = 0x80808080u;  // offset-binary zero
+  uint32_t out = flip * 0x01010101u;  // the stored byte of zero, four times
   if (n < N) {
     out = 0;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int64_t k = kbase + i;
-      const uint32_t u = (k < K) ? (uint32_t)(uint8_t)(plain[n * K + k] ^ (int8_t)0x80) : 0x80u;
+      const uint32_t u = (k < K) ? ((uint32_t)(uint8_t)plain[n * K + k] ^ flip) : flip;
       out |= u << (8 * i);
     }
   }
@@ -82,7 +84,7 @@ __global__ void pack_int8_kernel(const int8_t* __restrict__ plain, uint32_t* __r
 }
 
 __global__ void unpack_int8_kernel(const uint8_t* __restrict__ packed, int8_t* __restrict__ plain,
-                                   int64_t N, int64_t K, int64_t KT) {
+                                   int64_t N, int64_t K, int64_t KT, uint32_t flip) {
   const int64_t gid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (gid >= N * K) return;
   const int64_t n = gid / K, k = gid % K;
@@ -91,7 +93,7 @@ __global__ void unpack_int8_kernel(const uint8_t* __restrict__ packed, int8_t* _
   const int koff = k % kTileK8;
   const int c = koff / 16, i = koff % 16;
   const uint8_t u = packed[((nt * KT + kt) * 64 + (r + 16 * c)) * 16 + i];
-  plain[gid] = (int8_t)(u ^ 0x80u);
+  plain[gid] = (int8_t)(u ^ flip);
 }
 
 __global__ void pack_qparams_kernel(const float* __restrict__ scales, const float* __restrict__ zeros,
@@ -143,7 +145,8 @@ __global__ void dequant_weight_kernel(const uint8_t* __restrict__ packed, int we
   const int64_t n = gid / K8, k0 = (gid % K8) * 8;
   const int64_t nt = n / kTileN;
   const int r = n % kTileN;
-  const bool w4 = weight_dtype != WOQ_HIP_DTYPE_INT8;
+  const bool fp8 = weight_dtype == WOQ_HIP_DTYPE_FP8;
+  const bool w4 = weight_dtype != WOQ_HIP_DTYPE_INT8 && !fp8;
   const int tile_k = w4 ? kTileK4 : kTileK8;
   const int64_t kt = k0 / tile_k;
   const int koff = k0 % tile_k;
@@ -165,7 +168,7 @@ __global__ void dequant_weight_kernel(const uint8_t* __restrict__ packed, int we
     const int c = koff / 16, i0 = koff % 16;
     const uint8_t* p = packed + ((nt * KT + kt) * 64 + (r + 16 * c)) * 16 + i0;
 #pragma unroll
-    for (int e = 0; e < 8; ++e) w[e] = (float)p[e];
+    for (int e = 0; e < 8; ++e) w[e] = fp8 ? fp8_e4m3fn_to_f32(p[e]) : (float)p[e];
   }
   const bool nf4 = weight_dtype == WOQ_HIP_DTYPE_NF4;
 #pragma unroll
@@ -174,7 +177,8 @@ __global__ void dequant_weight_kernel(const uint8_t* __restrict__ packed, int we
     if (k >= K) break;
     // (q - z) first, then the scale, each in fp32 (woq_utils.h:147-161); NF4: table value times
     // scale (woq_utils.h:165-262)
-    const float v = nf4 ? __fmul_rn(kNf4Values[(int)w[e]], s) : __fmul_rn(__fsub_rn(w[e], z), s);
+    // float8: the converted byte times the scale (woq.h:728-741)
+    const float v = nf4 ? __fmul_rn(kNf4Values[(int)w[e]], s) : fp8 ? __fmul_rn(w[e], s) : __fmul_rn(__fsub_rn(w[e], z), s);
     store_act(out, out_dtype, n * K + k, v);
   }
 }
@@ -184,13 +188,14 @@ static inline unsigned blocks_for(int64_t n, int bs) { return (unsigned)((n + bs
 int launch_pack_weight(const void* plain, int weight_dtype, int64_t N, int64_t K, void* packed,
                        hipStream_t st) {
   const int64_t Np = woq_hip_padded_n(N), Kp = woq_hip_padded_k(weight_dtype, K);
-  const int tile_k = weight_dtype == WOQ_HIP_DTYPE_INT8 ? kTileK8 : kTileK4;
+  const bool w8 = weight_dtype == WOQ_HIP_DTYPE_INT8 || weight_dtype == WOQ_HIP_DTYPE_FP8;
+  const int tile_k = w8 ? kTileK8 : kTileK4;
   const int64_t KT = Kp / tile_k;
   const int64_t total = (Np / kTileN) * KT * (kTileBytes / 4);
   if (total == 0) return 0;
-  if (weight_dtype == WOQ_HIP_DTYPE_INT8)
-    pack_int8_kernel<<<blocks_for(total, 256), 256, 0, st>>>((const int8_t*)plain, (uint32_t*)packed, N,
-                                                             K, KT, total);
+  if (w8)
+    pack_int8_kernel<<<blocks_for(total, 256), 256, 0, st>>>((const int8_t*)plain, (uint32_t*)packed, N, K, KT, total,
+                                                             weight_dtype == WOQ_HIP_DTYPE_FP8 ? 0u : 0x80u);
   else
     pack_int4_kernel<<<blocks_for(total, 256), 256, 0, st>>>((const uint8_t*)plain, (uint32_t*)packed,
                                                              N, K, KT, total);
@@ -201,9 +206,10 @@ int launch_unpack_weight(const void* packed, int weight_dtype, int64_t N, int64_
                          hipStream_t st) {
   const int64_t Kp = woq_hip_padded_k(weight_dtype, K);
   if (N == 0 || K == 0) return 0;
-  if (weight_dtype == WOQ_HIP_DTYPE_INT8) {
-    unpack_int8_kernel<<<blocks_for(N * K, 256), 256, 0, st>>>((const uint8_t*)packed, (int8_t*)plain, N,
-                                                               K, Kp / kTileK8);
+  if (weight_dtype == WOQ_HIP_DTYPE_INT8 || weight_dtype == WOQ_HIP_DTYPE_FP8) {
+    unpack_int8_kernel<<<blocks_for(N * K, 256), 256, 0, st>>>((const uint8_t*)packed, (int8_t*)plain, N, K,
+                                                               Kp / kTileK8,
+                                                               weight_dtype == WOQ_HIP_DTYPE_FP8 ? 0u : 0x80u);
   } else {
     const int64_t total = N * ((K + 1) / 2);
     unpack_int4_kernel<<<blocks_for(total, 256), 256, 0, st>>>((const uint32_t*)packed, (uint8_t*)plain,
@@ -236,7 +242,7 @@ int launch_dequant_weight(const void* qweight, int weight_dtype, int64_t N, int6
                           const uint8_t* z8, int64_t G, void* out, int out_dtype, hipStream_t st) {
   if (N == 0 || K == 0) return 0;
   const int64_t Kp = woq_hip_padded_k(weight_dtype, K);
-  const int tile_k = weight_dtype == WOQ_HIP_DTYPE_INT8 ? kTileK8 : kTileK4;
+  const int tile_k = (weight_dtype == WOQ_HIP_DTYPE_INT8 || weight_dtype == WOQ_HIP_DTYPE_FP8) ? kTileK8 : kTileK4;
   const int64_t KG = G > 0 ? (K + G - 1) / G : 1;
   const int64_t total = N * ((K + 7) / 8);
   dequant_weight_kernel<<<blocks_for(total, 256), 256, 0, st>>>((const uint8_t*)qweight, weight_dtype, N,

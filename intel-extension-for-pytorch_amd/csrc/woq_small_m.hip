@@ -73,7 +73,8 @@ __device__ __forceinline__ LaneQ<WBITS, REGIME> make_laneq(uint16_t sbits, bool 
 
 template <int WBITS, int REGIME>
 __device__ __forceinline__ void dequant_tile(const u4& w, const LaneQ<WBITS, REGIME>& q,
-                                             typename RegimeTraits<REGIME>::vec8 (&a)[WBITS == 4 ? 4 : 2]) {
+                                             typename RegimeTraits<REGIME>::vec8 (&a)[WBITS == 4 ? 4 : 2],
+                                             bool fp8 = false) {
   if (WBITS == 4) {
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
@@ -81,6 +82,14 @@ __device__ __forceinline__ void dequant_tile(const u4& w, const LaneQ<WBITS, REG
         a[j] = dequant8_f16(w[j], q.nz, q.s2);
       else
         a[j] = dequant8_bf16(w[j], q.s, q.c);
+    }
+  } else if (fp8) {  // (uniform) float8 e4m3fn bytes
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      if constexpr (REGIME == kRegimeF16)
+        a[j] = dequant8_f16_fp8(w[2 * j], w[2 * j + 1], q.s);
+      else
+        a[j] = dequant8_bf16_fp8(w[2 * j], w[2 * j + 1], q.s);
     }
   } else {
 #pragma unroll
@@ -214,7 +223,7 @@ __global__ __launch_bounds__(1024) void woq_small_m_kernel(const SmallMArgs a) {
 #pragma unroll
           for (int j = 0; j < STEPS; ++j) aop[j] = bitcast<vec8>(nf4_dequant<REGIME>(wreg[t][i][j], sNf4, s));
         } else {
-          dequant_tile<WBITS, REGIME>(wreg[t][i], q, aop);
+          dequant_tile<WBITS, REGIME>(wreg[t][i], q, aop, WBITS == 8 && f.fp8);
         }
 #pragma unroll
         for (int j = 0; j < STEPS; ++j)

@@ -36,11 +36,14 @@ def padded_k(weight_dtype, K):
 
 
 def pack_weight(plain, weight_dtype, N, K):
-    """Plain [N, ceil(K/2)] uint8 (4-bit) or [N, K] int8 -> packed tiles [NT, KT, 1024] uint8."""
+    """Plain [N, ceil(K/2)] uint8 (4-bit), [N, K] int8, or [N, K] float8_e4m3fn / uint8 bytes (FP8) -> packed tiles
+    [NT, KT, 1024] uint8."""
     lib = _lib.load()
     _require_cuda(plain, "qweight")
     plain = plain.contiguous()
-    tk = _lib.TILE_K_INT8 if weight_dtype == _lib.DTYPE_INT8 else _lib.TILE_K_INT4
+    if weight_dtype == _lib.DTYPE_FP8 and plain.dtype != torch.uint8:
+        plain = plain.view(torch.uint8)
+    tk = _lib.TILE_K_INT8 if weight_dtype in _lib.DTYPES_8BIT else _lib.TILE_K_INT4
     nt, kt = padded_n(N) // _lib.TILE_N, padded_k(weight_dtype, K) // tk
     packed = torch.empty((nt, kt, _lib.TILE_BYTES), dtype=torch.uint8, device=plain.device)
     with torch.cuda.device(plain.device):
@@ -51,7 +54,9 @@ def pack_weight(plain, weight_dtype, N, K):
 def unpack_weight(packed, weight_dtype, N, K):
     lib = _lib.load()
     _require_cuda(packed, "packed weight")
-    if weight_dtype == _lib.DTYPE_INT8:
+    if weight_dtype == _lib.DTYPE_FP8:
+        plain = torch.empty((N, K), dtype=torch.float8_e4m3fn, device=packed.device)
+    elif weight_dtype == _lib.DTYPE_INT8:
         plain = torch.empty((N, K), dtype=torch.int8, device=packed.device)
     else:
         plain = torch.empty((N, (K + 1) // 2), dtype=torch.uint8, device=packed.device)
@@ -80,7 +85,7 @@ def pack_qparams(scales, zeros, weight_dtype):
         assert zeros.shape == scales.shape
         z8 = torch.empty((nt, KG, _lib.TILE_N), dtype=torch.uint8, device=dev)
     sz = None
-    if weight_dtype != _lib.DTYPE_INT8:
+    if weight_dtype not in _lib.DTYPES_8BIT:
         sz = torch.empty((nt, KG, _lib.TILE_N), dtype=torch.int32, device=dev)
     with torch.cuda.device(dev):
         _lib.check(

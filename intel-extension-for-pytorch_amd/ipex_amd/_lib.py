@@ -11,7 +11,8 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(os.path.dirname(_HERE), "lib", "libwoq_hip.so")
 
 # weight dtype / lowp mode / fusion codes of the C ABI
-DTYPE_INT8, DTYPE_INT4, DTYPE_NF4 = 1, 2, 3
+DTYPE_INT8, DTYPE_INT4, DTYPE_NF4, DTYPE_FP8 = 1, 2, 3, 4
+DTYPES_8BIT = (DTYPE_INT8, DTYPE_FP8)
 LOWP_NONE, LOWP_FP16, LOWP_BF16, LOWP_INT8 = 0, 1, 2, 3
 ACT_FP32, ACT_FP16, ACT_BF16 = 0, 1, 2
 FUSE_NONE, FUSE_GELU_ERF, FUSE_GELU_TANH, FUSE_RELU, FUSE_SILU = 0x0, 0x1, 0x2, 0x3, 0x4

@@ -182,7 +182,7 @@ class WeightOnlyQuantizedLinear(nn.Module):
             act_quant_mode = getattr(mod.qconfig, "act_quant_mode", act_quant_mode)
             if hasattr(mod.qconfig, "cache_weight_for_large_batch"):
                 cache_weight_for_large_batch = mod.qconfig.cache_weight_for_large_batch and lowp_mode in (2, 3)
-        supported = [torch.int32, torch.uint8, torch.int8, torch.quint4x2, torch.bfloat16, torch.float32]
+        supported = [torch.int32, torch.uint8, torch.int8, torch.quint4x2, torch.bfloat16, torch.float32, torch.float8_e4m3fn]
         assert qweight.dtype in supported, "Data type of quantized weight should be in {}, but got: {}".format(
             supported, qweight.dtype
         )

@@ -36,7 +36,7 @@ _current_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None) or (
 )
 _current_device = getattr(torch._C, "_cuda_getDevice", None) or torch.cuda.current_device
 
-WOQ_DTYPE_MAP = {"int8": _lib.DTYPE_INT8, "int4": _lib.DTYPE_INT4, "nf4": _lib.DTYPE_NF4}
+WOQ_DTYPE_MAP = {"int8": _lib.DTYPE_INT8, "int4": _lib.DTYPE_INT4, "nf4": _lib.DTYPE_NF4, "fp8": _lib.DTYPE_FP8}
 PLAIN_WEIGHT_FORMAT, GPTQ_WEIGHT_FORMAT, AWQ_WEIGHT_FORMAT = 0, 1, 2
 
 _contexts = {}
@@ -91,14 +91,23 @@ class WoqLinearOpContext:
         cache_weight_for_large_batch=False,
     ):
         weight_dtype = int(weight_dtype)
-        if weight_dtype not in (_lib.DTYPE_INT8, _lib.DTYPE_INT4, _lib.DTYPE_NF4):
+        if weight_dtype not in (_lib.DTYPE_INT8, _lib.DTYPE_INT4, _lib.DTYPE_NF4, _lib.DTYPE_FP8):
             raise RuntimeError(f"WOQ linear: unsupported weight dtype {weight_dtype}")
         if weight_dtype == _lib.DTYPE_NF4 and zero_points is not None:
             raise RuntimeError("WOQ: symmetric quantization is required for NF4 or INT8 with lowp-mode INT8")
+        if weight_dtype == _lib.DTYPE_FP8 and zero_points is not None:
+            raise RuntimeError("WOQ: FP8 weights take no zero points")
+        if weight_dtype == _lib.DTYPE_FP8 and int(lowp_mode) == _lib.LOWP_INT8:
+            raise RuntimeError("WOQ: lowp-mode INT8 does not take FP8 weights")
         N, K = int(weight_shape[0]), int(weight_shape[1])
         weight = _to_gpu(weight)
         dev = weight.device
-        if weight_dtype != _lib.DTYPE_INT8:
+        if weight_dtype == _lib.DTYPE_FP8:
+            # float8 e4m3fn values, or their bytes
+            if weight.dtype not in (torch.float8_e4m3fn, torch.uint8) or tuple(weight.shape) != (N, K):
+                raise RuntimeError(f"WOQ linear: fp8 weight must be float8_e4m3fn [{N}, {K}]")
+            weight = weight.view(torch.uint8)
+        elif weight_dtype != _lib.DTYPE_INT8:
             weight = weight.view(torch.uint8) if weight.dtype != torch.uint8 else weight
             if tuple(weight.shape) != (N, (K + 1) // 2):
                 raise RuntimeError(
@@ -179,6 +188,8 @@ class WoqLinearOpContext:
 
     # ---- reference method surface ----
     def get_weight(self):
+        if self.weight_dtype_ == _lib.DTYPE_FP8:
+            return self.at_weight_.view(torch.float8_e4m3fn)
         return self.at_weight_
 
     def get_bias(self):
@@ -227,8 +238,13 @@ class WoqLinearOpContext:
     # ---- pickling: always the plain format, re-prepacked on load (OpContext.h:363-403) ----
     def __getstate__(self):
         cpu = lambda t: None if t is None else t.detach().cpu()
+        weight = cpu(self.to_public(self.at_weight_))
+        if weight.dtype == torch.float8_e4m3fn:
+            # float8 tensors do not pickle with every torch version: the state carries their bytes,
+            # which the constructor takes as well
+            weight = weight.view(torch.uint8)
         return (
-            cpu(self.to_public(self.at_weight_)),
+            weight,
             self.weight_dtype_,
             list(self.weight_shape_),
             cpu(self.scales_plain_),

@@ -51,3 +51,18 @@ def make_int8_case(cfg, M, K, N, bias=True, group_size=-1):
     b = (0.02 * torch.randn(N, generator=_gen(cfg, 4))).to(torch.bfloat16) if bias else None
     return dict(x=x, qweight=qweight, scales=scales, zeros=None, bias=b, M=M, K=K, N=N,
                 group_size=group_size, weight_dtype=1)
+
+
+def make_fp8_case(cfg, M, K, N, bias=True, group_size=-1, x_dtype=torch.bfloat16):
+    """float8 e4m3fn weights: every byte except the two NaN codes, uniform (so all exponents and the
+    subnormals occur), fp32 scales uniform in [0.0005, 0.002] per output channel (or per group of
+    ``group_size`` input channels), no zero points, bias ~ N(0, 0.02)."""
+    x = torch.randn(M, K, generator=_gen(cfg, 0)).to(x_dtype)
+    code = torch.randint(0, 254, (N, K), dtype=torch.int16, generator=_gen(cfg, 1))
+    code = code + (code >= 0x7F).to(torch.int16)  # skips 0x7F; 0xFF is out of range
+    qweight = code.to(torch.uint8).view(torch.float8_e4m3fn)
+    shape = (N,) if group_size <= 0 else (N, (K + group_size - 1) // group_size)
+    scales = 0.0005 + 0.0015 * torch.rand(shape, generator=_gen(cfg, 2))
+    b = (0.02 * torch.randn(N, generator=_gen(cfg, 4))).to(x_dtype) if bias else None
+    return dict(x=x, qweight=qweight, scales=scales, zeros=None, bias=b, M=M, K=K, N=N,
+                group_size=group_size, weight_dtype=4)

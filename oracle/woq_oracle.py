@@ -34,6 +34,11 @@ How each function is pinned (see tests/test_oracle.py):
     extreme element maps to +-127 / 0 / 255, |x - q*s| <= s/2) over all 65536 bf16 patterns;
   * int8 block sums: exact integer arithmetic against a Python big-int loop;
   * NF4 table: the published normal-quantile construction (scipy), codes by brute force;
+  * float8 e4m3fn: the value table against torch's float8_e4m3fn -> float32 conversion on all 256 bytes
+    and the format's landmarks (448 the largest, 2^-6 the smallest normal, 2^-9 the smallest subnormal);
+    the reference kernels' conversion against that table on every normal code and +-0, and on the 16
+    codes where it differs against the values the reference's own comment names
+    (csrc/cpu/vec/vec512/vec512_fp8.h:94-98) worked out by hand;
   * MoE token lists / weighted scatter: an independent formulation (nonzero per expert) and exact
     rationals rounded once.
 PARITY UNPINNED (no fixture or invariant can fix them; they are below the stated tolerances):
@@ -49,7 +54,7 @@ PARITY UNPINNED (no fixture or invariant can fix them; they are below the stated
 """
 import numpy as np
 
-WOQ_DTYPE_INT8, WOQ_DTYPE_INT4, WOQ_DTYPE_NF4 = 1, 2, 3
+WOQ_DTYPE_INT8, WOQ_DTYPE_INT4, WOQ_DTYPE_NF4, WOQ_DTYPE_FP8 = 1, 2, 3, 4  # csrc/cpu/aten/utils/woq_defines.h:6-9
 LOWP_NONE, LOWP_FP16, LOWP_BF16, LOWP_INT8 = 0, 1, 2, 3
 SMALL_BATCH_THRESHOLD = 5  # IPEX_WOQ_SMALL_BATCH_THRESHOLD, woq.h:24
 
@@ -122,9 +127,45 @@ NF4_DEQUANT_TABLE = np.array(
 )
 
 
+def _fp8_e4m3fn_table():
+    """All 256 float8 e4m3fn values (the dtype of the reference's FP8 weights, torch.float8_e4m3fn:
+    weight_only_quantization.py:238, tests/cpu/test_quantization_default_recipe.py:2155-2226): 1 sign bit,
+    4 exponent bits with bias 7, 3 mantissa bits, no infinities, exponent 15 with mantissa 7 is NaN;
+    exponent 0 is subnormal (mantissa * 2^-9)."""
+    t = np.zeros(256, dtype=np.float32)
+    for b in range(256):
+        e, m = (b >> 3) & 15, b & 7
+        if e == 15 and m == 7:
+            v = np.nan
+        elif e == 0:
+            v = m * 2.0 ** -9
+        else:
+            v = (1.0 + m / 8.0) * 2.0 ** (e - 7)
+        t[b] = -v if b & 0x80 else v
+    return t
+
+
+FP8_E4M3FN_TABLE = _fp8_e4m3fn_table()
+
+
+def _fp8_e4m3fn_kernel_table():
+    """What the reference's weight-only kernels make of each float8 e4m3fn byte
+    (convert_fp8_e4m3_to_fp32, csrc/cpu/aten/utils/woq.h:465-485, restated on the integers): mantissa
+    << 20 | (exponent + 120) << 23, zeroed when the 7 low bits are zero, | sign << 24.  Equal to the
+    float8 value on +-0 and every normal code; the subnormal codes 0x01..0x07 come out as
+    (8 + m) * 2^-10 (float8: m * 2^-9) and the NaN codes 0x7F / 0xFF as +-480 (the conversion "without
+    denorm behavior" that csrc/cpu/vec/vec512/vec512_fp8.h:94-98 describes)."""
+    x = np.arange(256, dtype=np.uint32)
+    nonsign = np.where((x & 127) != 0, ((x & 7) << 20) | ((((x >> 3) & 15) + 120) << 23), 0).astype(np.uint32)
+    return (nonsign | ((x & 128) << 24)).astype(np.uint32).view(np.float32)
+
+
+FP8_E4M3FN_KERNEL_TABLE = _fp8_e4m3fn_kernel_table()
+
+
 def dequantize_woq_weight(qw, N, K, scales, zps, weight_dtype, group_size):
     """fp32 (q - z) * s; q - z first, then the scale, both in fp32.  zps None: symmetric (INT4
-    codes stand for code - 8).  NF4: table[code] * s, no zero point
+    codes stand for code - 8).  FP8: qw holds float8 e4m3fn bytes, each converted as the reference's kernels convert it, times s.  NF4: table[code] * s, no zero point
     (csrc/cpu/aten/utils/woq_utils.h:64-77, 108-131).  scales / zps: [N] or
     [N, ceil(K / group_size)]."""
     if weight_dtype == WOQ_DTYPE_NF4:
@@ -136,6 +177,11 @@ def dequantize_woq_weight(qw, N, K, scales, zps, weight_dtype, group_size):
             q = q - np.float32(8)
     elif weight_dtype == WOQ_DTYPE_INT8:
         q = np.asarray(qw, dtype=np.int8).astype(np.float32)
+    elif weight_dtype == WOQ_DTYPE_FP8:
+        # the byte converted to the compute type (exactly: 4 significant bits) times the scale
+        # (load_dequant_fp8, csrc/cpu/aten/utils/woq.h:728-741); no zero points
+        assert zps is None, "FP8 weights are symmetric"
+        q = FP8_E4M3FN_KERNEL_TABLE[np.asarray(qw).view(np.uint8)]
     else:
         raise NotImplementedError("oracle: weight dtype")
     s = np.asarray(scales, dtype=np.float32).reshape(N, -1)

@@ -11,7 +11,9 @@ def case_np(case):
     """Numpy view of a case from ipex_amd.utils.synthetic for the oracle."""
     return dict(
         x=to_np_f32(case["x"]),
-        qw=case["qweight"].cpu().numpy(),
+        qw=(case["qweight"].view(torch.uint8) if case["qweight"].dtype == torch.float8_e4m3fn else case["qweight"])
+        .cpu()
+        .numpy(),
         scales=to_np_f32(case["scales"]),
         zps=None if case["zeros"] is None else to_np_f32(case["zeros"]),
         bias=None if case["bias"] is None else to_np_f32(case["bias"]),

@@ -101,6 +101,50 @@ def test_default_qconfig_on_an_fp32_model_computes_in_fp32(cuda, weight_dtype, g
     assert torch.allclose(y.cpu(), ref, atol=1e-5, rtol=1e-5), float((y.cpu() - ref).abs().max())
 
 
+@pytest.mark.parametrize("M", [4, 1024])
+@pytest.mark.parametrize("has_bias", [True, False])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_fp8_weight_through_from_float_and_qweight(cuda, M, has_bias, dtype):
+    """The reference's own FP8 test (tests/cpu/test_quantization_default_recipe.py:2155-2226), same shapes,
+    recipe, expected value and tolerance: group-wise absmax / 448 scales, weight / scale as float8 e4m3fn,
+    compared with matmul on the dequantized weight in the compute dtype (fp16 for bf16 rows up to 4)."""
+    ipex = _ipex()
+    q = ipex.quantization
+    from ipex_amd.nn.modules import WeightOnlyQuantizedLinear
+
+    torch.manual_seed(2)
+    K = N = 1024
+    group_size = 128
+    lin = torch.nn.Linear(K, N, has_bias).eval()
+    data = torch.rand(M, K).to(dtype) * 0.1
+    weight = lin.weight.detach()
+    grouped = weight.view(N, K // group_size, group_size)
+    w_scales = grouped.abs().max(-1)[0] / 448.0
+    w_fp8 = (grouped / w_scales.unsqueeze(-1)).view(N, K).to(torch.float8_e4m3fn)
+    w_dq = (w_fp8.view(N, K // group_size, group_size).float() * w_scales.unsqueeze(-1)).view(N, K)
+    compute_dtype = torch.half if (dtype == torch.bfloat16 and M <= 4) else dtype
+    w_dq = w_dq.to(compute_dtype)
+    out1 = torch.matmul(data.to(compute_dtype).float(), w_dq.float().T).to(compute_dtype)
+    out1 = (out1 + lin.bias.detach()) if has_bias else out1.float()
+    lowp = q.WoqLowpMode.BF16 if dtype == torch.bfloat16 else q.WoqLowpMode.NONE
+    qmap = q.get_weight_only_quant_qconfig_mapping(weight_dtype=q.WoqWeightDtype.FP8, lowp_mode=lowp)
+    with torch.no_grad():
+        lin.qconfig = qmap.global_qconfig
+        woq = WeightOnlyQuantizedLinear.from_float_and_qweight(
+            lin, w_fp8.to(cuda), q.WoqWeightDtype.FP8, w_scales, None, lin.bias, group_size
+        )
+        assert woq.weight is not None and woq.weight.dtype == torch.float8_e4m3fn
+        out2 = woq(data.to(cuda)).float().cpu()
+    torch.testing.assert_close(out1.float(), out2, atol=1e-3, rtol=1e-3)
+    ctx = woq._op_context
+    assert torch.equal(ctx.to_public(ctx.get_weight()).view(torch.uint8).cpu(), w_fp8.view(torch.uint8))
+    # the registered context pickles with its float8 weight and gives the same output afterwards
+    ctx2 = pickle.loads(pickle.dumps(ctx))
+    assert ctx2.get_weight().dtype == torch.float8_e4m3fn
+    y2 = torch.ops.torch_ipex.ipex_woq_linear(data.to(cuda), ctx2.get_data_handle())
+    assert torch.equal(y2.float().cpu(), out2)
+
+
 def test_all_zero_bias_is_dropped_and_weight_emptied(cuda):
     ipex = _ipex()
     q = ipex.quantization

@@ -26,6 +26,12 @@ def _kernels():
     return _kernels
 
 
+def _lib_last_kernel():
+    from ipex_amd import _lib
+
+    return _lib.last_kernel()
+
+
 def _synthetic():
     from ipex_amd.utils import synthetic
 
@@ -709,6 +715,132 @@ def test_nf4_weight_cache_for_large_batch_matches_oracle(cuda):
     c = case_np(case)
     _, y_opt = O.woq_linear_opt_bf16(c["x"], "bf16", c["qw"], 64, 256, c["scales"], None, None, 3, 64)
     assert rel_l2(y, y_opt) <= REL_L2_OUT
+
+
+# ---------------------------------------------------------------------------------------------
+# float8 e4m3fn weights (WOQ_DTYPE_FP8): bytes converted as the reference's kernels convert them, times the scale
+# ---------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("N,K", [(16, 64), (1024, 1024), (37, 100), (1, 1)])
+def test_fp8_pack_unpack_roundtrip(cuda, N, K):
+    k = _kernels()
+    code = torch.randint(0, 256, (N, K), dtype=torch.int16, generator=torch.Generator().manual_seed(N + K)).to(torch.uint8)
+    plain = code.view(torch.float8_e4m3fn)
+    packed = k.pack_weight(plain.to(cuda), 4, N, K)
+    back = k.unpack_weight(packed, 4, N, K)
+    assert back.dtype == torch.float8_e4m3fn and torch.equal(back.view(torch.uint8).cpu(), code)
+    # the bytes of a float8 tensor may also be handed over as uint8
+    assert torch.equal(k.pack_weight(code.to(cuda), 4, N, K), packed)
+
+
+@pytest.mark.parametrize("G", [128, -1])
+def test_fp8_dequant_weight_bit_exact_on_every_byte(cuda, G):
+    k = _kernels()
+    N, K = 48, 512
+    g = torch.Generator().manual_seed(77)
+    code = torch.arange(N * K, dtype=torch.int32).reshape(N, K).remainder(256)
+    code = code[:, torch.randperm(K, generator=g)].to(torch.uint8)  # all 256 bytes in every row, NaN codes included
+    shape = (N, K // G) if G > 0 else (N,)
+    scales = 0.0005 + 0.0015 * torch.rand(shape, generator=g)
+    case = dict(x=torch.zeros(1, K, dtype=torch.bfloat16), qweight=code.view(torch.float8_e4m3fn), scales=scales,
+                zeros=None, bias=None, M=1, K=K, N=N, group_size=G, weight_dtype=4)
+    ctx = make_context(case, O.LOWP_BF16)
+    want = O.dequantize_woq_weight(code.numpy(), N, K, scales.numpy(), None, 4, G)
+    got = k.dequant_weight(ctx.at_weight_, 4, N, K, ctx.scales_list_[0], None, G)
+    assert np.array_equal(got.cpu().numpy().view(np.uint32), want.view(np.uint32))
+    got16 = k.dequant_weight(ctx.at_weight_, 4, N, K, ctx.scales_list_[0], None, G, torch.bfloat16)
+    assert np.array_equal(to_np_f32(got16), O.bf16_round(want))
+
+
+@pytest.mark.parametrize("M", [1, 4, 5, 16, 40, 64, 65, 200])
+@pytest.mark.parametrize("K,N,G", [(1024, 272, 128), (384, 48, 32), (1000, 100, -1)])
+def test_fp8_linear(cuda, M, K, N, G):
+    case = _synthetic().make_fp8_case(60, M, K, N, bias=(M % 2 == 0), group_size=G)
+    _check_fp(case, O.LOWP_BF16, label=f"fp8 M={M} K={K} N={N} G={G}")
+
+
+def test_fp8_other_lowp_modes_kernels_and_activations(cuda):
+    syn = _synthetic()
+    for M in (3, 70):
+        case = syn.make_fp8_case(61, M, 512, 96, bias=True, group_size=64)
+        _check_fp(case, O.LOWP_NONE, label=f"fp8 lowp NONE M={M}")
+        _check_fp(case, O.LOWP_FP16, label=f"fp8 lowp FP16 M={M}")
+    # the tiled kernel on few rows and the small-M kernel at its row limit agree with the oracle too
+    case = syn.make_fp8_case(62, 48, 640, 144, bias=False, group_size=128)
+    _check_fp(case, O.LOWP_BF16, force_kernel=2, label="fp8 tiled kernel M=48")
+    _check_fp(case, O.LOWP_BF16, force_kernel=1, label="fp8 small-M kernel M=48")
+    # fp16 activations: w = fp16(value * s), fp32 accumulation
+    case = syn.make_fp8_case(63, 9, 256, 64, bias=False, group_size=128, x_dtype=torch.float16)
+    ctx = make_context(case, O.LOWP_FP16)
+    c = case_np(case)
+    y = to_np_f32(ctx.run(case["x"].cuda()))
+    _, y_ref = O.woq_linear_ref(c["x"], "fp16", c["qw"], 64, 256, O._round_to(c["scales"], "fp16"), None, None, 4, 128, "fp16")
+    assert rel_l2(y, y_ref) <= REL_L2_OUT
+
+
+@pytest.mark.parametrize("M,K,N,G,bias", [(4, 1024, 1024, 128, True), (300, 1024, 272, 128, False), (37, 1000, 100, -1, True)])
+def test_fp8_fp32_compute(cuda, M, K, N, G, bias):
+    """fp32 activations under lowp_mode NONE: w = fp32(value * s) (fp32 scales), fp32 matrix instructions."""
+    case = _synthetic().make_fp8_case(64, M, K, N, bias=bias, group_size=G, x_dtype=torch.float32)
+    ctx = make_context(case, O.LOWP_NONE)
+    y = ctx.run(case["x"].cuda())
+    assert y.dtype == torch.float32
+    c = case_np(case)
+    acc, _ = O.woq_linear_ref(c["x"], "fp32", c["qw"], N, K, c["scales"], None, c["bias"], 4, G, "fp32")
+    assert rel_l2(y.cpu().numpy(), acc) <= 1e-5
+
+
+@pytest.mark.parametrize("M,K,N,G,bias", [(1, 1024, 544, 128, False), (7, 1024, 544, 128, True), (16, 2048, 64, -1, False),
+                                          (27, 1152, 96, 128, True), (50, 1024, 288, 256, False), (64, 2048, 544, 128, True)])
+@pytest.mark.parametrize("kernel", [7, 8, 9, 13, 14])  # the dequantizing decode kernel: automatic, 1 / 2 row-blocks, K split in two
+def test_fp8_decode_kernels(cuda, M, K, N, G, bias, kernel):
+    if kernel in (13, 14) and M > 32:
+        pytest.skip("split K takes at most 32 rows")
+    case = _synthetic().make_fp8_case(66, M, K, N, bias=bias, group_size=G)
+    # lowp_mode BF16 computes in fp16 below 5 rows (bf16 rows converted on the way in)
+    _check_fp(case, O.LOWP_BF16, force_kernel=kernel, label=f"fp8 kernel {kernel} M={M}")
+    assert _lib_last_kernel() == "woq_decode_dq_kernel"
+
+
+@pytest.mark.parametrize("M,K,N,G,bias", [(128, 1024, 512, 128, True), (70, 2560, 272, -1, False), (300, 1024, 1040, 256, True),
+                                          (65, 512, 144, 128, False)])
+@pytest.mark.parametrize("kernel", [0, 5, 6, 12, 19])  # automatic, 128 x 256, 128 x 128, 64 x 128 tiles, K split in two
+def test_fp8_prefill_kernel(cuda, M, K, N, G, bias, kernel):
+    case = _synthetic().make_fp8_case(67, M, K, N, bias=bias, group_size=G)
+    _check_fp(case, O.LOWP_BF16, force_kernel=kernel, label=f"fp8 prefill kernel {kernel} M={M}")
+    assert _lib_last_kernel() == "woq_gemm_w4_kernel"
+
+
+@pytest.mark.parametrize("regime", ["fp16", "bf16"])
+@pytest.mark.parametrize("kernel", [1, 2, 8, 6])  # small-M, tiled, dequantizing decode, prefill
+def test_fp8_unit_rows_read_out_the_dequantized_weight_bit_for_bit(cuda, regime, kernel):
+    """Row m of the activations is the unit vector e_k(m): the fp32 accumulator is then the kernel's own
+    dequantized weight w[n, k(m)] -- every byte (subnormal and NaN codes included) against the oracle's
+    conversion and single rounding, bit for bit."""
+    N, K, G = 64, 256, 128
+    g = torch.Generator().manual_seed(91)
+    code = torch.stack([torch.randperm(256, generator=g) for _ in range(N)]).to(torch.uint8)  # all bytes in every row
+    scales = 0.0005 + 0.0015 * torch.rand((N, K // G), generator=g)
+    xdt = torch.float16 if regime == "fp16" else torch.bfloat16
+    case = dict(x=None, qweight=code.view(torch.float8_e4m3fn), scales=scales, zeros=None, bias=None, M=0, K=K, N=N,
+                group_size=G, weight_dtype=4)
+    ctx = make_context(case, O.LOWP_FP16 if regime == "fp16" else O.LOWP_BF16)
+    want = O._round_to(O.dequantize_woq_weight(code.numpy(), N, K, O._round_to(scales.numpy(), regime), None, 4, G), regime)
+    rows = 64 if kernel in (1, 8) else 256
+    eye = torch.eye(K, dtype=xdt)
+    for k0 in range(0, K, rows):
+        acc = ctx.run(eye[k0:k0 + rows].cuda(), out_fp32=True, force_kernel=kernel).cpu().numpy()
+        assert np.array_equal(acc, want[:, k0:k0 + rows].T), (regime, kernel, k0)
+
+
+def test_fp8_rejections(cuda):
+    syn = _synthetic()
+    case = syn.make_fp8_case(65, 4, 256, 32, group_size=64)
+    with pytest.raises(RuntimeError, match="no zero points"):
+        make_context(dict(case, zeros=torch.zeros(32, 4)), O.LOWP_BF16)
+    with pytest.raises(RuntimeError, match="INT8 does not take FP8"):
+        make_context(case, O.LOWP_INT8, act_quant_mode=6)
+    with pytest.raises(RuntimeError, match="float8_e4m3fn"):
+        make_context(dict(case, qweight=case["qweight"].view(torch.uint8).view(torch.int8)), O.LOWP_BF16)
 
 
 def test_empty_batch(cuda):

@@ -160,6 +160,56 @@ def test_nf4_quantize_dequantize_roundtrip_error_bound():
     assert np.allclose(np.abs(w).reshape(8, 4, 32).max(axis=-1), amax, rtol=0, atol=1e-7)
 
 
+def test_fp8_e4m3fn_tables():
+    # the value table against an independent implementation: torch's float8_e4m3fn -> float32
+    t = O.FP8_E4M3FN_TABLE
+    want = torch.arange(256, dtype=torch.int16).to(torch.uint8).view(torch.float8_e4m3fn).float().numpy()
+    assert t.dtype == np.float32 and t.shape == (256,)
+    assert np.array_equal(np.isnan(t), np.isnan(want)) and list(np.flatnonzero(np.isnan(t))) == [0x7F, 0xFF]
+    ok = ~np.isnan(want)
+    assert np.array_equal(t[ok].view(np.uint32), want[ok].view(np.uint32))  # bit for bit, -0.0 included
+    # landmarks of the format
+    assert t[0x7E] == 448.0 and t[0x08] == 2.0**-6 and t[0x01] == 2.0**-9 and t[0x07] == 7 * 2.0**-9
+    assert t[0x38] == 1.0 and t[0xB8] == -1.0
+    # the reference kernels' conversion: the same on +-0 and on every normal code ...
+    k = O.FP8_E4M3FN_KERNEL_TABLE
+    normal = np.array([b for b in range(256) if (b & 0x7F) == 0 or ((b >> 3) & 15) >= 1 and (b & 0x7F) != 0x7F])
+    assert len(normal) == 256 - 16
+    assert np.array_equal(k[normal].view(np.uint32), t[normal].view(np.uint32))
+    # ... a subnormal code read as exponent -7 with a hidden one (0.0019..0.0137 "cannot be converted
+    # correctly", vec512_fp8.h:94-98): m = 1 -> 1.125 / 128, m = 7 -> 1.875 / 128; NaN codes -> 1.875 * 2^8
+    hand = {0x01: 0.0087890625, 0x02: 0.009765625, 0x03: 0.0107421875, 0x04: 0.01171875, 0x05: 0.0126953125,
+            0x06: 0.013671875, 0x07: 0.0146484375, 0x7F: 480.0}
+    for b, v in hand.items():
+        assert k[b] == np.float32(v) and k[b | 0x80] == np.float32(-v), hex(b)
+    # the largest deviation from the float8 value of a non-NaN code: code 0x01, 9 * 2^-10 - 2 * 2^-10
+    assert np.nanmax(np.abs(k - t)) == 7 * 2.0**-10
+
+
+def test_fp8_dequantize_and_linear_against_exact_rationals():
+    # every byte, two scale groups: (table value) * scale in fp32, and the GEMM on top of it
+    qw = np.arange(256, dtype=np.uint8).reshape(1, 256).repeat(2, 0)
+    qw[1] = qw[1, ::-1]
+    s = np.array([[0.5, 0.0078125], [3.0, 0.001953125]], dtype=np.float32)
+    w = O.dequantize_woq_weight(qw, 2, 256, s, None, O.WOQ_DTYPE_FP8, 128)
+    k = O.FP8_E4M3FN_KERNEL_TABLE
+    for n in range(2):
+        for c in range(256):
+            assert w[n, c] == np.float32(k[qw[n, c]]) * s[n, c // 128]
+    assert np.array_equal(O.dequantize_woq_weight(qw.view(np.int8), 2, 256, s, None, O.WOQ_DTYPE_FP8, 128), w)
+    with pytest.raises(AssertionError):
+        O.dequantize_woq_weight(qw, 2, 256, s, s, O.WOQ_DTYPE_FP8, 128)
+    rng = np.random.default_rng(5)
+    x = O.bf16_round(rng.standard_normal((3, 256)).astype(np.float32))
+    acc, y = O.woq_linear_ref(x, "bf16", qw, 2, 256, s, None, None, O.WOQ_DTYPE_FP8, 128, "bf16")
+    wb = O.bf16_round(w)
+    for m in range(3):
+        for n in range(2):
+            exact = sum(fractions.Fraction(float(x[m, c])) * fractions.Fraction(float(wb[n, c])) for c in range(256))
+            assert abs(float(exact) - acc[m, n]) <= 1e-9 * max(1.0, abs(float(exact)))
+            assert y[m, n] == O.bf16_round(np.float32(float(exact)))
+
+
 def test_moe_token_lists_and_weighted_scatter():
     rng = np.random.default_rng(11)
     T, topk, E, H = 9, 3, 5, 6
