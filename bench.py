@@ -238,6 +238,8 @@ def config_sweep(torch, lib, lib_mod, ops_mod, synthetic, dev, stream, steps):
         us = groups[4]
         if case["weight_dtype"] == 2:
             nbytes = algorithmic_bytes(M, K, N, G)
+        elif case["weight_dtype"] == 4:  # float8 bytes, bf16 scales per group
+            nbytes = N * K + N * ((K + G - 1) // G if G > 0 else 1) * 2 + M * K * 2 + M * N * 2
         else:
             nbytes = N * K + N * 4 + M * K * 2 + M * N * 2 + (N * 2 if case["bias"] is not None else 0)
         row = {"config": name, "M": M, "K": K, "N": N, "group_size": G, "us_per_launch": round(us, 2),
@@ -276,6 +278,9 @@ def config_sweep(torch, lib, lib_mod, ops_mod, synthetic, dev, stream, steps):
     run("extra: int4 g128 M=16 4096->14336 lowp INT8 per-row-and-K-block", synthetic.make_int4_case(5, 16, 4096, 14336, 128), 3, 7)
     run("extra: int4 g32 M=1 4096->14336 lowp INT8 per-row-and-K-block", synthetic.make_int4_case(5, 1, 4096, 14336, 32), 3, 7)
     run("extra: int8 per-channel M=2048 4096->11008 +bias (lowp BF16)", synthetic.make_int8_case(5, 2048, 4096, 11008))
+    run("extra: int4 g32 M=2048 qkv 4096->6144 (lowp BF16, 256 x 192 tiles)", synthetic.make_int4_case(5, 2048, 4096, 6144, 32))
+    run("extra: fp8 e4m3fn g128 M=1 4096->14336 (lowp BF16)", synthetic.make_fp8_case(5, 1, 4096, 14336, bias=False, group_size=128))
+    run("extra: fp8 e4m3fn g128 M=2048 4096->14336 (lowp BF16)", synthetic.make_fp8_case(5, 2048, 4096, 14336, bias=False, group_size=128))
     run("extra: int4 g128 M=16 4096->14336 lowp INT8 asymmetric per-row", synthetic.make_int4_case(5, 16, 4096, 14336, 128), 3, 2)
     run("extra: int4 g64 M=128 4096->14336 lowp INT8 per-row", synthetic.make_int4_case(5, 128, 4096, 14336, 64), 3, 6)
     run("extra: int8 per-channel M=128 4096->11008 +bias lowp INT8 per-row", synthetic.make_int8_case(5, 128, 4096, 11008), 3, 6)
@@ -405,6 +410,10 @@ def run_probe(name, torch, lib, lib_mod, ops_mod, synthetic, dev, stream):
         info.update(floor_probe(torch, lib, dev, stream))
         print(json.dumps(info))
         return
+    elif name == "mfma":
+        info.update(mfma_issue_probe(torch, lib, dev, stream))
+        print(json.dumps(info))
+        return
     else:
         raise SystemExit(f"unknown probe {name!r}")
     info["calibration_copy_bytes"] = _calibration_copy(torch, dev)
@@ -458,6 +467,40 @@ def floor_probe(torch, lib, dev, stream, groups=9, per_group=200):
     return out
 
 
+def mfma_issue_probe(torch, lib, dev, stream, iters=1500, repeats=5):
+    """What bounds the prefill GEMM's K loop, measured without it: 256 workgroups of four waves (one wave per
+    SIMD on every CU), each wave issuing `iters` x 16 independent v_mfma_f32_16x16x32_bf16 on random bf16
+    operands with V fp32 FMAs and L ds_read_b128 per 16 MFMAs spread between them.  Per mix: microseconds per
+    launch (median of `repeats`), nanoseconds per MFMA and wave, and the TFLOP/s of the whole chip.  The
+    prefill kernel's loop issues 40 VALU and 2.8 LDS reads per 16 MFMAs."""
+    src = torch.randn(3 * 256 * 8, device=dev).to(torch.bfloat16)  # 12 KiB: LDS tile, A and B fragments
+    st = ctypes.c_void_p(stream.cuda_stream)
+    rows = []
+    for valu, lds in ((0, 0), (16, 0), (32, 0), (40, 0), (48, 0), (64, 0), (0, 3), (0, 8), (0, 16), (32, 3), (40, 3),
+                      (48, 3), (20, 6)):
+        def launch():
+            rc = lib.woq_hip_probe_mfma_issue(ctypes.c_void_p(src.data_ptr()), valu, lds, 256, iters, None, st)
+            assert rc == 0, lib.woq_hip_last_error()
+
+        launch()
+        vals = []
+        for _ in range(repeats):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            torch.cuda.synchronize()
+            e0.record(stream)
+            launch()
+            e1.record(stream)
+            torch.cuda.synchronize()
+            vals.append(e0.elapsed_time(e1) * 1e3)
+        us = sorted(vals)[len(vals) // 2]
+        mfmas = iters * 16
+        rows.append({"valu_per_16_mfma": valu, "lds_reads_per_16_mfma": lds, "us_per_launch": round(us, 1),
+                     "ns_per_mfma_and_wave": round(us * 1e3 / mfmas, 2),
+                     "tflops": round(256 * 4 * mfmas * 16384 / us / 1e6, 1),
+                     "frac_of_bf16_mfma_peak": round(256 * 4 * mfmas * 16384 / us / 1e6 / MFMA_BF16_PEAK_TFLOPS, 3)})
+    return {"workgroups": 256, "waves_per_workgroup": 4, "mfma_per_wave": iters * 16, "mixes": rows}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -471,7 +514,7 @@ def main():
     ap.add_argument("--no-sweep", action="store_true", help="skip the other named configurations")
     ap.add_argument("--no-floor", action="store_true", help="skip the streaming-read / empty-kernel floor")
     ap.add_argument("--M", type=int, default=1, help="decode batch (1..16)")
-    ap.add_argument("--probe", choices=["decode", "decode_dq", "prefill", "floor"],
+    ap.add_argument("--probe", choices=["decode", "decode_dq", "prefill", "floor", "mfma"],
                     help="short fixed workload for a rocprofv3 run (counters or kernel trace) instead of the benchmark")
     ap.add_argument("--traffic-probe", action="store_true", help="same as --probe decode")
     args = ap.parse_args()

@@ -222,6 +222,13 @@ __global__ __launch_bounds__(256) void woq_gemm_w4_kernel(const FpArgs f, const 
   static_assert(kStepLoads < 64 && G4_NTW * TPS < 16, "s_waitcnt vmcnt is a 6-bit field");
   constexpr int kVmcntStep = 0x0F70 | (kStepLoads & 15) | ((kStepLoads >> 4) << 14);
 
+  // With one set of fragment registers (16 row tiles) a wave reads the 16 fragments of the next sub-step in one block,
+  // and four waves that do so at the same moment queue at the LDS: a ds_read_b128 issued next to vector work costs
+  // 10 clocks alone and about 40 when the three other waves issue theirs with it.  The waves therefore meet at the
+  // barrier in different blocks of the last sub-step -- wave w in block FETCH_T - w, the same moment for all -- and so
+  // reach the fetching block one block apart, in every sub-step (M = 2048, 4096 -> 6144: 92 us against 99 us).
+  constexpr int STAG_MAX = S::XA_SETS == 1 ? (S::FETCH_T < 3 ? S::FETCH_T : 3) : 0;
+  const int bar_t = S::FETCH_T - (wave < STAG_MAX ? wave : STAG_MAX);
   load_x(kt_lo, 0);
   dma_w(kt_lo, 0);
   dma_w(KT > kt_lo + 1 ? kt_lo + 1 : kt_lo, 1);
@@ -277,11 +284,19 @@ __global__ __launch_bounds__(256) void woq_gemm_w4_kernel(const FpArgs f, const 
           __builtin_amdgcn_sched_barrier(0);
         }
         if (j == 3 && t == 0) __builtin_amdgcn_s_waitcnt(kVmcntStep);  // tiles of step kt + 1 are in LDS
-        if (fetch_t && j == 3) {
-          // Written as an instruction, not as the barrier builtin: before that one the compiler
-          // waits for every outstanding load, the tiles requested for step kt + 2 included.
-          __builtin_amdgcn_s_waitcnt(kVmcntW);
-          asm volatile("s_barrier" ::: "memory");
+        if constexpr (STAG_MAX == 0) {
+          if (fetch_t && j == 3) {
+            // Written as an instruction, not as the barrier builtin: before that one the compiler
+            // waits for every outstanding load, the tiles requested for step kt + 2 included.
+            __builtin_amdgcn_s_waitcnt(kVmcntW);
+            asm volatile("s_barrier" ::: "memory");
+          }
+        } else {
+          // this wave's meeting block (see bar_t)
+          if (j == 3 && t <= S::FETCH_T && t >= S::FETCH_T - STAG_MAX && bar_t == t) {
+            __builtin_amdgcn_s_waitcnt(kVmcntW);
+            __builtin_amdgcn_s_barrier();
+          }
         }
         if (last_t && j == 3) {
 #pragma unroll
@@ -528,7 +543,7 @@ int launch_gemm_w4(const FpArgs& f, int wbits, int regime, hipStream_t st, int s
   // 256 rows x 192 columns (MT 16, NTW 3: 192 accumulator registers) dequantizes half as much per
   // MFMA but measured no faster per output (a workgroup takes 95-120 us for K = 4096 against 103 us
   // for the 17 % larger 128 x 448 one); it is chosen only where it tiles the problem into whole
-  // generations of 256 workgroups and the others do not (N = 6144, M = 2048: 101 us against 138 us).
+  // generations of 256 workgroups and the others do not (N = 6144, M = 2048: 93 us against 138 us).
   // A 256 x 256 shape would need all 256 accumulator registers; the register allocator then
   // copies accumulators through VGPRs and scratch, it measured slower and is not built.
   using S7 = G4Shape<8, 7>;

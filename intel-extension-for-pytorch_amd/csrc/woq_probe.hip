@@ -26,6 +26,50 @@ __global__ __launch_bounds__(1024) void probe_stream_read_kernel(const u4* __res
 
 __global__ __launch_bounds__(1024) void probe_empty_kernel() {}
 
+// What the matrix pipe of a SIMD sustains when the wave that feeds it also issues other work: `iters` rounds
+// of 16 independent v_mfma_f32_16x16x32_bf16 (sixteen accumulator tiles, operands loaded once from src), with
+// VALU fp32 FMAs on eight independent registers and LDS ds_read_b128 spread evenly between them -- VALU16 and
+// LDS16 per sixteen MFMAs.  One wave per SIMD (four waves per workgroup, one workgroup per CU when the grid is
+// the CU count).  The prefill GEMM's K loop issues 2.5 VALU and 0.17 LDS reads per MFMA.
+template <int VALU16, int LDS16>
+__global__ __launch_bounds__(256) void probe_mfma_issue_kernel(const u4* __restrict__ src, int iters, float* sink) {
+  __shared__ u4 lds[256];
+  lds[threadIdx.x] = src[threadIdx.x];
+  __syncthreads();
+  f4 acc[16];
+#pragma unroll
+  for (int i = 0; i < 16; ++i) acc[i] = f4{0.f, 0.f, 0.f, 0.f};
+  const u4 a = src[256 + threadIdx.x], b = src[512 + threadIdx.x];
+  float v[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) v[i] = 1.0f + 0.001f * (float)((threadIdx.x + i) & 7);
+  u4 l[4] = {a, a, a, a};
+  const uint32_t la = threadIdx.x * 16u;
+#pragma unroll 1
+  for (int it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(acc[i]) : "v"(a), "v"(b));
+#pragma unroll
+      for (int j = (i * VALU16) / 16; j < ((i + 1) * VALU16) / 16; ++j)
+        asm volatile("v_fma_f32 %0, %0, %1, %0" : "+v"(v[j & 7]) : "v"(v[7 - (j & 7)]));
+#pragma unroll
+      for (int j = (i * LDS16) / 16; j < ((i + 1) * LDS16) / 16; ++j)
+        asm volatile("ds_read_b128 %0, %1" : "=v"(l[j & 3]) : "v"(la));
+    }
+  }
+  // nothing in the loop reads what the LDS loads return (they come back in order), so the loop never waits for them
+  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+  float s = 0.f;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) s += acc[i][0] + acc[i][3];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) s += v[i];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) s += bitcast<float>(l[i][0]);
+  if (sink) sink[(size_t)blockIdx.x * 256 + threadIdx.x] = s;
+}
+
 }  // namespace woq
 
 using namespace woq;
@@ -60,6 +104,25 @@ int woq_hip_probe_empty(int64_t workgroups, int waves_per_wg, void* stream) {
     return set_error("probe_empty: bad launch shape");
   probe_empty_kernel<<<(unsigned)workgroups, waves_per_wg * 64, 0, (hipStream_t)stream>>>();
   return check_launch("probe_empty_kernel");
+}
+
+int woq_hip_probe_mfma_issue(const void* src, int valu_per_16, int lds_per_16, int64_t workgroups, int iters,
+                             float* sink, void* stream) {
+  if (!src) return set_error("probe_mfma_issue: src must hold 12 KiB of operand bytes");
+  if (workgroups < 1 || workgroups > 65536 || iters < 1) return set_error("probe_mfma_issue: bad launch shape");
+  hipStream_t st = (hipStream_t)stream;
+  const u4* s = (const u4*)src;
+  const unsigned g = (unsigned)workgroups;
+#define WOQ_PROBE_MIX(V, L)                                                \
+  if (valu_per_16 == V && lds_per_16 == L) {                               \
+    probe_mfma_issue_kernel<V, L><<<g, 256, 0, st>>>(s, iters, sink);      \
+    return check_launch("probe_mfma_issue_kernel");                        \
+  }
+  WOQ_PROBE_MIX(0, 0) WOQ_PROBE_MIX(16, 0) WOQ_PROBE_MIX(32, 0) WOQ_PROBE_MIX(40, 0) WOQ_PROBE_MIX(48, 0)
+  WOQ_PROBE_MIX(64, 0) WOQ_PROBE_MIX(0, 3) WOQ_PROBE_MIX(0, 8) WOQ_PROBE_MIX(0, 16) WOQ_PROBE_MIX(32, 3)
+  WOQ_PROBE_MIX(40, 3) WOQ_PROBE_MIX(48, 3) WOQ_PROBE_MIX(20, 6)
+#undef WOQ_PROBE_MIX
+  return set_error("probe_mfma_issue: no instance for %d VALU and %d LDS reads per 16 MFMAs", valu_per_16, lds_per_16);
 }
 
 }  // extern "C"

@@ -44,6 +44,7 @@ EXPORTS = [
     "woq_hip_moe_scale_add_rows",
     "woq_hip_probe_stream_read",
     "woq_hip_probe_empty",
+    "woq_hip_probe_mfma_issue",
 ]
 
 
@@ -148,6 +149,8 @@ def load():
         lib.woq_hip_probe_stream_read.argtypes = [vp, i64, i32, i32, vp, vp]
         lib.woq_hip_probe_empty.restype = i32
         lib.woq_hip_probe_empty.argtypes = [i64, i32, vp]
+        lib.woq_hip_probe_mfma_issue.restype = i32
+        lib.woq_hip_probe_mfma_issue.argtypes = [vp, i32, i32, i64, i32, vp, vp]
         if lib.woq_hip_abi_version() != 1:
             raise RuntimeError("libwoq_hip.so has an unexpected ABI version")
         _lib = lib
