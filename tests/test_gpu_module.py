@@ -213,6 +213,81 @@ def test_gptq_checkpoint_through_llm_front_door(cuda):
     assert torch.allclose(y, ref, atol=3e-2, rtol=2e-2)
 
 
+class _TinyLM(torch.nn.Module):
+    def __init__(self, K, H, N, V):
+        super().__init__()
+        self.norm = torch.nn.LayerNorm(K)
+        self.block = torch.nn.ModuleDict({"up": torch.nn.Linear(K, H, bias=False), "down": torch.nn.Linear(H, N, bias=True)})
+        self.lm_head = torch.nn.Linear(N, V, bias=False)
+
+    def forward(self, x):
+        return self.lm_head(self.block["down"](torch.nn.functional.silu(self.block["up"](self.norm(x)))))
+
+
+@pytest.mark.parametrize("method", ["gptq", "gptq_act_order", "awq", "fp8", "int8"])
+def test_model_from_low_precision_checkpoint(cuda, method):
+    """A whole model from a checkpoint's state dict, as ipex.llm.optimize(low_precision_checkpoint=...) builds it
+    (utils/weight_only_quantization.py:224-376): quantized linears from the checkpoint's tensors, the floating-point
+    lm_head and the LayerNorm parameters loaded as they are; against the same model on the dequantized weights."""
+    import checkpoints as C
+    ipex = _ipex()
+    q = ipex.quantization
+    from ipex_amd.utils.weight_only_quantization import _convert_woq_with_low_precision_checkpoint
+
+    gen = torch.Generator().manual_seed(11)
+    K, H, N, V, G = 256, 512, 128, 64, 64
+    sd = {"norm.weight": 1 + 0.1 * torch.randn(K, generator=gen), "norm.bias": 0.1 * torch.randn(K, generator=gen),
+          "lm_head.weight": 0.05 * torch.randn(V, N, generator=gen)}
+    dense = {}
+    quant_config = {"quant_method": method.split("_")[0]}
+    for name, (n_out, n_in) in {"block.up": (H, K), "block.down": (N, H)}.items():
+        if method in ("gptq", "gptq_act_order", "awq"):
+            codes = torch.randint(0, 16, (n_out, n_in), generator=gen)
+            zp = torch.randint(0, 16, (n_out, n_in // G), generator=gen)
+            sc = (0.002 + 0.006 * torch.rand(n_out, n_in // G, generator=gen)).half()
+            if method == "gptq_act_order":
+                g_idx = (torch.randperm(n_in, generator=gen) // G).to(torch.int32)
+                dense[name] = (codes - zp[:, g_idx.long()]).float() * sc.float()[:, g_idx.long()]
+                sd[name + ".g_idx"] = g_idx
+            else:
+                dense[name] = C.int4_dequant(codes, zp, sc, G)
+            qw, s2, qz = (C.awq_layer if method == "awq" else C.gptq_layer)(codes, zp, sc)
+            sd.update({name + ".qweight": qw, name + ".scales": s2, name + ".qzeros": qz})
+        elif method == "fp8":
+            w8, sinv, dq = C.fp8_layer(0.05 * torch.randn(n_out, n_in, generator=gen), 128, 128)
+            sd.update({name + ".weight": w8, name + ".weight_scale_inv": sinv})
+            dense[name] = dq
+            quant_config["weight_block_size"] = [128, 128]
+        else:
+            w8 = torch.randint(-127, 128, (n_out, n_in), generator=gen, dtype=torch.int8)
+            sc = 0.0005 + 0.001 * torch.rand(n_out, 1, generator=gen)
+            sd.update({name + ".weight": w8, name + ".weight_scale": sc})
+            dense[name] = w8.float() * sc
+    sd["block.down.bias"] = 0.1 * torch.randn(N, generator=gen)
+    for k in ("norm.weight", "norm.bias", "lm_head.weight", "block.down.bias"):  # a bf16 checkpoint
+        sd[k] = sd[k].to(torch.bfloat16)
+    model = _TinyLM(K, H, N, V).eval()
+    qmap = q.get_weight_only_quant_qconfig_mapping(weight_dtype=q.WoqWeightDtype.INT4, lowp_mode=q.WoqLowpMode.BF16)
+    sd_gpu = {k: v.to(cuda) for k, v in sd.items()}
+    woq = _convert_woq_with_low_precision_checkpoint(copy.deepcopy(model).to(cuda).to(torch.bfloat16), qmap, sd_gpu,
+                                                     quant_config, inplace=True)
+    assert type(woq.block["up"]).__name__ == "WeightOnlyQuantizedLinear" and type(woq.block["down"]).__name__ == "WeightOnlyQuantizedLinear"
+    assert isinstance(woq.lm_head, torch.nn.Linear) and torch.equal(woq.lm_head.weight.cpu(), sd["lm_head.weight"])
+    assert torch.equal(woq.norm.weight.cpu(), sd["norm.weight"])
+    # the same model on the dequantized weights, in fp32
+    ref = copy.deepcopy(model)
+    ref.load_state_dict({"norm.weight": sd["norm.weight"].float(), "norm.bias": sd["norm.bias"].float(),
+                         "lm_head.weight": sd["lm_head.weight"].float(), "block.up.weight": dense["block.up"],
+                         "block.down.weight": dense["block.down"], "block.down.bias": sd["block.down.bias"].float()})
+    for M in (3, 70):
+        x = torch.randn(M, K, generator=gen)
+        with torch.no_grad():
+            want = ref(x)
+            got = woq(x.to(cuda).to(torch.bfloat16)).float().cpu()
+        err = float((got - want).norm() / want.norm())
+        assert err < 2e-2, (method, M, err)
+
+
 def test_context_pickle_roundtrip(cuda):
     from ipex_amd.utils import synthetic
     from helpers import make_context

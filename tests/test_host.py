@@ -174,6 +174,65 @@ def test_gptq_and_awq_converters_roundtrip():
     assert torch.equal(s3, s.t()) and torch.equal(z3.long(), zp)
 
 
+def test_get_linear_parameters_per_checkpoint_kind():
+    """utils/weight_only_quantization.py:_get_linear_parameters against checkpoints built from known codes."""
+    import checkpoints as C
+    from ipex_amd.nn.modules.weight_only_quantization import WoqWeightFormat
+    from ipex_amd.utils import weight_only_quantization as W
+
+    g = torch.Generator().manual_seed(1)
+    N, K, G = 32, 256, 64
+    q = torch.randint(0, 16, (N, K), generator=g)
+    zp = torch.randint(0, 16, (N, K // G), generator=g)
+    s = (0.01 * torch.rand(N, K // G, generator=g)).half()
+    plain = ((q[:, 1::2] << 4) | q[:, ::2]).to(torch.uint8)
+    # GPTQ without act-order: tensors stay in the GPTQ layout, parameters go to [N, groups]
+    qw, sc, qz = C.gptq_layer(q, zp, s)
+    sd = {"m.fc.qweight": qw, "m.fc.scales": sc, "m.fc.qzeros": qz, "m.fc.g_idx": torch.arange(K, dtype=torch.int32) // G,
+          "m.fc.bias": torch.ones(N)}
+    w, s2, z2, b, gs, gi, fmt = W._get_linear_parameters("m.fc", sd, W.GPTQ_LOWP_CHECKPOINT_CONFIG, {"quant_method": "gptq"})
+    assert fmt == WoqWeightFormat.GPTQ_FORMAT and gs == G and gi is None and w is qw and torch.equal(b, torch.ones(N))
+    assert torch.equal(s2, s) and torch.equal(z2.long(), zp)
+    # ... with act-order: the plain layout (as int32 words along K) and g_idx kept
+    perm = torch.randperm(K, generator=g)
+    sd["m.fc.g_idx"] = (perm // G).to(torch.int32)
+    w, s2, z2, _, gs, gi, fmt = W._get_linear_parameters("m.fc", sd, W.GPTQ_LOWP_CHECKPOINT_CONFIG, {"quant_method": "gptq"})
+    assert fmt == WoqWeightFormat.PLAIN_FORMAT and gi is not None and gs == G
+    assert torch.equal(w.contiguous().view(torch.uint8), plain) and torch.equal(z2.long(), zp)
+    # ... and dropped when the config says there is none
+    w, *_, gi, fmt = W._get_linear_parameters("m.fc", sd, dict(W.GPTQ_LOWP_CHECKPOINT_CONFIG, desc_act=False), {"quant_method": "gptq"})
+    assert gi is None and fmt == WoqWeightFormat.GPTQ_FORMAT
+    # AWQ
+    qw, sc, qz = C.awq_layer(q, zp, s)
+    sd = {"m.fc.qweight": qw, "m.fc.scales": sc, "m.fc.qzeros": qz}
+    w, s2, z2, b, gs, gi, fmt = W._get_linear_parameters("m.fc", sd, W.AWQ_LOWP_CHECKPOINT_CONFIG, {"quant_method": "awq"})
+    assert fmt == WoqWeightFormat.AWQ_FORMAT and gs == G and gi is None and b is None and w is qw
+    assert torch.equal(s2, s) and torch.equal(z2.long(), zp)
+    # DeepSeek FP8: one scale per 16 x 64 block -> one per row and block of 64 columns
+    wf = torch.randn(40, 128, generator=g)
+    q8, sinv, dq = C.fp8_layer(wf, 16, 64)
+    sd = {"m.fc.weight": q8, "m.fc.weight_scale_inv": sinv}
+    w, s2, z2, b, gs, gi, fmt = W._get_linear_parameters("m.fc", sd, W.FP8_LOWP_CHECKPOINT_CONFIG,
+                                                        {"quant_method": "fp8", "weight_block_size": [16, 64]})
+    assert w is q8 and z2 is None and gs == 64 and fmt == WoqWeightFormat.PLAIN_FORMAT and tuple(s2.shape) == (40, 2)
+    assert torch.equal((q8.float().view(40, 2, 64) * s2[:, :, None]).view(40, 128), dq)
+    # round to nearest, 8 bits: int8 along K four per word, zero points stored minus one as uint8
+    q8i = torch.randint(-128, 128, (N, K), generator=g, dtype=torch.int8)
+    z8 = torch.randint(0, 256, (N, K // G), generator=g)
+    sd = {"m.fc.qweight": q8i.contiguous().view(torch.int32).t().contiguous(),
+          "m.fc.scales": s.t().contiguous().float(),
+          "m.fc.qzeros": ((z8 - 1) % 256).to(torch.uint8).t().contiguous().view(torch.int32)}
+    w, s2, z2, _, gs, gi, fmt = W._get_linear_parameters("m.fc", sd, W.RTN_LOWP_CHECKPOINT_CONFIG, {"quant_method": "rtn", "bits": 8})
+    assert w.dtype == torch.int8 and torch.equal(w, q8i) and gs == G and gi is None
+    assert torch.equal(z2.view(torch.uint8).long(), z8 % 256) and torch.equal(s2, s.float())
+    # per-channel INT8 and a layer the checkpoint keeps in floating point
+    sd = {"m.fc.weight": q8i, "m.fc.weight_scale": torch.rand(N, 1), "m.head.weight": torch.randn(8, N)}
+    w, s2, z2, _, gs, _, _ = W._get_linear_parameters("m.fc", sd, W.INT8_LOWP_CHECKPOINT_CONFIG, {"quant_method": "int8"})
+    assert w is q8i and gs == -1 and z2 is None and tuple(s2.shape) == (N, 1)
+    w, s2, *_ = W._get_linear_parameters("m.head", sd, W.INT8_LOWP_CHECKPOINT_CONFIG, {"quant_method": "int8"})
+    assert s2 is None and w is sd["m.head.weight"]
+
+
 def test_c_port_of_oracle_matches_numpy_oracle():
     import ctypes
 
