@@ -284,10 +284,63 @@ def config_sweep(torch, lib, lib_mod, ops_mod, synthetic, dev, stream, steps):
     run("extra: int4 g128 M=16 4096->14336 lowp INT8 asymmetric per-row", synthetic.make_int4_case(5, 16, 4096, 14336, 128), 3, 2)
     run("extra: int4 g64 M=128 4096->14336 lowp INT8 per-row", synthetic.make_int4_case(5, 128, 4096, 14336, 64), 3, 6)
     run("extra: int8 per-channel M=128 4096->11008 +bias lowp INT8 per-row", synthetic.make_int8_case(5, 128, 4096, 11008), 3, 6)
+    rows.extend(moe_layer_rows(torch, ops_mod, synthetic, dev))
     # fp32 compute: the reference's default qconfig (INT8 weights, lowp_mode NONE) on an fp32 model
     case = synthetic.make_int8_case(5, 2048, 4096, 11008)
     case["fp32_activations"] = True
     run("extra: int8 per-channel M=2048 4096->11008 +bias, fp32 activations, lowp NONE (fp32 MFMA)", case, 0)
+    return rows
+
+
+def moe_layer_rows(torch, ops_mod, synthetic, dev, experts=32, H=7168, I=2048, topk=8):
+    """One mixture-of-experts layer over INT4 g128 experts (gate / up 7168 -> 2048, down 2048 -> 7168, top-8 of 32
+    experts) through torch.ops.torch_ipex.deepseek_moe_woq: microseconds per layer, wall clock over 20 calls without
+    synchronization in between, with the routing sorted on the device and grouped launches (the default up to 64
+    tokens) and with the per-expert launches that read the routing on the host."""
+    import os
+    import time
+
+    def ctx(K, N, seed):
+        c = synthetic.make_int4_case(seed, 1, K, N, 128)
+        return ops_mod.WoqLinearOpContext(c["qweight"].to(dev), 2, [N, K], c["scales"].to(dev), c["zeros"].to(dev), None, None,
+                                          None, 128, 2, -1, False)
+
+    lists = [[ctx(H, I, 600 + e % 4) for e in range(experts)], [ctx(H, I, 610 + e % 4) for e in range(experts)],
+             [ctx(I, H, 620 + e % 4) for e in range(experts)]]
+    op = torch.ops.torch_ipex.deepseek_moe_woq
+    g = torch.Generator().manual_seed(7)
+    rows = []
+    saved = os.environ.get("IPEX_AMD_MOE_GROUPED")
+    try:
+        for T in (1, 16):
+            x = torch.randn(T, H, generator=g).to(torch.bfloat16).to(dev)
+            ids = torch.stack([torch.randperm(experts, generator=g)[:topk] for _ in range(T)]).to(dev)
+            rw = torch.softmax(torch.randn(T, topk, generator=g), -1).to(torch.bfloat16).to(dev)
+            us = {}
+            for mode in ("1", "0"):
+                os.environ["IPEX_AMD_MOE_GROUPED"] = mode
+                for _ in range(3):
+                    op(x, ids, lists[0], lists[1], lists[2], rw, False)
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                for _ in range(20):
+                    op(x, ids, lists[0], lists[1], lists[2], rw, False)
+                torch.cuda.synchronize()
+                us[mode] = (time.perf_counter() - t0) / 20 * 1e6
+            active = len(set(ids.flatten().tolist()))
+            wbytes = active * 3 * H * I // 2
+            rows.append({"config": f"extra: MoE layer, {experts} INT4 g128 experts 7168->2048->7168, top-{topk}, {T} token(s)",
+                         "tokens": T, "active_experts": active, "us_per_layer_grouped": round(us["1"], 1),
+                         "us_per_layer_per_expert_launches": round(us["0"], 1),
+                         "GB_per_s_of_active_weights": round(wbytes / us["1"] / 1e3, 1),
+                         "frac_of_hbm_peak": round(wbytes / us["1"] / 1e3 / HBM_PEAK_GBS, 3)})
+    finally:
+        if saved is None:
+            os.environ.pop("IPEX_AMD_MOE_GROUPED", None)
+        else:
+            os.environ["IPEX_AMD_MOE_GROUPED"] = saved
+    del lists
+    torch.cuda.empty_cache()
     return rows
 
 

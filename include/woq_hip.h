@@ -316,6 +316,51 @@ int woq_hip_moe_scale_add_rows(void* out, int dtype, int64_t T, int64_t H, const
                                const void* routing_weights, int64_t topk, const int64_t* top_x, const int64_t* idx,
                                int64_t n, void* stream);
 
+/*
+ * A whole mixture-of-experts layer without reading the routing on the host (deepseek_moe_woq, csrc/cpu/aten/MoE.cpp:290-328,
+ * whose expert loop runs on the host because its tensors live there).
+ *
+ * woq_hip_moe_route: topk_ids int64 [T, topk] on the device -> the (token, slot) entries sorted by expert, stable, so
+ *   that inside an expert the tokens ascend (get_expert_topx_idx, MoE.cpp:64-81).  All outputs have T * topk entries
+ *   (at most WOQ_HIP_MOE_ROUTE_MAX): x_row[p] = token of the entry at sorted position p; one slot per sorted position:
+ *   the first position of an expert carries the expert's id -- in slot_expert_lo if the expert has fewer than split_lo
+ *   rows, in slot_expert_mid if at most split_mid, else in slot_expert_hi, -1 in the others -- with slot_row0[p] = p and
+ *   slot_rows[p] = its row count, every other position -1; row_of[t, i] / slot_of[t, i] = sorted position and top-k slot of token t's i-th contribution in ascending
+ *   expert order (row_of -1: none).  An expert id outside [0, experts) contributes nothing.
+ * woq_hip_linear_grouped: one linear of every expert that has a slot, in one launch.  p describes one expert's problem
+ *   (all experts share N, K, group size, weight dtype INT4 or INT8, lowp_mode NONE / FP16 / BF16, post-op none / silu /
+ *   mul) with M = the bound on a slot's rows (1..64; it selects the compute type like woq_hip_linear's M, so a layer
+ *   under lowp_mode BF16 takes one call with M = 4 on the slots of experts with fewer than five rows and one with a
+ *   larger M on the others; M <= 16 and M > 16 also select a kernel with one or four row tiles, hence three tables); p's weight, scale, zero
+ *   point and bias pointers are ignored.  x: the rows the slots read, out / others[0]: [routed rows, N].  group: DEVICE
+ *   pointer to a woq_hip_moe_group.  Rows of a slot are row0 .. row0 + rows - 1 of out; they read row x_row[row] of x,
+ *   or the same row when x_row is NULL.  Needs what the dequantizing decode kernel needs: K a multiple of the weight tile,
+ *   a power-of-two or per-channel group size, an even number of 16-column blocks, rows in the compute type (bf16 rows
+ *   under fp16 compute: at most 16 per slot).
+ * woq_hip_moe_combine_rows: out[t, :] (accumulate != 0: its value; else zero) plus token t's contributions in row_of's order of
+ *   routing_weights[t, slot] * expert_out[row, :], added in row_of's order and rounded to the dtype after every addition: bit for bit what one
+ *   woq_hip_moe_scale_add_rows call per expert, experts ascending, leaves.
+ */
+#define WOQ_HIP_MOE_ROUTE_MAX 2048
+typedef struct woq_hip_moe_group {
+  const int32_t* slot_expert;      /* [slots] expert of the slot or -1 */
+  const int32_t* slot_row0;        /* [slots] */
+  const int32_t* slot_rows;        /* [slots] */
+  const int64_t* x_row;            /* [routed rows] or NULL */
+  const void* const* qweight;      /* [experts] packed weights */
+  const void* const* scales;       /* [experts] scales in the compute type of the call (fp16 or bf16 layout of woq_hip_pack_qparams) */
+  const uint8_t* const* zeros_u8;  /* [experts] or NULL (symmetric) */
+  const float* const* bias;        /* [experts] or NULL */
+} woq_hip_moe_group;
+int woq_hip_moe_route(const int64_t* topk_ids, int64_t T, int64_t topk, int64_t experts, int64_t split_lo,
+                      int64_t split_mid, int64_t* x_row, int32_t* slot_expert_lo, int32_t* slot_expert_mid,
+                      int32_t* slot_expert_hi, int32_t* slot_row0, int32_t* slot_rows, int32_t* row_of, int32_t* slot_of,
+                      void* stream);
+int woq_hip_linear_grouped(const woq_hip_linear_params* p, const void* group, int64_t slots);
+int woq_hip_moe_combine_rows(void* out, int dtype, int64_t T, int64_t H, const void* expert_out,
+                             const void* routing_weights, int64_t topk, const int32_t* row_of, const int32_t* slot_of,
+                             int accumulate, void* stream);
+
 /* Measurement probes (no counterpart in the reference): the floor of an HBM-bound launch on this GPU.
  *   probe_stream_read: reads `bytes` from src once, `kib_per_wave` (1, 2, 4 or 8) KiB per wave as one
  *                      non-temporal dwordx4 load per lane and KiB, `waves_per_wg` (1..16) waves per

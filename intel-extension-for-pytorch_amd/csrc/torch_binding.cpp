@@ -225,6 +225,14 @@ class WoqLinearOpContext : public torch::CustomClassHolder {
   Tensor get_scales() { return scales_plain_; }
   optional<Tensor> get_zero_points() { return zeros_plain_; }
   std::vector<int64_t> get_weight_shape() { return {N_, K_}; }
+  // What a grouped launch over many contexts (the experts of a mixture-of-experts layer) needs of each: the device
+  // addresses of the packed weight, the fp16 and bf16 scales, the zero points and the fp32 bias (0: none), then
+  // N, K, group size, weight dtype, lowp_mode, whether the input channels are permuted (g_idx), the device index.
+  std::vector<int64_t> kernel_pointers() {
+    auto addr = [](const Tensor& t) -> int64_t { return t.defined() ? (int64_t)(uintptr_t)t.data_ptr() : 0; };
+    return {addr(packed_), addr(q_.s16), addr(q_.sb16), q_.z8.has_value() ? addr(*q_.z8) : 0, addr(bias_f32_),
+            N_, K_, group_size_, weight_dtype_, lowp_mode_, g_src_.defined() ? 1 : 0, (int64_t)packed_.device().index()};
+  }
   optional<Tensor> get_g_idx() { return g_idx_; }
   // The reference keeps a dequantized bf16 copy of the weight for batches of 64 rows and more when
   // cache_weight_for_large_batch is set (csrc/cpu/jit/cpu/kernels/LinearWoqPacked.cpp:430-533), because
@@ -819,6 +827,7 @@ TORCH_LIBRARY_FRAGMENT(ipex_prepack, m) {
       .def("get_scales", &WoqLinearOpContext::get_scales)
       .def("get_zero_points", &WoqLinearOpContext::get_zero_points)
       .def("get_weight_shape", &WoqLinearOpContext::get_weight_shape)
+      .def("kernel_pointers", &WoqLinearOpContext::kernel_pointers)
       .def("get_g_idx", &WoqLinearOpContext::get_g_idx)
       .def("get_cached_weight", &WoqLinearOpContext::get_cached_weight)
       .def("get_cached_compensation", &WoqLinearOpContext::get_cached_compensation)

@@ -307,6 +307,49 @@ int woq_hip_linear(const woq_hip_linear_params* p) {
                      : launch_gemm(f, wbits, regime, st);
 }
 
+int woq_hip_linear_grouped(const woq_hip_linear_params* p, const void* group, int64_t slots) {
+  if (!p || !group) return set_error("woq_linear_grouped: null params or group table");
+  if (p->struct_size != sizeof(woq_hip_linear_params))
+    return set_error("woq_linear_grouped: struct_size %u does not match this library (%zu)", p->struct_size,
+                     sizeof(woq_hip_linear_params));
+  if (p->weight_dtype != WOQ_HIP_DTYPE_INT4 && p->weight_dtype != WOQ_HIP_DTYPE_INT8)
+    return set_error("woq_linear_grouped: INT4 and INT8 weights, got dtype %d", p->weight_dtype);
+  if (p->M < 1 || p->M > 64 || p->K <= 0 || p->N <= 0)
+    return set_error("woq_linear_grouped: 1..64 rows per slot, got M=%lld K=%lld N=%lld", (long long)p->M, (long long)p->K,
+                     (long long)p->N);
+  if (p->x_dtype != WOQ_HIP_ACT_BF16 && p->x_dtype != WOQ_HIP_ACT_FP16)
+    return set_error("woq_linear_grouped: bf16 or fp16 rows, got x_dtype %d", p->x_dtype);
+  if (p->out_dtype != p->x_dtype) return set_error("woq_linear_grouped: out_dtype must equal x_dtype");
+  if (p->lowp_mode < 0 || p->lowp_mode > 2) return set_error("woq_linear_grouped: lowp_mode NONE, FP16 or BF16, got %d", p->lowp_mode);
+  if (!p->x || !p->out) return set_error("woq_linear_grouped: null pointer argument");
+  if (p->group_size > 0 && p->group_size % 32 != 0)
+    return set_error("woq_linear_grouped: group_size %lld must be a multiple of 32 (or <= 0 for per-channel)",
+                     (long long)p->group_size);
+  if (p->fusion != WOQ_HIP_FUSE_NONE && p->fusion != WOQ_HIP_FUSE_SILU && p->fusion != WOQ_HIP_FUSE_MUL)
+    return set_error("woq_linear_grouped: post-op none, silu or mul, got 0x%x", p->fusion);
+  if (p->fusion == WOQ_HIP_FUSE_MUL && !p->others[0]) return set_error("woq_linear_grouped: mul needs others[0]");
+  const int wbits = p->weight_dtype == WOQ_HIP_DTYPE_INT8 ? 8 : 4;
+  const int tk = wbits == 4 ? kTileK4 : kTileK8;
+  const int64_t NT = woq_hip_padded_n(p->N) / kTileN;
+  const int64_t KT = woq_hip_padded_k(p->weight_dtype, p->K) / tk;
+  const int64_t G = p->group_size > 0 ? p->group_size : KT * tk;
+  const int64_t KG = p->group_size > 0 ? (p->K + G - 1) / G : 1;
+  // the regimes of woq_hip_linear (csrc/cpu/aten/kernels/WoqLinearKrnl.cpp:75-112), with M the bound on a slot's rows
+  int regime;
+  if (p->lowp_mode == WOQ_HIP_LOWP_FP16 || (p->lowp_mode == WOQ_HIP_LOWP_NONE && p->x_dtype == WOQ_HIP_ACT_FP16) ||
+      (p->lowp_mode == WOQ_HIP_LOWP_BF16 && p->M < 5))
+    regime = kRegimeF16;
+  else
+    regime = kRegimeBF16;
+  FpArgs f;
+  f.x = p->x; f.x_dtype = p->x_dtype; f.M = p->M; f.K = p->K; f.N = p->N; f.NT = NT; f.KT = KT;
+  f.qweight = nullptr; f.scales = nullptr; f.zeros = nullptr;  // per expert, from the group table
+  f.G = G; f.KG = KG; f.bias = nullptr; f.fusion = p->fusion;
+  f.other0 = p->others[0]; f.other1 = nullptr; f.out = p->out; f.out_dtype = p->out_dtype;
+  f.nf4 = 0; f.fp8 = 0;
+  return launch_decode_dq_grouped(f, wbits, regime, (const MoeGroup*)group, slots, (hipStream_t)p->stream);
+}
+
 int woq_hip_dequant_weight(const void* qweight, int weight_dtype, int64_t N, int64_t K, const float* scales_f32,
                            const uint8_t* zeros_u8, int64_t group_size, void* out, int out_dtype, void* stream) {
   if (!valid_wdtype(weight_dtype)) return set_error("dequant_weight: unsupported weight dtype %d", weight_dtype);
@@ -363,6 +406,31 @@ int woq_hip_moe_scale_add_rows(void* out, int dtype, int64_t T, int64_t H, const
                               (long long)T);
   return launch_moe_scale_add_rows(out, dtype, T, H, expert_out, routing_weights, topk, top_x, idx, n,
                                    (hipStream_t)stream);
+}
+
+int woq_hip_moe_route(const int64_t* topk_ids, int64_t T, int64_t topk, int64_t experts, int64_t split_lo,
+                      int64_t split_mid, int64_t* x_row, int32_t* slot_expert_lo, int32_t* slot_expert_mid,
+                      int32_t* slot_expert_hi, int32_t* slot_row0, int32_t* slot_rows, int32_t* row_of, int32_t* slot_of,
+                      void* stream) {
+  if (T < 0 || topk <= 0 || experts <= 0) return set_error("moe_route: bad size");
+  if (T * topk > WOQ_HIP_MOE_ROUTE_MAX)
+    return set_error("moe_route: at most %d (token, slot) entries, got %lld", WOQ_HIP_MOE_ROUTE_MAX, (long long)(T * topk));
+  if (T > 0 && (!topk_ids || !x_row || !slot_expert_lo || !slot_expert_mid || !slot_expert_hi || !slot_row0 || !slot_rows ||
+                !row_of || !slot_of))
+    return set_error("moe_route: null pointer");
+  return launch_moe_route(topk_ids, T, topk, experts, split_lo, split_mid, x_row, slot_expert_lo, slot_expert_mid,
+                          slot_expert_hi, slot_row0, slot_rows, row_of, slot_of, (hipStream_t)stream);
+}
+
+int woq_hip_moe_combine_rows(void* out, int dtype, int64_t T, int64_t H, const void* expert_out,
+                             const void* routing_weights, int64_t topk, const int32_t* row_of, const int32_t* slot_of,
+                             int accumulate, void* stream) {
+  if (dtype < 0 || dtype > 2) return set_error("moe_combine_rows: bad dtype %d", dtype);
+  if (T < 0 || H < 0 || topk <= 0) return set_error("moe_combine_rows: bad size");
+  if (T > 0 && H > 0 && (!out || !expert_out || !routing_weights || !row_of || !slot_of))
+    return set_error("moe_combine_rows: null pointer");
+  return launch_moe_combine_rows(out, dtype, T, H, expert_out, routing_weights, topk, row_of, slot_of, accumulate,
+                                 (hipStream_t)stream);
 }
 
 // ---- woq_hip_linear for callers that cannot allocate ----------------------------------------------

@@ -45,7 +45,18 @@ struct DecodeDqArgs {
   int KTs;      // K tiles per workgroup row (gridDim.y workgroups share the K tiles of a row-block set)
   float* partial;  // split K: [gridDim.y][gridDim.x] fp32 partial tiles
   int* counters;   // split K: [gridDim.x], zero between launches
+  // GROUPED instances (mixture of experts): the workgroups with blockIdx.z = s serve slot s, whose expert, first
+  // routed row and row count they read from device memory; the expert's tensors come from pointer tables.
+  const MoeGroup* grp;
 };
+
+// a pointer every lane of the wave loaded from the same address, moved to scalar registers
+template <typename T>
+__device__ __forceinline__ T* dq_uniform(T* p) {
+  const uint64_t v = (uint64_t)p;
+  const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+  return (T*)(((uint64_t)hi << 32) | lo);
+}
 
 template <int REGIME>
 __device__ __forceinline__ f4 dq_mfma(u4 a, u4 b, f4 c) {
@@ -83,7 +94,7 @@ struct G8Consts {
 // reference's fp16 kernel converts them per K block (csrc/cpu/aten/utils/woq.h:3076-3079) -- the common
 // case of a bf16 model under lowp_mode BF16 with fewer than five rows.  The rows then travel through
 // registers (16-byte loads, conversion, ds_write to the same swizzled places) instead of the LDS DMA.
-template <int REGIME, int WBITS, int MT, int NTW, bool NF4, bool XCONV, bool FP8>
+template <int REGIME, int WBITS, int MT, int NTW, bool NF4, bool XCONV, bool FP8, bool GROUPED>
 __global__ __launch_bounds__(512, 4) void woq_decode_dq_kernel(const DecodeDqArgs a) {
   static_assert(!XCONV || (REGIME == kRegimeF16 && MT == 1), "bf16 -> fp16 rows: fp16 regime, one row tile");
   using Geo = DqGeom<WBITS, MT>;
@@ -96,7 +107,35 @@ __global__ __launch_bounds__(512, 4) void woq_decode_dq_kernel(const DecodeDqArg
     nf4_fill_lut(sNf4, (int)threadIdx.x, (int)blockDim.x);
     __syncthreads();
   }
-  const FpArgs& f = a.f;
+  FpArgs fg;                      // GROUPED: this slot's problem
+  const int64_t* xrow = nullptr;  // GROUPED: routed row -> row of x, from xrow0 on
+  int64_t xrow0 = 0;
+  if constexpr (GROUPED) {
+    // every workgroup of a slot takes the same path, and nothing has been synchronized yet
+    const MoeGroup& g = *a.grp;
+    const int slot = (int)blockIdx.z;
+    const int e = __builtin_amdgcn_readfirstlane(g.slot_expert[slot]);
+    if (e < 0) return;
+    const int64_t row0 = __builtin_amdgcn_readfirstlane(g.slot_row0[slot]);
+    const int rows = __builtin_amdgcn_readfirstlane(g.slot_rows[slot]);
+    fg = a.f;
+    fg.M = rows < (int)fg.M ? rows : fg.M;
+    fg.qweight = dq_uniform((const uint8_t*)g.qweight[e]);
+    fg.scales = dq_uniform((const uint16_t*)g.scales[e]);
+    fg.zeros = g.zeros ? dq_uniform(g.zeros[e]) : nullptr;
+    fg.bias = g.bias ? dq_uniform(g.bias[e]) : nullptr;
+    const int64_t out_elt = fg.out_dtype == WOQ_HIP_ACT_FP32 ? 4 : 2, x_elt = 2;  // rows are 16-bit here
+    fg.out = (uint8_t*)fg.out + row0 * fg.N * out_elt;
+    if (fg.other0) fg.other0 = (const uint8_t*)fg.other0 + row0 * fg.N * x_elt;
+    if (fg.other1) fg.other1 = (const uint8_t*)fg.other1 + row0 * fg.N * x_elt;
+    if (g.x_row) {
+      xrow = g.x_row;
+      xrow0 = row0;
+    } else {
+      fg.x = (const uint8_t*)fg.x + row0 * fg.K * x_elt;
+    }
+  }
+  const FpArgs& f = GROUPED ? fg : a.f;
   const int W = a.W;
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
@@ -124,7 +163,10 @@ __global__ __launch_bounds__(512, 4) void woq_decode_dq_kernel(const DecodeDqArg
 #pragma unroll
   for (int i = 0; i < NX; ++i) {
     const int row = Geo::RPI * i + lane / Geo::LPR;
-    const int rowc = row < M ? row : M - 1;
+    int rowc = row < M ? row : M - 1;
+    if constexpr (GROUPED) {
+      if (xrow) rowc = (int)xrow[xrow0 + rowc];  // (the host bounds rows of x * K * 2 below 2^31)
+    }
     const int chunk = ((lane % Geo::LPR) ^ Geo::swz(row)) & (Geo::LPR - 1);
     xoff[i] = (uint32_t)(rowc * K + chunk * 8) * 2u;
   }
@@ -313,8 +355,8 @@ __global__ __launch_bounds__(512, 4) void woq_decode_dq_kernel(const DecodeDqArg
   if (threadIdx.x == 0) __hip_atomic_store(a.counters + blockIdx.x, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-template <int REGIME, int WBITS, int MT, int NTW, bool NF4 = false, bool XCONV = false, bool FP8 = false>
-static int launch_dq_cfg(DecodeDqArgs a, int splits, hipStream_t st) {
+template <int REGIME, int WBITS, int MT, int NTW, bool NF4 = false, bool XCONV = false, bool FP8 = false, bool GROUPED = false>
+static int launch_dq_cfg(DecodeDqArgs a, int splits, hipStream_t st, int slots = 1) {
   using Geo = DqGeom<WBITS, MT>;
   if (MT > 2 && splits > 1) return set_error("woq_decode_dq_kernel: split K takes at most 32 rows");
   // At most 64 KiB of activation buffers per workgroup, so that two workgroups share a CU -- unless
@@ -324,7 +366,7 @@ static int launch_dq_cfg(DecodeDqArgs a, int splits, hipStream_t st) {
   // four row tiles (33..64 rows) a wave's two buffers are 32 KiB and one workgroup of four waves takes
   // 128 KiB.  Sixteen waves of one row tile measured no faster than eight.
   constexpr int kLdsMax = 131072;
-  const dim3 grid((unsigned)(a.f.NT / NTW), (unsigned)splits);
+  const dim3 grid((unsigned)(a.f.NT / NTW), (unsigned)splits, (unsigned)slots);
   const bool alone = MT == 2 && grid.x * grid.y <= 256;
   const int lds_cap = (MT > 2 || alone) ? kLdsMax : 65536;
   const int max_w = lds_cap / (2 * Geo::SLICE);
@@ -334,7 +376,7 @@ static int launch_dq_cfg(DecodeDqArgs a, int splits, hipStream_t st) {
   size_t smem = (size_t)a.W * 2 * Geo::SLICE;
   const size_t red = (size_t)NTW * MT * a.W * 64 * sizeof(f4);
   if (red > smem) smem = red;
-  auto kern = woq_decode_dq_kernel<REGIME, WBITS, MT, NTW, NF4, XCONV, FP8>;
+  auto kern = woq_decode_dq_kernel<REGIME, WBITS, MT, NTW, NF4, XCONV, FP8, GROUPED>;
   if (MT >= 2) {
     // more than 64 KiB of LDS per workgroup needs an opt-in (once per kernel and process)
     static const hipError_t lds_optin =
@@ -395,6 +437,48 @@ static int launch_dq_nf4(const DecodeDqArgs& a, int ntw, int splits, hipStream_t
   return two_rows ? launch_dq_cfg<REGIME, 4, 2, 1, true>(a, splits, st) : launch_dq_cfg<REGIME, 4, 1, 1, true>(a, splits, st);
 }
 
+// Grouped launch over the slots of a mixture-of-experts layer: INT4 / INT8 weights, two row-blocks per workgroup, one
+// row tile (up to 16 rows per slot) or four (up to 64), K never split.  f describes one expert's problem with M = the
+// bound on a slot's rows; the slots' experts, rows and tensors come from grp (device memory).
+template <int REGIME, int WBITS>
+static int launch_dq_grouped_regime(const DecodeDqArgs& a, int slots, hipStream_t st) {
+  const bool four = a.f.M > 16;
+  if constexpr (REGIME == kRegimeF16) {
+    if (a.f.x_dtype == WOQ_HIP_ACT_BF16) {
+      if (four) return set_error("woq_linear_grouped: bf16 rows under fp16 compute take at most 16 rows per slot");
+      return launch_dq_cfg<REGIME, WBITS, 1, 2, false, true, false, true>(a, 1, st, slots);
+    }
+  }
+  return four ? launch_dq_cfg<REGIME, WBITS, 4, 2, false, false, false, true>(a, 1, st, slots)
+              : launch_dq_cfg<REGIME, WBITS, 1, 2, false, false, false, true>(a, 1, st, slots);
+}
+
+int launch_decode_dq_grouped(const FpArgs& f, int wbits, int regime, const MoeGroup* grp, int64_t slots, hipStream_t st) {
+  if (!grp || slots < 1 || slots > 65535) return set_error("woq_linear_grouped: 1..65535 slots and a group table");
+  if (f.nf4 || f.fp8) return set_error("woq_linear_grouped: INT4 and INT8 weights");
+  if (f.NT % 2 != 0) return set_error("woq_linear_grouped: an even number of row-blocks (N a multiple of 32 after padding)");
+  if (!decode_dq_applies(f, wbits, regime))
+    return set_error("woq_linear_grouped: at most 64 rows per slot, K a multiple of the weight tile, a power-of-two or "
+                     "per-channel group size and rows in the compute dtype (bf16 rows under fp16 compute: 16 per slot)");
+  DecodeDqArgs a;
+  a.f = f;
+  a.partial = nullptr;
+  a.counters = nullptr;
+  a.grp = grp;
+  a.W = 1;
+  a.KTs = (int)f.KT;
+  a.g_shift = 30;
+  if (f.G < f.KT * (wbits == 4 ? kTileK4 : kTileK8)) {
+    a.g_shift = 0;
+    while (((int64_t)1 << a.g_shift) < f.G) ++a.g_shift;
+  }
+  if (wbits == 4)
+    return regime == kRegimeF16 ? launch_dq_grouped_regime<kRegimeF16, 4>(a, (int)slots, st)
+                                : launch_dq_grouped_regime<kRegimeBF16, 4>(a, (int)slots, st);
+  return regime == kRegimeF16 ? launch_dq_grouped_regime<kRegimeF16, 8>(a, (int)slots, st)
+                              : launch_dq_grouped_regime<kRegimeBF16, 8>(a, (int)slots, st);
+}
+
 int64_t decode_dq_splitk_bytes(int64_t M, int64_t NT, int splits) {
   return (int64_t)splits * NT * (M > 16 ? 2 : 1) * 256 * (int64_t)sizeof(float);
 }
@@ -405,6 +489,7 @@ int launch_decode_dq(const FpArgs& f, int wbits, int regime, hipStream_t st, int
   a.f = f;
   a.partial = scratch ? scratch->partial : nullptr;
   a.counters = scratch ? scratch->counters : nullptr;
+  a.grp = nullptr;
   a.W = 1;
   a.KTs = (int)f.KT;
   a.g_shift = 30;

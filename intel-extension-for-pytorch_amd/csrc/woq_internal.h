@@ -36,6 +36,18 @@ struct FpArgs {
   int fp8;  // 8-bit weights are float8 e4m3fn bytes, not offset-binary integers (zeros == nullptr)
 };
 
+// Device-side description of a grouped launch over the experts of a mixture-of-experts layer (woq_hip_moe_group).
+struct MoeGroup {
+  const int32_t* slot_expert;  // [slots] expert of the slot, or -1: nothing to do
+  const int32_t* slot_row0;    // [slots] first routed row of the slot
+  const int32_t* slot_rows;    // [slots] its number of rows
+  const int64_t* x_row;        // [routed rows] row of x a routed row reads, or null: the routed row itself
+  const void* const* qweight;  // [experts] packed weights
+  const void* const* scales;   // [experts] scales in the regime's dtype
+  const uint8_t* const* zeros; // [experts] or null
+  const float* const* bias;    // [experts] or null
+};
+
 // Split-K scratch of the dequantizing decode kernel: fp32 partial tiles, and one counter per
 // row-block set that is zero between launches.
 struct SplitKScratch {
@@ -64,6 +76,11 @@ int launch_moe_gather_rows(const void* x, int x_dtype, int64_t T, int64_t H, con
                            hipStream_t st);
 int launch_moe_scale_add_rows(void* out, int dtype, int64_t T, int64_t H, const void* cur, const void* rw, int64_t topk,
                               const int64_t* top_x, const int64_t* idx, int64_t n, hipStream_t st);
+int launch_moe_route(const int64_t* ids, int64_t T, int64_t topk, int64_t experts, int64_t split_lo, int64_t split_mid,
+                     int64_t* x_row, int32_t* slot_lo, int32_t* slot_mid, int32_t* slot_hi, int32_t* slot_row0,
+                     int32_t* slot_rows, int32_t* row_of, int32_t* slot_of, hipStream_t st);
+int launch_moe_combine_rows(void* out, int dtype, int64_t T, int64_t H, const void* cur, const void* rw, int64_t topk,
+                            const int32_t* row_of, const int32_t* slot_of, int accumulate, hipStream_t st);
 int launch_dequant_weight(const void* qweight, int weight_dtype, int64_t N, int64_t K, const float* s32,
                           const uint8_t* z8, int64_t G, void* out, int out_dtype, hipStream_t st);
 
@@ -112,6 +129,7 @@ int launch_fp32(const Fp32Args& f, int wbits, hipStream_t st);
 // splits: workgroups that share the K tiles of a row-block set (1, 2 or 4; more than 1 needs the
 // scratch and at most 32 rows), 0 = automatic (only together with ntw = 0)
 bool decode_dq_applies(const FpArgs& f, int wbits, int regime);
+int launch_decode_dq_grouped(const FpArgs& f, int wbits, int regime, const MoeGroup* grp, int64_t slots, hipStream_t st);
 int launch_decode_dq(const FpArgs& f, int wbits, int regime, hipStream_t st, int ntw = 0, int splits = 1,
                      const SplitKScratch* scratch = nullptr);
 // Bytes of partial-tile scratch that `splits` workgroups per row-block set need.

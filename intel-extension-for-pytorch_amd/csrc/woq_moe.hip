@@ -90,6 +90,109 @@ __global__ void moe_scale_add_rows_kernel(void* __restrict__ out, const void* __
   }
 }
 
+// Routing of a whole layer on the device, for the grouped launches: one workgroup sorts the R = tokens x top-k
+// (token, slot) entries by expert -- stable, so that inside an expert the tokens ascend, the order of
+// get_expert_topx_idx (csrc/cpu/aten/MoE.cpp:64-81) -- and writes
+//   x_row[p]        token of the entry at sorted position p (the row of the hidden states it reads),
+//   slot_*[p]       a slot per sorted position: the first position of an expert carries the expert's id (in the table
+//                   of its size class: fewer than split_lo rows -> lo, at most split_mid -> mid, else hi; -1 in the
+//                   others) and its row count, every other position -1,
+//   row_of[t, i]    sorted position of token t's i-th contribution in ascending expert order (-1: none),
+//   slot_of[t, i]   its top-k slot.
+// An expert id outside [0, experts) contributes nothing.  R <= kMoeRouteMax entries, compared pairwise from LDS.
+constexpr int kMoeRouteMax = WOQ_HIP_MOE_ROUTE_MAX;
+__global__ __launch_bounds__(256) void moe_route_kernel(const int64_t* __restrict__ ids, int R, int topk, int experts,
+                                                        int split_lo, int split_mid, int64_t* __restrict__ x_row,
+                                                        int32_t* __restrict__ slot_lo, int32_t* __restrict__ slot_mid,
+                                                        int32_t* __restrict__ slot_hi,
+                                                        int32_t* __restrict__ slot_row0, int32_t* __restrict__ slot_rows,
+                                                        int32_t* __restrict__ row_of, int32_t* __restrict__ slot_of) {
+  __shared__ int se[kMoeRouteMax];
+  for (int i = threadIdx.x; i < R; i += blockDim.x) {
+    const int64_t e = ids[i];
+    se[i] = (e >= 0 && e < experts) ? (int)e : -1;
+    slot_lo[i] = -1;
+    slot_mid[i] = -1;
+    slot_hi[i] = -1;
+    slot_row0[i] = i;
+    slot_rows[i] = 0;
+    row_of[i] = -1;
+    slot_of[i] = 0;
+  }
+  __syncthreads();
+  for (int i = threadIdx.x; i < R; i += blockDim.x) {
+    const int e = se[i];
+    if (e < 0) continue;
+    int before = 0, rank = 0, count = 0;
+    for (int k = 0; k < R; ++k) {
+      const int ek = se[k];
+      before += (ek >= 0 && ek < e) ? 1 : 0;
+      rank += (ek == e && k < i) ? 1 : 0;
+      count += (ek == e) ? 1 : 0;
+    }
+    const int p = before + rank;
+    const int t = i / topk, j = i - t * topk;
+    x_row[p] = t;
+    if (rank == 0) {
+      (count < split_lo ? slot_lo : count <= split_mid ? slot_mid : slot_hi)[p] = e;
+      slot_rows[p] = count;
+    }
+    int ord = 0;
+    for (int jj = 0; jj < topk; ++jj) {
+      const int ek = se[t * topk + jj];
+      ord += (ek >= 0 && (ek < e || (ek == e && jj < j))) ? 1 : 0;
+    }
+    row_of[t * topk + ord] = p;
+    slot_of[t * topk + ord] = j;
+  }
+  // positions past the valid entries read token 0 (never used: no slot covers them)
+  int valid = 0;
+  for (int k = 0; k < R; ++k) valid += se[k] >= 0 ? 1 : 0;
+  for (int i = valid + threadIdx.x; i < R; i += blockDim.x) x_row[i] = 0;
+}
+
+// out[t, :] accumulates token t's contributions in the order row_of gives (ascending expert), each step rounded to the
+// output dtype -- what one moe_scale_add_rows launch per expert leaves in memory between the experts.
+template <int DTYPE>
+__global__ void moe_combine_rows_kernel(void* __restrict__ out, const void* __restrict__ cur, const void* __restrict__ rw,
+                                        int64_t topk, const int32_t* __restrict__ row_of,
+                                        const int32_t* __restrict__ slot_of, int64_t T, int64_t H, int64_t R,
+                                        bool accumulate) {
+  constexpr int PER = DTYPE == WOQ_HIP_ACT_FP32 ? 4 : 8;
+  const int64_t chunks = (H + PER - 1) / PER;
+  const int64_t g = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (g >= T * chunks) return;
+  const int64_t t = g / chunks, j0 = (g - t * chunks) * PER;
+  float o[PER];
+  for (int e = 0; e < PER; ++e) o[e] = (accumulate && j0 + e < H) ? load_act(out, DTYPE, t * H + j0 + e) : 0.0f;
+  // the contributions in groups of eight: all rows of a group are requested before the first addition, the additions
+  // then run in order
+  for (int64_t i0 = 0; i0 < topk; i0 += 8) {
+    float v[8][PER], w[8];
+    bool have[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int64_t r = i0 + i < topk ? (int64_t)row_of[t * topk + i0 + i] : -1;
+      have[i] = (uint64_t)r < (uint64_t)R;
+      w[i] = have[i] ? load_act(rw, DTYPE, t * topk + slot_of[t * topk + i0 + i]) : 0.0f;
+#pragma unroll
+      for (int e = 0; e < PER; ++e) v[i][e] = (have[i] && j0 + e < H) ? load_act(cur, DTYPE, r * H + j0 + e) : 0.0f;
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      if (!have[i]) continue;
+#pragma unroll
+      for (int e = 0; e < PER; ++e) {
+        const float s = moe_accumulate<DTYPE>(o[e], v[i][e], w[i]);
+        o[e] = DTYPE == WOQ_HIP_ACT_BF16   ? bf16_bits_to_f32(f32_to_bf16_bits(s))
+               : DTYPE == WOQ_HIP_ACT_FP16 ? f16_bits_to_f32(f32_to_f16_bits(s))
+                                           : s;
+      }
+    }
+  }
+  for (int e = 0; e < PER && j0 + e < H; ++e) store_act(out, DTYPE, t * H + j0 + e, o[e]);
+}
+
 static inline unsigned moe_blocks(int64_t n) { return (unsigned)((n + 255) / 256); }
 
 int launch_moe_gather_rows(const void* x, int x_dtype, int64_t T, int64_t H, const int64_t* rows, int64_t n, void* out,
@@ -120,6 +223,32 @@ int launch_moe_scale_add_rows(void* out, int dtype, int64_t T, int64_t H, const 
   else
     moe_scale_add_rows_kernel<WOQ_HIP_ACT_FP32><<<blocks, 256, 0, st>>>(out, cur, rw, topk, top_x, idx, n, H, T, vec);
   return check_launch("moe_scale_add_rows");
+}
+
+int launch_moe_route(const int64_t* ids, int64_t T, int64_t topk, int64_t experts, int64_t split_lo, int64_t split_mid,
+                     int64_t* x_row, int32_t* slot_lo, int32_t* slot_mid, int32_t* slot_hi, int32_t* slot_row0,
+                     int32_t* slot_rows, int32_t* row_of, int32_t* slot_of, hipStream_t st) {
+  const int64_t R = T * topk;
+  if (R == 0) return 0;
+  if (R > kMoeRouteMax) return set_error("moe_route: at most %d (token, slot) entries, got %lld", kMoeRouteMax, (long long)R);
+  moe_route_kernel<<<1, 256, 0, st>>>(ids, (int)R, (int)topk, (int)experts, (int)split_lo, (int)split_mid, x_row, slot_lo,
+                                       slot_mid, slot_hi, slot_row0, slot_rows, row_of, slot_of);
+  return check_launch("moe_route");
+}
+
+int launch_moe_combine_rows(void* out, int dtype, int64_t T, int64_t H, const void* cur, const void* rw, int64_t topk,
+                            const int32_t* row_of, const int32_t* slot_of, int accumulate, hipStream_t st) {
+  if (T == 0 || H == 0 || topk == 0) return 0;
+  const int per = dtype == WOQ_HIP_ACT_FP32 ? 4 : 8;
+  const unsigned blocks = moe_blocks(T * ((H + per - 1) / per));
+  const int64_t R = T * topk;
+  if (dtype == WOQ_HIP_ACT_BF16)
+    moe_combine_rows_kernel<WOQ_HIP_ACT_BF16><<<blocks, 256, 0, st>>>(out, cur, rw, topk, row_of, slot_of, T, H, R, accumulate != 0);
+  else if (dtype == WOQ_HIP_ACT_FP16)
+    moe_combine_rows_kernel<WOQ_HIP_ACT_FP16><<<blocks, 256, 0, st>>>(out, cur, rw, topk, row_of, slot_of, T, H, R, accumulate != 0);
+  else
+    moe_combine_rows_kernel<WOQ_HIP_ACT_FP32><<<blocks, 256, 0, st>>>(out, cur, rw, topk, row_of, slot_of, T, H, R, accumulate != 0);
+  return check_launch("moe_combine_rows");
 }
 
 }  // namespace woq

@@ -13,6 +13,7 @@ LIB_PATH = os.path.join(os.path.dirname(_HERE), "lib", "libwoq_hip.so")
 # weight dtype / lowp mode / fusion codes of the C ABI
 DTYPE_INT8, DTYPE_INT4, DTYPE_NF4, DTYPE_FP8 = 1, 2, 3, 4
 DTYPES_8BIT = (DTYPE_INT8, DTYPE_FP8)
+MOE_ROUTE_MAX = 2048  # WOQ_HIP_MOE_ROUTE_MAX
 LOWP_NONE, LOWP_FP16, LOWP_BF16, LOWP_INT8 = 0, 1, 2, 3
 ACT_FP32, ACT_FP16, ACT_BF16 = 0, 1, 2
 FUSE_NONE, FUSE_GELU_ERF, FUSE_GELU_TANH, FUSE_RELU, FUSE_SILU = 0x0, 0x1, 0x2, 0x3, 0x4
@@ -45,6 +46,9 @@ EXPORTS = [
     "woq_hip_probe_stream_read",
     "woq_hip_probe_empty",
     "woq_hip_probe_mfma_issue",
+    "woq_hip_moe_route",
+    "woq_hip_linear_grouped",
+    "woq_hip_moe_combine_rows",
 ]
 
 
@@ -149,6 +153,12 @@ def load():
         lib.woq_hip_probe_stream_read.argtypes = [vp, i64, i32, i32, vp, vp]
         lib.woq_hip_probe_empty.restype = i32
         lib.woq_hip_probe_empty.argtypes = [i64, i32, vp]
+        lib.woq_hip_moe_route.restype = i32
+        lib.woq_hip_moe_route.argtypes = [vp, i64, i64, i64, i64, i64, vp, vp, vp, vp, vp, vp, vp, vp, vp]
+        lib.woq_hip_linear_grouped.restype = i32
+        lib.woq_hip_linear_grouped.argtypes = [ctypes.POINTER(LinearParams), vp, i64]
+        lib.woq_hip_moe_combine_rows.restype = i32
+        lib.woq_hip_moe_combine_rows.argtypes = [vp, i32, i64, i64, vp, vp, i64, vp, vp, i32, vp]
         lib.woq_hip_probe_mfma_issue.restype = i32
         lib.woq_hip_probe_mfma_issue.argtypes = [vp, i32, i32, i64, i32, vp, vp]
         if lib.woq_hip_abi_version() != 1:

@@ -22,6 +22,7 @@ handles name Python objects and are understood by the functions of this module o
 """
 import contextlib
 import ctypes
+import os
 import threading
 import weakref
 from typing import List, Optional
@@ -651,6 +652,165 @@ def mixtral_moe_woq(hidden_states, top_x, idx, gate_wei, up_wei, down_wei, routi
     return _moe_expert(hidden_states, top_x.to(dev), idx.to(dev), gate_wei, up_wei, down_wei, routing_weights, output)
 
 
+# ---- a whole layer in grouped launches (decode sizes) -----------------------------------------------
+_MOE_PLANS = {}  # id of the gate list -> plan; the plan keeps the three lists alive, so the id stays theirs
+_MOE_PLAN_LIMIT = 128
+
+
+def _context_pointers(ctx):
+    """[qweight, fp16 scales, bf16 scales, zero points or 0, fp32 bias or 0, N, K, group size, weight dtype,
+    lowp_mode, has g_idx, device index] of a context of either binding."""
+    if _is_python_context(ctx):
+        ptr = lambda t: 0 if t is None else t.data_ptr()
+        N, K = ctx.weight_shape_
+        return [ctx.at_weight_.data_ptr(), ctx.scales_list_[1].data_ptr(), ctx.scales_list_[2].data_ptr(),
+                ptr(ctx.zeros_u8_), ptr(ctx.bias_f32_), N, K, ctx.group_size_, ctx.weight_dtype_, ctx.lowp_mode_,
+                0 if ctx.g_idx_ is None else 1, ctx.at_weight_.device.index]
+    return list(ctx.kernel_pointers())
+
+
+class _MoeGroupedPlan:
+    """What the grouped launches of one layer reuse from call to call: per linear (gate, up, down) the experts'
+    pointer tables and the woq_hip_moe_group structs on the device (one per size class of the experts: fewer than five
+    rows, which lowp_mode BF16 computes in fp16, up to 16 rows, up to 64), the routing buffers they point to and the
+    intermediate rows."""
+
+    def __init__(self, gate_ctx, up_ctx, down_ctx, device):
+        self.lists = (gate_ctx, up_ctx, down_ctx)
+        self.ok = False
+        infos = [[_context_pointers(c) for c in lst] for lst in self.lists]
+        self.shapes = []
+        for rows in infos:
+            first = rows[0]
+            same = all(r[5:11] == first[5:11] and (r[3] == 0) == (first[3] == 0) and (r[4] == 0) == (first[4] == 0)
+                       and r[11] == device.index for r in rows)
+            if not same or first[10] or first[8] not in (_lib.DTYPE_INT4, _lib.DTYPE_INT8) or first[9] not in (0, 1, 2):
+                return
+            self.shapes.append(dict(N=first[5], K=first[6], G=first[7], wd=first[8], lowp=first[9]))
+        g, u, d = self.shapes
+        if (g["N"], g["K"]) != (u["N"], u["K"]) or d["K"] != g["N"] or d["N"] != g["K"] or len({x["lowp"] for x in self.shapes}) != 1:
+            return
+        if any((-(-x["N"] // 16)) % 2 for x in self.shapes):  # the grouped kernel takes two 16-column blocks per workgroup
+            return
+        R = _lib.MOE_ROUTE_MAX
+        i32 = lambda: torch.empty(R, dtype=torch.int32, device=device)
+        self.x_row = torch.empty(R, dtype=torch.int64, device=device)
+        self.slots = [i32(), i32(), i32()]  # experts with few / up to 16 / up to 64 rows
+        self.slot_row0, self.slot_rows, self.row_of, self.slot_of = (i32() for _ in range(4))
+        self.tables = []
+        for rows in infos:
+            col = lambda k: torch.tensor([r[k] for r in rows], dtype=torch.int64, device=device)
+            self.tables.append(dict(qweight=col(0), s16=col(1), sb16=col(2), z8=col(3) if rows[0][3] else None,
+                                    bias=col(4) if rows[0][4] else None))
+        self.structs = {}
+        self.rows = {}  # dtype -> (act, inter, y) for the most routed rows seen
+        self.device = device
+        self.ok = True
+
+    def buffers(self, R, dtype):
+        have = self.rows.get(dtype)
+        if have is None or have[0].shape[0] < R:
+            N1, H = self.shapes[0]["N"], self.shapes[0]["K"]
+            mk = lambda n: torch.empty((R, n), dtype=dtype, device=self.device)
+            have = self.rows[dtype] = (mk(N1), mk(N1), mk(H))
+        return have
+
+    def group_struct(self, linear, cls, f16_scales, gather):
+        """Device copy of the woq_hip_moe_group of one launch (built once)."""
+        key = (linear, cls, f16_scales, gather)
+        st = self.structs.get(key)
+        if st is None:
+            t = self.tables[linear]
+            ptr = lambda x: 0 if x is None else x.data_ptr()
+            fields = [ptr(self.slots[cls]), ptr(self.slot_row0), ptr(self.slot_rows),
+                      ptr(self.x_row) if gather else 0, ptr(t["qweight"]), ptr(t["s16"] if f16_scales else t["sb16"]),
+                      ptr(t["z8"]), ptr(t["bias"])]
+            st = torch.tensor(fields, dtype=torch.int64, device=self.device)
+            self.structs[key] = st
+        return st
+
+
+def _moe_plan(gate_ctx, up_ctx, down_ctx, device):
+    key = id(gate_ctx)
+    plan = _MOE_PLANS.get(key)
+    if plan is None or plan.lists[0] is not gate_ctx or plan.lists[1] is not up_ctx or plan.lists[2] is not down_ctx:
+        if len(_MOE_PLANS) >= _MOE_PLAN_LIMIT:
+            _MOE_PLANS.clear()
+        plan = _MoeGroupedPlan(gate_ctx, up_ctx, down_ctx, device)
+        _MOE_PLANS[key] = plan
+    return plan
+
+
+def _f16_regime(lowp, x_dtype, rows):
+    return lowp == 1 or (lowp == 0 and x_dtype == torch.float16) or (lowp == 2 and rows < 5)
+
+
+def _deepseek_moe_grouped(hidden_states, topk_ids, gate_ctx, up_ctx, down_ctx, routing_weights):
+    """The layer in five to eleven launches and without reading the routing on the host: the routing is sorted on the
+    device, every linear runs once per compute type over all experts that have tokens (woq_hip_linear_grouped), and
+    the contributions of a token are added in ascending expert order.  Returns None when the layer does not fit
+    (more than 64 tokens, mixed experts, act-order, NF4 / FP8 / lowp INT8 ...): the caller then takes the per-expert path."""
+    x = hidden_states
+    if x.dim() != 2 or x.dtype not in (torch.bfloat16, torch.float16) or not x.is_contiguous() or x.data_ptr() % 16:
+        return None
+    T, H = x.shape
+    if topk_ids.dim() != 2 or topk_ids.shape[0] != T or not topk_ids.is_cuda or topk_ids.device != x.device:
+        return None
+    topk = topk_ids.shape[1]
+    if T == 0 or T > 64 or T * topk > _lib.MOE_ROUTE_MAX or T * H * 2 >= 2**31:
+        return None
+    if routing_weights.dtype != x.dtype or routing_weights.dim() != 2 or tuple(routing_weights.shape) != (T, topk) or not routing_weights.is_cuda:
+        return None
+    plan = _moe_plan(gate_ctx, up_ctx, down_ctx, x.device)
+    if not plan.ok or plan.shapes[0]["K"] != H:
+        return None
+    lowp = plan.shapes[0]["lowp"]
+    split = 5 if lowp == 2 else 0  # lowp_mode BF16: experts with fewer than five rows compute in fp16
+    # (size class, bound on its slots' rows): an expert has at most T rows, so the larger classes are empty for small T
+    launches = ([(0, 4)] if split else []) + ([(1, 16)] if T >= split else []) + ([(2, 64)] if T > 16 else [])
+    for cls, bound in launches:
+        f16 = _f16_regime(lowp, x.dtype, bound)
+        # rows must be in the compute type; bf16 rows under fp16 compute are converted for up to 16 rows per slot
+        if f16 and x.dtype == torch.bfloat16 and bound > 16:
+            return None
+        if not f16 and x.dtype == torch.float16:
+            return None
+    lib = _lib.load()
+    ids = topk_ids.to(torch.int64).contiguous()
+    rw = routing_weights.contiguous()
+    R = T * topk
+    N1 = plan.shapes[0]["N"]
+    act, inter, y = plan.buffers(R, x.dtype)  # calls on one stream follow each other
+    out = torch.empty_like(x)
+    code = _kernels._ACT_CODE[x.dtype]
+    with torch.cuda.device(x.device):
+        stream = _kernels._stream()
+        _lib.check(lib.woq_hip_moe_route(ids.data_ptr(), T, topk, len(gate_ctx), split, 16, plan.x_row.data_ptr(),
+                                         plan.slots[0].data_ptr(), plan.slots[1].data_ptr(), plan.slots[2].data_ptr(),
+                                         plan.slot_row0.data_ptr(), plan.slot_rows.data_ptr(), plan.row_of.data_ptr(),
+                                         plan.slot_of.data_ptr(), stream), "moe_route")
+        p = _lib.LinearParams()
+        p.struct_size = ctypes.sizeof(_lib.LinearParams)
+        p.x_dtype = p.out_dtype = code
+        p.stream = torch.cuda.current_stream().cuda_stream
+        p.lowp_mode = lowp
+        p.act_quant_mode = -1
+        steps = ((0, x, act, _lib.FUSE_SILU, None, True), (1, x, inter, _lib.FUSE_MUL, act, True),
+                 (2, inter, y, _lib.FUSE_NONE, None, False))
+        for li, src, dst, fusion, other, gather in steps:
+            sh = plan.shapes[li]
+            p.K, p.N, p.weight_dtype, p.group_size = sh["K"], sh["N"], sh["wd"], sh["G"]
+            p.x, p.out, p.fusion = src.data_ptr(), dst.data_ptr(), fusion
+            p.others[0] = other.data_ptr() if other is not None else None
+            for cls, bound in launches:
+                p.M = bound
+                g = plan.group_struct(li, cls, _f16_regime(lowp, x.dtype, bound), gather)
+                _lib.check(lib.woq_hip_linear_grouped(ctypes.byref(p), g.data_ptr(), R), "woq_linear_grouped")
+        _lib.check(lib.woq_hip_moe_combine_rows(out.data_ptr(), code, T, H, y.data_ptr(), rw.data_ptr(), topk,
+                                                plan.row_of.data_ptr(), plan.slot_of.data_ptr(), 0, stream), "moe_combine_rows")
+    return out
+
+
 def deepseek_moe_woq(hidden_states, topk_ids, gate_ctx, up_ctx, down_ctx, routing_weights, is_distributed):
     """All experts of a layer (csrc/cpu/aten/MoE.cpp:290-328): ``topk_ids`` [tokens, top-k] names the
     experts of every token, the three lists hold one WoqLinearOpContext per expert.  Experts are
@@ -663,6 +823,10 @@ def deepseek_moe_woq(hidden_states, topk_ids, gate_ctx, up_ctx, down_ctx, routin
     num_experts = len(gate_ctx)
     if len(up_ctx) != num_experts or len(down_ctx) != num_experts:
         raise RuntimeError("torch_ipex::deepseek_moe_woq: gate / up / down lists differ in length")
+    if topk_ids.numel() and os.environ.get("IPEX_AMD_MOE_GROUPED", "1") != "0":
+        grouped = _deepseek_moe_grouped(hidden_states, topk_ids, gate_ctx, up_ctx, down_ctx, routing_weights)
+        if grouped is not None:
+            return grouped
     output = torch.zeros_like(hidden_states)
     ids = topk_ids.detach().to("cpu", torch.int64)
     if ids.numel() == 0:

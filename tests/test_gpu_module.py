@@ -567,6 +567,181 @@ def test_deepseek_moe_woq_matches_per_expert_composition(cuda, T, topk):
     assert float(err) < 3e-2, float(err)
 
 
+def test_moe_route_against_the_oracle_token_lists(cuda):
+    """woq_hip_moe_route: sorted positions, slots per compute type and per-token contribution order against the
+    oracle's per-expert token lists (get_expert_topx_idx, MoE.cpp:64-81); ids outside the expert range drop out."""
+    from ipex_amd import _lib
+    from oracle import woq_oracle as O
+
+    lib = _lib.load()
+    g = torch.Generator().manual_seed(5)
+    for T, topk, E, split in ((1, 8, 64, 5), (16, 8, 32, 5), (64, 6, 9, 5), (33, 4, 7, 0), (256, 8, 300, 5)):
+        ids = torch.stack([torch.randperm(E, generator=g)[:topk] for _ in range(T)])
+        if T >= 16:
+            ids[3, 1], ids[7, 0] = -1, E + 3  # not experts
+        R = T * topk
+        dev = ids.to(cuda)
+        x_row = torch.full((R,), -7, dtype=torch.int64, device=cuda)
+        lo, mid, hi, row0, rows, row_of, slot_of = (torch.full((R,), -7, dtype=torch.int32, device=cuda) for _ in range(7))
+        rc = lib.woq_hip_moe_route(dev.data_ptr(), T, topk, E, split, 16, x_row.data_ptr(), lo.data_ptr(), mid.data_ptr(),
+                                   hi.data_ptr(), row0.data_ptr(), rows.data_ptr(), row_of.data_ptr(), slot_of.data_ptr(), None)
+        assert rc == 0, lib.woq_hip_last_error()
+        torch.cuda.synchronize()
+        valid = (ids >= 0) & (ids < E)
+        top_x, idx = O.expert_token_lists(torch.where(valid, ids, torch.full_like(ids, E)).numpy(), E + 1)
+        pos, want_row, want_lo, want_mid, want_hi, want_rows = 0, [], {}, {}, {}, {}
+        entry_pos = {}
+        for e in range(E):
+            n = len(top_x[e])
+            if n:
+                (want_lo if n < split else want_mid if n <= 16 else want_hi)[pos] = e
+                want_rows[pos] = n
+            for t, j in zip(top_x[e], idx[e]):
+                entry_pos[(int(t), int(j))] = pos
+                want_row.append(int(t))
+                pos += 1
+        assert x_row.cpu().tolist()[:pos] == want_row
+        assert row0.cpu().tolist() == list(range(R))
+        lo_c, mid_c, hi_c, rows_c = lo.cpu().tolist(), mid.cpu().tolist(), hi.cpu().tolist(), rows.cpu().tolist()
+        for p in range(R):
+            assert lo_c[p] == want_lo.get(p, -1) and mid_c[p] == want_mid.get(p, -1) and hi_c[p] == want_hi.get(p, -1), (T, p)
+            assert rows_c[p] == want_rows.get(p, 0)
+        ro, so = row_of.cpu().view(T, topk), slot_of.cpu().view(T, topk)
+        for t in range(T):
+            order = sorted((int(ids[t, j]), j) for j in range(topk) if bool(valid[t, j]))
+            for i in range(topk):
+                if i < len(order):
+                    assert int(ro[t, i]) == entry_pos[(t, order[i][1])] and int(so[t, i]) == order[i][1]
+                else:
+                    assert int(ro[t, i]) == -1
+
+
+@pytest.mark.parametrize("weight_dtype,lowp", [("INT4", "BF16"), ("INT8", "BF16"), ("INT4", "NONE")])
+@pytest.mark.parametrize("T,topk", [(1, 4), (5, 3), (16, 4), (40, 2), (64, 6)])
+def test_deepseek_moe_grouped_launches_equal_the_per_expert_path(cuda, monkeypatch, weight_dtype, lowp, T, topk):
+    """The layer in grouped launches (routing sorted on the device, one launch per linear and compute type over all
+    experts, contributions added in ascending expert order) against the per-expert path, which reads the routing on
+    the host: bit for bit, with experts that get one, a few, many or no tokens."""
+    from ipex_amd import _lib
+
+    ipex = _ipex()
+    E, H, I = 9, 256, 384
+    G = 64 if weight_dtype == "INT4" else -1
+    mk = lambda k, n, s: _woq_module(ipex, k, n, weight_dtype, G, lowp, bias=False, seed=s)
+    ctxs = [[mk(H, I, 300 + 3 * e)._op_context for e in range(E)], [mk(H, I, 301 + 3 * e)._op_context for e in range(E)],
+            [mk(I, H, 302 + 3 * e)._op_context for e in range(E)]]
+    g = torch.Generator().manual_seed(100 * T + topk)
+    hidden = torch.randn(T, H, generator=g).to(torch.bfloat16).to(cuda)
+    # skewed routing: expert 0 is popular, expert E - 1 never chosen
+    ids = torch.stack([torch.cat([torch.zeros(1, dtype=torch.int64), 1 + torch.randperm(E - 2, generator=g)[:topk - 1]]) if t % 3 else
+                       torch.randperm(E - 1, generator=g)[:topk] for t in range(T)]).to(cuda)
+    rw = torch.softmax(torch.randn(T, topk, generator=g), -1).to(torch.bfloat16).to(cuda)
+    op = torch.ops.torch_ipex.deepseek_moe_woq
+    monkeypatch.setenv("IPEX_AMD_MOE_GROUPED", "0")
+    want = op(hidden, ids, ctxs[0], ctxs[1], ctxs[2], rw, False)
+    assert _lib.last_kernel() == "moe_scale_add_rows"
+    monkeypatch.setenv("IPEX_AMD_MOE_GROUPED", "1")
+    got = op(hidden, ids, ctxs[0], ctxs[1], ctxs[2], rw, False)
+    assert _lib.last_kernel() == "moe_combine_rows"
+    assert torch.equal(got, want)
+    # again with other routing through the cached plan
+    ids2 = ids.flip(0).contiguous()
+    monkeypatch.setenv("IPEX_AMD_MOE_GROUPED", "0")
+    want2 = op(hidden, ids2, ctxs[0], ctxs[1], ctxs[2], rw, False)
+    monkeypatch.setenv("IPEX_AMD_MOE_GROUPED", "1")
+    assert torch.equal(op(hidden, ids2, ctxs[0], ctxs[1], ctxs[2], rw, False), want2)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("accumulate", [0, 1])
+def test_moe_combine_rows_bit_exact(cuda, dtype, accumulate):
+    """woq_hip_moe_combine_rows against the oracle's sequential weighted scatter applied expert by expert."""
+    from ipex_amd import _kernels, _lib
+    from oracle import woq_oracle as O
+
+    lib = _lib.load()
+    name = {torch.bfloat16: "bf16", torch.float16: "fp16", torch.float32: "fp32"}[dtype]
+    g = torch.Generator().manual_seed(3)
+    T, topk, E, H = 19, 10, 13, 100  # ten contributions: two groups of eight in the kernel; H not a multiple of 8
+    ids = torch.stack([torch.randperm(E, generator=g)[:topk] for _ in range(T)])
+    ids[2, 3] = -1
+    R = T * topk
+    bufs = [torch.empty(R, dtype=torch.int32, device=cuda) for _ in range(7)]
+    x_row = torch.empty(R, dtype=torch.int64, device=cuda)
+    rc = lib.woq_hip_moe_route(ids.to(cuda).data_ptr(), T, topk, E, 5, 16, x_row.data_ptr(), *[b.data_ptr() for b in bufs], None)
+    assert rc == 0, lib.woq_hip_last_error()
+    row_of, slot_of = bufs[5], bufs[6]
+    expert_out = torch.randn(R, H, generator=g).to(dtype)
+    rw = torch.rand(T, topk, generator=g).to(dtype)
+    out0 = torch.randn(T, H, generator=g).to(dtype)
+    out = out0.to(cuda).clone()
+    rc = lib.woq_hip_moe_combine_rows(out.data_ptr(), _kernels._ACT_CODE[dtype], T, H, expert_out.to(cuda).data_ptr(),
+                                      rw.to(cuda).data_ptr(), topk, row_of.data_ptr(), slot_of.data_ptr(), accumulate, None)
+    assert rc == 0, lib.woq_hip_last_error()
+    valid = (ids >= 0) & (ids < E)
+    top_x, idx = O.expert_token_lists(torch.where(valid, ids, torch.full_like(ids, E)).numpy(), E + 1)
+    want = out0.float().numpy() if accumulate else np.zeros((T, H), dtype=np.float32)
+    pos = 0
+    for e in range(E):
+        n = len(top_x[e])
+        want = O.moe_index_mul_index_add(want, expert_out[pos:pos + n].float().numpy(), rw.float().numpy(), top_x[e], idx[e], name)
+        pos += n
+    assert np.array_equal(out.float().cpu().numpy(), want)
+
+
+def test_deepseek_moe_grouped_groups_of_128_and_rejections(cuda, monkeypatch):
+    """Groups of 128: the per-expert path serves experts with fewer than five rows with the decode kernel that keeps the
+    weights as integers, the grouped path dequantizes them -- two roundings of the same product, compared to tolerance
+    and both against the float layer.  Then what the grouped entry point refuses."""
+    import ctypes
+    from ipex_amd import _lib
+
+    ipex = _ipex()
+    E, H, I, T, topk = 6, 512, 256, 3, 2
+    mk = lambda k, n, s: _woq_module(ipex, k, n, "INT4", 128, "BF16", bias=False, seed=s)
+    mods = [[mk(H, I, 400 + 3 * e) for e in range(E)], [mk(H, I, 401 + 3 * e) for e in range(E)], [mk(I, H, 402 + 3 * e) for e in range(E)]]
+    ctxs = [[m._op_context for m in ms] for ms in mods]
+    g = torch.Generator().manual_seed(9)
+    hidden = torch.randn(T, H, generator=g).to(torch.bfloat16).to(cuda)
+    ids = torch.stack([torch.randperm(E, generator=g)[:topk] for _ in range(T)]).to(cuda)
+    rw = torch.softmax(torch.randn(T, topk, generator=g), -1).to(torch.bfloat16).to(cuda)
+    op = torch.ops.torch_ipex.deepseek_moe_woq
+    monkeypatch.setenv("IPEX_AMD_MOE_GROUPED", "0")
+    a = op(hidden, ids, ctxs[0], ctxs[1], ctxs[2], rw, False).float()
+    monkeypatch.setenv("IPEX_AMD_MOE_GROUPED", "1")
+    b = op(hidden, ids, ctxs[0], ctxs[1], ctxs[2], rw, False).float()
+    assert _lib.last_kernel() == "moe_combine_rows"
+    assert float((a - b).norm() / a.norm()) < 6e-3
+    deq = lambda m: ipex.quantization.dequantize_per_block(
+        m._op_context.to_public(m._op_context.get_weight()).cpu(), m._op_context.get_scales().cpu(),
+        m._op_context.get_zero_points().cpu(), ipex.quantization.WoqWeightDtype.INT4, 128, [m.out_features, m.in_features])
+    dense = torch.zeros(T, H)
+    for t in range(T):
+        for j in range(topk):
+            e = int(ids[t, j])
+            xc = hidden[t].float().cpu()
+            ye = (torch.nn.functional.silu(deq(mods[0][e]) @ xc) * (deq(mods[1][e]) @ xc)) @ deq(mods[2][e]).t()
+            dense[t] += ye * float(rw[t, j])
+    for got in (a, b):
+        assert float((got.cpu() - dense).norm() / dense.norm()) < 2e-2
+    # the C entry point: what it refuses
+    lib = _lib.load()
+    p = _lib.LinearParams()
+    p.struct_size = ctypes.sizeof(_lib.LinearParams)
+    p.K, p.N, p.M, p.weight_dtype, p.group_size, p.lowp_mode = H, I, 16, 2, 128, 2
+    p.x_dtype = p.out_dtype = 2
+    p.x = p.out = hidden.data_ptr()
+    table = torch.zeros(8, dtype=torch.int64, device=cuda)
+    for change, text in ((dict(M=65), "rows per slot"), (dict(weight_dtype=3), "INT4 and INT8"), (dict(lowp_mode=3), "lowp_mode"),
+                         (dict(fusion=_lib.FUSE_GELU_ERF), "post-op"), (dict(N=48), "even number"), (dict(K=H + 64), "multiple of the weight tile")):
+        q = _lib.LinearParams.from_buffer_copy(p)
+        for k, v in change.items():
+            setattr(q, k, v)
+        assert lib.woq_hip_linear_grouped(ctypes.byref(q), table.data_ptr(), 4) != 0
+        assert text in lib.woq_hip_last_error().decode(), (change, lib.woq_hip_last_error())
+    assert lib.woq_hip_linear_grouped(ctypes.byref(p), None, 4) != 0
+
+
 def test_mixtral_moe_woq_single_expert_and_errors(cuda):
     ipex = _ipex()
     H, I, T = 128, 256, 6
