@@ -832,6 +832,29 @@ def test_fp8_unit_rows_read_out_the_dequantized_weight_bit_for_bit(cuda, regime,
         assert np.array_equal(acc, want[:, k0:k0 + rows].T), (regime, kernel, k0)
 
 
+@pytest.mark.parametrize("regime", ["fp16", "bf16"])
+@pytest.mark.parametrize("sym", [True, False])
+@pytest.mark.parametrize("kernel", [1, 2, 8, 6])  # small-M, tiled, dequantizing decode, prefill
+def test_int8_unit_rows_read_out_the_dequantized_weight_bit_for_bit(cuda, regime, sym, kernel):
+    """As for FP8: unit-vector rows make the fp32 accumulator the kernel's own w[n, k] = cd((q - z) * s), here for
+    every int8 code with and without zero points, against the oracle bit for bit."""
+    N, K, G = 64, 256, 128
+    g = torch.Generator().manual_seed(92)
+    q = torch.stack([torch.randperm(256, generator=g) for _ in range(N)]).sub(128).to(torch.int8)  # every code in every row
+    scales = 0.0005 + 0.0015 * torch.rand((N, K // G), generator=g)
+    zeros = None if sym else torch.randint(-128, 128, (N, K // G), generator=g).float()
+    xdt = torch.float16 if regime == "fp16" else torch.bfloat16
+    case = dict(x=None, qweight=q, scales=scales, zeros=zeros, bias=None, M=0, K=K, N=N, group_size=G, weight_dtype=1)
+    ctx = make_context(case, O.LOWP_FP16 if regime == "fp16" else O.LOWP_BF16)
+    want = O._round_to(O.dequantize_woq_weight(q.numpy(), N, K, O._round_to(scales.numpy(), regime),
+                                               None if sym else zeros.numpy(), 1, G), regime)
+    rows = 64 if kernel in (1, 8) else 256
+    eye = torch.eye(K, dtype=xdt)
+    for k0 in range(0, K, rows):
+        acc = ctx.run(eye[k0:k0 + rows].cuda(), out_fp32=True, force_kernel=kernel).cpu().numpy()
+        assert np.array_equal(acc, want[:, k0:k0 + rows].T), (regime, sym, kernel, k0)
+
+
 def test_fp8_rejections(cuda):
     syn = _synthetic()
     case = syn.make_fp8_case(65, 4, 256, 32, group_size=64)
