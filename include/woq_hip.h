@@ -326,7 +326,8 @@ int woq_hip_moe_scale_add_rows(void* out, int dtype, int64_t T, int64_t H, const
  *   the first position of an expert carries the expert's id -- in slot_expert_lo if the expert has fewer than split_lo
  *   rows, in slot_expert_mid if at most split_mid, else in slot_expert_hi, -1 in the others -- with slot_row0[p] = p and
  *   slot_rows[p] = its row count, every other position -1; row_of[t, i] / slot_of[t, i] = sorted position and top-k slot of token t's i-th contribution in ascending
- *   expert order (row_of -1: none).  An expert id outside [0, experts) contributes nothing.
+ *   expert order (row_of -1: none).  An expert id outside [0, experts) contributes nothing, and neither
+ *   do an expert's entries beyond its first 64 (a slot holds at most 64 rows).
  * woq_hip_linear_grouped: one linear of every expert that has a slot, in one launch.  p describes one expert's problem
  *   (all experts share N, K, group size, weight dtype INT4 or INT8, lowp_mode NONE / FP16 / BF16, post-op none / silu /
  *   mul) with M = the bound on a slot's rows (1..64; it selects the compute type like woq_hip_linear's M, so a layer

@@ -101,6 +101,7 @@ __global__ void moe_scale_add_rows_kernel(void* __restrict__ out, const void* __
 //   slot_of[t, i]   its top-k slot.
 // An expert id outside [0, experts) contributes nothing.  R <= kMoeRouteMax entries, compared pairwise from LDS.
 constexpr int kMoeRouteMax = WOQ_HIP_MOE_ROUTE_MAX;
+constexpr int kMoeSlotRowsMax = 64;
 __global__ __launch_bounds__(256) void moe_route_kernel(const int64_t* __restrict__ ids, int R, int topk, int experts,
                                                         int split_lo, int split_mid, int64_t* __restrict__ x_row,
                                                         int32_t* __restrict__ slot_lo, int32_t* __restrict__ slot_mid,
@@ -135,8 +136,10 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const int64_t* __restric
     x_row[p] = t;
     if (rank == 0) {
       (count < split_lo ? slot_lo : count <= split_mid ? slot_mid : slot_hi)[p] = e;
-      slot_rows[p] = count;
+      slot_rows[p] = count < kMoeSlotRowsMax ? count : kMoeSlotRowsMax;
     }
+    // a slot holds at most 64 rows (an expert gets more only if a token names it twice): the rest contribute nothing
+    if (rank >= kMoeSlotRowsMax) continue;
     int ord = 0;
     for (int jj = 0; jj < topk; ++jj) {
       const int ek = se[t * topk + jj];

@@ -653,7 +653,9 @@ def mixtral_moe_woq(hidden_states, top_x, idx, gate_wei, up_wei, down_wei, routi
 
 
 # ---- a whole layer in grouped launches (decode sizes) -----------------------------------------------
-_MOE_PLANS = {}  # id of the gate list -> plan; the plan keeps the three lists alive, so the id stays theirs
+# (id of the gate list, stream) -> plan; the plan keeps the three lists alive, so the id stays theirs.  One plan per
+# stream: its routing buffers and intermediate rows are reused from call to call, and calls on one stream follow each other.
+_MOE_PLANS = {}
 _MOE_PLAN_LIMIT = 128
 
 
@@ -731,7 +733,7 @@ class _MoeGroupedPlan:
 
 
 def _moe_plan(gate_ctx, up_ctx, down_ctx, device):
-    key = id(gate_ctx)
+    key = (id(gate_ctx), device.index, torch.cuda.current_stream(device).cuda_stream)
     plan = _MOE_PLANS.get(key)
     if plan is None or plan.lists[0] is not gate_ctx or plan.lists[1] is not up_ctx or plan.lists[2] is not down_ctx:
         if len(_MOE_PLANS) >= _MOE_PLAN_LIMIT:

@@ -616,6 +616,24 @@ def test_moe_route_against_the_oracle_token_lists(cuda):
                     assert int(ro[t, i]) == -1
 
 
+def test_moe_route_keeps_at_most_64_rows_of_an_expert(cuda):
+    from ipex_amd import _lib
+
+    lib = _lib.load()
+    T, topk, E = 80, 2, 5
+    ids = torch.stack([torch.tensor([2, 3 if t % 2 else 4]) for t in range(T)])  # expert 2 gets all 80 tokens
+    R = T * topk
+    x_row = torch.empty(R, dtype=torch.int64, device=cuda)
+    lo, mid, hi, row0, rows, row_of, slot_of = (torch.empty(R, dtype=torch.int32, device=cuda) for _ in range(7))
+    rc = lib.woq_hip_moe_route(ids.to(cuda).data_ptr(), T, topk, E, 5, 16, x_row.data_ptr(), lo.data_ptr(), mid.data_ptr(), hi.data_ptr(),
+                               row0.data_ptr(), rows.data_ptr(), row_of.data_ptr(), slot_of.data_ptr(), None)
+    assert rc == 0, lib.woq_hip_last_error()
+    assert int(hi[0]) == 2 and int(rows[0]) == 64 and x_row[:80].cpu().tolist() == list(range(80))
+    ro = row_of.cpu().view(T, topk)
+    assert ro[:64, 0].tolist() == list(range(64)) and bool((ro[64:, 0] == -1).all())
+    assert bool((ro[:, 1] >= 80).all())  # the other contribution of every token is kept
+
+
 @pytest.mark.parametrize("weight_dtype,lowp", [("INT4", "BF16"), ("INT8", "BF16"), ("INT4", "NONE")])
 @pytest.mark.parametrize("T,topk", [(1, 4), (5, 3), (16, 4), (40, 2), (64, 6)])
 def test_deepseek_moe_grouped_launches_equal_the_per_expert_path(cuda, monkeypatch, weight_dtype, lowp, T, topk):
