@@ -64,3 +64,48 @@ def test_graph_replays_match_eager(cuda):
         for (label, *_), a, b in zip(CASES, got, want):
             assert torch.equal(a, b), (label, rep)
         assert all(bool(torch.isfinite(y.float()).all()) for y in got)
+
+
+def test_moe_layer_graph_replays_with_new_routing(cuda):
+    """deepseek_moe_woq with its routing sorted on the device, captured once: the replays see new hidden states, new
+    expert ids and new routing weights (written into the captured tensors) and must equal the eager results -- the
+    captured launches have no shape that depends on the routing."""
+    import ipex_amd  # noqa: F401
+    from ipex_amd import _lib
+    from test_gpu_module import _woq_module
+
+    E, H, I, T, topk = 8, 256, 384, 6, 3
+    mk = lambda k, n, s: _woq_module(ipex_amd, k, n, "INT4", 64, "BF16", bias=False, seed=s)._op_context
+    gate, up, down = [mk(H, I, 700 + e) for e in range(E)], [mk(H, I, 720 + e) for e in range(E)], [mk(I, H, 740 + e) for e in range(E)]
+    op = torch.ops.torch_ipex.deepseek_moe_woq
+    gen = torch.Generator().manual_seed(3)
+
+    def draw():
+        hidden = torch.randn(T, H, generator=gen).to(torch.bfloat16)
+        ids = torch.stack([torch.randperm(E, generator=gen)[:topk] for _ in range(T)])
+        rw = torch.softmax(torch.randn(T, topk, generator=gen), -1).to(torch.bfloat16)
+        return hidden, ids, rw
+
+    static = [t.cuda() for t in draw()]
+    s = torch.cuda.Stream()
+    s.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(s):
+        op(static[0], static[1], gate, up, down, static[2], False)  # builds the layer's pointer tables and buffers
+        assert _lib.last_kernel() == "moe_combine_rows"
+    torch.cuda.current_stream().wait_stream(s)
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g, stream=s):
+        static_out = op(static[0], static[1], gate, up, down, static[2], False)
+    for rep in range(4):
+        new = draw()
+        if rep == 2:
+            new[1][:, 0] = 5  # every token to expert 5: one expert with six rows, the others with few or none
+        for dst, src in zip(static, new):
+            dst.copy_(src)
+        g.replay()
+        torch.cuda.synchronize()
+        got = static_out.clone()
+        want = op(*[t.cuda() for t in new[:2]], gate, up, down, new[2].cuda(), False)
+        torch.cuda.synchronize()
+        assert torch.equal(got, want), rep
