@@ -321,19 +321,23 @@ int woq_hip_moe_scale_add_rows(void* out, int dtype, int64_t T, int64_t H, const
  * whose expert loop runs on the host because its tensors live there).
  *
  * woq_hip_moe_route: topk_ids int64 [T, topk] on the device -> the (token, slot) entries sorted by expert, stable, so
- *   that inside an expert the tokens ascend (get_expert_topx_idx, MoE.cpp:64-81).  All outputs have T * topk entries
- *   (at most WOQ_HIP_MOE_ROUTE_MAX): x_row[p] = token of the entry at sorted position p; one slot per sorted position:
- *   the first position of an expert carries the expert's id -- in slot_expert_lo if the expert has fewer than split_lo
- *   rows, in slot_expert_mid if at most split_mid, else in slot_expert_hi, -1 in the others -- with slot_row0[p] = p and
- *   slot_rows[p] = its row count, every other position -1; row_of[t, i] / slot_of[t, i] = sorted position and top-k slot of token t's i-th contribution in ascending
- *   expert order (row_of -1: none).  An expert id outside [0, experts) contributes nothing, and neither
- *   do an expert's entries beyond its first 64 (a slot holds at most 64 rows).
+ *   that inside an expert the tokens ascend (get_expert_topx_idx, MoE.cpp:64-81).  x_row[p] (T * topk entries, at most
+ *   WOQ_HIP_MOE_ROUTE_MAX) = token of the entry at sorted position p.  slots: int32 [4][3][S], S >= min(T * topk, experts):
+ *   per size class the experts that have tokens, densely from index 0 in ascending expert order, as three arrays --
+ *   expert id (-1: unused entry), first sorted position, number of rows (at most 64).  Classes: 0 fewer than split_lo
+ *   rows, 1 at most split_mid, 2 more, 3 (only with use_single) exactly one row, taken out of class 0.
+ *   row_of[t, i] / slot_of[t, i] = sorted position and top-k slot of token t's i-th contribution in ascending expert
+ *   order (row_of -1: none).  An expert id outside [0, experts) contributes nothing, and neither do an expert's entries
+ *   beyond its first 64 (a slot holds at most 64 rows).
  * woq_hip_linear_grouped: one linear of every expert that has a slot, in one launch.  p describes one expert's problem
  *   (all experts share N, K, group size, weight dtype INT4 or INT8, lowp_mode NONE / FP16 / BF16, post-op none / silu /
  *   mul) with M = the bound on a slot's rows (1..64; it selects the compute type like woq_hip_linear's M, so a layer
  *   under lowp_mode BF16 takes one call with M = 4 on the slots of experts with fewer than five rows and one with a
- *   larger M on the others; M <= 16 and M > 16 also select a kernel with one or four row tiles, hence three tables); p's weight, scale, zero
- *   point and bias pointers are ignored.  x: the rows the slots read, out / others[0]: [routed rows, N].  group: DEVICE
+ *   larger M on the others; M <= 16 and M > 16 also select a kernel with one or four row tiles, hence the size classes); p's weight, scale, zero
+ *   point and bias pointers are ignored -- except that a non-NULL scale_zero_f16x2 says that the group's scales table
+ *   holds the experts' (fp16 scale, fp16 128 + zero) dword tables: the call then runs the single-row decode kernel
+ *   (M must be 1: one row per slot, the class of experts with exactly one row; 4-bit weights in groups of 128 * 2^k, K a multiple of 256,
+ *   fp16 compute).  x: the rows the slots read, out / others[0]: [routed rows, N].  group: DEVICE
  *   pointer to a woq_hip_moe_group.  Rows of a slot are row0 .. row0 + rows - 1 of out; they read row x_row[row] of x,
  *   or the same row when x_row is NULL.  Needs what the dequantizing decode kernel needs: K a multiple of the weight tile,
  *   a power-of-two or per-channel group size, an even number of 16-column blocks, rows in the compute type (bf16 rows
@@ -354,9 +358,8 @@ typedef struct woq_hip_moe_group {
   const float* const* bias;        /* [experts] or NULL */
 } woq_hip_moe_group;
 int woq_hip_moe_route(const int64_t* topk_ids, int64_t T, int64_t topk, int64_t experts, int64_t split_lo,
-                      int64_t split_mid, int64_t* x_row, int32_t* slot_expert_lo, int32_t* slot_expert_mid,
-                      int32_t* slot_expert_hi, int32_t* slot_row0, int32_t* slot_rows, int32_t* row_of, int32_t* slot_of,
-                      void* stream);
+                      int64_t split_mid, int use_single, int64_t S, int64_t* x_row, int32_t* slots, int32_t* row_of,
+                      int32_t* slot_of, void* stream);
 int woq_hip_linear_grouped(const woq_hip_linear_params* p, const void* group, int64_t slots);
 int woq_hip_moe_combine_rows(void* out, int dtype, int64_t T, int64_t H, const void* expert_out,
                              const void* routing_weights, int64_t topk, const int32_t* row_of, const int32_t* slot_of,

@@ -227,11 +227,13 @@ class WoqLinearOpContext : public torch::CustomClassHolder {
   std::vector<int64_t> get_weight_shape() { return {N_, K_}; }
   // What a grouped launch over many contexts (the experts of a mixture-of-experts layer) needs of each: the device
   // addresses of the packed weight, the fp16 and bf16 scales, the zero points and the fp32 bias (0: none), then
-  // N, K, group size, weight dtype, lowp_mode, whether the input channels are permuted (g_idx), the device index.
+  // N, K, group size, weight dtype, lowp_mode, whether the input channels are permuted (g_idx), the device index,
+  // and the (fp16 scale, fp16 128 + zero) dword table of the single-row decode kernel (0: none).
   std::vector<int64_t> kernel_pointers() {
     auto addr = [](const Tensor& t) -> int64_t { return t.defined() ? (int64_t)(uintptr_t)t.data_ptr() : 0; };
     return {addr(packed_), addr(q_.s16), addr(q_.sb16), q_.z8.has_value() ? addr(*q_.z8) : 0, addr(bias_f32_),
-            N_, K_, group_size_, weight_dtype_, lowp_mode_, g_src_.defined() ? 1 : 0, (int64_t)packed_.device().index()};
+            N_, K_, group_size_, weight_dtype_, lowp_mode_, g_src_.defined() ? 1 : 0, (int64_t)packed_.device().index(),
+            q_.sz.has_value() ? addr(*q_.sz) : 0};
   }
   optional<Tensor> get_g_idx() { return g_idx_; }
   // The reference keeps a dequantized bf16 copy of the weight for batches of 64 rows and more when

@@ -347,6 +347,16 @@ int woq_hip_linear_grouped(const woq_hip_linear_params* p, const void* group, in
   f.G = G; f.KG = KG; f.bias = nullptr; f.fusion = p->fusion;
   f.other0 = p->others[0]; f.other1 = nullptr; f.out = p->out; f.out_dtype = p->out_dtype;
   f.nf4 = 0; f.fp8 = 0;
+  if (p->scale_zero_f16x2) {
+    // one routed row per slot on the single-row decode kernel: the group's scales table holds the experts'
+    // (fp16 scale, fp16 128 + zero) dword tables
+    if (p->M != 1) return set_error("woq_linear_grouped: (scale, zero) dword tables go with one row per slot (M = 1)");
+    f.scales = nullptr;
+    if (!decode_kernel_applies(f, wbits, regime, (const uint32_t*)p->scale_zero_f16x2))
+      return set_error("woq_linear_grouped: the single-row kernel takes 4-bit weights in groups of 128 x 2^k, fp16 compute "
+                       "and K a multiple of 256");
+    return launch_decode_grouped(f, (const MoeGroup*)group, slots, (hipStream_t)p->stream);
+  }
   return launch_decode_dq_grouped(f, wbits, regime, (const MoeGroup*)group, slots, (hipStream_t)p->stream);
 }
 
@@ -409,17 +419,16 @@ int woq_hip_moe_scale_add_rows(void* out, int dtype, int64_t T, int64_t H, const
 }
 
 int woq_hip_moe_route(const int64_t* topk_ids, int64_t T, int64_t topk, int64_t experts, int64_t split_lo,
-                      int64_t split_mid, int64_t* x_row, int32_t* slot_expert_lo, int32_t* slot_expert_mid,
-                      int32_t* slot_expert_hi, int32_t* slot_row0, int32_t* slot_rows, int32_t* row_of, int32_t* slot_of,
-                      void* stream) {
+                      int64_t split_mid, int use_single, int64_t S, int64_t* x_row, int32_t* slots, int32_t* row_of,
+                      int32_t* slot_of, void* stream) {
   if (T < 0 || topk <= 0 || experts <= 0) return set_error("moe_route: bad size");
   if (T * topk > WOQ_HIP_MOE_ROUTE_MAX)
     return set_error("moe_route: at most %d (token, slot) entries, got %lld", WOQ_HIP_MOE_ROUTE_MAX, (long long)(T * topk));
-  if (T > 0 && (!topk_ids || !x_row || !slot_expert_lo || !slot_expert_mid || !slot_expert_hi || !slot_row0 || !slot_rows ||
-                !row_of || !slot_of))
-    return set_error("moe_route: null pointer");
-  return launch_moe_route(topk_ids, T, topk, experts, split_lo, split_mid, x_row, slot_expert_lo, slot_expert_mid,
-                          slot_expert_hi, slot_row0, slot_rows, row_of, slot_of, (hipStream_t)stream);
+  const int64_t need = T * topk < experts ? T * topk : experts;  // experts that can have tokens
+  if (S < need) return set_error("moe_route: slot tables of %lld entries, %lld experts can have tokens", (long long)S, (long long)need);
+  if (T > 0 && (!topk_ids || !x_row || !slots || !row_of || !slot_of)) return set_error("moe_route: null pointer");
+  return launch_moe_route(topk_ids, T, topk, experts, split_lo, split_mid, use_single, S, x_row, slots, row_of, slot_of,
+                          (hipStream_t)stream);
 }
 
 int woq_hip_moe_combine_rows(void* out, int dtype, int64_t T, int64_t H, const void* expert_out,

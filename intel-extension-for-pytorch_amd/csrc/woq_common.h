@@ -277,6 +277,14 @@ __device__ __forceinline__ void epilogue_store(const Epilogue& e, int64_t m, int
   store_act(e.out, e.out_dtype, idx, y);
 }
 
+// a pointer every lane of the wave loaded from the same address, moved to scalar registers
+template <typename T>
+__device__ __forceinline__ T* dq_uniform(T* p) {
+  const uint64_t v = (uint64_t)p;
+  const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+  return (T*)(((uint64_t)hi << 32) | lo);
+}
+
 // ---- 4-bit weights as MFMA operands: one packed dword (8 weights of one row) -> 8 bf16 / fp16 ----
 // Per-lane dequantization constants of one weight row and quantization group.
 template <int REGIME>

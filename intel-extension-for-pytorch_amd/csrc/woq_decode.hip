@@ -211,8 +211,27 @@ __global__ __launch_bounds__(1024, 8) void woq_decode_kernel(const DecodeArgs a)
 //     against -1 as above;
 //   * every row of the A operand is the one activation row, so every row of D is the result: a lane
 //     scales and accumulates one element per tile instead of four.
-template <bool XBF16, int NTW, int KPW, bool ONE_ROUND>
-__global__ __launch_bounds__(KPW == 2 ? 1024 : 512, KPW == 2 ? 8 : 4) void woq_decode_m1_kernel(const DecodeArgs a) {
+// GROUPED (mixture of experts): the workgroups with blockIdx.z = s serve slot s, one routed row of one expert, whose
+// packed weight, (scale, zero) table and bias come from pointer tables in device memory; an empty slot exits.
+template <bool XBF16, int NTW, int KPW, bool ONE_ROUND, bool GROUPED>
+__global__ __launch_bounds__(KPW == 2 ? 1024 : 512, KPW == 2 ? 8 : 4) void woq_decode_m1_kernel(const DecodeArgs a_in) {
+  DecodeArgs ag;
+  if constexpr (GROUPED) {
+    const MoeGroup& g = *a_in.grp;
+    const int slot = (int)blockIdx.z;
+    const int e = __builtin_amdgcn_readfirstlane(g.slot_expert[slot]);
+    if (e < 0) return;  // the whole workgroup, before anything is synchronized
+    const int64_t row = __builtin_amdgcn_readfirstlane(g.slot_row0[slot]);
+    const int64_t xr = g.x_row ? (int64_t)__builtin_amdgcn_readfirstlane((int)g.x_row[row]) : row;
+    ag = a_in;
+    ag.qweight = dq_uniform((const uint8_t*)g.qweight[e]);
+    ag.sz = dq_uniform((const uint32_t*)g.scales[e]);
+    ag.bias = g.bias ? dq_uniform(g.bias[e]) : nullptr;
+    ag.x = a_in.x + xr * a_in.K;
+    ag.out = (uint8_t*)a_in.out + row * a_in.N * 2;
+    if (a_in.other0) ag.other0 = (const uint8_t*)a_in.other0 + row * a_in.N * 2;
+  }
+  const DecodeArgs& a = GROUPED ? ag : a_in;
   constexpr int SLICE = KPW * kTileK4;  // K elements of one wave per round
   extern __shared__ __align__(16) uint8_t smem[];
   const int W = a.W;
@@ -367,9 +386,13 @@ __global__ __launch_bounds__(KPW == 2 ? 1024 : 512, KPW == 2 ? 8 : 4) void woq_d
 }
 
 template <bool XBF16, int NTW, int KPW, bool ONE_ROUND>
-static int launch_decode_m1_cfg(const DecodeArgs& a, hipStream_t st) {
+static int launch_decode_m1_cfg(const DecodeArgs& a, hipStream_t st, int slots = 0) {
   const size_t smem = (size_t)NTW * 16 * 16 * sizeof(float) + (size_t)a.W * KPW * kTileK4 * sizeof(uint16_t);
-  woq_decode_m1_kernel<XBF16, NTW, KPW, ONE_ROUND><<<(unsigned)((a.NT + NTW - 1) / NTW), a.W * 64, smem, st>>>(a);
+  const unsigned grid = (unsigned)((a.NT + NTW - 1) / NTW);
+  if (slots > 0)
+    woq_decode_m1_kernel<XBF16, NTW, KPW, ONE_ROUND, true><<<dim3(grid, 1, (unsigned)slots), a.W * 64, smem, st>>>(a);
+  else
+    woq_decode_m1_kernel<XBF16, NTW, KPW, ONE_ROUND, false><<<grid, a.W * 64, smem, st>>>(a);
   return check_launch("woq_decode_m1_kernel");
 }
 
@@ -395,8 +418,19 @@ bool decode_kernel_applies(const FpArgs& f, int wbits, int regime, const uint32_
          (tpg & (tpg - 1)) == 0 && (f.K % (kDecodeKPW * kTileK4)) == 0 && (f.x_dtype == WOQ_HIP_ACT_BF16 || f.x_dtype == WOQ_HIP_ACT_FP16);
 }
 
-int launch_decode(const FpArgs& f, const uint32_t* sz, hipStream_t st) {
+static int launch_decode_impl(const FpArgs& f, const uint32_t* sz, hipStream_t st, const MoeGroup* grp, int slots);
+
+int launch_decode(const FpArgs& f, const uint32_t* sz, hipStream_t st) { return launch_decode_impl(f, sz, st, nullptr, 0); }
+
+int launch_decode_grouped(const FpArgs& f, const MoeGroup* grp, int64_t slots, hipStream_t st) {
+  if (!grp || slots < 1 || slots > 65535) return set_error("woq_linear_grouped: 1..65535 slots and a group table");
+  if (f.M != 1) return set_error("woq_linear_grouped: the single-row kernel takes one row per slot");
+  return launch_decode_impl(f, nullptr, st, grp, (int)slots);
+}
+
+static int launch_decode_impl(const FpArgs& f, const uint32_t* sz, hipStream_t st, const MoeGroup* grp, int slots) {
   DecodeArgs a;
+  a.grp = grp;
   a.x = (const uint16_t*)f.x;
   a.x_dtype = f.x_dtype;
   a.M = f.M; a.K = f.K; a.N = f.N; a.NT = f.NT; a.KT = f.KT;
@@ -429,11 +463,11 @@ int launch_decode(const FpArgs& f, const uint32_t* sz, hipStream_t st) {
     const int64_t waves2 = (f.NT / (two ? 2 : 1)) * ((f.KT + 1) / 2);
     if (waves2 <= 2048 && f.KT % 4 == 0 && f.KT / 4 <= 8) {
       a.W = (int)(f.KT / 4);
-      if (xf16) return two ? launch_decode_m1_cfg<false, 2, 4, true>(a, st) : launch_decode_m1_cfg<false, 1, 4, true>(a, st);
-      return two ? launch_decode_m1_cfg<true, 2, 4, true>(a, st) : launch_decode_m1_cfg<true, 1, 4, true>(a, st);
+      if (xf16) return two ? launch_decode_m1_cfg<false, 2, 4, true>(a, st, slots) : launch_decode_m1_cfg<false, 1, 4, true>(a, st, slots);
+      return two ? launch_decode_m1_cfg<true, 2, 4, true>(a, st, slots) : launch_decode_m1_cfg<true, 1, 4, true>(a, st, slots);
     }
 #define WOQ_DECODE_M1(XB, NTW) \
-  (one_round ? launch_decode_m1_cfg<XB, NTW, 2, true>(a, st) : launch_decode_m1_cfg<XB, NTW, 2, false>(a, st))
+  (one_round ? launch_decode_m1_cfg<XB, NTW, 2, true>(a, st, slots) : launch_decode_m1_cfg<XB, NTW, 2, false>(a, st, slots))
     if (xf16) return two ? WOQ_DECODE_M1(false, 2) : WOQ_DECODE_M1(false, 1);
     return two ? WOQ_DECODE_M1(true, 2) : WOQ_DECODE_M1(true, 1);
 #undef WOQ_DECODE_M1

@@ -50,13 +50,7 @@ struct DecodeDqArgs {
   const MoeGroup* grp;
 };
 
-// a pointer every lane of the wave loaded from the same address, moved to scalar registers
-template <typename T>
-__device__ __forceinline__ T* dq_uniform(T* p) {
-  const uint64_t v = (uint64_t)p;
-  const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
-  return (T*)(((uint64_t)hi << 32) | lo);
-}
+
 
 template <int REGIME>
 __device__ __forceinline__ f4 dq_mfma(u4 a, u4 b, f4 c) {

@@ -16,6 +16,18 @@ int check_launch(const char* what);
 struct Epilogue;
 
 // Arguments common to the floating-point kernels (small-M streaming and tiled GEMM).
+// Device-side description of a grouped launch over the experts of a mixture-of-experts layer (woq_hip_moe_group).
+struct MoeGroup {
+  const int32_t* slot_expert;  // [slots] expert of the slot, or -1: nothing to do
+  const int32_t* slot_row0;    // [slots] first routed row of the slot
+  const int32_t* slot_rows;    // [slots] its number of rows
+  const int64_t* x_row;        // [routed rows] row of x a routed row reads, or null: the routed row itself
+  const void* const* qweight;  // [experts] packed weights
+  const void* const* scales;   // [experts] scales in the regime's dtype
+  const uint8_t* const* zeros; // [experts] or null
+  const float* const* bias;    // [experts] or null
+};
+
 struct FpArgs {
   const void* x;
   int x_dtype;
@@ -34,18 +46,6 @@ struct FpArgs {
   int out_dtype;
   int nf4;  // 4-bit codes index the NF4 table instead of standing for integers (zeros == nullptr)
   int fp8;  // 8-bit weights are float8 e4m3fn bytes, not offset-binary integers (zeros == nullptr)
-};
-
-// Device-side description of a grouped launch over the experts of a mixture-of-experts layer (woq_hip_moe_group).
-struct MoeGroup {
-  const int32_t* slot_expert;  // [slots] expert of the slot, or -1: nothing to do
-  const int32_t* slot_row0;    // [slots] first routed row of the slot
-  const int32_t* slot_rows;    // [slots] its number of rows
-  const int64_t* x_row;        // [routed rows] row of x a routed row reads, or null: the routed row itself
-  const void* const* qweight;  // [experts] packed weights
-  const void* const* scales;   // [experts] scales in the regime's dtype
-  const uint8_t* const* zeros; // [experts] or null
-  const float* const* bias;    // [experts] or null
 };
 
 // Split-K scratch of the dequantizing decode kernel: fp32 partial tiles, and one counter per
@@ -77,8 +77,8 @@ int launch_moe_gather_rows(const void* x, int x_dtype, int64_t T, int64_t H, con
 int launch_moe_scale_add_rows(void* out, int dtype, int64_t T, int64_t H, const void* cur, const void* rw, int64_t topk,
                               const int64_t* top_x, const int64_t* idx, int64_t n, hipStream_t st);
 int launch_moe_route(const int64_t* ids, int64_t T, int64_t topk, int64_t experts, int64_t split_lo, int64_t split_mid,
-                     int64_t* x_row, int32_t* slot_lo, int32_t* slot_mid, int32_t* slot_hi, int32_t* slot_row0,
-                     int32_t* slot_rows, int32_t* row_of, int32_t* slot_of, hipStream_t st);
+                     int use_single, int64_t S, int64_t* x_row, int32_t* slots, int32_t* row_of, int32_t* slot_of,
+                     hipStream_t st);
 int launch_moe_combine_rows(void* out, int dtype, int64_t T, int64_t H, const void* cur, const void* rw, int64_t topk,
                             const int32_t* row_of, const int32_t* slot_of, int accumulate, hipStream_t st);
 int launch_dequant_weight(const void* qweight, int weight_dtype, int64_t N, int64_t K, const float* s32,
@@ -101,9 +101,12 @@ struct DecodeArgs {
   int W;
   int tpg_shift;  // log2(G / 128)
   uint32_t wbytes, szbytes;  // extents of qweight and sz: the single-row kernel addresses them with 32-bit offsets
+  const MoeGroup* grp;       // GROUPED instances of the single-row kernel: one routed row per slot (blockIdx.z)
 };
 bool decode_kernel_applies(const FpArgs& f, int wbits, int regime, const uint32_t* sz);
 int launch_decode(const FpArgs& f, const uint32_t* sz, hipStream_t st);
+// One routed row per slot, the experts' (scale, zero) dword tables in grp->scales.
+int launch_decode_grouped(const FpArgs& f, const MoeGroup* grp, int64_t slots, hipStream_t st);
 
 // fp32 compute (woq_fp32.hip): lowp_mode NONE with fp32 activations; fp32 scales, one-byte zero
 // points, fp32 output.

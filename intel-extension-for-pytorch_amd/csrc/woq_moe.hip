@@ -94,34 +94,35 @@ __global__ void moe_scale_add_rows_kernel(void* __restrict__ out, const void* __
 // (token, slot) entries by expert -- stable, so that inside an expert the tokens ascend, the order of
 // get_expert_topx_idx (csrc/cpu/aten/MoE.cpp:64-81) -- and writes
 //   x_row[p]        token of the entry at sorted position p (the row of the hidden states it reads),
-//   slot_*[p]       a slot per sorted position: the first position of an expert carries the expert's id (in the table
-//                   of its size class: fewer than split_lo rows -> lo, at most split_mid -> mid, else hi; -1 in the
-//                   others) and its row count, every other position -1,
+//   slots           [4 classes][expert, first row, rows][S]: the experts that have tokens, densely from index 0 and in
+//                   ascending expert order, by size class -- 0: fewer than split_lo rows, 1: at most split_mid,
+//                   2: more, 3 (use_single): exactly one row (taken out of class 0) -- unused entries expert -1,
 //   row_of[t, i]    sorted position of token t's i-th contribution in ascending expert order (-1: none),
 //   slot_of[t, i]   its top-k slot.
 // An expert id outside [0, experts) contributes nothing.  R <= kMoeRouteMax entries, compared pairwise from LDS.
 constexpr int kMoeRouteMax = WOQ_HIP_MOE_ROUTE_MAX;
 constexpr int kMoeSlotRowsMax = 64;
 __global__ __launch_bounds__(256) void moe_route_kernel(const int64_t* __restrict__ ids, int R, int topk, int experts,
-                                                        int split_lo, int split_mid, int64_t* __restrict__ x_row,
-                                                        int32_t* __restrict__ slot_lo, int32_t* __restrict__ slot_mid,
-                                                        int32_t* __restrict__ slot_hi,
-                                                        int32_t* __restrict__ slot_row0, int32_t* __restrict__ slot_rows,
+                                                        int split_lo, int split_mid, int use_single, int S,
+                                                        int64_t* __restrict__ x_row, int32_t* __restrict__ slots,
                                                         int32_t* __restrict__ row_of, int32_t* __restrict__ slot_of) {
   __shared__ int se[kMoeRouteMax];
+  __shared__ int8_t cls_of[kMoeRouteMax];  // size class of the expert whose first sorted position this is, or -1
   for (int i = threadIdx.x; i < R; i += blockDim.x) {
     const int64_t e = ids[i];
     se[i] = (e >= 0 && e < experts) ? (int)e : -1;
-    slot_lo[i] = -1;
-    slot_mid[i] = -1;
-    slot_hi[i] = -1;
-    slot_row0[i] = i;
-    slot_rows[i] = 0;
+    cls_of[i] = -1;
     row_of[i] = -1;
     slot_of[i] = 0;
   }
+  for (int i = threadIdx.x; i < 12 * S; i += blockDim.x) slots[i] = (i / S) % 3 == 0 ? -1 : 0;
   __syncthreads();
-  for (int i = threadIdx.x; i < R; i += blockDim.x) {
+  int my_p[kMoeRouteMax / 256], my_e[kMoeRouteMax / 256], my_n[kMoeRouteMax / 256];
+#pragma unroll
+  for (int u = 0; u < kMoeRouteMax / 256; ++u) {
+    my_p[u] = -1;
+    const int i = (int)threadIdx.x + u * 256;
+    if (i >= R) continue;
     const int e = se[i];
     if (e < 0) continue;
     int before = 0, rank = 0, count = 0;
@@ -135,8 +136,11 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const int64_t* __restric
     const int t = i / topk, j = i - t * topk;
     x_row[p] = t;
     if (rank == 0) {
-      (count < split_lo ? slot_lo : count <= split_mid ? slot_mid : slot_hi)[p] = e;
-      slot_rows[p] = count < kMoeSlotRowsMax ? count : kMoeSlotRowsMax;
+      const int cls = (use_single && count == 1) ? 3 : count < split_lo ? 0 : count <= split_mid ? 1 : 2;
+      cls_of[p] = (int8_t)cls;
+      my_p[u] = p;
+      my_e[u] = e;
+      my_n[u] = count < kMoeSlotRowsMax ? count : kMoeSlotRowsMax;
     }
     // a slot holds at most 64 rows (an expert gets more only if a token names it twice): the rest contribute nothing
     if (rank >= kMoeSlotRowsMax) continue;
@@ -147,6 +151,22 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const int64_t* __restric
     }
     row_of[t * topk + ord] = p;
     slot_of[t * topk + ord] = j;
+  }
+  __syncthreads();
+  // dense index of an expert inside its class: the experts of that class at earlier sorted positions
+#pragma unroll
+  for (int u = 0; u < kMoeRouteMax / 256; ++u) {
+    const int p = my_p[u];
+    if (p < 0) continue;
+    const int cls = cls_of[p];
+    int idx = 0;
+    for (int k = 0; k < p; ++k) idx += cls_of[k] == cls ? 1 : 0;
+    if (idx < S) {
+      int32_t* const tab = slots + (size_t)cls * 3 * S;
+      tab[idx] = my_e[u];
+      tab[S + idx] = p;
+      tab[2 * S + idx] = my_n[u];
+    }
   }
   // positions past the valid entries read token 0 (never used: no slot covers them)
   int valid = 0;
@@ -229,13 +249,13 @@ int launch_moe_scale_add_rows(void* out, int dtype, int64_t T, int64_t H, const 
 }
 
 int launch_moe_route(const int64_t* ids, int64_t T, int64_t topk, int64_t experts, int64_t split_lo, int64_t split_mid,
-                     int64_t* x_row, int32_t* slot_lo, int32_t* slot_mid, int32_t* slot_hi, int32_t* slot_row0,
-                     int32_t* slot_rows, int32_t* row_of, int32_t* slot_of, hipStream_t st) {
+                     int use_single, int64_t S, int64_t* x_row, int32_t* slots, int32_t* row_of, int32_t* slot_of,
+                     hipStream_t st) {
   const int64_t R = T * topk;
   if (R == 0) return 0;
   if (R > kMoeRouteMax) return set_error("moe_route: at most %d (token, slot) entries, got %lld", kMoeRouteMax, (long long)R);
-  moe_route_kernel<<<1, 256, 0, st>>>(ids, (int)R, (int)topk, (int)experts, (int)split_lo, (int)split_mid, x_row, slot_lo,
-                                       slot_mid, slot_hi, slot_row0, slot_rows, row_of, slot_of);
+  moe_route_kernel<<<1, 256, 0, st>>>(ids, (int)R, (int)topk, (int)experts, (int)split_lo, (int)split_mid, use_single, (int)S,
+                                       x_row, slots, row_of, slot_of);
   return check_launch("moe_route");
 }
 

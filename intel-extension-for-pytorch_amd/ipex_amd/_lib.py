@@ -154,7 +154,7 @@ def load():
         lib.woq_hip_probe_empty.restype = i32
         lib.woq_hip_probe_empty.argtypes = [i64, i32, vp]
         lib.woq_hip_moe_route.restype = i32
-        lib.woq_hip_moe_route.argtypes = [vp, i64, i64, i64, i64, i64, vp, vp, vp, vp, vp, vp, vp, vp, vp]
+        lib.woq_hip_moe_route.argtypes = [vp, i64, i64, i64, i64, i64, i32, i64, vp, vp, vp, vp, vp]
         lib.woq_hip_linear_grouped.restype = i32
         lib.woq_hip_linear_grouped.argtypes = [ctypes.POINTER(LinearParams), vp, i64]
         lib.woq_hip_moe_combine_rows.restype = i32

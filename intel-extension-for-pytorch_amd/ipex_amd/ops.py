@@ -661,13 +661,13 @@ _MOE_PLAN_LIMIT = 128
 
 def _context_pointers(ctx):
     """[qweight, fp16 scales, bf16 scales, zero points or 0, fp32 bias or 0, N, K, group size, weight dtype,
-    lowp_mode, has g_idx, device index] of a context of either binding."""
+    lowp_mode, has g_idx, device index, (scale, zero) dword table or 0] of a context of either binding."""
     if _is_python_context(ctx):
         ptr = lambda t: 0 if t is None else t.data_ptr()
         N, K = ctx.weight_shape_
         return [ctx.at_weight_.data_ptr(), ctx.scales_list_[1].data_ptr(), ctx.scales_list_[2].data_ptr(),
                 ptr(ctx.zeros_u8_), ptr(ctx.bias_f32_), N, K, ctx.group_size_, ctx.weight_dtype_, ctx.lowp_mode_,
-                0 if ctx.g_idx_ is None else 1, ctx.at_weight_.device.index]
+                0 if ctx.g_idx_ is None else 1, ctx.at_weight_.device.index, ptr(ctx.scale_zero_f16x2_)]
     return list(ctx.kernel_pointers())
 
 
@@ -685,7 +685,7 @@ class _MoeGroupedPlan:
         for rows in infos:
             first = rows[0]
             same = all(r[5:11] == first[5:11] and (r[3] == 0) == (first[3] == 0) and (r[4] == 0) == (first[4] == 0)
-                       and r[11] == device.index for r in rows)
+                       and (r[12] == 0) == (first[12] == 0) and r[11] == device.index for r in rows)
             if not same or first[10] or first[8] not in (_lib.DTYPE_INT4, _lib.DTYPE_INT8) or first[9] not in (0, 1, 2):
                 return
             self.shapes.append(dict(N=first[5], K=first[6], G=first[7], wd=first[8], lowp=first[9]))
@@ -697,13 +697,20 @@ class _MoeGroupedPlan:
         R = _lib.MOE_ROUTE_MAX
         i32 = lambda: torch.empty(R, dtype=torch.int32, device=device)
         self.x_row = torch.empty(R, dtype=torch.int64, device=device)
-        self.slots = [i32(), i32(), i32()]  # experts with few / up to 16 / up to 64 rows
-        self.slot_row0, self.slot_rows, self.row_of, self.slot_of = (i32() for _ in range(4))
+        # slot tables [class][expert, first row, rows][S]: experts with few / up to 16 / up to 64 rows / exactly one row
+        self.S = len(gate_ctx)
+        self.slots = torch.empty((4, 3, self.S), dtype=torch.int32, device=device)
+        self.row_of, self.slot_of = i32(), i32()
         self.tables = []
         for rows in infos:
             col = lambda k: torch.tensor([r[k] for r in rows], dtype=torch.int64, device=device)
             self.tables.append(dict(qweight=col(0), s16=col(1), sb16=col(2), z8=col(3) if rows[0][3] else None,
-                                    bias=col(4) if rows[0][4] else None))
+                                    bias=col(4) if rows[0][4] else None, sz=col(12) if rows[0][12] else None))
+        # the single-row decode kernel serves the experts with fewer than five rows where all three linears have its
+        # (scale, zero) tables: 4-bit weights in groups of 128 x 2^k, K a multiple of 256
+        self.single_row = all(t["sz"] is not None for t in self.tables) and all(
+            x["wd"] == _lib.DTYPE_INT4 and x["K"] % 256 == 0 and x["G"] % 128 == 0 and (x["G"] // 128) & (x["G"] // 128 - 1) == 0
+            for x in self.shapes)
         self.structs = {}
         self.rows = {}  # dtype -> (act, inter, y) for the most routed rows seen
         self.device = device
@@ -718,15 +725,18 @@ class _MoeGroupedPlan:
         return have
 
     def group_struct(self, linear, cls, f16_scales, gather):
-        """Device copy of the woq_hip_moe_group of one launch (built once)."""
+        """Device copy of the woq_hip_moe_group of one launch (built once).  Class 3: one slot per row, with the
+        (scale, zero) dword tables in place of the scales."""
         key = (linear, cls, f16_scales, gather)
         st = self.structs.get(key)
         if st is None:
             t = self.tables[linear]
             ptr = lambda x: 0 if x is None else x.data_ptr()
-            fields = [ptr(self.slots[cls]), ptr(self.slot_row0), ptr(self.slot_rows),
-                      ptr(self.x_row) if gather else 0, ptr(t["qweight"]), ptr(t["s16"] if f16_scales else t["sb16"]),
-                      ptr(t["z8"]), ptr(t["bias"])]
+            tab = [ptr(self.slots[cls, i]) for i in range(3)] + [ptr(self.x_row) if gather else 0]
+            if cls == 3:
+                fields = tab + [ptr(t["qweight"]), ptr(t["sz"]), 0, ptr(t["bias"])]
+            else:
+                fields = tab + [ptr(t["qweight"]), ptr(t["s16"] if f16_scales else t["sb16"]), ptr(t["z8"]), ptr(t["bias"])]
             st = torch.tensor(fields, dtype=torch.int64, device=self.device)
             self.structs[key] = st
         return st
@@ -748,7 +758,7 @@ def _f16_regime(lowp, x_dtype, rows):
 
 
 def _deepseek_moe_grouped(hidden_states, topk_ids, gate_ctx, up_ctx, down_ctx, routing_weights):
-    """The layer in five to eleven launches and without reading the routing on the host: the routing is sorted on the
+    """The layer in five to fourteen launches and without reading the routing on the host: the routing is sorted on the
     device, every linear runs once per compute type over all experts that have tokens (woq_hip_linear_grouped), and
     the contributions of a token are added in ascending expert order.  Returns None when the layer does not fit
     (more than 64 tokens, mixed experts, act-order, NF4 / FP8 / lowp INT8 ...): the caller then takes the per-expert path."""
@@ -769,7 +779,10 @@ def _deepseek_moe_grouped(hidden_states, topk_ids, gate_ctx, up_ctx, down_ctx, r
     lowp = plan.shapes[0]["lowp"]
     split = 5 if lowp == 2 else 0  # lowp_mode BF16: experts with fewer than five rows compute in fp16
     # (size class, bound on its slots' rows): an expert has at most T rows, so the larger classes are empty for small T
-    launches = ([(0, 4)] if split else []) + ([(1, 16)] if T >= split else []) + ([(2, 64)] if T > 16 else [])
+    # experts with exactly one row (most of them in a layer with many experts and few tokens) on the single-row kernel
+    single = bool(split) and plan.single_row
+    launches = ([(3, 1)] if single else []) + ([(0, 4)] if split and (T > 1 or not single) else []) + \
+               ([(1, 16)] if T >= split else []) + ([(2, 64)] if T > 16 else [])
     for cls, bound in launches:
         f16 = _f16_regime(lowp, x.dtype, bound)
         # rows must be in the compute type; bf16 rows under fp16 compute are converted for up to 16 rows per slot
@@ -787,10 +800,10 @@ def _deepseek_moe_grouped(hidden_states, topk_ids, gate_ctx, up_ctx, down_ctx, r
     code = _kernels._ACT_CODE[x.dtype]
     with torch.cuda.device(x.device):
         stream = _kernels._stream()
-        _lib.check(lib.woq_hip_moe_route(ids.data_ptr(), T, topk, len(gate_ctx), split, 16, plan.x_row.data_ptr(),
-                                         plan.slots[0].data_ptr(), plan.slots[1].data_ptr(), plan.slots[2].data_ptr(),
-                                         plan.slot_row0.data_ptr(), plan.slot_rows.data_ptr(), plan.row_of.data_ptr(),
+        _lib.check(lib.woq_hip_moe_route(ids.data_ptr(), T, topk, len(gate_ctx), split, 16, int(single), plan.S,
+                                         plan.x_row.data_ptr(), plan.slots.data_ptr(), plan.row_of.data_ptr(),
                                          plan.slot_of.data_ptr(), stream), "moe_route")
+        nslots = min(R, plan.S)  # experts that can have tokens: the tables are dense
         p = _lib.LinearParams()
         p.struct_size = ctypes.sizeof(_lib.LinearParams)
         p.x_dtype = p.out_dtype = code
@@ -806,8 +819,10 @@ def _deepseek_moe_grouped(hidden_states, topk_ids, gate_ctx, up_ctx, down_ctx, r
             p.others[0] = other.data_ptr() if other is not None else None
             for cls, bound in launches:
                 p.M = bound
+                # (a non-null value tells the entry point that the group's scales are (scale, zero) dword tables)
+                p.scale_zero_f16x2 = plan.tables[li]["sz"].data_ptr() if cls == 3 else None
                 g = plan.group_struct(li, cls, _f16_regime(lowp, x.dtype, bound), gather)
-                _lib.check(lib.woq_hip_linear_grouped(ctypes.byref(p), g.data_ptr(), R), "woq_linear_grouped")
+                _lib.check(lib.woq_hip_linear_grouped(ctypes.byref(p), g.data_ptr(), nslots), "woq_linear_grouped")
         _lib.check(lib.woq_hip_moe_combine_rows(out.data_ptr(), code, T, H, y.data_ptr(), rw.data_ptr(), topk,
                                                 plan.row_of.data_ptr(), plan.slot_of.data_ptr(), 0, stream), "moe_combine_rows")
     return out

@@ -582,30 +582,35 @@ def test_moe_route_against_the_oracle_token_lists(cuda):
         R = T * topk
         dev = ids.to(cuda)
         x_row = torch.full((R,), -7, dtype=torch.int64, device=cuda)
-        lo, mid, hi, row0, rows, row_of, slot_of = (torch.full((R,), -7, dtype=torch.int32, device=cuda) for _ in range(7))
-        rc = lib.woq_hip_moe_route(dev.data_ptr(), T, topk, E, split, 16, x_row.data_ptr(), lo.data_ptr(), mid.data_ptr(),
-                                   hi.data_ptr(), row0.data_ptr(), rows.data_ptr(), row_of.data_ptr(), slot_of.data_ptr(), None)
+        row_of, slot_of = (torch.full((R,), -7, dtype=torch.int32, device=cuda) for _ in range(2))
+        single = split > 1 and T != 33
+        S = min(R, E) + (T == 16)  # also tables longer than needed
+        slots = torch.full((4, 3, S), -7, dtype=torch.int32, device=cuda)
+        assert lib.woq_hip_moe_route(dev.data_ptr(), T, topk, E, split, 16, int(single), min(R, E) - 1, x_row.data_ptr(),
+                                     slots.data_ptr(), row_of.data_ptr(), slot_of.data_ptr(), None) != 0  # tables too short
+        rc = lib.woq_hip_moe_route(dev.data_ptr(), T, topk, E, split, 16, int(single), S, x_row.data_ptr(),
+                                   slots.data_ptr(), row_of.data_ptr(), slot_of.data_ptr(), None)
         assert rc == 0, lib.woq_hip_last_error()
         torch.cuda.synchronize()
         valid = (ids >= 0) & (ids < E)
         top_x, idx = O.expert_token_lists(torch.where(valid, ids, torch.full_like(ids, E)).numpy(), E + 1)
-        pos, want_row, want_lo, want_mid, want_hi, want_rows = 0, [], {}, {}, {}, {}
+        pos, want_row, want = 0, [], [[], [], [], []]  # per class: (expert, first sorted position, rows)
         entry_pos = {}
         for e in range(E):
             n = len(top_x[e])
             if n:
-                (want_lo if n < split else want_mid if n <= 16 else want_hi)[pos] = e
-                want_rows[pos] = n
+                cls = 3 if single and n == 1 else 0 if n < split else 1 if n <= 16 else 2
+                want[cls].append((e, pos, min(n, 64)))
             for t, j in zip(top_x[e], idx[e]):
                 entry_pos[(int(t), int(j))] = pos
                 want_row.append(int(t))
                 pos += 1
         assert x_row.cpu().tolist()[:pos] == want_row
-        assert row0.cpu().tolist() == list(range(R))
-        lo_c, mid_c, hi_c, rows_c = lo.cpu().tolist(), mid.cpu().tolist(), hi.cpu().tolist(), rows.cpu().tolist()
-        for p in range(R):
-            assert lo_c[p] == want_lo.get(p, -1) and mid_c[p] == want_mid.get(p, -1) and hi_c[p] == want_hi.get(p, -1), (T, p)
-            assert rows_c[p] == want_rows.get(p, 0)
+        got = slots.cpu()
+        for cls in range(4):
+            n = len(want[cls])
+            assert [tuple(int(got[cls, i, k]) for i in range(3)) for k in range(n)] == want[cls], (T, cls)
+            assert got[cls, 0, n:].eq(-1).all(), (T, cls)
         ro, so = row_of.cpu().view(T, topk), slot_of.cpu().view(T, topk)
         for t in range(T):
             order = sorted((int(ids[t, j]), j) for j in range(topk) if bool(valid[t, j]))
@@ -624,11 +629,13 @@ def test_moe_route_keeps_at_most_64_rows_of_an_expert(cuda):
     ids = torch.stack([torch.tensor([2, 3 if t % 2 else 4]) for t in range(T)])  # expert 2 gets all 80 tokens
     R = T * topk
     x_row = torch.empty(R, dtype=torch.int64, device=cuda)
-    lo, mid, hi, row0, rows, row_of, slot_of = (torch.empty(R, dtype=torch.int32, device=cuda) for _ in range(7))
-    rc = lib.woq_hip_moe_route(ids.to(cuda).data_ptr(), T, topk, E, 5, 16, x_row.data_ptr(), lo.data_ptr(), mid.data_ptr(), hi.data_ptr(),
-                               row0.data_ptr(), rows.data_ptr(), row_of.data_ptr(), slot_of.data_ptr(), None)
+    row_of, slot_of = (torch.empty(R, dtype=torch.int32, device=cuda) for _ in range(2))
+    slots = torch.empty((4, 3, E), dtype=torch.int32, device=cuda)
+    rc = lib.woq_hip_moe_route(ids.to(cuda).data_ptr(), T, topk, E, 5, 16, 1, E, x_row.data_ptr(), slots.data_ptr(),
+                               row_of.data_ptr(), slot_of.data_ptr(), None)
     assert rc == 0, lib.woq_hip_last_error()
-    assert int(hi[0]) == 2 and int(rows[0]) == 64 and x_row[:80].cpu().tolist() == list(range(80))
+    assert slots[2, :, 0].cpu().tolist() == [2, 0, 64] and x_row[:80].cpu().tolist() == list(range(80))
+    assert slots[2, 0, 1:].cpu().tolist() == [3, 4, -1, -1] and slots[2, 1, 1:3].cpu().tolist() == [80, 120]
     ro = row_of.cpu().view(T, topk)
     assert ro[:64, 0].tolist() == list(range(64)) and bool((ro[64:, 0] == -1).all())
     assert bool((ro[:, 1] >= 80).all())  # the other contribution of every token is kept
@@ -684,11 +691,12 @@ def test_moe_combine_rows_bit_exact(cuda, dtype, accumulate):
     ids = torch.stack([torch.randperm(E, generator=g)[:topk] for _ in range(T)])
     ids[2, 3] = -1
     R = T * topk
-    bufs = [torch.empty(R, dtype=torch.int32, device=cuda) for _ in range(7)]
+    row_of, slot_of = (torch.empty(R, dtype=torch.int32, device=cuda) for _ in range(2))
+    slots = torch.empty((4, 3, E), dtype=torch.int32, device=cuda)
     x_row = torch.empty(R, dtype=torch.int64, device=cuda)
-    rc = lib.woq_hip_moe_route(ids.to(cuda).data_ptr(), T, topk, E, 5, 16, x_row.data_ptr(), *[b.data_ptr() for b in bufs], None)
+    rc = lib.woq_hip_moe_route(ids.to(cuda).data_ptr(), T, topk, E, 5, 16, 0, E, x_row.data_ptr(), slots.data_ptr(),
+                               row_of.data_ptr(), slot_of.data_ptr(), None)
     assert rc == 0, lib.woq_hip_last_error()
-    row_of, slot_of = bufs[5], bufs[6]
     expert_out = torch.randn(R, H, generator=g).to(dtype)
     rw = torch.rand(T, topk, generator=g).to(dtype)
     out0 = torch.randn(T, H, generator=g).to(dtype)
