@@ -451,8 +451,10 @@ def run_probe(name, torch, lib, lib_mod, ops_mod, synthetic, dev, stream):
         K, N, G, Mp = 4096, 14336, 128, 2048
         case = synthetic.make_int4_case(3, Mp, K, N, G, outliers=True)
         info["launches"] = []
-        for lowp, aq in ((2, -1), (3, 6)):
+        # (third: lowp_mode BF16 on the kernel that dequantizes once per workgroup into LDS)
+        for lowp, aq, forced in ((2, -1, 0), (3, 6, 0), (2, -1, 21)):
             params, keep = _rotating_params(torch, lib_mod, ops_mod, case, lowp, dev, stream, min_bytes=1, act_quant_mode=aq)
+            params[0].force_kernel = forced
             for _ in range(20):
                 assert lib.woq_hip_linear(ctypes.byref(params[0])) == 0, lib.woq_hip_last_error()
             torch.cuda.synchronize()
@@ -744,13 +746,15 @@ def main():
         pre = {}
         # its own fixed counts, whatever --steps says: 60 warm-up launches, then five regions of 40
         warm_p, steps_p, groups_p = 60, 40, 5
-        for name, lowp, aq in (("bf16", 2, -1), ("int8", 3, 6)):
+        # (bf16_lds_tile: the same problem on the kernel that dequantizes once per workgroup into LDS, force_kernel 21)
+        for name, lowp, aq, forced in (("bf16", 2, -1, 0), ("int8", 3, 6, 0), ("bf16_lds_tile", 2, -1, 21)):
             ws = None
             wbytes = lib.woq_hip_linear_workspace_bytes(Mp, K, lowp, aq, G)
             if wbytes:
                 ws = torch.empty(wbytes, dtype=torch.uint8, device=dev)
             pp = build_params(_lib, xp, keep[0], outp, lowp, aq, ws)
             pp.stream = stream.cuda_stream
+            pp.force_kernel = forced
             time_steps(torch, lib, [pp], 1, warm_p, stream)
             _, ms = time_groups(torch, lib, [pp], steps_p, stream, groups=groups_p)
             us = ms * 1e3 / steps_p
@@ -781,6 +785,7 @@ def main():
             "flops_per_step": flops,
             "lowp_bf16": pre["bf16"],
             "lowp_int8_per_row": pre["int8"],
+            "lowp_bf16_dequantized_tile_in_lds": pre["bf16_lds_tile"],
             "dense_bf16_vendor_gemm_same_shape": {"us_per_step": round(us_d, 2),
                                                   "tflops": round(flops / (us_d * 1e-6) / 1e12, 1)},
             "frac_of_bf16_mfma_peak": round(pre["bf16"]["tflops"] / MFMA_BF16_PEAK_TFLOPS, 4),

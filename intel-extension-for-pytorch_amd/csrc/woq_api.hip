@@ -293,6 +293,12 @@ int woq_hip_linear(const woq_hip_linear_params* p) {
       kernel = w4 ? 3 : 2;
   }
   if (kernel == 1 && p->M > 64) return set_error("woq_linear: the small-M kernel takes M <= 64");
+  if (kernel == 21) {
+    if (!gemm_w4s_applies(f, wbits, regime))
+      return set_error("woq_linear: the prefill kernel with the dequantized tile in LDS takes 4-bit integer weights, "
+                       "K %% 128 == 0, a power-of-two or per-channel group size and activations in the compute dtype");
+    return launch_gemm_w4s(f, regime, st);
+  }
   const int w4_shape = kernel == 4 ? 7 : kernel == 5 ? 4 : kernel == 6 ? 2 : kernel == 11 ? 163
                        : (kernel == 12 || kernel == 19 || kernel == 20) ? 42 : 0;
   // forced shapes run unsplit, 19 / 20 split K in two / four; the automatic choice may split

@@ -116,7 +116,10 @@ __global__ __launch_bounds__(256) void woq_gemm_w4_kernel(const FpArgs f, const 
   for (int i = 0; i < G4_XLOADS; ++i) {
     const int rowl = (wave * G4_XLOADS + i) * 4 + c;
     const int rowc = m0 + rowl < M ? rowl : M - 1 - m0;
-    const int chunk = r ^ (rowl & 15);
+    // (4-bit weights: the chunk 4 c + j of lane column c and sub-step j is kept at slot 4 j + c, so that the four
+    // lane columns of a row read slots that differ in their low bits: chunks 8 apart share their banks)
+    const int slot = r ^ (rowl & 15);
+    const int chunk = WBITS == 4 ? ((slot & 3) << 2) | (slot >> 2) : slot;
     xoff[i] = (uint32_t)(rowc * K + chunk * 8) * 2u;
   }
   // All global addresses are a wave-uniform 64-bit base plus a 32-bit per-lane byte offset that
@@ -135,8 +138,8 @@ __global__ __launch_bounds__(256) void woq_gemm_w4_kernel(const FpArgs f, const 
   uint32_t rd[4];
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
-    const int chunk = WBITS == 4 ? c * 4 + j : 8 * (j / 2) + 2 * c + (j % 2);
-    rd[j] = (uint32_t)(r * 256 + ((chunk ^ r) << 4));
+    const int slot = WBITS == 4 ? j * 4 + c : 8 * (j / 2) + 2 * c + (j % 2);
+    rd[j] = (uint32_t)(r * 256 + ((slot ^ r) << 4));
   }
 
   // ---- weights of one K tile: one dwordx4 + one (scale, zero) per row-block and lane.  Symmetric

@@ -148,6 +148,8 @@ bool gemm_w4_applies(const FpArgs& f, int wbits, int regime);
 // 64 x 128 tiles, 0 = by cost model; 8-bit weights: 4, 2, 42 or 0
 // splits: workgroups that share the K steps of a tile (64 x 128 shape only; 2 or 4 need the scratch),
 // 0 = by problem size, 1 = none
+bool gemm_w4s_applies(const FpArgs& f, int wbits, int regime);
+int launch_gemm_w4s(const FpArgs& f, int regime, hipStream_t st);
 int launch_gemm_w4(const FpArgs& f, int wbits, int regime, hipStream_t st, int shape = 0, int splits = 0,
                    const SplitKScratch* scratch = nullptr);
 

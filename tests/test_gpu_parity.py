@@ -246,7 +246,7 @@ def test_both_kernels_agree_on_mid_m(cuda, M):
         (150, 256, 450, 128, True),  # N not a multiple of 8: element-wise stores
     ],
 )
-@pytest.mark.parametrize("shape", [3, 4, 5, 6, 11, 12])  # cost model, then 448 / 256 / 128 columns per workgroup, then 256 rows x 192, 64 x 128
+@pytest.mark.parametrize("shape", [3, 4, 5, 6, 11, 12, 21])  # cost model, then 448 / 256 / 128 columns per workgroup, then 256 rows x 192, 64 x 128, then the kernel with the dequantized tile in LDS
 def test_w4_prefill_kernel(cuda, M, K, N, G, bias, shape):
     case = _synthetic().make_int4_case(20, M, K, N, G, bias=bias)
     _check_fp(case, O.LOWP_BF16, force_kernel=shape, label=f"w4 prefill M={M} K={K} N={N} G={G} kernel={shape}")
@@ -362,6 +362,51 @@ def test_w4_prefill_kernel_rejects_other_shapes(cuda):
     ctx = make_context(case, O.LOWP_BF16)
     with pytest.raises(RuntimeError, match="prefill kernel takes"):
         ctx.run(case["x"].cuda(), force_kernel=3)
+    with pytest.raises(RuntimeError, match="dequantized tile in LDS takes"):
+        ctx.run(case["x"].cuda(), force_kernel=21)
+    int8 = _synthetic().make_int8_case(24, 70, 256, 64, 128)
+    with pytest.raises(RuntimeError, match="dequantized tile in LDS takes"):
+        make_context(int8, O.LOWP_BF16).run(int8["x"].cuda(), force_kernel=21)
+
+
+def test_w4_prefill_kernel_with_the_tile_in_lds(cuda):
+    """force_kernel 21 (256 x 224 workgroup tiles, weights dequantized once per workgroup into LDS): symmetric
+    weights, the fp16 regime, post-ops through the staging tile, and agreement with the register-resident kernel
+    (another order of the fp32 sums: the K values of an MFMA are grouped differently)."""
+    from ipex_amd import _lib
+
+    syn = _synthetic()
+    case = syn.make_int4_case(21, 260, 512, 464, 128, bias=True)
+    case["zeros"] = None
+    _check_fp(case, O.LOWP_BF16, force_kernel=21, label="w4 prefill with the tile in LDS, symmetric")
+    ctx = make_context(case, O.LOWP_BF16)
+    x = case["x"].cuda()
+    a, b = to_np_f32(ctx.run(x, force_kernel=21)), to_np_f32(ctx.run(x, force_kernel=3))
+    assert bool(np.all((bf16_ulp_diff(a, b) <= 1) | (np.abs(a - b) <= 1e-4)))
+    assert torch.equal(ctx.run(x, force_kernel=21), ctx.run(x, force_kernel=21))
+    # post-ops and an fp32 output go through the per-wave staging tile
+    other = torch.randn(260, 464, generator=torch.Generator().manual_seed(4)).bfloat16().cuda()
+    base = ctx.run(x, out_fp32=True, force_kernel=21)
+    assert max_abs(base.cpu().numpy(), ctx.run(x, out_fp32=True, force_kernel=3).cpu().numpy()) <= MAX_ABS_ACC
+    y = ctx.run(x, force_kernel=21)
+    assert torch.equal(ctx.run(x, fusion=_lib.FUSE_ADD, others=(other,), force_kernel=21), (y.float() + other.float()).bfloat16())
+    assert torch.equal(ctx.run(x, fusion=_lib.FUSE_RELU, force_kernel=21), torch.relu(y))
+    # fp16 regime
+    M, K, N, G = 140, 512, 464, 128
+    case = syn.make_int4_case(22, M, K, N, G, bias=True, scale_dtype=torch.float16)
+    case["x"] = case["x"].to(torch.float16)
+    ctx = make_context(case, O.LOWP_FP16)
+    x = case["x"].cuda()
+    y = to_np_f32(ctx.run(x, force_kernel=21))
+    acc = ctx.run(x, out_fp32=True, force_kernel=21).cpu().numpy()
+    c = case_np(case)
+    acc_ref, y_ref = O.woq_linear_ref(c["x"], "fp16", c["qw"], N, K, c["scales"], c["zps"], c["bias"], 2, G, "fp16")
+    assert max_abs(acc, acc_ref) <= MAX_ABS_ACC
+    assert rel_l2(y, y_ref) <= REL_L2_OUT
+    # groups of 32 (two groups inside a lane's K step) and per-channel scales, K = 128 (two K steps)
+    for G2, K2 in ((32, 384), (-1, 128)):
+        _check_fp(syn.make_int4_case(25, 257, K2, 240, G2, bias=False), O.LOWP_BF16, force_kernel=21,
+                  label=f"w4 prefill with the tile in LDS, G={G2} K={K2}")
 
 
 @pytest.mark.parametrize(
