@@ -524,17 +524,18 @@ def floor_probe(torch, lib, dev, stream, groups=9, per_group=200):
 
 def mfma_issue_probe(torch, lib, dev, stream, iters=1500, repeats=5):
     """What bounds the prefill GEMM's K loop, measured without it: 256 workgroups of four waves (one wave per
-    SIMD on every CU), each wave issuing `iters` x 16 independent v_mfma_f32_16x16x32_bf16 on random bf16
+    SIMD on every CU; some mixes again with eight, two per SIMD), each wave issuing `iters` x 16 independent v_mfma_f32_16x16x32_bf16 on random bf16
     operands with V fp32 FMAs and L ds_read_b128 per 16 MFMAs spread between them.  Per mix: microseconds per
     launch (median of `repeats`), nanoseconds per MFMA and wave, and the TFLOP/s of the whole chip.  The
     prefill kernel's loop issues 40 VALU and 2.8 LDS reads per 16 MFMAs."""
     src = torch.randn(3 * 256 * 8, device=dev).to(torch.bfloat16)  # 12 KiB: LDS tile, A and B fragments
     st = ctypes.c_void_p(stream.cuda_stream)
     rows = []
-    for valu, lds in ((0, 0), (16, 0), (32, 0), (40, 0), (48, 0), (64, 0), (0, 3), (0, 8), (0, 16), (32, 3), (40, 3),
-                      (48, 3), (20, 6)):
+    one = [(0, 0), (16, 0), (32, 0), (40, 0), (48, 0), (64, 0), (0, 3), (0, 8), (0, 16), (32, 3), (40, 3), (48, 3), (20, 6)]
+    two = [(0, 0), (40, 0), (40, 3), (48, 3), (20, 6)]
+    for waves, valu, lds in [(4, v, l) for v, l in one] + [(8, v, l) for v, l in two]:
         def launch():
-            rc = lib.woq_hip_probe_mfma_issue(ctypes.c_void_p(src.data_ptr()), valu, lds, 256, iters, None, st)
+            rc = lib.woq_hip_probe_mfma_issue(ctypes.c_void_p(src.data_ptr()), valu, lds, 256, waves, iters, None, st)
             assert rc == 0, lib.woq_hip_last_error()
 
         launch()
@@ -549,11 +550,11 @@ def mfma_issue_probe(torch, lib, dev, stream, iters=1500, repeats=5):
             vals.append(e0.elapsed_time(e1) * 1e3)
         us = sorted(vals)[len(vals) // 2]
         mfmas = iters * 16
-        rows.append({"valu_per_16_mfma": valu, "lds_reads_per_16_mfma": lds, "us_per_launch": round(us, 1),
-                     "ns_per_mfma_and_wave": round(us * 1e3 / mfmas, 2),
-                     "tflops": round(256 * 4 * mfmas * 16384 / us / 1e6, 1),
-                     "frac_of_bf16_mfma_peak": round(256 * 4 * mfmas * 16384 / us / 1e6 / MFMA_BF16_PEAK_TFLOPS, 3)})
-    return {"workgroups": 256, "waves_per_workgroup": 4, "mfma_per_wave": iters * 16, "mixes": rows}
+        rows.append({"waves_per_workgroup": waves, "valu_per_16_mfma": valu, "lds_reads_per_16_mfma": lds,
+                     "us_per_launch": round(us, 1), "ns_per_mfma_and_wave": round(us * 1e3 / mfmas, 2),
+                     "tflops": round(256 * waves * mfmas * 16384 / us / 1e6, 1),
+                     "frac_of_bf16_mfma_peak": round(256 * waves * mfmas * 16384 / us / 1e6 / MFMA_BF16_PEAK_TFLOPS, 3)})
+    return {"workgroups": 256, "mfma_per_wave": iters * 16, "mixes": rows}
 
 
 def main():

@@ -376,13 +376,13 @@ int woq_hip_moe_combine_rows(void* out, int dtype, int64_t T, int64_t H, const v
 int woq_hip_probe_stream_read(const void* src, int64_t bytes, int waves_per_wg, int kib_per_wave, void* sink,
                               void* stream);
 int woq_hip_probe_empty(int64_t workgroups, int waves_per_wg, void* stream);
-/*   probe_mfma_issue:  the matrix-instruction rate of one wave per SIMD that also issues other work: each of the
- *                      4 waves of a workgroup runs `iters` rounds of 16 independent v_mfma_f32_16x16x32_bf16 with
+/*   probe_mfma_issue:  the matrix-instruction rate of waves that also issue other work: each of the 4 or 8 waves
+ *                      of a workgroup (one or two per SIMD) runs `iters` rounds of 16 independent v_mfma_f32_16x16x32_bf16 with
  *                      `valu_per_16` fp32 FMAs and `lds_per_16` ds_read_b128 spread between them (instances:
  *                      (0,0) (16,0) (32,0) (40,0) (48,0) (64,0) (0,3) (0,8) (0,16) (32,3) (40,3) (48,3) (20,6));
- *                      src: 12 KiB of operand bytes; sink: NULL or workgroups * 256 floats. */
-int woq_hip_probe_mfma_issue(const void* src, int valu_per_16, int lds_per_16, int64_t workgroups, int iters,
-                             float* sink, void* stream);
+ *                      src: 12 KiB of operand bytes; sink: NULL or one float per thread. */
+int woq_hip_probe_mfma_issue(const void* src, int valu_per_16, int lds_per_16, int64_t workgroups,
+                             int waves_per_workgroup, int iters, float* sink, void* stream);
 
 #ifdef __cplusplus
 }

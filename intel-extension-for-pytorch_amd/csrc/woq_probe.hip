@@ -30,21 +30,23 @@ __global__ __launch_bounds__(1024) void probe_empty_kernel() {}
 // of 16 independent v_mfma_f32_16x16x32_bf16 (sixteen accumulator tiles, operands loaded once from src), with
 // VALU fp32 FMAs on eight independent registers and LDS ds_read_b128 spread evenly between them -- VALU16 and
 // LDS16 per sixteen MFMAs.  One wave per SIMD (four waves per workgroup, one workgroup per CU when the grid is
-// the CU count).  The prefill GEMM's K loop issues 2.5 VALU and 0.17 LDS reads per MFMA.
+// the CU count) or two (eight waves: the other wave's instructions then run under this one's MFMAs).  The prefill
+// GEMM's K loop issues 2.5 VALU and 0.17 LDS reads per MFMA.
 template <int VALU16, int LDS16>
-__global__ __launch_bounds__(256) void probe_mfma_issue_kernel(const u4* __restrict__ src, int iters, float* sink) {
+__global__ __launch_bounds__(512) void probe_mfma_issue_kernel(const u4* __restrict__ src, int iters, float* sink) {
   __shared__ u4 lds[256];
-  lds[threadIdx.x] = src[threadIdx.x];
+  const uint32_t tid = threadIdx.x & 255u;
+  if (threadIdx.x < 256) lds[tid] = src[tid];
   __syncthreads();
   f4 acc[16];
 #pragma unroll
   for (int i = 0; i < 16; ++i) acc[i] = f4{0.f, 0.f, 0.f, 0.f};
-  const u4 a = src[256 + threadIdx.x], b = src[512 + threadIdx.x];
+  const u4 a = src[256 + tid], b = src[512 + tid];
   float v[8];
 #pragma unroll
-  for (int i = 0; i < 8; ++i) v[i] = 1.0f + 0.001f * (float)((threadIdx.x + i) & 7);
+  for (int i = 0; i < 8; ++i) v[i] = 1.0f + 0.001f * (float)((tid + i) & 7);
   u4 l[4] = {a, a, a, a};
-  const uint32_t la = threadIdx.x * 16u;
+  const uint32_t la = tid * 16u;
 #pragma unroll 1
   for (int it = 0; it < iters; ++it) {
 #pragma unroll
@@ -67,7 +69,7 @@ __global__ __launch_bounds__(256) void probe_mfma_issue_kernel(const u4* __restr
   for (int i = 0; i < 8; ++i) s += v[i];
 #pragma unroll
   for (int i = 0; i < 4; ++i) s += bitcast<float>(l[i][0]);
-  if (sink) sink[(size_t)blockIdx.x * 256 + threadIdx.x] = s;
+  if (sink) sink[(size_t)blockIdx.x * blockDim.x + threadIdx.x] = s;
 }
 
 }  // namespace woq
@@ -106,16 +108,18 @@ int woq_hip_probe_empty(int64_t workgroups, int waves_per_wg, void* stream) {
   return check_launch("probe_empty_kernel");
 }
 
-int woq_hip_probe_mfma_issue(const void* src, int valu_per_16, int lds_per_16, int64_t workgroups, int iters,
-                             float* sink, void* stream) {
+int woq_hip_probe_mfma_issue(const void* src, int valu_per_16, int lds_per_16, int64_t workgroups,
+                             int waves_per_workgroup, int iters, float* sink, void* stream) {
   if (!src) return set_error("probe_mfma_issue: src must hold 12 KiB of operand bytes");
-  if (workgroups < 1 || workgroups > 65536 || iters < 1) return set_error("probe_mfma_issue: bad launch shape");
+  if (workgroups < 1 || workgroups > 65536 || iters < 1 || (waves_per_workgroup != 4 && waves_per_workgroup != 8))
+    return set_error("probe_mfma_issue: bad launch shape (4 or 8 waves per workgroup)");
+  const unsigned threads = 64u * (unsigned)waves_per_workgroup;
   hipStream_t st = (hipStream_t)stream;
   const u4* s = (const u4*)src;
   const unsigned g = (unsigned)workgroups;
 #define WOQ_PROBE_MIX(V, L)                                                \
   if (valu_per_16 == V && lds_per_16 == L) {                               \
-    probe_mfma_issue_kernel<V, L><<<g, 256, 0, st>>>(s, iters, sink);      \
+    probe_mfma_issue_kernel<V, L><<<g, threads, 0, st>>>(s, iters, sink);  \
     return check_launch("probe_mfma_issue_kernel");                        \
   }
   WOQ_PROBE_MIX(0, 0) WOQ_PROBE_MIX(16, 0) WOQ_PROBE_MIX(32, 0) WOQ_PROBE_MIX(40, 0) WOQ_PROBE_MIX(48, 0)

@@ -160,7 +160,7 @@ def load():
         lib.woq_hip_moe_combine_rows.restype = i32
         lib.woq_hip_moe_combine_rows.argtypes = [vp, i32, i64, i64, vp, vp, i64, vp, vp, i32, vp]
         lib.woq_hip_probe_mfma_issue.restype = i32
-        lib.woq_hip_probe_mfma_issue.argtypes = [vp, i32, i32, i64, i32, vp, vp]
+        lib.woq_hip_probe_mfma_issue.argtypes = [vp, i32, i32, i64, i32, i32, vp, vp]
         if lib.woq_hip_abi_version() != 1:
             raise RuntimeError("libwoq_hip.so has an unexpected ABI version")
         _lib = lib
