@@ -327,7 +327,8 @@ int woq_hip_moe_scale_add_rows(void* out, int dtype, int64_t T, int64_t H, const
  *   WOQ_HIP_MOE_ROUTE_MAX) = token of the entry at sorted position p.  slots: int32 [4][3][S], S >= min(T * topk, experts):
  *   per size class the experts that have tokens, densely from index 0 in ascending expert order, as three arrays --
  *   expert id (-1: unused entry), first sorted position, number of rows (at most 64).  Classes: 0 fewer than split_lo
- *   rows, 1 at most split_mid, 2 more, 3 (only with use_single) exactly one row, taken out of class 0.
+ *   rows, 1 at most split_mid, 2 more, 3 (use_single = 1) exactly one row, taken out of class 0.  use_single = 2:
+ *   every sorted position is a slot of one row in class 3, at its own index (S >= T * topk; for a single token).
  *   row_of[t, i] / slot_of[t, i] = sorted position and top-k slot of token t's i-th contribution in ascending expert
  *   order (row_of -1: none).  An expert id outside [0, experts) contributes nothing, and neither do an expert's entries
  *   beyond its first 64 (a slot holds at most 64 rows).

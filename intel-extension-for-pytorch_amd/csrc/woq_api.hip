@@ -430,7 +430,9 @@ int woq_hip_moe_route(const int64_t* topk_ids, int64_t T, int64_t topk, int64_t 
   if (T < 0 || topk <= 0 || experts <= 0) return set_error("moe_route: bad size");
   if (T * topk > WOQ_HIP_MOE_ROUTE_MAX)
     return set_error("moe_route: at most %d (token, slot) entries, got %lld", WOQ_HIP_MOE_ROUTE_MAX, (long long)(T * topk));
-  const int64_t need = T * topk < experts ? T * topk : experts;  // experts that can have tokens
+  if (use_single < 0 || use_single > 2) return set_error("moe_route: use_single is 0, 1 or 2");
+  // experts that can have tokens; with a slot per sorted position, the positions
+  const int64_t need = use_single == 2 ? T * topk : (T * topk < experts ? T * topk : experts);
   if (S < need) return set_error("moe_route: slot tables of %lld entries, %lld experts can have tokens", (long long)S, (long long)need);
   if (T > 0 && (!topk_ids || !x_row || !slots || !row_of || !slot_of)) return set_error("moe_route: null pointer");
   return launch_moe_route(topk_ids, T, topk, experts, split_lo, split_mid, use_single, S, x_row, slots, row_of, slot_of,

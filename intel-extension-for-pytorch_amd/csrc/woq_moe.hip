@@ -96,7 +96,9 @@ __global__ void moe_scale_add_rows_kernel(void* __restrict__ out, const void* __
 //   x_row[p]        token of the entry at sorted position p (the row of the hidden states it reads),
 //   slots           [4 classes][expert, first row, rows][S]: the experts that have tokens, densely from index 0 and in
 //                   ascending expert order, by size class -- 0: fewer than split_lo rows, 1: at most split_mid,
-//                   2: more, 3 (use_single): exactly one row (taken out of class 0) -- unused entries expert -1,
+//                   2: more, 3 (use_single 1): exactly one row (taken out of class 0) -- unused entries expert -1;
+//                   use_single 2: every sorted position p is a slot of one row in class 3, at index p (an expert
+//                   named twice then has two slots; for a single token, where that costs nothing),
 //   row_of[t, i]    sorted position of token t's i-th contribution in ascending expert order (-1: none),
 //   slot_of[t, i]   its top-k slot.
 // An expert id outside [0, experts) contributes nothing.  R <= kMoeRouteMax entries, compared pairwise from LDS.
@@ -135,7 +137,14 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const int64_t* __restric
     const int p = before + rank;
     const int t = i / topk, j = i - t * topk;
     x_row[p] = t;
-    if (rank == 0) {
+    if (use_single == 2) {
+      if (p < S) {
+        int32_t* const tab = slots + (size_t)3 * 3 * S;
+        tab[p] = e;
+        tab[S + p] = p;
+        tab[2 * S + p] = 1;
+      }
+    } else if (rank == 0) {
       const int cls = (use_single && count == 1) ? 3 : count < split_lo ? 0 : count <= split_mid ? 1 : 2;
       cls_of[p] = (int8_t)cls;
       my_p[u] = p;

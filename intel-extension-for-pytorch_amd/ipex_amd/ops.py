@@ -780,8 +780,10 @@ def _deepseek_moe_grouped(hidden_states, topk_ids, gate_ctx, up_ctx, down_ctx, r
     split = 5 if lowp == 2 else 0  # lowp_mode BF16: experts with fewer than five rows compute in fp16
     # (size class, bound on its slots' rows): an expert has at most T rows, so the larger classes are empty for small T
     # experts with exactly one row (most of them in a layer with many experts and few tokens) on the single-row kernel
-    single = bool(split) and plan.single_row
-    launches = ([(3, 1)] if single else []) + ([(0, 4)] if split and (T > 1 or not single) else []) + \
+    single = plan.single_row and _f16_regime(lowp, x.dtype, 1)
+    # a single token: every (token, slot) entry is a slot of its own (an expert named twice included)
+    each = single and T == 1 and topk <= plan.S
+    launches = [(3, 1)] if each else ([(3, 1)] if single else []) + ([(0, 4)] if split else []) + \
                ([(1, 16)] if T >= split else []) + ([(2, 64)] if T > 16 else [])
     for cls, bound in launches:
         f16 = _f16_regime(lowp, x.dtype, bound)
@@ -800,10 +802,10 @@ def _deepseek_moe_grouped(hidden_states, topk_ids, gate_ctx, up_ctx, down_ctx, r
     code = _kernels._ACT_CODE[x.dtype]
     with torch.cuda.device(x.device):
         stream = _kernels._stream()
-        _lib.check(lib.woq_hip_moe_route(ids.data_ptr(), T, topk, len(gate_ctx), split, 16, int(single), plan.S,
+        _lib.check(lib.woq_hip_moe_route(ids.data_ptr(), T, topk, len(gate_ctx), split, 16, 2 if each else int(single), plan.S,
                                          plan.x_row.data_ptr(), plan.slots.data_ptr(), plan.row_of.data_ptr(),
                                          plan.slot_of.data_ptr(), stream), "moe_route")
-        nslots = min(R, plan.S)  # experts that can have tokens: the tables are dense
+        nslots = R if each else min(R, plan.S)  # experts that can have tokens: the tables are dense
         p = _lib.LinearParams()
         p.struct_size = ctypes.sizeof(_lib.LinearParams)
         p.x_dtype = p.out_dtype = code

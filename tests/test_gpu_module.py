@@ -677,6 +677,60 @@ def test_deepseek_moe_grouped_launches_equal_the_per_expert_path(cuda, monkeypat
     assert torch.equal(op(hidden, ids2, ctxs[0], ctxs[1], ctxs[2], rw, False), want2)
 
 
+def test_moe_route_with_a_slot_per_position(cuda):
+    """use_single = 2 (what a single token gets): every sorted position is a one-row slot of its own in class 3."""
+    from ipex_amd import _lib
+
+    lib = _lib.load()
+    ids = torch.tensor([[5, 2, 5, 0, 7, 2]])  # experts 2 and 5 named twice
+    T, topk, E, S = 1, 6, 8, 8
+    x_row = torch.full((6,), -7, dtype=torch.int64, device=cuda)
+    row_of, slot_of = (torch.full((6,), -7, dtype=torch.int32, device=cuda) for _ in range(2))
+    slots = torch.full((4, 3, S), -7, dtype=torch.int32, device=cuda)
+    args = (ids.to(cuda).data_ptr(), T, topk, E, 5, 16)
+    assert lib.woq_hip_moe_route(*args, 2, 5, x_row.data_ptr(), slots.data_ptr(), row_of.data_ptr(), slot_of.data_ptr(), None) != 0
+    assert lib.woq_hip_moe_route(*args, 3, S, x_row.data_ptr(), slots.data_ptr(), row_of.data_ptr(), slot_of.data_ptr(), None) != 0
+    rc = lib.woq_hip_moe_route(*args, 2, S, x_row.data_ptr(), slots.data_ptr(), row_of.data_ptr(), slot_of.data_ptr(), None)
+    assert rc == 0, lib.woq_hip_last_error()
+    got = slots.cpu()
+    assert got[3, 0].tolist() == [0, 2, 2, 5, 5, 7, -1, -1]
+    assert got[3, 1, :6].tolist() == [0, 1, 2, 3, 4, 5] and got[3, 2, :6].tolist() == [1] * 6
+    assert bool(got[:3, 0].eq(-1).all())
+    assert row_of.cpu().tolist() == [0, 1, 2, 3, 4, 5] and slot_of.cpu().tolist() == [3, 1, 5, 0, 2, 4]
+
+
+@pytest.mark.parametrize("lowp,G", [("BF16", 128), ("BF16", 64), ("FP16", 128), ("NONE", 64)])
+@pytest.mark.parametrize("T", [1, 3])
+def test_deepseek_moe_grouped_with_an_expert_named_twice(cuda, monkeypatch, lowp, G, T):
+    """Top-k lists that name an expert twice: in the grouped launches both entries are rows of that expert, each with
+    its own routing weight."""
+    from ipex_amd import _lib
+
+    ipex = _ipex()
+    E, H, I, topk = 6, 256, 256, 4
+    mk = lambda k, n, s: _woq_module(ipex, k, n, "INT4", G, lowp, bias=False, seed=s)
+    ctxs = [[mk(H, I, 500 + 3 * e)._op_context for e in range(E)], [mk(H, I, 501 + 3 * e)._op_context for e in range(E)],
+            [mk(I, H, 502 + 3 * e)._op_context for e in range(E)]]
+    g = torch.Generator().manual_seed(T)
+    xdt = torch.float16 if lowp == "FP16" else torch.bfloat16
+    hidden = torch.randn(T, H, generator=g).to(xdt).to(cuda)
+    ids = torch.tensor([[3, 1, 3, 5], [0, 0, 0, 0], [2, 4, 1, 2]][:T]).to(cuda)
+    rw = torch.softmax(torch.randn(T, topk, generator=g), -1).to(xdt).to(cuda)
+    op = torch.ops.torch_ipex.deepseek_moe_woq
+    monkeypatch.setenv("IPEX_AMD_MOE_GROUPED", "1")
+    got = op(hidden, ids, ctxs[0], ctxs[1], ctxs[2], rw, False)
+    assert _lib.last_kernel() == "moe_combine_rows"
+    # the same layer one top-k column at a time (no expert is named twice inside a column), summed in float
+    want = torch.zeros(T, H)
+    for j in range(topk):
+        want += op(hidden, ids[:, j:j + 1].contiguous(), ctxs[0], ctxs[1], ctxs[2], rw[:, j:j + 1].contiguous(), False).float().cpu()
+    assert float((got.float().cpu() - want).norm() / want.norm()) < 8e-3
+    # the per-expert path refuses such lists (its scatter adds a token's row once per expert)
+    monkeypatch.setenv("IPEX_AMD_MOE_GROUPED", "0")
+    with pytest.raises(RuntimeError, match="a token may appear once"):
+        op(hidden, ids, ctxs[0], ctxs[1], ctxs[2], rw, False)
+
+
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
 @pytest.mark.parametrize("accumulate", [0, 1])
 def test_moe_combine_rows_bit_exact(cuda, dtype, accumulate):
