@@ -855,12 +855,25 @@ def deepseek_moe_woq(hidden_states, topk_ids, gate_ctx, up_ctx, down_ctx, routin
     topk = ids.shape[1]
     order = torch.argsort(ids.reshape(-1), stable=True)  # by expert, then token, then slot
     counts = torch.bincount(ids.reshape(-1), minlength=num_experts).tolist()
-    routed = torch.stack([order // topk, order % topk]).to(hidden_states.device)
+    tokens = order // topk
+    routed = torch.stack([tokens, order % topk]).to(hidden_states.device)
     start = 0
     for e, n in enumerate(counts):
         if n:
-            _moe_expert(hidden_states, routed[0, start:start + n], routed[1, start:start + n], gate_ctx[e], up_ctx[e],
-                        down_ctx[e], routing_weights, output)
+            tok = tokens[start:start + n]
+            if n > 1 and bool((tok[1:] == tok[:-1]).any()):
+                # a token names this expert more than once: the scatter adds one row per token, so the entries go in
+                # rounds, the k-th mention of every token in round k
+                first = torch.cat([torch.ones(1, dtype=torch.bool), tok[1:] != tok[:-1]])
+                pos = torch.arange(n)
+                mention = pos - torch.cummax(torch.where(first, pos, torch.zeros_like(pos)), 0).values
+                for k in range(int(mention.max()) + 1):
+                    sel = (start + torch.nonzero(mention == k).flatten()).to(hidden_states.device)
+                    _moe_expert(hidden_states, routed[0].index_select(0, sel), routed[1].index_select(0, sel), gate_ctx[e],
+                                up_ctx[e], down_ctx[e], routing_weights, output)
+            else:
+                _moe_expert(hidden_states, routed[0, start:start + n], routed[1, start:start + n], gate_ctx[e], up_ctx[e],
+                            down_ctx[e], routing_weights, output)
         start += n
     return output
 

@@ -725,10 +725,11 @@ def test_deepseek_moe_grouped_with_an_expert_named_twice(cuda, monkeypatch, lowp
     for j in range(topk):
         want += op(hidden, ids[:, j:j + 1].contiguous(), ctxs[0], ctxs[1], ctxs[2], rw[:, j:j + 1].contiguous(), False).float().cpu()
     assert float((got.float().cpu() - want).norm() / want.norm()) < 8e-3
-    # the per-expert path refuses such lists (its scatter adds a token's row once per expert)
+    # the per-expert path runs the mentions of a token in rounds (its scatter adds one row per token)
     monkeypatch.setenv("IPEX_AMD_MOE_GROUPED", "0")
-    with pytest.raises(RuntimeError, match="a token may appear once"):
-        op(hidden, ids, ctxs[0], ctxs[1], ctxs[2], rw, False)
+    per_expert = op(hidden, ids, ctxs[0], ctxs[1], ctxs[2], rw, False)
+    assert _lib.last_kernel() == "moe_scale_add_rows"
+    assert float((per_expert.float().cpu() - want).norm() / want.norm()) < 8e-3
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
