@@ -1,5 +1,5 @@
 // Decode kernel for the fp16 regime (M < 5 under lowp_mode BF16 or FP16) with 4-bit weights and
-// group sizes that are multiples of 128, or 32: HBM-bound weight streaming.
+// group sizes that are multiples of 128, or 64, or 32: HBM-bound weight streaming.
 //
 // Reference counterpart: the small-batch FMA micro-kernel, which keeps the weights as exact small
 // integers and applies the group scale to the block sum (csrc/cpu/aten/utils/woq.h:775-951:
@@ -48,14 +48,16 @@ __device__ __forceinline__ f4 mfma16(u4 a, u4 b, f4 c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_bf16(bitcast<b8>(a), bitcast<b8>(b), c, 0, 0, 0);
 }
 
-// G32 (groups of 32 input channels): a lane column's 32 K values of a tile are one group, but an MFMA sums over the
-// four lane columns.  The rows of the A operand keep the groups apart: row 4 g + m carries activation row m in lane
-// column g only and zeros elsewhere (read from a zeroed LDS slice), so lane column c accumulates the sums over group c
-// alone for the four activation rows and applies that group's (scale, zero) dword; the four lane columns are added
-// at the end.
-template <bool XF16, int NTW, int MAXM, bool ONE_ROUND, bool G32>
+// GPT = 4 or 2 groups per K tile (groups of 32 or 64 input channels): a lane column's 32 K values of a tile belong to
+// one group, but an MFMA sums over the four lane columns.  The rows of the A operand keep the groups apart: row
+// 4 g + m carries activation row m in the lane columns of group g only and zeros elsewhere (read from a zeroed LDS
+// slice), so lane column c accumulates the sums over group c alone for the four activation rows and applies that
+// group's (scale, zero) dword; the lane columns are added at the end.
+template <bool XF16, int NTW, int MAXM, bool ONE_ROUND, int GPT>
 __global__ __launch_bounds__(1024, 8) void woq_decode_kernel(const DecodeArgs a) {
-  static_assert(!G32 || MAXM == 4, "four activation rows times four groups fill the 16 rows of the A operand");
+  static_assert(GPT == 1 || GPT == 2 || GPT == 4, "groups of 128 x 2^k, 64 or 32");
+  constexpr bool G32 = GPT > 1;  // the groups of a tile are kept apart
+  static_assert(!G32 || MAXM == 4, "four activation rows times up to four groups fill the 16 rows of the A operand");
   constexpr int KPW = kDecodeKPW;
   constexpr int SLICE = KPW * kTileK4;  // K elements of one wave per round
   constexpr int XROWS = MAXM + (G32 ? 1 : 0);  // LDS rows of a wave: its activation slices (and one of zeros)
@@ -92,7 +94,7 @@ __global__ __launch_bounds__(1024, 8) void woq_decode_kernel(const DecodeArgs a)
   const int xlane = lane & (KPW * 16 - 1);  // lanes 32..63 mirror 0..31
   // row of the A operand -> LDS row: the activation row itself (rows past MAXM mirror row 0), or with G32 row r % 4
   // in lane column r / 4 and the zero slice in the others
-  const int xrow = G32 ? (c == (r >> 2) ? (r & 3) : MAXM) : (r < MAXM ? r : 0);
+  const int xrow = G32 ? ((r >> 2) < GPT && (c >> (GPT == 2 ? 1 : 0)) == (r >> 2) ? (r & 3) : MAXM) : (r < MAXM ? r : 0);
   const __amdgpu_buffer_rsrc_t wrs = __builtin_amdgcn_make_buffer_rsrc((void*)a.qweight, 0, (int)a.wbytes, 0x00020000);
   const __amdgpu_buffer_rsrc_t srs = __builtin_amdgcn_make_buffer_rsrc((void*)a.sz, 0, (int)a.szbytes, 0x00020000);
 
@@ -123,15 +125,15 @@ __global__ __launch_bounds__(1024, 8) void woq_decode_kernel(const DecodeArgs a)
     // unit (decode_kernel_applies keeps weights of 4 GiB and more away) ----
     u4 wreg[NTW][KPW];
     uint32_t szreg[NTW][KPW];
-    // (G32: lane column c takes the dword of group 4 kt + c, 64 bytes after the one of group 4 kt + c - 1)
-    const int lane16 = lane * 16, r4 = G32 ? lane * 4 : r * 4;
+    // (several groups per tile: lane column c takes the dword of group GPT kt + c % GPT, 64 bytes per group)
+    const int lane16 = lane * 16, r4 = ((c & (GPT - 1)) * 16 + r) * 4;
 #pragma unroll
     for (int i = 0; i < KPW; ++i) {
 #pragma unroll
       for (int t = 0; t < NTW; ++t) {
         const uint32_t nt = (uint32_t)nt0 + t;
         const int woff = (int)((nt * (uint32_t)KT + (uint32_t)(ktw + i)) * (uint32_t)kTileBytes);
-        const uint32_t grp = G32 ? (uint32_t)(ktw + i) * 4u : (uint32_t)(ktw + i) >> tpg_shift;
+        const uint32_t grp = G32 ? (uint32_t)(ktw + i) * (uint32_t)GPT : (uint32_t)(ktw + i) >> tpg_shift;
         const int soff = (int)((nt * (uint32_t)KG + grp) * (uint32_t)(kTileN * sizeof(uint32_t)));
         wreg[t][i] = __builtin_amdgcn_raw_buffer_load_b128(wrs, lane16, woff, 2);  // non-temporal
         szreg[t][i] = __builtin_amdgcn_raw_buffer_load_b32(srs, r4, soff, 0);
@@ -181,14 +183,15 @@ __global__ __launch_bounds__(1024, 8) void woq_decode_kernel(const DecodeArgs a)
   }
 
   // ---- combine the waves' partial sums in wave order, then bias / rounding / store ----
-  // G32: a lane column holds the terms of its own groups; the four are added here
+  // several groups per tile: a lane column holds the terms of its own groups (columns without a group hold
+  // zeros); they are added here
   if constexpr (G32) {
 #pragma unroll
     for (int t = 0; t < NTW; ++t)
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
         acc[t][e] += __shfl_xor(acc[t][e], 16);
-        acc[t][e] += __shfl_xor(acc[t][e], 32);
+        if constexpr (GPT == 4) acc[t][e] += __shfl_xor(acc[t][e], 32);
       }
   }
   // Only lanes 0..15 hold rows m = 0..3 (M <= 4); they publish their four accumulators.
@@ -237,13 +240,17 @@ __global__ __launch_bounds__(1024, 8) void woq_decode_kernel(const DecodeArgs a)
 //     scales and accumulates one element per tile instead of four.
 // GROUPED (mixture of experts): the workgroups with blockIdx.z = s serve slot s, one routed row of one expert, whose
 // packed weight, (scale, zero) table and bias come from pointer tables in device memory; an empty slot exits.
-// G32 (groups of 32 input channels): a lane column's 32 K values of a tile are one group, but an MFMA sums over the
-// four lane columns.  The 15 spare rows of the A operand keep the groups apart: row m carries the activations of lane
-// column m / 4 only and zeros elsewhere (read from a zeroed LDS slice, no instruction more), so D[4 c][n] -- the
-// accumulator register the kernel uses anyway -- is the sum over group c alone, in lane column c, which applies that
-// group's (scale, zero) dword; the four lane columns are added at the end.
-template <bool XBF16, int NTW, int KPW, bool ONE_ROUND, bool GROUPED, bool G32>
+// GPT = 4 or 2 groups per K tile (groups of 32 or 64 input channels): a lane column's 32 K values of a tile belong to
+// one group, but an MFMA sums over the four lane columns.  The 15 spare rows of the A operand keep the groups apart:
+// row m carries the activations of the lane columns of one group only -- the group of lane column m / 4 -- and zeros
+// elsewhere (read from a zeroed LDS slice, no instruction more), so D[4 c][n] -- the accumulator register the kernel
+// uses anyway -- is the sum over the group of lane column c alone, and that lane column applies the group's
+// (scale, zero) dword; one lane column per group is added at the end.
+template <bool XBF16, int NTW, int KPW, bool ONE_ROUND, bool GROUPED, int GPT>
 __global__ __launch_bounds__(KPW == 2 ? 1024 : 512, KPW == 2 ? 8 : 4) void woq_decode_m1_kernel(const DecodeArgs a_in) {
+  static_assert(GPT == 1 || GPT == 2 || GPT == 4, "groups of 128 x 2^k, 64 or 32");
+  constexpr bool G32 = GPT > 1;       // the groups of a tile are kept apart
+  constexpr int CS = GPT == 2 ? 1 : 0;  // lane columns per group, as a shift
   static_assert(!(GROUPED && G32), "grouped launches take groups of 128 x 2^k");
   DecodeArgs ag;
   if constexpr (GROUPED) {
@@ -321,8 +328,8 @@ __global__ __launch_bounds__(KPW == 2 ? 1024 : 512, KPW == 2 ? 8 : 4) void woq_d
 
     u4 wreg[NTW][KPW];
     uint32_t szreg[NTW][KPW];
-    // (G32: lane column c takes the dword of group 4 kt + c, 64 bytes after the one of group 4 kt + c - 1)
-    const int lane16 = lane * 16, r4 = G32 ? lane * 4 : r * 4;
+    // (several groups per tile: lane column c takes the dword of its group GPT kt + c / (4 / GPT), 64 bytes per group)
+    const int lane16 = lane * 16, r4 = G32 ? ((c >> CS) * 16 + r) * 4 : r * 4;
     // requested in the order of use: K tile by K tile, row-block by row-block, each tile with its parameters
 #pragma unroll
     for (int i = 0; i < KPW; ++i) {
@@ -330,7 +337,7 @@ __global__ __launch_bounds__(KPW == 2 ? 1024 : 512, KPW == 2 ? 8 : 4) void woq_d
       for (int t = 0; t < NTW; ++t) {
         const uint32_t nt = (uint32_t)nt0 + t;
         const int woff = (int)((nt * (uint32_t)KT + (uint32_t)(ktw + i)) * (uint32_t)kTileBytes);
-        const uint32_t grp = G32 ? (uint32_t)(ktw + i) * 4u : (uint32_t)(ktw + i) >> tpg_shift;
+        const uint32_t grp = G32 ? (uint32_t)(ktw + i) * (uint32_t)GPT : (uint32_t)(ktw + i) >> tpg_shift;
         const int soff = (int)((nt * (uint32_t)KG + grp) * (uint32_t)(kTileN * sizeof(uint32_t)));
         wreg[t][i] = __builtin_amdgcn_raw_buffer_load_b128(wrs, lane16, woff, 2);  // non-temporal
         szreg[t][i] = __builtin_amdgcn_raw_buffer_load_b32(srs, r4, soff, 0);
@@ -360,8 +367,9 @@ __global__ __launch_bounds__(KPW == 2 ? 1024 : 512, KPW == 2 ? 8 : 4) void woq_d
 #pragma unroll
     for (int i = 0; i < KPW; ++i) {
       u4 xa[4];
-      // (G32: row r of the A operand carries lane column r / 4 only; the other lanes read the zero slice)
-      const uint16_t* const xsrc = (!G32 || c == (r >> 2)) ? sx : sx + SLICE;
+      // (several groups per tile: row r of the A operand carries the lane columns of the group of lane column r / 4
+      // only; the other lanes read the zero slice)
+      const uint16_t* const xsrc = (!G32 || (c >> CS) == (r >> (2 + CS))) ? sx : sx + SLICE;
 #pragma unroll
       for (int j = 0; j < 4; ++j) xa[j] = *(const u4*)(xsrc + i * kTileK4 + c * 32 + j * 8);
       f4 dk = f4{0.f, 0.f, 0.f, 0.f};
@@ -395,11 +403,12 @@ __global__ __launch_bounds__(KPW == 2 ? 1024 : 512, KPW == 2 ? 8 : 4) void woq_d
   if (W < 16 && threadIdx.x < NTW * 16) {
     for (int w = W; w < 16; ++w) red[threadIdx.x * 16 + w] = 0.f;
   }
-  // G32: a lane column holds the terms of its own groups; the four are added here
+  // several groups per tile: a lane column holds the terms of its own group (with two groups, lane columns c and
+  // c + 1 the same ones); one lane column per group is added here
   if constexpr (G32) {
 #pragma unroll
     for (int t = 0; t < NTW; ++t) {
-      acc[t] += __shfl_xor(acc[t], 16);
+      if constexpr (GPT == 4) acc[t] += __shfl_xor(acc[t], 16);
       acc[t] += __shfl_xor(acc[t], 32);
     }
   }
@@ -433,23 +442,25 @@ __global__ __launch_bounds__(KPW == 2 ? 1024 : 512, KPW == 2 ? 8 : 4) void woq_d
 
 template <bool XBF16, int NTW, int KPW, bool ONE_ROUND>
 static int launch_decode_m1_cfg(const DecodeArgs& a, hipStream_t st, int slots = 0) {
-  const bool g32 = a.G == 32;
-  const size_t smem = (size_t)NTW * 16 * 16 * sizeof(float) + (size_t)a.W * KPW * kTileK4 * sizeof(uint16_t) * (g32 ? 2 : 1);
+  const bool apart = a.G == 32 || a.G == 64;  // several groups per K tile
+  const size_t smem = (size_t)NTW * 16 * 16 * sizeof(float) + (size_t)a.W * KPW * kTileK4 * sizeof(uint16_t) * (apart ? 2 : 1);
   const unsigned grid = (unsigned)((a.NT + NTW - 1) / NTW);
   if (slots > 0)
-    woq_decode_m1_kernel<XBF16, NTW, KPW, ONE_ROUND, true, false><<<dim3(grid, 1, (unsigned)slots), a.W * 64, smem, st>>>(a);
-  else if (g32)
-    woq_decode_m1_kernel<XBF16, NTW, KPW, ONE_ROUND, false, true><<<grid, a.W * 64, smem, st>>>(a);
+    woq_decode_m1_kernel<XBF16, NTW, KPW, ONE_ROUND, true, 1><<<dim3(grid, 1, (unsigned)slots), a.W * 64, smem, st>>>(a);
+  else if (a.G == 32)
+    woq_decode_m1_kernel<XBF16, NTW, KPW, ONE_ROUND, false, 4><<<grid, a.W * 64, smem, st>>>(a);
+  else if (a.G == 64)
+    woq_decode_m1_kernel<XBF16, NTW, KPW, ONE_ROUND, false, 2><<<grid, a.W * 64, smem, st>>>(a);
   else
-    woq_decode_m1_kernel<XBF16, NTW, KPW, ONE_ROUND, false, false><<<grid, a.W * 64, smem, st>>>(a);
+    woq_decode_m1_kernel<XBF16, NTW, KPW, ONE_ROUND, false, 1><<<grid, a.W * 64, smem, st>>>(a);
   return check_launch("woq_decode_m1_kernel");
 }
 
-template <bool XF16, int NTW, int MAXM, bool ONE_ROUND, bool G32>
+template <bool XF16, int NTW, int MAXM, bool ONE_ROUND, int GPT>
 static int launch_decode_cfg_g(const DecodeArgs& a, hipStream_t st) {
   const size_t smem = (size_t)NTW * a.W * 16 * sizeof(f4) +
-                      (size_t)a.W * (MAXM + (G32 ? 1 : 0)) * kDecodeKPW * kTileK4 * sizeof(uint16_t);
-  auto kern = woq_decode_kernel<XF16, NTW, MAXM, ONE_ROUND, G32>;
+                      (size_t)a.W * (MAXM + (GPT > 1 ? 1 : 0)) * kDecodeKPW * kTileK4 * sizeof(uint16_t);
+  auto kern = woq_decode_kernel<XF16, NTW, MAXM, ONE_ROUND, GPT>;
   if (smem > 64 * 1024) {
     hipError_t err = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
     if (err != hipSuccess) return set_error("hipFuncSetAttribute: %s", hipGetErrorString(err));
@@ -461,16 +472,17 @@ static int launch_decode_cfg_g(const DecodeArgs& a, hipStream_t st) {
 
 template <bool XF16, int NTW, int MAXM, bool ONE_ROUND>
 static int launch_decode_cfg(const DecodeArgs& a, hipStream_t st) {
-  return a.G == 32 ? launch_decode_cfg_g<XF16, NTW, MAXM, ONE_ROUND, true>(a, st)
-                   : launch_decode_cfg_g<XF16, NTW, MAXM, ONE_ROUND, false>(a, st);
+  return a.G == 32   ? launch_decode_cfg_g<XF16, NTW, MAXM, ONE_ROUND, 4>(a, st)
+         : a.G == 64 ? launch_decode_cfg_g<XF16, NTW, MAXM, ONE_ROUND, 2>(a, st)
+                     : launch_decode_cfg_g<XF16, NTW, MAXM, ONE_ROUND, 1>(a, st);
 }
 
 bool decode_kernel_applies(const FpArgs& f, int wbits, int regime, const uint32_t* sz) {
   const int64_t tpg = f.G / kTileK4;
   // the kernels address the packed weight and its parameters with 32-bit offsets
   if (f.NT * f.KT * kTileBytes >= ((int64_t)1 << 32) || f.NT * f.KG * kTileN * 4 >= ((int64_t)1 << 32)) return false;
-  // groups of 128 x 2^k, or of 32
-  const bool groups = ((f.G % kTileK4) == 0 && (tpg & (tpg - 1)) == 0) || f.G == 32;
+  // groups of 128 x 2^k, of 64 or of 32
+  const bool groups = ((f.G % kTileK4) == 0 && (tpg & (tpg - 1)) == 0) || f.G == 32 || f.G == 64;
   return sz != nullptr && wbits == 4 && regime == kRegimeF16 && f.M <= 4 && groups &&
          (f.K % (kDecodeKPW * kTileK4)) == 0 && (f.x_dtype == WOQ_HIP_ACT_BF16 || f.x_dtype == WOQ_HIP_ACT_FP16);
 }

@@ -531,7 +531,8 @@ def test_deepseek_moe_woq_matches_per_expert_composition(cuda, T, topk):
     from oracle import woq_oracle as O
 
     ipex = _ipex()
-    E, H, I = 5, 256, 384
+    # (K not a multiple of 256 in any linear: experts with few rows then run the dequantizing kernel on both paths)
+    E, H, I = 5, 384, 640
     gate, up, down = _moe_layer(ipex, E, H, I, 100)
     g = torch.Generator().manual_seed(T)
     hidden = torch.randn(T, H, generator=g).to(torch.bfloat16)
@@ -650,7 +651,8 @@ def test_deepseek_moe_grouped_launches_equal_the_per_expert_path(cuda, monkeypat
     from ipex_amd import _lib
 
     ipex = _ipex()
-    E, H, I = 9, 256, 384
+    # (K not a multiple of 256 in any linear: experts with few rows then run the dequantizing kernel on both paths)
+    E, H, I = 9, 384, 640
     G = 64 if weight_dtype == "INT4" else -1
     mk = lambda k, n, s: _woq_module(ipex, k, n, weight_dtype, G, lowp, bias=False, seed=s)
     ctxs = [[mk(H, I, 300 + 3 * e)._op_context for e in range(E)], [mk(H, I, 301 + 3 * e)._op_context for e in range(E)],

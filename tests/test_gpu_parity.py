@@ -1897,16 +1897,17 @@ def test_single_row_decode_with_four_k_tiles_per_wave(cuda, K, N):
         (8192, 8192, True),    # several rounds with two row-blocks
     ],
 )
-def test_decode_kernels_with_groups_of_32(cuda, K, N, bias):
-    """Up to four rows with groups of 32 input channels on the integer-weight decode kernels: the four groups of a K
-    tile stay apart in rows of the MFMA's activation operand.  Symmetric weights and fp16 rows (lowp_mode FP16) as
-    well; five and more rows keep the dequantizing kernel."""
+@pytest.mark.parametrize("G", [32, 64])
+def test_decode_kernels_with_groups_of_32_and_64(cuda, K, N, bias, G):
+    """Up to four rows with groups of 32 or 64 input channels on the integer-weight decode kernels: the four or two
+    groups of a K tile stay apart in rows of the MFMA's activation operand.  Symmetric weights and fp16 rows
+    (lowp_mode FP16) as well; five and more rows keep the dequantizing kernel."""
     from ipex_amd import _lib
 
     syn = _synthetic()
     cols = None if N * K <= 4096 * 4096 else np.arange(0, N, 7)
-    case = syn.make_int4_case(78, 1, K, N, 32, bias=bias)
-    _check_fp(case, O.LOWP_BF16, cols=cols, label=f"M=1 G=32 K={K} N={N}")
+    case = syn.make_int4_case(78, 1, K, N, G, bias=bias)
+    _check_fp(case, O.LOWP_BF16, cols=cols, label=f"M=1 G={G} K={K} N={N}")
     assert _lib.last_kernel() == "woq_decode_m1_kernel"
     ctx = make_context(case, O.LOWP_BF16)
     x = case["x"].cuda()
@@ -1914,7 +1915,7 @@ def test_decode_kernels_with_groups_of_32(cuda, K, N, bias):
     assert rel_l2(a, b) <= 2e-3
     assert torch.equal(ctx.run(x), ctx.run(x))
     sym = dict(case, zeros=None)
-    _check_fp(sym, O.LOWP_BF16, cols=cols, label=f"M=1 G=32 symmetric K={K} N={N}")
+    _check_fp(sym, O.LOWP_BF16, cols=cols, label=f"M=1 G={G} symmetric K={K} N={N}")
     case16 = dict(case)
     case16["x"] = case["x"].to(torch.float16)
     ctx16 = make_context(case16, O.LOWP_FP16)
@@ -1922,16 +1923,16 @@ def test_decode_kernels_with_groups_of_32(cuda, K, N, bias):
     y = to_np_f32(ctx16.run(case16["x"].cuda()))
     assert _lib.last_kernel() == "woq_decode_m1_kernel"
     if cols is None:
-        _, want = O.woq_linear_ref(c["x"], "fp16", c["qw"], N, K, O._round_to(c["scales"], "fp16"), c["zps"], c["bias"], 2, 32, "fp16")
+        _, want = O.woq_linear_ref(c["x"], "fp16", c["qw"], N, K, O._round_to(c["scales"], "fp16"), c["zps"], c["bias"], 2, G, "fp16")
         assert rel_l2(y, want) <= REL_L2_OUT
     # two to four rows: the same arrangement with row 4 g + m of the A operand for group g of activation row m
     for M in (2, 3, 4):
-        more = syn.make_int4_case(79 + M, M, K, N, 32, bias=bias)
-        _check_fp(more, O.LOWP_BF16, cols=cols, label=f"M={M} G=32 K={K} N={N}")
+        more = syn.make_int4_case(79 + M, M, K, N, G, bias=bias)
+        _check_fp(more, O.LOWP_BF16, cols=cols, label=f"M={M} G={G} K={K} N={N}")
         assert _lib.last_kernel() == "woq_decode_kernel"
         ctxm = make_context(more, O.LOWP_BF16)
         xm = more["x"].cuda()
         assert rel_l2(to_np_f32(ctxm.run(xm)), to_np_f32(ctxm.run(xm, force_kernel=1))) <= 2e-3
-    five = syn.make_int4_case(85, 5, K, N, 32, bias=bias)
+    five = syn.make_int4_case(85, 5, K, N, G, bias=bias)
     make_context(five, O.LOWP_BF16).run(five["x"].cuda())
     assert _lib.last_kernel() == "woq_decode_dq_kernel"
