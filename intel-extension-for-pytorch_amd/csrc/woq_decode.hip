@@ -251,7 +251,6 @@ __global__ __launch_bounds__(KPW == 2 ? 1024 : 512, KPW == 2 ? 8 : 4) void woq_d
   static_assert(GPT == 1 || GPT == 2 || GPT == 4, "groups of 128 x 2^k, 64 or 32");
   constexpr bool G32 = GPT > 1;       // the groups of a tile are kept apart
   constexpr int CS = GPT == 2 ? 1 : 0;  // lane columns per group, as a shift
-  static_assert(!(GROUPED && G32), "grouped launches take groups of 128 x 2^k");
   DecodeArgs ag;
   if constexpr (GROUPED) {
     const MoeGroup& g = *a_in.grp;
@@ -445,8 +444,13 @@ static int launch_decode_m1_cfg(const DecodeArgs& a, hipStream_t st, int slots =
   const bool apart = a.G == 32 || a.G == 64;  // several groups per K tile
   const size_t smem = (size_t)NTW * 16 * 16 * sizeof(float) + (size_t)a.W * KPW * kTileK4 * sizeof(uint16_t) * (apart ? 2 : 1);
   const unsigned grid = (unsigned)((a.NT + NTW - 1) / NTW);
-  if (slots > 0)
-    woq_decode_m1_kernel<XBF16, NTW, KPW, ONE_ROUND, true, 1><<<dim3(grid, 1, (unsigned)slots), a.W * 64, smem, st>>>(a);
+  const dim3 ggrid(grid, 1, (unsigned)(slots > 0 ? slots : 1));
+  if (slots > 0 && a.G == 32)
+    woq_decode_m1_kernel<XBF16, NTW, KPW, ONE_ROUND, true, 4><<<ggrid, a.W * 64, smem, st>>>(a);
+  else if (slots > 0 && a.G == 64)
+    woq_decode_m1_kernel<XBF16, NTW, KPW, ONE_ROUND, true, 2><<<ggrid, a.W * 64, smem, st>>>(a);
+  else if (slots > 0)
+    woq_decode_m1_kernel<XBF16, NTW, KPW, ONE_ROUND, true, 1><<<ggrid, a.W * 64, smem, st>>>(a);
   else if (a.G == 32)
     woq_decode_m1_kernel<XBF16, NTW, KPW, ONE_ROUND, false, 4><<<grid, a.W * 64, smem, st>>>(a);
   else if (a.G == 64)
@@ -494,7 +498,6 @@ int launch_decode(const FpArgs& f, const uint32_t* sz, hipStream_t st) { return 
 int launch_decode_grouped(const FpArgs& f, const MoeGroup* grp, int64_t slots, hipStream_t st) {
   if (!grp || slots < 1 || slots > 65535) return set_error("woq_linear_grouped: 1..65535 slots and a group table");
   if (f.M != 1) return set_error("woq_linear_grouped: the single-row kernel takes one row per slot");
-  if (f.G % kTileK4 != 0) return set_error("woq_linear_grouped: the single-row kernel takes groups of 128 x 2^k");
   return launch_decode_impl(f, nullptr, st, grp, (int)slots);
 }
 

@@ -706,10 +706,11 @@ class _MoeGroupedPlan:
             col = lambda k: torch.tensor([r[k] for r in rows], dtype=torch.int64, device=device)
             self.tables.append(dict(qweight=col(0), s16=col(1), sb16=col(2), z8=col(3) if rows[0][3] else None,
                                     bias=col(4) if rows[0][4] else None, sz=col(12) if rows[0][12] else None))
-        # the single-row decode kernel serves the experts with fewer than five rows where all three linears have its
-        # (scale, zero) tables: 4-bit weights in groups of 128 x 2^k, K a multiple of 256
+        # the single-row decode kernel serves the experts with one row where all three linears have its
+        # (scale, zero) tables: 4-bit weights in groups of 32, 64 or 128 x 2^k, K a multiple of 256
         self.single_row = all(t["sz"] is not None for t in self.tables) and all(
-            x["wd"] == _lib.DTYPE_INT4 and x["K"] % 256 == 0 and x["G"] % 128 == 0 and (x["G"] // 128) & (x["G"] // 128 - 1) == 0
+            x["wd"] == _lib.DTYPE_INT4 and x["K"] % 256 == 0 and (x["G"] in (32, 64) or (
+                x["G"] % 128 == 0 and (x["G"] // 128) & (x["G"] // 128 - 1) == 0))
             for x in self.shapes)
         self.structs = {}
         self.rows = {}  # dtype -> (act, inter, y) for the most routed rows seen

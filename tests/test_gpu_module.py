@@ -701,6 +701,30 @@ def test_moe_route_with_a_slot_per_position(cuda):
     assert row_of.cpu().tolist() == [0, 1, 2, 3, 4, 5] and slot_of.cpu().tolist() == [3, 1, 5, 0, 2, 4]
 
 
+@pytest.mark.parametrize("G", [32, 64, 128])
+def test_deepseek_moe_grouped_single_token_is_the_per_expert_result(cuda, monkeypatch, G):
+    """One token: every expert it names has one row, which both paths give to the single-row decode kernel (groups of
+    32, 64 and 128): bit for bit."""
+    from ipex_amd import _lib
+
+    ipex = _ipex()
+    E, H, I, topk = 7, 512, 256, 4
+    mk = lambda k, n, s: _woq_module(ipex, k, n, "INT4", G, "BF16", bias=False, seed=s)
+    ctxs = [[mk(H, I, 600 + 3 * e)._op_context for e in range(E)], [mk(H, I, 601 + 3 * e)._op_context for e in range(E)],
+            [mk(I, H, 602 + 3 * e)._op_context for e in range(E)]]
+    g = torch.Generator().manual_seed(G)
+    hidden = torch.randn(1, H, generator=g).to(torch.bfloat16).to(cuda)
+    ids = torch.randperm(E, generator=g)[:topk].reshape(1, topk).to(cuda)
+    rw = torch.softmax(torch.randn(1, topk, generator=g), -1).to(torch.bfloat16).to(cuda)
+    op = torch.ops.torch_ipex.deepseek_moe_woq
+    monkeypatch.setenv("IPEX_AMD_MOE_GROUPED", "0")
+    want = op(hidden, ids, ctxs[0], ctxs[1], ctxs[2], rw, False)
+    monkeypatch.setenv("IPEX_AMD_MOE_GROUPED", "1")
+    got = op(hidden, ids, ctxs[0], ctxs[1], ctxs[2], rw, False)
+    assert _lib.last_kernel() == "moe_combine_rows"
+    assert torch.equal(got, want)
+
+
 @pytest.mark.parametrize("lowp,G", [("BF16", 128), ("BF16", 64), ("FP16", 128), ("NONE", 64)])
 @pytest.mark.parametrize("T", [1, 3])
 def test_deepseek_moe_grouped_with_an_expert_named_twice(cuda, monkeypatch, lowp, G, T):
