@@ -745,8 +745,9 @@ def main():
         outp = torch.empty(Mp, N, dtype=torch.bfloat16, device=dev)
         flops = 2.0 * Mp * K * N
         pre = {}
-        # its own fixed counts, whatever --steps says: 60 warm-up launches, then five regions of 40
-        warm_p, steps_p, groups_p = 60, 40, 5
+        # its own fixed counts, whatever --steps says: 200 warm-up launches (the clock needs about 150 launches of this
+        # kernel to settle after the decode phase: 245 us per launch at first, 198 us from then on), then five regions of 40
+        warm_p, steps_p, groups_p = 200, 40, 5
         # (bf16_lds_tile: the same problem on the kernel that dequantizes once per workgroup into LDS, force_kernel 21)
         for name, lowp, aq, forced in (("bf16", 2, -1, 0), ("int8", 3, 6, 0), ("bf16_lds_tile", 2, -1, 21)):
             ws = None
