@@ -339,7 +339,7 @@ int woq_hip_moe_scale_add_rows(void* out, int dtype, int64_t T, int64_t H, const
  *   larger M on the others; M <= 16 and M > 16 also select a kernel with one or four row tiles, hence the size classes); p's weight, scale, zero
  *   point and bias pointers are ignored -- except that a non-NULL scale_zero_f16x2 says that the group's scales table
  *   holds the experts' (fp16 scale, fp16 128 + zero) dword tables: the call then runs the single-row decode kernel
- *   (M must be 1: one row per slot, the class of experts with exactly one row; 4-bit weights in groups of 32, 64 or 128 * 2^k, K a multiple of 256,
+ *   (M must be at most 4: the classes of experts with exactly one row and with fewer than five; 4-bit weights in groups of 32, 64 or 128 * 2^k, K a multiple of 256,
  *   fp16 compute).  x: the rows the slots read, out / others[0]: [routed rows, N].  group: DEVICE
  *   pointer to a woq_hip_moe_group.  Rows of a slot are row0 .. row0 + rows - 1 of out; they read row x_row[row] of x,
  *   or the same row when x_row is NULL.  Needs what the dequantizing decode kernel needs: K a multiple of the weight tile,

@@ -354,13 +354,13 @@ int woq_hip_linear_grouped(const woq_hip_linear_params* p, const void* group, in
   f.other0 = p->others[0]; f.other1 = nullptr; f.out = p->out; f.out_dtype = p->out_dtype;
   f.nf4 = 0; f.fp8 = 0;
   if (p->scale_zero_f16x2) {
-    // one routed row per slot on the single-row decode kernel: the group's scales table holds the experts'
-    // (fp16 scale, fp16 128 + zero) dword tables
-    if (p->M != 1) return set_error("woq_linear_grouped: (scale, zero) dword tables go with one row per slot (M = 1)");
+    // up to four routed rows per slot on the integer-weight decode kernels: the group's scales table holds the
+    // experts' (fp16 scale, fp16 128 + zero) dword tables
+    if (p->M > 4) return set_error("woq_linear_grouped: (scale, zero) dword tables go with at most four rows per slot (M <= 4)");
     f.scales = nullptr;
     if (!decode_kernel_applies(f, wbits, regime, (const uint32_t*)p->scale_zero_f16x2))
-      return set_error("woq_linear_grouped: the single-row kernel takes 4-bit weights in groups of 128 x 2^k, fp16 compute "
-                       "and K a multiple of 256");
+      return set_error("woq_linear_grouped: the integer-weight decode kernels take 4-bit weights in groups of 32, 64 or "
+                       "128 x 2^k, fp16 compute and K a multiple of 256");
     return launch_decode_grouped(f, (const MoeGroup*)group, slots, (hipStream_t)p->stream);
   }
   return launch_decode_dq_grouped(f, wbits, regime, (const MoeGroup*)group, slots, (hipStream_t)p->stream);

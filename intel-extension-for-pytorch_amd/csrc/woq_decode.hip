@@ -53,9 +53,34 @@ __device__ __forceinline__ f4 mfma16(u4 a, u4 b, f4 c) {
 // 4 g + m carries activation row m in the lane columns of group g only and zeros elsewhere (read from a zeroed LDS
 // slice), so lane column c accumulates the sums over group c alone for the four activation rows and applies that
 // group's (scale, zero) dword; the lane columns are added at the end.
-template <bool XF16, int NTW, int MAXM, bool ONE_ROUND, int GPT>
-__global__ __launch_bounds__(1024, 8) void woq_decode_kernel(const DecodeArgs a) {
+// GROUPED (mixture of experts): the workgroups with blockIdx.z = s serve slot s, up to four routed rows of one expert,
+// whose packed weight, (scale, zero) table and bias come from pointer tables in device memory; an empty slot exits.
+template <bool XF16, int NTW, int MAXM, bool ONE_ROUND, int GPT, bool GROUPED>
+__global__ __launch_bounds__(1024, 8) void woq_decode_kernel(const DecodeArgs a_in) {
   static_assert(GPT == 1 || GPT == 2 || GPT == 4, "groups of 128 x 2^k, 64 or 32");
+  DecodeArgs ag;
+  int64_t xr[MAXM];  // GROUPED: the rows of x that the slot's rows read
+  if constexpr (GROUPED) {
+    const MoeGroup& g = *a_in.grp;
+    const int slot = (int)blockIdx.z;
+    const int e = __builtin_amdgcn_readfirstlane(g.slot_expert[slot]);
+    if (e < 0) return;  // the whole workgroup, before anything is synchronized
+    const int64_t row0 = __builtin_amdgcn_readfirstlane(g.slot_row0[slot]);
+    const int rows = __builtin_amdgcn_readfirstlane(g.slot_rows[slot]);
+    ag = a_in;
+    ag.M = rows < MAXM ? rows : MAXM;
+    ag.qweight = dq_uniform((const uint8_t*)g.qweight[e]);
+    ag.sz = dq_uniform((const uint32_t*)g.scales[e]);
+    ag.bias = g.bias ? dq_uniform(g.bias[e]) : nullptr;
+    ag.out = (uint8_t*)a_in.out + row0 * a_in.N * 2;
+    if (a_in.other0) ag.other0 = (const uint8_t*)a_in.other0 + row0 * a_in.N * 2;
+#pragma unroll
+    for (int m = 0; m < MAXM; ++m) {
+      const int64_t row = row0 + (m < (int)ag.M ? m : (int)ag.M - 1);
+      xr[m] = g.x_row ? (int64_t)__builtin_amdgcn_readfirstlane((int)g.x_row[row]) : row;
+    }
+  }
+  const DecodeArgs& a = GROUPED ? ag : a_in;
   constexpr bool G32 = GPT > 1;  // the groups of a tile are kept apart
   static_assert(!G32 || MAXM == 4, "four activation rows times up to four groups fill the 16 rows of the A operand");
   constexpr int KPW = kDecodeKPW;
@@ -115,7 +140,7 @@ __global__ __launch_bounds__(1024, 8) void woq_decode_kernel(const DecodeArgs a)
     const uint8_t* xbase = (const uint8_t*)a.x + (size_t)ktw * kTileK4 * 2;  // uniform
 #pragma unroll
     for (int m = 0; m < MAXM; ++m) {
-      const int mm = m < M ? m : M - 1;
+      const int64_t mm = GROUPED ? xr[m] : (int64_t)(m < M ? m : M - 1);
       xs[m] = *(const u4*)(xbase + (size_t)mm * K * 2 + (uint32_t)xlane * 16u);
     }
 
@@ -460,25 +485,29 @@ static int launch_decode_m1_cfg(const DecodeArgs& a, hipStream_t st, int slots =
   return check_launch("woq_decode_m1_kernel");
 }
 
-template <bool XF16, int NTW, int MAXM, bool ONE_ROUND, int GPT>
-static int launch_decode_cfg_g(const DecodeArgs& a, hipStream_t st) {
+template <bool XF16, int NTW, int MAXM, bool ONE_ROUND, int GPT, bool GROUPED>
+static int launch_decode_cfg_g(const DecodeArgs& a, hipStream_t st, int slots) {
   const size_t smem = (size_t)NTW * a.W * 16 * sizeof(f4) +
                       (size_t)a.W * (MAXM + (GPT > 1 ? 1 : 0)) * kDecodeKPW * kTileK4 * sizeof(uint16_t);
-  auto kern = woq_decode_kernel<XF16, NTW, MAXM, ONE_ROUND, GPT>;
+  auto kern = woq_decode_kernel<XF16, NTW, MAXM, ONE_ROUND, GPT, GROUPED>;
   if (smem > 64 * 1024) {
     hipError_t err = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
     if (err != hipSuccess) return set_error("hipFuncSetAttribute: %s", hipGetErrorString(err));
   }
-  const unsigned grid = (unsigned)((a.NT + NTW - 1) / NTW);
+  const dim3 grid((unsigned)((a.NT + NTW - 1) / NTW), 1, (unsigned)(GROUPED ? slots : 1));
   kern<<<grid, a.W * 64, smem, st>>>(a);
   return check_launch("woq_decode_kernel");
 }
 
 template <bool XF16, int NTW, int MAXM, bool ONE_ROUND>
-static int launch_decode_cfg(const DecodeArgs& a, hipStream_t st) {
-  return a.G == 32   ? launch_decode_cfg_g<XF16, NTW, MAXM, ONE_ROUND, 4>(a, st)
-         : a.G == 64 ? launch_decode_cfg_g<XF16, NTW, MAXM, ONE_ROUND, 2>(a, st)
-                     : launch_decode_cfg_g<XF16, NTW, MAXM, ONE_ROUND, 1>(a, st);
+static int launch_decode_cfg(const DecodeArgs& a, hipStream_t st, int slots = 0) {
+  if (slots > 0)
+    return a.G == 32   ? launch_decode_cfg_g<XF16, NTW, MAXM, ONE_ROUND, 4, true>(a, st, slots)
+           : a.G == 64 ? launch_decode_cfg_g<XF16, NTW, MAXM, ONE_ROUND, 2, true>(a, st, slots)
+                       : launch_decode_cfg_g<XF16, NTW, MAXM, ONE_ROUND, 1, true>(a, st, slots);
+  return a.G == 32   ? launch_decode_cfg_g<XF16, NTW, MAXM, ONE_ROUND, 4, false>(a, st, 0)
+         : a.G == 64 ? launch_decode_cfg_g<XF16, NTW, MAXM, ONE_ROUND, 2, false>(a, st, 0)
+                     : launch_decode_cfg_g<XF16, NTW, MAXM, ONE_ROUND, 1, false>(a, st, 0);
 }
 
 bool decode_kernel_applies(const FpArgs& f, int wbits, int regime, const uint32_t* sz) {
@@ -497,7 +526,7 @@ int launch_decode(const FpArgs& f, const uint32_t* sz, hipStream_t st) { return 
 
 int launch_decode_grouped(const FpArgs& f, const MoeGroup* grp, int64_t slots, hipStream_t st) {
   if (!grp || slots < 1 || slots > 65535) return set_error("woq_linear_grouped: 1..65535 slots and a group table");
-  if (f.M != 1) return set_error("woq_linear_grouped: the single-row kernel takes one row per slot");
+  if (f.M < 1 || f.M > 4) return set_error("woq_linear_grouped: the integer-weight decode kernels take up to four rows per slot");
   return launch_decode_impl(f, nullptr, st, grp, (int)slots);
 }
 
@@ -546,7 +575,7 @@ static int launch_decode_impl(const FpArgs& f, const uint32_t* sz, hipStream_t s
 #undef WOQ_DECODE_M1
   }
 #define WOQ_DECODE(XF, NTW) \
-  (one_round ? launch_decode_cfg<XF, NTW, 4, true>(a, st) : launch_decode_cfg<XF, NTW, 4, false>(a, st))
+  (one_round ? launch_decode_cfg<XF, NTW, 4, true>(a, st, slots) : launch_decode_cfg<XF, NTW, 4, false>(a, st, slots))
   if (xf16) return two ? WOQ_DECODE(true, 2) : WOQ_DECODE(true, 1);
   return two ? WOQ_DECODE(false, 2) : WOQ_DECODE(false, 1);
 #undef WOQ_DECODE

@@ -725,16 +725,16 @@ class _MoeGroupedPlan:
             have = self.rows[dtype] = (mk(N1), mk(N1), mk(H))
         return have
 
-    def group_struct(self, linear, cls, f16_scales, gather):
-        """Device copy of the woq_hip_moe_group of one launch (built once).  Class 3: one slot per row, with the
-        (scale, zero) dword tables in place of the scales."""
-        key = (linear, cls, f16_scales, gather)
+    def group_struct(self, linear, cls, f16_scales, gather, sz=False):
+        """Device copy of the woq_hip_moe_group of one launch (built once).  ``sz``: for the integer-weight decode
+        kernels, with the (scale, zero) dword tables in place of the scales."""
+        key = (linear, cls, f16_scales, gather, sz)
         st = self.structs.get(key)
         if st is None:
             t = self.tables[linear]
             ptr = lambda x: 0 if x is None else x.data_ptr()
             tab = [ptr(self.slots[cls, i]) for i in range(3)] + [ptr(self.x_row) if gather else 0]
-            if cls == 3:
+            if sz:
                 fields = tab + [ptr(t["qweight"]), ptr(t["sz"]), 0, ptr(t["bias"])]
             else:
                 fields = tab + [ptr(t["qweight"]), ptr(t["s16"] if f16_scales else t["sb16"]), ptr(t["z8"]), ptr(t["bias"])]
@@ -778,10 +778,13 @@ def _deepseek_moe_grouped(hidden_states, topk_ids, gate_ctx, up_ctx, down_ctx, r
     if not plan.ok or plan.shapes[0]["K"] != H:
         return None
     lowp = plan.shapes[0]["lowp"]
-    split = 5 if lowp == 2 else 0  # lowp_mode BF16: experts with fewer than five rows compute in fp16
-    # (size class, bound on its slots' rows): an expert has at most T rows, so the larger classes are empty for small T
-    # experts with exactly one row (most of them in a layer with many experts and few tokens) on the single-row kernel
+    # experts with fewer than five rows on the integer-weight decode kernels, as woq_hip_linear serves them, where
+    # such rows compute in fp16 and the layer has the kernels' tables; those with exactly one row (most of them in a
+    # layer with many experts and few tokens) on the single-row kernel
     single = plan.single_row and _f16_regime(lowp, x.dtype, 1)
+    # lowp_mode BF16: experts with fewer than five rows compute in fp16, a class of their own
+    split = 5 if (lowp == 2 or single) else 0
+    # (size class, bound on its slots' rows): an expert has at most T rows, so the larger classes are empty for small T
     # a single token: every (token, slot) entry is a slot of its own (an expert named twice included)
     each = single and T == 1 and topk <= plan.S
     launches = [(3, 1)] if each else ([(3, 1)] if single else []) + ([(0, 4)] if split else []) + \
@@ -823,8 +826,9 @@ def _deepseek_moe_grouped(hidden_states, topk_ids, gate_ctx, up_ctx, down_ctx, r
             for cls, bound in launches:
                 p.M = bound
                 # (a non-null value tells the entry point that the group's scales are (scale, zero) dword tables)
-                p.scale_zero_f16x2 = plan.tables[li]["sz"].data_ptr() if cls == 3 else None
-                g = plan.group_struct(li, cls, _f16_regime(lowp, x.dtype, bound), gather)
+                sz = cls == 3 or (cls == 0 and single)
+                p.scale_zero_f16x2 = plan.tables[li]["sz"].data_ptr() if sz else None
+                g = plan.group_struct(li, cls, _f16_regime(lowp, x.dtype, bound), gather, sz)
                 _lib.check(lib.woq_hip_linear_grouped(ctypes.byref(p), g.data_ptr(), nslots), "woq_linear_grouped")
         _lib.check(lib.woq_hip_moe_combine_rows(out.data_ptr(), code, T, H, y.data_ptr(), rw.data_ptr(), topk,
                                                 plan.row_of.data_ptr(), plan.slot_of.data_ptr(), 0, stream), "moe_combine_rows")

@@ -702,20 +702,23 @@ def test_moe_route_with_a_slot_per_position(cuda):
 
 
 @pytest.mark.parametrize("G", [32, 64, 128])
-def test_deepseek_moe_grouped_single_token_is_the_per_expert_result(cuda, monkeypatch, G):
-    """One token: every expert it names has one row, which both paths give to the single-row decode kernel (groups of
-    32, 64 and 128): bit for bit."""
+@pytest.mark.parametrize("T,lowp", [(1, "BF16"), (3, "BF16"), (8, "BF16"), (16, "BF16"), (5, "FP16")])
+def test_deepseek_moe_grouped_is_the_per_expert_result_up_to_16_rows(cuda, monkeypatch, G, T, lowp):
+    """Experts with one row run the single-row decode kernel on both paths, those with two to four rows the other
+    integer-weight decode kernel, those with five to sixteen the dequantizing one (groups of 32, 64 and 128, K a
+    multiple of 256): bit for bit."""
     from ipex_amd import _lib
 
     ipex = _ipex()
     E, H, I, topk = 7, 512, 256, 4
-    mk = lambda k, n, s: _woq_module(ipex, k, n, "INT4", G, "BF16", bias=False, seed=s)
+    mk = lambda k, n, s: _woq_module(ipex, k, n, "INT4", G, lowp, bias=False, seed=s)
     ctxs = [[mk(H, I, 600 + 3 * e)._op_context for e in range(E)], [mk(H, I, 601 + 3 * e)._op_context for e in range(E)],
             [mk(I, H, 602 + 3 * e)._op_context for e in range(E)]]
-    g = torch.Generator().manual_seed(G)
-    hidden = torch.randn(1, H, generator=g).to(torch.bfloat16).to(cuda)
-    ids = torch.randperm(E, generator=g)[:topk].reshape(1, topk).to(cuda)
-    rw = torch.softmax(torch.randn(1, topk, generator=g), -1).to(torch.bfloat16).to(cuda)
+    g = torch.Generator().manual_seed(G + T)
+    xdt = torch.float16 if lowp == "FP16" else torch.bfloat16
+    hidden = torch.randn(T, H, generator=g).to(xdt).to(cuda)
+    ids = torch.stack([torch.randperm(E, generator=g)[:topk] for _ in range(T)]).to(cuda)
+    rw = torch.softmax(torch.randn(T, topk, generator=g), -1).to(xdt).to(cuda)
     op = torch.ops.torch_ipex.deepseek_moe_woq
     monkeypatch.setenv("IPEX_AMD_MOE_GROUPED", "0")
     want = op(hidden, ids, ctxs[0], ctxs[1], ctxs[2], rw, False)
