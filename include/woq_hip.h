@@ -242,7 +242,9 @@ typedef struct woq_hip_linear_params {
    * (1, 2), (2, 2), (4, 2), (2, 4), (4, 4): needs workspace and split_k_counters;
    * 19 / 20 = the prefill GEMM with 64 x 128 tiles and K shared by two / four workgroups per tile (same needs);
    * 21 = prefill GEMM that dequantizes each weight once per workgroup into an LDS tile (256 rows x 224 columns,
-   * 8 waves; 4-bit integer weights, otherwise the conditions of 3).
+   * 8 waves; 4-bit integer weights, otherwise the conditions of 3);
+   * 22 = the dequantizing decode kernel (M <= 32, INT4 / INT8 weights) with three weight row-blocks per workgroup,
+   * which need not divide the row-blocks.
    * NF4 weights: 0, 1, 2, 7, 8, 9, 13, 14, 16 only.
    * fp32 compute (lowp_mode NONE with fp32 activations, csrc/cpu/aten/kernels/WoqLinearKrnl.cpp:142-158;
    * also lowp_mode INT8 on fp32 activations) has one kernel of its own and takes 0 only */

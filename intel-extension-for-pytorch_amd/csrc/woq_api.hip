@@ -280,6 +280,11 @@ int woq_hip_linear(const woq_hip_linear_params* p) {
     // 7: row-blocks per workgroup and K splits by shape; 8..10: that many row-blocks, K not split
     return launch_decode_dq(f, wbits, regime, st, kernel == 10 ? 4 : kernel - 7, kernel == 7 ? 0 : 1, &scratch);
   }
+  if (kernel == 22) {  // three row-blocks per workgroup (they need not divide the row-blocks), K not split
+    if (!decode_dq_applies(f, wbits, regime))
+      return set_error("woq_linear: the dequantizing decode kernel does not take this problem");
+    return launch_decode_dq(f, wbits, regime, st, 3, 1, &scratch);
+  }
   if (kernel >= 13 && kernel <= 17) {
     static const int kNtw[5] = {1, 2, 4, 2, 4}, kSplits[5] = {2, 2, 2, 4, 4};
     if (!decode_dq_applies(f, wbits, regime))

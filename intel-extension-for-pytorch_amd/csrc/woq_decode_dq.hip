@@ -174,9 +174,12 @@ __global__ __launch_bounds__(512, 4) void woq_decode_dq_kernel(const DecodeDqArg
   const uint8_t* zbase[NTW];
 #pragma unroll
   for (int t = 0; t < NTW; ++t) {
-    wbase[t] = f.qweight + (size_t)(nt0 + t) * KT * kTileBytes;
-    sbase[t] = (const uint8_t*)(f.scales + (size_t)(nt0 + t) * KG * kTileN);
-    zbase[t] = has_z ? f.zeros + (size_t)(nt0 + t) * KG * kTileN : sbase[t];
+    // three row-blocks per workgroup need not divide the row-blocks: the last workgroup reads its
+    // missing ones from the last real row-block, and the store below drops their columns (n >= N)
+    const int64_t nt = nt0 + t < f.NT ? nt0 + t : f.NT - 1;
+    wbase[t] = f.qweight + (size_t)nt * KT * kTileBytes;
+    sbase[t] = (const uint8_t*)(f.scales + (size_t)nt * KG * kTileN);
+    zbase[t] = has_z ? f.zeros + (size_t)nt * KG * kTileN : sbase[t];
   }
 
   u4 wnext[NTW];
@@ -360,7 +363,7 @@ static int launch_dq_cfg(DecodeDqArgs a, int splits, hipStream_t st, int slots =
   // four row tiles (33..64 rows) a wave's two buffers are 32 KiB and one workgroup of four waves takes
   // 128 KiB.  Sixteen waves of one row tile measured no faster than eight.
   constexpr int kLdsMax = 131072;
-  const dim3 grid((unsigned)(a.f.NT / NTW), (unsigned)splits, (unsigned)slots);
+  const dim3 grid((unsigned)((a.f.NT + NTW - 1) / NTW), (unsigned)splits, (unsigned)slots);
   const bool alone = MT == 2 && grid.x * grid.y <= 256;
   const int lds_cap = (MT > 2 || alone) ? kLdsMax : 65536;
   const int max_w = lds_cap / (2 * Geo::SLICE);
@@ -401,16 +404,28 @@ static int launch_dq_regime(const DecodeDqArgs& a, int ntw, int splits, hipStrea
   if constexpr (REGIME == kRegimeF16) {
     if (a.f.x_dtype == WOQ_HIP_ACT_BF16) {  // one row tile, rows converted to fp16 on the way in
       if (ntw == 4) return launch_dq_cfg<REGIME, WBITS, 1, 4, false, true, FP8>(a, splits, st);
+      if (ntw == 3) {
+        if constexpr (FP8)
+          return set_error("woq_decode_dq_kernel: FP8 weights take 1, 2 or 4 row-blocks per workgroup");
+        else
+          return launch_dq_cfg<REGIME, WBITS, 1, 3, false, true>(a, splits, st);
+      }
       if (ntw == 2) return launch_dq_cfg<REGIME, WBITS, 1, 2, false, true, FP8>(a, splits, st);
       return launch_dq_cfg<REGIME, WBITS, 1, 1, false, true, FP8>(a, splits, st);
     }
   }
   if (mt == 4) {
     // 33..64 rows: one or two row-blocks per workgroup (four would leave too few workgroups)
-    if (ntw == 4) return set_error("woq_decode_dq_kernel: 33..64 rows take 1 or 2 row-blocks per workgroup");
+    if (ntw > 2) return set_error("woq_decode_dq_kernel: 33..64 rows take 1 or 2 row-blocks per workgroup");
     return ntw == 2 ? launch_dq_cfg<REGIME, WBITS, 4, 2, false, false, FP8>(a, splits, st) : launch_dq_cfg<REGIME, WBITS, 4, 1, false, false, FP8>(a, splits, st);
   }
   const bool two_rows = mt == 2;
+  if (ntw == 3) {
+    if constexpr (FP8)
+      return set_error("woq_decode_dq_kernel: FP8 weights take 1, 2 or 4 row-blocks per workgroup");
+    else
+      return two_rows ? launch_dq_cfg<REGIME, WBITS, 2, 3>(a, splits, st) : launch_dq_cfg<REGIME, WBITS, 1, 3>(a, splits, st);
+  }
   if (ntw == 4) return two_rows ? launch_dq_cfg<REGIME, WBITS, 2, 4, false, false, FP8>(a, splits, st) : launch_dq_cfg<REGIME, WBITS, 1, 4, false, false, FP8>(a, splits, st);
   if (ntw == 2) return two_rows ? launch_dq_cfg<REGIME, WBITS, 2, 2, false, false, FP8>(a, splits, st) : launch_dq_cfg<REGIME, WBITS, 1, 2, false, false, FP8>(a, splits, st);
   return two_rows ? launch_dq_cfg<REGIME, WBITS, 2, 1, false, false, FP8>(a, splits, st) : launch_dq_cfg<REGIME, WBITS, 1, 1, false, false, FP8>(a, splits, st);
@@ -491,18 +506,26 @@ int launch_decode_dq(const FpArgs& f, int wbits, int regime, hipStream_t st, int
     a.g_shift = 0;
     while (((int64_t)1 << a.g_shift) < f.G) ++a.g_shift;
   }
-  if (ntw != 0 && ntw != 1 && ntw != 2 && ntw != 4)
-    return set_error("woq_decode_dq_kernel: 1, 2 or 4 row-blocks per workgroup, got %d", ntw);
-  if (ntw != 0 && f.NT % ntw != 0)
+  if (ntw < 0 || ntw > 4)
+    return set_error("woq_decode_dq_kernel: 1 to 4 row-blocks per workgroup, got %d", ntw);
+  if (ntw == 3 && splits > 1) return set_error("woq_decode_dq_kernel: three row-blocks per workgroup run unsplit");
+  if (ntw != 0 && ntw != 3 && f.NT % ntw != 0)
     return set_error("woq_decode_dq_kernel: %d row-blocks per workgroup do not divide %lld", ntw, (long long)f.NT);
   // More row-blocks per workgroup re-read the activations less often (every workgroup streams all
   // of x through LDS); fewer make more workgroups, which small N needs to fill the chip.  Measured at
   // M = 16 / 32: 4096 -> 14336 (896 row-blocks) 14.4 / 11.4 / 10.7 us with 1 / 2 / 4, 4096 -> 6144 (384)
   // 8.5 / 7.0 / 9.7 us, 14336 -> 4096 (256) 12.9 / 15.5 / 24.5 us.  33..64 rows (four row tiles, no
   // variant with four row-blocks) have four times the activation bytes per workgroup.
+  // Between 513 and 768 row-blocks neither two nor four per workgroup fill the 256 CUs (two: a second,
+  // partial round of workgroups; four: 129..192 workgroups), three do: 4096 -> 11008 (688 row-blocks) INT4
+  // G = 128 at M = 8 / 16 / 32 takes 8.4 / 8.8 / 10.8 us against 9.9 / 10.2 / 12.5 us with four (INT8 per
+  // channel at M = 32: 12.8 against 14.5 us), 4096 -> 8704 at M = 32 10.5 us against 13.7 us with two; at 832
+  // row-blocks three make 278 workgroups and lose (17.3 against 12.7 us).
   const bool auto_ntw = ntw == 0;
   if (ntw == 0) {
-    if (f.M <= 32 && !f.nf4 && f.NT >= 640 && f.NT % 4 == 0)
+    if (f.M <= 32 && !f.nf4 && !f.fp8 && f.NT > 512 && f.NT <= 768)
+      ntw = 3;
+    else if (f.M <= 32 && !f.nf4 && f.NT >= 640 && f.NT % 4 == 0)
       ntw = 4;
     else
       ntw = (f.NT >= 384 && f.NT % 2 == 0) ? 2 : 1;
@@ -537,7 +560,7 @@ int launch_decode_dq(const FpArgs& f, int wbits, int regime, hipStream_t st, int
   if (f.nf4) {
     if (wbits != 4 || f.zeros) return set_error("woq_decode_dq_kernel: NF4 weights are 4-bit and symmetric");
 
-    if (ntw == 4) return set_error("woq_decode_dq_kernel: NF4 weights take 1 or 2 row-blocks per workgroup");
+    if (ntw > 2) return set_error("woq_decode_dq_kernel: NF4 weights take 1 or 2 row-blocks per workgroup");
     return regime == kRegimeF16 ? launch_dq_nf4<kRegimeF16>(a, ntw, splits, st)
                                 : launch_dq_nf4<kRegimeBF16>(a, ntw, splits, st);
   }

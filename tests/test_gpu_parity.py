@@ -420,9 +420,9 @@ def test_w4_prefill_kernel_with_the_tile_in_lds(cuda):
         (3, 256, 80, 256, True),  # bf16 regime is forced below by lowp NONE
     ],
 )
-@pytest.mark.parametrize("kernel", [7, 8, 9, 10])  # automatic, then 1 / 2 / 4 row-blocks per workgroup
+@pytest.mark.parametrize("kernel", [7, 8, 9, 10, 22])  # automatic, then 1 / 2 / 4 / 3 row-blocks per workgroup
 def test_dequantizing_decode_kernel(cuda, M, K, N, G, bias, kernel):
-    ntw = {7: 1, 8: 1, 9: 2, 10: 4}[kernel]
+    ntw = {7: 1, 8: 1, 9: 2, 10: 4, 22: 1}[kernel]  # three need not divide the row-blocks
     if (N // 16) % ntw:
         pytest.skip("row-blocks per workgroup must divide N / 16")
     case = _synthetic().make_int4_case(24, M, K, N, G, bias=bias)
@@ -431,7 +431,7 @@ def test_dequantizing_decode_kernel(cuda, M, K, N, G, bias, kernel):
 
 
 @pytest.mark.parametrize("M", [1, 7, 16, 17, 32])
-@pytest.mark.parametrize("kernel", [7, 9, 10])
+@pytest.mark.parametrize("kernel", [7, 9, 10, 22])
 def test_dequantizing_decode_kernel_int8_weights(cuda, M, kernel):
     """8-bit weights (64 K values per tile) and two row tiles (M > 16)."""
     case = _synthetic().make_int8_case(33, M, 704, 128)  # 11 K tiles: a partial last round
@@ -454,12 +454,26 @@ def test_dequantizing_decode_kernel_four_row_tiles(cuda, M, K, N, G, bias, kerne
     _check_fp(case, O.LOWP_BF16, force_kernel=kernel, label=f"decode dq int4 M={M} K={K} N={N} G={G} kernel={kernel}")
 
 
+@pytest.mark.parametrize("M,N,G", [(6, 8200, 128), (16, 11008, -1), (17, 8208, 64), (32, 12288, 128)])
+def test_dequantizing_decode_kernel_three_row_blocks_by_shape(cuda, M, N, G):
+    """513..768 row-blocks: the automatic choice is three per workgroup, whose last workgroup may hold
+    fewer (8200 columns: 513 row-blocks, the last one partial); the forced form gives the same bits."""
+    case = _synthetic().make_int4_case(58, M, 256, N, G, bias=True)
+    _check_fp(case, O.LOWP_BF16, label=f"decode dq three row-blocks M={M} N={N} G={G}")
+    ctx = make_context(case, O.LOWP_BF16)
+    x = case["x"].cuda()
+    assert torch.equal(ctx.run(x), ctx.run(x, force_kernel=22))
+    assert _lib_last_kernel() == "woq_decode_dq_kernel"
+
+
 def test_dequantizing_decode_kernel_four_row_tiles_int8_weights_and_rejections(cuda):
     case = _synthetic().make_int8_case(36, 48, 704, 128)
     _check_fp(case, O.LOWP_BF16, force_kernel=7, label="decode dq int8 weights M=48")
     ctx = make_context(case, O.LOWP_BF16)
     with pytest.raises(RuntimeError, match="row-blocks"):
         ctx.run(case["x"].cuda(), force_kernel=10)
+    with pytest.raises(RuntimeError, match="row-blocks"):
+        ctx.run(case["x"].cuda(), force_kernel=22)
     nf4 = _synthetic().make_nf4_case(37, 40, 512, 64, 128)
     for kernel in (0, 7, 8, 9, 1):  # four row tiles of NF4 codes, then the small-M kernel
         _check_fp(nf4, O.LOWP_BF16, force_kernel=kernel, label=f"nf4 M=40 kernel={kernel}")
@@ -473,12 +487,12 @@ def test_dequantizing_decode_kernel_four_row_tiles_int8_weights_and_rejections(c
     [(1, 1024, 64, 32, False), (2, 4096, 1024, 64, True), (4, 1152, 96, -1, True), (3, 512, 128, 32, False),
      (4, 256, 64, 256, True)],
 )
-@pytest.mark.parametrize("kernel", [0, 8, 9, 10, 13, 14])
+@pytest.mark.parametrize("kernel", [0, 8, 9, 10, 13, 14, 22])
 def test_dequantizing_decode_kernel_bf16_rows_under_fp16_compute(cuda, M, K, N, G, bias, kernel):
     """lowp_mode BF16 with fewer than five bf16 rows computes in fp16 (the reference converts the rows
     per K block): group sizes the integer-weight decode kernel does not take go through this kernel,
     which converts the rows on the way into LDS."""
-    ntw = {0: 1, 8: 1, 9: 2, 10: 4, 13: 1, 14: 2}[kernel]
+    ntw = {0: 1, 8: 1, 9: 2, 10: 4, 13: 1, 14: 2, 22: 1}[kernel]
     if (N // 16) % ntw:
         pytest.skip("row-blocks per workgroup must divide N / 16")
     case = _synthetic().make_int4_case(54, M, K, N, G, bias=bias)
