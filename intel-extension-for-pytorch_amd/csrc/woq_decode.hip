@@ -552,7 +552,11 @@ static int launch_decode_impl(const FpArgs& f, const uint32_t* sz, hipStream_t s
   }
   a.W = (int)w;
   const bool xf16 = f.x_dtype == WOQ_HIP_ACT_FP16;
-  const bool two = f.NT >= 512 && f.NT % 2 == 0;
+  // Two row-blocks per workgroup from 512 row-blocks on; a single row only above 768: up to there one
+  // row-block per workgroup spreads more evenly over the 256 CUs (M = 1: 8192 -> 10240 9.6 us against
+  // 11.7 us, 4096 -> 8192 5.2 against 5.4 us, 4096 -> 11008 6.5 against 6.7 us; 4096 -> 14336 the other
+  // way round, 7.1 against 7.8 us; M = 4, 4096 -> 11008: 7.4 us with two against 7.7 us).
+  const bool two = f.NT % 2 == 0 && (f.M == 1 ? f.NT > 768 : f.NT >= 512);
   a.wbytes = (uint32_t)(f.NT * f.KT * kTileBytes);  // below 4 GiB (decode_kernel_applies)
   a.szbytes = (uint32_t)(f.NT * f.KG * kTileN * (int64_t)sizeof(uint32_t));
   const bool one_row = f.M == 1;
