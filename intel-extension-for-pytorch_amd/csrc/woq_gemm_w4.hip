@@ -585,7 +585,13 @@ int launch_gemm_w4(const FpArgs& f, int wbits, int regime, hipStream_t st, int s
                                 : launch_shape<kRegimeBF16, S42>(f, g_shift, st, splits, scratch);
   }
   if (splits > 1) return set_error("woq_gemm_w4_kernel: K is split for the 64 x 128 shape only");
-  const double c7 = shape_cost<S7>(f), c4 = shape_cost<S4>(f), c2 = shape_cost<S2>(f);
+  const double c7 = shape_cost<S7>(f), c4 = shape_cost<S4>(f);
+  // 128 x 128 tiles of 4-bit weights: two workgroups share a CU, so beyond two generations the CUs stay
+  // evenly loaded (fractional generations), and a generation measured 0.53 of a 128 x 256 one (37 against
+  // 70 us at K = 4096).  M = 1024, 4096 -> 11008 (688 workgroups): 101 us against 124 us with 128 x 448
+  // tiles (200 workgroups); M = 1024 / 2048, 8192 -> 10240: 180 / 313 us against 207 / 329 us.
+  const double wgs2 = (double)((f.NT * kTileN + S2::BN - 1) / S2::BN) * (double)((f.M + S2::BM - 1) / S2::BM);
+  const double c2 = wgs2 <= 512 ? shape_cost<S2>(f) : wgs2 / 256.0 * 2.7;
   if (shape == 0) {
     shape = (c7 <= c4 && c7 <= c2) ? 7 : (c4 <= c2 ? 4 : 2);
     const int64_t wgs_t = ((f.NT * kTileN + ST::BN - 1) / ST::BN) * ((f.M + ST::BM - 1) / ST::BM);
