@@ -454,6 +454,20 @@ def test_dequantizing_decode_kernel_four_row_tiles(cuda, M, K, N, G, bias, kerne
     _check_fp(case, O.LOWP_BF16, force_kernel=kernel, label=f"decode dq int4 M={M} K={K} N={N} G={G} kernel={kernel}")
 
 
+@pytest.mark.parametrize("M,N,G", [(16, 4112, 128), (40, 4650, 32), (9, 10256, -1), (20, 13000, 64)])
+def test_dequantizing_decode_kernel_row_blocks_that_do_not_divide(cuda, M, N, G):
+    """The automatic choice of two (above 256 row-blocks) or four (from 640) row-blocks per workgroup with a
+    count of row-blocks they do not divide: 257, 291, 641 and 813."""
+    case = _synthetic().make_int4_case(59, M, 256, N, G, bias=True)
+    _check_fp(case, O.LOWP_BF16, label=f"decode dq ragged row-blocks M={M} N={N} G={G}")
+    assert _lib_last_kernel() == "woq_decode_dq_kernel"
+    # one row-block per workgroup gives the same bits while the waves per workgroup agree (one or four row tiles)
+    if M <= 16:
+        ctx = make_context(case, O.LOWP_BF16)
+        x = case["x"].cuda()
+        assert torch.equal(ctx.run(x), ctx.run(x, force_kernel=8))
+
+
 @pytest.mark.parametrize("M,N,G", [(6, 8200, 128), (16, 11008, -1), (17, 8208, 64), (32, 12288, 128)])
 def test_dequantizing_decode_kernel_three_row_blocks_by_shape(cuda, M, N, G):
     """513..768 row-blocks: the automatic choice is three per workgroup, whose last workgroup may hold
