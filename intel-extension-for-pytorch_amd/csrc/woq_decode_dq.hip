@@ -516,20 +516,32 @@ int launch_decode_dq(const FpArgs& f, int wbits, int regime, hipStream_t st, int
   // M = 16 / 32: 4096 -> 14336 (896 row-blocks) 14.4 / 11.4 / 10.7 us with 1 / 2 / 4, 4096 -> 6144 (384)
   // 8.5 / 7.0 / 9.7 us, 14336 -> 4096 (256) 12.9 / 15.5 / 24.5 us.  33..64 rows (four row tiles, no
   // variant with four row-blocks) have four times the activation bytes per workgroup.
-  // Between 513 and 768 row-blocks neither two nor four per workgroup fill the 256 CUs (two: a second,
-  // partial round of workgroups; four: 129..192 workgroups), three do: 4096 -> 11008 (688 row-blocks) INT4
-  // G = 128 at M = 8 / 16 / 32 takes 8.4 / 8.8 / 10.8 us against 9.9 / 10.2 / 12.5 us with four (INT8 per
-  // channel at M = 32: 12.8 against 14.5 us), 4096 -> 8704 at M = 32 10.5 us against 13.7 us with two; at 832
-  // row-blocks three make 278 workgroups and lose (17.3 against 12.7 us).
+  // Up to 32 rows: the count with the shortest schedule -- generations of 256 workgroups (one per CU and
+  // round; a second workgroup on a CU shares its vector pipes) times a workgroup's length, which is its
+  // row-blocks plus a fixed part for streaming the activations (about half a row-block's worth, from the
+  // 1 / 2 / 4 figures above); ties go to the larger count.  That gives 1 up to 256 row-blocks, 2 up to 512
+  // (288 row-blocks, M = 16 / 32: 6.9 / 8.4 us against 8.3 / 10.9 us with one), 3 up to 768 (4096 -> 11008, 688
+  // row-blocks: INT4 G = 128 at M = 8 / 16 / 32 8.4 / 8.8 / 10.8 us against 9.9 / 10.2 / 12.5 us with four, INT8
+  // per channel at M = 32 12.8 against 14.5 us), 4 up to 1024 (at 832 row-blocks three make 278 workgroups
+  // and lose, 17.3 against 12.7 us), then whichever of 3 and 4 wastes less of the last generation (1376
+  // row-blocks: three).  A count that does not divide the row-blocks is fine: the last workgroup repeats
+  // the last row-block.
   const bool auto_ntw = ntw == 0;
   if (ntw == 0) {
-    if (f.M <= 32 && !f.nf4 && !f.fp8 && f.NT > 512 && f.NT <= 768)
-      ntw = 3;
-    else if (f.M <= 32 && !f.nf4 && f.NT >= 640)
-      ntw = 4;
-    else
-      ntw = f.NT > 256 ? 2 : 1;  // 288 row-blocks, M = 16 / 32 / 64: 6.9 / 8.4 / 13.9 us against 8.3 / 10.9 / 20.6 us with one
-    // (a count that does not divide the row-blocks is fine here: the last workgroup repeats the last row-block)
+    if (f.M <= 32 && !f.nf4) {
+      double best = 0.0;
+      for (int cand = 1; cand <= 4; ++cand) {
+        if (cand == 3 && f.fp8) continue;  // no such instances
+        const int64_t wgs = (f.NT + cand - 1) / cand;
+        const double cost = (double)((wgs + 255) / 256) * (cand * 1.9 + 1.0);
+        if (ntw == 0 || cost <= best) {
+          best = cost;
+          ntw = cand;
+        }
+      }
+    } else {
+      ntw = f.NT > 256 ? 2 : 1;  // 288 row-blocks, M = 64: 13.9 us against 20.6 us with one
+    }
   }
   // Few output columns and a long K: one row-block per workgroup fills the chip but re-reads the
   // activations once per 16 columns.  Two workgroups per row-block set, each with half of the K tiles
