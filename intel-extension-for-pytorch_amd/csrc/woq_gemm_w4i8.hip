@@ -897,7 +897,8 @@ int launch_gemm_w4i8(const Int8Args& a, const uint8_t* xq, int64_t ldq, const fl
     // (up to four rows: only above 768 row-blocks; below, single row-blocks spread more evenly over the
     // CUs -- M = 1 with its activation quantization, 4096 -> 11008: 8.9 against 10.1 us, 8192 -> 10240: 13.8
     // against 15.3 us; 16 and 32 rows measured the same either way)
-    const int ntw = (gsub * mt <= 2 && a.NT >= (a.M <= 4 ? 769 : 512) && a.NT % 2 == 0) ? 2 : 1;
+    // (17..32 rows: from 258 row-blocks on -- 288..512 row-blocks at M = 32: 10.5-10.9 us against 11.6-12.0 us)
+    const int ntw = (gsub * mt <= 2 && a.NT >= (a.M <= 4 ? 769 : a.M > 16 ? 258 : 512) && a.NT % 2 == 0) ? 2 : 1;
     const int slice = mt * 16 * kTileK4;
     int w = 65536 / (2 * slice);  // at most 64 KiB of activation slices
     if (w > 8) w = 8;

@@ -1136,7 +1136,7 @@ def test_int8_lowp_other_groups(cuda, G, M):
 @pytest.mark.parametrize("mode", [4, 5, 6, 7])
 @pytest.mark.parametrize("M,K,N,G", [(17, 1024, 272, 128), (32, 2048, 1040, 64), (9, 512, 144, 32), (16, 1152, 96, -1),
                                      (25, 1024, 8208, 256), (2, 384, 48, 64), (30, 1024, 272, 32), (64, 512, 144, 64),
-                                     (41, 1024, 96, 64)])
+                                     (41, 1024, 96, 64), (20, 512, 4128, 128), (1, 512, 8224, 128), (4, 256, 12320, -1)])
 def test_int8_lowp_decode_kernel(cuda, mode, M, K, N, G):
     """The int8 MFMA decode kernel: one or two row tiles, groups of 32 / 64 as K blocks inside a tile,
     two row-blocks per workgroup for wide layers; the general kernel (debug run) supplies the bit-exact
