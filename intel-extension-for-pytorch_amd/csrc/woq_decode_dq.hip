@@ -89,7 +89,7 @@ struct G8Consts {
 // case of a bf16 model under lowp_mode BF16 with fewer than five rows.  The rows then travel through
 // registers (16-byte loads, conversion, ds_write to the same swizzled places) instead of the LDS DMA.
 template <int REGIME, int WBITS, int MT, int NTW, bool NF4, bool XCONV, bool FP8, bool GROUPED>
-__global__ __launch_bounds__(512, 4) void woq_decode_dq_kernel(const DecodeDqArgs a) {
+__global__ __launch_bounds__(512, (MT * NTW > 8 ? 2 : 4)) void woq_decode_dq_kernel(const DecodeDqArgs a) {
   static_assert(!XCONV || (REGIME == kRegimeF16 && MT == 1), "bf16 -> fp16 rows: fp16 regime, one row tile");
   using Geo = DqGeom<WBITS, MT>;
   constexpr int TK = Geo::TK, NJ = Geo::NJ, NX = Geo::NX, SLICE = Geo::SLICE;
@@ -415,8 +415,13 @@ static int launch_dq_regime(const DecodeDqArgs& a, int ntw, int splits, hipStrea
     }
   }
   if (mt == 4) {
-    // 33..64 rows: one or two row-blocks per workgroup (four would leave too few workgroups)
-    if (ntw > 2) return set_error("woq_decode_dq_kernel: 33..64 rows take 1 or 2 row-blocks per workgroup");
+    // 33..64 rows: one, two or (integer weights: 16 accumulator tiles, so two waves per SIMD at most, which
+    // is what the 128 KiB of activation buffers of four waves allow anyway) four row-blocks per workgroup
+    if (ntw == 3 || (ntw == 4 && FP8))
+      return set_error("woq_decode_dq_kernel: 33..64 rows take 1, 2 or (integer weights) 4 row-blocks per workgroup");
+    if constexpr (!FP8) {
+      if (ntw == 4) return launch_dq_cfg<REGIME, WBITS, 4, 4>(a, splits, st);
+    }
     return ntw == 2 ? launch_dq_cfg<REGIME, WBITS, 4, 2, false, false, FP8>(a, splits, st) : launch_dq_cfg<REGIME, WBITS, 4, 1, false, false, FP8>(a, splits, st);
   }
   const bool two_rows = mt == 2;
@@ -534,6 +539,18 @@ int launch_decode_dq(const FpArgs& f, int wbits, int regime, hipStream_t st, int
         if (cand == 3 && f.fp8) continue;  // no such instances
         const int64_t wgs = (f.NT + cand - 1) / cand;
         const double cost = (double)((wgs + 255) / 256) * (cand * 1.9 + 1.0);
+        if (ntw == 0 || cost <= best) {
+          best = cost;
+          ntw = cand;
+        }
+      }
+    } else if (f.M > 32 && !f.nf4 && !f.fp8) {
+      // four row tiles: streaming 33..64 activation rows is the larger part of a workgroup's time (256
+      // workgroups of one / two row-blocks at M = 64: 11.7 / 14.3 us), so the same rule with that fixed part
+      double best = 0.0;
+      for (int cand = 1; cand <= 4; cand *= 2) {
+        const int64_t wgs = (f.NT + cand - 1) / cand;
+        const double cost = (double)((wgs + 255) / 256) * (cand * 2.5 + 7.0);
         if (ntw == 0 || cost <= best) {
           best = cost;
           ntw = cand;

@@ -447,14 +447,16 @@ def test_dequantizing_decode_kernel_two_row_tiles_int4(cuda, M, K, N, G):
 
 @pytest.mark.parametrize("M,K,N,G,bias", [(33, 1024, 96, 128, True), (64, 2048, 544, 32, False), (50, 384, 96, -1, True),
                                           (64, 512, 768, 128, False)])
-@pytest.mark.parametrize("kernel", [0, 8, 9])  # automatic, then one / two row-blocks per workgroup
+@pytest.mark.parametrize("kernel", [0, 8, 9, 10])  # automatic, then one / two / four row-blocks per workgroup
 def test_dequantizing_decode_kernel_four_row_tiles(cuda, M, K, N, G, bias, kernel):
     """33..64 rows: four row tiles per wave, 128 KiB of activation buffers per workgroup."""
+    if kernel == 10 and (N // 16) % 4:
+        pytest.skip("row-blocks per workgroup must divide N / 16")
     case = _synthetic().make_int4_case(35, M, K, N, G, bias=bias)
     _check_fp(case, O.LOWP_BF16, force_kernel=kernel, label=f"decode dq int4 M={M} K={K} N={N} G={G} kernel={kernel}")
 
 
-@pytest.mark.parametrize("M,N,G", [(16, 4112, 128), (40, 4650, 32), (9, 10256, -1), (20, 13000, 64)])
+@pytest.mark.parametrize("M,N,G", [(16, 4112, 128), (40, 4650, 32), (9, 10256, -1), (20, 13000, 64), (50, 9232, 128)])
 def test_dequantizing_decode_kernel_row_blocks_that_do_not_divide(cuda, M, N, G):
     """The automatic choice of two (above 256 row-blocks) or four (from 640) row-blocks per workgroup with a
     count of row-blocks they do not divide: 257, 291, 641 and 813."""
@@ -483,11 +485,13 @@ def test_dequantizing_decode_kernel_three_row_blocks_by_shape(cuda, M, N, G):
 def test_dequantizing_decode_kernel_four_row_tiles_int8_weights_and_rejections(cuda):
     case = _synthetic().make_int8_case(36, 48, 704, 128)
     _check_fp(case, O.LOWP_BF16, force_kernel=7, label="decode dq int8 weights M=48")
+    _check_fp(case, O.LOWP_BF16, force_kernel=10, label="decode dq int8 weights M=48, four row-blocks per workgroup")
     ctx = make_context(case, O.LOWP_BF16)
     with pytest.raises(RuntimeError, match="row-blocks"):
-        ctx.run(case["x"].cuda(), force_kernel=10)
-    with pytest.raises(RuntimeError, match="row-blocks"):
         ctx.run(case["x"].cuda(), force_kernel=22)
+    fp8 = _synthetic().make_fp8_case(36, 48, 512, 128, bias=False, group_size=128)
+    with pytest.raises(RuntimeError, match="row-blocks"):
+        make_context(fp8, O.LOWP_BF16).run(fp8["x"].cuda(), force_kernel=10)
     nf4 = _synthetic().make_nf4_case(37, 40, 512, 64, 128)
     for kernel in (0, 7, 8, 9, 1):  # four row tiles of NF4 codes, then the small-M kernel
         _check_fp(nf4, O.LOWP_BF16, force_kernel=kernel, label=f"nf4 M=40 kernel={kernel}")
