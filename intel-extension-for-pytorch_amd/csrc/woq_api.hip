@@ -268,11 +268,11 @@ int woq_hip_linear(const woq_hip_linear_params* p) {
   }
   if (kernel == 0 && decode_kernel_applies(f, wbits, regime, p->scale_zero_f16x2))
     return launch_decode(f, p->scale_zero_f16x2, st);
-  // 33..64 rows: the decode kernel with four row tiles, except for very wide layers, where the
-  // prefill kernel's activation reuse wins (M = 64, 4096 -> 14336: 27 us against 37 us and 58 us for the
-  // small-M kernel; 4096 -> 28672: 51 us against 42 us)
+  // 33..64 rows: the decode kernel with four row tiles while its workgroups of four row-blocks fit one
+  // generation (up to 1024 row-blocks), the prefill kernel's 64 x 128 tiles beyond (M = 64, 4096 -> 14336 /
+  // 16384: 20.7 / 21.2 us against 29 us; 4096 -> 22016 / 28672: 38.5 / 39.3 us against 29.7 / 30.9 us)
   const bool w4 = gemm_w4_applies(f, wbits, regime);
-  if (kernel == 0 && decode_dq_applies(f, wbits, regime) && !(p->M > 32 && w4 && p->N >= 16384)) kernel = 7;
+  if (kernel == 0 && decode_dq_applies(f, wbits, regime) && !(p->M > 32 && w4 && p->N > 16384)) kernel = 7;
   if (kernel >= 7 && kernel <= 10) {
     if (!decode_dq_applies(f, wbits, regime))
       return set_error("woq_linear: the dequantizing decode kernel takes M <= 64, K a multiple of the weight tile, a "
