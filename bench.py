@@ -60,6 +60,7 @@ def build_params(lib_mod, x, ctx, out, lowp_mode, act_quant_mode=-1, workspace=N
     p.scales_bf16 = ctx.scales_list_[2].data_ptr()
     p.zeros_u8 = ctx.zeros_u8_.data_ptr() if ctx.zeros_u8_ is not None else None
     p.scale_zero_f16x2 = ctx.scale_zero_f16x2_.data_ptr() if ctx.scale_zero_f16x2_ is not None else None
+    p.scale_zero_bf16 = ctx.scale_zero_bf16_.data_ptr() if ctx.scale_zero_bf16_ is not None else None
     p.group_size = ctx.group_size_
     p.bias = ctx.bias_f32_.data_ptr() if ctx.bias_f32_ is not None else None
     p.lowp_mode = lowp_mode
@@ -211,6 +212,7 @@ def _rotating_params(torch, lib_mod, ops_mod, case, lowp_mode, dev, stream, min_
             c.scales_list_ = [t.clone() for t in ctx0.scales_list_]
             c.zeros_u8_ = None if ctx0.zeros_u8_ is None else ctx0.zeros_u8_.clone()
             c.scale_zero_f16x2_ = None if ctx0.scale_zero_f16x2_ is None else ctx0.scale_zero_f16x2_.clone()
+            c.scale_zero_bf16_ = None if ctx0.scale_zero_bf16_ is None else ctx0.scale_zero_bf16_.clone()
         keep.append(c)
         p = build_params(lib_mod, x, c, out, lowp_mode, act_quant_mode, ws)
         p.stream = stream.cuda_stream
@@ -618,6 +620,7 @@ def main():
             c.scales_list_ = [t.clone() for t in ctx0.scales_list_]
             c.zeros_u8_ = ctx0.zeros_u8_.clone()
             c.scale_zero_f16x2_ = ctx0.scale_zero_f16x2_.clone()
+            c.scale_zero_bf16_ = None if ctx0.scale_zero_bf16_ is None else ctx0.scale_zero_bf16_.clone()
         keep.append(c)
         p = build_params(_lib, x, c, out, 2)
         p.stream = stream.cuda_stream

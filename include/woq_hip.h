@@ -157,11 +157,18 @@ int woq_hip_unpack_weight(const void* packed, int weight_dtype, int64_t N, int64
  *   scale_zero_f16x2 (may be NULL): one dword per (row, group) for the decode kernel, low half =
  *   fp16 scale, high half = fp16 (128 + zero point) (symmetric 4-bit weights: 128 + 8); only
  *   meaningful for 4-bit weights.
+ *   scale_zero_bf16 (may be NULL): one dword per (row, group) for the bf16 kernels on integer weights
+ *   (INT4, INT8), so that they load a group's parameters with one request: high half = bf16 scale (the
+ *   rounding of scales_bf16), low half = an fp16 number, 1024 + zero point for 4-bit weights (symmetric:
+ *   1024 + 8; the kernels read a nibble q as the fp16 number 1024 + q), the stored byte of zeros_u8 for
+ *   8-bit weights (symmetric: 128).  No counterpart in the reference, which keeps scales and zero points
+ *   in separate tensors (ContextLinearWoq.h:104-133).
  * Padding rows get scale 1, zero 0 (LinearWoqPacked.cpp:344-361).
  */
 int woq_hip_pack_qparams(const float* scales, const float* zeros, int weight_dtype, int64_t N,
                          int64_t KG, float* scales_f32, void* scales_f16, void* scales_bf16,
-                         uint8_t* zeros_u8, uint32_t* scale_zero_f16x2, void* stream);
+                         uint8_t* zeros_u8, uint32_t* scale_zero_f16x2, uint32_t* scale_zero_bf16,
+                         void* stream);
 
 /* zp[i][j] = (zp32[i][j/8] >> (4*(j%8))) & 0xf, written as fp32 [rows, cols]. */
 int woq_hip_unpack_int4_zeros(const int32_t* zp32, int64_t rows, int64_t cols,
@@ -195,6 +202,9 @@ typedef struct woq_hip_linear_params {
   const void* scales_bf16;
   const uint8_t* zeros_u8; /* NULL: symmetric weights */
   const uint32_t* scale_zero_f16x2; /* from woq_hip_pack_qparams; NULL disables the decode kernel */
+  const uint32_t* scale_zero_bf16;  /* from woq_hip_pack_qparams, optional: with it the bf16 kernels on INT4 /
+                                     * INT8 weights load one dword per (row, group) instead of a scale and a zero
+                                     * point; results are the same bit for bit */
   int64_t group_size;       /* <= 0: per output channel */
   const float* bias;        /* fp32 [N] or NULL */
 
@@ -260,6 +270,13 @@ int64_t woq_hip_linear_workspace_bytes(int64_t M, int64_t K, int32_t lowp_mode,
  * in the floating-point modes (decode kernel up to 32 rows; prefill GEMM when its 64 x 128 tiles are
  * at most 128); 0 where it never does.  No counterpart in the reference. */
 int64_t woq_hip_linear_split_k_workspace_bytes(int64_t M, int64_t N);
+
+/* The same size for the problems on which woq_hip_linear shares K between workgroups BY ITSELF (force_kernel 0):
+ * few output tiles and a long K -- 5..32 rows with K >= 8192 and N <= 4096 in the floating-point modes, more than
+ * 64 rows with K >= 4096 and M * N <= 2^20 in every mode -- and 0 for every other problem, where scratch and
+ * counters would go unused.  A caller that allocates per call asks this function; there is no second copy of the
+ * rule to keep in step.  No counterpart in the reference. */
+int64_t woq_hip_linear_auto_split_k_workspace_bytes(int64_t M, int64_t K, int64_t N, int32_t lowp_mode);
 
 /* K-block of the int8 path: min(group_size, 128), per-channel -> 128
  * (get_block_k, csrc/cpu/aten/Linear.cpp:362-376). */

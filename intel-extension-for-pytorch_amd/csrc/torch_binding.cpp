@@ -142,7 +142,7 @@ static Tensor dequant_weight(const Tensor& packed, int64_t wd, int64_t N, int64_
 
 struct PackedQParams {
   Tensor s32, s16, sb16;
-  optional<Tensor> z8, sz;
+  optional<Tensor> z8, sz, szb;
 };
 
 static PackedQParams pack_qparams(const Tensor& scales_in, const optional<Tensor>& zeros_in, int64_t wd) {
@@ -160,11 +160,13 @@ static PackedQParams pack_qparams(const Tensor& scales_in, const optional<Tensor
     q.z8 = at::empty({nt, KG, WOQ_HIP_TILE_N}, opt.dtype(at::kByte));
   }
   if (!is_8bit(wd)) q.sz = at::empty({nt, KG, WOQ_HIP_TILE_N}, opt.dtype(at::kInt));
+  if (wd == WOQ_HIP_DTYPE_INT4 || wd == WOQ_HIP_DTYPE_INT8) q.szb = at::empty({nt, KG, WOQ_HIP_TILE_N}, opt.dtype(at::kInt));
   DeviceScope scope(scales);
   check_rc(woq_hip_pack_qparams(scales.data_ptr<float>(), zeros.defined() ? zeros.data_ptr<float>() : nullptr, (int)wd,
                                 N, KG, q.s32.data_ptr<float>(), q.s16.data_ptr(), q.sb16.data_ptr(),
                                 q.z8.has_value() ? q.z8->data_ptr<uint8_t>() : nullptr,
-                                q.sz.has_value() ? (uint32_t*)q.sz->data_ptr() : nullptr, current_stream(scales)),
+                                q.sz.has_value() ? (uint32_t*)q.sz->data_ptr() : nullptr,
+                                q.szb.has_value() ? (uint32_t*)q.szb->data_ptr() : nullptr, current_stream(scales)),
            "pack_qparams");
   return q;
 }
@@ -429,6 +431,7 @@ class WoqLinearOpContext : public torch::CustomClassHolder {
     p.scales_bf16 = q_.sb16.data_ptr();
     p.zeros_u8 = q_.z8.has_value() ? q_.z8->data_ptr<uint8_t>() : nullptr;
     p.scale_zero_f16x2 = q_.sz.has_value() ? (const uint32_t*)q_.sz->data_ptr() : nullptr;
+    p.scale_zero_bf16 = q_.szb.has_value() ? (const uint32_t*)q_.szb->data_ptr() : nullptr;
     p.group_size = group_size_;
     p.bias = bias_f32_.defined() ? bias_f32_.data_ptr<float>() : nullptr;
     p.lowp_mode = (int32_t)lowp_mode_;
@@ -437,6 +440,9 @@ class WoqLinearOpContext : public torch::CustomClassHolder {
     std::vector<Tensor> keep;
     for (size_t i = 0; i < others.size() && i < 2; ++i) {
       TORCH_CHECK(others[i].numel() == M * N_, "woq_linear: post-op operand must have the output's shape");
+      TORCH_CHECK(others[i].is_cuda() && others[i].device() == x.device(),
+                  "woq_linear: expected all tensors to be on the same device, but the post-op operand is on ",
+                  others[i].device(), " and the input on ", x.device());
       keep.push_back(others[i].to(x.scalar_type()).contiguous());
       p.others[i] = keep.back().data_ptr();
     }
@@ -447,11 +453,10 @@ class WoqLinearOpContext : public torch::CustomClassHolder {
     const bool int8 = lowp_mode_ == WOQ_HIP_LOWP_INT8;
     int64_t wbytes = int8 ? woq_hip_linear_workspace_bytes(M, K_, WOQ_HIP_LOWP_INT8, (int32_t)act_quant_mode_, group_size_) : 0;
     optional<Tensor> counters;
-    if ((!int8 && M <= 32 && K_ >= 8192 && N_ <= 4096) || (M > 64 && K_ >= 4096 && M * N_ <= 1048576)) {
-      // long K and few output tiles: scratch with which the kernels may share K between workgroups
-      // (the library decides), and the zeroed counters of this stream
-      const int64_t extra = woq_hip_linear_split_k_workspace_bytes(M, N_);
-      if (extra > 0) counters = split_k_counters(x2);
+    // long K and few output tiles: scratch with which the kernels share K between workgroups, and the zeroed
+    // counters of this stream (the library says for which problems it would use them)
+    if (const int64_t extra = woq_hip_linear_auto_split_k_workspace_bytes(M, K_, N_, (int32_t)lowp_mode_)) {
+      counters = split_k_counters(x2);
       if (counters.has_value()) wbytes = (wbytes + 255) / 256 * 256 + extra;
     }
     Tensor ws;
@@ -499,6 +504,8 @@ static c10::intrusive_ptr<WoqLinearOpContext> context_from_handle(const Tensor& 
   TORCH_CHECK(handle.scalar_type() == at::kLong && handle.numel() == 1 && handle.is_cpu(), op,
               ": W_prepack must be the 1-element int64 tensor of get_data_handle()");
   const int64_t key = handle.data_ptr<int64_t>()[0];
+  // (the ctypes twin of the Python package hands out negative handles, so that neither kind resolves as the other)
+  TORCH_CHECK(key > 0, op, ": this handle does not come from a torch.classes.ipex_prepack.WoqLinearOpContext");
   c10::intrusive_ptr<WoqLinearOpContext> ctx;
   {
     std::lock_guard<std::mutex> lock(ctx_mutex());
@@ -706,11 +713,44 @@ static Tensor woq_linear_v2(const Tensor& input_in, const Tensor& qweight, c10::
   Tensor input = input_in;
   if (g_idx.has_value() && wd == WOQ_HIP_DTYPE_INT4 && group_size > 0) {
     // the packed weight from woq_linear_pack_weight is already sorted by group
+    TORCH_CHECK(g_idx->numel() == input.size(-1), "g_idx size and weight shape mismatch");
     const Tensor src = at::argsort(g_idx->to(input.device()).to(at::kLong).reshape({-1}), true, -1, false).to(at::kInt).contiguous();
     input = shuffle_activations(input, src);
   }
   TORCH_CHECK(input.size(-1) == K, "WOQ linear: input and weight shapes do not match, got k = ", input.size(-1),
               " and ", K, " respectively.");
+  // The tensor arguments go to the kernels as raw device pointers: each must live on the input's GPU and have the
+  // dtype and size of woq_linear_pack_weight's outputs for [N, K] and this group size, or the kernels would read
+  // host memory or past the end of an allocation.
+  TORCH_CHECK(N > 0 && K > 0, "IPEX WOQ: weight_shape must be positive, got [", N, ", ", K, "]");
+  auto on_input_device = [&](const Tensor& t, const char* what) {
+    TORCH_CHECK(t.is_cuda() && t.device() == input.device(), "torch_ipex::woq_linear: expected all tensors to be on the "
+                "same device, but ", what, " is on ", t.device(), " and the input on ", input.device());
+    TORCH_CHECK(t.is_contiguous(), "torch_ipex::woq_linear: ", what, " must be contiguous");
+  };
+  on_input_device(qweight, "the packed weight");
+  TORCH_CHECK((int64_t)qweight.nbytes() == woq_hip_packed_weight_bytes((int)wd, N, K), "torch_ipex::woq_linear: the packed "
+              "weight has ", qweight.nbytes(), " bytes, expected ", woq_hip_packed_weight_bytes((int)wd, N, K), " for [", N,
+              ", ", K, "] (the first output of woq_linear_pack_weight)");
+  const int64_t KG = group_size > 0 ? (K + group_size - 1) / group_size : 1;
+  const int64_t qcount = woq_hip_padded_n(N) / WOQ_HIP_TILE_N * KG * WOQ_HIP_TILE_N;
+  static const at::ScalarType kScaleTypes[3] = {at::kFloat, at::kHalf, at::kBFloat16};
+  for (int i = 0; i < 3; ++i) {
+    on_input_device(weight_scales[i], "a scale tensor");
+    TORCH_CHECK(weight_scales[i].scalar_type() == kScaleTypes[i] && weight_scales[i].numel() == qcount,
+                "torch_ipex::woq_linear: scales[", i, "] must be ", kScaleTypes[i], " with ", qcount,
+                " elements ([N/16, K/G, 16]), got ", weight_scales[i].scalar_type(), " with ", weight_scales[i].numel());
+  }
+  if (weight_zeros.has_value()) {
+    const Tensor& z8 = (*weight_zeros)[3];
+    on_input_device(z8, "the zero points");
+    TORCH_CHECK(z8.scalar_type() == at::kByte && z8.numel() == qcount, "torch_ipex::woq_linear: zeros[3] must be uint8 "
+                "with ", qcount, " elements ([N/16, K/G, 16]), got ", z8.scalar_type(), " with ", z8.numel());
+  }
+  if (bias.has_value()) {
+    on_input_device((*bias)[0], "the bias");
+    TORCH_CHECK((*bias)[0].numel() == N, "torch_ipex::woq_linear: bias has ", (*bias)[0].numel(), " elements, expected ", N);
+  }
   Tensor x2 = input.reshape({-1, K}).contiguous();
   if ((uintptr_t)x2.data_ptr() % 16) x2 = x2.clone();
   const int64_t M = x2.size(0);

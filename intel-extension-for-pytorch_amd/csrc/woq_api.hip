@@ -42,7 +42,7 @@ extern "C" {
 
 const char* woq_hip_last_error(void) { return g_err; }
 
-int woq_hip_abi_version(void) { return 1; }
+int woq_hip_abi_version(void) { return 2; }
 
 const char* woq_hip_last_kernel(void) { return g_last_kernel; }
 
@@ -76,14 +76,14 @@ int woq_hip_unpack_weight(const void* packed, int weight_dtype, int64_t N, int64
 
 int woq_hip_pack_qparams(const float* scales, const float* zeros, int weight_dtype, int64_t N, int64_t KG,
                          float* scales_f32, void* scales_f16, void* scales_bf16, uint8_t* zeros_u8,
-                         uint32_t* scale_zero_f16x2, void* stream) {
+                         uint32_t* scale_zero_f16x2, uint32_t* scale_zero_bf16, void* stream) {
   if (!valid_wdtype(weight_dtype)) return set_error("pack_qparams: unsupported weight dtype %d", weight_dtype);
   if (N < 0 || KG < 1) return set_error("pack_qparams: bad shape N=%lld KG=%lld", (long long)N, (long long)KG);
   if (N > 0 && (!scales || !scales_f32 || !scales_f16 || !scales_bf16))
     return set_error("pack_qparams: null scales pointer");
   if (zeros && !zeros_u8) return set_error("pack_qparams: zeros given but zeros_u8 is null");
   return launch_pack_qparams(scales, zeros, weight_dtype, N, KG, scales_f32, scales_f16, scales_bf16, zeros_u8,
-                             scale_zero_f16x2, (hipStream_t)stream);
+                             scale_zero_f16x2, scale_zero_bf16, (hipStream_t)stream);
 }
 
 int woq_hip_unpack_int4_zeros(const int32_t* zp32, int64_t rows, int64_t cols, int64_t cols_zp32, float* out,
@@ -134,6 +134,14 @@ int64_t woq_hip_linear_split_k_workspace_bytes(int64_t M, int64_t N) {
   const int64_t NT = woq_hip_padded_n(N) / kTileN;
   if (NT > 4 * kSplitKCounters) return 0;
   return decode_dq_splitk_bytes(M, NT, kSplitKMax);
+}
+
+int64_t woq_hip_linear_auto_split_k_workspace_bytes(int64_t M, int64_t K, int64_t N, int32_t lowp_mode) {
+  const bool int8 = lowp_mode == WOQ_HIP_LOWP_INT8;
+  // the dequantizing decode kernel (launch_decode_dq) and the 64 x 128 tiles of the prefill GEMMs (pick_splits)
+  const bool decode = !int8 && M >= 5 && M <= 32 && K >= 8192 && N <= 4096;
+  const bool prefill = M > 64 && K >= 4096 && M * N <= 1048576;
+  return decode || prefill ? woq_hip_linear_split_k_workspace_bytes(M, N) : 0;
 }
 
 int woq_hip_linear(const woq_hip_linear_params* p) {
@@ -251,6 +259,7 @@ int woq_hip_linear(const woq_hip_linear_params* p) {
   f.other0 = p->others[0]; f.other1 = p->others[1]; f.out = p->out; f.out_dtype = p->out_dtype;
   f.nf4 = nf4 ? 1 : 0;
   f.fp8 = fp8 ? 1 : 0;
+  f.szb = (regime == kRegimeBF16 && !nf4 && !fp8) ? p->scale_zero_bf16 : nullptr;
   SplitKScratch scratch;
   if (p->split_k_counters && p->workspace && p->workspace_bytes > 0) {
     scratch.partial = (float*)p->workspace;
@@ -355,6 +364,7 @@ int woq_hip_linear_grouped(const woq_hip_linear_params* p, const void* group, in
   FpArgs f;
   f.x = p->x; f.x_dtype = p->x_dtype; f.M = p->M; f.K = p->K; f.N = p->N; f.NT = NT; f.KT = KT;
   f.qweight = nullptr; f.scales = nullptr; f.zeros = nullptr;  // per expert, from the group table
+  f.szb = nullptr;
   f.G = G; f.KG = KG; f.bias = nullptr; f.fusion = p->fusion;
   f.other0 = p->others[0]; f.other1 = nullptr; f.out = p->out; f.out_dtype = p->out_dtype;
   f.nf4 = 0; f.fp8 = 0;
@@ -510,8 +520,8 @@ int woq_hip_linear_noalloc(const woq_hip_linear_params* p) {
   // Sharing K between workgroups is an option, not a need: offered for the problems it pays for (few
   // output tiles and a long K) while its scratch fits behind the quantized activations.
   bool split = false;
-  if ((!int8 && p->M <= 32 && p->K >= 8192 && p->N <= 4096) || (p->M > 64 && p->K >= 4096 && p->M * p->N <= 1048576)) {
-    const int64_t extra = woq_hip_linear_split_k_workspace_bytes(p->M, p->N);
+  {
+    const int64_t extra = woq_hip_linear_auto_split_k_workspace_bytes(p->M, p->K, p->N, p->lowp_mode);
     const int64_t base = (need + 255) / 256 * 256;
     if (extra > 0 && base + extra <= kNoAllocWorkspaceBytes) {
       need = base + extra;

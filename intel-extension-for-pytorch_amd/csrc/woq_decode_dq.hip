@@ -31,6 +31,8 @@
 // writes its fp32 partial tile to scratch memory, and the workgroup that arrives last at the
 // row-block set's counter (no workgroup ever waits) adds the S partial tiles in split order and runs
 // the epilogue.  The sum order is fixed, so the result does not depend on the arrival order.
+#include <type_traits>
+
 #include "woq_common.h"
 #include "woq_internal.h"
 
@@ -88,9 +90,40 @@ struct G8Consts {
 // reference's fp16 kernel converts them per K block (csrc/cpu/aten/utils/woq.h:3076-3079) -- the common
 // case of a bf16 model under lowp_mode BF16 with fewer than five rows.  The rows then travel through
 // registers (16-byte loads, conversion, ds_write to the same swizzled places) instead of the LDS DMA.
-template <int REGIME, int WBITS, int MT, int NTW, bool NF4, bool XCONV, bool FP8, bool GROUPED>
+// Constants of one (row, group) from its merged dword, bf16 scale << 16 | an fp16 number: 4-bit weights
+// w = (1024 + q) * s + c = (64 + q) * s + c64 with the fp16 number 1024 + z (a nibble is read as 1024 + q, or as
+// 64 + q in place at bits 4..7); 8-bit weights w = u * s + c with the fp16 number the stored zero byte.  All exact
+// in fp32, so the one rounding is the conversion to bf16, as with separate scale and zero point.
+struct DqConstsM {
+  float s, c, c64;
+  template <int WBITS>
+  __device__ __forceinline__ void set(uint32_t pd) {
+    s = bitcast<float>(pd & 0xFFFF0000u);
+    const _Float16 h = bitcast<_Float16>((uint16_t)(pd & 0xFFFFu));
+    c = -((float)h * s);
+    if constexpr (WBITS == 4) c64 = __builtin_fmaf(960.0f, s, c);
+  }
+};
+__device__ __forceinline__ u4 dq_dequant_m(uint32_t d, const G4Masks& k, uint32_t magic64, const DqConstsM& q) {
+  u4 r;
+  const f2 f0 = g4_fma_pair((d & k.lo) | k.magic, q.s, q.c);
+  const f2 f1 = g4_fma_pair((d & k.hi) | magic64, q.s, q.c64);
+  r[0] = g4_cvt_pair(f0);
+  const uint32_t d8 = d >> 8;
+  const f2 f2_ = g4_fma_pair((d8 & k.lo) | k.magic, q.s, q.c);
+  r[1] = g4_cvt_pair(f1);
+  const f2 f3 = g4_fma_pair((d8 & k.hi) | magic64, q.s, q.c64);
+  r[2] = g4_cvt_pair(f2_);
+  r[3] = g4_cvt_pair(f3);
+  return r;
+}
+
+// SZB (bf16 compute, integer weights, not GROUPED): scale and zero point of a (row, group) come as one dword
+// (f.szb): one request and three vector instructions per row-block and round instead of two and eight.
+template <int REGIME, int WBITS, int MT, int NTW, bool NF4, bool XCONV, bool FP8, bool GROUPED, bool SZB = false>
 __global__ __launch_bounds__(512, (MT * NTW > 8 ? 2 : 4)) void woq_decode_dq_kernel(const DecodeDqArgs a) {
   static_assert(!XCONV || (REGIME == kRegimeF16 && MT == 1), "bf16 -> fp16 rows: fp16 regime, one row tile");
+  static_assert(!SZB || (REGIME == kRegimeBF16 && !NF4 && !FP8 && !GROUPED), "merged parameters: bf16 compute, integer weights");
   using Geo = DqGeom<WBITS, MT>;
   constexpr int TK = Geo::TK, NJ = Geo::NJ, NX = Geo::NX, SLICE = Geo::SLICE;
   static_assert(!NF4 || WBITS == 4, "NF4 codes are 4 bits wide");
@@ -143,6 +176,8 @@ __global__ __launch_bounds__(512, (MT * NTW > 8 ? 2 : 4)) void woq_decode_dq_ker
   asm volatile("s_mov_b32 %0, 0x000F000F" : "=s"(km.lo));
   asm volatile("s_mov_b32 %0, 0x00F000F0" : "=s"(km.hi));
   asm volatile("v_mov_b32 %0, 0x64006400" : "=v"(km.magic));
+  uint32_t magic64 = 0;  // fp16 64 twice
+  if constexpr (SZB && WBITS == 4) asm volatile("v_mov_b32 %0, 0x54005400" : "=v"(magic64));
 
   f4 acc[NTW][MT];
 #pragma unroll
@@ -178,16 +213,25 @@ __global__ __launch_bounds__(512, (MT * NTW > 8 ? 2 : 4)) void woq_decode_dq_ker
     // missing ones from the last real row-block, and the store below drops their columns (n >= N)
     const int64_t nt = nt0 + t < f.NT ? nt0 + t : f.NT - 1;
     wbase[t] = f.qweight + (size_t)nt * KT * kTileBytes;
-    sbase[t] = (const uint8_t*)(f.scales + (size_t)nt * KG * kTileN);
-    zbase[t] = has_z ? f.zeros + (size_t)nt * KG * kTileN : sbase[t];
+    if constexpr (SZB) {
+      sbase[t] = (const uint8_t*)f.szb + (size_t)nt * KG * (kTileN * 4);
+      zbase[t] = sbase[t];
+    } else {
+      sbase[t] = (const uint8_t*)(f.scales + (size_t)nt * KG * kTileN);
+      zbase[t] = has_z ? f.zeros + (size_t)nt * KG * kTileN : sbase[t];
+    }
   }
 
-  u4 wnext[NTW];
-  uint16_t snext[NTW];
-  uint8_t znext[NTW];
+  // Two register sets for the tiles and parameters in flight: round i computes from set i % 2 while the
+  // requests of round i + 1 fill the other, so nothing is copied between rounds.
+  u4 wq[2][NTW];
+  uint16_t sq[2][SZB ? 1 : NTW];
+  uint8_t zq[2][SZB ? 1 : NTW];
+  uint32_t mq[2][SZB ? NTW : 1];
   u4 xnext[XCONV ? NX : 1];  // XCONV: the next round's activation rows, still bf16
-  // every request of one round: activations into LDS buffer `buf`, tiles and parameters into registers
-  auto request = [&](int kt, int buf) {
+  // every request of one round: activations into LDS buffer `buf`, tiles and parameters into register set `buf`
+  auto request = [&](int kt, auto bufc) {
+    constexpr int buf = decltype(bufc)::value;
     // uniform base + 32-bit offset; instructions whose rows lie entirely past M are skipped
     // (their LDS bytes stay undefined: an MFMA output row depends on its own A row only)
     const uint32_t ko = (uint32_t)kt * Geo::ROWB;
@@ -206,9 +250,13 @@ __global__ __launch_bounds__(512, (MT * NTW > 8 ? 2 : 4)) void woq_decode_dq_ker
     const uint32_t wo = (uint32_t)kt * kTileBytes + woff;
 #pragma unroll
     for (int t = 0; t < NTW; ++t) {
-      wnext[t] = __builtin_nontemporal_load((const u4*)(wbase[t] + wo));
-      snext[t] = *(const uint16_t*)(sbase[t] + (uint32_t)(qoff * 2u));
-      znext[t] = *(zbase[t] + qoff);  // raw: any use here would wait for the load inside the request
+      wq[buf][t] = __builtin_nontemporal_load((const u4*)(wbase[t] + wo));
+      if constexpr (SZB) {
+        mq[buf][t] = *(const uint32_t*)(sbase[t] + (uint32_t)(qoff * 4u));
+      } else {
+        sq[buf][t] = *(const uint16_t*)(sbase[t] + (uint32_t)(qoff * 2u));
+        zq[buf][t] = *(zbase[t] + qoff);  // raw: any use here would wait for the load inside the request
+      }
     }
   };
 
@@ -216,22 +264,31 @@ __global__ __launch_bounds__(512, (MT * NTW > 8 ? 2 : 4)) void woq_decode_dq_ker
   // wave with no tile left idles until the sum.
   const int kt0 = (int)blockIdx.y * a.KTs;
   const int kt1 = kt0 + a.KTs < KT ? kt0 + a.KTs : KT;
-  if (kt0 + wave < kt1) request(kt0 + wave, 0);
-#pragma unroll 1
-  for (int kt = kt0 + wave, buf = 0; kt < kt1; kt += W, buf ^= 1) {
-    u4 wreg[NTW];
-    G4Consts<REGIME> qc4[WBITS == 4 ? NTW : 1];
+  using Buf0 = std::integral_constant<int, 0>;
+  using Buf1 = std::integral_constant<int, 1>;
+  if (kt0 + wave < kt1) request(kt0 + wave, Buf0{});
+  // one round: K tile kt from register set and LDS buffer `buf`
+  auto round = [&](const int kt, auto bufc) {
+    constexpr int buf = decltype(bufc)::value;
+    const u4 (&wreg)[NTW] = wq[buf];
+    G4Consts<REGIME> qc4[WBITS == 4 && !SZB ? NTW : 1];
     G8Consts qc8[WBITS == 8 || NF4 ? NTW : 1];
+    DqConstsM qm[SZB ? NTW : 1];
 #pragma unroll
     for (int t = 0; t < NTW; ++t) {
-      wreg[t] = wnext[t];
-      if constexpr (NF4) {
-        qc8[t].s = REGIME == kRegimeF16 ? f16_bits_to_f32(snext[t]) : bf16_bits_to_f32(snext[t]);
+      if constexpr (SZB) {
+        qm[t].template set<WBITS>(mq[buf][t]);
+        if constexpr (WBITS == 8) {
+          qc8[t].s = qm[t].s;
+          qc8[t].c = qm[t].c;
+        }
+      } else if constexpr (NF4) {
+        qc8[t].s = REGIME == kRegimeF16 ? f16_bits_to_f32(sq[buf][t]) : bf16_bits_to_f32(sq[buf][t]);
       } else if constexpr (WBITS == 4) {
-        qc4[t].set(snext[t], has_z ? (float)znext[t] : 8.0f);
+        qc4[t].set(sq[buf][t], has_z ? (float)zq[buf][t] : 8.0f);
       } else {
-        qc8[t].s = REGIME == kRegimeF16 ? f16_bits_to_f32(snext[t]) : bf16_bits_to_f32(snext[t]);
-        qc8[t].c = -((has_z ? (float)znext[t] : 128.0f) * qc8[t].s);
+        qc8[t].s = REGIME == kRegimeF16 ? f16_bits_to_f32(sq[buf][t]) : bf16_bits_to_f32(sq[buf][t]);
+        qc8[t].c = -((has_z ? (float)zq[buf][t] : 128.0f) * qc8[t].s);
       }
     }
     // The compiler does not order LDS reads after the LDS-writing loads: wait for them here.
@@ -251,7 +308,7 @@ __global__ __launch_bounds__(512, (MT * NTW > 8 ? 2 : 4)) void woq_decode_dq_ker
           *(u4*)(sx + buf * SLICE + i * 1024 + lane * 16) = h;
         }
     }
-    if (kt + W < kt1) request(kt + W, buf ^ 1);
+    if (kt + W < kt1) request(kt + W, std::integral_constant<int, buf ^ 1>{});
     __builtin_amdgcn_sched_barrier(0);
 
 #pragma unroll
@@ -264,6 +321,8 @@ __global__ __launch_bounds__(512, (MT * NTW > 8 ? 2 : 4)) void woq_decode_dq_ker
         u4 bop;
         if constexpr (NF4) {
           bop = nf4_dequant<REGIME>(wreg[t][j], sNf4, qc8[t].s);
+        } else if constexpr (WBITS == 4 && SZB) {
+          bop = dq_dequant_m(wreg[t][j], km, magic64, qm[t]);
         } else if constexpr (WBITS == 4) {
           bop = g4_dequant(wreg[t][j], km, qc4[t]);
         } else if constexpr (FP8) {
@@ -280,6 +339,11 @@ __global__ __launch_bounds__(512, (MT * NTW > 8 ? 2 : 4)) void woq_decode_dq_ker
         for (int mt = 0; mt < MT; ++mt) acc[t][mt] = dq_mfma<REGIME>(xa[mt], bop, acc[t][mt]);
       }
     }
+  };
+#pragma unroll 1
+  for (int kt = kt0 + wave; kt < kt1; kt += 2 * W) {
+    round(kt, Buf0{});
+    if (kt + W < kt1) round(kt + W, Buf1{});
   }
 
   // ---- combine the waves' partial sums in wave order, then bias / rounding / store ----
@@ -352,8 +416,8 @@ __global__ __launch_bounds__(512, (MT * NTW > 8 ? 2 : 4)) void woq_decode_dq_ker
   if (threadIdx.x == 0) __hip_atomic_store(a.counters + blockIdx.x, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-template <int REGIME, int WBITS, int MT, int NTW, bool NF4 = false, bool XCONV = false, bool FP8 = false, bool GROUPED = false>
-static int launch_dq_cfg(DecodeDqArgs a, int splits, hipStream_t st, int slots = 1) {
+template <int REGIME, int WBITS, int MT, int NTW, bool NF4, bool XCONV, bool FP8, bool GROUPED, bool SZB>
+static int launch_dq_cfg_impl(DecodeDqArgs a, int splits, hipStream_t st, int slots) {
   using Geo = DqGeom<WBITS, MT>;
   if (MT > 2 && splits > 1) return set_error("woq_decode_dq_kernel: split K takes at most 32 rows");
   // At most 64 KiB of activation buffers per workgroup, so that two workgroups share a CU -- unless
@@ -373,7 +437,7 @@ static int launch_dq_cfg(DecodeDqArgs a, int splits, hipStream_t st, int slots =
   size_t smem = (size_t)a.W * 2 * Geo::SLICE;
   const size_t red = (size_t)NTW * MT * a.W * 64 * sizeof(f4);
   if (red > smem) smem = red;
-  auto kern = woq_decode_dq_kernel<REGIME, WBITS, MT, NTW, NF4, XCONV, FP8, GROUPED>;
+  auto kern = woq_decode_dq_kernel<REGIME, WBITS, MT, NTW, NF4, XCONV, FP8, GROUPED, SZB>;
   if (MT >= 2) {
     // more than 64 KiB of LDS per workgroup needs an opt-in (once per kernel and process)
     static const hipError_t lds_optin =
@@ -383,6 +447,15 @@ static int launch_dq_cfg(DecodeDqArgs a, int splits, hipStream_t st, int slots =
   }
   kern<<<grid, a.W * 64, smem, st>>>(a);
   return check_launch("woq_decode_dq_kernel");
+}
+
+template <int REGIME, int WBITS, int MT, int NTW, bool NF4 = false, bool XCONV = false, bool FP8 = false, bool GROUPED = false>
+static int launch_dq_cfg(DecodeDqArgs a, int splits, hipStream_t st, int slots = 1) {
+  if constexpr (REGIME == kRegimeBF16 && !NF4 && !FP8 && !GROUPED && !XCONV) {
+    // the caller's merged (scale, zero) dword table: one parameter request per row-block and round
+    if (a.f.szb) return launch_dq_cfg_impl<REGIME, WBITS, MT, NTW, NF4, XCONV, FP8, GROUPED, true>(a, splits, st, slots);
+  }
+  return launch_dq_cfg_impl<REGIME, WBITS, MT, NTW, NF4, XCONV, FP8, GROUPED, false>(a, splits, st, slots);
 }
 
 // At most 64 rows already in the compute dtype (or up to 16 bf16 rows for fp16 compute), whole K tiles, and (4-bit) a group size whose

@@ -27,7 +27,12 @@
 //     step of 128 is then two packed tiles per row-block (a tile is 16 rows x 64 bytes), sub-step j
 //     takes dwords 2 (j % 2), 2 (j % 2) + 1 of tile j / 2 -- the K offsets 64 (j / 2) + 16 c + 8 (j % 2)
 //     of lane column c -- and the A fragment is read from the matching 16-byte chunk; 20 VALU
-//     instructions per B operand (byte -> float, fma, pack) against 17.
+//     instructions per B operand (byte -> float, fma, pack) against 17;
+//   * MERGED instances (4-bit weights, bf16 compute, when the caller passes the table): the scale and the
+//     zero point of a (row, group) come as one dword, bf16 scale << 16 | fp16 (1024 + zero), and the two
+//     nibble positions are read as the fp16 numbers 1024 + q and 64 + q, so that one scale serves both:
+//     7 instead of 14 parameter requests and 21 instead of 56 vector instructions per K step and wave
+//     (M = 2048, 4096 -> 14336: 198 against 202-206 us on the same boxes; same bits out).
 #include "woq_common.h"
 #include "woq_internal.h"
 
@@ -74,7 +79,33 @@ typedef const __attribute__((address_space(1))) void* global_ptr_t;
 // lie in the registers, and the workgroup that arrives last at the tile's counter adds the partial
 // tiles in z order (its own from the registers) and runs the epilogue.  Nobody waits; the order of
 // the sum is fixed.  All scratch accesses are relaxed device-scope atomics, as in the decode kernel.
-template <int REGIME, class S, int WBITS, bool FP8>
+// Constants of one (row, group) from its merged dword: w = (1024 + q) * s + c = (64 + q) * s + c64, both
+// exact in fp32 (an 11-bit integer times an 8-bit significand), so the fma result is the exact product
+// (q - z) * s and the one rounding is the conversion to bf16, as with separate scale and zero point.
+struct G4ConstsM {
+  float s, c, c64;
+  __device__ __forceinline__ void set(uint32_t pd) {
+    s = bitcast<float>(pd & 0xFFFF0000u);
+    const _Float16 h = bitcast<_Float16>((uint16_t)(pd & 0xFFFFu));
+    c = -((float)h * s);
+    c64 = __builtin_fmaf(960.0f, s, c);
+  }
+};
+__device__ __forceinline__ u4 g4_dequant_m(uint32_t d, const G4Masks& k, uint32_t magic64, const G4ConstsM& q) {
+  u4 r;
+  const f2 f0 = g4_fma_pair((d & k.lo) | k.magic, q.s, q.c);
+  const f2 f1 = g4_fma_pair((d & k.hi) | magic64, q.s, q.c64);
+  r[0] = g4_cvt_pair(f0);
+  const uint32_t d8 = d >> 8;
+  const f2 f2_ = g4_fma_pair((d8 & k.lo) | k.magic, q.s, q.c);
+  r[1] = g4_cvt_pair(f1);
+  const f2 f3 = g4_fma_pair((d8 & k.hi) | magic64, q.s, q.c64);
+  r[2] = g4_cvt_pair(f2_);
+  r[3] = g4_cvt_pair(f3);
+  return r;
+}
+
+template <int REGIME, class S, int WBITS, bool FP8, bool MERGED = false>
 __global__ __launch_bounds__(256) void woq_gemm_w4_kernel(const FpArgs f, const int g_shift, float* const sk_partial,
                                                           int* const sk_counters, const int kts) {
   constexpr int TPS = WBITS / 4;  // packed tiles per row-block and K step of 128
@@ -101,6 +132,8 @@ __global__ __launch_bounds__(256) void woq_gemm_w4_kernel(const FpArgs f, const 
   asm volatile("s_mov_b32 %0, 0x000F000F" : "=s"(km.lo));
   asm volatile("s_mov_b32 %0, 0x00F000F0" : "=s"(km.hi));
   asm volatile("v_mov_b32 %0, 0x64006400" : "=v"(km.magic));
+  uint32_t magic64;  // fp16 64 twice: a nibble in place at bits 4..7 reads as 64 + q
+  asm volatile("v_mov_b32 %0, 0x54005400" : "=v"(magic64));
 
   f4 acc[G4_MT][G4_NTW];
 #pragma unroll
@@ -148,12 +181,14 @@ __global__ __launch_bounds__(256) void woq_gemm_w4_kernel(const FpArgs f, const 
   const uint8_t* wbase[G4_NTW];
   const uint8_t* sbase[G4_NTW];
   const uint8_t* zbase[G4_NTW];
+  const uint8_t* mbase[G4_NTW];
 #pragma unroll
   for (int t = 0; t < G4_NTW; ++t) {
     const int nt = nt0 + t < NT ? nt0 + t : NT - 1;
     wbase[t] = f.qweight + (size_t)nt * KTW * kTileBytes;
     sbase[t] = (const uint8_t*)(f.scales + (size_t)nt * KG * kTileN);
     zbase[t] = has_z ? f.zeros + (size_t)nt * KG * kTileN : sbase[t];
+    mbase[t] = (const uint8_t*)f.szb + (size_t)nt * KG * (kTileN * 4);
   }
   const uint32_t woff = (uint32_t)lane * 16u;
   auto load_q = [&](int kt, uint16_t (&s)[G4_NTW], uint8_t (&z)[G4_NTW]) {
@@ -166,6 +201,13 @@ __global__ __launch_bounds__(256) void woq_gemm_w4_kernel(const FpArgs f, const 
       const uint8_t zb = *(zbase[t] + qoff);
       z[t] = has_z ? zb : (uint8_t)(WBITS == 4 ? 8 : 128);  // symmetric: the stored code of zero
     }
+  };
+  auto load_m = [&](int kt, uint32_t (&p)[G4_NTW]) {
+    int g = (kt * kTileK4 + c * 32) >> g_shift;
+    g = g < KG ? g : KG - 1;
+    const uint32_t qoff = (uint32_t)(g * kTileN + r) * 4u;
+#pragma unroll
+    for (int t = 0; t < G4_NTW; ++t) p[t] = *(const uint32_t*)(mbase[t] + qoff);
   };
   // The packed tiles of a K step travel global -> LDS -> registers: the LDS stage costs no
   // registers while the load is in flight, which lets the tiles be requested two steps ahead.
@@ -189,9 +231,13 @@ __global__ __launch_bounds__(256) void woq_gemm_w4_kernel(const FpArgs f, const 
   uint16_t sr[G4_NTW];
   uint8_t zr[G4_NTW];
   G4Consts<REGIME> qc[WBITS == 4 ? G4_NTW : 1];
+  G4ConstsM qm[G4_NTW];
+  uint32_t mr[G4_NTW];
   float q8s[WBITS == 8 ? G4_NTW : 1], q8c[WBITS == 8 ? G4_NTW : 1];  // 8-bit: scale, -(128 + z) * scale
   auto set_q = [&](int t, uint16_t sbits, float z) {
-    if constexpr (WBITS == 4) {
+    if constexpr (MERGED) {
+      qm[t].set(mr[t]);
+    } else if constexpr (WBITS == 4) {
       qc[t].set(sbits, z);
     } else {
       q8s[t] = REGIME == kRegimeF16 ? f16_bits_to_f32(sbits) : bf16_bits_to_f32(sbits);
@@ -200,7 +246,9 @@ __global__ __launch_bounds__(256) void woq_gemm_w4_kernel(const FpArgs f, const 
   };
   // B operand of row-block t, K sub-step j
   auto deq = [&](int t, int j) -> u4 {
-    if constexpr (WBITS == 4) {
+    if constexpr (MERGED) {
+      return g4_dequant_m(wr[t][0][j], km, magic64, qm[t]);
+    } else if constexpr (WBITS == 4) {
       return g4_dequant(wr[t][0][j], km, qc[t]);
     } else {
       const uint32_t d0 = wr[t][j / 2][2 * (j % 2)], d1 = wr[t][j / 2][2 * (j % 2) + 1];
@@ -220,8 +268,9 @@ __global__ __launch_bounds__(256) void woq_gemm_w4_kernel(const FpArgs f, const 
   // s_waitcnt immediates (vmcnt in bits 3:0 and 15:14; expcnt 6:4 and lgkmcnt 11:8 left at maximum)
   constexpr int kVmcnt0 = 0x0F70, kLgkmcnt0 = 0xC07F;
   constexpr int kVmcntW = 0x0F70 | (G4_NTW * TPS);  // all but the last loads (one weight stage) have landed
-  // everything older than one whole step of loads (2 NTW parameter loads, XLOADS + NTW * TPS LDS loads)
-  constexpr int kStepLoads = (2 + TPS) * G4_NTW + G4_XLOADS;
+  // everything older than one whole step of loads (2 NTW parameter loads -- merged: NTW --, XLOADS + NTW * TPS
+  // LDS loads)
+  constexpr int kStepLoads = ((MERGED ? 1 : 2) + TPS) * G4_NTW + G4_XLOADS;
   static_assert(kStepLoads < 64 && G4_NTW * TPS < 16, "s_waitcnt vmcnt is a 6-bit field");
   constexpr int kVmcntStep = 0x0F70 | (kStepLoads & 15) | ((kStepLoads >> 4) << 14);
 
@@ -235,7 +284,7 @@ __global__ __launch_bounds__(256) void woq_gemm_w4_kernel(const FpArgs f, const 
   load_x(kt_lo, 0);
   dma_w(kt_lo, 0);
   dma_w(KT > kt_lo + 1 ? kt_lo + 1 : kt_lo, 1);
-  load_q(kt_lo, sr, zr);
+  if constexpr (MERGED) load_m(kt_lo, mr); else load_q(kt_lo, sr, zr);
   __builtin_amdgcn_s_waitcnt(kVmcnt0);
   __syncthreads();
 #pragma unroll
@@ -264,7 +313,7 @@ __global__ __launch_bounds__(256) void woq_gemm_w4_kernel(const FpArgs f, const 
     // kt + 2 into the stage that held step kt.  Past the end the last step is requested again. ----
     const int kt1 = kt + 1 < KT ? kt + 1 : KT - 1;
     const int kt2 = kt + 2 < KT ? kt + 2 : KT - 1;
-    load_q(kt1, sr, zr);
+    if constexpr (MERGED) load_m(kt1, mr); else load_q(kt1, sr, zr);
     load_x(kt1, (kt & 1) ^ 1);
     __builtin_amdgcn_sched_barrier(0);
 
@@ -496,6 +545,18 @@ static int launch_shape(const FpArgs& f, int g_shift, hipStream_t st, int splits
     if (!scratch || !scratch->partial || !scratch->counters || scratch->bytes < need || tiles > kSplitKCounters)
       return set_error("woq_gemm_w4_kernel: split K needs %lld bytes of workspace, the counter array and at most %d "
                        "tiles", (long long)need, kSplitKCounters);
+  }
+  if constexpr (REGIME == kRegimeBF16 && WBITS == 4) {
+    if (f.szb) {  // scale and zero point of a (row, group) in one dword
+      static const hipError_t lds_optin_m =
+          hipFuncSetAttribute(reinterpret_cast<const void*>(&woq_gemm_w4_kernel<REGIME, S, WBITS, FP8, true>),
+                              hipFuncAttributeMaxDynamicSharedMemorySize, kLds);
+      if (lds_optin_m != hipSuccess)
+        return set_error("woq_gemm_w4_kernel: LDS opt-in failed: %s", hipGetErrorString(lds_optin_m));
+      woq_gemm_w4_kernel<REGIME, S, WBITS, FP8, true><<<grid, 256, kLds, st>>>(
+          f, g_shift, splits > 1 ? scratch->partial : nullptr, splits > 1 ? scratch->counters : nullptr, kts);
+      return check_launch("woq_gemm_w4_kernel");
+    }
   }
   woq_gemm_w4_kernel<REGIME, S, WBITS, FP8><<<grid, 256, kLds, st>>>(f, g_shift, splits > 1 ? scratch->partial : nullptr,
                                                                  splits > 1 ? scratch->counters : nullptr, kts);

@@ -36,6 +36,9 @@ struct FpArgs {
   const uint8_t* qweight;
   const uint16_t* scales;  // fp16 bits (fp16 regime) or bf16 bits (bf16 regime), [NT][KG][16]
   const uint8_t* zeros;    // [NT][KG][16] or nullptr
+  // bf16 regime, integer weights, optional: [NT][KG][16] dwords, bf16 scale << 16 | fp16 (1024 + zero) (4-bit
+  // weights) or fp16 (stored zero byte) (8-bit weights): one load instead of two per (row, group)
+  const uint32_t* szb;
   int64_t G;               // group size in K elements (per-channel: >= padded K)
   int64_t KG;
   const float* bias;
@@ -64,7 +67,7 @@ int launch_pack_weight(const void* plain, int weight_dtype, int64_t N, int64_t K
 int launch_unpack_weight(const void* packed, int weight_dtype, int64_t N, int64_t K, void* plain,
                          hipStream_t st);
 int launch_pack_qparams(const float* scales, const float* zeros, int weight_dtype, int64_t N, int64_t KG,
-                        float* s32, void* s16, void* sb16, uint8_t* z8, uint32_t* sz, hipStream_t st);
+                        float* s32, void* s16, void* sb16, uint8_t* z8, uint32_t* sz, uint32_t* szb, hipStream_t st);
 int launch_unpack_int4_zeros(const int32_t* zp32, int64_t rows, int64_t cols, int64_t cols_zp32,
                              float* out, hipStream_t st);
 int launch_convert_activations(const void* src, int src_dtype, void* dst, int dst_dtype, int64_t count, hipStream_t st);

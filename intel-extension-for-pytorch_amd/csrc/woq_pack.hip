@@ -100,7 +100,7 @@ __global__ void pack_qparams_kernel(const float* __restrict__ scales, const floa
                                     int weight_dtype, int64_t N, int64_t Np, int64_t KG,
                                     float* __restrict__ s32, uint16_t* __restrict__ s16,
                                     uint16_t* __restrict__ sb16, uint8_t* __restrict__ z8,
-                                    uint32_t* __restrict__ sz) {
+                                    uint32_t* __restrict__ sz, uint32_t* __restrict__ szb) {
   const int64_t gid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (gid >= Np * KG) return;
   const int r = gid % kTileN;
@@ -123,6 +123,14 @@ __global__ void pack_qparams_kernel(const float* __restrict__ scales, const floa
   if (sz) {
     const float zz = 128.0f + (zeros ? z : (n < N ? 8.0f : 0.0f));
     sz[gid] = (uint32_t)f32_to_f16_bits(s) | ((uint32_t)f32_to_f16_bits(zz) << 16);
+  }
+  if (szb) {
+    // what the bf16 kernels subtract from the stored code: the zero point byte as stored (8-bit weights:
+    // offset-binary), the code of zero for symmetric weights; 4-bit weights get the 1024 of the fp16 number
+    // 1024 + q that their nibbles are read as
+    const bool w8 = weight_dtype == WOQ_HIP_DTYPE_INT8;
+    const float zc = zeros ? z + (w8 ? 128.0f : 0.0f) : (w8 ? 128.0f : 8.0f);
+    szb[gid] = ((uint32_t)f32_to_bf16_bits(s) << 16) | (uint32_t)f32_to_f16_bits(zc + (w8 ? 0.0f : 1024.0f));
   }
 }
 
@@ -219,13 +227,13 @@ int launch_unpack_weight(const void* packed, int weight_dtype, int64_t N, int64_
 }
 
 int launch_pack_qparams(const float* scales, const float* zeros, int weight_dtype, int64_t N, int64_t KG,
-                        float* s32, void* s16, void* sb16, uint8_t* z8, uint32_t* sz, hipStream_t st) {
+                        float* s32, void* s16, void* sb16, uint8_t* z8, uint32_t* sz, uint32_t* szb, hipStream_t st) {
   const int64_t Np = woq_hip_padded_n(N);
   const int64_t total = Np * KG;
   if (total == 0) return 0;
   pack_qparams_kernel<<<blocks_for(total, 256), 256, 0, st>>>(scales, zeros, weight_dtype, N, Np, KG, s32,
                                                               (uint16_t*)s16, (uint16_t*)sb16,
-                                                              zeros ? z8 : nullptr, sz);
+                                                              zeros ? z8 : nullptr, sz, szb);
   return check_launch("pack_qparams");
 }
 

@@ -69,7 +69,8 @@ def unpack_weight(packed, weight_dtype, N, K):
 
 def pack_qparams(scales, zeros, weight_dtype):
     """scales / zeros: fp32 [N, KG] -> ([NT, KG, 16] fp32, fp16, bf16, uint8-or-None, packed
-    (fp16 scale, fp16 128 + zero) dwords-or-None)."""
+    (fp16 scale, fp16 128 + zero) dwords-or-None, packed (bf16 scale, fp16 zero code) dwords-or-None: the
+    last for INT4 and INT8 weights, which the bf16 kernels then read with one load per (row, group))."""
     lib = _lib.load()
     _require_cuda(scales, "scales")
     scales = scales.to(torch.float32).contiguous()
@@ -87,15 +88,18 @@ def pack_qparams(scales, zeros, weight_dtype):
     sz = None
     if weight_dtype not in _lib.DTYPES_8BIT:
         sz = torch.empty((nt, KG, _lib.TILE_N), dtype=torch.int32, device=dev)
+    szb = None
+    if weight_dtype in (_lib.DTYPE_INT4, _lib.DTYPE_INT8):
+        szb = torch.empty((nt, KG, _lib.TILE_N), dtype=torch.int32, device=dev)
     with torch.cuda.device(dev):
         _lib.check(
             lib.woq_hip_pack_qparams(
                 _ptr(scales), _ptr(zeros), weight_dtype, N, KG, _ptr(s32), _ptr(s16), _ptr(sb16), _ptr(z8), _ptr(sz),
-                _stream()
+                _ptr(szb), _stream()
             ),
             "pack_qparams",
         )
-    return s32, s16, sb16, z8, sz
+    return s32, s16, sb16, z8, sz, szb
 
 
 def unpack_int4_zeros(zp32, cols):
@@ -187,6 +191,7 @@ def linear(
     debug_block_sums=False,
     noalloc=False,
     out_dtype=None,
+    scale_zero_bf16=None,
 ):
     """y = x @ dequant(W)^T (+ bias, post-op).  x: [..., K]; returns [..., N] in x.dtype, or the
     fp32 accumulator when ``out_fp32``.  With ``debug_block_sums`` also returns the int32 sum of
@@ -219,6 +224,7 @@ def linear(
     p.scales_bf16 = scales_bf16.data_ptr()
     p.zeros_u8 = zeros_u8.data_ptr() if zeros_u8 is not None else None
     p.scale_zero_f16x2 = scale_zero_f16x2.data_ptr() if scale_zero_f16x2 is not None else None
+    p.scale_zero_bf16 = scale_zero_bf16.data_ptr() if scale_zero_bf16 is not None else None
     p.group_size = group_size
     p.bias = bias_f32.data_ptr() if bias_f32 is not None else None
     p.lowp_mode = lowp_mode

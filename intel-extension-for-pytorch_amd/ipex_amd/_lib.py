@@ -34,6 +34,7 @@ EXPORTS = [
     "woq_hip_dynamic_quant",
     "woq_hip_linear_workspace_bytes",
     "woq_hip_linear_split_k_workspace_bytes",
+    "woq_hip_linear_auto_split_k_workspace_bytes",
     "woq_hip_int8_block_k",
     "woq_hip_linear",
     "woq_hip_linear_noalloc",
@@ -69,6 +70,7 @@ class LinearParams(ctypes.Structure):
         ("scales_bf16", ctypes.c_void_p),
         ("zeros_u8", ctypes.c_void_p),
         ("scale_zero_f16x2", ctypes.c_void_p),
+        ("scale_zero_bf16", ctypes.c_void_p),
         ("group_size", ctypes.c_int64),
         ("bias", ctypes.c_void_p),
         ("lowp_mode", ctypes.c_int32),
@@ -122,7 +124,7 @@ def load():
         lib.woq_hip_unpack_weight.restype = i32
         lib.woq_hip_unpack_weight.argtypes = [vp, i32, i64, i64, vp, vp]
         lib.woq_hip_pack_qparams.restype = i32
-        lib.woq_hip_pack_qparams.argtypes = [vp, vp, i32, i64, i64, vp, vp, vp, vp, vp, vp]
+        lib.woq_hip_pack_qparams.argtypes = [vp, vp, i32, i64, i64, vp, vp, vp, vp, vp, vp, vp]
         lib.woq_hip_unpack_int4_zeros.restype = i32
         lib.woq_hip_unpack_int4_zeros.argtypes = [vp, i64, i64, i64, vp, vp]
         lib.woq_hip_dynamic_quant.restype = i32
@@ -131,6 +133,8 @@ def load():
         lib.woq_hip_linear_workspace_bytes.argtypes = [i64, i64, ctypes.c_int32, ctypes.c_int32, i64]
         lib.woq_hip_linear_split_k_workspace_bytes.restype = i64
         lib.woq_hip_linear_split_k_workspace_bytes.argtypes = [i64, i64]
+        lib.woq_hip_linear_auto_split_k_workspace_bytes.restype = i64
+        lib.woq_hip_linear_auto_split_k_workspace_bytes.argtypes = [i64, i64, i64, i32]
         lib.woq_hip_int8_block_k.restype = i64
         lib.woq_hip_int8_block_k.argtypes = [i64, i64]
         lib.woq_hip_linear.restype = i32
@@ -161,7 +165,7 @@ def load():
         lib.woq_hip_moe_combine_rows.argtypes = [vp, i32, i64, i64, vp, vp, i64, vp, vp, i32, vp]
         lib.woq_hip_probe_mfma_issue.restype = i32
         lib.woq_hip_probe_mfma_issue.argtypes = [vp, i32, i32, i64, i32, i32, vp, vp]
-        if lib.woq_hip_abi_version() != 1:
+        if lib.woq_hip_abi_version() != 2:
             raise RuntimeError("libwoq_hip.so has an unexpected ABI version")
         _lib = lib
     return _lib

@@ -42,7 +42,9 @@ PLAIN_WEIGHT_FORMAT, GPTQ_WEIGHT_FORMAT, AWQ_WEIGHT_FORMAT = 0, 1, 2
 
 _contexts = {}
 _contexts_lock = threading.Lock()
-_next_handle = [1]
+# Handles of this ctypes twin are negative, those of the registered custom class (torch_binding.cpp) positive:
+# a handle of one kind given to an operator of the other kind raises instead of naming some live context there.
+_next_handle = [-1]
 
 
 def _to_gpu(t, device=None):
@@ -166,10 +168,11 @@ class WoqLinearOpContext:
         self.at_bias_ = _to_gpu(bias, dev)
         self.bias_f32_ = self.at_bias_.to(torch.float32).contiguous() if self.at_bias_ is not None else None
         self.at_weight_ = _kernels.pack_weight(weight, weight_dtype, N, K)
-        s32, s16, sb16, z8, sz = _kernels.pack_qparams(scales, zero_points, weight_dtype)
+        s32, s16, sb16, z8, sz, szb = _kernels.pack_qparams(scales, zero_points, weight_dtype)
         self.scales_list_ = [s32, s16, sb16]
         self.zeros_u8_ = z8
         self.scale_zero_f16x2_ = sz
+        self.scale_zero_bf16_ = szb
         self.scales_plain_ = scales if group_size > 0 else scales.reshape(N)
         self.zero_points_plain_ = (
             None if zero_points is None else (zero_points if group_size > 0 else zero_points.reshape(N))
@@ -177,7 +180,7 @@ class WoqLinearOpContext:
         self.cached_compensation_ = None
         with _contexts_lock:
             self._handle = _next_handle[0]
-            _next_handle[0] += 1
+            _next_handle[0] -= 1
             _contexts[self._handle] = weakref.ref(self)
 
     def __del__(self):
@@ -283,6 +286,7 @@ class WoqLinearOpContext:
             p.scales_bf16 = self.scales_list_[2].data_ptr()
             p.zeros_u8 = self.zeros_u8_.data_ptr() if self.zeros_u8_ is not None else None
             p.scale_zero_f16x2 = self.scale_zero_f16x2_.data_ptr() if self.scale_zero_f16x2_ is not None else None
+            p.scale_zero_bf16 = self.scale_zero_bf16_.data_ptr() if self.scale_zero_bf16_ is not None else None
             p.group_size = self.group_size_
             p.bias = self.bias_f32_.data_ptr() if self.bias_f32_ is not None else None
             p.lowp_mode = self.lowp_mode_
@@ -323,12 +327,11 @@ class WoqLinearOpContext:
             int8 = self.lowp_mode_ == _lib.LOWP_INT8
             if int8:  # the quantized activations and their scales
                 wbytes = lib.woq_hip_linear_workspace_bytes(M, K, _lib.LOWP_INT8, self.act_quant_mode_, self.group_size_)
-            if ((M <= 32 and K >= 8192 and N <= 4096) and not int8) or (M > 64 and K >= 4096 and M * N <= 1048576):
-                # long K and few output tiles: scratch with which the decode kernel or the prefill GEMMs may
-                # share K between workgroups (the library decides), and the zeroed counters of this stream
-                extra = lib.woq_hip_linear_split_k_workspace_bytes(M, N)
-                if extra > 0:
-                    counters = _kernels._split_k_counters(x.device)
+            # long K and few output tiles: scratch with which the decode kernel or the prefill GEMMs share K
+            # between workgroups, and the zeroed counters of this stream (the library says for which problems)
+            extra = lib.woq_hip_linear_auto_split_k_workspace_bytes(M, K, N, self.lowp_mode_)
+            if extra > 0:
+                counters = _kernels._split_k_counters(x.device)
                 if counters is not None:
                     wbytes = (wbytes + 255) // 256 * 256 + extra
             if wbytes > 0:
@@ -391,6 +394,7 @@ class WoqLinearOpContext:
             self.lowp_mode_,
             self.act_quant_mode_,
             scale_zero_f16x2=self.scale_zero_f16x2_,
+            scale_zero_bf16=self.scale_zero_bf16_,
             fusion=fusion,
             others=others,
             **kw,
@@ -401,6 +405,11 @@ def _context_from_handle(handle):
     if handle.dtype != torch.int64 or handle.numel() != 1:
         raise RuntimeError("ipex_woq_linear: W_prepack must be the 1-element int64 tensor of get_data_handle()")
     key = handle.item()
+    if key > 0:
+        raise RuntimeError(
+            "ipex_woq_linear: this handle belongs to a torch.classes.ipex_prepack.WoqLinearOpContext; pass it to "
+            "torch.ops.torch_ipex.*, not to the ctypes twin in ipex_amd.ops"
+        )
     ref = _contexts.get(key)  # a single dict read: atomic under the interpreter lock
     ctx = ref() if ref is not None else None
     if ctx is None:

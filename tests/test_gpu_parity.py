@@ -84,7 +84,7 @@ def test_qparams_layout(cuda):
     N, KG = 40, 3
     s = torch.rand(N, KG) + 0.5
     z = torch.randint(0, 16, (N, KG)).float()
-    s32, s16, sb16, z8, sz = k.pack_qparams(s.to(cuda), z.to(cuda), 2)
+    s32, s16, sb16, z8, sz, szb = k.pack_qparams(s.to(cuda), z.to(cuda), 2)
     assert s32.shape == (3, KG, 16)
     sp = torch.ones(48, KG)
     sp[:N] = s
@@ -98,6 +98,19 @@ def test_qparams_layout(cuda):
     assert torch.equal(halves[..., 0], s16.cpu())
     want_z = 128 + zp.view(3, 16, KG).permute(0, 2, 1)
     assert torch.equal(halves[..., 1].float(), want_z)
+    # the bf16 kernels' dword: bf16 scale in the high half, the fp16 number 1024 + zero in the low half
+    m = szb.cpu()
+    assert torch.equal((m >> 16).to(torch.int16).view(torch.bfloat16), sb16.cpu())
+    assert torch.equal((m & 0xFFFF).to(torch.int16).view(torch.float16).float(), 1024 + zp.view(3, 16, KG).permute(0, 2, 1))
+    # symmetric 4-bit weights: the code of zero is 8; 8-bit weights: the stored byte (offset-binary), 128 when symmetric
+    assert torch.equal((k.pack_qparams(s.to(cuda), None, 2)[5].cpu() & 0xFFFF)[:2], torch.full((2, KG, 16), 0x6408, dtype=torch.int32))
+    z8b = torch.randint(-128, 128, (N, KG)).float()
+    m8 = k.pack_qparams(s.to(cuda), z8b.to(cuda), 1)[5].cpu()
+    zp8 = torch.zeros(48, KG)
+    zp8[:N] = z8b
+    assert torch.equal((m8 & 0xFFFF).to(torch.int16).view(torch.float16).float(), 128 + zp8.view(3, 16, KG).permute(0, 2, 1))
+    assert torch.equal((k.pack_qparams(s.to(cuda), None, 1)[5].cpu() & 0xFFFF), torch.full((3, KG, 16), 0x5800, dtype=torch.int32))
+    assert k.pack_qparams(s.to(cuda), None, 3)[5] is None  # NF4: no such table
 
 
 def test_compressed_zero_points(cuda):
@@ -179,6 +192,36 @@ def _check_fp(case, lowp_mode, ctx=None, cols=None, force_kernel=0, label=""):
         assert stats["rel_l2_out_vs_opt_fp16"] <= 6e-3, (label, stats)
     print(label, stats)
     return stats
+
+
+@pytest.mark.parametrize(
+    "kind,M,K,N,G,sym,bias",
+    [("int4", 16, 1024, 272, 128, False, True), ("int4", 8, 512, 96, 32, False, False), ("int4", 32, 384, 48, -1, True, True),
+     ("int4", 64, 1024, 544, 64, False, False), ("int4", 200, 1024, 512, 128, False, True), ("int4", 130, 512, 300, 32, True, False),
+     ("int4", 2048, 512, 448, 256, False, False), ("int8", 32, 512, 176, -1, True, True), ("int8", 7, 256, 64, 64, False, False)],
+)
+def test_merged_scale_zero_table_changes_no_bit(cuda, kind, M, K, N, G, sym, bias):
+    """The bf16 kernels read scale and zero point from one dword when the caller passes the merged table and from two
+    arrays when it does not (the registered woq_linear operator of the reference's argument list): the same bits out."""
+    syn = _synthetic()
+    if kind == "int4":
+        case = syn.make_int4_case(11, M, K, N, G, bias=bias)
+        if sym:
+            case["zeros"] = None
+    else:
+        case = syn.make_int8_case(11, M, K, N, group_size=G, bias=bias)
+        if not sym:
+            case["zeros"] = torch.randint(-128, 128, case["scales"].shape, generator=torch.Generator().manual_seed(5)).float()
+    ctx = make_context(case, O.LOWP_BF16)
+    assert ctx.scale_zero_bf16_ is not None
+    x = case["x"].cuda()
+    with_table = ctx.run(x, out_fp32=True)
+    kernel = _lib_last_kernel()
+    table, ctx.scale_zero_bf16_ = ctx.scale_zero_bf16_, None
+    without = ctx.run(x, out_fp32=True)
+    assert _lib_last_kernel() == kernel
+    ctx.scale_zero_bf16_ = table
+    assert torch.equal(with_table, without), (kernel, (with_table - without).abs().max().item())
 
 
 def test_c0_int4_g128_m1(cuda):

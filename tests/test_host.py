@@ -23,7 +23,7 @@ def test_library_exports_every_declared_symbol():
     lib = _lib.load()
     for name in declared:
         assert hasattr(lib, name), name
-    assert lib.woq_hip_abi_version() == 1
+    assert lib.woq_hip_abi_version() == 2
     # pure host-side helpers can be called without a GPU
     assert lib.woq_hip_padded_n(500) == 512
     assert lib.woq_hip_padded_k(2, 4096) == 4096 and lib.woq_hip_padded_k(2, 4097) == 4224
@@ -308,3 +308,24 @@ def test_ops_are_registered_with_reference_schemas():
     for name in ("weight_only_qlinear_prepack", "weight_only_qlinear_prepack_int4", "woq_linear_pack_weight",
                  "woq_linear_unpack_weight"):
         assert hasattr(torch.ops.ipex_prepack, name)
+
+
+def test_auto_split_k_predicate_is_the_library_s():
+    """The problems on which woq_hip_linear shares K between workgroups by itself, asked of the library (pure host
+    arithmetic): few output tiles and a long K; everything else gets no scratch."""
+    from ipex_amd import _lib
+
+    lib = _lib.load()
+    f = lib.woq_hip_linear_auto_split_k_workspace_bytes
+    full = lib.woq_hip_linear_split_k_workspace_bytes
+    BF16, INT8 = _lib.LOWP_BF16, _lib.LOWP_INT8
+    assert f(16, 14336, 4096, BF16) == full(16, 4096) > 0  # down projection at decode
+    assert f(16, 4096, 14336, BF16) == 0  # enough row-blocks
+    assert f(16, 4096, 4096, BF16) == 0  # K too short
+    assert f(4, 14336, 4096, BF16) == 0  # fewer than five rows: the integer-weight decode kernels never split
+    assert f(33, 14336, 4096, BF16) == 0
+    assert f(16, 14336, 4096, INT8) == 0  # the int8 decode kernel does not split
+    assert f(128, 4096, 4096, BF16) == full(128, 4096) > 0
+    assert f(128, 4096, 4096, INT8) == full(128, 4096)
+    assert f(2048, 4096, 14336, BF16) == 0
+    assert f(128, 2048, 4096, BF16) == 0
