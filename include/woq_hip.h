@@ -107,6 +107,11 @@ const char* woq_hip_last_error(void);
 /* ABI version; bumped whenever a struct or a layout below changes. */
 int woq_hip_abi_version(void);
 
+/* Rows below which lowp_mode BF16 computes in fp16 (the reference's fp16 kernel) instead of bf16: the value of the
+ * environment's IPEX_WOQ_SMALL_BATCH_THRESHOLD when the library first needed it, 5 by default
+ * (csrc/cpu/aten/utils/woq.h:24, csrc/cpu/aten/kernels/WoqLinearKrnl.cpp:77, 93). */
+int woq_hip_small_batch_threshold(void);
+
 /* Name of the kernel the calling thread enqueued last through any entry point below ("" before the
  * first launch), e.g. "woq_gemm_w4i8_kernel": lets a test or a profile script state which kernel served
  * a call.  No counterpart in the reference, whose kernel choice is visible only in its dispatch code
@@ -294,7 +299,8 @@ int woq_hip_linear(const woq_hip_linear_params* p);
  * before anything is launched; K is shared between workgroups only while that scratch fits as well.
  * Allocates nothing, on the device or through any library.  All calls on one GPU share the array: calls
  * that may overlap in time on one GPU (different streams, concurrent graph launches) race and must be
- * serialised by the caller. */
+ * serialised by the caller.  The first call on a device that needs the array looks up its address, which cannot
+ * happen under stream capture: such a call is rejected, so make one call on the device before capturing. */
 #define WOQ_HIP_NOALLOC_MAX_WORKSPACE_BYTES (12 * 1024 * 1024)
 int woq_hip_linear_noalloc(const woq_hip_linear_params* p);
 
@@ -386,23 +392,6 @@ int woq_hip_linear_grouped(const woq_hip_linear_params* p, const void* group, in
 int woq_hip_moe_combine_rows(void* out, int dtype, int64_t T, int64_t H, const void* expert_out,
                              const void* routing_weights, int64_t topk, const int32_t* row_of, const int32_t* slot_of,
                              int accumulate, void* stream);
-
-/* Measurement probes (no counterpart in the reference): the floor of an HBM-bound launch on this GPU.
- *   probe_stream_read: reads `bytes` from src once, `kib_per_wave` (1, 2, 4 or 8) KiB per wave as one
- *                      non-temporal dwordx4 load per lane and KiB, `waves_per_wg` (1..16) waves per
- *                      workgroup, no arithmetic, nothing written (sink, one dword, may be NULL);
- *                      bytes must be whole workgroups.
- *   probe_empty:       an empty kernel of the given grid. */
-int woq_hip_probe_stream_read(const void* src, int64_t bytes, int waves_per_wg, int kib_per_wave, void* sink,
-                              void* stream);
-int woq_hip_probe_empty(int64_t workgroups, int waves_per_wg, void* stream);
-/*   probe_mfma_issue:  the matrix-instruction rate of waves that also issue other work: each of the 4 or 8 waves
- *                      of a workgroup (one or two per SIMD) runs `iters` rounds of 16 independent v_mfma_f32_16x16x32_bf16 with
- *                      `valu_per_16` fp32 FMAs and `lds_per_16` ds_read_b128 spread between them (instances:
- *                      (0,0) (16,0) (32,0) (40,0) (48,0) (64,0) (0,3) (0,8) (0,16) (32,3) (40,3) (48,3) (20,6));
- *                      src: 12 KiB of operand bytes; sink: NULL or one float per thread. */
-int woq_hip_probe_mfma_issue(const void* src, int valu_per_16, int lds_per_16, int64_t workgroups,
-                             int waves_per_workgroup, int iters, float* sink, void* stream);
 
 #ifdef __cplusplus
 }

@@ -3,8 +3,14 @@
 // flight together, non-temporal like the decode kernels' weight stream) and an empty kernel of the
 // same grid.  They let a benchmark state the floor that bounds an HBM-bound launch of a given size
 // next to the time of the kernel itself.  No counterpart in the reference.
+//
+// Built into a library of its own (libwoq_bench_probes.so) that only the benchmark loads: the product library and its
+// C ABI carry no measurement code.  Entry points return 0, -1 for arguments they do not take, or the hipError_t of
+// the launch.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
 #include "woq_common.h"
-#include "woq_internal.h"
 
 namespace woq {
 
@@ -76,18 +82,20 @@ __global__ __launch_bounds__(512) void probe_mfma_issue_kernel(const u4* __restr
 
 using namespace woq;
 
+static int bad_args() { return -1; }
+static int launched() { return (int)hipGetLastError(); }
+
 extern "C" {
 
-int woq_hip_probe_stream_read(const void* src, int64_t bytes, int waves_per_wg, int kib_per_wave, void* sink,
+int woq_bench_probe_stream_read(const void* src, int64_t bytes, int waves_per_wg, int kib_per_wave, void* sink,
                               void* stream) {
-  if (!src || bytes <= 0) return set_error("probe_stream_read: null source or no bytes");
-  if (waves_per_wg < 1 || waves_per_wg > 16) return set_error("probe_stream_read: 1..16 waves per workgroup");
+  if (!src || bytes <= 0) return bad_args();
+  if (waves_per_wg < 1 || waves_per_wg > 16) return bad_args();
   const int64_t per_wg = (int64_t)waves_per_wg * kib_per_wave * 1024;
   if (per_wg <= 0 || bytes % per_wg != 0)
-    return set_error("probe_stream_read: %lld bytes are not whole workgroups of %d waves x %d KiB", (long long)bytes,
-                     waves_per_wg, kib_per_wave);
+    return bad_args();
   const int64_t grid = bytes / per_wg;
-  if (grid > 0x7fffffff) return set_error("probe_stream_read: too many workgroups");
+  if (grid > 0x7fffffff) return bad_args();
   hipStream_t st = (hipStream_t)stream;
   const u4* s = (const u4*)src;
   uint32_t* k = (uint32_t*)sink;
@@ -96,23 +104,23 @@ int woq_hip_probe_stream_read(const void* src, int64_t bytes, int waves_per_wg, 
     case 2: probe_stream_read_kernel<2><<<(unsigned)grid, waves_per_wg * 64, 0, st>>>(s, k); break;
     case 4: probe_stream_read_kernel<4><<<(unsigned)grid, waves_per_wg * 64, 0, st>>>(s, k); break;
     case 8: probe_stream_read_kernel<8><<<(unsigned)grid, waves_per_wg * 64, 0, st>>>(s, k); break;
-    default: return set_error("probe_stream_read: kib_per_wave must be 1, 2, 4 or 8");
+    default: return bad_args();
   }
-  return check_launch("probe_stream_read_kernel");
+  return launched();
 }
 
-int woq_hip_probe_empty(int64_t workgroups, int waves_per_wg, void* stream) {
+int woq_bench_probe_empty(int64_t workgroups, int waves_per_wg, void* stream) {
   if (workgroups < 1 || workgroups > 0x7fffffff || waves_per_wg < 1 || waves_per_wg > 16)
-    return set_error("probe_empty: bad launch shape");
+    return bad_args();
   probe_empty_kernel<<<(unsigned)workgroups, waves_per_wg * 64, 0, (hipStream_t)stream>>>();
-  return check_launch("probe_empty_kernel");
+  return launched();
 }
 
-int woq_hip_probe_mfma_issue(const void* src, int valu_per_16, int lds_per_16, int64_t workgroups,
+int woq_bench_probe_mfma_issue(const void* src, int valu_per_16, int lds_per_16, int64_t workgroups,
                              int waves_per_workgroup, int iters, float* sink, void* stream) {
-  if (!src) return set_error("probe_mfma_issue: src must hold 12 KiB of operand bytes");
+  if (!src) return bad_args();
   if (workgroups < 1 || workgroups > 65536 || iters < 1 || (waves_per_workgroup != 4 && waves_per_workgroup != 8))
-    return set_error("probe_mfma_issue: bad launch shape (4 or 8 waves per workgroup)");
+    return bad_args();
   const unsigned threads = 64u * (unsigned)waves_per_workgroup;
   hipStream_t st = (hipStream_t)stream;
   const u4* s = (const u4*)src;
@@ -120,13 +128,13 @@ int woq_hip_probe_mfma_issue(const void* src, int valu_per_16, int lds_per_16, i
 #define WOQ_PROBE_MIX(V, L)                                                \
   if (valu_per_16 == V && lds_per_16 == L) {                               \
     probe_mfma_issue_kernel<V, L><<<g, threads, 0, st>>>(s, iters, sink);  \
-    return check_launch("probe_mfma_issue_kernel");                        \
+    return launched();                        \
   }
   WOQ_PROBE_MIX(0, 0) WOQ_PROBE_MIX(16, 0) WOQ_PROBE_MIX(32, 0) WOQ_PROBE_MIX(40, 0) WOQ_PROBE_MIX(48, 0)
   WOQ_PROBE_MIX(64, 0) WOQ_PROBE_MIX(0, 3) WOQ_PROBE_MIX(0, 8) WOQ_PROBE_MIX(0, 16) WOQ_PROBE_MIX(32, 3)
   WOQ_PROBE_MIX(40, 3) WOQ_PROBE_MIX(48, 3) WOQ_PROBE_MIX(20, 6)
 #undef WOQ_PROBE_MIX
-  return set_error("probe_mfma_issue: no instance for %d VALU and %d LDS reads per 16 MFMAs", valu_per_16, lds_per_16);
+  return bad_args();
 }
 
 }  // extern "C"

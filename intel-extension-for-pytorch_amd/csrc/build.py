@@ -15,7 +15,9 @@ from concurrent.futures import ThreadPoolExecutor
 HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_DIR = os.path.join(os.path.dirname(HERE), "lib")
 OBJ_DIR = os.path.join(HERE, "build")
-SOURCES = ["woq_api.hip", "woq_pack.hip", "woq_small_m.hip", "woq_decode.hip", "woq_decode_dq.hip", "woq_gemm.hip", "woq_gemm_w4.hip", "woq_gemm_w4s.hip", "woq_int8.hip", "woq_moe.hip", "woq_gemm_w4i8.hip", "woq_act_quant.hip", "woq_fp32.hip", "woq_probe.hip"]
+SOURCES = ["woq_api.hip", "woq_pack.hip", "woq_small_m.hip", "woq_decode.hip", "woq_decode_dq.hip", "woq_gemm.hip", "woq_gemm_w4.hip", "woq_gemm_w4s.hip", "woq_int8.hip", "woq_moe.hip", "woq_gemm_w4i8.hip", "woq_act_quant.hip", "woq_fp32.hip"]
+# measurement probes of bench.py: a library of their own, so that the product library carries none
+PROBE_SOURCE = "bench_probes.hip"
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
     "--offload-arch=gfx950",
@@ -33,6 +35,24 @@ def lib_path():
 
 def torch_lib_path():
     return os.path.join(LIB_DIR, "libwoq_torch.so")
+
+
+def probe_lib_path():
+    return os.path.join(LIB_DIR, "libwoq_bench_probes.so")
+
+
+def build_probes(verbose=True, incremental=False):
+    """hipcc on bench_probes.hip -> ../lib/libwoq_bench_probes.so (loaded by bench.py only)."""
+    src, out = os.path.join(HERE, PROBE_SOURCE), probe_lib_path()
+    if incremental and os.path.exists(out) and os.path.getmtime(out) > max(
+            os.path.getmtime(src), os.path.getmtime(os.path.join(HERE, "woq_common.h"))):
+        return out
+    res = subprocess.run([HIPCC, *FLAGS, "-shared", src, "-o", out], capture_output=True, text=True)
+    if res.returncode != 0:
+        raise RuntimeError("hipcc failed for bench_probes.hip:\n" + res.stderr[-4000:])
+    if verbose:
+        print("built", out)
+    return out
 
 
 def build_torch_binding(verbose=True, incremental=False):
@@ -97,6 +117,7 @@ def build(jobs=4, verbose=True, incremental=False):
     if verbose:
         print("built", lib_path())
     build_torch_binding(verbose, incremental)
+    build_probes(verbose, incremental)
     return lib_path()
 
 

@@ -192,6 +192,9 @@ static optional<Tensor> split_k_counters(const Tensor& like) {
 
 // ---- the prepack context ----------------------------------------------------------------------------
 static std::atomic<int64_t> g_next_handle{1};
+// Bumped whenever a context changes or frees its device arrays (load_from_ctx, release): whoever caches the
+// addresses of kernel_pointers() compares it before every use.
+static std::atomic<int64_t> g_context_epoch{0};
 static void unregister_context(int64_t handle);
 
 // Prepacked weight and quantization parameters of one linear layer (ContextLinearWoq /
@@ -213,6 +216,7 @@ class WoqLinearOpContext : public torch::CustomClassHolder {
   // Runs when the last owner lets go (the table of live contexts holds a weak reference, so this, not the
   // destructor, is the first thing to happen): the handle stops resolving and the device memory is freed.
   void release_resources() override {
+    g_context_epoch.fetch_add(1);
     unregister_context(handle_);
     packed_ = Tensor();
     q_ = PackedQParams();
@@ -271,6 +275,7 @@ class WoqLinearOpContext : public torch::CustomClassHolder {
   }
   void load_from_ctx(const c10::intrusive_ptr<WoqLinearOpContext>& other) {
     const int64_t keep = handle_;
+    g_context_epoch.fetch_add(1);
     copy_state(*other);
     handle_ = keep;
   }
@@ -889,6 +894,8 @@ TORCH_LIBRARY_FRAGMENT(ipex_prepack, m) {
       "woq_linear_pack_weight(Tensor W, str W_dtype, int[] W_shape, Tensor scales, Tensor? zero_points, Tensor? B, "
       "Tensor? g_idx, int group_size, int lowp_mode) -> (Tensor, Tensor[], Tensor[]?, Tensor[]?, Tensor?)");
   m.def("woq_linear_unpack_weight(Tensor W, str W_dtype, int[] W_shape, int lowp_mode) -> Tensor");
+  // no counterpart in the reference: see g_context_epoch
+  m.def("woq_context_epoch() -> int", []() -> int64_t { return g_context_epoch.load(); });
 }
 
 // The prepack ops take checkpoint tensors wherever they live (the reference registers them for CPU

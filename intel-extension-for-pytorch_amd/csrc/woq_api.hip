@@ -1,6 +1,7 @@
 // extern "C" entry points: argument validation, regime / kernel selection, launches.
 #include <stdarg.h>
 #include <stdio.h>
+#include <stdlib.h>
 #include <string.h>
 
 #include <mutex>
@@ -34,6 +35,19 @@ static bool valid_wdtype(int d) {
 }
 static bool wdtype_is_8bit(int d) { return d == WOQ_HIP_DTYPE_INT8 || d == WOQ_HIP_DTYPE_FP8; }
 
+// Rows below which lowp_mode BF16 computes in fp16: IPEX_WOQ_SMALL_BATCH_THRESHOLD, default 5, read once
+// (csrc/cpu/aten/utils/woq.h:24, used at csrc/cpu/aten/kernels/WoqLinearKrnl.cpp:77, 93).
+static int small_batch_threshold() {
+  static const int value = [] {
+    const char* env = getenv("IPEX_WOQ_SMALL_BATCH_THRESHOLD");
+    if (!env || !*env) return 5;
+    char* end = nullptr;
+    const long v = strtol(env, &end, 10);
+    return (end && *end == '\0' && v >= 0 && v <= 1 << 20) ? (int)v : 5;
+  }();
+  return value;
+}
+
 }  // namespace woq
 
 using namespace woq;
@@ -43,6 +57,8 @@ extern "C" {
 const char* woq_hip_last_error(void) { return g_err; }
 
 int woq_hip_abi_version(void) { return 2; }
+
+int woq_hip_small_batch_threshold(void) { return small_batch_threshold(); }
 
 const char* woq_hip_last_kernel(void) { return g_last_kernel; }
 
@@ -229,11 +245,11 @@ int woq_hip_linear(const woq_hip_linear_params* p) {
     }
   }
 
-  // Floating-point regimes (csrc/cpu/aten/kernels/WoqLinearKrnl.cpp:75-112; the small-batch
-  // threshold 5 is IPEX_WOQ_SMALL_BATCH_THRESHOLD, csrc/cpu/aten/utils/woq.h:24).
+  // Floating-point regimes (csrc/cpu/aten/kernels/WoqLinearKrnl.cpp:75-112; the small-batch threshold
+  // is the environment's IPEX_WOQ_SMALL_BATCH_THRESHOLD, 5 by default, csrc/cpu/aten/utils/woq.h:24).
   int regime;
   if (lowp == WOQ_HIP_LOWP_FP16 || (lowp == WOQ_HIP_LOWP_NONE && p->x_dtype == WOQ_HIP_ACT_FP16) ||
-      (lowp == WOQ_HIP_LOWP_BF16 && p->M < 5)) {
+      (lowp == WOQ_HIP_LOWP_BF16 && p->M < small_batch_threshold())) {
     regime = kRegimeF16;
   } else if ((lowp == WOQ_HIP_LOWP_NONE && p->x_dtype == WOQ_HIP_ACT_BF16) || lowp == WOQ_HIP_LOWP_BF16) {
     regime = kRegimeBF16;
@@ -357,7 +373,7 @@ int woq_hip_linear_grouped(const woq_hip_linear_params* p, const void* group, in
   // the regimes of woq_hip_linear (csrc/cpu/aten/kernels/WoqLinearKrnl.cpp:75-112), with M the bound on a slot's rows
   int regime;
   if (p->lowp_mode == WOQ_HIP_LOWP_FP16 || (p->lowp_mode == WOQ_HIP_LOWP_NONE && p->x_dtype == WOQ_HIP_ACT_FP16) ||
-      (p->lowp_mode == WOQ_HIP_LOWP_BF16 && p->M < 5))
+      (p->lowp_mode == WOQ_HIP_LOWP_BF16 && p->M < small_batch_threshold()))
     regime = kRegimeF16;
   else
     regime = kRegimeBF16;
@@ -477,13 +493,19 @@ constexpr int kMaxDevices = 64;
 static std::mutex g_scratch_mutex;
 static unsigned char* g_scratch_ptr[kMaxDevices] = {};
 
-static int scratch_of_current_device(unsigned char** out) {
+static int scratch_of_current_device(unsigned char** out, hipStream_t stream) {
   int dev = -1;
   hipError_t err = hipGetDevice(&dev);
   if (err != hipSuccess) return set_error("woq_linear_noalloc: hipGetDevice: %s", hipGetErrorString(err));
   if (dev < 0 || dev >= kMaxDevices) return set_error("woq_linear_noalloc: device index %d out of range", dev);
   std::lock_guard<std::mutex> lock(g_scratch_mutex);
   if (!g_scratch_ptr[dev]) {
+    // The address is looked up once per device, and not under stream capture (the lookup may load the code
+    // object, which a capturing stream does not allow): the first call on a device must come before the capture.
+    hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(stream, &status) != hipSuccess || status != hipStreamCaptureStatusNone)
+      return set_error("woq_linear_noalloc: the first call on a device looks up the resident scratch and cannot be "
+                       "captured; call woq_hip_linear_noalloc once on this device before capturing");
     void* ptr = nullptr;
     err = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
     if (err != hipSuccess || !ptr)
@@ -494,7 +516,7 @@ static int scratch_of_current_device(unsigned char** out) {
   return 0;
 }
 
-__global__ void zero_counters_kernel(int32_t* p, int n) {
+static __global__ void woq_zero_counters_kernel(int32_t* p, int n) {
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
   if (i < n) p[i] = 0;
 }
@@ -531,16 +553,16 @@ int woq_hip_linear_noalloc(const woq_hip_linear_params* p) {
   woq_hip_linear_params q = *p;
   if (need > 0) {
     unsigned char* ptr = nullptr;
-    if (int rc = scratch_of_current_device(&ptr)) return rc;
+    if (int rc = scratch_of_current_device(&ptr, (hipStream_t)p->stream)) return rc;
     q.workspace = ptr + kNoAllocCounterBytes;
     q.workspace_bytes = need;
     if (split) {
       // every finished launch leaves the counters at zero; a fill kernel (not a memset node, so that the
       // call can be captured into a HIP graph) makes that hold whatever ran before
       q.split_k_counters = (int32_t*)ptr;
-      zero_counters_kernel<<<(kSplitKCounters + 255) / 256, 256, 0, (hipStream_t)p->stream>>>(q.split_k_counters,
-                                                                                              kSplitKCounters);
-      if (int rc = check_launch("zero_counters_kernel")) return rc;
+      woq_zero_counters_kernel<<<(kSplitKCounters + 255) / 256, 256, 0, (hipStream_t)p->stream>>>(q.split_k_counters,
+                                                                                                  kSplitKCounters);
+      if (int rc = check_launch("woq_zero_counters_kernel")) return rc;
     }
   }
   return woq_hip_linear(&q);

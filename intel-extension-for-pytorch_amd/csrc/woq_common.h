@@ -314,6 +314,14 @@ struct G4Consts<kRegimeF16> {
   }
 };
 
+// Chunk swizzle of an LDS row of 128 bytes (8 chunks of 16 bytes; chunk q of row m is kept at q ^ swz_row128(m)):
+// distinct over any 8 consecutive rows, and over the even and the odd rows of 16, so that a fragment read -- 16
+// rows x one chunk per lane column -- touches every 16-byte bank group once whether the LDS serves 8 lanes x
+// 128 bytes or 16 lanes x 256 bytes at a time.  (With (m / 2) % 8 instead, rows m and m + 1 share a chunk
+// position and their lanes meet in the same banks when 8 lanes are served together: the bank-conflict counter
+// read 14.7 M cycles per launch of the int8 prefill kernel, of 33 M LDS-active ones.)
+__device__ __forceinline__ int swz_row128(int row) { return ((row >> 1) & 3) | (((row ^ (row >> 3)) & 1) << 2); }
+
 struct G4Masks {
   uint32_t lo, hi, magic;  // 0x000F000F, 0x00F000F0, fp16 1024 twice
 };

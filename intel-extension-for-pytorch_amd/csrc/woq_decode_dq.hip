@@ -18,7 +18,7 @@
 // Activations: a wave copies the rows of its K tile (16, 32 or 64 rows x 256 bytes for 4-bit weights,
 // x 128 bytes for 8-bit ones) straight into its private slice of LDS (global_load_lds_dwordx4:
 // fully coalesced, no registers) and reads the operand fragments from there; chunk p of row m sits
-// at p ^ m (p ^ (m / 2) for the 128-byte rows) so the fragment reads are conflict-free.  Reading
+// at p ^ m (p ^ swz_row128(m) for the 128-byte rows) so the fragment reads are conflict-free.  Reading
 // the fragments from global memory directly costs the same number of instructions but each one
 // gathers 64 separate 16-byte pieces, which made the texture addresser the bottleneck (M = 16:
 // 19.7 us against 13.9 us at M = 8 for the same weights).  Rows past M re-read row M - 1 and their
@@ -76,7 +76,7 @@ struct DqGeom {
   static constexpr int SLICE = MT * 16 * ROWB;    // one buffer of one wave
   static constexpr int NX = SLICE / 1024;         // LDS-load instructions per buffer
   static constexpr int NJ = TK / 32;              // MFMAs (32 K values each) per tile
-  static __device__ __forceinline__ int swz(int row) { return WBITS == 4 ? (row & 15) : ((row >> 1) & 7); }
+  static __device__ __forceinline__ int swz(int row) { return WBITS == 4 ? (row & 15) : swz_row128(row); }
 };
 
 // 8-bit weights: per-lane scale and offset of one row, c = -(128 + z) * s for the offset-binary

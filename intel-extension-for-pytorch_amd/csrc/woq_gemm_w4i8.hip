@@ -12,7 +12,7 @@
 // weight is decoded once per 64 rows by exactly one wave and never stored.  The activations
 // (already quantized, each group of eight in the order the nibble decode produces) and the packed
 // tiles go from global memory straight into LDS (global_load_lds_dwordx4), two K steps ahead; 16-byte
-// chunk p of activation row m sits at chunk p ^ ((m / 2) % 8), which makes the fragment reads
+// chunk p of activation row m sits at chunk p ^ swz_row128(m), which makes the fragment reads
 // conflict-free for 128-byte rows.
 // The int32 sums of a K step (128 K values = the reference's K block) are scaled into fp32
 // accumulators right away: four VALU instructions per output element and step, which is what
@@ -204,14 +204,14 @@ __global__ __launch_bounds__(256, (GSUB > 1 ? 2 : 3)) void woq_gemm_w4i8_kernel(
   int32_t za_next = 0;
 
   // ---- activations: load i of wave w fills LDS KiB number w * XLOADS + i of a buffer: rows
-  // 8 (w * XLOADS + i) + lane / 8, physical chunk lane % 8 = logical chunk ^ ((row / 2) % 8).
+  // 8 (w * XLOADS + i) + lane / 8, physical chunk lane % 8 = logical chunk ^ swz_row128(row).
   // Rows past M re-read row M - 1; their results are never stored. ----
   uint32_t xoff[W8_XLOADS];
 #pragma unroll
   for (int i = 0; i < W8_XLOADS; ++i) {
     const int rowl = (wave * W8_XLOADS + i) * 8 + (lane >> 3);
     const int rowc = m0 + rowl < M ? rowl : M - 1 - m0;
-    const int chunk = (lane & 7) ^ ((rowl >> 1) & 7);
+    const int chunk = (lane & 7) ^ swz_row128(rowl);
     xoff[i] = (uint32_t)(rowc * (int)a.ldq + chunk * 16);
   }
   const uint8_t* xbase = a.xq + (int64_t)m0 * a.ldq;
@@ -227,7 +227,7 @@ __global__ __launch_bounds__(256, (GSUB > 1 ? 2 : 3)) void woq_gemm_w4i8_kernel(
   uint32_t rd[2];
 #pragma unroll
   for (int j = 0; j < 2; ++j)
-    rd[j] = (uint32_t)(r * 128 + (((WBITS == 4 ? 2 * c + j : 4 * j + c) ^ ((r >> 1) & 7)) << 4));
+    rd[j] = (uint32_t)(r * 128 + (((WBITS == 4 ? 2 * c + j : 4 * j + c) ^ swz_row128(r)) << 4));
 
   // ---- weights ----
   const bool has_z = a.zeros != nullptr;
@@ -604,19 +604,19 @@ __global__ __launch_bounds__(512, (GSUB * MT > 4 ? 2 : 4)) void woq_decode_w4i8_
     for (int mt = 0; mt < MT; ++mt) acc[t][mt] = f4{0.f, 0.f, 0.f, 0.f};
 
   // activation load i fills LDS bytes [1024 i, +1024) of a buffer: rows 8 i + lane / 8, physical
-  // chunk lane % 8 = logical chunk ^ ((row / 2) % 8); rows past M re-read row M - 1
+  // chunk lane % 8 = logical chunk ^ swz_row128(row); rows past M re-read row M - 1
   uint32_t xoff[NX];
 #pragma unroll
   for (int i = 0; i < NX; ++i) {
     const int row = 8 * i + (lane >> 3);
     const int rowc = row < M ? row : M - 1;
-    const int chunk = (lane & 7) ^ ((row >> 1) & 7);
+    const int chunk = (lane & 7) ^ swz_row128(row);
     xoff[i] = (uint32_t)(rowc * (int)k.ldq + chunk * 16);
   }
   uint32_t rd[2];  // A fragment of MFMA j in row tile 0: row r, logical chunk 2 c + j (8-bit weights: 4 j + c)
 #pragma unroll
   for (int j = 0; j < 2; ++j)
-    rd[j] = (uint32_t)(r * 128 + ((((WBITS == 4 ? 2 * c + j : 4 * j + c)) ^ ((r >> 1) & 7)) << 4));
+    rd[j] = (uint32_t)(r * 128 + ((((WBITS == 4 ? 2 * c + j : 4 * j + c)) ^ swz_row128(r)) << 4));
 
   const bool has_z = k.zeros != nullptr;
   const uint8_t* wbase[NTW];

@@ -50,8 +50,7 @@ static_assert(GS_LDS <= 160 * 1024 && 8 * 16 * GS_SSTRIDE * 4 <= GS_LDS, "a work
 typedef __attribute__((address_space(3))) void* gs_lds_ptr_t;
 typedef const __attribute__((address_space(1))) void* gs_global_ptr_t;
 
-// Chunk swizzle of a row (128 bytes): distinct over any 8 consecutive rows, and over the even and the odd rows of 16.
-__device__ __forceinline__ int gs_swz(int row) { return ((row >> 1) & 3) | (((row ^ (row >> 3)) & 1) << 2); }
+__device__ __forceinline__ int gs_swz(int row) { return swz_row128(row); }
 
 template <int REGIME>
 __device__ __forceinline__ f4 gs_mfma(u4 a, u4 b, f4 c) {

@@ -23,6 +23,7 @@ TILE_N, TILE_BYTES, TILE_K_INT4, TILE_K_INT8 = 16, 1024, 128, 64
 EXPORTS = [
     "woq_hip_last_error",
     "woq_hip_abi_version",
+    "woq_hip_small_batch_threshold",
     "woq_hip_last_kernel",
     "woq_hip_padded_n",
     "woq_hip_padded_k",
@@ -44,9 +45,6 @@ EXPORTS = [
     "woq_hip_shuffle_int4_weight",
     "woq_hip_moe_gather_rows",
     "woq_hip_moe_scale_add_rows",
-    "woq_hip_probe_stream_read",
-    "woq_hip_probe_empty",
-    "woq_hip_probe_mfma_issue",
     "woq_hip_moe_route",
     "woq_hip_linear_grouped",
     "woq_hip_moe_combine_rows",
@@ -111,6 +109,8 @@ def load():
         lib.woq_hip_last_error.restype = ctypes.c_char_p
         lib.woq_hip_last_error.argtypes = []
         lib.woq_hip_abi_version.restype = i32
+        lib.woq_hip_small_batch_threshold.restype = i32
+        lib.woq_hip_small_batch_threshold.argtypes = []
         lib.woq_hip_last_kernel.restype = ctypes.c_char_p
         lib.woq_hip_last_kernel.argtypes = []
         lib.woq_hip_padded_n.restype = i64
@@ -153,18 +153,12 @@ def load():
         lib.woq_hip_moe_gather_rows.argtypes = [vp, i32, i64, i64, vp, i64, vp, vp]
         lib.woq_hip_moe_scale_add_rows.restype = i32
         lib.woq_hip_moe_scale_add_rows.argtypes = [vp, i32, i64, i64, vp, vp, i64, vp, vp, i64, vp]
-        lib.woq_hip_probe_stream_read.restype = i32
-        lib.woq_hip_probe_stream_read.argtypes = [vp, i64, i32, i32, vp, vp]
-        lib.woq_hip_probe_empty.restype = i32
-        lib.woq_hip_probe_empty.argtypes = [i64, i32, vp]
         lib.woq_hip_moe_route.restype = i32
         lib.woq_hip_moe_route.argtypes = [vp, i64, i64, i64, i64, i64, i32, i64, vp, vp, vp, vp, vp]
         lib.woq_hip_linear_grouped.restype = i32
         lib.woq_hip_linear_grouped.argtypes = [ctypes.POINTER(LinearParams), vp, i64]
         lib.woq_hip_moe_combine_rows.restype = i32
         lib.woq_hip_moe_combine_rows.argtypes = [vp, i32, i64, i64, vp, vp, i64, vp, vp, i32, vp]
-        lib.woq_hip_probe_mfma_issue.restype = i32
-        lib.woq_hip_probe_mfma_issue.argtypes = [vp, i32, i32, i64, i32, i32, vp, vp]
         if lib.woq_hip_abi_version() != 2:
             raise RuntimeError("libwoq_hip.so has an unexpected ABI version")
         _lib = lib

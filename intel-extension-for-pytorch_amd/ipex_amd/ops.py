@@ -42,6 +42,9 @@ PLAIN_WEIGHT_FORMAT, GPTQ_WEIGHT_FORMAT, AWQ_WEIGHT_FORMAT = 0, 1, 2
 
 _contexts = {}
 _contexts_lock = threading.Lock()
+# Bumped whenever a context of this module changes or frees its device arrays (load_from_ctx, destruction): whoever
+# caches device addresses of contexts (the grouped mixture-of-experts plans) compares it before every use.
+_context_epoch = [0]
 # Handles of this ctypes twin are negative, those of the registered custom class (torch_binding.cpp) positive:
 # a handle of one kind given to an operator of the other kind raises instead of naming some live context there.
 _next_handle = [-1]
@@ -185,6 +188,7 @@ class WoqLinearOpContext:
 
     def __del__(self):
         try:
+            _context_epoch[0] += 1
             with _contexts_lock:
                 _contexts.pop(self._handle, None)
         except Exception:
@@ -236,6 +240,7 @@ class WoqLinearOpContext:
         return torch.tensor([self._handle], dtype=torch.int64)
 
     def load_from_ctx(self, other):
+        _context_epoch[0] += 1
         self.__dict__.pop("_tls", None)  # cached parameter blocks point at the old tensors
         self.__dict__.update({k: v for k, v in other.__dict__.items() if k not in ("_handle", "_tls")})
 
@@ -623,6 +628,8 @@ def _is_python_context(ctx):
 def _run_context(ctx, x, fusion=_lib.FUSE_NONE, others=()):
     """One linear of an expert: ``ctx`` is a ``torch.classes.ipex_prepack.WoqLinearOpContext`` (the
     registered operators, by handle) or the ctypes twin of this module."""
+    if isinstance(ctx, torch.Tensor) and ctx.numel() == 1 and ctx.dtype == torch.int64 and ctx.item() < 0:
+        ctx = _context_from_handle(ctx)  # a handle of the ctypes twin (negative), resolved here
     if _is_python_context(ctx):
         return ctx.run(x, fusion=fusion, others=others)
     h = ctx if isinstance(ctx, torch.Tensor) else ctx.get_data_handle()
@@ -662,10 +669,21 @@ def mixtral_moe_woq(hidden_states, top_x, idx, gate_wei, up_wei, down_wei, routi
 
 
 # ---- a whole layer in grouped launches (decode sizes) -----------------------------------------------
-# (id of the gate list, stream) -> plan; the plan keeps the three lists alive, so the id stays theirs.  One plan per
-# stream: its routing buffers and intermediate rows are reused from call to call, and calls on one stream follow each other.
+# (identities of the experts' contexts, device, stream) -> plan.  A plan snapshots device addresses of its contexts and
+# holds none of them alive; it is valid while no context anywhere has changed or freed its arrays since the snapshot
+# (_context_epochs), which is checked before every use.  One plan per stream: its routing buffers are reused from call
+# to call, and calls on one stream follow each other.
 _MOE_PLANS = {}
 _MOE_PLAN_LIMIT = 128
+# (device, stream, dtype, intermediate width, hidden width) -> (act, inter, y) rows for the largest routing the grouped
+# path takes, allocated once and never moved, so that a HIP graph captured over a layer keeps valid addresses; shared
+# by all layers of those widths (calls on one stream follow each other).
+_MOE_ROWS = {}
+
+
+def _context_epochs():
+    """(epoch of this module's contexts, epoch of the registered custom class's contexts)."""
+    return _context_epoch[0], int(torch.ops.ipex_prepack.woq_context_epoch())
 
 
 def _context_pointers(ctx):
@@ -687,9 +705,9 @@ class _MoeGroupedPlan:
     intermediate rows."""
 
     def __init__(self, gate_ctx, up_ctx, down_ctx, device):
-        self.lists = (gate_ctx, up_ctx, down_ctx)
+        self.epochs = _context_epochs()  # before the snapshot: a change during it makes the plan stale, not wrong
         self.ok = False
-        infos = [[_context_pointers(c) for c in lst] for lst in self.lists]
+        infos = [[_context_pointers(c) for c in lst] for lst in (gate_ctx, up_ctx, down_ctx)]
         self.shapes = []
         for rows in infos:
             first = rows[0]
@@ -722,16 +740,16 @@ class _MoeGroupedPlan:
                 x["G"] % 128 == 0 and (x["G"] // 128) & (x["G"] // 128 - 1) == 0))
             for x in self.shapes)
         self.structs = {}
-        self.rows = {}  # dtype -> (act, inter, y) for the most routed rows seen
         self.device = device
         self.ok = True
 
-    def buffers(self, R, dtype):
-        have = self.rows.get(dtype)
-        if have is None or have[0].shape[0] < R:
-            N1, H = self.shapes[0]["N"], self.shapes[0]["K"]
-            mk = lambda n: torch.empty((R, n), dtype=dtype, device=self.device)
-            have = self.rows[dtype] = (mk(N1), mk(N1), mk(H))
+    def buffers(self, dtype, stream):
+        N1, H = self.shapes[0]["N"], self.shapes[0]["K"]
+        key = (self.device.index, stream, dtype, N1, H)
+        have = _MOE_ROWS.get(key)
+        if have is None:
+            mk = lambda n: torch.empty((_lib.MOE_ROUTE_MAX, n), dtype=dtype, device=self.device)
+            have = _MOE_ROWS[key] = (mk(N1), mk(N1), mk(H))
         return have
 
     def group_struct(self, linear, cls, f16_scales, gather, sz=False):
@@ -752,10 +770,12 @@ class _MoeGroupedPlan:
         return st
 
 
-def _moe_plan(gate_ctx, up_ctx, down_ctx, device):
-    key = (id(gate_ctx), device.index, torch.cuda.current_stream(device).cuda_stream)
+def _moe_plan(gate_ctx, up_ctx, down_ctx, device, stream):
+    # the contexts themselves, not the lists that hold them: a caller may build the lists anew for every call, or
+    # replace an expert inside a list
+    key = (tuple(map(id, gate_ctx)), tuple(map(id, up_ctx)), tuple(map(id, down_ctx)), device.index, stream)
     plan = _MOE_PLANS.get(key)
-    if plan is None or plan.lists[0] is not gate_ctx or plan.lists[1] is not up_ctx or plan.lists[2] is not down_ctx:
+    if plan is None or plan.epochs != _context_epochs():
         if len(_MOE_PLANS) >= _MOE_PLAN_LIMIT:
             _MOE_PLANS.clear()
         plan = _MoeGroupedPlan(gate_ctx, up_ctx, down_ctx, device)
@@ -763,8 +783,13 @@ def _moe_plan(gate_ctx, up_ctx, down_ctx, device):
     return plan
 
 
+def _small_batch_threshold():
+    """Rows below which lowp_mode BF16 computes in fp16: the library's reading of IPEX_WOQ_SMALL_BATCH_THRESHOLD."""
+    return (_lib._lib or _lib.load()).woq_hip_small_batch_threshold()
+
+
 def _f16_regime(lowp, x_dtype, rows):
-    return lowp == 1 or (lowp == 0 and x_dtype == torch.float16) or (lowp == 2 and rows < 5)
+    return lowp == 1 or (lowp == 0 and x_dtype == torch.float16) or (lowp == 2 and rows < _small_batch_threshold())
 
 
 def _deepseek_moe_grouped(hidden_states, topk_ids, gate_ctx, up_ctx, down_ctx, routing_weights):
@@ -775,6 +800,8 @@ def _deepseek_moe_grouped(hidden_states, topk_ids, gate_ctx, up_ctx, down_ctx, r
     x = hidden_states
     if x.dim() != 2 or x.dtype not in (torch.bfloat16, torch.float16) or not x.is_contiguous() or x.data_ptr() % 16:
         return None
+    if _small_batch_threshold() != 5:  # the size classes below are cut for the default threshold
+        return None
     T, H = x.shape
     if topk_ids.dim() != 2 or topk_ids.shape[0] != T or not topk_ids.is_cuda or topk_ids.device != x.device:
         return None
@@ -783,7 +810,8 @@ def _deepseek_moe_grouped(hidden_states, topk_ids, gate_ctx, up_ctx, down_ctx, r
         return None
     if routing_weights.dtype != x.dtype or routing_weights.dim() != 2 or tuple(routing_weights.shape) != (T, topk) or not routing_weights.is_cuda:
         return None
-    plan = _moe_plan(gate_ctx, up_ctx, down_ctx, x.device)
+    raw_stream = _current_raw_stream(x.device.index)
+    plan = _moe_plan(gate_ctx, up_ctx, down_ctx, x.device, raw_stream)
     if not plan.ok or plan.shapes[0]["K"] != H:
         return None
     lowp = plan.shapes[0]["lowp"]
@@ -793,11 +821,13 @@ def _deepseek_moe_grouped(hidden_states, topk_ids, gate_ctx, up_ctx, down_ctx, r
     single = plan.single_row and _f16_regime(lowp, x.dtype, 1)
     # lowp_mode BF16: experts with fewer than five rows compute in fp16, a class of their own
     split = 5 if (lowp == 2 or single) else 0
-    # (size class, bound on its slots' rows): an expert has at most T rows, so the larger classes are empty for small T
+    # (size class, bound on its slots' rows): an expert has at most T * topk entries (a token may name it in several of
+    # its slots), so the larger classes are empty while that bound is small
     # a single token: every (token, slot) entry is a slot of its own (an expert named twice included)
     each = single and T == 1 and topk <= plan.S
+    most = T * topk
     launches = [(3, 1)] if each else ([(3, 1)] if single else []) + ([(0, 4)] if split else []) + \
-               ([(1, 16)] if T >= split else []) + ([(2, 64)] if T > 16 else [])
+               ([(1, 16)] if most >= split else []) + ([(2, 64)] if most > 16 else [])
     for cls, bound in launches:
         f16 = _f16_regime(lowp, x.dtype, bound)
         # rows must be in the compute type; bf16 rows under fp16 compute are converted for up to 16 rows per slot
@@ -810,7 +840,7 @@ def _deepseek_moe_grouped(hidden_states, topk_ids, gate_ctx, up_ctx, down_ctx, r
     rw = routing_weights.contiguous()
     R = T * topk
     N1 = plan.shapes[0]["N"]
-    act, inter, y = plan.buffers(R, x.dtype)  # calls on one stream follow each other
+    act, inter, y = plan.buffers(x.dtype, raw_stream)  # calls on one stream follow each other
     out = torch.empty_like(x)
     code = _kernels._ACT_CODE[x.dtype]
     with torch.cuda.device(x.device):

@@ -10,6 +10,8 @@
  *     w = bf16((q - z) * s) with the subtraction and the product in fp32, bf16 x bf16 products
  *     accumulated in fp32, fp32 bias, caller rounds the result;
  *   - the fallback's fp16 regime for M < 5 (woq.h:3511-3613): w = fp16((q - z) * s);
+ *   - the optimized fp16 kernel for M < 5 (woq.h:775-951): fp16 fused multiply-adds on integer
+ *     weights per K block of 64, the scale applied to the block sum, fp16 accumulators;
  *   - per-row symmetric activation quantization (woq_dynamic_quant.h:1608-1648) and the int8
  *     block sums + fp32 epilogue (woq.h:2172-2186).
  * The reference blocks N by 32 and K by 64 for AVX-512 / AMX; this port keeps the plain
@@ -93,6 +95,58 @@ void woq_ref_linear_int4(const uint16_t* x, int64_t M, int64_t K, int64_t N, con
     free(w);
   }
   free(xf);
+}
+
+/* double -> fp16 with ONE rounding to nearest even (through a float rounded to odd). */
+static inline float round_f16_from_double(double d) {
+  float f = (float)d;
+  if ((double)f != d) {
+    uint32_t u;
+    memcpy(&u, &f, 4);
+    if (fabs((double)f) > fabs(d)) u -= 1;  /* towards zero */
+    u |= 1u;                                /* sticky bit */
+    memcpy(&f, &u, 4);
+  }
+  return round_f16(f);
+}
+
+/*
+ * The optimized fp16 kernel of the reference for fewer than five rows (GemmMicroKernel<half>,
+ * csrc/cpu/aten/utils/woq.h:775-951): activations rounded to fp16; per output and K block of
+ * block_k values vc = 0, vc = fma16(x_k, q_k - z, vc) for k ascending, then C = fma16(s, vc, C); C starts
+ * at the fp16 bias or 0 and is the fp16 result (returned as float).  fma16 = a * b + c rounded once to
+ * fp16: the products and sums of the inner chain are exact in double; the outer fma goes through the
+ * double-precision fma, whose own rounding could only matter when |C| exceeds |s * vc| by 2^30.
+ */
+void woq_ref_linear_int4_fp16_chain(const uint16_t* x, int64_t M, int64_t K, int64_t N, const uint8_t* qw,
+                                    const float* scales, const float* zeros, int64_t G, int64_t block_k,
+                                    const float* bias, int64_t n0, int64_t n1, float* out) {
+  const int64_t KG = G > 0 ? (K + G - 1) / G : 1;
+  const int64_t row_bytes = (K + 1) / 2;
+  float* xh = (float*)malloc(sizeof(float) * (size_t)(M * K));
+  for (int64_t i = 0; i < M * K; ++i) xh[i] = round_f16(bf16_to_f32(x[i]));
+#pragma omp parallel for schedule(static)
+  for (int64_t n = n0; n < n1; ++n) {
+    const uint8_t* qrow = qw + n * row_bytes;
+    for (int64_t m = 0; m < M; ++m) {
+      const float* xr = xh + m * K;
+      float C = bias ? round_f16(bias[n]) : 0.f;
+      for (int64_t k0 = 0; k0 < K; k0 += block_k) {
+        const int64_t g = G > 0 ? k0 / G : 0;
+        const float z = zeros ? round_f16(zeros[n * KG + g]) : 8.0f;
+        const float s = round_f16(scales[n * KG + g]);
+        float vc = 0.f;
+        for (int64_t k = k0; k < k0 + block_k && k < K; ++k) {
+          const uint8_t byte = qrow[k >> 1];
+          const float w = (float)((k & 1) ? (byte >> 4) : (byte & 0xF)) - z;
+          vc = round_f16_from_double((double)xr[k] * (double)w + (double)vc);
+        }
+        C = round_f16_from_double(fma((double)s, (double)vc, (double)C));
+      }
+      out[m * N + n] = C;
+    }
+  }
+  free(xh);
 }
 
 /* Per-row symmetric int8 quantization: s = max|x| / 127, q = clamp(rint(x / s), -128, 127). */

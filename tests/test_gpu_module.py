@@ -344,6 +344,74 @@ def test_context_free_op_matches_module(cuda):
         torch.ops.torch_ipex.woq_linear(x, packed, "int3", [96, 512], scales, zeros, bias, None, 128, 2, -1, None)
 
 
+def test_context_free_op_rejects_tensors_it_could_not_read(cuda):
+    """torch_ipex::woq_linear hands its tensor arguments to the kernels as raw device pointers: a tensor on the CPU, of
+    another dtype or of a size that does not fit [N, K] and the group size must raise, not reach a kernel."""
+    from ipex_amd.utils import synthetic
+
+    case = synthetic.make_int4_case(34, 6, 512, 96, 128, bias=True)
+    x = case["x"].to(cuda)
+    packed, scales, zeros, bias, comp = torch.ops.ipex_prepack.woq_linear_pack_weight(
+        case["qweight"].to(cuda), "int4", [96, 512], case["scales"].to(cuda), case["zeros"].to(cuda),
+        case["bias"].to(cuda), None, 128, 2,
+    )
+    call = lambda **kw: torch.ops.torch_ipex.woq_linear(
+        kw.get("x", x), kw.get("packed", packed), "int4", kw.get("shape", [96, 512]), kw.get("scales", scales),
+        kw.get("zeros", zeros), kw.get("bias", bias), None, kw.get("G", 128), 2, -1, None)
+    call()
+    cpu_list = lambda ts, i: [t.cpu() if j == i else t for j, t in enumerate(ts)]
+    with pytest.raises(RuntimeError, match="same device"):
+        call(packed=packed.cpu())
+    for i in range(3):
+        with pytest.raises(RuntimeError, match="same device"):
+            call(scales=cpu_list(scales, i))
+    with pytest.raises(RuntimeError, match="same device"):
+        call(zeros=cpu_list(zeros, 3))
+    with pytest.raises(RuntimeError, match="same device"):
+        call(bias=cpu_list(bias, 0))
+    with pytest.raises(RuntimeError, match="packed weight has"):
+        call(shape=[192, 512])  # twice the rows the packed tensor holds
+    with pytest.raises(RuntimeError, match="packed weight has"):
+        call(packed=packed.reshape(-1)[:-1024])
+    with pytest.raises(RuntimeError, match=r"scales\[1\] must be"):
+        call(scales=[scales[0], scales[1].float(), scales[2]])
+    with pytest.raises(RuntimeError, match=r"scales\[0\] must be"):
+        call(G=64)  # twice the groups the tables hold
+    with pytest.raises(RuntimeError, match=r"zeros\[3\] must be uint8"):
+        call(zeros=[zeros[0], zeros[1], zeros[2], zeros[3].to(torch.int32)])
+    with pytest.raises(RuntimeError, match="bias has"):
+        call(bias=[b[:50] for b in bias])
+    with pytest.raises(RuntimeError, match="weight_shape must be positive"):
+        call(shape=[0, 512], x=x)
+    # a post-op operand on the CPU is rejected by the context's operators as well
+    from helpers import make_torch_context
+
+    tctx = make_torch_context(case, 2)
+    other = torch.zeros(6, 96, dtype=torch.bfloat16)
+    with pytest.raises(RuntimeError, match="same device"):
+        torch.ops.torch_ipex.woq_linear_add(x, tctx.get_data_handle(), [other])
+    torch.ops.torch_ipex.woq_linear_add(x, tctx.get_data_handle(), [other.to(cuda)])
+
+
+def test_handles_of_the_two_bindings_do_not_cross(cuda):
+    """The ctypes twin (ipex_amd.ops) and the registered custom class number their contexts apart: a handle of one kind
+    given to an operator of the other raises instead of resolving to some live context of that kind."""
+    from ipex_amd import ops
+    from ipex_amd.utils import synthetic
+    from helpers import make_context, make_torch_context
+
+    case = synthetic.make_int4_case(35, 3, 256, 32, 128)
+    twin, registered = make_context(case, 2), make_torch_context(case, 2)
+    x = case["x"].to(cuda)
+    assert twin.get_data_handle().item() < 0 < registered.get_data_handle().item()
+    with pytest.raises(RuntimeError, match="does not come from"):
+        torch.ops.torch_ipex.ipex_woq_linear(x, twin.get_data_handle())
+    with pytest.raises(RuntimeError, match="belongs to a torch.classes"):
+        ops.ipex_woq_linear(x, registered.get_data_handle())
+    assert torch.equal(ops.ipex_woq_linear(x, twin.get_data_handle()),
+                       torch.ops.torch_ipex.ipex_woq_linear(x, registered.get_data_handle()))
+
+
 def test_k_mismatch_and_bad_arguments(cuda):
     from ipex_amd import ops
     from ipex_amd.utils import synthetic

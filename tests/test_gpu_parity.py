@@ -136,14 +136,28 @@ def test_dequant_weight_bit_exact(cuda, G):
 # ---------------------------------------------------------------------------------------------
 # floating-point paths
 # ---------------------------------------------------------------------------------------------
-def _check_fp(case, lowp_mode, ctx=None, cols=None, force_kernel=0, label=""):
-    """Runs the HIP path twice (output dtype and fp32 accumulator) and checks both oracles."""
+def _shipped_binding_output(case, lowp_mode, act_quant_mode=-1, g_idx=None):
+    """The same call through what a user of the package gets: the registered prepack operator, the TorchScript custom
+    class it returns and torch.ops.torch_ipex.ipex_woq_linear (lib/libwoq_torch.so)."""
+    tctx = make_torch_context(case, lowp_mode, act_quant_mode, g_idx=g_idx)
+    return torch.ops.torch_ipex.ipex_woq_linear(case["x"].cuda(), tctx.get_data_handle())
+
+
+def _check_fp(case, lowp_mode, ctx=None, cols=None, force_kernel=0, label="", shipped=False):
+    """Runs the HIP path twice (output dtype and fp32 accumulator) and checks both oracles.  ``shipped``: the output
+    of the registered operator on the custom class must equal, bit for bit, the output of the ctypes twin that the
+    oracle comparisons below are made on."""
     k = _kernels()
     ctx = ctx or make_context(case, lowp_mode)
     x = case["x"].cuda()
     N, K, G = case["N"], case["K"], case["group_size"]
     kw = dict(force_kernel=force_kernel)
-    y = to_np_f32(ctx.run(x, **kw))
+    y_t = ctx.run(x, **kw)
+    if shipped:
+        assert force_kernel == 0
+        y_s = _shipped_binding_output(case, lowp_mode)
+        assert y_s.dtype == y_t.dtype and torch.equal(y_s, y_t), (label, "registered operator differs from the ctypes twin")
+    y = to_np_f32(y_t)
     acc = ctx.run(x, out_fp32=True, **kw).cpu().numpy()
     c = case_np(case)
     M = c["x"].shape[0]
@@ -226,7 +240,43 @@ def test_merged_scale_zero_table_changes_no_bit(cuda, kind, M, K, N, G, sym, bia
 
 def test_c0_int4_g128_m1(cuda):
     case = _synthetic().make_int4_case(0, 1, 4096, 4096, 128)
-    _check_fp(case, O.LOWP_BF16, label="C0")
+    _check_fp(case, O.LOWP_BF16, label="C0", shipped=True)
+
+
+def test_single_row_kernel_converts_bf16_rows_toward_zero_outside_fp16_s_normal_range(cuda):
+    """The one-row decode kernel turns its bf16 row into fp16 with round-toward-zero (v_cvt_pkrtz_f16_f32): exact for
+    every bf16 value inside fp16's normal range, and a documented deviation from the reference's round-to-nearest
+    outside it -- below 2^-14 a value between two fp16 subnormals goes to the smaller one, and beyond 65504 the row
+    saturates at the largest finite fp16 instead of overflowing to infinity.  One planted activation at a time reads
+    the converted value out of the fp32 accumulator: acc[n] = fp16(x_k) * (q[n, k] - z[n]) * s[n]."""
+    K, N, G = 1024, 64, 128
+    case = _synthetic().make_int4_case(41, 1, K, N, G)
+    ctx = make_context(case, O.LOWP_BF16)
+    q = O.unpack_int4(case["qweight"].numpy())[:, :K].astype(np.float64)
+    s16 = case["scales"].numpy().astype(np.float16).astype(np.float64)  # fp16 scales in this regime
+    z = case["zeros"].numpy().astype(np.float64)
+    planted = [
+        # (value, what the kernel's conversion gives, what round-to-nearest-even gives)
+        (1.75 * 2.0 ** -24, 1.0 * 2.0 ** -24, 2.0 * 2.0 ** -24),    # between the first two subnormals
+        (-1.75 * 2.0 ** -24, -1.0 * 2.0 ** -24, -2.0 * 2.0 ** -24),
+        (1.5 * 2.0 ** -16, 1.5 * 2.0 ** -16, 1.5 * 2.0 ** -16),    # a subnormal that is exact: no deviation
+        (1.0078125 * 2.0 ** -14, 1.0078125 * 2.0 ** -14, 1.0078125 * 2.0 ** -14),  # normal range: exact
+        (99840.0, 65504.0, float("inf")),                            # beyond the largest finite fp16
+        (-3.0e38, -65504.0, float("-inf")),
+    ]
+    for k, (value, rtz, rne) in zip((3, 200, 517, 640, 901, 1023), planted):
+        x = torch.zeros(1, K, dtype=torch.bfloat16)
+        x[0, k] = value
+        assert float(x[0, k]) == value or abs(value) > 1e38  # representable in bf16 (the last one rounds, far beyond fp16)
+        acc = ctx.run(x.cuda(), out_fp32=True).double().cpu().numpy()[0]
+        assert _lib_last_kernel() == "woq_decode_m1_kernel"
+        w = (q[:, k] - z[:, k // G]) * s16[:, k // G]
+        want = rtz * w
+        assert np.all(np.isfinite(acc))
+        assert np.allclose(acc, want, rtol=1e-6, atol=0.0), (value, float(np.abs(acc - want).max()))
+        if rne != rtz:  # and it is not what round-to-nearest would have given
+            with np.errstate(invalid="ignore"):
+                assert not np.allclose(acc[w != 0], (rne * w)[w != 0], rtol=1e-3, atol=0.0)
 
 
 @pytest.mark.parametrize("M", [1, 4, 8, 16])
@@ -234,23 +284,23 @@ def test_c0_int4_g128_m1(cuda):
 def test_c2_decode_sweep(cuda, M, K, N):
     case = _synthetic().make_int4_case(2, M, K, N, 128)
     cols = np.arange(0, N, 7)  # every 7th output column keeps the oracle in seconds
-    _check_fp(case, O.LOWP_BF16, cols=cols, label=f"C2 M={M} K={K} N={N}")
+    _check_fp(case, O.LOWP_BF16, cols=cols, label=f"C2 M={M} K={K} N={N}", shipped=True)
 
 
 def test_c1_int8_per_channel_bias(cuda):
     case = _synthetic().make_int8_case(1, 32, 4096, 11008)
-    _check_fp(case, O.LOWP_BF16, cols=np.arange(0, 11008, 5), label="C1")
+    _check_fp(case, O.LOWP_BF16, cols=np.arange(0, 11008, 5), label="C1", shipped=True)
 
 
 @pytest.mark.parametrize("K,N", [(4096, 6144), (4096, 4096), (4096, 28672), (14336, 4096)])
 def test_c4_block_g32_m16(cuda, K, N):
     case = _synthetic().make_int4_case(4, 16, K, N, 32)
-    _check_fp(case, O.LOWP_BF16, cols=np.arange(0, N, 9), label=f"C4 K={K} N={N}")
+    _check_fp(case, O.LOWP_BF16, cols=np.arange(0, N, 9), label=f"C4 K={K} N={N}", shipped=True)
 
 
 def test_c3_prefill_bf16(cuda):
     case = _synthetic().make_int4_case(3, 2048, 4096, 14336, 128, outliers=True)
-    _check_fp(case, O.LOWP_BF16, cols=np.arange(0, 14336, 29), label="C3 bf16")
+    _check_fp(case, O.LOWP_BF16, cols=np.arange(0, 14336, 29), label="C3 bf16", shipped=True)
 
 
 @pytest.mark.parametrize("M", [1, 3, 5, 17, 33, 64, 65, 130, 257])
@@ -1085,12 +1135,15 @@ def test_dynamic_quant_all_bf16_patterns(cuda):
         assert np.array_equal(q.cpu().numpy(), q_ref)
 
 
-def _check_int8(case, mode, cols=None, debug=True, label=""):
+def _check_int8(case, mode, cols=None, debug=True, label="", shipped=False):
     ctx = make_context(case, O.LOWP_INT8, mode)
     x = case["x"].cuda()
     N, K, G = case["N"], case["K"], case["group_size"]
     c = case_np(case)
-    y = to_np_f32(ctx.run(x))
+    y_t = ctx.run(x)
+    if shipped:  # the registered operator on the custom class: the same bits
+        assert torch.equal(_shipped_binding_output(case, O.LOWP_INT8, mode), y_t), (label, "registered operator differs")
+    y = to_np_f32(y_t)
     # the accumulators of the kernel that serves the call, and (debug) those of the general kernel with
     # its block sums
     acc = ctx.run(x, out_fp32=True).cpu().numpy()
@@ -1263,7 +1316,7 @@ def test_int8_lowp_int8_weights_split_k(cuda, mode):
 
 def test_c3_prefill_int8(cuda):
     case = _synthetic().make_int4_case(3, 2048, 4096, 14336, 128, outliers=True)
-    _check_int8(case, 6, cols=np.arange(0, 14336, 61), debug=False, label="C3 int8 per-M")
+    _check_int8(case, 6, cols=np.arange(0, 14336, 61), debug=False, label="C3 int8 per-M", shipped=True)
     # bit-exact int32 block sums on a slice small enough to hold [M, N, K/128]
     small = dict(case)
     small["x"] = case["x"][:96]
@@ -1650,6 +1703,10 @@ def test_g_idx_matches_the_group_sorted_problem(cuda, M):
         ctx2 = pickle.loads(pickle.dumps(ctx))
         x = case["x"].cuda()
         assert torch.equal(ctx2.run(x), ctx.run(x))
+        # the registered operator on the custom class built with the same g_idx: the same bits
+        assert torch.equal(_shipped_binding_output(case, O.LOWP_BF16, g_idx=g_idx), ctx.run(x)), name
+        assert torch.equal(_shipped_binding_output(case, O.LOWP_INT8, 6, g_idx=g_idx),
+                           make_context(sorted_case, O.LOWP_INT8, 6).run(sorted_case["x"].cuda())), name
         # lowp INT8 goes through the same shuffles: identical to the context of the sorted problem
         ctx_i8 = ops.WoqLinearOpContext(
             case["qweight"].cuda(), 2, [N, K], case["scales"].cuda(), case["zeros"].cuda(), case["bias"].cuda(),
@@ -1682,6 +1739,8 @@ def test_g_idx_under_lowp_fp16_with_bf16_rows(cuda, M):
         ref = make_context(sorted_case, O.LOWP_FP16)
         y = ctx.run(case["x"].cuda())
         assert torch.equal(y, ref.run(sorted_case["x"].cuda())), name
+        # the registered operator on the custom class: one shuffle there too
+        assert torch.equal(_shipped_binding_output(case, O.LOWP_FP16, g_idx=g_idx), y), name
         c = case_np(sorted_case)
         _, want = O.woq_linear_ref(c["x"], "bf16", c["qw"], N, K, O._round_to(c["scales"], "fp16"), c["zps"], c["bias"],
                                    2, G, "fp16")

@@ -257,6 +257,12 @@ def test_c_port_of_oracle_matches_numpy_oracle():
                                 bias.ctypes.data, regime, 0, N, acc.ctypes.data)
         want, _ = O.woq_linear_ref(x, "bf16", qw, N, K, sc, zp, bias, 2, G, cd)
         assert np.max(np.abs(acc - want)) < 1e-4
+    # the optimized fp16 kernel's chain of fp16 fused multiply-adds: the same bits as the numpy restatement
+    lib.woq_ref_linear_int4_fp16_chain.argtypes = [vp, i64, i64, i64, vp, vp, vp, i64, i64, vp, i64, i64, vp]
+    for b in (bias, None):
+        lib.woq_ref_linear_int4_fp16_chain(xb.ctypes.data, M, K, N, qw.ctypes.data, sc.ctypes.data, zp.ctypes.data, G, 64,
+                                           None if b is None else b.ctypes.data, 0, N, acc.ctypes.data)
+        assert np.array_equal(O.bf16_round(acc), O.woq_linear_opt_fp16(x, qw, N, K, sc, zp, b, 2, G))
     # int8 path: quantization and block sums are exact, epilogue to fp32 rounding
     xq = np.zeros((M, K), dtype=np.int8)
     sa = np.zeros(M, dtype=np.float32)

@@ -87,3 +87,49 @@ def test_noalloc_plain_calls_and_rejections(cuda):
     p.workspace, p.workspace_bytes = x.data_ptr(), 1024
     assert _lib.load().woq_hip_linear_noalloc(ctypes.byref(p)) != 0
     assert b"must be null" in _lib.load().woq_hip_last_error()
+
+
+def test_noalloc_calls_captured_into_a_graph_replay_like_eager(cuda):
+    """What the entry point is for: a split-K call (counters re-zeroed by a fill kernel, partial tiles in the
+    resident scratch) and a lowp INT8 call (quantized activations there) recorded into one HIP graph after a
+    warm-up call outside the capture, replayed several times on new inputs with eager work in between; every
+    replay equals the eager woq_hip_linear result bit for bit."""
+    from ipex_amd import _kernels, _lib
+
+    syn = _synthetic()
+    split = syn.make_int4_case(56, 16, 8192, 512, 128, bias=True)
+    int8 = syn.make_int4_case(57, 150, 1024, 272, 128, bias=True, outliers=True)
+    ctxs = [make_context(split, O.LOWP_BF16), make_context(int8, O.LOWP_INT8, 6)]
+    xs = [split["x"].cuda(), int8["x"].cuda()]
+    static_x = [x.clone() for x in xs]
+
+    def call(ctx, x, noalloc):
+        N, K = ctx.weight_shape_
+        return _kernels.linear(x, ctx.at_weight_, ctx.weight_dtype_, N, K, *ctx.scales_list_, ctx.zeros_u8_,
+                               ctx.group_size_, ctx.bias_f32_, ctx.lowp_mode_, ctx.act_quant_mode_,
+                               scale_zero_f16x2=ctx.scale_zero_f16x2_, scale_zero_bf16=ctx.scale_zero_bf16_, noalloc=noalloc)
+
+    s = torch.cuda.Stream()
+    s.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(s):
+        kernels = []
+        for ctx, x in zip(ctxs, static_x):  # the warm-up: the scratch address of this device is looked up here
+            call(ctx, x, True)
+            kernels.append(_lib.last_kernel())
+    assert kernels == ["woq_decode_dq_kernel", "woq_gemm_w4i8_kernel"]
+    torch.cuda.current_stream().wait_stream(s)
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g, stream=s):
+        static_y = [call(ctx, x, True) for ctx, x in zip(ctxs, static_x)]
+    gen = torch.Generator(device="cpu").manual_seed(3)
+    for rep in range(4):
+        for sx, x in zip(static_x, xs):
+            sx.copy_((torch.randn(x.shape, generator=gen) * (1.0 + rep)).to(x.dtype))
+        g.replay()
+        torch.cuda.synchronize()
+        got = [y.clone() for y in static_y]
+        want = [call(ctx, x, False) for ctx, x in zip(ctxs, static_x)]  # eager work between the replays
+        torch.cuda.synchronize()
+        for a, b in zip(got, want):
+            assert torch.equal(a, b), rep
