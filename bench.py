@@ -548,9 +548,15 @@ def run_probe(name, torch, lib, lib_mod, ops_mod, synthetic, dev, stream):
         case = synthetic.make_int4_case(3, Mp, K, N, G, outliers=True)
         info["launches"] = []
         # (third: lowp_mode BF16 on the kernel that dequantizes once per workgroup into LDS)
-        for lowp, aq, forced in ((2, -1, 0), (3, 6, 0), (2, -1, 21)):
+        # (fourth: lowp_mode BF16 with cache_weight_for_large_batch, the dense kernel on the bf16 copy)
+        from ipex_amd import _kernels as kernels_mod
+        for lowp, aq, forced in ((2, -1, 0), (3, 6, 0), (2, -1, 21), (2, -1, 23)):
             params, keep = _rotating_params(torch, lib_mod, ops_mod, case, lowp, dev, stream, min_bytes=1, act_quant_mode=aq)
             params[0].force_kernel = forced
+            if forced == 23:
+                c = keep[2]
+                keep.append(kernels_mod.dense_weight(c.at_weight_, c.weight_dtype_, N, K, c.scales_list_[2], c.zeros_u8_, G))
+                params[0].dense_bf16 = keep[-1].data_ptr()
             for _ in range(20):
                 assert lib.woq_hip_linear(ctypes.byref(params[0])) == 0, lib.woq_hip_last_error()
             torch.cuda.synchronize()
@@ -917,10 +923,44 @@ def main():
                          "kernel": _lib.last_kernel()}
             if name == "bf16":
                 outp_host = outp.cpu()
+                # the same kernel with every launch reading its weights from HBM (rotating over the decode phase's
+                # copies), for the comparison with the dense copy below
+                rot = []
+                for c in keep[:12]:
+                    q = build_params(_lib, xp, c, outp, lowp, aq, ws)
+                    q.stream = stream.cuda_stream
+                    rot.append(q)
+                _, ms_r = time_groups(torch, lib, rot, steps_p, stream, groups=groups_p)
+                pre[name]["us_per_step_rotating_%d_copies" % len(rot)] = round(ms_r * 1e3 / steps_p, 2)
+                del rot
             if lowp == 3:  # integer products: against the i8 MFMA peak
                 pre[name]["frac_of_i8_mfma_peak"] = round(pre[name]["tflops"] / MFMA_I8_PEAK_TOPS, 4)
                 pre[name]["peak_tops"] = MFMA_I8_PEAK_TOPS
                 pre[name]["includes"] = "the activation quantization kernel"
+        # cache_weight_for_large_batch: the same problem on the dense bf16 copy of the weight (four times the packed
+        # bytes), first on one copy like the rows above, then rotating over three (351 MB: every launch reads its
+        # weights from HBM)
+        dense_copies = [_kernels.dense_weight(keep[0].at_weight_, keep[0].weight_dtype_, N, K, keep[0].scales_list_[2],
+                                              keep[0].zeros_u8_, G) for _ in range(3)]
+        cached = []
+        for d in dense_copies:
+            pp = build_params(_lib, xp, keep[0], outp, 2, -1, None)
+            pp.stream = stream.cuda_stream
+            pp.dense_bf16 = d.data_ptr()
+            cached.append(pp)
+        time_steps(torch, lib, cached[:1], 1, warm_p, stream)
+        _, ms = time_groups(torch, lib, cached[:1], steps_p, stream, groups=groups_p)
+        us = ms * 1e3 / steps_p
+        same_bits = bool(torch.equal(outp.cpu(), outp_host))
+        _, ms_r = time_groups(torch, lib, cached, steps_p, stream, groups=groups_p)
+        pre["bf16_weight_cache"] = {
+            "us_per_step": round(us, 2), "tflops": round(flops / (us * 1e-6) / 1e12, 1), "kernel": _lib.last_kernel(),
+            "frac_of_bf16_mfma_peak": round(flops / (us * 1e-6) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4),
+            "us_per_step_rotating_3_copies": round(ms_r * 1e3 / steps_p, 2),
+            "dense_copy_bytes": dense_copies[0].numel() * 2,
+            "output_equals_lowp_bf16_bit_for_bit": same_bits,
+        }
+        del dense_copies, cached
         # For scale: the vendor's dense bf16 GEMM (torch.matmul) on the same activations and the
         # already dequantized weight.  It does no dequantization; its rate on random data is what
         # this chip sustains for the shape (the clock drops under MFMA load with non-zero operands).
@@ -947,6 +987,7 @@ def main():
             "lowp_bf16": pre["bf16"],
             "lowp_int8_per_row": pre["int8"],
             "lowp_bf16_dequantized_tile_in_lds": pre["bf16_lds_tile"],
+            "lowp_bf16_cache_weight_for_large_batch": pre["bf16_weight_cache"],
             "dense_bf16_vendor_gemm_same_shape": {"us_per_step": round(us_d, 2),
                                                   "tflops": round(flops / (us_d * 1e-6) / 1e12, 1)},
             "frac_of_bf16_mfma_peak": round(pre["bf16"]["tflops"] / MFMA_BF16_PEAK_TFLOPS, 4),

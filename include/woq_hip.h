@@ -210,6 +210,9 @@ typedef struct woq_hip_linear_params {
   const uint32_t* scale_zero_bf16;  /* from woq_hip_pack_qparams, optional: with it the bf16 kernels on INT4 /
                                      * INT8 weights load one dword per (row, group) instead of a scale and a zero
                                      * point; results are the same bit for bit */
+  const void* dense_bf16;   /* from woq_hip_dense_weight, optional (cache_weight_for_large_batch): with it, lowp_mode
+                             * BF16 on bf16 activations runs batches of at least woq_hip_weight_cache_batch_threshold()
+                             * rows on the dense copy where that is the faster kernel; same results */
   int64_t group_size;       /* <= 0: per output channel */
   const float* bias;        /* fp32 [N] or NULL */
 
@@ -259,8 +262,10 @@ typedef struct woq_hip_linear_params {
    * 21 = prefill GEMM that dequantizes each weight once per workgroup into an LDS tile (256 rows x 224 columns,
    * 8 waves; 4-bit integer weights, otherwise the conditions of 3);
    * 22 = the dequantizing decode kernel (M <= 32, INT4 / INT8 weights) with three weight row-blocks per workgroup,
-   * which need not divide the row-blocks.
-   * NF4 weights: 0, 1, 2, 7, 8, 9, 13, 14, 16 only.
+   * which need not divide the row-blocks;
+   * 23 = dense bf16 GEMM on dense_bf16 (lowp_mode BF16, bf16 activations, K % 128 == 0; any M), workgroup shape by
+   * cost model; 24 / 25 / 26 = the same with 448 / 256 / 128 columns per workgroup.
+   * NF4 weights: 0, 1, 2, 7, 8, 9, 13, 14, 16 and 23..26 only.
    * fp32 compute (lowp_mode NONE with fp32 activations, csrc/cpu/aten/kernels/WoqLinearKrnl.cpp:142-158;
    * also lowp_mode INT8 on fp32 activations) has one kernel of its own and takes 0 only */
   int32_t force_kernel;
@@ -309,6 +314,21 @@ int woq_hip_linear_noalloc(const woq_hip_linear_params* p);
 int woq_hip_dequant_weight(const void* qweight, int weight_dtype, int64_t N, int64_t K,
                            const float* scales_f32, const uint8_t* zeros_u8,
                            int64_t group_size, void* out, int out_dtype, void* stream);
+
+/* Dense bf16 copy of a packed weight for large batches: what the reference caches under
+ * cache_weight_for_large_batch with lowp_mode BF16 (csrc/cpu/jit/cpu/kernels/LinearWoqPacked.cpp:430-486: the weight
+ * dequantized with the bf16 scales, w = bf16((q - z) * s), blocked for its GEMM; :511-526 uses it for at least
+ * IPEX_WOQ_WEIGHT_CACHE_BATCH_THRESHOLD rows).  Here the copy is laid out as the MFMA operands of the dense kernel
+ * ([K / 128][padded N / 16][4][64] fragments of 16 bytes), four times the packed 4-bit bytes.
+ * woq_hip_dense_weight_bytes: size of the copy, or 0 where none can be made (K not a multiple of 128, or a copy of
+ * 2 GiB and more).  woq_hip_dense_weight: writes it from the packed weight, the bf16 scales and the zero point
+ * bytes of woq_hip_pack_qparams.  woq_hip_weight_cache_batch_threshold: rows from which woq_hip_linear uses the
+ * copy, the environment's IPEX_WOQ_WEIGHT_CACHE_BATCH_THRESHOLD when the library first needed it, 64 by default
+ * (LinearWoqPacked.cpp:17-18). */
+int64_t woq_hip_dense_weight_bytes(int32_t weight_dtype, int64_t N, int64_t K);
+int woq_hip_dense_weight(const void* qweight, int32_t weight_dtype, int64_t N, int64_t K, const void* scales_bf16,
+                         const uint8_t* zeros_u8, int64_t group_size, void* dense, void* stream);
+int woq_hip_weight_cache_batch_threshold(void);
 
 /* dst[i] = src[i] converted, round to nearest even; dtypes WOQ_HIP_ACT_*; count elements.  With it a
  * caller runs lowp_mode FP16 on a bf16 tensor of any number of rows through the fp16 kernels: convert

@@ -15,7 +15,7 @@ from concurrent.futures import ThreadPoolExecutor
 HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_DIR = os.path.join(os.path.dirname(HERE), "lib")
 OBJ_DIR = os.path.join(HERE, "build")
-SOURCES = ["woq_api.hip", "woq_pack.hip", "woq_small_m.hip", "woq_decode.hip", "woq_decode_dq.hip", "woq_gemm.hip", "woq_gemm_w4.hip", "woq_gemm_w4s.hip", "woq_int8.hip", "woq_moe.hip", "woq_gemm_w4i8.hip", "woq_act_quant.hip", "woq_fp32.hip"]
+SOURCES = ["woq_api.hip", "woq_pack.hip", "woq_small_m.hip", "woq_decode.hip", "woq_decode_dq.hip", "woq_gemm.hip", "woq_gemm_w4.hip", "woq_gemm_w4s.hip", "woq_gemm_dense.hip", "woq_int8.hip", "woq_moe.hip", "woq_gemm_w4i8.hip", "woq_act_quant.hip", "woq_fp32.hip"]
 # measurement probes of bench.py: a library of their own, so that the product library carries none
 PROBE_SOURCE = "bench_probes.hip"
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")

@@ -242,12 +242,11 @@ class WoqLinearOpContext : public torch::CustomClassHolder {
             q_.sz.has_value() ? addr(*q_.sz) : 0};
   }
   optional<Tensor> get_g_idx() { return g_idx_; }
-  // The reference keeps a dequantized bf16 copy of the weight for batches of 64 rows and more when
-  // cache_weight_for_large_batch is set (csrc/cpu/jit/cpu/kernels/LinearWoqPacked.cpp:430-533), because
-  // its kernel dequantizes a weight block again for every 64 rows.  The prefill kernels here dequantize
-  // in registers once per 128 rows and run within 15 % of a dense bf16 GEMM on the same shape, so the
-  // flag is accepted, kept and pickled, and no copy (four times the packed weight's memory) is made.
-  optional<Tensor> get_cached_weight() { return c10::nullopt; }
+  // The dequantized bf16 copy of the weight that cache_weight_for_large_batch asks for under lowp_mode BF16
+  // (csrc/cpu/jit/cpu/kernels/LinearWoqPacked.cpp:430-486), in the operand layout of the dense kernel
+  // ([K / 128][padded N / 16][4][64][8] bf16); nothing where the flag is off or no copy can be made
+  // (K not a multiple of 128).  Made at prepack time, not on the first large batch: a forward call mutates nothing.
+  optional<Tensor> get_cached_weight() { return dense_.defined() ? optional<Tensor>(dense_) : c10::nullopt; }
   // The reference caches the column sums of an int8 copy of the weight for lowp_mode INT8
   // (LinearWoqPacked.cpp:485-508); here the int8 MFMA kernels read the stored codes and form those sums
   // on the fly, so there is nothing to cache.
@@ -394,12 +393,25 @@ class WoqLinearOpContext : public torch::CustomClassHolder {
     bias_f32_ = bias_.has_value() ? bias_->to(at::kFloat).contiguous() : Tensor();
     packed_ = pack_weight(weight, weight_dtype, N, K);
     q_ = pack_qparams(scales, zps, weight_dtype);
+    dense_ = Tensor();
+    if (cache_weight && lowp_mode == WOQ_HIP_LOWP_BF16) {
+      if (const int64_t bytes = woq_hip_dense_weight_bytes((int32_t)weight_dtype, N, K)) {
+        const int64_t nt = woq_hip_padded_n(N) / WOQ_HIP_TILE_N;
+        TORCH_CHECK(bytes == K / 128 * nt * 4 * 64 * 16, "WOQ linear: unexpected size of the dense copy");
+        dense_ = at::empty({K / 128, nt, 4, 64, 8}, packed_.options().dtype(at::kBFloat16));
+        DeviceScope scope(packed_);
+        check_rc(woq_hip_dense_weight(packed_.data_ptr(), (int32_t)weight_dtype, N, K, q_.sb16.data_ptr(),
+                                      q_.z8.has_value() ? q_.z8->data_ptr<uint8_t>() : nullptr, group_size,
+                                      dense_.data_ptr(), current_stream(packed_)),
+                 "woq_linear_prepack");
+      }
+    }
     scales_plain_ = group_size > 0 ? scales : scales.reshape({N});
     zeros_plain_ = zps.has_value() ? optional<Tensor>(group_size > 0 ? *zps : zps->reshape({N})) : c10::nullopt;
   }
 
   void copy_state(const WoqLinearOpContext& o) {
-    packed_ = o.packed_; q_ = o.q_; bias_ = o.bias_; bias_f32_ = o.bias_f32_; scales_plain_ = o.scales_plain_;
+    packed_ = o.packed_; q_ = o.q_; dense_ = o.dense_; bias_ = o.bias_; bias_f32_ = o.bias_f32_; scales_plain_ = o.scales_plain_;
     zeros_plain_ = o.zeros_plain_; g_idx_ = o.g_idx_; g_src_ = o.g_src_; g_dst_ = o.g_dst_;
     N_ = o.N_; K_ = o.K_; group_size_ = o.group_size_;
     weight_dtype_ = o.weight_dtype_; lowp_mode_ = o.lowp_mode_; act_quant_mode_ = o.act_quant_mode_;
@@ -437,6 +449,7 @@ class WoqLinearOpContext : public torch::CustomClassHolder {
     p.zeros_u8 = q_.z8.has_value() ? q_.z8->data_ptr<uint8_t>() : nullptr;
     p.scale_zero_f16x2 = q_.sz.has_value() ? (const uint32_t*)q_.sz->data_ptr() : nullptr;
     p.scale_zero_bf16 = q_.szb.has_value() ? (const uint32_t*)q_.szb->data_ptr() : nullptr;
+    p.dense_bf16 = dense_.defined() ? dense_.data_ptr() : nullptr;
     p.group_size = group_size_;
     p.bias = bias_f32_.defined() ? bias_f32_.data_ptr<float>() : nullptr;
     p.lowp_mode = (int32_t)lowp_mode_;
@@ -477,6 +490,7 @@ class WoqLinearOpContext : public torch::CustomClassHolder {
 
   Tensor packed_;
   PackedQParams q_;
+  Tensor dense_;  // cache_weight_for_large_batch under lowp_mode BF16: the dense bf16 copy, or undefined
   optional<Tensor> bias_;
   Tensor bias_f32_;
   Tensor scales_plain_;

@@ -48,6 +48,19 @@ static int small_batch_threshold() {
   return value;
 }
 
+// Rows from which lowp_mode BF16 uses the dense copy of the weight when the caller holds one:
+// IPEX_WOQ_WEIGHT_CACHE_BATCH_THRESHOLD, default 64, read once (csrc/cpu/jit/cpu/kernels/LinearWoqPacked.cpp:17-18, 517).
+static int weight_cache_batch_threshold() {
+  static const int value = [] {
+    const char* env = getenv("IPEX_WOQ_WEIGHT_CACHE_BATCH_THRESHOLD");
+    if (!env || !*env) return 64;
+    char* end = nullptr;
+    const long v = strtol(env, &end, 10);
+    return (end && *end == '\0' && v >= 0 && v <= 1 << 20) ? (int)v : 64;
+  }();
+  return value;
+}
+
 }  // namespace woq
 
 using namespace woq;
@@ -56,7 +69,28 @@ extern "C" {
 
 const char* woq_hip_last_error(void) { return g_err; }
 
-int woq_hip_abi_version(void) { return 2; }
+int woq_hip_abi_version(void) { return 3; }
+
+int woq_hip_weight_cache_batch_threshold(void) { return weight_cache_batch_threshold(); }
+
+int64_t woq_hip_dense_weight_bytes(int32_t weight_dtype, int64_t N, int64_t K) {
+  if (!valid_wdtype(weight_dtype) || N <= 0 || K <= 0 || K % 128 != 0) return 0;
+  const int64_t bytes = woq_hip_padded_n(N) * K * 2;
+  return bytes < (int64_t)1 << 31 ? bytes : 0;
+}
+
+int woq_hip_dense_weight(const void* qweight, int32_t weight_dtype, int64_t N, int64_t K, const void* scales_bf16,
+                         const uint8_t* zeros_u8, int64_t group_size, void* dense, void* stream) {
+  if (!valid_wdtype(weight_dtype)) return set_error("dense_weight: unsupported weight dtype %d", weight_dtype);
+  if (woq_hip_dense_weight_bytes(weight_dtype, N, K) == 0)
+    return set_error("dense_weight: no dense copy for N=%lld K=%lld (K must be a multiple of 128, the copy below 2 GiB)",
+                     (long long)N, (long long)K);
+  if (!qweight || !scales_bf16 || !dense) return set_error("dense_weight: null pointer");
+  if (group_size > 0 && group_size % 32 != 0) return set_error("dense_weight: group_size must be a multiple of 32");
+  const int64_t G = group_size > 0 ? group_size : woq_hip_padded_k(weight_dtype, K);
+  return launch_dense_weight(qweight, weight_dtype, N, K, (const uint16_t*)scales_bf16, zeros_u8, G, dense,
+                             (hipStream_t)stream);
+}
 
 int woq_hip_small_batch_threshold(void) { return small_batch_threshold(); }
 
@@ -284,6 +318,22 @@ int woq_hip_linear(const woq_hip_linear_params* p) {
   }
 
   int kernel = p->force_kernel;
+  // The dense copy (cache_weight_for_large_batch, csrc/cpu/jit/cpu/kernels/LinearWoqPacked.cpp:511-526: lowp_mode
+  // BF16, at least the threshold's rows): same operands into the same MFMAs as the kernels below, so same results.
+  if (kernel >= 23 && kernel <= 26) {
+    if (!p->dense_bf16 || regime != kRegimeBF16 || !gemm_dense_applies(f))
+      return set_error("woq_linear: the dense kernel takes dense_bf16, bf16 compute on bf16 activations and "
+                       "K %% 128 == 0");
+    return launch_gemm_dense(f, p->dense_bf16, wbits, st, kernel == 23 ? 0 : kernel == 24 ? 7 : kernel == 25 ? 4 : 2);
+  }
+  if (kernel == 0 && p->dense_bf16 && lowp == WOQ_HIP_LOWP_BF16 && regime == kRegimeBF16 &&
+      p->M >= weight_cache_batch_threshold() && p->M > 64 && gemm_dense_applies(f)) {
+    // ... where it is the faster kernel: against the prefill kernel that dequantizes in registers (a quarter of the
+    // bytes for the same MFMAs, and shapes of 64 rows) by the two cost models; weights that kernel does not take
+    // (NF4, groups that split a lane's K values) run on the general tiled kernel, which the dense one always beats
+    if (!gemm_w4_applies(f, wbits, regime) || gemm_dense_cost(f) < 0.97 * gemm_w4_cost(f, wbits))
+      return launch_gemm_dense(f, p->dense_bf16, wbits, st, 0);
+  }
   if (nf4) {
     // table lookups instead of the integer decode: the dequantizing decode kernel and the two
     // general kernels carry them

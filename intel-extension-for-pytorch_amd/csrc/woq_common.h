@@ -62,6 +62,26 @@ __host__ __device__ __forceinline__ constexpr int nibble_pos(int e) {
   return (e & 1) ? 4 + (e >> 1) : (e >> 1);
 }
 
+// ---- workgroup -> tile, by XCD ------------------------------------------------------------------
+// Workgroups are handed to the eight XCDs round robin in dispatch order (x fastest), and each XCD has an L2 of
+// its own.  With a grid whose width is no multiple of eight, the tiles of one XCD would be scattered over every
+// column block, and every L2 would fetch the whole weight.  This maps the dispatch order onto tiles so that an XCD
+// works on a contiguous range of them: tiles are numbered in bands of four column blocks (x fastest inside a band,
+// then y, then the next band), XCD k takes the k-th eighth of that numbering.  For a width that is a multiple of
+// 32 and any height this is what the hardware order gives anyway (four column blocks per XCD, rows in order).
+__device__ __forceinline__ void xcd_tile(int& tx, int& ty) {
+  const int gx = (int)gridDim.x, gy = (int)gridDim.y;
+  const int total = gx * gy;
+  const int id = (int)(blockIdx.y * gridDim.x + blockIdx.x);
+  const int xcd = id & 7, slot = id >> 3;
+  const int lin = xcd * (total >> 3) + (xcd < (total & 7) ? xcd : (total & 7)) + slot;
+  const int band = lin / (4 * gy);
+  const int within = lin - band * (4 * gy);
+  const int bw = gx - 4 * band < 4 ? gx - 4 * band : 4;
+  ty = within / bw;
+  tx = 4 * band + within - ty * bw;
+}
+
 // ---- 4-bit decode -------------------------------------------------------------------
 // (d >> 4v) & 0x000F000F | 0x6400_6400 is the fp16 pair (1024 + q[2v], 1024 + q[2v+1]).
 __device__ __forceinline__ h2 nib_pair_f16(uint32_t d, int v, uint32_t mask, uint32_t magic) {
@@ -317,9 +337,9 @@ struct G4Consts<kRegimeF16> {
 // Chunk swizzle of an LDS row of 128 bytes (8 chunks of 16 bytes; chunk q of row m is kept at q ^ swz_row128(m)):
 // distinct over any 8 consecutive rows, and over the even and the odd rows of 16, so that a fragment read -- 16
 // rows x one chunk per lane column -- touches every 16-byte bank group once whether the LDS serves 8 lanes x
-// 128 bytes or 16 lanes x 256 bytes at a time.  (With (m / 2) % 8 instead, rows m and m + 1 share a chunk
-// position and their lanes meet in the same banks when 8 lanes are served together: the bank-conflict counter
-// read 14.7 M cycles per launch of the int8 prefill kernel, of 33 M LDS-active ones.)
+// 128 bytes or 16 lanes x 256 bytes at a time.  (The prefill kernel with the dequantized tile in LDS reads its bf16
+// tiles this way with the bank-conflict counter at zero; the int8 kernels' fragment reads -- chunk 2 c + j instead of
+// 4 s + c -- still count four conflict cycles each, as they did with (m / 2) % 8, behind vector work that bounds them.)
 __device__ __forceinline__ int swz_row128(int row) { return ((row >> 1) & 3) | (((row ^ (row >> 3)) & 1) << 2); }
 
 struct G4Masks {

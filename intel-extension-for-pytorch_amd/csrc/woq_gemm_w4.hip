@@ -33,6 +33,8 @@
 //     nibble positions are read as the fp16 numbers 1024 + q and 64 + q, so that one scale serves both:
 //     7 instead of 14 parameter requests and 21 instead of 56 vector instructions per K step and wave
 //     (M = 2048, 4096 -> 14336: 198 against 202-206 us on the same boxes; same bits out).
+#include <algorithm>
+
 #include "woq_common.h"
 #include "woq_internal.h"
 
@@ -125,8 +127,10 @@ __global__ __launch_bounds__(256) void woq_gemm_w4_kernel(const FpArgs f, const 
   // that of its number whatever the split
   const int kt_lo = (int)blockIdx.z * kts;
   const int KT = KTW / TPS < kt_lo + kts ? KTW / TPS : kt_lo + kts;
-  const int m0 = blockIdx.y * G4_BM;
-  const int nt0 = (blockIdx.x * G4_WAVES + wave) * G4_NTW;  // first row-block of this wave
+  int bx, by;  // this workgroup's tile, by XCD (xcd_tile)
+  xcd_tile(bx, by);
+  const int m0 = by * G4_BM;
+  const int nt0 = (bx * G4_WAVES + wave) * G4_NTW;  // first row-block of this wave
 
   G4Masks km;
   asm volatile("s_mov_b32 %0, 0x000F000F" : "=s"(km.lo));
@@ -460,13 +464,14 @@ __global__ __launch_bounds__(256) void woq_gemm_w4_kernel(const FpArgs f, const 
   // (the output may be the other 16-bit type than the activations: fp16 rows converted from a bf16 tensor)
   const bool out_f16 = f.out_dtype == WOQ_HIP_ACT_FP16;
   const bool fast = f.fusion == WOQ_HIP_FUSE_NONE && (out_f16 || f.out_dtype == WOQ_HIP_ACT_BF16) && (f.N % 4) == 0 &&
-                    ncol0 + G4_NTW * kTileN <= f.N && (((uintptr_t)f.out & 7) | ((uintptr_t)f.bias & 15)) == 0;
+                    (((uintptr_t)f.out & 7) | ((uintptr_t)f.bias & 15)) == 0;
   const bool hb = f.bias != nullptr;
   if (fast) {
     f4 bias4[G4_NTW];
 #pragma unroll
     for (int t = 0; t < G4_NTW; ++t)
-      bias4[t] = hb ? *(const f4*)(f.bias + ncol0 + t * kTileN + 4 * c) : f4{0.f, 0.f, 0.f, 0.f};
+      bias4[t] = hb && ncol0 + t * kTileN + 4 * c < f.N ? *(const f4*)(f.bias + ncol0 + t * kTileN + 4 * c)
+                                                        : f4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int mt = 0; mt < G4_MT; ++mt) {
       const int m = m0 + mt * 16 + r;
@@ -486,7 +491,7 @@ __global__ __launch_bounds__(256) void woq_gemm_w4_kernel(const FpArgs f, const 
             o[0] = bitcast<uint32_t>(__builtin_convertvector(f2{y0, y1}, b2));
             o[1] = bitcast<uint32_t>(__builtin_convertvector(f2{y2, y3}, b2));
           }
-          *(u2*)(row + t * kTileN) = o;
+          if (ncol0 + t * kTileN + 4 * c < f.N) *(u2*)(row + t * kTileN) = o;  // (N % 4 == 0: all four or none)
         }
       }
     }
@@ -592,6 +597,26 @@ static int launch8(const FpArgs& f, int regime, int g_shift, hipStream_t st, int
                                 : launch_shape<kRegimeBF16, S, 8, true>(f, g_shift, st, splits, scratch);
   return regime == kRegimeF16 ? launch_shape<kRegimeF16, S, 8>(f, g_shift, st, splits, scratch)
                               : launch_shape<kRegimeBF16, S, 8>(f, g_shift, st, splits, scratch);
+}
+
+// Estimated time of the automatic choice below, in microseconds, for the comparison with the dense kernel
+// (gemm_dense_cost): per 4096 input channels a generation of 256 workgroups measured 92 / 58 / 37 us with 7 / 4 / 2
+// row-blocks per wave, the 64 x 128 shape 27 us while it fits one generation; the 128 x 128 shape beyond 512
+// workgroups (two share a CU) 68 us per 512 and 24-68 us for the rest; 8-bit weights a fifth more.
+double gemm_w4_cost(const FpArgs& f, int wbits) {
+  auto wgs = [&](int bm, int bn) { return ((f.NT * kTileN + bn - 1) / bn) * ((f.M + bm - 1) / bm); };
+  auto gens = [](int64_t w) { return (double)((w + 255) / 256); };
+  const int64_t w42 = wgs(64, 128), w2 = wgs(128, 128);
+  double c;
+  if (w42 <= 256) {
+    c = 27.0;
+  } else {
+    const int64_t rem = w2 % 512;
+    const double c2 = w2 <= 512 ? gens(w2) * 37.0 : 68.0 * (double)(w2 / 512) + (rem ? 24.0 + 44.0 * (double)rem / 512.0 : 0.0);
+    c = std::min(gens(wgs(128, 256)) * 58.0, c2);
+    if (wbits == 4) c = std::min(c, gens(wgs(128, 448)) * 92.0);
+  }
+  return c * (wbits == 8 ? 1.2 : 1.0) * (double)f.K / 4096.0;
 }
 
 int launch_gemm_w4(const FpArgs& f, int wbits, int regime, hipStream_t st, int shape, int splits,

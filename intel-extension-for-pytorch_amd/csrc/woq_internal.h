@@ -155,6 +155,16 @@ bool gemm_w4s_applies(const FpArgs& f, int wbits, int regime);
 int launch_gemm_w4s(const FpArgs& f, int regime, hipStream_t st);
 int launch_gemm_w4(const FpArgs& f, int wbits, int regime, hipStream_t st, int shape = 0, int splits = 0,
                    const SplitKScratch* scratch = nullptr);
+// Dense bf16 GEMM on the fragment-laid copy that launch_dense_weight writes (woq_gemm_dense.hip): bf16 activations,
+// K % 128 == 0; wbits selects the assignment of K values to lanes that the copy was written with;
+// shape: row-blocks per wave (7, 4 or 2), 0 = by cost model
+bool gemm_dense_applies(const FpArgs& f);
+// estimated microseconds of the dense kernel / of launch_gemm_w4's automatic choice on this problem
+double gemm_dense_cost(const FpArgs& f);
+double gemm_w4_cost(const FpArgs& f, int wbits);
+int launch_gemm_dense(const FpArgs& f, const void* dense, int wbits, hipStream_t st, int shape = 0);
+int launch_dense_weight(const void* qweight, int weight_dtype, int64_t N, int64_t K, const uint16_t* sb16,
+                        const uint8_t* z8, int64_t G, void* out, hipStream_t st);
 
 struct Int8Args {
   const void* x;

@@ -259,6 +259,70 @@ int launch_dequant_weight(const void* qweight, int weight_dtype, int64_t N, int6
   return check_launch("dequant_weight");
 }
 
+// ---- dense bf16 copy for large batches --------------------------------------------------------
+// The weight as the bf16 kernels would dequantize it, w = bf16((q - z) * s) with s the bf16 scale
+// (csrc/cpu/jit/cpu/kernels/LinearWoqPacked.cpp:430-486 caches the same values, blocked for its GEMM), laid out as
+// the MFMA operands of woq_gemm_dense_kernel: [K / 128][NT][4][64] fragments of 16 bytes, fragment (kt, nt, j, lane)
+// holding row 16 nt + lane % 16 and the eight K values 128 kt + 8 chunk .. + 7, chunk = 4 (lane / 16) + j for 4-bit
+// codes and 8 (j / 2) + 2 (lane / 16) + j % 2 for bytes -- the K values that the same lane and K sub-step of
+// woq_gemm_w4_kernel take from the packed tile, so that the two kernels feed identical operands to identical
+// instructions.  One thread per fragment.
+__global__ void dense_weight_kernel(const uint8_t* __restrict__ packed, int weight_dtype, int64_t NT, int64_t KT128,
+                                    int64_t KT, const uint16_t* __restrict__ sb16, const uint8_t* __restrict__ z8,
+                                    int64_t G, int64_t KG, u4* __restrict__ out) {
+  const int64_t gid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (gid >= KT128 * NT * 256) return;
+  const int lane = (int)(gid & 63), j = (int)((gid >> 6) & 3);
+  const int64_t nt = (gid >> 8) % NT, kt128 = (gid >> 8) / NT;
+  const int r = lane & 15, c = lane >> 4;
+  const bool fp8 = weight_dtype == WOQ_HIP_DTYPE_FP8;
+  const bool w4 = weight_dtype != WOQ_HIP_DTYPE_INT8 && !fp8;
+  const bool nf4 = weight_dtype == WOQ_HIP_DTYPE_NF4;
+  const int chunk = w4 ? 4 * c + j : 8 * (j / 2) + 2 * c + (j % 2);
+  const int64_t k0 = kt128 * 128 + chunk * 8;
+  int64_t g = G > 0 ? k0 / G : 0;
+  if (g >= KG) g = KG - 1;
+  const float s = bf16_bits_to_f32(sb16[(nt * KG + g) * kTileN + r]);
+  const float z = z8 ? (float)z8[(nt * KG + g) * kTileN + r] : (w4 ? 8.0f : 128.0f);
+  float w[8];
+  if (w4) {
+    const uint32_t d = ((const uint32_t*)packed)[((nt * KT + kt128) * 64 + lane) * 4 + j];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) w[e] = (float)((d >> (4 * nibble_pos(e))) & 0xFu);
+  } else {
+    const int64_t kt = k0 / kTileK8;
+    const int koff = (int)(k0 % kTileK8);
+    const uint8_t* p = packed + ((nt * KT + kt) * 64 + (r + 16 * (koff / 16))) * 16 + koff % 16;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) w[e] = fp8 ? fp8_e4m3fn_to_f32(p[e]) : (float)p[e];
+  }
+  uint32_t o[4];
+#pragma unroll
+  for (int e = 0; e < 8; e += 2) {
+    float v[2];
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+      v[h] = nf4 ? __fmul_rn(kNf4Values[(int)w[e + h]], s)
+                 : fp8 ? __fmul_rn(w[e + h], s) : __fmul_rn(__fsub_rn(w[e + h], z), s);
+    o[e / 2] = (uint32_t)f32_to_bf16_bits(v[0]) | ((uint32_t)f32_to_bf16_bits(v[1]) << 16);
+  }
+  out[gid] = u4{o[0], o[1], o[2], o[3]};
+}
+
+int launch_dense_weight(const void* qweight, int weight_dtype, int64_t N, int64_t K, const uint16_t* sb16,
+                        const uint8_t* z8, int64_t G, void* out, hipStream_t st) {
+  if (N == 0 || K == 0) return 0;
+  if (K % 128 != 0) return set_error("dense_weight: K = %lld is not a multiple of 128", (long long)K);
+  const bool w8 = weight_dtype == WOQ_HIP_DTYPE_INT8 || weight_dtype == WOQ_HIP_DTYPE_FP8;
+  const int64_t NT = (N + kTileN - 1) / kTileN, KT128 = K / 128;
+  const int64_t KT = woq_hip_padded_k(weight_dtype, K) / (w8 ? kTileK8 : kTileK4);
+  const int64_t KG = G > 0 ? (K + G - 1) / G : 1;
+  const int64_t total = KT128 * NT * 256;
+  dense_weight_kernel<<<blocks_for(total, 256), 256, 0, st>>>((const uint8_t*)qweight, weight_dtype, NT, KT128, KT,
+                                                              sb16, z8, G, KG, (u4*)out);
+  return check_launch("dense_weight");
+}
+
 // ---- GPTQ act-order (g_idx): channel shuffles -------------------------------------------------
 // Reference: woq_shuffle_tensor_by_group_idx / woq_shuffle_weight_back_by_group_idx
 // (csrc/cpu/jit/cpu/kernels/LinearWoqPacked.cpp:777-954).  Channel j moves to position

@@ -102,6 +102,27 @@ def pack_qparams(scales, zeros, weight_dtype):
     return s32, s16, sb16, z8, sz, szb
 
 
+def dense_weight(qweight, weight_dtype, N, K, scales_bf16, zeros_u8, group_size):
+    """Dense bf16 copy of a packed weight in the operand layout of the dense kernel
+    ([K / 128, padded N / 16, 4, 64, 8] bf16), or None where none can be made (K % 128 != 0)."""
+    lib = _lib.load()
+    _require_cuda(qweight, "weight")
+    nbytes = lib.woq_hip_dense_weight_bytes(weight_dtype, N, K)
+    if nbytes == 0:
+        return None
+    nt = padded_n(N) // _lib.TILE_N
+    out = torch.empty((K // 128, nt, 4, 64, 8), dtype=torch.bfloat16, device=qweight.device)
+    assert out.numel() * 2 == nbytes
+    with torch.cuda.device(qweight.device):
+        _lib.check(
+            lib.woq_hip_dense_weight(
+                _ptr(qweight), weight_dtype, N, K, _ptr(scales_bf16), _ptr(zeros_u8), group_size, _ptr(out), _stream()
+            ),
+            "dense_weight",
+        )
+    return out
+
+
 def unpack_int4_zeros(zp32, cols):
     """int32-compressed zero points [rows, ceil(cols/8)] -> fp32 [rows, cols]."""
     lib = _lib.load()
@@ -192,6 +213,7 @@ def linear(
     noalloc=False,
     out_dtype=None,
     scale_zero_bf16=None,
+    dense_bf16=None,
 ):
     """y = x @ dequant(W)^T (+ bias, post-op).  x: [..., K]; returns [..., N] in x.dtype, or the
     fp32 accumulator when ``out_fp32``.  With ``debug_block_sums`` also returns the int32 sum of
@@ -225,6 +247,7 @@ def linear(
     p.zeros_u8 = zeros_u8.data_ptr() if zeros_u8 is not None else None
     p.scale_zero_f16x2 = scale_zero_f16x2.data_ptr() if scale_zero_f16x2 is not None else None
     p.scale_zero_bf16 = scale_zero_bf16.data_ptr() if scale_zero_bf16 is not None else None
+    p.dense_bf16 = dense_bf16.data_ptr() if dense_bf16 is not None else None
     p.group_size = group_size
     p.bias = bias_f32.data_ptr() if bias_f32 is not None else None
     p.lowp_mode = lowp_mode

@@ -24,6 +24,9 @@ EXPORTS = [
     "woq_hip_last_error",
     "woq_hip_abi_version",
     "woq_hip_small_batch_threshold",
+    "woq_hip_weight_cache_batch_threshold",
+    "woq_hip_dense_weight_bytes",
+    "woq_hip_dense_weight",
     "woq_hip_last_kernel",
     "woq_hip_padded_n",
     "woq_hip_padded_k",
@@ -69,6 +72,7 @@ class LinearParams(ctypes.Structure):
         ("zeros_u8", ctypes.c_void_p),
         ("scale_zero_f16x2", ctypes.c_void_p),
         ("scale_zero_bf16", ctypes.c_void_p),
+        ("dense_bf16", ctypes.c_void_p),
         ("group_size", ctypes.c_int64),
         ("bias", ctypes.c_void_p),
         ("lowp_mode", ctypes.c_int32),
@@ -111,6 +115,12 @@ def load():
         lib.woq_hip_abi_version.restype = i32
         lib.woq_hip_small_batch_threshold.restype = i32
         lib.woq_hip_small_batch_threshold.argtypes = []
+        lib.woq_hip_weight_cache_batch_threshold.restype = i32
+        lib.woq_hip_weight_cache_batch_threshold.argtypes = []
+        lib.woq_hip_dense_weight_bytes.restype = i64
+        lib.woq_hip_dense_weight_bytes.argtypes = [ctypes.c_int32, i64, i64]
+        lib.woq_hip_dense_weight.restype = i32
+        lib.woq_hip_dense_weight.argtypes = [vp, ctypes.c_int32, i64, i64, vp, vp, i64, vp, vp]
         lib.woq_hip_last_kernel.restype = ctypes.c_char_p
         lib.woq_hip_last_kernel.argtypes = []
         lib.woq_hip_padded_n.restype = i64
@@ -159,7 +169,7 @@ def load():
         lib.woq_hip_linear_grouped.argtypes = [ctypes.POINTER(LinearParams), vp, i64]
         lib.woq_hip_moe_combine_rows.restype = i32
         lib.woq_hip_moe_combine_rows.argtypes = [vp, i32, i64, i64, vp, vp, i64, vp, vp, i32, vp]
-        if lib.woq_hip_abi_version() != 2:
+        if lib.woq_hip_abi_version() != 3:
             raise RuntimeError("libwoq_hip.so has an unexpected ABI version")
         _lib = lib
     return _lib

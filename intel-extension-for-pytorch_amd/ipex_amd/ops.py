@@ -176,6 +176,13 @@ class WoqLinearOpContext:
         self.zeros_u8_ = z8
         self.scale_zero_f16x2_ = sz
         self.scale_zero_bf16_ = szb
+        # cache_weight_for_large_batch under lowp_mode BF16 (LinearWoqPacked.cpp:430-486): the dense bf16 copy, made
+        # at prepack time so that a forward call mutates nothing; None where the flag is off or K % 128 != 0
+        self.cached_weight_ = None
+        if self.cache_weight_for_large_batch_ and self.lowp_mode_ == _lib.LOWP_BF16:
+            self.cached_weight_ = _kernels.dense_weight(
+                self.at_weight_, weight_dtype, N, K, sb16, z8, group_size
+            )
         self.scales_plain_ = scales if group_size > 0 else scales.reshape(N)
         self.zero_points_plain_ = (
             None if zero_points is None else (zero_points if group_size > 0 else zero_points.reshape(N))
@@ -216,11 +223,9 @@ class WoqLinearOpContext:
         return self.g_idx_
 
     def get_cached_weight(self):
-        """Always None: ``cache_weight_for_large_batch`` is accepted, kept and pickled, but no dequantized
-        copy of the weight is made.  The reference caches one for batches of 64 rows and more because its
-        kernel dequantizes a block again for every 64 rows (LinearWoqPacked.cpp:430-533); the prefill
-        kernels here dequantize in registers once per 128 rows."""
-        return None
+        """The dequantized bf16 copy of the weight that ``cache_weight_for_large_batch`` asks for under lowp_mode
+        BF16 (LinearWoqPacked.cpp:430-486), in the operand layout of the dense kernel; None otherwise."""
+        return self.cached_weight_
 
     def get_cached_compensation(self):
         return self.cached_compensation_
@@ -292,6 +297,7 @@ class WoqLinearOpContext:
             p.zeros_u8 = self.zeros_u8_.data_ptr() if self.zeros_u8_ is not None else None
             p.scale_zero_f16x2 = self.scale_zero_f16x2_.data_ptr() if self.scale_zero_f16x2_ is not None else None
             p.scale_zero_bf16 = self.scale_zero_bf16_.data_ptr() if self.scale_zero_bf16_ is not None else None
+            p.dense_bf16 = self.cached_weight_.data_ptr() if self.cached_weight_ is not None else None
             p.group_size = self.group_size_
             p.bias = self.bias_f32_.data_ptr() if self.bias_f32_ is not None else None
             p.lowp_mode = self.lowp_mode_
@@ -400,6 +406,7 @@ class WoqLinearOpContext:
             self.act_quant_mode_,
             scale_zero_f16x2=self.scale_zero_f16x2_,
             scale_zero_bf16=self.scale_zero_bf16_,
+            dense_bf16=self.cached_weight_,
             fusion=fusion,
             others=others,
             **kw,

@@ -432,24 +432,37 @@ def test_k_mismatch_and_bad_arguments(cuda):
                                torch.ones(32, device=cuda), torch.zeros(32, device=cuda), None, None, None, -1, 3, 6)
 
 
-def test_weight_cache_flag_is_accepted_and_changes_nothing(cuda):
-    """cache_weight_for_large_batch (tests/cpu/test_quantization_default_recipe.py:1522-1579): the flag is
-    taken, kept and pickled; large batches run on the same prefill kernel with or without it (no dense
-    copy of the weight is made), so the results are bit-identical."""
+def test_weight_cache_flag_keeps_a_dense_copy_and_changes_no_result(cuda):
+    """cache_weight_for_large_batch (tests/cpu/test_quantization_default_recipe.py:1522-1579): under lowp_mode BF16
+    the context keeps a dequantized bf16 copy of the weight (get_cached_weight), made again when a pickled context
+    is loaded; results with and without it are bit-identical, through both bindings, below and above the batch size
+    from which the copy is used."""
+    from ipex_amd import _lib
     from ipex_amd.utils import synthetic
     from helpers import make_context, make_torch_context
 
-    case = synthetic.make_int4_case(34, 80, 512, 144, 128, bias=True)
+    case = synthetic.make_int4_case(34, 640, 512, 8192, 128, bias=True)
     x = case["x"].to(cuda)
-    y_plain = make_context(case, 2).run(x)
+    plain = make_context(case, 2)
+    y_plain = plain.run(x)
+    assert plain.get_cached_weight() is None and _lib.last_kernel() == "woq_gemm_w4_kernel"
     cached = make_context(case, 2, cache=True)
-    assert torch.equal(cached.run(x), y_plain) and cached.get_cached_weight() is None
-    assert pickle.loads(pickle.dumps(cached)).cache_weight_for_large_batch_ is True
+    assert tuple(cached.get_cached_weight().shape) == (4, 512, 4, 64, 8)
+    assert torch.equal(cached.run(x), y_plain) and _lib.last_kernel() == "woq_gemm_dense_kernel"
+    assert torch.equal(cached.run(x[:80]), plain.run(x[:80]))
+    again = pickle.loads(pickle.dumps(cached))
+    assert again.cache_weight_for_large_batch_ is True
+    assert torch.equal(again.get_cached_weight(), cached.get_cached_weight())
     tc = make_torch_context(case, 2, cache=True)
+    assert torch.equal(tc.get_cached_weight(), cached.get_cached_weight())
     assert torch.equal(torch.ops.torch_ipex.ipex_woq_linear(x, tc.get_data_handle()), y_plain)
-    assert tc.get_cached_weight() is None
+    assert _lib.last_kernel() == "woq_gemm_dense_kernel"
+    assert torch.equal(torch.ops.torch_ipex.ipex_woq_linear(x[:80], tc.get_data_handle()), plain.run(x[:80]))
     tc2 = pickle.loads(pickle.dumps(tc))
+    assert torch.equal(tc2.get_cached_weight(), cached.get_cached_weight())
     assert torch.equal(torch.ops.torch_ipex.ipex_woq_linear(x, tc2.get_data_handle()), y_plain)
+    assert make_torch_context(case, 2).get_cached_weight() is None
+    assert make_torch_context(case, 3, act_quant_mode=6, cache=True).get_cached_weight() is None
 
 
 def test_fused_ops_through_torch_ops(cuda):

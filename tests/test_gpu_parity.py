@@ -38,6 +38,12 @@ def _synthetic():
     return synthetic
 
 
+def _lib_mod():
+    from ipex_amd import _lib
+
+    return _lib
+
+
 # ---------------------------------------------------------------------------------------------
 # prepack: integer-exact, invertible
 # ---------------------------------------------------------------------------------------------
@@ -236,6 +242,159 @@ def test_merged_scale_zero_table_changes_no_bit(cuda, kind, M, K, N, G, sym, bia
     assert _lib_last_kernel() == kernel
     ctx.scale_zero_bf16_ = table
     assert torch.equal(with_table, without), (kernel, (with_table - without).abs().max().item())
+
+
+# ---------------------------------------------------------------------------------------------
+# cache_weight_for_large_batch: the dense bf16 copy and the kernel that runs on it
+# ---------------------------------------------------------------------------------------------
+def _dense_case(kind, M, K, N, G, sym=False, bias=False, seed=21):
+    syn = _synthetic()
+    if kind == "int4":
+        case = syn.make_int4_case(seed, M, K, N, G, bias=bias)
+        if sym:
+            case["zeros"] = None
+    elif kind == "int8":
+        case = syn.make_int8_case(seed, M, K, N, group_size=G, bias=bias)
+        if not sym:
+            case["zeros"] = torch.randint(-128, 128, case["scales"].shape, generator=torch.Generator().manual_seed(5)).float()
+    elif kind == "nf4":
+        case = syn.make_nf4_case(seed, M, K, N, G, bias=bias)
+    else:
+        case = syn.make_fp8_case(seed, M, K, N, bias=bias, group_size=G)
+    return case
+
+
+def _dense_copy_as_matrix(dense, N, K, wbits):
+    """[K / 128, NT, 4, 64, 8] fragments -> [padded N, K]: fragment (kt, nt, j, lane) holds row 16 nt + lane % 16 and
+    the K values 128 kt + 8 chunk .. + 7 with chunk = 4 (lane / 16) + j for 4-bit codes and
+    8 (j / 2) + 2 (lane / 16) + j % 2 for bytes."""
+    d = dense.view(torch.int16).cpu().numpy().view(np.uint16)
+    KT, NT = d.shape[0], d.shape[1]
+    out = np.zeros((NT * 16, K), dtype=np.uint16)
+    for j in range(4):
+        for c in range(4):
+            chunk = 4 * c + j if wbits == 4 else 8 * (j // 2) + 2 * c + (j % 2)
+            for kt in range(KT):
+                k0 = 128 * kt + 8 * chunk
+                # lanes 16 c .. 16 c + 15 are rows 0..15 of every row-block
+                out[:, k0:k0 + 8] = d[kt, :, j, 16 * c:16 * c + 16, :].reshape(NT * 16, 8)
+    return out
+
+
+@pytest.mark.parametrize(
+    "kind,K,N,G,sym",
+    [("int4", 512, 80, 128, False), ("int4", 256, 33, 32, True), ("int4", 384, 48, -1, False), ("int8", 256, 40, -1, True),
+     ("int8", 512, 32, 128, False), ("nf4", 256, 48, 64, True), ("fp8", 384, 24, 128, True)],
+)
+def test_dense_copy_is_the_bf16_dequantized_weight(cuda, kind, K, N, G, sym):
+    """The copy that cache_weight_for_large_batch keeps (LinearWoqPacked.cpp:430-486) against the oracle's
+    dequantization with the bf16 scales, bit for bit, through the documented fragment layout."""
+    case = _dense_case(kind, 4, K, N, G, sym=sym)
+    ctx = make_context(case, O.LOWP_BF16, cache=True)
+    dense = ctx.get_cached_weight()
+    NT = (N + 15) // 16
+    assert dense is not None and tuple(dense.shape) == (K // 128, NT, 4, 64, 8) and dense.dtype == torch.bfloat16
+    c = case_np(case)
+    w = O.dequantize_woq_weight(c["qw"], N, K, O._round_to(c["scales"], "bf16"), c["zps"], case["weight_dtype"], G)
+    want = O.f32_to_bf16_bits(w)
+    got = _dense_copy_as_matrix(dense, N, K, 8 if kind in ("int8", "fp8") else 4)
+    assert np.array_equal(got[:N], want), kind
+
+
+@pytest.mark.parametrize(
+    "kind,M,K,N,G,sym,bias",
+    [("int4", 130, 512, 448, 128, False, True), ("int4", 128, 1024, 500, 32, True, False),
+     ("int4", 257, 384, 300, -1, False, True), ("int4", 64, 256, 1024, 64, False, False),
+     ("int8", 96, 512, 272, 128, True, True), ("int8", 200, 256, 128, -1, False, False)],
+)
+@pytest.mark.parametrize("shape_kernels", [(24, 4), (25, 5), (26, 6)])
+def test_dense_kernel_equals_the_dequantizing_prefill_kernel_bit_for_bit(cuda, kind, M, K, N, G, sym, bias, shape_kernels):
+    """woq_gemm_dense_kernel on the copy feeds the MFMAs the operands that woq_gemm_w4_kernel dequantizes on the fly,
+    in the same order: fp32 accumulators and rounded outputs are equal for every workgroup shape (ragged M, N and the
+    row-blocks past N included), with and without bias."""
+    dense_k, w4_k = shape_kernels
+    if kind == "int8" and w4_k == 4:
+        pytest.skip("8-bit weights have no 448-column shape in the dequantizing kernel")
+    case = _dense_case(kind, M, K, N, G, sym=sym, bias=bias)
+    ctx = make_context(case, O.LOWP_BF16, cache=True)
+    x = case["x"].cuda()
+    for fp32 in (True, False):
+        y_dense = ctx.run(x, out_fp32=fp32, force_kernel=dense_k)
+        assert _lib_last_kernel() == "woq_gemm_dense_kernel"
+        y_w4 = ctx.run(x, out_fp32=fp32, force_kernel=w4_k)
+        assert _lib_last_kernel() == "woq_gemm_w4_kernel"
+        assert torch.equal(y_dense, y_w4), (kind, fp32, (y_dense.float() - y_w4.float()).abs().max().item())
+
+
+@pytest.mark.parametrize("kind,G", [("nf4", 64), ("fp8", 128), ("int4", 128)])
+def test_dense_kernel_against_the_oracle(cuda, kind, G):
+    """Every weight format through the dense kernel (force_kernel 23) against the optimized bf16 oracle, to the bars
+    of the other bf16 kernels; NF4 and FP8 have no dequantizing prefill kernel of the same accumulation order to be
+    compared with bit for bit."""
+    case = _dense_case(kind, 150, 512, 176, G, sym=True, bias=True)
+    ctx = make_context(case, O.LOWP_BF16, cache=True)
+    _check_fp(case, O.LOWP_BF16, ctx=ctx, force_kernel=23, label=f"dense {kind}")
+    assert _lib_last_kernel() == "woq_gemm_dense_kernel"
+
+
+def test_dense_kernel_post_ops_equal_the_dequantizing_kernel(cuda):
+    lib = _lib_mod()
+    case = _dense_case("int4", 160, 256, 144, 128, bias=True)
+    ctx = make_context(case, O.LOWP_BF16, cache=True)
+    x = case["x"].cuda()
+    g = torch.Generator().manual_seed(3)
+    o0 = torch.randn(160, 144, generator=g).to(torch.bfloat16).cuda()
+    o1 = torch.randn(160, 144, generator=g).to(torch.bfloat16).cuda()
+    for fusion, others in [(lib.FUSE_GELU_ERF, ()), (lib.FUSE_SILU, ()), (lib.FUSE_ADD, (o0,)), (lib.FUSE_MUL, (o0,)),
+                           (lib.FUSE_ADD_ADD, (o0, o1))]:
+        a = ctx.run(x, fusion=fusion, others=others, force_kernel=23)
+        assert _lib_last_kernel() == "woq_gemm_dense_kernel"
+        b = ctx.run(x, fusion=fusion, others=others, force_kernel=3)
+        assert torch.equal(a, b), fusion
+
+
+def test_weight_cache_serves_large_batches_only(cuda):
+    """With the copy, lowp_mode BF16 runs batches of at least IPEX_WOQ_WEIGHT_CACHE_BATCH_THRESHOLD rows (64) on the
+    dense kernel where the library's cost models make it the faster one (its 128-row tiles must fill the chip: here
+    1536 rows on a wide layer); smaller ones and contexts without the flag stay on the kernels that read the packed
+    weight.  Same bits either way."""
+    lib = _lib_mod().load()
+    assert lib.woq_hip_weight_cache_batch_threshold() == 64
+    case = _dense_case("int4", 1536, 512, 7168, 128)
+    cached, plain = make_context(case, O.LOWP_BF16, cache=True), make_context(case, O.LOWP_BF16)
+    assert plain.get_cached_weight() is None
+    x = case["x"].cuda()
+    y = cached.run(x)
+    assert _lib_last_kernel() == "woq_gemm_dense_kernel"
+    y_plain = plain.run(x)
+    assert _lib_last_kernel() == "woq_gemm_w4_kernel"
+    assert torch.equal(y, y_plain)
+    for rows in (1, 16, 63, 200):
+        y = cached.run(x[:rows])
+        assert _lib_last_kernel() != "woq_gemm_dense_kernel", rows
+        assert torch.equal(y, plain.run(x[:rows])), rows
+    # lowp_mode INT8 and K that is no multiple of 128 keep no copy (LinearWoqPacked.cpp:443-447 has its own conditions)
+    assert make_context(case, O.LOWP_INT8, act_quant_mode=6, cache=True).get_cached_weight() is None
+    odd = _dense_case("int4", 8, 192, 64, 64)
+    assert make_context(odd, O.LOWP_BF16, cache=True).get_cached_weight() is None
+    # a forced dense kernel without a copy is an error, not a fallback
+    with pytest.raises(RuntimeError, match="dense"):
+        plain.run(x, force_kernel=23)
+
+
+def test_c3_prefill_bf16_with_weight_cache(cuda):
+    """The named prefill configuration with cache_weight_for_large_batch: served by the dense kernel, equal bit for
+    bit to the run without the flag, and within the bars of the oracle like that one."""
+    case = _synthetic().make_int4_case(3, 2048, 4096, 14336, 128, outliers=True)
+    ctx = make_context(case, O.LOWP_BF16, cache=True)
+    x = case["x"].cuda()
+    y = ctx.run(x)
+    assert _lib_last_kernel() == "woq_gemm_dense_kernel"
+    y_plain = make_context(case, O.LOWP_BF16).run(x)
+    assert _lib_last_kernel() == "woq_gemm_w4_kernel"
+    assert torch.equal(y, y_plain)
+    _check_fp(case, O.LOWP_BF16, ctx=ctx, cols=np.arange(0, 14336, 29), label="C3 bf16 dense")
+    assert _lib_last_kernel() == "woq_gemm_dense_kernel"
 
 
 def test_c0_int4_g128_m1(cuda):

@@ -23,13 +23,19 @@ def test_library_exports_every_declared_symbol():
     lib = _lib.load()
     for name in declared:
         assert hasattr(lib, name), name
-    assert lib.woq_hip_abi_version() == 2
+    assert lib.woq_hip_abi_version() == 3
     # pure host-side helpers can be called without a GPU
     assert lib.woq_hip_padded_n(500) == 512
     assert lib.woq_hip_padded_k(2, 4096) == 4096 and lib.woq_hip_padded_k(2, 4097) == 4224
     assert lib.woq_hip_padded_k(1, 100) == 128
     assert lib.woq_hip_packed_weight_bytes(2, 14336, 4096) == 14336 * 4096 // 2
     assert [lib.woq_hip_int8_block_k(g, 4096) for g in (-1, 32, 64, 128, 256)] == [128, 32, 64, 128, 128]
+    # the dense bf16 copy of cache_weight_for_large_batch: two bytes per weight over the padded rows, none where K is
+    # no multiple of 128 or the copy would reach 2 GiB
+    assert lib.woq_hip_dense_weight_bytes(2, 14336, 4096) == 14336 * 4096 * 2
+    assert lib.woq_hip_dense_weight_bytes(1, 500, 256) == 512 * 256 * 2
+    assert lib.woq_hip_dense_weight_bytes(2, 64, 192) == 0 and lib.woq_hip_dense_weight_bytes(2, 65536, 16384) == 0
+    assert lib.woq_hip_weight_cache_batch_threshold() == 64
 
 
 def test_params_struct_size_is_checked():
