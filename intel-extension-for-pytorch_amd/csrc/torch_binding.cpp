@@ -714,6 +714,94 @@ static Tensor woq_linear_binary(const Tensor& input, const Tensor& W_prepack, co
   return context_from_handle(W_prepack, "torch_ipex::woq_linear_<post-op>")->run(input, FUSION, o);
 }
 
+// ---- mixture of experts over WOQ linears (csrc/cpu/aten/MoE.cpp:260-328) -------------------------------
+// One expert: gather its tokens, down(up(x) * silu(gate(x))), weighted accumulation into `output`
+// (mixtral_moe_woq_kernl_impl, csrc/cpu/aten/kernels/MoEKrnl.cpp:254-284).
+static Tensor moe_expert(const Tensor& hidden, const Tensor& top_x_in, const Tensor& idx_in, WoqLinearOpContext& gate,
+                         WoqLinearOpContext& up, WoqLinearOpContext& down, const Tensor& routing_weights, Tensor output,
+                         const char* op) {
+  const auto dev = hidden.device();
+  TORCH_CHECK(hidden.dim() == 2 && output.dim() == 2 && output.sizes() == hidden.sizes() && output.is_contiguous() &&
+                  output.device() == dev && output.scalar_type() == hidden.scalar_type(),
+              op, ": hidden_states and output must be [tokens, hidden] tensors of one dtype on one device, output contiguous");
+  TORCH_CHECK(routing_weights.dim() == 2 && routing_weights.size(0) == hidden.size(0) && routing_weights.device() == dev &&
+                  routing_weights.scalar_type() == hidden.scalar_type(),
+              op, ": routing_weights must be [tokens, top-k] in the dtype and on the device of hidden_states");
+  const Tensor x = hidden.contiguous(), rw = routing_weights.contiguous();
+  const Tensor top_x = top_x_in.to(dev, at::kLong).contiguous(), idx = idx_in.to(dev, at::kLong).contiguous();
+  const int64_t n = top_x.numel(), T = x.size(0), H = x.size(1);
+  TORCH_CHECK(idx.numel() == n, op, ": top_x and idx differ in length");
+  Tensor cur = at::empty({n, H}, x.options());
+  DeviceScope scope(x);
+  check_rc(woq_hip_moe_gather_rows(x.data_ptr(), act_code(x.scalar_type()), T, H, top_x.data_ptr<int64_t>(), n,
+                                   cur.data_ptr(), current_stream(x)), op);
+  const Tensor act = gate.run(cur, WOQ_HIP_FUSE_SILU, {});
+  const Tensor out = down.run(up.run(cur, WOQ_HIP_FUSE_MUL, {act}), WOQ_HIP_FUSE_NONE, {}).contiguous();
+  TORCH_CHECK(out.dim() == 2 && out.size(0) == n && out.size(1) == H, op, ": the down projection must return to the hidden width");
+  check_rc(woq_hip_moe_scale_add_rows(output.data_ptr(), act_code(output.scalar_type()), T, H, out.data_ptr(), rw.data_ptr(),
+                                      rw.size(1), top_x.data_ptr<int64_t>(), idx.data_ptr<int64_t>(), n, current_stream(x)),
+           op);
+  return output;
+}
+
+static Tensor mixtral_moe_woq(const Tensor& hidden_states, const Tensor& top_x, const Tensor& idx, const Tensor& gate_wei,
+                              const Tensor& up_wei, const Tensor& down_wei, const Tensor& routing_weights, Tensor output,
+                              bool is_distributed) {
+  const char* op = "torch_ipex::mixtral_moe_woq";
+  require_gpu_input(hidden_states, op);
+  TORCH_CHECK(!is_distributed, op, ": is_distributed=True needs an all-reduce, which this one-GPU build does not have");
+  if (top_x.size(0) == 0) return output;
+  auto gate = context_from_handle(gate_wei, op), up = context_from_handle(up_wei, op), down = context_from_handle(down_wei, op);
+  return moe_expert(hidden_states, top_x, idx, *gate, *up, *down, routing_weights, output, op);
+}
+
+// All experts of a layer: the routing table is read on the host, as the reference does (its tensors live there), and
+// the experts are visited in ascending order, inside an expert the tokens in ascending order (get_expert_topx_idx,
+// MoE.cpp:64-81), which fixes the order of the additions into a token's row.  The Python package puts a form without
+// the host read in front of this one (grouped launches, ipex_amd/ops.py).
+static Tensor deepseek_moe_woq(const Tensor& hidden_states, const Tensor& topk_ids,
+                               std::vector<c10::intrusive_ptr<WoqLinearOpContext>> gate_ctx,
+                               std::vector<c10::intrusive_ptr<WoqLinearOpContext>> up_ctx,
+                               std::vector<c10::intrusive_ptr<WoqLinearOpContext>> down_ctx, const Tensor& routing_weights,
+                               bool is_distributed) {
+  const char* op = "torch_ipex::deepseek_moe_woq";
+  require_gpu_input(hidden_states, op);
+  TORCH_CHECK(!is_distributed, op, ": is_distributed=True needs an all-reduce, which this one-GPU build does not have");
+  const int64_t experts = (int64_t)gate_ctx.size();
+  TORCH_CHECK((int64_t)up_ctx.size() == experts && (int64_t)down_ctx.size() == experts, op,
+              ": gate / up / down lists differ in length");
+  Tensor output = at::zeros_like(hidden_states, at::MemoryFormat::Contiguous);
+  const Tensor ids = topk_ids.detach().to(at::kCPU, at::kLong).contiguous();
+  if (ids.numel() == 0) return output;
+  TORCH_CHECK(ids.dim() == 2 && ids.size(0) == hidden_states.size(0), op, ": topk_ids must be [tokens, top-k]");
+  const int64_t T = ids.size(0), topk = ids.size(1);
+  const int64_t* id = ids.data_ptr<int64_t>();
+  // per expert the (token, slot) entries in ascending token order; a token that names an expert more than once has
+  // its k-th mention in round k (the scatter adds one row per token and call)
+  std::vector<std::vector<std::vector<int64_t>>> tok(experts), slot(experts);
+  for (int64_t t = 0; t < T; ++t) {
+    std::vector<int64_t> mentions(0);
+    for (int64_t k = 0; k < topk; ++k) {
+      const int64_t e = id[t * topk + k];
+      TORCH_CHECK(e >= 0 && e < experts, op, ": expert ids must lie in [0, ", experts, ")");
+      int64_t round = 0;
+      for (int64_t j = 0; j < k; ++j) round += id[t * topk + j] == e;
+      if ((int64_t)tok[e].size() <= round) { tok[e].resize(round + 1); slot[e].resize(round + 1); }
+      tok[e][round].push_back(t);
+      slot[e][round].push_back(k);
+    }
+  }
+  const auto opt = at::TensorOptions().dtype(at::kLong);
+  for (int64_t e = 0; e < experts; ++e) {
+    for (size_t round = 0; round < tok[e].size(); ++round) {
+      if (tok[e][round].empty()) continue;
+      const Tensor top_x = at::tensor(tok[e][round], opt), idx = at::tensor(slot[e][round], opt);
+      moe_expert(hidden_states, top_x, idx, *gate_ctx[e], *up_ctx[e], *down_ctx[e], routing_weights, output, op);
+    }
+  }
+  return output;
+}
+
 // Context-free forward (woq_linear_forward_v2, csrc/cpu/aten/Linear.cpp:556-617); the tensor arguments
 // are the outputs of woq_linear_pack_weight.
 static Tensor woq_linear_v2(const Tensor& input_in, const Tensor& qweight, c10::string_view weight_dtype,
@@ -936,6 +1024,16 @@ TORCH_LIBRARY_FRAGMENT(torch_ipex, m) {
       "woq_linear(Tensor _0, Tensor _1, str _2, int[] _3, Tensor[] _4, Tensor[]? _5, Tensor[]? _6, Tensor? _7, int _8, "
       "int _9, int _10, Tensor? _11 = None) -> Tensor");
   m.def("dequantize_nf4(Tensor t, Tensor scales, int group_size, ScalarType out_dtype) -> Tensor");
+  // (csrc/cpu/aten/MoE.cpp:455-472; output is accumulated into and returned)
+  m.def(
+      "mixtral_moe_woq(Tensor hidden_states, Tensor top_x, Tensor idx, Tensor gate_wei, Tensor up_wei, "
+      "Tensor down_wei, Tensor routing_weights, Tensor(a!) output, bool is_distributed) -> Tensor(a!)");
+  m.def(
+      "deepseek_moe_woq(Tensor hidden_states, Tensor topk_ids, "
+      "__torch__.torch.classes.ipex_prepack.WoqLinearOpContext[] gate_ctx, "
+      "__torch__.torch.classes.ipex_prepack.WoqLinearOpContext[] up_ctx, "
+      "__torch__.torch.classes.ipex_prepack.WoqLinearOpContext[] down_ctx, "
+      "Tensor routing_weights, bool is_distributed) -> Tensor");
 }
 
 TORCH_LIBRARY_IMPL(torch_ipex, CUDA, m) {
@@ -949,6 +1047,14 @@ TORCH_LIBRARY_IMPL(torch_ipex, CUDA, m) {
   m.impl("woq_linear_mul", TORCH_FN((woq_linear_binary<WOQ_HIP_FUSE_MUL, 1>)));
   m.impl("woq_linear", TORCH_FN(woq_linear_v2));
   m.impl("dequantize_nf4", TORCH_FN(dequantize_nf4));
+  m.impl("deepseek_moe_woq", TORCH_FN(deepseek_moe_woq));
+}
+
+// The handles of mixtral_moe_woq are CPU tensors beside GPU activations, so no backend key can be computed from the
+// arguments alone: registered for every backend, it checks the device of hidden_states itself.  (The Python package
+// registers a CUDA kernel in front of it that also resolves the handles of its ctypes contexts.)
+TORCH_LIBRARY_IMPL(torch_ipex, CompositeExplicitAutograd, m) {
+  m.impl("mixtral_moe_woq", TORCH_FN(mixtral_moe_woq));
 }
 
 // Tensors on the CPU reach these kernels, whose only work is the error: this build has no CPU path.

@@ -941,13 +941,12 @@ def register():
     if _registered:
         return
     _lib.load_torch_binding()
-    tl = torch.library.Library("torch_ipex", "FRAGMENT")
+    # The binding defines mixtral_moe_woq / deepseek_moe_woq over the registered custom class (per-expert launches,
+    # routing read on the host).  In front of them: a kernel for mixtral_moe_woq that also resolves the handles of this
+    # module's ctypes contexts, and deepseek_moe_woq as a function that takes contexts of either binding and runs small
+    # batches in grouped launches without reading the routing on the host.
+    tl = torch.library.Library("torch_ipex", "IMPL")
     _libs.append(tl)
-    tl.define(
-        "mixtral_moe_woq(Tensor hidden_states, Tensor top_x, Tensor idx, Tensor gate_wei, Tensor up_wei, "
-        "Tensor down_wei, Tensor routing_weights, Tensor(a!) output, bool is_distributed) -> Tensor(a!)"
-    )
-    tl.impl("mixtral_moe_woq", mixtral_moe_woq, "CompositeExplicitAutograd")
-    # takes lists of context objects, which no operator schema can name
+    tl.impl("mixtral_moe_woq", mixtral_moe_woq, "CUDA")
     setattr(torch.ops.torch_ipex, "deepseek_moe_woq", deepseek_moe_woq)
     _registered = True

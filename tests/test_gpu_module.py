@@ -649,6 +649,71 @@ def test_deepseek_moe_woq_matches_per_expert_composition(cuda, T, topk):
     assert float(err) < 3e-2, float(err)
 
 
+_BINDING_ALONE = r"""
+import sys
+import torch
+
+torch.ops.load_library(sys.argv[1])  # the operator / custom-class binding; the Python package is never imported
+d = torch.load(sys.argv[2])
+E, G = d["E"], d["G"]
+mk = lambda w, s, z, n, k: torch.ops.ipex_prepack.weight_only_qlinear_prepack(
+    w.cuda(), 2, [n, k], s.cuda(), z.cuda(), None, None, None, G, 2, -1, False)
+H, I = d["H"], d["I"]
+gate = [mk(*d["gate"][e], I, H) for e in range(E)]
+up = [mk(*d["up"][e], I, H) for e in range(E)]
+down = [mk(*d["down"][e], H, I) for e in range(E)]
+hidden, ids, rw = d["hidden"].cuda(), d["ids"].cuda(), d["rw"].cuda()
+layer = torch.ops.torch_ipex.deepseek_moe_woq(hidden, ids, gate, up, down, rw, False)
+one_by_one = torch.zeros_like(hidden)
+for e in range(E):
+    tok, slot = (d["ids"] == e).nonzero(as_tuple=True)
+    r = torch.ops.torch_ipex.mixtral_moe_woq(hidden, tok, slot, gate[e].get_data_handle(), up[e].get_data_handle(),
+                                             down[e].get_data_handle(), rw, one_by_one, False)
+    assert r.data_ptr() == one_by_one.data_ptr()
+torch.save({"layer": layer.cpu(), "one_by_one": one_by_one.cpu()}, sys.argv[3])
+"""
+
+
+def test_moe_operators_of_the_binding_without_the_python_package(cuda, tmp_path, monkeypatch):
+    """torch_ipex::mixtral_moe_woq and deepseek_moe_woq as the C++ binding registers them (csrc/cpu/aten/MoE.cpp:260-328,
+    455-472), in a process that loads only libwoq_torch.so -- what a TorchScript consumer has: equal, bit for bit, to
+    the Python package's per-expert path on the same experts and routing."""
+    import subprocess
+    import sys
+
+    from ipex_amd import _lib
+    from ipex_amd.utils import synthetic
+
+    E, H, I, G, T, topk = 4, 256, 384, 64, 9, 2
+    layer = {"E": E, "H": H, "I": I, "G": G}
+    for i, (name, n, k) in enumerate((("gate", I, H), ("up", I, H), ("down", H, I))):
+        layer[name] = []
+        for e in range(E):
+            c = synthetic.make_int4_case(500 + 3 * e + i, 1, k, n, G)
+            layer[name].append((c["qweight"], c["scales"], c["zeros"]))
+    g = torch.Generator().manual_seed(77)
+    layer["hidden"] = torch.randn(T, H, generator=g).to(torch.bfloat16)
+    layer["ids"] = torch.stack([torch.randperm(E, generator=g)[:topk] for _ in range(T)])
+    layer["rw"] = torch.softmax(torch.randn(T, topk, generator=g), -1).to(torch.bfloat16)
+    torch.save(layer, tmp_path / "layer.pt")
+    (tmp_path / "alone.py").write_text(_BINDING_ALONE)
+    run = subprocess.run([sys.executable, str(tmp_path / "alone.py"), _lib.TORCH_LIB_PATH, str(tmp_path / "layer.pt"),
+                          str(tmp_path / "out.pt")], capture_output=True, text=True, timeout=300)
+    assert run.returncode == 0, run.stderr[-3000:]
+    alone = torch.load(tmp_path / "out.pt")
+    assert torch.equal(alone["layer"], alone["one_by_one"])
+
+    ctx = lambda w, s, z, n, k: torch.ops.ipex_prepack.weight_only_qlinear_prepack(
+        w.to(cuda), 2, [n, k], s.to(cuda), z.to(cuda), None, None, None, G, 2, -1, False)
+    gate = [ctx(*layer["gate"][e], I, H) for e in range(E)]
+    up = [ctx(*layer["up"][e], I, H) for e in range(E)]
+    down = [ctx(*layer["down"][e], H, I) for e in range(E)]
+    monkeypatch.setenv("IPEX_AMD_MOE_GROUPED", "0")
+    want = torch.ops.torch_ipex.deepseek_moe_woq(layer["hidden"].to(cuda), layer["ids"].to(cuda), gate, up, down,
+                                                 layer["rw"].to(cuda), False)
+    assert torch.equal(alone["layer"], want.cpu())
+
+
 def test_moe_route_against_the_oracle_token_lists(cuda):
     """woq_hip_moe_route: sorted positions, slots per compute type and per-token contribution order against the
     oracle's per-expert token lists (get_expert_topx_idx, MoE.cpp:64-81); ids outside the expert range drop out."""

@@ -382,6 +382,27 @@ def test_weight_cache_serves_large_batches_only(cuda):
         plain.run(x, force_kernel=23)
 
 
+def test_weight_cache_with_act_order(cuda):
+    """GPTQ act-order with cache_weight_for_large_batch: the dense copy is made from the weight whose input channels
+    are already sorted by group, and the activations are shuffled per call as without the copy -- same bits as the
+    context without the flag, through the dense kernel."""
+    from ipex_amd import ops
+
+    M, K, N, G = 200, 512, 160, 128
+    case = _synthetic().make_int4_case(33, M, K, N, G, bias=True)
+    perm = torch.randperm(K, generator=torch.Generator().manual_seed(9))
+    g_idx = (torch.arange(K) // G)[perm]
+    make = lambda cache: ops.WoqLinearOpContext(
+        case["qweight"].cuda(), 2, [N, K], case["scales"].cuda(), case["zeros"].cuda(), case["bias"].cuda(),
+        g_idx, None, G, O.LOWP_BF16, -1, cache)
+    cached, plain = make(True), make(False)
+    assert cached.get_cached_weight() is not None and plain.get_cached_weight() is None
+    x = case["x"].cuda()
+    y = cached.run(x, force_kernel=23)
+    assert _lib_last_kernel() == "woq_gemm_dense_kernel"
+    assert torch.equal(y, plain.run(x, force_kernel=3))
+
+
 def test_c3_prefill_bf16_with_weight_cache(cuda):
     """The named prefill configuration with cache_weight_for_large_batch: served by the dense kernel, equal bit for
     bit to the run without the flag, and within the bars of the oracle like that one."""

@@ -341,3 +341,27 @@ def test_auto_split_k_predicate_is_the_library_s():
     assert f(128, 4096, 4096, INT8) == full(128, 4096)
     assert f(2048, 4096, 14336, BF16) == 0
     assert f(128, 2048, 4096, BF16) == 0
+
+
+def test_environment_knobs_of_the_reference_are_read_by_the_library():
+    """IPEX_WOQ_SMALL_BATCH_THRESHOLD (csrc/cpu/aten/utils/woq.h:24) and IPEX_WOQ_WEIGHT_CACHE_BATCH_THRESHOLD
+    (csrc/cpu/jit/cpu/kernels/LinearWoqPacked.cpp:17-18) are read once per process by the library; values that are
+    not whole numbers leave the defaults (5 and 64).  Each setting in a process of its own."""
+    import subprocess
+    import sys
+
+    code = (
+        "import sys; sys.path.insert(0, %r); from ipex_amd import _lib; lib = _lib.load(); "
+        "print(lib.woq_hip_small_batch_threshold(), lib.woq_hip_weight_cache_batch_threshold())"
+    ) % os.path.join(ROOT, "intel-extension-for-pytorch_amd")
+
+    def run(**env):
+        e = {k: v for k, v in os.environ.items() if not k.startswith("IPEX_WOQ_")}
+        e.update(env)
+        out = subprocess.run([sys.executable, "-c", code], env=e, capture_output=True, text=True, timeout=120)
+        assert out.returncode == 0, out.stderr[-2000:]
+        return out.stdout.split()[-2:]
+
+    assert run() == ["5", "64"]
+    assert run(IPEX_WOQ_SMALL_BATCH_THRESHOLD="9", IPEX_WOQ_WEIGHT_CACHE_BATCH_THRESHOLD="256") == ["9", "256"]
+    assert run(IPEX_WOQ_SMALL_BATCH_THRESHOLD="many", IPEX_WOQ_WEIGHT_CACHE_BATCH_THRESHOLD="-3") == ["5", "64"]
