@@ -230,9 +230,15 @@ def config_sweep(torch, lib, lib_mod, ops_mod, synthetic, dev, stream, steps):
     and outputs."""
     rows = []
 
-    def run(name, case, lowp=2, aq=-1):
+    def run(name, case, lowp=2, aq=-1, weight_cache=False):
         M, K, N, G = case["M"], case["K"], case["N"], case["group_size"]
         params, keep = _rotating_params(torch, lib_mod, ops_mod, case, lowp, dev, stream, act_quant_mode=aq)
+        if weight_cache:
+            # cache_weight_for_large_batch: a dense bf16 copy beside every packed copy (woq_hip_dense_weight)
+            from ipex_amd import _kernels as kernels_mod
+            for p, c in zip(params, keep[2:]):
+                keep.append(kernels_mod.dense_weight(c.at_weight_, c.weight_dtype_, N, K, c.scales_list_[2], c.zeros_u8_, G))
+                p.dense_bf16 = keep[-1].data_ptr()
         # Each configuration starts after an idle period (its inputs are generated on the host) and
         # the first few thousand launches after one run up to 10 % slower; single groups of a few
         # hundred launches also scatter by +-5 %.  So: a warm-up as long as one group, then nine
@@ -257,6 +263,8 @@ def config_sweep(torch, lib, lib_mod, ops_mod, synthetic, dev, stream, steps):
         else:
             row["GB_per_s"] = round(nbytes / us / 1e3, 1)
             row["frac_of_hbm_peak"] = round(nbytes / us / 1e3 / HBM_PEAK_GBS, 3)
+        if weight_cache:
+            row["kernel"] = lib_mod.last_kernel()
         rows.append(row)
         del params, keep
         torch.cuda.empty_cache()
@@ -285,6 +293,14 @@ def config_sweep(torch, lib, lib_mod, ops_mod, synthetic, dev, stream, steps):
     run("extra: int4 g32 M=2048 qkv 4096->6144 (lowp BF16, 256 x 192 tiles)", synthetic.make_int4_case(5, 2048, 4096, 6144, 32))
     run("extra: fp8 e4m3fn g128 M=1 4096->14336 (lowp BF16)", synthetic.make_fp8_case(5, 1, 4096, 14336, bias=False, group_size=128))
     run("extra: fp8 e4m3fn g128 M=2048 4096->14336 (lowp BF16)", synthetic.make_fp8_case(5, 2048, 4096, 14336, bias=False, group_size=128))
+    # the same large batches with cache_weight_for_large_batch (dense bf16 copy, rotating like the packed copies)
+    run("extra: int8 per-channel M=2048 4096->11008 +bias (lowp BF16, cache_weight_for_large_batch)",
+        synthetic.make_int8_case(5, 2048, 4096, 11008), weight_cache=True)
+    run("extra: fp8 e4m3fn g128 M=2048 4096->14336 (lowp BF16, cache_weight_for_large_batch)",
+        synthetic.make_fp8_case(5, 2048, 4096, 14336, bias=False, group_size=128), weight_cache=True)
+    run("extra: int4 g128 M=1024 4096->14336 (lowp BF16)", synthetic.make_int4_case(5, 1024, 4096, 14336, 128))
+    run("extra: int4 g128 M=1024 4096->14336 (lowp BF16, cache_weight_for_large_batch)",
+        synthetic.make_int4_case(5, 1024, 4096, 14336, 128), weight_cache=True)
     run("extra: int4 g128 M=16 4096->14336 lowp INT8 asymmetric per-row", synthetic.make_int4_case(5, 16, 4096, 14336, 128), 3, 2)
     run("extra: int4 g64 M=128 4096->14336 lowp INT8 per-row", synthetic.make_int4_case(5, 128, 4096, 14336, 64), 3, 6)
     run("extra: int8 per-channel M=128 4096->11008 +bias lowp INT8 per-row", synthetic.make_int8_case(5, 128, 4096, 11008), 3, 6)
