@@ -272,7 +272,7 @@ __global__ __launch_bounds__(1024, 8) void woq_decode_kernel(const DecodeArgs a_
 // uses anyway -- is the sum over the group of lane column c alone, and that lane column applies the group's
 // (scale, zero) dword; one lane column per group is added at the end.
 template <bool XBF16, int NTW, int KPW, bool ONE_ROUND, bool GROUPED, int GPT>
-__global__ __launch_bounds__(KPW == 2 ? 1024 : 512, KPW == 2 ? 8 : 4) void woq_decode_m1_kernel(const DecodeArgs a_in) {
+__global__ __launch_bounds__(KPW == 4 ? 512 : 1024, KPW == 2 ? 8 : 4) void woq_decode_m1_kernel(const DecodeArgs a_in) {
   static_assert(GPT == 1 || GPT == 2 || GPT == 4, "groups of 128 x 2^k, 64 or 32");
   constexpr bool G32 = GPT > 1;       // the groups of a tile are kept apart
   constexpr int CS = GPT == 2 ? 1 : 0;  // lane columns per group, as a shift
@@ -305,7 +305,9 @@ __global__ __launch_bounds__(KPW == 2 ? 1024 : 512, KPW == 2 ? 8 : 4) void woq_d
   uint16_t* sx = (uint16_t*)smem + (size_t)wave * SLICE * (G32 ? 2 : 1);
   float* red = (float*)(smem + (size_t)W * SLICE * (G32 ? 2 : 1) * sizeof(uint16_t));  // [NTW][16 columns][16 waves]
   if constexpr (G32) {
-    if (lane * 8 < SLICE) *(u4*)(sx + SLICE + lane * 8) = u4{0u, 0u, 0u, 0u};
+#pragma unroll
+    for (int o = 0; o < SLICE; o += 512)
+      if (o + lane * 8 < SLICE) *(u4*)(sx + SLICE + o + lane * 8) = u4{0u, 0u, 0u, 0u};
   }
 
   // buffer resources over the packed weight and its parameters: a load then takes the resource, one
@@ -333,8 +335,9 @@ __global__ __launch_bounds__(KPW == 2 ? 1024 : 512, KPW == 2 ? 8 : 4) void woq_d
 
   const int KT = (int)a.KT, KG = (int)a.KG;
   const int tpg_shift = a.tpg_shift;
-  static_assert(KPW == 2 || KPW == 4, "two or four K tiles per wave and round");
-  const int xlane = lane & (KPW * 16 - 1);  // lanes 32..63 mirror 0..31
+  static_assert(KPW == 2 || KPW == 4 || KPW == 8, "two, four or eight K tiles per wave and round");
+  constexpr int XL = KPW * 16 > 64 ? KPW * 16 / 64 : 1;  // 16-byte pieces of the slice per lane
+  const int xlane = lane & (KPW * 16 - 1);  // (two tiles: lanes 32..63 mirror 0..31)
   // What the last instructions of the kernel need from the argument block, loaded with the rest of it
   // and kept in scalar registers: left to itself the compiler reads them behind the barrier, one
   // dependent scalar load after the other in the only part of the kernel that nothing overlaps.
@@ -348,7 +351,9 @@ __global__ __launch_bounds__(KPW == 2 ? 1024 : 512, KPW == 2 ? 8 : 4) void woq_d
     if (!ONE_ROUND && ktw >= KT) break;
 
     const uint8_t* xbase = (const uint8_t*)a.x + (uint32_t)ktw * (kTileK4 * 2);  // uniform
-    const u4 xs = *(const u4*)(xbase + (uint32_t)xlane * 16u);
+    u4 xs[XL];
+#pragma unroll
+    for (int l = 0; l < XL; ++l) xs[l] = *(const u4*)(xbase + (uint32_t)(xlane + 64 * l) * 16u);
 
     u4 wreg[NTW][KPW];
     uint32_t szreg[NTW][KPW];
@@ -378,15 +383,18 @@ __global__ __launch_bounds__(KPW == 2 ? 1024 : 512, KPW == 2 ? 8 : 4) void woq_d
     }
     __builtin_amdgcn_sched_barrier(0);
 
-    u4 xh = xs;
-    if constexpr (XBF16) {
 #pragma unroll
-      for (int v = 0; v < 4; ++v) {
-        const float lo = bitcast<float>(xs[v] << 16), hi = bitcast<float>(xs[v] & 0xFFFF0000u);
-        xh[v] = bitcast<uint32_t>(__builtin_amdgcn_cvt_pkrtz(lo, hi));  // exact for every fp16-normal value
+    for (int l = 0; l < XL; ++l) {
+      u4 xh = xs[l];
+      if constexpr (XBF16) {
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+          const float lo = bitcast<float>(xs[l][v] << 16), hi = bitcast<float>(xs[l][v] & 0xFFFF0000u);
+          xh[v] = bitcast<uint32_t>(__builtin_amdgcn_cvt_pkrtz(lo, hi));  // exact for every fp16-normal value
+        }
       }
+      *(u4*)(sx + (xlane + 64 * l) * 8) = xh;
     }
-    *(u4*)(sx + xlane * 8) = xh;
 
 #pragma unroll
     for (int i = 0; i < KPW; ++i) {
@@ -561,6 +569,14 @@ static int launch_decode_impl(const FpArgs& f, const uint32_t* sz, hipStream_t s
   a.szbytes = (uint32_t)(f.NT * f.KG * kTileN * (int64_t)sizeof(uint32_t));
   const bool one_row = f.M == 1;
   const bool one_round = f.KT == (int64_t)a.W * kDecodeKPW;
+  if (one_row && !one_round && f.KT % 8 == 0 && f.KT / 8 <= 16 && f.G != 32 && f.G != 64) {
+    // A long K in one round: eight K tiles per wave (8 KiB in flight per wave, a budget of 128 registers) instead of
+    // several rounds of two, each of which waits for its own requests (M = 1, 14336 -> 4096: 7.48 against 7.71 us,
+    // 8192 -> 8192 8.04 against 8.39 us; with groups of 32 the larger zeroed slice makes it a loss, 8.6 against 8.2 us).
+    a.W = (int)(f.KT / 8);
+    if (xf16) return two ? launch_decode_m1_cfg<false, 2, 8, true>(a, st, slots) : launch_decode_m1_cfg<false, 1, 8, true>(a, st, slots);
+    return two ? launch_decode_m1_cfg<true, 2, 8, true>(a, st, slots) : launch_decode_m1_cfg<true, 1, 8, true>(a, st, slots);
+  }
   if (one_row) {
     // Four K tiles per wave (half the waves, each with twice the bytes in flight) where two tiles per
     // wave would leave at most two waves per SIMD anyway: the per-wave overhead then weighs more than
