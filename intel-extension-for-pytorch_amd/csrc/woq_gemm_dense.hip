@@ -144,20 +144,26 @@ __global__ __launch_bounds__(256) void woq_gemm_dense_kernel(const GdArgs a) {
   constexpr int kVmcntBar = 0x0F70 | (NBAR & 15) | ((NBAR >> 4) << 14);
   static_assert(NBLK - 1 + XLOADS < 64, "s_waitcnt vmcnt is a 6-bit field");
 
+  // Prologue: the activations of step 0, then the fragments of step 0 in the order the blocks use them -- all but
+  // the last block's, which block 0 of the loop requests like in every later step (a load whose value nothing reads
+  // would leave its registers free for other uses while it is still in flight).  Only the activations are waited
+  // for here; the loop's per-block waits cover the fragments (the loads behind fragment b -- the rest of the
+  // prologue, the activations of step 1, the refills up to block b -- are as many as in a later step), so the first
+  // MFMAs start when the first fragments are there, not the last.
   load_x(0, 0);
 #pragma unroll
-  for (int t = 0; t < NTW; ++t) {
-    bf[0][t] = gd_load_b<0>(bbase[t], boff);
-    bf[1][t] = gd_load_b<1>(bbase[t], boff);
-    bf[2][t] = gd_load_b<2>(bbase[t], boff);
-    bf[3][t] = gd_load_b<3>(bbase[t], boff);
+  for (int t = 0; t < NTW; ++t) bf[0][t] = gd_load_b<0>(bbase[t], boff);
+#pragma unroll
+  for (int t = 0; t < NTW; ++t) bf[1][t] = gd_load_b<1>(bbase[t], boff);
+#pragma unroll
+  for (int t = 0; t < NTW; ++t) bf[2][t] = gd_load_b<2>(bbase[t], boff);
+#pragma unroll
+  for (int t = 0; t + 1 < NTW; ++t) bf[3][t] = gd_load_b<3>(bbase[t], boff);
+  {
+    constexpr int kVmcntX = 0x0F70 | ((NBLK - 1) & 15) | (((NBLK - 1) >> 4) << 14);  // all but the fragment loads
+    __builtin_amdgcn_s_waitcnt(kVmcntX);
+    asm volatile("s_barrier" ::: "memory");
   }
-  __builtin_amdgcn_s_waitcnt(kVmcnt0);
-#pragma unroll
-  for (int j = 0; j < 4; ++j)
-#pragma unroll
-    for (int t = 0; t < NTW; ++t) asm volatile("" : "+v"(bf[j][t]));
-  __syncthreads();
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) xa[0][mt] = *(const u4*)(sX + mt * 4096 + rd[0]);
   // (the accumulators pass through an opaque statement on both sides of the loop so that they stay whole vectors)
