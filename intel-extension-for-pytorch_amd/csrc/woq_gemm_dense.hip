@@ -20,9 +20,15 @@
 //     that the next block needs (loads return in order: 4 NTW - 1 refills and the XLOADS activation loads of a
 //     step are younger than it).
 //
-// M = 2048, 4096 -> 14336: 184-188 us where woq_gemm_w4_kernel takes 202-204 us; of that the MFMAs with barrier and
-// epilogue alone take 134 us, the A fragments from LDS 9 us, the weight loads 18 us when they hit in L2 and 12 us
-// more from HBM (the dense copy is four times the packed bytes), the activation loads 9 + 2 us.
+// M = 2048, 4096 -> 14336: 166-176 us with one weight copy (cache-resident between launches) and 185-194 us when every
+// launch reads a fresh 117 MB copy from HBM, where woq_gemm_w4_kernel takes 192-205 and 204-215 us.  Stand-alone builds
+// with one part removed at a time (from HBM, 185 us): the MFMAs with barrier and epilogue alone 134 us, the A fragments
+// from LDS 9 us, the weight loads 18 us when they hit in L2 and 12 us more from HBM (the dense copy is four times the
+// packed bytes), the activation loads 9 + 2 us.
+//
+// The inline loads write their registers when the data arrives, not where the instruction stands: a load whose value
+// the program never reads would leave its registers free for the compiler to reuse while it is still in flight.
+// Every load here is therefore followed, on every path, by a wait that is tied to its registers.
 #include <algorithm>
 
 #include "woq_common.h"
