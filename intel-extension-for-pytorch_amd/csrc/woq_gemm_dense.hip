@@ -7,7 +7,7 @@
 // the operand stream of woq_gemm_w4_kernel with the dequantization already done (dense_weight_kernel writes it):
 //
 //   * same workgroup as woq_gemm_w4_kernel -- 4 waves, one per SIMD, wave w owns NTW weight row-blocks for all
-//     16 MT rows; the activations travel global -> LDS (double buffered, swizzled) -> A fragments exactly as
+//     16 MT rows; the activations travel global -> LDS (two to four buffers, swizzled) -> A fragments exactly as
 //     there, and the MFMAs see the same operands in the same order, so the results are bit-identical to the
 //     kernel that dequantizes on the fly;
 //   * a weight fragment (16 rows x 8 K values per lane = 1 KiB per wave) is private to its wave, so it goes from
@@ -25,6 +25,11 @@
 // with one part removed at a time (from HBM, 185 us): the MFMAs with barrier and epilogue alone 134 us, the A fragments
 // from LDS 9 us, the weight loads 18 us when they hit in L2 and 12 us more from HBM (the dense copy is four times the
 // packed bytes), the activation loads 9 + 2 us.
+// A lone, partly filled generation of the narrow shapes is bound by what one CU can pull in (64 KiB per K step of the
+// narrowest shape, about 70 GB/s per CU): 4096 input channels take 30 us on 128-column tiles with the activations
+// three steps ahead (35 us one step ahead) where the MFMAs need 14 us, and a deeper fragment ring in registers on
+// top of that changes nothing; woq_gemm_w4_kernel moves a quarter of the weight bytes and takes 24-28 us there, so
+// the copy pays from about 256 rows up, not below.
 //
 // The inline loads write their registers when the data arrives, not where the instruction stands: a load whose value
 // the program never reads would leave its registers free for the compiler to reuse while it is still in flight.
@@ -47,7 +52,6 @@ struct GdShape {
   static constexpr int BN = GD_WAVES * NTW * kTileN;
   static constexpr int XBYTES = BM * 128 * 2;                 // one activation buffer: BM rows x 128 K values
   static constexpr int XLOADS = XBYTES / (GD_WAVES * 1024);   // LDS loads per wave and buffer
-  static constexpr int LDS_BYTES = 2 * XBYTES;
   static constexpr int SSTRIDE = NTW * kTileN + 4;            // fp32 row stride of the epilogue staging tile
   static constexpr int FETCH_T = NTW >= 2 ? NTW - 2 : 0;      // block that reads the next sub-step's A fragments
   static constexpr int NBLK = 4 * NTW;                        // blocks (row-block x K sub-step) of a K step
@@ -76,7 +80,12 @@ __device__ __forceinline__ u4 gd_load_b(const uint8_t* base, uint32_t off) {
   return v;
 }
 
-template <class S>
+// XD: how many K steps ahead the activations are requested (XD + 1 buffers in LDS).  Because loads return in order,
+// the barrier's wait for the activations of the next step also retires every fragment requested before them: XD
+// bounds how long any load may take.  One step of the widest shape (28 blocks of 8 MFMAs) is long enough; one of the
+// narrowest (8 blocks) is not, and when its workgroups are too few for two to share a CU (which hides the same
+// latency with half the LDS each) it runs with XD = 3.
+template <class S, int XD>
 __global__ __launch_bounds__(256) void woq_gemm_dense_kernel(const GdArgs a) {
   constexpr int MT = S::MT, NTW = S::NTW, BM = S::BM, XBYTES = S::XBYTES, XLOADS = S::XLOADS, NBLK = S::NBLK,
                 SSTRIDE = S::SSTRIDE;
@@ -143,20 +152,24 @@ __global__ __launch_bounds__(256) void woq_gemm_dense_kernel(const GdArgs a) {
   u4 bf[4][NTW];
   u4 xa[2][MT];
   constexpr int kVmcnt0 = 0x0F70;
-  // barrier block: the activation loads of the next step (issued at the top of this one) have landed when at most
-  // the refills issued since are outstanding; two fewer than were issued, for slack
-  constexpr int BARB = 3 * NTW + S::FETCH_T;
+  // barrier block: the activation loads of the next step (issued at the top of step kt + 1 - XD) have landed when at
+  // most the loads issued since are outstanding (XD - 1 whole steps' and this step's refills so far); two fewer than
+  // were issued, for slack
+  constexpr int NXB = XD + 1;
+  constexpr int BARB = (XD - 1) * (NBLK + XLOADS) + 3 * NTW + S::FETCH_T;
   constexpr int NBAR = BARB >= 2 ? BARB - 2 : 0;
+  static_assert(NBAR < 64, "s_waitcnt vmcnt is a 6-bit field");
   constexpr int kVmcntBar = 0x0F70 | (NBAR & 15) | ((NBAR >> 4) << 14);
   static_assert(NBLK - 1 + XLOADS < 64, "s_waitcnt vmcnt is a 6-bit field");
 
-  // Prologue: the activations of step 0, then the fragments of step 0 in the order the blocks use them -- all but
+  // Prologue: the activations of the first XD steps, then the fragments of step 0 in the order the blocks use them -- all but
   // the last block's, which block 0 of the loop requests like in every later step (a load whose value nothing reads
   // would leave its registers free for other uses while it is still in flight).  Only the activations are waited
   // for here; the loop's per-block waits cover the fragments (the loads behind fragment b -- the rest of the
-  // prologue, the activations of step 1, the refills up to block b -- are as many as in a later step), so the first
-  // MFMAs start when the first fragments are there, not the last.
-  load_x(0, 0);
+  // prologue, the activations requested at the top of step 0, the refills up to block b -- are as many as in a later
+  // step), so the first MFMAs start when the first fragments are there, not the last.
+#pragma unroll
+  for (int st = 0; st < XD; ++st) load_x(st < KT ? st : KT - 1, st);
 #pragma unroll
   for (int t = 0; t < NTW; ++t) bf[0][t] = gd_load_b<0>(bbase[t], boff);
 #pragma unroll
@@ -178,11 +191,16 @@ __global__ __launch_bounds__(256) void woq_gemm_dense_kernel(const GdArgs a) {
 #pragma unroll
     for (int t = 0; t < NTW; ++t) asm volatile("" : "+a"(acc[mt][t]));
 
+  int xb = 0;  // the activation buffer of step kt: kt % NXB
   for (int kt = 0; kt < KT; ++kt) {
-    const uint8_t* xs = sX + (kt & 1) * XBYTES;
-    const uint8_t* xsn = sX + ((kt & 1) ^ 1) * XBYTES;
+    const int xbn = xb + 1 == NXB ? 0 : xb + 1, xbp = xb == 0 ? NXB - 1 : xb - 1;
+    const uint8_t* xs = sX + xb * XBYTES;
+    const uint8_t* xsn = sX + xbn * XBYTES;
     const int kt1 = kt + 1 < KT ? kt + 1 : KT - 1;  // past the end the last step is requested again
-    load_x(kt1, (kt & 1) ^ 1);
+    // step kt + XD goes into the buffer of step kt - 1, which every wave has left (that step's barrier stands behind
+    // its last read of it)
+    load_x(kt + XD < KT ? kt + XD : KT - 1, xbp);
+    xb = xbn;
     const uint32_t bko0 = boff + (uint32_t)kt * kstride;
     const uint32_t bko1 = boff + (uint32_t)kt1 * kstride;
     __builtin_amdgcn_sched_barrier(0);
@@ -295,23 +313,35 @@ __global__ __launch_bounds__(256) void woq_gemm_dense_kernel(const GdArgs a) {
   }
 }
 
-template <class S>
-int launch_dense_shape(const GdArgs& a, hipStream_t st) {
-  static_assert(S::LDS_BYTES <= 160 * 1024 && GD_WAVES * 16 * S::SSTRIDE * 4 <= S::LDS_BYTES, "a workgroup's LDS");
-  static const hipError_t lds_optin = hipFuncSetAttribute(reinterpret_cast<const void*>(&woq_gemm_dense_kernel<S>),
-                                                          hipFuncAttributeMaxDynamicSharedMemorySize, S::LDS_BYTES);
+template <class S, int XD>
+int launch_dense_shape_xd(const GdArgs& a, dim3 grid, hipStream_t st) {
+  constexpr int LDS_BYTES = (XD + 1) * S::XBYTES;
+  static_assert(LDS_BYTES <= 160 * 1024 && GD_WAVES * 16 * S::SSTRIDE * 4 <= LDS_BYTES, "a workgroup's LDS");
+  static const hipError_t lds_optin =
+      hipFuncSetAttribute(reinterpret_cast<const void*>(&woq_gemm_dense_kernel<S, XD>),
+                          hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
   if (lds_optin != hipSuccess)
     return set_error("woq_gemm_dense_kernel: LDS opt-in failed: %s", hipGetErrorString(lds_optin));
-  dim3 grid((unsigned)((a.f.NT * kTileN + S::BN - 1) / S::BN), (unsigned)((a.f.M + S::BM - 1) / S::BM));
-  woq_gemm_dense_kernel<S><<<grid, 256, S::LDS_BYTES, st>>>(a);
+  woq_gemm_dense_kernel<S, XD><<<grid, 256, LDS_BYTES, st>>>(a);
   return check_launch("woq_gemm_dense_kernel");
+}
+
+template <class S>
+int launch_dense_shape(const GdArgs& a, hipStream_t st) {
+  dim3 grid((unsigned)((a.f.NT * kTileN + S::BN - 1) / S::BN), (unsigned)((a.f.M + S::BM - 1) / S::BM));
+  // the narrowest shape with one workgroup per CU at most (256 CUs): deeper prefetch instead of a second workgroup
+  if constexpr (S::NTW <= 2) {
+    if ((int64_t)grid.x * grid.y <= 256) return launch_dense_shape_xd<S, 3>(a, grid, st);
+  }
+  return launch_dense_shape_xd<S, 1>(a, grid, st);
 }
 
 // Estimated time of a shape, in microseconds per 4096 input channels, from measurements: a full generation of 256
 // workgroups takes 88 / 54 / 40 us with 7 / 4 / 2 row-blocks per wave; a partial one, alone or behind full ones, is bound
 // by the latency of its weight loads rather than by the chip and takes 66 / 43 / 34 us when nearly empty, rising
 // (with the square of its fill) to the full figure (so the narrow shapes are far from proportional, and two workgroups past a generation
-// cost almost a whole one).
+// cost almost a whole one).  The narrowest shape alone on the chip (256 workgroups at most, deeper prefetch) takes
+// 29.5 us nearly empty and 34.5 us full.
 template <class S>
 double dense_shape_cost(const FpArgs& f) {
   const int64_t wgs = ((f.NT * kTileN + S::BN - 1) / S::BN) * ((f.M + S::BM - 1) / S::BM);
@@ -319,6 +349,7 @@ double dense_shape_cost(const FpArgs& f) {
   const double t_low = S::NTW == 7 ? 66.0 : S::NTW == 4 ? 43.0 : 34.0;
   const int64_t full = wgs / 256, rem = wgs % 256;
   const double fill = (double)rem / 256.0;
+  if (S::NTW <= 2 && wgs <= 256) return 29.5 + 5.0 * (double)wgs / 256.0 * (double)wgs / 256.0;
   return t_full * (double)full + (rem ? t_low + (t_full - t_low) * fill * fill : 0.0);
 }
 

@@ -306,7 +306,9 @@ def test_dense_copy_is_the_bf16_dequantized_weight(cuda, kind, K, N, G, sym):
     [("int4", 130, 512, 448, 128, False, True), ("int4", 128, 1024, 500, 32, True, False),
      ("int4", 257, 384, 300, -1, False, True), ("int4", 64, 256, 1024, 64, False, False),
      ("int8", 96, 512, 272, 128, True, True), ("int8", 200, 256, 128, -1, False, False),
-     ("int4", 70, 128, 176, 128, False, True), ("int4", 5, 256, 64, 32, False, False)],
+     ("int4", 70, 128, 176, 128, False, True), ("int4", 5, 256, 64, 32, False, False),
+     # more than 256 workgroups of the narrowest shape (its variant without the deeper activation prefetch)
+     ("int4", 2100, 256, 2064, 128, False, True), ("int4", 300, 640, 200, 128, False, False)],
 )
 @pytest.mark.parametrize("shape_kernels", [(24, 4), (25, 5), (26, 6)])
 def test_dense_kernel_equals_the_dequantizing_prefill_kernel_bit_for_bit(cuda, kind, M, K, N, G, sym, bias, shape_kernels):
