@@ -32,7 +32,7 @@ MFMA_I8_PEAK_TOPS = 5000.0      # MI355X dense int8, published
 # the figure comes from two rocprofv3 --pmc runs of `bench.py --probe decode` (FETCH_SIZE 15291.09 KiB and
 # WRITE_SIZE 28.00 KiB per dispatch, scaled by what the same counters read for a 256 MiB copy: x2.000 and
 # x1.000), whose summary is the file named beside it; keyed by (M, K, N, group size).  Other shapes: null.
-PROFILED_HBM_BYTES_PER_LAUNCH = {(1, 4096, 14336, 128): 31353978}
+PROFILED_HBM_BYTES_PER_LAUNCH = {(1, 4096, 14336, 128): 31354382}
 PROFILED_HBM_BYTES_SOURCE = "profiles/woq_decode_m1_kernel_M1_4096x14336_g128.hbm_traffic_and_counters.txt"
 # Launches that precede every timed region whatever --warmup says: the first milliseconds after an idle
 # period run 3-10 % slower (clocks, translation caches).
