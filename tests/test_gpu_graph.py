@@ -15,7 +15,7 @@ def _synthetic():
     return synthetic
 
 
-# (label, M, K, N, G, lowp_mode, act_quant_mode)
+# (label, M, K, N, G, lowp_mode, act_quant_mode[, cache_weight_for_large_batch])
 CASES = [
     ("fp16-regime decode kernel", 1, 1024, 256, 128, 2, -1),
     ("dequantizing decode kernel", 16, 1024, 256, 32, 2, -1),
@@ -24,15 +24,16 @@ CASES = [
     ("lowp INT8 prefill, scales per row", 200, 1024, 512, 128, 3, 6),
     ("lowp INT8 prefill, scales per row and K block", 130, 1024, 256, 128, 3, 7),
     ("lowp INT8 small batch", 8, 1024, 256, 128, 3, 6),
+    ("prefill GEMM on the dense copy of the weight cache", 1536, 512, 7168, 128, 2, -1, True),
 ]
 
 
 def test_graph_replays_match_eager(cuda):
     syn = _synthetic()
     ctxs, xs = [], []
-    for i, (_, M, K, N, G, lowp, aq) in enumerate(CASES):
+    for i, (_, M, K, N, G, lowp, aq, *cache) in enumerate(CASES):
         case = syn.make_int4_case(60 + i, M, K, N, G, bias=(i % 2 == 0))
-        ctxs.append(make_context(case, lowp, aq))
+        ctxs.append(make_context(case, lowp, aq, cache=bool(cache)))
         xs.append(case["x"].cuda())
     static_x = [x.clone() for x in xs]
 
@@ -46,6 +47,8 @@ def test_graph_replays_match_eager(cuda):
         run_all()
     torch.cuda.current_stream().wait_stream(s)
     torch.cuda.synchronize()
+    from ipex_amd import _lib
+    assert _lib.last_kernel() == "woq_gemm_dense_kernel"  # the last case runs on the copy
 
     g = torch.cuda.CUDAGraph()
     with torch.cuda.graph(g, stream=s):
