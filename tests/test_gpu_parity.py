@@ -419,6 +419,14 @@ def test_c3_prefill_bf16_with_weight_cache(cuda):
     assert torch.equal(y, y_plain)
     _check_fp(case, O.LOWP_BF16, ctx=ctx, cols=np.arange(0, 14336, 29), label="C3 bf16 dense")
     assert _lib_last_kernel() == "woq_gemm_dense_kernel"
+    # the same through the registered prepack operator, the custom class and torch.ops (the copy is made by the C++
+    # binding at prepack time and handed to the library on every call)
+    tctx = make_torch_context(case, O.LOWP_BF16, cache=True)
+    y_shipped = torch.ops.torch_ipex.ipex_woq_linear(x, tctx.get_data_handle())
+    assert _lib_last_kernel() == "woq_gemm_dense_kernel"
+    assert y_shipped.dtype == y.dtype and torch.equal(y_shipped, y)
+    cached = tctx.get_cached_weight()
+    assert cached is not None and cached.dtype == torch.bfloat16 and cached.numel() == 14336 * 4096
 
 
 def test_c0_int4_g128_m1(cuda):
